@@ -1,0 +1,270 @@
+"""ctypes binding of the CPU oracle (oracle/librnb_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by bench.py's
+cpu_baseline leg.  The shipped package (runnburn_amd) never imports this module.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "librnb_oracle.so")
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14  # ggml type ids (crates/rnb-loader/src/gguf/types.rs:5-41)
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
+
+Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
+Q8_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (32,))])
+assert Q8K_DTYPE.itemsize == 292 and Q8_DTYPE.itemsize == 36
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (make).  Returns the library path."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-s"] + (["-B"] if force else []), check=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        vp, sz, u32, u64, i32, f32 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_uint64, C.c_int, C.c_float
+        L.rnbo_f16_to_f32.restype = f32
+        L.rnbo_f16_to_f32.argtypes = [C.c_uint16]
+        L.rnbo_f32_to_f16.restype = C.c_uint16
+        L.rnbo_f32_to_f16.argtypes = [f32]
+        L.rnbo_nearest_int.restype = i32
+        L.rnbo_nearest_int.argtypes = [f32]
+        L.rnbo_get_scale_min_k4.restype = None
+        L.rnbo_get_scale_min_k4.argtypes = [i32, vp, vp, vp]
+        for name in ("rnbo_dequantize_q8_0", "rnbo_dequantize_q4_k", "rnbo_dequantize_q6_k"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [vp, sz, vp]
+        for name in ("rnbo_quantize_q8k", "rnbo_quantize_q8"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [vp, sz, vp]
+        for name in ("rnbo_dot_q4k_q8k", "rnbo_dot_q6k_q8k", "rnbo_dot_q8_0_q8", "rnbo_dot_q8_0_f32",
+                     "rnbo_dot_q4k_q8k_avx2", "rnbo_dot_q6k_q8k_avx2"):
+            getattr(L, name).restype = f32
+            getattr(L, name).argtypes = [vp, vp, sz]
+        for name in ("rnbo_dot_q4k_q8k_f64", "rnbo_dot_q6k_q8k_f64", "rnbo_dot_q8_0_q8_f64"):
+            getattr(L, name).restype = C.c_double
+            getattr(L, name).argtypes = [vp, vp, sz]
+        for name in ("rnbo_gemv", "rnbo_gemv_f64", "rnbo_gemv_avx2"):
+            getattr(L, name).restype = i32
+            getattr(L, name).argtypes = [u32, vp, sz, sz, vp, sz, vp, i32]
+        L.rnbo_gemv_q8_0_f32act.restype = i32
+        L.rnbo_gemv_q8_0_f32act.argtypes = [vp, sz, sz, vp, sz, vp, i32]
+        L.rnbo_silu_mul_inplace.restype = None
+        L.rnbo_silu_mul_inplace.argtypes = [vp, vp, sz]
+        L.rnbo_route_topk.restype = sz
+        L.rnbo_route_topk.argtypes = [vp, sz, sz, vp, vp]
+        L.rnbo_moe_sparse_experts_by_token.restype = i32
+        L.rnbo_moe_sparse_experts_by_token.argtypes = [vp, vp, vp, sz, vp, vp, vp, sz, sz, u32, sz, sz,
+                                                       vp, vp, i32]
+        for name in ("rnbo_quantize_row_q4_k", "rnbo_quantize_row_q6_k", "rnbo_quantize_row_q8_0"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [vp, sz, vp]
+        L.rnbo_fill_normal.restype = None
+        L.rnbo_fill_normal.argtypes = [vp, sz, u64, f32]
+        L.rnbo_make_weights.restype = i32
+        L.rnbo_make_weights.argtypes = [u32, sz, sz, u64, f32, vp, i32]
+        L.rnbo_have_avx2.restype = i32
+        L.rnbo_have_avx2.argtypes = []
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray) -> C.c_void_p:
+    return C.c_void_p(a.ctypes.data)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a) -> np.ndarray:
+    if isinstance(a, (bytes, bytearray, memoryview)):
+        a = np.frombuffer(a, dtype=np.uint8)
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+# ---- scalar helpers -----------------------------------------------------------------
+
+def f16_to_f32(bits: int) -> float:
+    return float(lib().rnbo_f16_to_f32(bits))
+
+
+def f32_to_f16(value: float) -> int:
+    return int(lib().rnbo_f32_to_f16(C.c_float(value)))
+
+
+def nearest_int(value: float) -> int:
+    return int(lib().rnbo_nearest_int(C.c_float(value)))
+
+
+def get_scale_min_k4(j: int, q12) -> tuple[int, int]:
+    q = _u8(q12)
+    assert q.size == 12
+    sc, mn = C.c_uint8(), C.c_uint8()
+    lib().rnbo_get_scale_min_k4(j, _p(q), C.byref(sc), C.byref(mn))
+    return sc.value, mn.value
+
+
+# ---- dequantisers -------------------------------------------------------------------
+
+def dequantize(quant: int, blocks) -> np.ndarray:
+    b = _u8(blocks)
+    n = b.size // BLOCK_BYTES[quant]
+    assert n * BLOCK_BYTES[quant] == b.size
+    out = np.empty(n * BLOCK_ELEMS[quant], dtype=np.float32)
+    fn = {Q8_0: "rnbo_dequantize_q8_0", Q4_K: "rnbo_dequantize_q4_k", Q6_K: "rnbo_dequantize_q6_k"}[quant]
+    getattr(lib(), fn)(_p(b), n, _p(out))
+    return out
+
+
+# ---- activation quantisers ----------------------------------------------------------
+
+def quantize_q8k(x) -> np.ndarray:
+    x = _f32(x).ravel()
+    assert x.size % 256 == 0
+    out = np.zeros(x.size // 256, dtype=Q8K_DTYPE)
+    lib().rnbo_quantize_q8k(_p(x), x.size, _p(out))
+    return out
+
+
+def quantize_q8(x) -> np.ndarray:
+    x = _f32(x).ravel()
+    assert x.size % 32 == 0
+    out = np.zeros(x.size // 32, dtype=Q8_DTYPE)
+    lib().rnbo_quantize_q8(_p(x), x.size, _p(out))
+    return out
+
+
+# ---- row dots -----------------------------------------------------------------------
+
+def dot(quant: int, row, act: np.ndarray, gold: bool = False, avx2: bool = False) -> float:
+    r = _u8(row)
+    nb = r.size // BLOCK_BYTES[quant]
+    assert act.size == nb
+    base = {Q8_0: "rnbo_dot_q8_0_q8", Q4_K: "rnbo_dot_q4k_q8k", Q6_K: "rnbo_dot_q6k_q8k"}[quant]
+    if gold:
+        base += "_f64"
+    elif avx2:
+        base += "_avx2"
+    act = np.ascontiguousarray(act)
+    return float(getattr(lib(), base)(_p(r), _p(act), nb))
+
+
+def dot_q8_0_f32(row, x) -> float:
+    r, x = _u8(row), _f32(x)
+    return float(lib().rnbo_dot_q8_0_f32(_p(r), _p(x), r.size // 34))
+
+
+# ---- drivers ------------------------------------------------------------------------
+
+def gemv(quant: int, w, rows: int, cols: int, x, gold: bool = False, avx2: bool = False,
+         n_threads: int = 0) -> np.ndarray:
+    """out[seq][rows]; x is [seq][cols] (or [cols])."""
+    w, x = _u8(w), _f32(x)
+    seq = x.size // cols
+    assert x.size == seq * cols
+    assert w.size == rows * (cols // BLOCK_ELEMS[quant]) * BLOCK_BYTES[quant]
+    out = np.empty((seq, rows), dtype=np.float64 if gold else np.float32)
+    fn = "rnbo_gemv_f64" if gold else ("rnbo_gemv_avx2" if avx2 else "rnbo_gemv")
+    rc = getattr(lib(), fn)(quant, _p(w), rows, cols, _p(x), seq, _p(out), n_threads)
+    if rc != 0:
+        raise RuntimeError(f"{fn} failed with code {rc}")
+    return out
+
+
+def gemv_q8_0_f32act(w, rows: int, cols: int, x, n_threads: int = 0) -> np.ndarray:
+    w, x = _u8(w), _f32(x)
+    seq = x.size // cols
+    out = np.empty((seq, rows), dtype=np.float32)
+    rc = lib().rnbo_gemv_q8_0_f32act(_p(w), rows, cols, _p(x), seq, _p(out), n_threads)
+    if rc != 0:
+        raise RuntimeError(f"rnbo_gemv_q8_0_f32act failed with code {rc}")
+    return out
+
+
+# ---- MoE ----------------------------------------------------------------------------
+
+def silu_mul(gate, up) -> np.ndarray:
+    g, u = _f32(gate).copy(), _f32(up)
+    lib().rnbo_silu_mul_inplace(_p(g), _p(u), g.size)
+    return g
+
+
+def route_topk(logits, k: int) -> tuple[np.ndarray, np.ndarray]:
+    lg = _f32(logits)
+    idx = np.zeros(min(k, lg.size), dtype=np.uint32)
+    w = np.zeros(min(k, lg.size), dtype=np.float32)
+    n = lib().rnbo_route_topk(_p(lg), lg.size, k, _p(idx), _p(w))
+    return idx[:n], w[:n]
+
+
+def moe_sparse_experts_by_token(gate_all, up_all, down_all, n_expert: int, expert_ids, route, token_ids,
+                                token_count: int, down_quant: int, n_ff: int, n_embd: int, x,
+                                n_threads: int = 0) -> np.ndarray:
+    g, u, d = _u8(gate_all), _u8(up_all), _u8(down_all)
+    e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
+    r = _f32(route)
+    t = np.ascontiguousarray(token_ids, dtype=np.uint32)
+    x = _f32(x)
+    assert x.size == token_count * n_embd
+    out = np.empty((token_count, n_embd), dtype=np.float32)
+    rc = lib().rnbo_moe_sparse_experts_by_token(_p(g), _p(u), _p(d), n_expert, _p(e), _p(r), _p(t), e.size,
+                                                token_count, down_quant, n_ff, n_embd, _p(x), _p(out),
+                                                n_threads)
+    if rc != 0:
+        raise RuntimeError(f"rnbo_moe_sparse_experts_by_token failed with code {rc}")
+    return out
+
+
+# ---- input generation ---------------------------------------------------------------
+
+def quantize_row(quant: int, x) -> np.ndarray:
+    x = _f32(x).ravel()
+    assert x.size % BLOCK_ELEMS[quant] == 0
+    out = np.zeros(x.size // BLOCK_ELEMS[quant] * BLOCK_BYTES[quant], dtype=np.uint8)
+    fn = {Q8_0: "rnbo_quantize_row_q8_0", Q4_K: "rnbo_quantize_row_q4_k", Q6_K: "rnbo_quantize_row_q6_k"}[quant]
+    getattr(lib(), fn)(_p(x), x.size, _p(out))
+    return out
+
+
+def fill_normal(n: int, seed: int, sigma: float = 1.0) -> np.ndarray:
+    out = np.empty(n, dtype=np.float32)
+    lib().rnbo_fill_normal(_p(out), n, seed, sigma)
+    return out
+
+
+def make_weights(quant: int, rows: int, cols: int, seed: int, sigma: float = 0.02,
+                 n_threads: int = 0) -> np.ndarray:
+    out = np.empty(rows * (cols // BLOCK_ELEMS[quant]) * BLOCK_BYTES[quant], dtype=np.uint8)
+    rc = lib().rnbo_make_weights(quant, rows, cols, seed, sigma, _p(out), n_threads)
+    if rc != 0:
+        raise RuntimeError(f"rnbo_make_weights failed with code {rc}")
+    return out
+
+
+def have_avx2() -> bool:
+    return bool(lib().rnbo_have_avx2())
+
+
+def tensor_seed(config: str, tensor: str, base: int = 20240607) -> int:
+    """Seed per tensor = hash(config id, tensor name) mixed with the base seed (FNV-1a 64)."""
+    h = 0xcbf29ce484222325
+    for ch in f"{base}:{config}:{tensor}".encode():
+        h = ((h ^ ch) * 0x100000001b3) & 0xFFFFFFFFFFFFFFFF
+    return h

@@ -1,0 +1,109 @@
+/*
+ * rnb_oracle.h -- CPU restatement of runNburn's rnb-cpu quantized-matmul arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker that the HIP kernels are
+ * compared against and the CPU baseline that is timed beside them.  It is never linked
+ * into, loaded by, or called from the shipped library (runnburn_amd/librnb_hip.so).
+ *
+ * Every function cites the reference source (paths relative to the reference checkout)
+ * whose arithmetic it restates.  The reference is a Rust workspace and no Rust toolchain
+ * exists here, so the oracle is pinned against the known-answer vectors in the
+ * reference's own unit tests and against independent mathematical checks (see
+ * tests/test_oracle_*.py).
+ *
+ * Pin status per function is listed in rnb_oracle.c's header comment.
+ */
+#ifndef RNB_ORACLE_H
+#define RNB_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RNBO_QK_K 256
+#define RNBO_Q8_0_BLOCK_BYTES 34
+#define RNBO_Q4_K_BLOCK_BYTES 144
+#define RNBO_Q6_K_BLOCK_BYTES 210
+
+/* Q8_K activation block, crates/rnb-cpu/src/gemm/activation_q8.rs:66-72 (repr(C), 292 B). */
+typedef struct {
+    float d;
+    int8_t qs[256];
+    int16_t bsums[16];
+} rnbo_q8k_block;
+
+/* 32-wide activation block, crates/rnb-cpu/src/gemm/activation_q8.rs:7-10 (36 B). */
+typedef struct {
+    float d;
+    int8_t qs[32];
+} rnbo_q8_block;
+
+/* ---- scalar helpers ------------------------------------------------------------ */
+float rnbo_f16_to_f32(uint16_t bits);
+uint16_t rnbo_f32_to_f16(float value);
+void rnbo_get_scale_min_k4(int j, const uint8_t *q12, uint8_t *sc, uint8_t *mn);
+int rnbo_nearest_int(float fval);
+
+/* ---- dequantisers (element order of the formats) -------------------------------- */
+void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_q4_k(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_q6_k(const uint8_t *blocks, size_t n_blocks, float *out);
+
+/* ---- activation quantisers (bit-exact contract) --------------------------------- */
+void rnbo_quantize_q8k(const float *x, size_t n, rnbo_q8k_block *out);
+void rnbo_quantize_q8(const float *x, size_t n, rnbo_q8_block *out);
+
+/* ---- row dots ------------------------------------------------------------------- */
+float rnbo_dot_q4k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_q6k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_q8_0_q8(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
+float rnbo_dot_q8_0_f32(const uint8_t *row, const float *x, size_t n_blocks);
+/* f64-accumulated "gold" forms of the same integer arithmetic */
+double rnbo_dot_q4k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+double rnbo_dot_q6k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+double rnbo_dot_q8_0_q8_f64(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
+
+/* ---- GEMV / GEMM drivers: out[s*rows + row], x is [seq_len][cols] --------------- */
+/* quant: 8 = Q8_0 (Q8 x Q8_0 integer form), 12 = Q4_K, 14 = Q6_K (ggml type ids).  */
+int rnbo_gemv(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
+              size_t seq_len, float *out, int n_threads);
+int rnbo_gemv_f64(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
+                  size_t seq_len, double *out, int n_threads);
+/* x86 default for Q8_0: f32 activations, no activation quantisation. */
+int rnbo_gemv_q8_0_f32act(const uint8_t *w, size_t rows, size_t cols, const float *x,
+                          size_t seq_len, float *out, int n_threads);
+
+/* ---- MoE ------------------------------------------------------------------------ */
+void rnbo_silu_mul_inplace(float *gate, const float *up, size_t n);
+size_t rnbo_route_topk(const float *logits, size_t n_expert, size_t k, uint32_t *idx_out,
+                       float *weights_out);
+int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_all,
+                                     const uint8_t *down_all, size_t n_expert,
+                                     const uint32_t *expert_ids, const float *route,
+                                     const uint32_t *token_ids, size_t n_slots, size_t token_count,
+                                     uint32_t down_quant, size_t n_ff, size_t n_embd,
+                                     const float *x, float *out, int n_threads);
+
+/* ---- input generation (not on the GPU path) ------------------------------------- */
+void rnbo_quantize_row_q4_k(const float *x, size_t n, uint8_t *out);
+void rnbo_quantize_row_q6_k(const float *x, size_t n, uint8_t *out);
+void rnbo_quantize_row_q8_0(const float *x, size_t n, uint8_t *out);
+void rnbo_fill_normal(float *out, size_t n, uint64_t seed, float sigma);
+/* rows x cols fp32 N(0, sigma) from `seed`, quantised row by row; multi-threaded.    */
+int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, float sigma,
+                      uint8_t *out, int n_threads);
+
+/* ---- x86 production-order restatement (AVX2+FMA), used as the timed CPU baseline - */
+int rnbo_have_avx2(void);
+float rnbo_dot_q4k_q8k_avx2(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_q6k_q8k_avx2(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+int rnbo_gemv_avx2(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
+                   size_t seq_len, float *out, int n_threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,469 @@
+"""Pins the CPU oracle WITHOUT running the reference (Rust; no toolchain here): every check is
+either a known-answer vector held by the reference's own unit tests (cited per test), or an
+independent numpy statement of the public format / a mathematical identity, chosen so that a
+dropped term, wrong shift or transposed index fails."""
+import math
+
+import numpy as np
+import pytest
+
+from tests import npref
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+# ---- f16 ----------------------------------------------------------------------------
+
+def test_f16_to_f32_all_bit_patterns(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([oracle.f16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_f32_to_f16_round_to_nearest_even(oracle):
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(0.02),
+        rng.standard_normal(5000).astype(np.float32) * np.float32(1e-6),   # f16 subnormals / underflow
+        rng.standard_normal(5000).astype(np.float32) * np.float32(3e4),    # near overflow
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, 5.96e-8, 2.98e-8, 2.9802322e-8,
+                  6.1035156e-5, 6.0975552e-5, 1.0009766, 1.00048828125, 1.00146484375], dtype=np.float32),
+    ])
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.f32_to_f16(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    # raw constants the reference's tests write by hand (quant_gemv.rs:1226-1227, 1451)
+    assert oracle.f16_to_f32(0x3C00) == 1.0 and oracle.f16_to_f32(0x3800) == 0.5
+
+
+# ---- 6-bit scale/min unpack -----------------------------------------------------------
+
+def test_get_scale_min_k4_known_vector(oracle):
+    # bytes used by crates/rnb-backend/cuda/src/runtime/tests.rs:12494, decoded by hand from
+    # the format: j<4 low six bits; j>=4 low nibble / high nibble of byte j+4 plus top two bits.
+    q = [3, 5, 7, 11, 13, 17, 19, 23, 0x21, 0x43, 0x65, 0x07]
+    want = [(3, 13), (5, 17), (7, 19), (11, 23), (1, 2), (3, 4), (5, 6), (7, 0)]
+    assert [oracle.get_scale_min_k4(j, q) for j in range(8)] == want
+    # with top bits set: byte0 = 0xC3 -> scale4 gets (3<<4), byte4 = 0x8D -> min4 gets (2<<4)
+    q2 = [0xC3, 5, 7, 11, 0x8D, 17, 19, 23, 0x21, 0x43, 0x65, 0x07]
+    assert oracle.get_scale_min_k4(0, q2) == (3, 13)
+    assert oracle.get_scale_min_k4(4, q2) == (1 | (3 << 4), 2 | (2 << 4))
+
+
+def test_get_scale_min_k4_roundtrip_all_positions(oracle):
+    rng = np.random.default_rng(2)
+    for _ in range(200):
+        sc = rng.integers(0, 64, 8)
+        mn = rng.integers(0, 64, 8)
+        q = npref.pack_scales_k4(sc, mn)
+        got = [oracle.get_scale_min_k4(j, q) for j in range(8)]
+        assert got == list(zip(sc.tolist(), mn.tolist()))
+
+
+def test_nearest_int_is_round_half_even(oracle):
+    for v, want in [(0.5, 0), (1.5, 2), (2.5, 2), (-0.5, 0), (-1.5, -2), (-2.5, -2), (3.49, 3), (-3.51, -4),
+                    (4194303.0, 4194303), (-4194303.0, -4194303)]:
+        assert oracle.nearest_int(v) == want
+
+
+# ---- dequantisers: element order and arithmetic ------------------------------------------
+
+def _random_q4k(rng, n):
+    blocks = []
+    for _ in range(n):
+        blocks.append(npref.make_q4k_block(rng.uniform(1e-4, 5e-3), rng.uniform(1e-4, 5e-3),
+                                           rng.integers(0, 64, 8), rng.integers(0, 64, 8),
+                                           rng.integers(0, 16, 256)))
+    return np.concatenate(blocks)
+
+
+def _random_q6k(rng, n):
+    blocks = []
+    for _ in range(n):
+        blocks.append(npref.make_q6k_block(rng.uniform(-5e-4, 5e-4), rng.integers(-128, 128, 16),
+                                           rng.integers(0, 64, 256)))
+    return np.concatenate(blocks)
+
+
+def _random_q8_0(rng, n):
+    return np.concatenate([npref.make_q8_0_block(rng.uniform(1e-4, 1e-2), rng.integers(-128, 128, 32))
+                           for _ in range(n)])
+
+
+def test_dequantize_q4k_places_each_nibble(oracle):
+    # one-hot: a single nibble set -> exactly one output differs from the "-dmin*mn" background
+    for elem in [0, 31, 32, 63, 64, 100, 255]:
+        nib = np.zeros(256, dtype=np.uint8)
+        nib[elem] = 9
+        blk = npref.make_q4k_block(1.0, 0.0, np.arange(1, 9), np.zeros(8), nib)
+        y = oracle.dequantize(Q4_K, blk)
+        want = np.zeros(256, dtype=np.float32)
+        want[elem] = 9.0 * (elem // 32 + 1)
+        assert np.array_equal(y, want)
+    rng = np.random.default_rng(3)
+    blocks = _random_q4k(rng, 64)
+    got = oracle.dequantize(Q4_K, blocks).astype(np.float64)
+    want = npref.dequant_q4k_f64(blocks)
+    assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
+
+
+def test_dequantize_q6k_places_each_value(oracle):
+    for elem in [0, 15, 16, 31, 32, 64, 96, 127, 128, 200, 255]:
+        q = np.full(256, 32, dtype=np.uint8)  # stored 32 == signed 0
+        q[elem] = 32 + 7
+        blk = npref.make_q6k_block(1.0, np.arange(1, 17), q)
+        y = oracle.dequantize(Q6_K, blk)
+        want = np.zeros(256, dtype=np.float32)
+        want[elem] = 7.0 * (elem // 16 + 1)
+        assert np.array_equal(y, want), elem
+    rng = np.random.default_rng(4)
+    blocks = _random_q6k(rng, 64)
+    got = oracle.dequantize(Q6_K, blocks).astype(np.float64)
+    want = npref.dequant_q6k_f64(blocks)
+    assert np.allclose(got, want, rtol=0, atol=1e-6 * np.abs(want).max())
+
+
+def test_dequantize_q8_0(oracle):
+    rng = np.random.default_rng(5)
+    blocks = _random_q8_0(rng, 50)
+    got = oracle.dequantize(Q8_0, blocks).astype(np.float64)
+    assert np.allclose(got, npref.dequant_q8_0_f64(blocks), rtol=1e-7, atol=0)
+
+
+# ---- Q8_K activation quantiser: the reference's exact vectors --------------------------
+
+def test_q8k_reference_vectors(oracle):
+    """crates/rnb-cpu/src/gemm/activation_q8.rs:179-217"""
+    z = oracle.quantize_q8k(np.zeros(256, np.float32))[0]
+    assert z["d"] == 0.0 and not z["qs"].any() and not z["bsums"].any()
+
+    ties = np.zeros(256, np.float32)
+    ties[0] = 127.0
+    ties[1:7] = [-0.5, -1.5, -2.5, 0.5, 1.5, 2.5]
+    b = oracle.quantize_q8k(ties)[0]
+    assert b["d"] == -1.0
+    assert b["qs"][1:7].tolist() == [0, 2, 2, 0, -2, -2]
+
+    fp = np.zeros(256, np.float32)
+    fp[0], fp[1] = 127.0, -127.0
+    b = oracle.quantize_q8k(fp)[0]
+    assert b["d"] == -1.0 and b["qs"][:2].tolist() == [-127, 127]
+
+    fn = np.zeros(256, np.float32)
+    fn[0], fn[1] = -127.0, 127.0
+    b = oracle.quantize_q8k(fn)[0]
+    assert b["d"] == 1.0 and b["qs"][:2].tolist() == [-127, 127]
+
+    bd = np.zeros(256, np.float32)
+    bd[15], bd[16], bd[255] = -1.0, -2.0, 127.0
+    b = oracle.quantize_q8k(bd)[0]
+    assert b["bsums"][0] == 1 and b["bsums"][1] == 2
+    assert not b["bsums"][2:15].any() and b["bsums"][15] == -127
+
+
+def test_q8k_matches_numpy_statement(oracle):
+    # the reference's batch generator (activation_q8.rs:221-224) plus gaussian data
+    idx = np.arange(16 * 256)
+    x1 = ((idx * 73 + 19) % 2001).astype(np.float32) - 1000.0
+    x2 = np.random.default_rng(6).standard_normal(64 * 256).astype(np.float32)
+    for x in (x1, x2):
+        got = oracle.quantize_q8k(x)
+        d, qs, bsums = npref.quantize_q8k_np(x)
+        assert np.array_equal(got["d"].view(np.uint32), d.view(np.uint32))
+        assert np.array_equal(got["qs"], qs)
+        assert np.array_equal(got["bsums"], bsums)
+    # d is 1/iscale, not max/-127: a value where the two differ in the last bit must follow 1/iscale
+    x = np.zeros(256, np.float32)
+    x[3] = np.float32(0.3)
+    b = oracle.quantize_q8k(x)[0]
+    iscale = np.float32(-127.0) / np.float32(0.3)
+    assert b["d"] == np.float32(1.0) / iscale and b["qs"][3] == -127
+
+
+def test_q8_activation_quantiser(oracle):
+    """crates/rnb-cpu/src/gemm/activation_q8.rs:14-32: d = amax/127 (f32), round half AWAY, clamp [-128,127]."""
+    x = np.zeros(32, np.float32)
+    x[0] = 127.0
+    x[1:7] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5]
+    b = oracle.quantize_q8(x)[0]
+    assert b["d"] == 1.0
+    assert b["qs"][:7].tolist() == [127, 1, 2, 3, -1, -2, -3]
+    z = oracle.quantize_q8(np.zeros(32, np.float32))[0]
+    assert z["d"] == 0.0 and not z["qs"].any()
+    xr = np.random.default_rng(7).standard_normal(32 * 100).astype(np.float32)
+    got = oracle.quantize_q8(xr)
+    d, qs = npref.quantize_q8_np(xr)
+    assert np.array_equal(got["d"].view(np.uint32), d.view(np.uint32))
+    assert np.array_equal(got["qs"], qs)
+
+
+# ---- Q4_K x Q8_K dot ------------------------------------------------------------------
+
+def _act_from_parts(d, qs, bsums=None):
+    from oracle.oracle import Q8K_DTYPE
+
+    qs = np.asarray(qs, dtype=np.int8).reshape(-1, 256)
+    a = np.zeros(qs.shape[0], dtype=Q8K_DTYPE)
+    a["d"] = d
+    a["qs"] = qs
+    a["bsums"] = qs.astype(np.int16).reshape(-1, 16, 16).sum(axis=2) if bsums is None else bsums
+    return a
+
+
+def test_q4k_dot_reference_closed_forms(oracle):
+    """crates/rnb-cpu/src/gemm/tile_q4k.rs:2019-2151: zero input -> 0; zero scales -> 0; one sub-block -> 2560."""
+    raw_scales = np.full(12, 10, np.uint8)
+    blk = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(0.5), np.uint8),
+                          raw_scales, np.full(128, 0x88, np.uint8)])
+    act = _act_from_parts(1.0, np.zeros(256, np.int8))
+    assert oracle.dot(Q4_K, blk, act) == 0.0
+
+    blk2 = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(1.0), np.uint8),
+                           np.zeros(12, np.uint8), np.full(128, 0x88, np.uint8)])
+    act2 = _act_from_parts(1.0, np.zeros(256, np.int8), bsums=np.full((1, 16), 50, np.int16))
+    assert oracle.dot(Q4_K, blk2, act2) == 0.0
+
+    sc = np.zeros(12, np.uint8)
+    sc[0] = 10
+    blk3 = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(0.0), np.uint8),
+                           sc, np.full(128, 0x88, np.uint8)])
+    q = np.zeros(256, np.int8)
+    q[:32] = 1
+    assert oracle.dot(Q4_K, blk3, _act_from_parts(1.0, q)) == 2560.0
+    assert oracle.dot(Q4_K, blk3, _act_from_parts(1.0, q), avx2=True) == 2560.0
+
+
+def test_q4k_dot_equals_f64_dequant_identity(oracle):
+    """integer path == sum dequant(W)[i] * (d_x*q_x[i]) computed independently in f64 (the invariant of
+    crates/rnb-cpu/src/gemm/avx2_dot.rs:949-983, here exact instead of loose)."""
+    rng = np.random.default_rng(8)
+    for nb in (1, 2, 7, 16):
+        row = _random_q4k(rng, nb)
+        x = rng.standard_normal(nb * 256).astype(np.float32)
+        act = oracle.quantize_q8k(x)
+        want = float(np.dot(npref.dequant_q4k_f64(row), npref.deq_act_q8k_f64(act)))
+        gold = oracle.dot(Q4_K, row, act, gold=True)
+        assert gold == pytest.approx(want, rel=1e-11, abs=1e-12)
+        scale = float(np.sum(np.abs(npref.dequant_q4k_f64(row) * npref.deq_act_q8k_f64(act))))
+        assert abs(oracle.dot(Q4_K, row, act) - want) <= 4e-7 * scale
+        assert abs(oracle.dot(Q4_K, row, act, avx2=True) - want) <= 4e-7 * scale
+
+
+def test_q4k_mins_use_32_wide_bsums(oracle):
+    # dmin term only: nibbles 0, mins 1..8, bsums chosen per 16 -> summ = sum mn[k]*(bsums[2k]+bsums[2k+1])
+    blk = npref.make_q4k_block(0.0, 1.0, np.zeros(8), np.arange(1, 9), np.zeros(256))
+    bs = np.arange(1, 17, dtype=np.int16).reshape(1, 16)
+    act = _act_from_parts(2.0, np.zeros(256, np.int8), bsums=bs)
+    summ = sum((k + 1) * (bs[0, 2 * k] + bs[0, 2 * k + 1]) for k in range(8))
+    assert oracle.dot(Q4_K, blk, act) == -2.0 * summ
+    assert oracle.dot(Q4_K, blk, act, avx2=True) == -2.0 * summ
+
+
+# ---- Q6_K x Q8_K dot ------------------------------------------------------------------
+
+def test_q6k_dot_equals_f64_dequant_identity(oracle):
+    rng = np.random.default_rng(9)
+    for nb in (1, 3, 16, 56):
+        row = _random_q6k(rng, nb)
+        x = rng.standard_normal(nb * 256).astype(np.float32)
+        act = oracle.quantize_q8k(x)
+        want = float(np.dot(npref.dequant_q6k_f64(row), npref.deq_act_q8k_f64(act)))
+        assert oracle.dot(Q6_K, row, act, gold=True) == pytest.approx(want, rel=1e-11, abs=1e-14)
+        scale = float(np.sum(np.abs(npref.dequant_q6k_f64(row) * npref.deq_act_q8k_f64(act))))
+        assert abs(oracle.dot(Q6_K, row, act) - want) <= 4e-7 * scale
+        assert abs(oracle.dot(Q6_K, row, act, avx2=True) - want) <= 4e-7 * scale
+
+
+def test_q6k_bsums_identity(oracle):
+    """sum sc*(q-32)*x == sum sc*q*x - 32*sum sc[sb]*bsums[sb] (crates/rnb-cpu/src/gemm/avx2_dot.rs:824,880)."""
+    rng = np.random.default_rng(10)
+    row = _random_q6k(rng, 1)
+    x = rng.standard_normal(256).astype(np.float32)
+    act = oracle.quantize_q8k(x)
+    d, sc, q = npref.split_q6k(row)
+    u = (q + 32).reshape(16, 16)
+    a = act["qs"][0].astype(np.int64).reshape(16, 16)
+    lhs = int(np.sum(sc[0][:, None] * (u - 32) * a))
+    rhs = int(np.sum(sc[0][:, None] * u * a)) - 32 * int(np.sum(sc[0] * act["bsums"][0].astype(np.int64)))
+    assert lhs == rhs
+    got = oracle.dot(Q6_K, row, act, gold=True)
+    assert got == pytest.approx(float(d[0]) * float(act["d"][0]) * lhs, rel=1e-12)
+
+
+# ---- Q8_0 ----------------------------------------------------------------------------
+
+REF_Q8_0_BYTES = bytes([0x00, 0x3C] + list(range(1, 33)) + [0x00, 0x3C] + list(range(32, 0, -1)))
+
+
+def test_q8_0_reference_seq_major_vector(oracle):
+    """crates/rnb-cpu/src/gemm/quant_gemv.rs:1448-1464: rows 1..32 / 32..1, d = 1, x = 1 -> 528 everywhere,
+    output index s*rows + row."""
+    x = np.ones(64, np.float32)
+    out = oracle.gemv_q8_0_f32act(REF_Q8_0_BYTES, 2, 32, x)
+    assert out.shape == (2, 2) and np.all(out == 528.0)
+    # distinguishable rows/tokens to pin the layout itself
+    x2 = np.concatenate([np.ones(32, np.float32), 2 * np.ones(32, np.float32)])
+    w = np.concatenate([npref.make_q8_0_block(1.0, np.ones(32)), npref.make_q8_0_block(1.0, 3 * np.ones(32))])
+    out = oracle.gemv_q8_0_f32act(w, 2, 32, x2)
+    assert out.ravel().tolist() == [32.0, 96.0, 64.0, 192.0]
+    out_q = oracle.gemv(Q8_0, w, 2, 32, x2)
+    assert np.allclose(out_q.ravel(), [32.0, 96.0, 64.0, 192.0], rtol=1e-6)
+
+
+def test_q8_0_q8_matches_engine_oracle(oracle):
+    """crates/rnb-llm/src/engine/tests.rs:6872-6896: out = d_x * sum(w*q) when d_w = 1."""
+    values = np.array([(i % 7) - 3 for i in range(64)], dtype=np.int8)
+    w = np.concatenate([npref.make_q8_0_block(1.0, values[:32]), npref.make_q8_0_block(1.0, values[32:])])
+    x = (np.arange(32, dtype=np.float32) - 16.0) * 0.25
+    act = oracle.quantize_q8(x)
+    out = oracle.gemv(Q8_0, w, 2, 32, x)[0]
+    for r in range(2):
+        dot = int(np.dot(values[32 * r:32 * r + 32].astype(np.int64), act["qs"][0].astype(np.int64)))
+        assert abs(out[r] - float(act["d"][0]) * dot) < 1e-5
+
+
+def test_q8_0_q8_equals_f64_identity(oracle):
+    rng = np.random.default_rng(11)
+    row = _random_q8_0(rng, 128)
+    x = rng.standard_normal(4096).astype(np.float32)
+    act = oracle.quantize_q8(x)
+    ax = (act["qs"].astype(np.float64) * act["d"].astype(np.float64)[:, None]).reshape(-1)
+    want = float(np.dot(npref.dequant_q8_0_f64(row), ax))
+    assert oracle.dot(Q8_0, row, act, gold=True) == pytest.approx(want, rel=1e-11)
+    assert oracle.dot(Q8_0, row, act) == pytest.approx(want, rel=2e-5)
+    assert oracle.dot_q8_0_f32(row, x) == pytest.approx(float(np.dot(npref.dequant_q8_0_f64(row), x.astype(np.float64))), rel=2e-5, abs=1e-5)
+
+
+# ---- drivers --------------------------------------------------------------------------
+
+@pytest.mark.parametrize("quant,maker", [(Q4_K, _random_q4k), (Q6_K, _random_q6k)])
+def test_gemv_driver_layout_and_row_independence(oracle, quant, maker):
+    rng = np.random.default_rng(12)
+    rows, nb, seq = 5, 2, 3
+    w = maker(rng, rows * nb)
+    x = rng.standard_normal((seq, nb * 256)).astype(np.float32)
+    out = oracle.gemv(quant, w, rows, nb * 256, x)
+    rb = w.size // rows
+    for s in range(seq):
+        act = oracle.quantize_q8k(x[s])
+        for r in range(rows):
+            assert out[s, r] == np.float32(oracle.dot(quant, w[r * rb:(r + 1) * rb], act))
+    gold = oracle.gemv(quant, w, rows, nb * 256, x, gold=True)
+    assert np.allclose(out, gold, rtol=1e-4, atol=1e-6)
+    fast = oracle.gemv(quant, w, rows, nb * 256, x, avx2=True)
+    assert np.allclose(fast, gold, rtol=1e-4, atol=1e-6)
+    # 1 thread == many threads, bitwise (rows are independent)
+    assert np.array_equal(oracle.gemv(quant, w, rows, nb * 256, x, n_threads=1), out)
+
+
+# ---- router ---------------------------------------------------------------------------
+
+def test_router_reference_vectors(oracle):
+    """crates/rnb-llm/src/engine/models/shared_expert_moe/routing.rs:272-318"""
+    idx, w = oracle.route_topk([0.0, 4.0, 3.0, 2.0], 2)
+    assert idx.tolist() == [1, 2] and abs(w.sum() - 1.0) < 1e-6 and w[0] > w[1]
+    idx, w = oracle.route_topk([1.0, 4.0, 4.0, -2.0, 3.0], 3)
+    assert idx.tolist() == [1, 2, 4]
+    e4, e3 = 1.0, math.exp(-1.0)
+    s = e4 + e4 + e3
+    assert np.allclose(w, [e4 / s, e4 / s, e3 / s], atol=1e-6)
+
+
+def test_router_against_numpy_sort(oracle):
+    rng = np.random.default_rng(13)
+    for _ in range(20):
+        lg = rng.standard_normal(128).astype(np.float32)
+        idx, w = oracle.route_topk(lg, 8)
+        order = np.lexsort((np.arange(128), -lg))[:8]  # logit desc, ties -> lower id
+        assert idx.tolist() == order.tolist()
+        e = np.exp(lg[order].astype(np.float64) - float(lg[order[0]]))
+        assert np.allclose(w, e / e.sum(), rtol=1e-5)
+
+
+# ---- SiLU * up ------------------------------------------------------------------------
+
+def test_silu_mul(oracle):
+    g = np.array([0.0, 1.0, -1.0, 5.0, -20.0, 30.0], np.float32)
+    u = np.array([2.0, 3.0, 4.0, -1.0, 1.0, 0.5], np.float32)
+    want = g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64))) * u
+    assert np.allclose(oracle.silu_mul(g, u), want, rtol=1e-6, atol=1e-12)
+
+
+# ---- MoE ------------------------------------------------------------------------------
+
+def test_moe_matches_f32_dequant_statement(oracle):
+    """The reference's CUDA-test oracle (crates/rnb-backend/cuda/src/runtime/tests.rs:29561-29584) is an
+    f32-dequant statement of gate/up -> SiLU*up -> Q6_K down -> route-weighted sum; the integer path agrees
+    with an independent f64 dequant statement up to activation-quantisation noise (~1e-2 relative)."""
+    n_expert, n_ff, n_embd = 4, 256, 512
+    w_gate = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, 101)
+    w_up = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, 102)
+    w_down = oracle.make_weights(Q6_K, n_expert * n_embd, n_ff, 103)
+    x = oracle.fill_normal(2 * n_embd, 104).reshape(2, n_embd)
+    expert_ids = np.array([2, 0, 3, 1, 2], np.uint32)
+    token_ids = np.array([0, 0, 0, 1, 1], np.uint32)
+    route = np.array([0.5, 0.3, 0.2, 0.6, 0.4], np.float32)
+    out = oracle.moe_sparse_experts_by_token(w_gate, w_up, w_down, n_expert, expert_ids, route, token_ids, 2,
+                                             Q6_K, n_ff, n_embd, x)
+    G = npref.dequant_q4k_f64(w_gate).reshape(n_expert, n_ff, n_embd)
+    U = npref.dequant_q4k_f64(w_up).reshape(n_expert, n_ff, n_embd)
+    D = npref.dequant_q6k_f64(w_down).reshape(n_expert, n_embd, n_ff)
+    want = np.zeros((2, n_embd))
+    for e, t, r in zip(expert_ids, token_ids, route):
+        g = G[e] @ x[t].astype(np.float64)
+        u = U[e] @ x[t].astype(np.float64)
+        a = g / (1.0 + np.exp(-g)) * u
+        want[t] += r * (D[e] @ a)
+    err = np.abs(out - want).max() / np.abs(want).max()
+    assert err < 3e-2, err
+    # exact composition: one slot == gemv(gate), gemv(up), silu, gemv(down) * w, bitwise
+    pg = n_ff * (n_embd // 256) * 144
+    pd = n_embd * (n_ff // 256) * 210
+    g = oracle.gemv(Q4_K, w_gate[2 * pg:3 * pg], n_ff, n_embd, x[0])[0]
+    u = oracle.gemv(Q4_K, w_up[2 * pg:3 * pg], n_ff, n_embd, x[0])[0]
+    a = oracle.silu_mul(g, u)
+    o = oracle.gemv(Q6_K, w_down[2 * pd:3 * pd], n_embd, n_ff, a)[0] * np.float32(0.5)
+    one = oracle.moe_sparse_experts_by_token(w_gate, w_up, w_down, n_expert, [2], [0.5], [0], 1, Q6_K, n_ff,
+                                             n_embd, x[0])
+    assert np.array_equal(one[0], o)
+    # token batching does not change a (token, expert) result: 1-token call == row of the 2-token call
+    solo = oracle.moe_sparse_experts_by_token(w_gate, w_up, w_down, n_expert, expert_ids[:3], route[:3],
+                                              [0, 0, 0], 1, Q6_K, n_ff, n_embd, x[0])
+    assert np.array_equal(solo[0], out[0])
+
+
+# ---- weight generators (input generation only) -----------------------------------------
+
+def test_q4k_quantiser_roundtrip_property(oracle):
+    """crates/rnb-cpu/src/quantize/quant.rs:766-798: quantise -> dequantise cosine >= 0.97.  Byte parity with
+    the Rust quantiser is UNPINNED (cannot run it); GPU and oracle consume identical bytes regardless."""
+    x = oracle.fill_normal(256 * 40, 21, 0.02)
+    y = oracle.dequantize(Q4_K, oracle.quantize_row(Q4_K, x))
+    cos = float(np.dot(x, y) / (np.linalg.norm(x) * np.linalg.norm(y)))
+    assert cos >= 0.97
+    assert np.sqrt(np.mean((x - y) ** 2)) / np.sqrt(np.mean(x ** 2)) < 0.1
+
+
+def test_q6k_q8_0_generators_roundtrip(oracle):
+    x = oracle.fill_normal(256 * 40, 22, 0.02)
+    y6 = oracle.dequantize(Q6_K, oracle.quantize_row(Q6_K, x))
+    assert np.sqrt(np.mean((x - y6) ** 2)) / np.sqrt(np.mean(x ** 2)) < 0.03
+    y8 = oracle.dequantize(Q8_0, oracle.quantize_row(Q8_0, x))
+    assert np.sqrt(np.mean((x - y8) ** 2)) / np.sqrt(np.mean(x ** 2)) < 0.01
+    # scales spread over the 6-bit / int8 range as for real weights
+    d, dmin, sc, mn, nib = npref.split_q4k(oracle.quantize_row(Q4_K, x))
+    assert sc.max() == 63 and nib.max() == 15 and nib.min() == 0
+
+
+def test_generator_is_counter_based_and_normal(oracle):
+    a = oracle.fill_normal(100000, 5, 1.0)
+    assert abs(a.mean()) < 0.02 and abs(a.std() - 1.0) < 0.02
+    w1 = oracle.make_weights(Q4_K, 8, 512, 77, n_threads=1)
+    w2 = oracle.make_weights(Q4_K, 8, 512, 77, n_threads=4)
+    assert np.array_equal(w1, w2)
+    row3 = oracle.quantize_row(Q4_K, oracle.fill_normal(8 * 512, 77, 0.02)[3 * 512:4 * 512])
+    assert np.array_equal(w1[3 * 288:4 * 288], row3)
