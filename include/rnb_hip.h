@@ -1,0 +1,152 @@
+/*
+ * rnb_hip.h -- C ABI of the MI355X (gfx950) backend for runNburn's quantized matmul path.
+ *
+ * Every entry point states the reference interface it replaces (paths relative to the
+ * reference checkout).  The ABI uses plain pointers and sizes only; all functions return an
+ * rnb_hip_status and leave a message retrievable with rnb_hip_last_error() (thread-local).
+ *
+ * Semantics are those of the reference's rnb-cpu crate: activations are quantised on the
+ * device to Q8_K (256-wide, crates/rnb-cpu/src/gemm/activation_q8.rs:149-173) for Q4_K / Q6_K
+ * weights and to the 32-wide f32-scale Q8 block (:14-32) for Q8_0 weights; weight blocks are
+ * consumed exactly as stored in GGUF (34 / 144 / 210 bytes, no repack, no requantisation).
+ *
+ * Threading model (crates/rnb-backend/cuda/src/runtime.rs:9): one process-global state behind
+ * a mutex, opened lazily on first use, one device, one stream.  Host-pointer entry points
+ * block until the result is in the caller's buffer.  `_dev` entry points only enqueue on the
+ * library stream (rnb_hip_stream()) and return.
+ */
+#ifndef RNB_HIP_H
+#define RNB_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error classes of crates/rnb-backend/api/src/lib.rs:55-108 (BackendErrorKind) plus NO_DEVICE so
+ * that callers can skip like crates/rnb-backend/cuda/src/runtime/tests.rs:22831-22834. */
+typedef enum {
+    RNB_HIP_OK = 0,
+    RNB_HIP_INVALID_REQUEST = 1,
+    RNB_HIP_UNSUPPORTED_OP = 2,
+    RNB_HIP_EXECUTION_FAILED = 3,
+    RNB_HIP_NO_DEVICE = 4
+} rnb_hip_status;
+
+/* ggml type ids, crates/rnb-loader/src/gguf/types.rs:5-41 */
+#define RNB_GGML_Q8_0 8u
+#define RNB_GGML_Q4_K 12u
+#define RNB_GGML_Q6_K 14u
+
+/* BackendOp, crates/rnb-backend/api/src/lib.rs:12-18 */
+#define RNB_OP_MATMUL 0
+#define RNB_OP_ATTENTION 1
+#define RNB_OP_GDN 2
+#define RNB_OP_MOE 3
+#define RNB_OP_SAMPLER 4
+
+/* ---- trait facade: crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend) ------------ */
+/* kind(): the reference's BackendKind (:2-9) has no HIP variant; this returns the ordinal a new
+ * `Hip` variant appended to that enum would take (6). */
+int rnb_hip_backend_kind(void);
+/* capabilities(): 1 when `op` (RNB_OP_*) executes on this backend, else 0. */
+int rnb_hip_backend_supports(int op);
+/* 1 when (op, ggml quant id) is supported: MatMul x {Q8_0,Q4_K,Q6_K}; MoE x gate/up Q4_K with
+ * down Q4_K|Q6_K (pass the down quant). */
+int rnb_hip_backend_supports_quant(int op, uint32_t quant);
+
+/* ---- lifecycle / diagnostics -------------------------------------------------------------- */
+/* CudaState::open (crates/rnb-backend/cuda/src/runtime/state/init.rs:75-118): opens device
+ * RNB_HIP_DEVICE (default 0) lazily; explicit call returns RNB_HIP_NO_DEVICE when none opens. */
+int rnb_hip_init(void);
+const char *rnb_hip_last_error(void);
+int rnb_hip_device_name(char *buf, size_t buf_len);
+/* cuStreamSynchronize at the end of every reference call (runtime/gemv.rs:285-295) */
+int rnb_hip_sync(void);
+/* DeviceTransferCounters, crates/rnb-backend/api/src/lib.rs:213-242 */
+int rnb_hip_transfer_counters(uint64_t *h2d_bytes, uint64_t *d2h_bytes);
+/* the library's only stream, as a hipStream_t */
+void *rnb_hip_stream(void);
+
+/* ---- weight residency: crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:399-405,757-851 */
+/* prewarm_q4k_weights (api/quant_api.rs:952): upload host ranges untouched and keep them
+ * resident, keyed by (pointer, length, sampled fingerprint).  Sub-ranges of a resident range
+ * resolve to parent + offset (q4k_cache.rs:722-741). */
+int rnb_hip_prewarm(const uint8_t *const *ptrs, const size_t *lens, size_t n);
+/* drop a resident range (call before unmapping the host bytes) */
+int rnb_hip_release(const uint8_t *ptr, size_t len);
+int rnb_hip_resident_bytes(uint64_t *bytes, uint64_t *entries);
+
+/* ---- activation quantisers (bit-exact contract) --------------------------------------------- */
+/* quantize_input_q8k, crates/rnb-cpu/src/gemm/activation_q8.rs:109-139: n floats (n % 256 == 0)
+ * -> n/256 blocks of {f32 d; i8 qs[256]; i16 bsums[16]} = 292 bytes each, computed on the device. */
+int rnb_hip_quantize_q8k(const float *x, size_t n, void *out_blocks, size_t out_bytes);
+/* quantize_input_q8, activation_q8.rs:14-32: n floats (n % 32 == 0) -> n/32 blocks of
+ * {f32 d; i8 qs[32]} = 36 bytes each. */
+int rnb_hip_quantize_q8(const float *x, size_t n, void *out_blocks, size_t out_bytes);
+
+/* ---- operator surface, host in / host out ------------------------------------------------- */
+/* q4k_gemv / q4k_gemv_into, crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-238,340-365:
+ * out[row] = Q4_K row . Q8_K(x);  x_len == cols, out_len >= rows. */
+int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                     size_t x_len, float *out, size_t out_len);
+/* q4k_gemv_batch, quant_api.rs:2283-2319: seq_len = x_len / cols, out[s*rows + row],
+ * out_len >= seq_len*rows.  seq_len >= 16 takes the int8-MFMA GEMM. */
+int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                           const float *x, size_t x_len, float *out, size_t out_len);
+/* q6k_gemv / q6k_gemv_into, quant_api.rs:2071-2168 */
+int rnb_hip_q6k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                     size_t x_len, float *out, size_t out_len);
+/* q6k_gemv_batch, quant_api.rs:3919-3955 */
+int rnb_hip_q6k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                           const float *x, size_t x_len, float *out, size_t out_len);
+/* q8_0_gemv, quant_api.rs:498-505 (validation in q5_basic_gemv :1983-2028); semantics are the
+ * Q8 x Q8_0 integer dot of crates/rnb-cpu/src/gemm/neon_dot.rs:376-436 */
+int rnb_hip_q8_0_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+/* q8_0_gemv_batch, quant_api.rs:807-822 */
+int rnb_hip_q8_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
+
+/* qwen35_sparse_experts_selected_base_by_token, crates/rnb-backend/cuda/src/runtime/api/
+ * qwen_moe_api.rs:2529-2541 (validation: runtime/helpers.rs:1496-1600, 2747-2800): whole-layer
+ * expert tensors + per-slot (expert id, route weight, token id).  Gate/up are Q4_K
+ * [n_expert][n_ff][n_embd]; down is [n_expert][n_embd][n_ff] in `down_quant` (12 = Q4_K,
+ * 14 = Q6_K).  out[token][n_embd] = sum over that token's slots, in slot order, of
+ * route * W_down[e] . Q8_K(silu(W_gate[e] . Q8_K(x)) * (W_up[e] . Q8_K(x))). */
+int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len,
+                                        const uint8_t *up_all, size_t up_len,
+                                        const uint8_t *down_all, size_t down_len,
+                                        const uint32_t *expert_ids, const float *route_weights,
+                                        const uint32_t *token_ids, size_t n_slots,
+                                        size_t token_count, uint32_t down_quant, size_t n_ff,
+                                        size_t n_embd, const float *x, size_t x_len, float *out,
+                                        size_t out_len);
+
+/* ---- device-resident variants --------------------------------------------------------------
+ * The reference's device-input entry points (quant_api.rs:242-330 take `input_dev: u64`) keep
+ * activations on the device between operators.  These take device pointers for weights, input
+ * and output, enqueue on the library stream and return without synchronising. */
+void *rnb_hip_dev_alloc(size_t bytes);
+int rnb_hip_dev_free(void *ptr);
+int rnb_hip_dev_upload(void *dst_dev, const void *src_host, size_t bytes);
+int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes);
+/* quant: RNB_GGML_*; x_dev [seq_len][cols] f32 (16-byte aligned); out_dev [seq_len][rows] f32 */
+int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
+                     const float *x_dev, size_t seq_len, float *out_dev);
+/* device-resident form of rnb_hip_moe_sparse_experts_by_token: weights, x and out on the device;
+ * the slot arrays stay on the host (the caller routes on the host, as the reference does). */
+int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev,
+                                            const void *down_dev, size_t n_expert,
+                                            const uint32_t *expert_ids,
+                                            const float *route_weights, const uint32_t *token_ids,
+                                            size_t n_slots, size_t token_count,
+                                            uint32_t down_quant, size_t n_ff, size_t n_embd,
+                                            const float *x_dev, float *out_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

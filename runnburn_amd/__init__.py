@@ -1,0 +1,54 @@
+"""runnburn_amd -- MI355X (gfx950) backend for runNburn's quantized matmul hot path.
+
+Python mirror of the reference's operator surface over the C ABI in include/rnb_hip.h.  The
+functions keep the reference's names, argument meaning and error behaviour:
+`Result<Vec<f32>, String>` becomes "return an array or raise BackendError(message)".
+
+  q4k_gemv / q4k_gemv_into / q4k_gemv_batch   crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-238, 2283-2319
+  q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
+  q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
+  qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
+  HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
+
+There is no CPU fallback: when librnb_hip.so is missing or no gfx950 device opens, every
+operator raises.
+"""
+from __future__ import annotations
+
+from .binding import (  # noqa: F401
+    BackendError,
+    HipBackend,
+    DeviceBuffer,
+    GGML_Q4_K,
+    GGML_Q6_K,
+    GGML_Q8_0,
+    OP_MATMUL,
+    OP_MOE,
+    STATUS_NAMES,
+    device_available,
+    device_name,
+    gemv_dev,
+    last_error,
+    lib,
+    lib_path,
+    moe_sparse_experts_by_token_dev,
+    prewarm,
+    q4k_gemv,
+    q4k_gemv_batch,
+    q4k_gemv_into,
+    q6k_gemv,
+    q6k_gemv_batch,
+    q6k_gemv_into,
+    q8_0_gemv,
+    q8_0_gemv_batch,
+    quantize_input_q8,
+    quantize_input_q8k,
+    qwen35_sparse_experts_selected_base_by_token,
+    release,
+    resident_bytes,
+    stream_handle,
+    sync,
+    transfer_counters,
+)
+
+__all__ = [name for name in dir() if not name.startswith("_")]

@@ -1,0 +1,329 @@
+"""ctypes binding of librnb_hip.so and the host-side mirror of the reference's operator functions."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Sequence
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_PKG, "librnb_hip.so")
+
+GGML_Q8_0, GGML_Q4_K, GGML_Q6_K = 8, 12, 14
+OP_MATMUL, OP_ATTENTION, OP_GDN, OP_MOE, OP_SAMPLER = 0, 1, 2, 3, 4
+STATUS_NAMES = {0: "Ok", 1: "InvalidRequest", 2: "UnsupportedOp", 3: "ExecutionFailed", 4: "NoDevice"}
+
+# every symbol include/rnb_hip.h declares: (name, restype, argtypes)
+_vp, _sz, _u32, _u64p, _i = C.c_void_p, C.c_size_t, C.c_uint32, C.POINTER(C.c_uint64), C.c_int
+_MATMUL_ARGS = [_vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz]
+SYMBOLS = [
+    ("rnb_hip_backend_kind", _i, []),
+    ("rnb_hip_backend_supports", _i, [_i]),
+    ("rnb_hip_backend_supports_quant", _i, [_i, _u32]),
+    ("rnb_hip_init", _i, []),
+    ("rnb_hip_last_error", C.c_char_p, []),
+    ("rnb_hip_device_name", _i, [C.c_char_p, _sz]),
+    ("rnb_hip_sync", _i, []),
+    ("rnb_hip_transfer_counters", _i, [_u64p, _u64p]),
+    ("rnb_hip_stream", _vp, []),
+    ("rnb_hip_prewarm", _i, [C.POINTER(_vp), C.POINTER(_sz), _sz]),
+    ("rnb_hip_release", _i, [_vp, _sz]),
+    ("rnb_hip_resident_bytes", _i, [_u64p, _u64p]),
+    ("rnb_hip_quantize_q8k", _i, [_vp, _sz, _vp, _sz]),
+    ("rnb_hip_quantize_q8", _i, [_vp, _sz, _vp, _sz]),
+    ("rnb_hip_q4k_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_q4k_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_q6k_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_q6k_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_q8_0_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_q8_0_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_moe_sparse_experts_by_token", _i,
+     [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
+    ("rnb_hip_dev_alloc", _vp, [_sz]),
+    ("rnb_hip_dev_free", _i, [_vp]),
+    ("rnb_hip_dev_upload", _i, [_vp, _vp, _sz]),
+    ("rnb_hip_dev_download", _i, [_vp, _vp, _sz]),
+    ("rnb_hip_gemv_dev", _i, [_u32, _vp, _sz, _sz, _vp, _sz, _vp]),
+    ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
+     [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
+]
+
+Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
+Q8_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (32,))])
+
+
+class BackendError(RuntimeError):
+    """BackendError of crates/rnb-backend/api/src/lib.rs:55-108: kind + message."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(message)
+        self.status = status
+        self.kind = STATUS_NAMES.get(status, str(status))
+        self.message = message
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def lib() -> C.CDLL:
+    """Loads the HIP extension.  Raises when it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(f"{_LIB_PATH} is missing: build it with `python -m runnburn_amd.build` "
+                              "(hipcc --offload-arch=gfx950); runnburn_amd has no CPU fallback")
+        L = C.CDLL(_LIB_PATH)
+        for name, restype, argtypes in SYMBOLS:
+            fn = getattr(L, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = L
+    return _lib
+
+
+def last_error() -> str:
+    msg = lib().rnb_hip_last_error()
+    return msg.decode("utf-8", "replace") if msg else ""
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise BackendError(status, last_error())
+
+
+def device_available() -> bool:
+    return lib().rnb_hip_init() == 0
+
+
+def device_name() -> str:
+    buf = C.create_string_buffer(256)
+    _check(lib().rnb_hip_device_name(buf, 256))
+    return buf.value.decode()
+
+
+def sync() -> None:
+    _check(lib().rnb_hip_sync())
+
+
+def stream_handle() -> int:
+    return int(lib().rnb_hip_stream() or 0)
+
+
+def transfer_counters() -> tuple[int, int]:
+    a, b = C.c_uint64(), C.c_uint64()
+    _check(lib().rnb_hip_transfer_counters(C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def resident_bytes() -> tuple[int, int]:
+    a, b = C.c_uint64(), C.c_uint64()
+    _check(lib().rnb_hip_resident_bytes(C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def _bytes_view(w) -> np.ndarray:
+    if isinstance(w, np.ndarray):
+        if w.dtype != np.uint8 or not w.flags.c_contiguous:
+            raise TypeError("weights must be a C-contiguous uint8 array (raw GGUF block bytes)")
+        return w
+    return np.frombuffer(w, dtype=np.uint8)
+
+
+def _f32(x) -> np.ndarray:
+    return np.ascontiguousarray(x, dtype=np.float32)
+
+
+def _ptr(a: np.ndarray) -> C.c_void_p:
+    return C.c_void_p(a.ctypes.data)
+
+
+def prewarm(weights: Sequence) -> None:
+    """prewarm_q4k_weights(&[&[u8]]), quant_api.rs:952"""
+    views = [_bytes_view(w) for w in weights]
+    n = len(views)
+    ptrs = (_vp * n)(*[v.ctypes.data for v in views])
+    lens = (_sz * n)(*[v.size for v in views])
+    _check(lib().rnb_hip_prewarm(ptrs, lens, n))
+
+
+def release(weights) -> None:
+    v = _bytes_view(weights)
+    _check(lib().rnb_hip_release(_ptr(v), v.size))
+
+
+# ---- activation quantisers ---------------------------------------------------------------
+
+def quantize_input_q8k(x) -> np.ndarray:
+    """quantize_input_q8k, crates/rnb-cpu/src/gemm/activation_q8.rs:109-119, computed on the device."""
+    x = _f32(x).ravel()
+    out = np.zeros(x.size // 256 if x.size % 256 == 0 else 0, dtype=Q8K_DTYPE)
+    _check(lib().rnb_hip_quantize_q8k(_ptr(x), x.size, _ptr(out), out.nbytes))
+    return out
+
+
+def quantize_input_q8(x) -> np.ndarray:
+    """quantize_input_q8, crates/rnb-cpu/src/gemm/activation_q8.rs:14-32, computed on the device."""
+    x = _f32(x).ravel()
+    out = np.zeros(x.size // 32 if x.size % 32 == 0 else 0, dtype=Q8_DTYPE)
+    _check(lib().rnb_hip_quantize_q8(_ptr(x), x.size, _ptr(out), out.nbytes))
+    return out
+
+
+# ---- operator surface ---------------------------------------------------------------------
+
+def _gemv(fn_name: str, weights, rows: int, cols: int, x) -> np.ndarray:
+    w, x = _bytes_view(weights), _f32(x).ravel()
+    out = np.empty(rows, dtype=np.float32)
+    _check(getattr(lib(), fn_name)(_ptr(w), w.size, rows, cols, _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+def _gemv_into(fn_name: str, weights, rows: int, cols: int, x, output: np.ndarray) -> None:
+    w, x = _bytes_view(weights), _f32(x).ravel()
+    if output.dtype != np.float32 or not output.flags.c_contiguous:
+        raise TypeError("output must be a C-contiguous float32 array")
+    _check(getattr(lib(), fn_name)(_ptr(w), w.size, rows, cols, _ptr(x), x.size, _ptr(output), output.size))
+
+
+def _gemv_batch(fn_name: str, weights, rows: int, cols: int, x) -> np.ndarray:
+    w, x = _bytes_view(weights), _f32(x).ravel()
+    seq = x.size // cols if cols and x.size % cols == 0 else 0
+    out = np.empty((seq, rows), dtype=np.float32)
+    _check(getattr(lib(), fn_name)(_ptr(w), w.size, rows, cols, _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+def q4k_gemv(weights, rows, cols, input):  # noqa: A002 - the reference's argument name
+    return _gemv("rnb_hip_q4k_gemv", weights, rows, cols, input)
+
+
+def q4k_gemv_into(weights, rows, cols, input, output):  # noqa: A002
+    _gemv_into("rnb_hip_q4k_gemv", weights, rows, cols, input, output)
+
+
+def q4k_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    """seq_len = len(input) / cols; returns out[seq][rows]"""
+    return _gemv_batch("rnb_hip_q4k_gemv_batch", weights, rows, cols, input)
+
+
+def q6k_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_q6k_gemv", weights, rows, cols, input)
+
+
+def q6k_gemv_into(weights, rows, cols, input, output):  # noqa: A002
+    _gemv_into("rnb_hip_q6k_gemv", weights, rows, cols, input, output)
+
+
+def q6k_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_q6k_gemv_batch", weights, rows, cols, input)
+
+
+def q8_0_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_q8_0_gemv", weights, rows, cols, input)
+
+
+def q8_0_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_q8_0_gemv_batch", weights, rows, cols, input)
+
+
+def qwen35_sparse_experts_selected_base_by_token(gate_all, up_all, down_all, expert_ids, route_weights, token_ids,
+                                                 token_count: int, down_quant: int, n_ff: int, n_embd: int,
+                                                 input) -> np.ndarray:  # noqa: A002
+    """api/qwen_moe_api.rs:2529-2541; returns out[token_count][n_embd]."""
+    g, u, d = _bytes_view(gate_all), _bytes_view(up_all), _bytes_view(down_all)
+    e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
+    r = _f32(route_weights).ravel()
+    t = np.ascontiguousarray(token_ids, dtype=np.uint32)
+    if not (e.size == r.size == t.size):
+        raise BackendError(1, f"Qwen35 full-layer token-batch length mismatch: expert={e.size} route={r.size} "
+                              f"token={t.size}")
+    x = _f32(input).ravel()
+    out = np.empty((token_count, n_embd), dtype=np.float32)
+    _check(lib().rnb_hip_moe_sparse_experts_by_token(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, _ptr(e),
+                                                     _ptr(r), _ptr(t), e.size, token_count, down_quant, n_ff, n_embd,
+                                                     _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+# ---- device-resident helpers (benchmarks, fused callers) -----------------------------------
+
+class DeviceBuffer:
+    """A hipMalloc'd range owned by the library's device."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        self.ptr = lib().rnb_hip_dev_alloc(self.nbytes)
+        if not self.ptr:
+            raise BackendError(3, last_error())
+
+    @classmethod
+    def from_host(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        buf = cls(a.nbytes)
+        _check(lib().rnb_hip_dev_upload(buf.ptr, _ptr(a), a.nbytes))
+        return buf
+
+    def to_host(self, dtype, count: Optional[int] = None) -> np.ndarray:
+        dt = np.dtype(dtype)
+        n = self.nbytes // dt.itemsize if count is None else count
+        out = np.empty(n, dtype=dt)
+        _check(lib().rnb_hip_dev_download(_ptr(out), self.ptr, out.nbytes))
+        return out
+
+    def free(self) -> None:
+        if self.ptr:
+            lib().rnb_hip_dev_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def gemv_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, x: DeviceBuffer, seq_len: int,
+             out: DeviceBuffer) -> None:
+    """Enqueue activation quantisation + GEMV/GEMM on the library stream; does not synchronise."""
+    _check(lib().rnb_hip_gemv_dev(quant, w.ptr, rows, cols, x.ptr, seq_len, out.ptr))
+
+
+def moe_sparse_experts_by_token_dev(gate: DeviceBuffer, up: DeviceBuffer, down: DeviceBuffer, n_expert: int,
+                                    expert_ids, route_weights, token_ids, token_count: int, down_quant: int,
+                                    n_ff: int, n_embd: int, x: DeviceBuffer, out: DeviceBuffer) -> None:
+    e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
+    r = _f32(route_weights).ravel()
+    t = np.ascontiguousarray(token_ids, dtype=np.uint32)
+    _check(lib().rnb_hip_moe_sparse_experts_by_token_dev(gate.ptr, up.ptr, down.ptr, n_expert, _ptr(e), _ptr(r),
+                                                         _ptr(t), e.size, token_count, down_quant, n_ff, n_embd,
+                                                         x.ptr, out.ptr))
+
+
+# ---- trait facade --------------------------------------------------------------------------
+
+class HipBackend:
+    """Capability facade in the shape of `trait Backend` (crates/rnb-backend/api/src/lib.rs:1281-1285).
+    Like CudaBackend::execute (crates/rnb-backend/cuda/src/lib.rs:193-195), execute() does not run
+    requests: real work flows through the operator functions above."""
+
+    def kind(self) -> str:
+        return "Hip"
+
+    def kind_ordinal(self) -> int:
+        return lib().rnb_hip_backend_kind()
+
+    def capabilities(self) -> dict:
+        names = {OP_MATMUL: "MatMul", OP_ATTENTION: "Attention", OP_GDN: "Gdn", OP_MOE: "MoE", OP_SAMPLER: "Sampler"}
+        return {name: bool(lib().rnb_hip_backend_supports(op)) for op, name in names.items()}
+
+    def supports_quant(self, op: int, quant: int) -> bool:
+        return bool(lib().rnb_hip_backend_supports_quant(op, quant))
+
+    def execute(self, request) -> None:
+        raise BackendError(2, "HipBackend::execute: requests are served by the operator functions "
+                              "(q4k_gemv, q6k_gemv, q8_0_gemv, *_batch, qwen35_sparse_experts_*)")

@@ -1,0 +1,568 @@
+// extern "C" surface of the HIP backend (include/rnb_hip.h): validation with the reference's
+// messages, staging through pinned bounce buffers, kernel sequencing on the single stream.
+#include "../../include/rnb_hip.h"
+
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+#include "state.h"
+
+using namespace rnb;
+
+namespace {
+
+struct QuantInfo {
+    const char *label;
+    size_t elems;
+    size_t bytes;
+};
+
+bool quant_info(uint32_t quant, QuantInfo *qi) {
+    switch (quant) {
+    case kQ8_0: *qi = {"Q8_0", 32, kQ8_0Bytes}; return true;
+    case kQ4K: *qi = {"Q4_K", 256, kQ4KBytes}; return true;
+    case kQ6K: *qi = {"Q6_K", 256, kQ6KBytes}; return true;
+    default: return false;
+    }
+}
+
+int fail(int status, const std::string &msg) {
+    set_last_error(msg);
+    return status;
+}
+
+int hip_fail(const char *what, hipError_t e) {
+    return fail(RNB_HIP_EXECUTION_FAILED, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                      \
+    do {                                                   \
+        hipError_t _e = (expr);                            \
+        if (_e != hipSuccess) return hip_fail(#expr, _e);  \
+    } while (0)
+
+// Quantise seq*cols staged floats on the device into the state's activation scratch.
+int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view) {
+    const size_t n = seq * cols;
+    HIP_TRY(s.act_qs.reserve(n));
+    if (quant == kQ8_0) {
+        HIP_TRY(s.act_d.reserve(n / 32 * sizeof(float)));
+        launch_quantize_q8(x_dev, n / 32, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.stream);
+        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), nullptr};
+    } else {
+        HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
+        HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
+        launch_quantize_q8k(x_dev, n / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
+                            s.stream);
+        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
+    }
+    HIP_TRY(hipGetLastError());
+    return RNB_HIP_OK;
+}
+
+// Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
+constexpr size_t kGemmMinSeq = 16;
+
+int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, const float *x_dev,
+                   size_t seq, float *out_dev) {
+    ActView act;
+    int st = quantize_activations(s, quant, x_dev, seq, cols, &act);
+    if (st != RNB_HIP_OK) return st;
+    const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
+    if (quant == kQ4K) {
+        if (seq >= kGemmMinSeq)
+            launch_gemm_q4k_mfma(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+        else
+            launch_gemv_q4k(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+    } else if (quant == kQ6K) {
+        launch_gemv_q6k(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+    } else {
+        launch_gemv_q8_0(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
+    }
+    HIP_TRY(hipGetLastError());
+    return RNB_HIP_OK;
+}
+
+// Validation order and messages: crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-206 (gemv),
+// :340-358 (gemv_into), :2283-2307 (batch), :1983-2009 / :2030-2057 (Q8_0).
+int validate_matmul(const QuantInfo &qi, size_t w_len, size_t rows, size_t cols, size_t x_len, size_t out_len,
+                    bool batch, size_t *seq_out) {
+    const std::string label = qi.label;
+    if (cols == 0 || cols % qi.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    label + " cols must be divisible by " + std::to_string(qi.elems) + ", got " + std::to_string(cols));
+    size_t seq = 1;
+    if (batch) {
+        if (x_len % cols != 0)
+            return fail(RNB_HIP_INVALID_REQUEST, label + " batch input length " + std::to_string(x_len) +
+                                                     " is not divisible by cols " + std::to_string(cols));
+        seq = x_len / cols;
+    }
+    const size_t row_bytes = cols / qi.elems * qi.bytes;
+    if (w_len != rows * row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " weight byte mismatch: got " + std::to_string(w_len) +
+                                                 ", expected " + std::to_string(rows * row_bytes));
+    if (!batch && x_len != cols && out_len >= rows)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " input length mismatch: got " + std::to_string(x_len) +
+                                                 ", expected " + std::to_string(cols));
+    if (!batch && (x_len != cols || out_len < rows))
+        return fail(RNB_HIP_INVALID_REQUEST, label + " shape mismatch: input=" + std::to_string(x_len) +
+                                                 " output=" + std::to_string(out_len) + " expected input=" +
+                                                 std::to_string(cols) + " output>=" + std::to_string(rows));
+    if (batch && out_len < seq * rows)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " shape mismatch: input=" + std::to_string(x_len) +
+                                                 " output=" + std::to_string(out_len) + " expected output>=" +
+                                                 std::to_string(seq * rows));
+    if (rows > 0x7fffffffu || seq > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " shape out of range: rows=" + std::to_string(rows) +
+                                                 " seq_len=" + std::to_string(seq));
+    *seq_out = seq;
+    return RNB_HIP_OK;
+}
+
+int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                size_t x_len, float *out, size_t out_len, bool batch) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    size_t seq = 0;
+    int st = validate_matmul(qi, w_len, rows, cols, x_len, out_len, batch, &seq);
+    if (st != RNB_HIP_OK) return st;
+    if ((w_len && !w) || (x_len && !x) || (out_len && !out))
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " null pointer argument");
+    if (rows == 0 || seq == 0) return RNB_HIP_OK;
+
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *w_dev = nullptr;
+    HIP_TRY(s.resident_ptr(w, w_len, &w_dev));
+    const size_t in_bytes = seq * cols * sizeof(float), out_bytes = seq * rows * sizeof(float);
+    HIP_TRY(s.bounce_in.reserve(in_bytes));
+    HIP_TRY(s.bounce_out.reserve(out_bytes));
+    HIP_TRY(s.x_f32.reserve(in_bytes));
+    HIP_TRY(s.out_f32.reserve(out_bytes));
+    std::memcpy(s.bounce_in.ptr, x, in_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += in_bytes;
+    st = run_matmul_dev(s, quant, w_dev, rows, cols, s.x_f32.as<float>(), seq, s.out_f32.as<float>());
+    if (st != RNB_HIP_OK) return st;
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += out_bytes;
+    std::memcpy(out, s.bounce_out.ptr, out_bytes);
+    return RNB_HIP_OK;
+}
+
+// ---- MoE ------------------------------------------------------------------------------------
+
+struct MoeShape {
+    size_t per_gate, per_down, n_expert, nb_in, nb_mid;
+};
+
+// Messages: crates/rnb-backend/cuda/src/runtime/helpers.rs:1570-1600 (selected-base shape) and
+// :2747-2800 (full-layer token batch).
+int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t *expert_ids,
+                 const uint32_t *token_ids, size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff,
+                 size_t n_embd, size_t x_len, size_t out_len, MoeShape *shape) {
+    if (x_len != token_count * n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer input length mismatch: got " + std::to_string(x_len) +
+                                                 ", expected " + std::to_string(token_count * n_embd));
+    if (n_embd == 0 || n_ff == 0 || n_embd % 256 != 0 || n_ff % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer dims must be divisible by 256, got n_ff=" +
+                                                 std::to_string(n_ff) + " n_embd=" + std::to_string(n_embd));
+    for (size_t i = 0; i < n_slots; i++)
+        if (token_ids[i] >= token_count)
+            return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer token id out of range");
+    size_t down_block;
+    switch (down_quant) {
+    case kQ4K: down_block = kQ4KBytes; break;
+    case kQ6K: down_block = kQ6KBytes; break;
+    default:
+        return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported Qwen35 HIP down quant code " + std::to_string(down_quant));
+    }
+    MoeShape sh;
+    sh.nb_in = n_embd / 256;
+    sh.nb_mid = n_ff / 256;
+    sh.per_gate = n_ff * sh.nb_in * kQ4KBytes;
+    sh.per_down = n_embd * sh.nb_mid * down_block;
+    if (gate_len % sh.per_gate != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base gate length is not expert-aligned: len=" +
+                                                 std::to_string(gate_len) + " per_expert=" + std::to_string(sh.per_gate));
+    sh.n_expert = gate_len / sh.per_gate;
+    if (up_len != sh.n_expert * sh.per_gate)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base up length mismatch: len=" + std::to_string(up_len) +
+                                                 " expected=" + std::to_string(sh.n_expert * sh.per_gate));
+    if (down_len != sh.n_expert * sh.per_down)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base down length mismatch: len=" +
+                                                 std::to_string(down_len) + " expected=" +
+                                                 std::to_string(sh.n_expert * sh.per_down));
+    for (size_t i = 0; i < n_slots; i++)
+        if (expert_ids[i] >= sh.n_expert)
+            return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base expert id out of range: id=" +
+                                                     std::to_string(expert_ids[i]) + " n_expert=" +
+                                                     std::to_string(sh.n_expert));
+    if (out_len < token_count * n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer output length mismatch: got " +
+                                                 std::to_string(out_len) + ", expected >= " +
+                                                 std::to_string(token_count * n_embd));
+    if (n_slots > 0x0fffffffu || token_count > 0x0fffffffu)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer slot count out of range");
+    *shape = sh;
+    return RNB_HIP_OK;
+}
+
+// Device-side sequence for the gathered expert path.  x_dev [token_count][n_embd], out_dev likewise.
+int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev,
+                const MoeShape &sh, const uint32_t *expert_ids, const float *route, const uint32_t *token_ids,
+                size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
+                const float *x_dev, float *out_dev) {
+    if (token_count == 0) return RNB_HIP_OK;
+    // host tables: expert[n], token[n], route[n], tok_offsets[T+1], tok_slots[n]
+    const size_t table_words = 4 * n_slots + token_count + 1;
+    HIP_TRY(s.bounce_tables.reserve(table_words * 4));
+    HIP_TRY(s.moe_tables.reserve(table_words * 4));
+    uint32_t *h = s.bounce_tables.as<uint32_t>();
+    uint32_t *h_expert = h, *h_token = h + n_slots;
+    float *h_route = reinterpret_cast<float *>(h + 2 * n_slots);
+    uint32_t *h_off = h + 3 * n_slots, *h_list = h_off + token_count + 1;
+    HIP_TRY(hipStreamSynchronize(s.stream));  // the previous call's table upload must have drained
+    std::memcpy(h_expert, expert_ids, n_slots * 4);
+    std::memcpy(h_token, token_ids, n_slots * 4);
+    std::memcpy(h_route, route, n_slots * 4);
+    std::vector<uint32_t> counts(token_count + 1, 0);
+    for (size_t i = 0; i < n_slots; i++) counts[token_ids[i] + 1]++;
+    for (size_t t = 0; t < token_count; t++) counts[t + 1] += counts[t];
+    std::memcpy(h_off, counts.data(), (token_count + 1) * 4);
+    for (size_t i = 0; i < n_slots; i++) h_list[counts[token_ids[i]]++] = static_cast<uint32_t>(i);  // slot order kept
+    uint32_t *d = s.moe_tables.as<uint32_t>();
+    HIP_TRY(hipMemcpyAsync(d, h, table_words * 4, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += table_words * 4;
+    MoeSlots slots{d, d + n_slots, reinterpret_cast<const float *>(d + 2 * n_slots), static_cast<uint32_t>(n_slots)};
+    const uint32_t *d_off = d + 3 * n_slots, *d_list = d_off + token_count + 1;
+
+    if (n_slots == 0) {  // nothing routed: the reduce kernel alone writes the zero rows
+        launch_moe_reduce(nullptr, d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
+                          static_cast<uint32_t>(n_embd), s.stream);
+        HIP_TRY(hipGetLastError());
+        return RNB_HIP_OK;
+    }
+    ActView act;
+    int st = quantize_activations(s, kQ4K, x_dev, token_count, n_embd, &act);
+    if (st != RNB_HIP_OK) return st;
+    HIP_TRY(s.moe_mid.reserve(n_slots * n_ff * sizeof(float)));
+    HIP_TRY(s.moe_mid_qs.reserve(n_slots * n_ff));
+    HIP_TRY(s.moe_mid_d.reserve(n_slots * sh.nb_mid * sizeof(float)));
+    HIP_TRY(s.moe_mid_bsums.reserve(n_slots * sh.nb_mid * 16 * sizeof(int16_t)));
+    HIP_TRY(s.moe_slot_out.reserve(n_slots * n_embd * sizeof(float)));
+    launch_moe_gate_up(gate_dev, up_dev, act, slots, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
+                       static_cast<uint32_t>(sh.nb_in), s.stream);
+    launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
+                        s.moe_mid_bsums.as<int16_t>(), s.stream);
+    ActView mid{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>()};
+    launch_moe_down(down_dev, down_quant, mid, slots, s.moe_slot_out.as<float>(), static_cast<uint32_t>(n_embd),
+                    static_cast<uint32_t>(sh.nb_mid), s.stream);
+    launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
+                      static_cast<uint32_t>(n_embd), s.stream);
+    HIP_TRY(hipGetLastError());
+    return RNB_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rnb_hip_backend_kind(void) { return 6; }
+
+int rnb_hip_backend_supports(int op) { return (op == RNB_OP_MATMUL || op == RNB_OP_MOE) ? 1 : 0; }
+
+int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
+    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || quant == kQ4K || quant == kQ6K) ? 1 : 0;
+    if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ6K) ? 1 : 0;
+    return 0;
+}
+
+int rnb_hip_init(void) {
+    Guard g;
+    return g.state ? RNB_HIP_OK : g.status;
+}
+
+const char *rnb_hip_last_error(void) { return last_error_cstr(); }
+
+int rnb_hip_device_name(char *buf, size_t buf_len) {
+    Guard g;
+    if (!g.state) return g.status;
+    if (!buf || buf_len == 0) return fail(RNB_HIP_INVALID_REQUEST, "device_name: empty buffer");
+    std::strncpy(buf, g.state->device_name.c_str(), buf_len - 1);
+    buf[buf_len - 1] = 0;
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_sync(void) {
+    Guard g;
+    if (!g.state) return g.status;
+    HIP_TRY(hipStreamSynchronize(g.state->stream));
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_transfer_counters(uint64_t *h2d_bytes, uint64_t *d2h_bytes) {
+    Guard g;
+    if (!g.state) return g.status;
+    if (h2d_bytes) *h2d_bytes = g.state->h2d_bytes;
+    if (d2h_bytes) *d2h_bytes = g.state->d2h_bytes;
+    return RNB_HIP_OK;
+}
+
+void *rnb_hip_stream(void) {
+    Guard g;
+    return g.state ? static_cast<void *>(g.state->stream) : nullptr;
+}
+
+int rnb_hip_prewarm(const uint8_t *const *ptrs, const size_t *lens, size_t n) {
+    Guard g;
+    if (!g.state) return g.status;
+    for (size_t i = 0; i < n; i++) {
+        if (!ptrs[i] || lens[i] == 0) continue;
+        const uint8_t *dev = nullptr;
+        HIP_TRY(g.state->resident_ptr(ptrs[i], lens[i], &dev, /*pin=*/true));
+    }
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_release(const uint8_t *ptr, size_t len) {
+    Guard g;
+    if (!g.state) return g.status;
+    if (!g.state->release(ptr, len)) return fail(RNB_HIP_INVALID_REQUEST, "release: range is not resident");
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_resident_bytes(uint64_t *bytes, uint64_t *entries) {
+    Guard g;
+    if (!g.state) return g.status;
+    if (bytes) *bytes = g.state->resident_bytes;
+    if (entries) *entries = g.state->residents.size();
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_quantize_q8k(const float *x, size_t n, void *out_blocks, size_t out_bytes) {
+    if (n % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_K input length must be divisible by 256, got " + std::to_string(n));
+    const size_t nb = n / 256;
+    if (out_bytes < nb * 292)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_K output byte mismatch: got " + std::to_string(out_bytes) +
+                                                 ", expected " + std::to_string(nb * 292));
+    if (nb == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    HIP_TRY(s.bounce_in.reserve(n * 4));
+    HIP_TRY(s.x_f32.reserve(n * 4));
+    std::memcpy(s.bounce_in.ptr, x, n * 4);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, n * 4, hipMemcpyHostToDevice, s.stream));
+    ActView act;
+    int st = quantize_activations(s, kQ4K, s.x_f32.as<float>(), 1, n, &act);
+    if (st != RNB_HIP_OK) return st;
+    const size_t qs_b = n, d_b = nb * 4, bs_b = nb * 32;
+    HIP_TRY(s.bounce_out.reserve(qs_b + d_b + bs_b));
+    uint8_t *h = s.bounce_out.as<uint8_t>();
+    HIP_TRY(hipMemcpyAsync(h, act.qs, qs_b, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipMemcpyAsync(h + qs_b, act.d, d_b, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipMemcpyAsync(h + qs_b + d_b, act.bsums, bs_b, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.h2d_bytes += n * 4;
+    s.d2h_bytes += qs_b + d_b + bs_b;
+    // repack the device structure-of-arrays into the reference's 292-byte repr(C) block
+    uint8_t *o = static_cast<uint8_t *>(out_blocks);
+    for (size_t b = 0; b < nb; b++) {
+        std::memcpy(o + b * 292, h + qs_b + b * 4, 4);
+        std::memcpy(o + b * 292 + 4, h + b * 256, 256);
+        std::memcpy(o + b * 292 + 260, h + qs_b + d_b + b * 32, 32);
+    }
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_quantize_q8(const float *x, size_t n, void *out_blocks, size_t out_bytes) {
+    if (n % 32 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8 input length must be divisible by 32, got " + std::to_string(n));
+    const size_t nb = n / 32;
+    if (out_bytes < nb * 36)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8 output byte mismatch: got " + std::to_string(out_bytes) +
+                                                 ", expected " + std::to_string(nb * 36));
+    if (nb == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    HIP_TRY(s.bounce_in.reserve(n * 4));
+    HIP_TRY(s.x_f32.reserve(n * 4 + 1024));
+    std::memcpy(s.bounce_in.ptr, x, n * 4);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, n * 4, hipMemcpyHostToDevice, s.stream));
+    ActView act;
+    int st = quantize_activations(s, kQ8_0, s.x_f32.as<float>(), 1, n, &act);
+    if (st != RNB_HIP_OK) return st;
+    HIP_TRY(s.bounce_out.reserve(n + nb * 4));
+    uint8_t *h = s.bounce_out.as<uint8_t>();
+    HIP_TRY(hipMemcpyAsync(h, act.qs, n, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipMemcpyAsync(h + n, act.d, nb * 4, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.h2d_bytes += n * 4;
+    s.d2h_bytes += n + nb * 4;
+    uint8_t *o = static_cast<uint8_t *>(out_blocks);
+    for (size_t b = 0; b < nb; b++) {
+        std::memcpy(o + b * 36, h + n + b * 4, 4);
+        std::memcpy(o + b * 36 + 4, h + b * 32, 32);
+    }
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                     float *out, size_t out_len) {
+    return matmul_host(kQ4K, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                           float *out, size_t out_len) {
+    return matmul_host(kQ4K, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+int rnb_hip_q6k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                     float *out, size_t out_len) {
+    return matmul_host(kQ6K, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q6k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                           float *out, size_t out_len) {
+    return matmul_host(kQ6K, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+int rnb_hip_q8_0_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                      float *out, size_t out_len) {
+    return matmul_host(kQ8_0, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q8_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                            float *out, size_t out_len) {
+    return matmul_host(kQ8_0, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+
+int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len, const uint8_t *up_all,
+                                        size_t up_len, const uint8_t *down_all, size_t down_len,
+                                        const uint32_t *expert_ids, const float *route_weights,
+                                        const uint32_t *token_ids, size_t n_slots, size_t token_count,
+                                        uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x, size_t x_len,
+                                        float *out, size_t out_len) {
+    MoeShape sh;
+    int st = validate_moe(gate_len, up_len, down_len, expert_ids, token_ids, n_slots, token_count, down_quant, n_ff,
+                          n_embd, x_len, out_len, &sh);
+    if (st != RNB_HIP_OK) return st;
+    if (token_count == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *gate_dev = nullptr, *up_dev = nullptr, *down_dev = nullptr;
+    HIP_TRY(s.resident_ptr(gate_all, gate_len, &gate_dev));
+    HIP_TRY(s.resident_ptr(up_all, up_len, &up_dev));
+    HIP_TRY(s.resident_ptr(down_all, down_len, &down_dev));
+    const size_t io_bytes = token_count * n_embd * sizeof(float);
+    HIP_TRY(s.bounce_in.reserve(io_bytes));
+    HIP_TRY(s.bounce_out.reserve(io_bytes));
+    HIP_TRY(s.x_f32.reserve(io_bytes));
+    HIP_TRY(s.out_f32.reserve(io_bytes));
+    std::memcpy(s.bounce_in.ptr, x, io_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, io_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += io_bytes;
+    st = run_moe_dev(s, gate_dev, up_dev, down_dev, sh, expert_ids, route_weights, token_ids, n_slots, token_count,
+                     down_quant, n_ff, n_embd, s.x_f32.as<float>(), s.out_f32.as<float>());
+    if (st != RNB_HIP_OK) return st;
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, io_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += io_bytes;
+    std::memcpy(out, s.bounce_out.ptr, io_bytes);
+    return RNB_HIP_OK;
+}
+
+// ---- device-resident variants ------------------------------------------------------------------
+
+void *rnb_hip_dev_alloc(size_t bytes) {
+    Guard g;
+    if (!g.state) return nullptr;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        hip_fail("hipMalloc", e);
+        return nullptr;
+    }
+    return p;
+}
+
+int rnb_hip_dev_free(void *ptr) {
+    Guard g;
+    if (!g.state) return g.status;
+    HIP_TRY(hipStreamSynchronize(g.state->stream));
+    HIP_TRY(hipFree(ptr));
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_dev_upload(void *dst_dev, const void *src_host, size_t bytes) {
+    Guard g;
+    if (!g.state) return g.status;
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, g.state->stream));
+    HIP_TRY(hipStreamSynchronize(g.state->stream));
+    g.state->h2d_bytes += bytes;
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes) {
+    Guard g;
+    if (!g.state) return g.status;
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.state->stream));
+    HIP_TRY(hipStreamSynchronize(g.state->stream));
+    g.state->d2h_bytes += bytes;
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols, const float *x_dev, size_t seq_len,
+                     float *out_dev) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    if (cols == 0 || cols % qi.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " cols must be divisible by " +
+                                                 std::to_string(qi.elems) + ", got " + std::to_string(cols));
+    if (!w_dev || !x_dev || !out_dev) return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " null device pointer");
+    if ((reinterpret_cast<uintptr_t>(w_dev) | reinterpret_cast<uintptr_t>(x_dev)) & 15u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " device pointers must be 16-byte aligned");
+    if (rows > 0x7fffffffu || seq_len > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " shape out of range");
+    if (rows == 0 || seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    return run_matmul_dev(*g.state, quant, static_cast<const uint8_t *>(w_dev), rows, cols, x_dev, seq_len, out_dev);
+}
+
+int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev, const void *down_dev,
+                                            size_t n_expert, const uint32_t *expert_ids, const float *route_weights,
+                                            const uint32_t *token_ids, size_t n_slots, size_t token_count,
+                                            uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x_dev,
+                                            float *out_dev) {
+    if (n_embd == 0 || n_ff == 0 || n_embd % 256 != 0 || n_ff % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer dims must be divisible by 256, got n_ff=" +
+                                                 std::to_string(n_ff) + " n_embd=" + std::to_string(n_embd));
+    const size_t down_block = down_quant == kQ4K ? kQ4KBytes : kQ6KBytes;
+    if (down_quant != kQ4K && down_quant != kQ6K)
+        return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported Qwen35 HIP down quant code " + std::to_string(down_quant));
+    MoeShape sh;
+    sh.nb_in = n_embd / 256;
+    sh.nb_mid = n_ff / 256;
+    sh.per_gate = n_ff * sh.nb_in * kQ4KBytes;
+    sh.per_down = n_embd * sh.nb_mid * down_block;
+    sh.n_expert = n_expert;
+    MoeShape checked;
+    int st = validate_moe(n_expert * sh.per_gate, n_expert * sh.per_gate, n_expert * sh.per_down, expert_ids, token_ids,
+                          n_slots, token_count, down_quant, n_ff, n_embd, token_count * n_embd, token_count * n_embd,
+                          &checked);
+    if (st != RNB_HIP_OK) return st;
+    if (!gate_dev || !up_dev || !down_dev || !x_dev || !out_dev)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer null device pointer");
+    Guard g;
+    if (!g.state) return g.status;
+    return run_moe_dev(*g.state, static_cast<const uint8_t *>(gate_dev), static_cast<const uint8_t *>(up_dev),
+                       static_cast<const uint8_t *>(down_dev), sh, expert_ids, route_weights, token_ids, n_slots,
+                       token_count, down_quant, n_ff, n_embd, x_dev, out_dev);
+}
+
+}  // extern "C"

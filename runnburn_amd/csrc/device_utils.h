@@ -1,0 +1,75 @@
+// Device-side helpers shared by the gfx950 kernels: wave64 reductions, unaligned vector loads,
+// fp16 decode and the Q4_K 6-bit scale/min unpack.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rnb {
+
+constexpr int kWave = 64;
+
+// GGUF blocks of 210 / 34 bytes are only 2-byte aligned inside a row.  gfx950 global loads
+// accept any alignment (the queue runs in unaligned access mode); the reduced-alignment
+// typedefs keep the compiler from assuming more than is true.
+typedef uint4 __attribute__((aligned(2))) uint4_a2;
+typedef uint2 __attribute__((aligned(2))) uint2_a2;
+typedef uint32_t __attribute__((aligned(2))) uint32_a2;
+
+__device__ __forceinline__ uint4 ld_u4_a2(const uint8_t *p) { return *reinterpret_cast<const uint4_a2 *>(p); }
+__device__ __forceinline__ uint2 ld_u2_a2(const uint8_t *p) { return *reinterpret_cast<const uint2_a2 *>(p); }
+__device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) { return *reinterpret_cast<const uint32_a2 *>(p); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(bits & 0xffffu)));
+}
+__device__ __forceinline__ float ld_f16(const uint8_t *p) {
+    return f16_bits_to_f32(*reinterpret_cast<const unsigned short *>(p));
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
+}
+
+// sum over the 64 lanes of a wave; every lane gets the total
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// sum over aligned groups of `width` lanes (width a power of two <= 64)
+template <int width>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+template <int width>
+__device__ __forceinline__ int group_sum_i(int v) {
+#pragma unroll
+    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// The 12 scale bytes of a Q4_K block as three dwords -> four dwords of packed 6-bit values:
+// sc[0..3], sc[4..7], mn[0..3], mn[4..7] (one byte each).
+struct Q4KScales {
+    uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+};
+__device__ __forceinline__ Q4KScales unpack_q4k_scales(uint32_t u0, uint32_t u1, uint32_t u2) {
+    Q4KScales s;
+    s.sc_lo = u0 & 0x3f3f3f3fu;
+    s.mn_lo = u1 & 0x3f3f3f3fu;
+    s.sc_hi = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
+    s.mn_hi = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
+    return s;
+}
+// byte j (0..7) of an (lo, hi) pair of packed dwords
+__device__ __forceinline__ int byte_of(uint32_t lo, uint32_t hi, int j) {
+    const uint32_t wsel = (j & 4) ? hi : lo;
+    return static_cast<int>((wsel >> ((j & 3) * 8)) & 0xffu);
+}
+
+}  // namespace rnb

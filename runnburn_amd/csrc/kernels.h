@@ -1,0 +1,62 @@
+// Kernel launchers of the gfx950 quantized-matmul backend (internal; the public surface is
+// include/rnb_hip.h).  All launchers only enqueue on `stream`.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace rnb {
+
+constexpr uint32_t kQ8_0 = 8, kQ4K = 12, kQ6K = 14;
+constexpr size_t kQ8_0Bytes = 34, kQ4KBytes = 144, kQ6KBytes = 210;
+
+// Device layout of quantised activations (structure of arrays, one set per call):
+//   Q8_K:  qs    int8  [seq][K]          (16-byte aligned rows, K % 256 == 0)
+//          d     f32   [seq][K/256]
+//          bsums int16 [seq][K/256][16]  (sums of 16 consecutive qs)
+//   Q8:    qs    int8  [seq][K]
+//          d     f32   [seq][K/32]
+struct ActView {
+    const int8_t *qs;
+    const float *d;
+    const int16_t *bsums;  // null for the 32-wide Q8 form
+};
+
+// x: f32, 16-byte aligned, n_blocks*256 values
+void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
+                         hipStream_t stream);
+// x: f32, 16-byte aligned, n_blocks*32 values; n_blocks % 8 == 0 not required
+void launch_quantize_q8(const float *x, size_t n_blocks, int8_t *qs, float *d, hipStream_t stream);
+
+// out[s*rows + row] for s < seq; weights row-major packed blocks, base 16-byte aligned
+void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
+                     uint32_t seq, hipStream_t stream);
+void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
+                     uint32_t seq, hipStream_t stream);
+void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,
+                      uint32_t seq, hipStream_t stream);
+
+// Q4_K x Q8_K GEMM on int8 MFMA; same contract as launch_gemv_q4k, intended for seq >= 16
+void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream);
+
+// ---- gathered sparse-MoE ------------------------------------------------------------------
+struct MoeSlots {
+    const uint32_t *expert;  // [n_slots] device
+    const uint32_t *token;   // [n_slots] device
+    const float *route;      // [n_slots] device
+    uint32_t n_slots;
+};
+// mid[slot][n_ff] = silu(Wg[e] . h_tok) * (Wu[e] . h_tok); act = Q8_K(x) per token
+void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeSlots slots,
+                        float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
+// slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot]))
+void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeSlots slots,
+                     float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
+// out[token][n_embd] = sum of slot_out over the token's slots, in list order;
+// tok_offsets [token_count+1], tok_slots [n_slots] (CSR built by the host)
+void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,
+                       float *out, uint32_t token_count, uint32_t n_embd, hipStream_t stream);
+
+}  // namespace rnb

@@ -1,0 +1,125 @@
+"""No-GPU checks of the C-ABI library: it loads, exports every symbol include/rnb_hip.h declares,
+validates requests with the reference's messages before touching a device, and reports a
+distinguishable NoDevice status so callers can skip (crates/rnb-backend/cuda/src/runtime/tests.rs:22831-22834)."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import runnburn_amd as rnb
+from runnburn_amd import binding
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rnb_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rnb_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 25
+    L = rnb.lib()
+    for name in names:
+        assert hasattr(L, name), f"{name} declared in include/rnb_hip.h but not exported"
+    bound = {s[0] for s in binding.SYMBOLS}
+    assert bound == set(names), (sorted(bound - set(names)), sorted(set(names) - bound))
+
+
+def test_trait_facade():
+    b = rnb.HipBackend()
+    assert b.kind() == "Hip" and b.kind_ordinal() == 6
+    caps = b.capabilities()
+    assert caps == {"MatMul": True, "Attention": False, "Gdn": False, "MoE": True, "Sampler": False}
+    assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q4_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q8_0)
+    assert not b.supports_quant(rnb.OP_MATMUL, 13)  # Q5_K is not on this path
+    with pytest.raises(rnb.BackendError) as ei:
+        b.execute(object())
+    assert ei.value.kind == "UnsupportedOp"
+
+
+def _err(fn, *args):
+    with pytest.raises(rnb.BackendError) as ei:
+        fn(*args)
+    return ei.value
+
+
+def test_matmul_validation_messages_match_reference():
+    """crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:189-206, 352-358, 2289-2307, 1992-2009"""
+    z = np.zeros
+    e = _err(rnb.q4k_gemv, z(144, np.uint8), 1, 255, z(255, np.float32))
+    assert (e.kind, str(e)) == ("InvalidRequest", "Q4_K cols must be divisible by 256, got 255")
+    e = _err(rnb.q4k_gemv, z(143, np.uint8), 1, 256, z(256, np.float32))
+    assert str(e) == "Q4_K weight byte mismatch: got 143, expected 144"
+    e = _err(rnb.q4k_gemv, z(144, np.uint8), 1, 256, z(255, np.float32))
+    assert str(e) == "Q4_K input length mismatch: got 255, expected 256"
+    out = np.zeros(1, np.float32)
+    e = _err(rnb.q4k_gemv_into, z(288, np.uint8), 2, 256, z(256, np.float32), out)
+    assert str(e) == "Q4_K shape mismatch: input=256 output=1 expected input=256 output>=2"
+    e = _err(rnb.q4k_gemv_batch, z(144, np.uint8), 1, 256, z(300, np.float32))
+    assert str(e) == "Q4_K batch input length 300 is not divisible by cols 256"
+    e = _err(rnb.q6k_gemv, z(210, np.uint8), 1, 100, z(100, np.float32))
+    assert str(e) == "Q6_K cols must be divisible by 256, got 100"
+    e = _err(rnb.q6k_gemv, z(200, np.uint8), 1, 256, z(256, np.float32))
+    assert str(e) == "Q6_K weight byte mismatch: got 200, expected 210"
+    e = _err(rnb.q6k_gemv_batch, z(210, np.uint8), 1, 256, z(257, np.float32))
+    assert str(e) == "Q6_K batch input length 257 is not divisible by cols 256"
+    e = _err(rnb.q8_0_gemv, z(34, np.uint8), 1, 31, z(31, np.float32))
+    assert str(e) == "Q8_0 cols must be divisible by 32, got 31"
+    e = _err(rnb.q8_0_gemv, z(35, np.uint8), 1, 32, z(32, np.float32))
+    assert str(e) == "Q8_0 weight byte mismatch: got 35, expected 34"
+    e = _err(rnb.q8_0_gemv, z(34, np.uint8), 1, 32, z(33, np.float32))
+    assert str(e) == "Q8_0 input length mismatch: got 33, expected 32"
+
+
+def test_moe_validation_messages():
+    """crates/rnb-backend/cuda/src/runtime/helpers.rs:1570-1600, 2747-2800"""
+    z = np.zeros
+    n_ff, n_embd = 256, 256
+    per_gate, per_down = n_ff * 144, n_embd * 210
+    g, u, d = z(2 * per_gate, np.uint8), z(2 * per_gate, np.uint8), z(2 * per_down, np.uint8)
+    x = z(n_embd, np.float32)
+    call = rnb.qwen35_sparse_experts_selected_base_by_token
+    e = _err(call, g, u, d, [0], [1.0], [0], 1, 14, n_ff, n_embd, z(10, np.float32))
+    assert str(e) == "Qwen35 full-layer input length mismatch: got 10, expected 256"
+    e = _err(call, g, u, d, [0], [1.0], [0], 1, 14, 100, n_embd, x)
+    assert str(e) == "Qwen35 full-layer dims must be divisible by 256, got n_ff=100 n_embd=256"
+    e = _err(call, g, u, d, [0], [1.0], [1], 1, 14, n_ff, n_embd, x)
+    assert str(e) == "Qwen35 full-layer token id out of range"
+    e = _err(call, g, u, d, [0], [1.0], [0], 1, 13, n_ff, n_embd, x)
+    assert e.kind == "UnsupportedOp" and "down quant code 13" in str(e)
+    e = _err(call, g[:-1], u, d, [0], [1.0], [0], 1, 14, n_ff, n_embd, x)
+    assert str(e).startswith("Qwen35 selected-base gate length is not expert-aligned")
+    e = _err(call, g, u[:per_gate], d, [0], [1.0], [0], 1, 14, n_ff, n_embd, x)
+    assert str(e).startswith("Qwen35 selected-base up length mismatch")
+    e = _err(call, g, u, d, [2], [1.0], [0], 1, 14, n_ff, n_embd, x)
+    assert str(e).startswith("Qwen35 selected-base expert id out of range")
+    e = _err(call, g, u, d, [0, 1], [1.0], [0], 1, 14, n_ff, n_embd, x)
+    assert "length mismatch" in str(e)
+
+
+def test_quantizer_validation():
+    e = _err(rnb.quantize_input_q8k, np.zeros(100, np.float32))
+    assert str(e) == "Q8_K input length must be divisible by 256, got 100"
+    e = _err(rnb.quantize_input_q8, np.zeros(33, np.float32))
+    assert str(e) == "Q8 input length must be divisible by 32, got 33"
+
+
+def test_no_device_is_distinguishable_and_there_is_no_fallback():
+    if rnb.device_available():
+        pytest.skip("a device is present; the NoDevice path is exercised on CPU-only hosts")
+    e = _err(rnb.q4k_gemv, np.zeros(144, np.uint8), 1, 256, np.zeros(256, np.float32))
+    assert e.kind == "NoDevice" and str(e).startswith("no HIP device")
+    assert rnb.stream_handle() == 0
+
+
+def test_product_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "runnburn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower().replace("test oracle", ""), f"{f} mentions the oracle"

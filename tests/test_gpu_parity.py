@@ -1,0 +1,397 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on identical
+seeded inputs.  Activation quantisation must be bit-exact; f32 outputs must satisfy the reference's
+abs-or-rel row check (crates/rnb-backend/cuda/src/runtime/tests.rs:28525-28541) with
+rel = 1e-3 and abs floor = 1e-3 * rms(ref), and are additionally held to 2e-5 * rms against the
+f64-accumulated form of the same integer arithmetic."""
+import numpy as np
+import pytest
+
+from tests import npref
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+REL = 1e-3          # tolerance named by the task: max relative error 1e-3 per row
+TIGHT = 2e-5        # what f32 summation-order differences actually allow, relative to rms
+
+
+def check_close(got, ref, gold=None, label=""):
+    assert np.all(np.isfinite(got)), f"{label}: non-finite output"
+    bad, diff, tol = npref.close_rows(got, ref, rel=REL)
+    assert bad.size == 0, f"{label}: {bad.size} rows outside max(1e-3*rms, 1e-3*|ref|); worst diff {diff.max()}"
+    if gold is not None:
+        g = np.asarray(gold, dtype=np.float64).ravel()
+        rms = float(np.sqrt(np.mean(g * g))) or 1.0
+        worst = float(np.abs(np.asarray(got, dtype=np.float64).ravel() - g).max())
+        assert worst <= TIGHT * rms, f"{label}: |gpu - f64 gold| = {worst} > {TIGHT} * rms ({rms})"
+
+
+def gemv_fn(rnb, quant, batch=False):
+    table = {(Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q6_K, False): rnb.q6k_gemv,
+             (Q6_K, True): rnb.q6k_gemv_batch, (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
+    return table[(quant, batch)]
+
+
+# ---- activation quantisers: bit-exact ---------------------------------------------------------
+
+def _q8k_inputs(oracle):
+    rng = np.random.default_rng(100)
+    cases = {}
+    cases["gauss"] = oracle.fill_normal(512 * 4096 // 8, 1, 1.0)
+    idx = np.arange(16 * 256)
+    cases["ref_batch"] = ((idx * 73 + 19) % 2001).astype(np.float32) - 1000.0  # activation_q8.rs:221-224
+    t = np.zeros(256 * 6, np.float32)
+    t[256] = 127.0
+    t[257:263] = [-0.5, -1.5, -2.5, 0.5, 1.5, 2.5]           # ties, activation_q8.rs:188-193
+    t[512], t[513] = 127.0, -127.0                            # first-max sign rule
+    t[768], t[769] = -127.0, 127.0
+    t[1024 + 15], t[1024 + 16], t[1024 + 255] = -1.0, -2.0, 127.0  # bsums boundaries
+    t[1280 + 200] = -3.0e-39                                  # subnormal-only block
+    cases["reference_vectors"] = t
+    tie = np.zeros(256, np.float32)
+    tie[[7, 100, 255]] = [-2.0, 2.0, 2.0]                     # equal |x|: the first (negative) one must win
+    cases["first_of_equal_magnitudes"] = tie
+    cases["tiny_and_huge"] = np.concatenate([rng.standard_normal(256).astype(np.float32) * np.float32(1e-30),
+                                             rng.standard_normal(256).astype(np.float32) * np.float32(1e30)])
+    cases["half_integers"] = (rng.integers(-254, 255, 2048).astype(np.float32) * np.float32(0.5))
+    return cases
+
+
+def test_q8k_activation_quantiser_bit_exact(rnb, oracle):
+    for name, x in _q8k_inputs(oracle).items():
+        got = rnb.quantize_input_q8k(x)
+        want = oracle.quantize_q8k(x)
+        assert np.array_equal(got["d"].view(np.uint32), want["d"].view(np.uint32)), name
+        assert np.array_equal(got["qs"], want["qs"]), name
+        assert np.array_equal(got["bsums"], want["bsums"]), name
+    b = rnb.quantize_input_q8k(_q8k_inputs(oracle)["reference_vectors"])
+    assert b["d"][1] == -1.0 and b["qs"][1][1:7].tolist() == [0, 2, 2, 0, -2, -2]
+    assert b["qs"][2][:2].tolist() == [-127, 127] and b["d"][3] == 1.0
+    assert b["bsums"][4][0] == 1 and b["bsums"][4][1] == 2 and b["bsums"][4][15] == -127
+
+
+def test_q8_activation_quantiser_bit_exact(rnb, oracle):
+    rng = np.random.default_rng(101)
+    xs = [oracle.fill_normal(4096, 2, 1.0), np.zeros(64, np.float32),
+          rng.integers(-254, 255, 32 * 9).astype(np.float32) * np.float32(0.5),   # 9 blocks: ragged last wave
+          rng.standard_normal(32 * 64 * 5 + 32).astype(np.float32) * np.float32(1e-20)]
+    for x in xs:
+        got, want = rnb.quantize_input_q8(x), oracle.quantize_q8(x)
+        assert np.array_equal(got["d"].view(np.uint32), want["d"].view(np.uint32))
+        assert np.array_equal(got["qs"], want["qs"])
+
+
+# ---- the reference's known-answer vectors through the device ------------------------------------
+
+def test_reference_closed_forms_on_device(rnb):
+    """crates/rnb-cpu/src/gemm/tile_q4k.rs:2019-2151 (0 / 0 / 2560 per row) and
+    crates/rnb-cpu/src/gemm/quant_gemv.rs:1448-1464 (528, seq-major)."""
+    rows = 8
+    sc = np.zeros(8, np.int64)
+    sc[0] = 10
+    nib = np.full(256, 8)
+    blk = npref.make_q4k_block(1.0, 0.0, sc, np.zeros(8), nib)
+    w = np.tile(blk, rows)
+    x = np.zeros(256, np.float32)
+    x[:32] = 1.0  # Q8_K: d = -1/127, q = -127 -> d*q = 1 exactly per element
+    out = rnb.q4k_gemv(w, rows, 256, x)
+    assert np.allclose(out, 2560.0, rtol=1e-6)
+    assert np.all(rnb.q4k_gemv(w, rows, 256, np.zeros(256, np.float32)) == 0.0)
+    w0 = np.tile(npref.make_q4k_block(1.0, 1.0, np.zeros(8), np.zeros(8), nib), rows)
+    assert np.all(rnb.q4k_gemv(w0, rows, 256, x) == 0.0)
+
+    ref_bytes = np.frombuffer(bytes([0x00, 0x3C] + list(range(1, 33)) + [0x00, 0x3C] + list(range(32, 0, -1))),
+                              dtype=np.uint8)
+    out = rnb.q8_0_gemv_batch(ref_bytes, 2, 32, np.ones(64, np.float32))
+    assert out.shape == (2, 2) and np.allclose(out, 528.0, rtol=1e-6)
+    w2 = np.concatenate([npref.make_q8_0_block(1.0, np.ones(32)), npref.make_q8_0_block(1.0, 3 * np.ones(32))])
+    x2 = np.concatenate([np.ones(32, np.float32), 2 * np.ones(32, np.float32)])
+    assert np.allclose(rnb.q8_0_gemv_batch(w2, 2, 32, x2).ravel(), [32.0, 96.0, 64.0, 192.0], rtol=1e-6)
+
+
+# ---- GEMV: shapes around every edge of the lane mapping ------------------------------------------
+
+@pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("rows,nblk", [(1, 1), (3, 2), (4, 3), (5, 5), (7, 8), (9, 9), (64, 16), (33, 17), (6, 56)])
+def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
+    cols = nblk * 256
+    w = oracle.make_weights(quant, rows, cols, 1000 + rows * 31 + nblk)
+    x = oracle.fill_normal(cols, 2000 + rows + nblk, 1.0)
+    got = gemv_fn(rnb, quant)(w, rows, cols, x)
+    ref = oracle.gemv(quant, w, rows, cols, x)[0]
+    gold = oracle.gemv(quant, w, rows, cols, x, gold=True)[0]
+    check_close(got, ref, gold, f"quant {quant} rows {rows} nblk {nblk}")
+
+
+@pytest.mark.parametrize("quant,cols", [(Q8_0, 32), (Q8_0, 96), (Q8_0, 32 * 65), (Q8_0, 32 * 129)])
+def test_q8_0_gemv_block_counts_off_the_wave_size(rnb, oracle, quant, cols):
+    rows = 6
+    w = oracle.make_weights(quant, rows, cols, 3000 + cols)
+    x = oracle.fill_normal(cols, 3001 + cols, 1.0)
+    check_close(rnb.q8_0_gemv(w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x)[0],
+                oracle.gemv(quant, w, rows, cols, x, gold=True)[0], f"q8_0 cols {cols}")
+
+
+def test_gemv_extreme_blocks(rnb, oracle):
+    """all-max nibbles, negative Q6_K scales, zero / subnormal f16 scales, a zero activation block"""
+    rng = np.random.default_rng(7)
+    nblk, rows = 4, 8
+    x = oracle.fill_normal(nblk * 256, 11, 1.0)
+    x[256:512] = 0.0
+    blocks = []
+    for r in range(rows):
+        for b in range(nblk):
+            d = [1.0, 0.0, 6e-8, 2.0 ** -14][(r + b) % 4]
+            blocks.append(npref.make_q4k_block(d, [0.5, 6e-8, 0.0, 1.0][(r + b) % 4], np.full(8, 63), np.full(8, 63),
+                                               np.full(256, 15) if b % 2 == 0 else rng.integers(0, 16, 256)))
+    w = np.concatenate(blocks)
+    check_close(rnb.q4k_gemv(w, rows, nblk * 256, x), oracle.gemv(Q4_K, w, rows, nblk * 256, x)[0],
+                oracle.gemv(Q4_K, w, rows, nblk * 256, x, gold=True)[0], "q4k extremes")
+    blocks = []
+    for r in range(rows):
+        for b in range(nblk):
+            d = [1.0, -0.5, 6e-8, 0.0][(r + b) % 4]
+            scales = np.full(16, -128) if b == 0 else rng.integers(-128, 128, 16)
+            q = np.full(256, 63) if b == 1 else (np.zeros(256) if b == 2 else rng.integers(0, 64, 256))
+            blocks.append(npref.make_q6k_block(d, scales, q))
+    w = np.concatenate(blocks)
+    check_close(rnb.q6k_gemv(w, rows, nblk * 256, x), oracle.gemv(Q6_K, w, rows, nblk * 256, x)[0],
+                oracle.gemv(Q6_K, w, rows, nblk * 256, x, gold=True)[0], "q6k extremes")
+    w = np.concatenate([npref.make_q8_0_block([1.0, 0.0, 6e-8, -2.0][i % 4],
+                                              np.full(32, -128) if i % 3 == 0 else rng.integers(-128, 128, 32))
+                        for i in range(rows * 32)])
+    check_close(rnb.q8_0_gemv(w, rows, 1024, x), oracle.gemv(Q8_0, w, rows, 1024, x)[0],
+                oracle.gemv(Q8_0, w, rows, 1024, x, gold=True)[0], "q8_0 extremes")
+
+
+def test_unaligned_host_weights_and_subrange_residency(rnb, oracle):
+    """Rows at odd host byte offsets must give identical results (crates/rnb-cpu/src/gemm/quant_gemv.rs:1257-1296);
+    a sub-range of a resident parent resolves to parent + offset (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:722-741)."""
+    rows, cols = 16, 1024
+    for quant in (Q4_K, Q6_K, Q8_0):
+        w = oracle.make_weights(quant, rows, cols, 42 + quant)
+        x = oracle.fill_normal(cols, 43, 1.0)
+        base = gemv_fn(rnb, quant)(w, rows, cols, x)
+        buf = np.zeros(w.size + 3, np.uint8)
+        buf[1:1 + w.size] = w
+        shifted = buf[1:1 + w.size]
+        assert shifted.ctypes.data % 2 == 1
+        assert np.array_equal(gemv_fn(rnb, quant)(shifted, rows, cols, x), base)
+        rnb.release(shifted)
+        # parent resident, call with the second half of the rows
+        rnb.prewarm([w])
+        before = rnb.transfer_counters()[0]
+        half = w[w.size // 2:]
+        got = gemv_fn(rnb, quant)(half, rows // 2, cols, x)
+        after = rnb.transfer_counters()[0]
+        assert np.array_equal(got, base[rows // 2:])
+        assert after - before == cols * 4, "the sub-range must not be uploaded again"
+        rnb.release(w)
+
+
+def test_resident_cache_notices_changed_bytes(rnb, oracle):
+    rows, cols = 8, 512
+    w = oracle.make_weights(Q4_K, rows, cols, 5).copy()
+    x = oracle.fill_normal(cols, 6, 1.0)
+    a = rnb.q4k_gemv(w, rows, cols, x)
+    w[:] = oracle.make_weights(Q4_K, rows, cols, 6)
+    b = rnb.q4k_gemv(w, rows, cols, x)
+    check_close(b, oracle.gemv(Q4_K, w, rows, cols, x)[0], None, "changed bytes at the same address")
+    assert not np.array_equal(a, b)
+    rnb.release(w)
+
+
+def test_unpinned_resident_never_serves_a_subrange(rnb, oracle):
+    """Host memory of an unpinned resident may be freed and reused: a later, smaller weight tensor that lands
+    inside the old address range must be uploaded, not resolved against the stale device copy."""
+    rows, cols = 16, 512
+    rb = cols // 256 * 144
+    buf = np.zeros(rows * rb, np.uint8)
+    buf[:] = oracle.make_weights(Q4_K, rows, cols, 31)
+    x = oracle.fill_normal(cols, 32, 1.0)
+    rnb.q4k_gemv(buf, rows, cols, x)                      # unpinned resident covering all of buf
+    buf[:] = oracle.make_weights(Q4_K, rows, cols, 33)    # "freed and reused"
+    inner = buf[4 * rb:12 * rb]
+    got = rnb.q4k_gemv(inner, 8, cols, x)
+    check_close(got, oracle.gemv(Q4_K, inner, 8, cols, x)[0], None, "sub-range of a stale unpinned resident")
+    rnb.release(inner)
+    rnb.q4k_gemv(buf, rows, cols, x)
+    rnb.release(buf)
+
+
+def test_gemv_into_and_zero_sized(rnb, oracle):
+    rows, cols = 5, 512
+    w = oracle.make_weights(Q6_K, rows, cols, 8)
+    x = oracle.fill_normal(cols, 9, 1.0)
+    out = np.full(rows + 3, -7.0, np.float32)
+    rnb.q6k_gemv_into(w, rows, cols, x, out)
+    assert np.array_equal(out[:rows], rnb.q6k_gemv(w, rows, cols, x)) and np.all(out[rows:] == -7.0)
+    assert rnb.q4k_gemv(np.zeros(0, np.uint8), 0, 256, np.zeros(256, np.float32)).size == 0
+    assert rnb.q4k_gemv_batch(np.zeros(144, np.uint8), 1, 256, np.zeros(0, np.float32)).shape == (0, 1)
+
+
+# ---- batches: seq-major layout, ragged token counts ----------------------------------------------
+
+@pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("seq", [2, 3, 15])
+def test_gemv_batch_small(rnb, oracle, quant, seq):
+    rows, cols = 37, 768
+    w = oracle.make_weights(quant, rows, cols, 50 + quant)
+    x = oracle.fill_normal(seq * cols, 60 + seq, 1.0)
+    got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+    assert got.shape == (seq, rows)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"batch quant {quant} seq {seq}")
+
+
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33),
+                                           (1, 1, 16), (257, 5, 40)])
+def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
+    cols = nblk * 256
+    w = oracle.make_weights(Q4_K, rows, cols, 70 + rows)
+    x = oracle.fill_normal(seq * cols, 80 + seq, 1.0)
+    got = rnb.q4k_gemv_batch(w, rows, cols, x)
+    check_close(got, oracle.gemv(Q4_K, w, rows, cols, x), oracle.gemv(Q4_K, w, rows, cols, x, gold=True),
+                f"gemm rows {rows} nblk {nblk} seq {seq}")
+
+
+def test_q4k_gemm_extreme_blocks(rnb, oracle):
+    rng = np.random.default_rng(17)
+    rows, nblk, seq = 40, 3, 24
+    blocks = [npref.make_q4k_block([1.0, 0.0, 6e-8, 2.0 ** -14][i % 4], [0.5, 1.0, 0.0, 6e-8][i % 4],
+                                   np.full(8, 63) if i % 2 else rng.integers(0, 64, 8), rng.integers(0, 64, 8),
+                                   np.full(256, 15) if i % 3 == 0 else rng.integers(0, 16, 256))
+              for i in range(rows * nblk)]
+    w = np.concatenate(blocks)
+    x = oracle.fill_normal(seq * nblk * 256, 18, 1.0).reshape(seq, -1)
+    x[3, 256:512] = 0.0
+    x[5] = 0.0
+    got = rnb.q4k_gemv_batch(w, rows, nblk * 256, x)
+    assert np.all(got[5] == 0.0)
+    check_close(got, oracle.gemv(Q4_K, w, rows, nblk * 256, x), oracle.gemv(Q4_K, w, rows, nblk * 256, x, gold=True),
+                "gemm extremes")
+
+
+# ---- the BASELINE configurations at full size ------------------------------------------------------
+
+def _full_gemv(rnb, oracle, quant, rows, cols, name):
+    w = oracle.make_weights(quant, rows, cols, oracle.tensor_seed(name, "weight"))
+    x = oracle.fill_normal(cols, oracle.tensor_seed(name, "x"), 1.0)
+    got = gemv_fn(rnb, quant)(w, rows, cols, x)
+    ref = oracle.gemv(quant, w, rows, cols, x)[0]
+    gold = oracle.gemv(quant, w, rows, cols, x, gold=True)[0]
+    check_close(got, ref, gold, name)
+    # size-independent properties: x -> 2x doubles every output bit-for-bit (power-of-two scaling commutes
+    # with the activation quantiser), x = 0 gives exact zeros, and reversing the row order reverses the output
+    assert np.array_equal(gemv_fn(rnb, quant)(w, rows, cols, 2.0 * x), 2.0 * got)
+    assert np.all(gemv_fn(rnb, quant)(w, rows, cols, np.zeros(cols, np.float32)) == 0.0)
+    rb = w.size // rows
+    w_rev = np.ascontiguousarray(w.reshape(rows, rb)[::-1]).reshape(-1)
+    assert np.array_equal(gemv_fn(rnb, quant)(w_rev, rows, cols, x), got[::-1])
+    rnb.release(w_rev)
+    rnb.release(w)
+
+
+def test_config1_q8_0_gemv_4096x4096(rnb, oracle):
+    _full_gemv(rnb, oracle, Q8_0, 4096, 4096, "cfg1")
+
+
+def test_config2_q4k_gemv_14336x4096(rnb, oracle):
+    _full_gemv(rnb, oracle, Q4_K, 14336, 4096, "cfg2")
+
+
+def test_config3a_q6k_gemv_4096x14336(rnb, oracle):
+    _full_gemv(rnb, oracle, Q6_K, 4096, 14336, "cfg3a")
+
+
+def test_config3b_q6k_gemv_lm_head_128256x4096(rnb, oracle):
+    _full_gemv(rnb, oracle, Q6_K, 128256, 4096, "cfg3b")
+
+
+def test_config4_q4k_gemm_512x4096_to_14336(rnb, oracle):
+    rows, cols, seq = 14336, 4096, 512
+    w = oracle.make_weights(Q4_K, rows, cols, oracle.tensor_seed("cfg2", "weight"))
+    x = oracle.fill_normal(seq * cols, oracle.tensor_seed("cfg4", "x"), 1.0)
+    got = rnb.q4k_gemv_batch(w, rows, cols, x)
+    assert got.shape == (seq, rows)
+    rb = cols // 256 * 144
+    # oracle on three row bands (first, an interior band straddling tile edges, last): all 512 tokens each
+    for lo, hi in ((0, 160), (7001, 7161), (rows - 160, rows)):
+        ws = w[lo * rb:hi * rb]
+        ref = oracle.gemv(Q4_K, ws, hi - lo, cols, x)
+        gold = oracle.gemv(Q4_K, ws, hi - lo, cols, x, gold=True)
+        check_close(got[:, lo:hi], ref, gold, f"cfg4 rows {lo}:{hi}")
+    # every row for a spread of tokens: the GEMM must agree with the decode GEMV path on the same x
+    for s in (0, 31, 32, 255, 511):
+        one = rnb.q4k_gemv(w, rows, cols, x[s * cols:(s + 1) * cols])
+        check_close(got[s], one, None, f"cfg4 token {s} vs GEMV")
+    # property: a token's result does not depend on its neighbours (permute tokens -> permuted output, bitwise)
+    perm = np.random.default_rng(3).permutation(seq)
+    got_p = rnb.q4k_gemv_batch(w, rows, cols, x.reshape(seq, cols)[perm])
+    assert np.array_equal(got_p, got[perm])
+    rnb.release(w)
+
+
+# ---- sparse MoE ----------------------------------------------------------------------------------
+
+def _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, seed, down_quant=Q6_K):
+    gate = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, oracle.tensor_seed(f"moe{seed}", "gate"))
+    up = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, oracle.tensor_seed(f"moe{seed}", "up"))
+    down = oracle.make_weights(down_quant, n_expert * n_embd, n_ff, oracle.tensor_seed(f"moe{seed}", "down"))
+    x = oracle.fill_normal(tokens * n_embd, oracle.tensor_seed(f"moe{seed}", "x"), 1.0)
+    logits = oracle.fill_normal(tokens * n_expert, oracle.tensor_seed(f"moe{seed}", "logits"), 1.0)
+    eids, route, tids = [], [], []
+    for t in range(tokens):
+        idx, wts = oracle.route_topk(logits[t * n_expert:(t + 1) * n_expert], k)
+        eids += idx.tolist()
+        route += wts.tolist()
+        tids += [t] * len(idx)
+    return gate, up, down, x, np.array(eids, np.uint32), np.array(route, np.float32), np.array(tids, np.uint32)
+
+
+@pytest.mark.parametrize("tokens,down_quant", [(1, Q6_K), (3, Q6_K), (2, Q4_K)])
+def test_moe_small(rnb, oracle, tokens, down_quant):
+    n_expert, n_ff, n_embd, k = 8, 512, 768, 3
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 1, down_quant)
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"moe tokens {tokens}")
+    for w in (gate, up, down):
+        rnb.release(w)
+
+
+def test_moe_unrouted_token_and_empty_slot_list(rnb, oracle):
+    n_expert, n_ff, n_embd = 4, 256, 256
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, 3, 2, 2)
+    keep = t != 1  # token 1 gets no expert: its row must be exactly zero
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e[keep], r[keep], t[keep], 3, Q6_K, n_ff,
+                                                           n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e[keep], r[keep], t[keep], 3, Q6_K, n_ff,
+                                             n_embd, x)
+    assert np.all(got[1] == 0.0)
+    check_close(got, ref, None, "moe with an unrouted token")
+    none = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e[:0], r[:0], t[:0], 3, Q6_K, n_ff, n_embd, x)
+    assert none.shape == (3, n_embd) and np.all(none == 0.0)
+    for w in (gate, up, down):
+        rnb.release(w)
+
+
+@pytest.mark.parametrize("tokens", [1, 64])
+def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
+    n_expert, n_ff, n_embd, k = 128, 768, 2048, 8
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 5)
+    # callers hand prefill slots sorted by (expert, token) (crates/rnb-llm/.../shared_expert_moe/prefill.rs:1410-1458)
+    if tokens > 1:
+        order = np.lexsort((t, e))
+        e, r, t = e[order], r[order], t[order]
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
+    check_close(got, ref, None, f"cfg5 tokens {tokens}")
+    if tokens > 1:
+        # a (token, expert) result does not depend on batching: token 7 alone == row 7 of the batch
+        sel = t == 7
+        solo = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e[sel], r[sel], np.zeros(sel.sum(), np.uint32),
+                                                                1, Q6_K, n_ff, n_embd, x[7 * n_embd:8 * n_embd])
+        assert np.array_equal(solo[0], got[7])
+    for w in (gate, up, down):
+        rnb.release(w)
