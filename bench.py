@@ -1,0 +1,440 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline (BASELINE.json metric, configs[1]): Q4_K decode GEMV, weights 14336 x 4096 (Llama-3-8B FFN
+up/gate), one token.  A step = one pass of the path over one batch of synthetic input, inputs
+already resident in HBM: device-side Q8_K quantisation of the activation + the GEMV kernel.
+Steps rotate over enough distinct weight copies to exceed the 256 MiB Infinity Cache, so the
+weights of every step come from HBM.
+
+Prints ONE JSON line on stdout (progress goes to stderr):
+  value      whole-job GB/s = algorithmic bytes per step * K / wall time of K steps
+  roofline   the GEMV kernel alone: algorithmic bytes per launch / mean kernel duration measured with
+             HIP events on the library's stream, against the 8 TB/s HBM peak
+  cpu_baseline  the CPU restatement of rnb-cpu's x86 path (oracle/, AVX2+FMA, row-chunk threads) timed on
+             the host cores on the same workload
+  secondary  the other BASELINE configs (kernel-level, same protocol), Q4_K prefill GEMM in TOP/s
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA, POP/s -> TOP/s
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
+MALL_BYTES = 256 << 20
+
+
+def log(msg: str) -> None:
+    print(msg, file=sys.stderr, flush=True)
+
+
+# ---- synthetic weights: fp32 N(0, 0.02) fitted to valid GGUF blocks with numpy -------------------
+# (block layouts are the real ones; the fit is a plain vectorised min/max fit -- the kernels' speed
+# does not depend on the values)
+
+def _f16_bytes(a: np.ndarray) -> np.ndarray:
+    return a.astype(np.float16).view(np.uint8).reshape(*a.shape, 2)
+
+
+def synth_q8_0(rng, rows, cols):
+    x = rng.standard_normal((rows, cols // 32, 32), dtype=np.float32) * np.float32(0.02)
+    d = (np.abs(x).max(axis=2) / 127.0).astype(np.float16)
+    df = np.maximum(d.astype(np.float32), 1e-12)
+    q = np.clip(np.rint(x / df[..., None]), -127, 127).astype(np.int8)
+    out = np.empty((rows, cols // 32, 34), np.uint8)
+    out[..., 0:2] = d.view(np.uint8).reshape(rows, cols // 32, 2)
+    out[..., 2:] = q.view(np.uint8)
+    return out.reshape(-1)
+
+
+def synth_q4_k(rng, rows, cols):
+    nb = cols // 256
+    x = rng.standard_normal((rows, nb, 8, 32), dtype=np.float32) * np.float32(0.02)
+    lo = np.minimum(x.min(axis=3), 0.0)
+    hi = x.max(axis=3)
+    scale = (hi - lo) / 15.0
+    mins = -lo
+    d = (scale.max(axis=2) / 63.0).astype(np.float16)
+    dmin = (mins.max(axis=2) / 63.0).astype(np.float16)
+    df = np.maximum(d.astype(np.float32), 1e-12)[..., None]
+    dmf = np.maximum(dmin.astype(np.float32), 1e-12)[..., None]
+    sc = np.clip(np.rint(scale / df), 0, 63).astype(np.uint8)
+    mn = np.clip(np.rint(mins / dmf), 0, 63).astype(np.uint8)
+    step = np.maximum(df * sc, 1e-12)[..., None]
+    q = np.clip(np.rint((x + (dmf * mn)[..., None]) / step), 0, 15).astype(np.uint8)
+    out = np.empty((rows, nb, 144), np.uint8)
+    out[..., 0:2] = d.view(np.uint8).reshape(rows, nb, 2)
+    out[..., 2:4] = dmin.view(np.uint8).reshape(rows, nb, 2)
+    out[..., 4:8] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
+    out[..., 8:12] = (mn[..., 0:4] & 63) | ((mn[..., 4:8] >> 4) << 6)
+    out[..., 12:16] = (sc[..., 4:8] & 15) | ((mn[..., 4:8] & 15) << 4)
+    qg = q.reshape(rows, nb, 4, 2, 32)
+    out[..., 16:] = (qg[:, :, :, 0, :] | (qg[:, :, :, 1, :] << 4)).reshape(rows, nb, 128)
+    return out.reshape(-1)
+
+
+def synth_q6_k(rng, rows, cols):
+    nb = cols // 256
+    x = rng.standard_normal((rows, nb, 16, 16), dtype=np.float32) * np.float32(0.02)
+    scale = np.abs(x).max(axis=3) / 31.0
+    d = (scale.max(axis=2) / 127.0).astype(np.float16)
+    df = np.maximum(d.astype(np.float32), 1e-12)[..., None]
+    sc = np.clip(np.rint(scale / df), 1, 127).astype(np.int8)
+    q = (np.clip(np.rint(x / (df * sc)[..., None]), -32, 31) + 32).astype(np.uint8)
+    q = q.reshape(rows, nb, 2, 4, 32)  # half, quarter, l
+    out = np.empty((rows, nb, 210), np.uint8)
+    ql = np.empty((rows, nb, 2, 64), np.uint8)
+    ql[..., 0:32] = (q[:, :, :, 0] & 15) | ((q[:, :, :, 2] & 15) << 4)
+    ql[..., 32:64] = (q[:, :, :, 1] & 15) | ((q[:, :, :, 3] & 15) << 4)
+    qh = (q[:, :, :, 0] >> 4) | ((q[:, :, :, 1] >> 4) << 2) | ((q[:, :, :, 2] >> 4) << 4) | ((q[:, :, :, 3] >> 4) << 6)
+    out[..., 0:128] = ql.reshape(rows, nb, 128)
+    out[..., 128:192] = qh.reshape(rows, nb, 64)
+    out[..., 192:208] = sc.view(np.uint8)
+    out[..., 208:210] = d.view(np.uint8).reshape(rows, nb, 2)
+    return out.reshape(-1)
+
+
+SYNTH = {Q8_0: synth_q8_0, Q4_K: synth_q4_k, Q6_K: synth_q6_k}
+
+
+def synth_weights(quant, rows, cols, seed, distinct_rows=16384):
+    """rows x cols packed weights; beyond `distinct_rows` the generated rows repeat (addresses differ, so
+    cache behaviour is that of fully distinct data)."""
+    rng = np.random.default_rng(seed)
+    gen = min(rows, distinct_rows)
+    parts = [SYNTH[quant](rng, min(4096, gen - r0), cols) for r0 in range(0, gen, 4096)]
+    base = np.concatenate(parts)
+    if gen == rows:
+        return base
+    reps = -(-rows // gen)
+    rb = cols // BLOCK_ELEMS[quant] * BLOCK_BYTES[quant]
+    return np.tile(base, reps)[:rows * rb].copy()
+
+
+# ---- HIP events on the library stream (ctypes on the runtime the library already loaded) ----------
+
+class Hip:
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.rt.hipEventDestroy.argtypes = [C.c_void_p]
+        self.rt.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        self.rt.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        self.rt.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        self.rt.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        self.rt.hipGraphDestroy.argtypes = [C.c_void_p]
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with hipError {rc}")
+
+    def event(self):
+        ev = C.c_void_p()
+        self.check(self.rt.hipEventCreate(C.byref(ev)), "hipEventCreate")
+        return ev
+
+    def record(self, ev, stream):
+        self.check(self.rt.hipEventRecord(ev, stream), "hipEventRecord")
+
+    def elapsed_ms(self, a, b):
+        self.check(self.rt.hipEventSynchronize(b), "hipEventSynchronize")
+        ms = C.c_float()
+        self.check(self.rt.hipEventElapsedTime(C.byref(ms), a, b), "hipEventElapsedTime")
+        return float(ms.value)
+
+
+def kernel_times_ms(hip, stream, launch, n, pre=None):
+    """Mean/median duration of `launch(i)` over n launches: one event pair per launch on the stream the
+    kernel runs on.  `pre(i)` is enqueued before the start event (e.g. the activation quantiser)."""
+    starts = [hip.event() for _ in range(n)]
+    stops = [hip.event() for _ in range(n)]
+    for i in range(n):
+        if pre is not None:
+            pre(i)
+        hip.record(starts[i], stream)
+        launch(i)
+        hip.record(stops[i], stream)
+    t = np.array([hip.elapsed_ms(starts[i], stops[i]) for i in range(n)])
+    for ev in starts + stops:
+        hip.rt.hipEventDestroy(ev)
+    return t
+
+
+def wall_steps(rnb, step, n):
+    rnb.sync()
+    t0 = time.perf_counter()
+    for i in range(n):
+        step(i)
+    rnb.sync()
+    return (time.perf_counter() - t0) * 1e3
+
+
+def graph_steps(hip, rnb, stream, step, per_graph, n_graphs):
+    """Capture `per_graph` steps into one HIP graph and replay it `n_graphs` times; returns wall ms."""
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.check(hip.rt.hipStreamBeginCapture(stream, 2), "hipStreamBeginCapture")  # 2 = relaxed
+    try:
+        for i in range(per_graph):
+            step(i)
+    finally:
+        rc = hip.rt.hipStreamEndCapture(stream, C.byref(graph))
+    hip.check(rc, "hipStreamEndCapture")
+    hip.check(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0), "hipGraphInstantiate")
+    for _ in range(3):
+        hip.check(hip.rt.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+    rnb.sync()
+    t0 = time.perf_counter()
+    for _ in range(n_graphs):
+        hip.rt.hipGraphLaunch(gexec, stream)
+    rnb.sync()
+    ms = (time.perf_counter() - t0) * 1e3
+    hip.rt.hipGraphExecDestroy(gexec)
+    hip.rt.hipGraphDestroy(graph)
+    return ms
+
+
+# ---- algorithmic bytes (weights once + quantised activations once + f32 outputs once) --------------
+
+def gemv_bytes(quant, rows, cols, seq=1):
+    w = rows * (cols // BLOCK_ELEMS[quant]) * BLOCK_BYTES[quant]
+    act = seq * (cols // 32 * 36 if quant == Q8_0 else cols // 256 * 292)
+    return w + act + seq * rows * 4
+
+
+def copies_for(nbytes):
+    return max(2, -(-2 * MALL_BYTES // nbytes))
+
+
+def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, name, want_graph=True):
+    w_host = synth_weights(quant, rows, cols, seed)
+    n_copies = copies_for(w_host.nbytes)
+    log(f"[{name}] weights {w_host.nbytes / 1e6:.1f} MB x {n_copies} device copies")
+    w_dev = [rnb.DeviceBuffer.from_host(w_host) for _ in range(n_copies)]
+    x = (np.random.default_rng(seed + 1).standard_normal(seq * cols)).astype(np.float32)
+    x_dev = rnb.DeviceBuffer.from_host(x)
+    out_dev = rnb.DeviceBuffer(seq * rows * 4)
+
+    def step(i):
+        rnb.gemv_dev(quant, w_dev[i % n_copies], rows, cols, x_dev, seq, out_dev)
+
+    for i in range(warmup):
+        step(i)
+    wall_ms = wall_steps(rnb, step, steps)
+    res = {"wall_ms_per_step": wall_ms / steps, "launch": "stream"}
+    if want_graph:
+        try:
+            per = n_copies if steps >= n_copies else steps
+            reps = max(1, steps // per)
+            g_ms = graph_steps(hip, rnb, stream, step, per, reps)
+            res["graph_ms_per_step"] = g_ms / (per * reps)
+        except Exception as exc:  # keep the stream number if capture is unavailable
+            log(f"[{name}] graph replay unavailable: {exc}")
+    rnb.quantize_dev(quant, x_dev, seq, cols)
+    t = kernel_times_ms(hip, stream, lambda i: rnb.gemv_quantized_dev(quant, w_dev[i % n_copies], rows, cols, seq, out_dev),
+                        min(steps, 1000))
+    res["kernel_ms_mean"] = float(t.mean())
+    res["kernel_ms_median"] = float(np.median(t))
+    res["kernel_ms_p10"] = float(np.percentile(t, 10))
+    res["kernel_ms_p90"] = float(np.percentile(t, 90))
+    # cache-resident variant (one copy, weights may stay in the 256 MiB Infinity Cache): labelled, never `value`
+    t1 = kernel_times_ms(hip, stream, lambda i: rnb.gemv_quantized_dev(quant, w_dev[0], rows, cols, seq, out_dev),
+                         min(steps, 300))
+    res["kernel_ms_mean_cache_resident"] = float(t1.mean())
+    res["bytes"] = gemv_bytes(quant, rows, cols, seq)
+    res["copies"] = n_copies
+    out = out_dev.to_host(np.float32)
+    for b in w_dev:
+        b.free()
+    x_dev.free()
+    out_dev.free()
+    return res, w_host, x, out
+
+
+def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=8.0):
+    """The CPU leg: rnb-cpu's x86 path restated in oracle/ (AVX2+FMA dots, contiguous row chunks per
+    thread), timed on this host; also checks the GPU result against it (abs-or-rel 1e-3)."""
+    from oracle import oracle as ora
+
+    ora.lib()
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = min(threads, os.cpu_count() or threads)
+    fn = (lambda: ora.gemv(quant, w_host, rows, cols, x, avx2=True, n_threads=threads)) if ora.have_avx2() else \
+        (lambda: ora.gemv(quant, w_host, rows, cols, x, n_threads=threads))
+    ref = fn()
+    for _ in range(2):
+        fn()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 200 and time.perf_counter() - t_start < budget_s:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    e = np.asarray(ref, np.float64).ravel()
+    g = np.asarray(gpu_out, np.float64).ravel()
+    tol = np.maximum(1e-3 * np.sqrt(np.mean(e * e)), 1e-3 * np.abs(e))
+    ok = bool(np.all(np.abs(g - e) <= tol))
+    return {"value": gemv_bytes(quant, rows, cols, x.size // cols) / med / 1e9, "unit": "GB/s", "cores": threads,
+            "kind": "port", "sample": f"{len(times)} full passes of the same {rows}x{cols} GEMV, median",
+            "ms": med * 1e3, "isa": "avx2+fma" if ora.have_avx2() else "scalar", "gpu_matches_cpu": ok}
+
+
+def bench_moe(rnb, hip, stream, tokens, steps, seed):
+    n_expert, n_ff, n_embd, k = 128, 768, 2048, 8
+    gen = 16  # distinct experts generated; tiled to 128 (addresses differ)
+    per_gate = n_ff * (n_embd // 256) * 144
+    per_down = n_embd * (n_ff // 256) * 210
+    g = np.tile(synth_weights(Q4_K, gen * n_ff, n_embd, seed), n_expert // gen)
+    u = np.tile(synth_weights(Q4_K, gen * n_ff, n_embd, seed + 1), n_expert // gen)
+    d = np.tile(synth_weights(Q6_K, gen * n_embd, n_ff, seed + 2), n_expert // gen)
+    gd, ud, dd = (rnb.DeviceBuffer.from_host(a) for a in (g, u, d))
+    rng = np.random.default_rng(seed + 3)
+    x_dev = rnb.DeviceBuffer.from_host(rng.standard_normal(tokens * n_embd).astype(np.float32))
+    out_dev = rnb.DeviceBuffer(tokens * n_embd * 4)
+    routes = []
+    for it in range(8):  # the route changes per iteration, so 392 MB of experts are cycled through
+        logits = rng.standard_normal((tokens, n_expert)).astype(np.float32)
+        idx = np.argsort(-logits, axis=1, kind="stable")[:, :k]
+        sel = np.take_along_axis(logits, idx, axis=1)
+        wts = np.exp(sel - sel[:, :1])
+        wts = (wts / wts.sum(axis=1, keepdims=True)).astype(np.float32)
+        e = idx.reshape(-1).astype(np.uint32)
+        t = np.repeat(np.arange(tokens, dtype=np.uint32), k)
+        r = wts.reshape(-1)
+        if tokens > 1:
+            order = np.lexsort((t, e))
+            e, t, r = e[order], t[order], r[order]
+        routes.append((e, r, t))
+
+    def step(i):
+        e, r, t = routes[i % len(routes)]
+        rnb.moe_sparse_experts_by_token_dev(gd, ud, dd, n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, x_dev, out_dev)
+
+    for i in range(10):
+        step(i)
+    tms = kernel_times_ms(hip, stream, step, min(steps, 200))
+    distinct = float(np.mean([len(np.unique(rt[0])) for rt in routes]))
+    weight_bytes = distinct * (2 * per_gate + per_down)
+    nbytes = weight_bytes + tokens * k * 292 + tokens * n_embd * 4
+    for b in (gd, ud, dd, x_dev, out_dev):
+        b.free()
+    ms = float(tms.mean())
+    return {"workload": f"cfg5 sparse MoE 128 experts top-8, hidden 2048, ffn 768, tokens={tokens}", "ms": ms,
+            "distinct_experts_mean": distinct, "bytes": nbytes, "GB/s": nbytes / ms / 1e6,
+            "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "ops": 2 * tokens * k * 3 * n_ff * n_embd,
+            "note": "events around the whole call (table upload + quantise + gate/up + re-quantise + down + reduce)"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--quick", action="store_true", help="headline config only (skip the secondary configs)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures the single-GPU hot path only: every box in this build has one GPU, and the path "
+            "has no collectives (it shards by weight rows / by expert). Run with --gpus 1.")
+        return 2
+
+    import runnburn_amd as rnb  # raises when librnb_hip.so has not been built: no fallback
+
+    if not rnb.device_available():
+        log(f"no MI355X device: {rnb.last_error()}")
+        return 3
+    hip = Hip()
+    stream = C.c_void_p(rnb.stream_handle())
+    log(f"device: {rnb.device_name()}")
+
+    rows, cols = 14336, 4096
+    main_res, w_host, x, gpu_out = bench_matmul(rnb, hip, stream, Q4_K, rows, cols, 1, args.steps, args.warmup, 20240607,
+                                                "cfg2 q4k gemv")
+    nbytes = main_res["bytes"]
+    step_ms = min(main_res["wall_ms_per_step"], main_res.get("graph_ms_per_step", float("inf")))
+    launch = "graph" if main_res.get("graph_ms_per_step", float("inf")) <= main_res["wall_ms_per_step"] else "stream"
+    achieved = nbytes / main_res["kernel_ms_mean"] / 1e6
+    result = {
+        "metric": "Q4_K decode GEMV HBM GB/s (% of 8 TB/s); prefill GEMM TOPS (% MFMA)",
+        "value": nbytes / step_ms / 1e6,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u4 x i8 -> i32, f32 scales",
+        "data": "synthetic: fp32 N(0,0.02) weights fitted to GGUF Q4_K blocks, fp32 N(0,1) activation, seeded",
+        "config": {"workload": "configs[1]: Q4_K decode GEMV, weights 14336x4096 (Llama-3-8B FFN up/gate), 1 token, "
+                               "step = device Q8_K quantisation + GEMV", "rows": rows, "cols": cols, "tokens": 1,
+                   "weight_copies_rotated": main_res["copies"], "step_launch": launch,
+                   "stream_ms_per_step": main_res["wall_ms_per_step"],
+                   "graph_ms_per_step": main_res.get("graph_ms_per_step")},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gemv_q4k_kernel",
+                     "bytes_per_launch": nbytes, "kernel_ms_mean": main_res["kernel_ms_mean"],
+                     "kernel_ms_median": main_res["kernel_ms_median"],
+                     "cache_resident_GBps": nbytes / main_res["kernel_ms_mean_cache_resident"] / 1e6},
+    }
+    if not args.no_cpu_baseline:
+        try:
+            result["cpu_baseline"] = cpu_baseline_gemv(Q4_K, w_host, rows, cols, x, gpu_out)
+        except Exception as exc:
+            log(f"cpu baseline failed: {exc}")
+            result["cpu_baseline"] = None
+    del w_host
+
+    if not args.quick:
+        sec = {}
+        s2 = max(50, min(args.steps, 500))
+        for key, quant, r, c, seq in (("cfg1_q8_0_gemv_4096x4096", Q8_0, 4096, 4096, 1),
+                                      ("cfg3a_q6k_gemv_4096x14336", Q6_K, 4096, 14336, 1),
+                                      ("cfg3b_q6k_gemv_128256x4096", Q6_K, 128256, 4096, 1)):
+            try:
+                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, seq, s2 if r < 100000 else 60, 10, 7 + r, key,
+                                            want_graph=False)
+                gbps = res["bytes"] / res["kernel_ms_mean"] / 1e6
+                sec[key] = {"kernel_ms_mean": res["kernel_ms_mean"], "bytes": res["bytes"], "GB/s": gbps,
+                            "hbm_frac": gbps / HBM_PEAK_GBPS, "copies": res["copies"],
+                            "cache_resident_GB/s": res["bytes"] / res["kernel_ms_mean_cache_resident"] / 1e6}
+            except Exception as exc:
+                sec[key] = {"error": str(exc)}
+        try:
+            res, _, _, _ = bench_matmul(rnb, hip, stream, Q4_K, 14336, 4096, 512, 40, 5, 99, "cfg4 q4k gemm",
+                                        want_graph=False)
+            ops = 2 * 512 * 14336 * 4096
+            tops = ops / res["kernel_ms_mean"] / 1e9
+            sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"kernel_ms_mean": res["kernel_ms_mean"], "ops": ops, "TOP/s": tops,
+                                                      "mfma_frac": tops / INT8_PEAK_TOPS}
+        except Exception as exc:
+            sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"error": str(exc)}
+        for tokens in (1, 64):
+            try:
+                sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens)
+            except Exception as exc:
+                sec[f"cfg5_moe_tokens{tokens}"] = {"error": str(exc)}
+        result["secondary"] = sec
+
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

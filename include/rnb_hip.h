@@ -136,6 +136,15 @@ int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes);
 /* quant: RNB_GGML_*; x_dev [seq_len][cols] f32 (16-byte aligned); out_dev [seq_len][rows] f32 */
 int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
                      const float *x_dev, size_t seq_len, float *out_dev);
+/* The two halves of rnb_hip_gemv_dev, for callers that feed several weight matrices from one
+ * activation (the reference quantises once for gate+up / QKV: rnb_quantize_q8_1_by_32 followed by
+ * rnb_q4k_gate_up_gemv_* in crates/rnb-backend/cuda/cuda/kernels/quant_gemv.cuh:700-1267).
+ * rnb_hip_quantize_dev fills the library's activation scratch from x_dev [seq_len][cols];
+ * rnb_hip_gemv_quantized_dev multiplies a weight matrix with whatever the scratch holds and must
+ * be given the same quant family (Q8_0 -> 32-wide Q8, Q4_K/Q6_K -> Q8_K), cols and seq_len. */
+int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols);
+int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
+                               size_t seq_len, float *out_dev);
 /* device-resident form of rnb_hip_moe_sparse_experts_by_token: weights, x and out on the device;
  * the slot arrays stay on the host (the caller routes on the host, as the reference does). */
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev,

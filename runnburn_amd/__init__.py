@@ -28,6 +28,8 @@ from .binding import (  # noqa: F401
     device_available,
     device_name,
     gemv_dev,
+    gemv_quantized_dev,
+    quantize_dev,
     last_error,
     lib,
     lib_path,

@@ -45,6 +45,8 @@ SYMBOLS = [
     ("rnb_hip_dev_upload", _i, [_vp, _vp, _sz]),
     ("rnb_hip_dev_download", _i, [_vp, _vp, _sz]),
     ("rnb_hip_gemv_dev", _i, [_u32, _vp, _sz, _sz, _vp, _sz, _vp]),
+    ("rnb_hip_quantize_dev", _i, [_u32, _vp, _sz, _sz]),
+    ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
 ]
@@ -291,6 +293,16 @@ def gemv_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, x: DeviceBuffer,
              out: DeviceBuffer) -> None:
     """Enqueue activation quantisation + GEMV/GEMM on the library stream; does not synchronise."""
     _check(lib().rnb_hip_gemv_dev(quant, w.ptr, rows, cols, x.ptr, seq_len, out.ptr))
+
+
+def quantize_dev(quant: int, x: DeviceBuffer, seq_len: int, cols: int) -> None:
+    """Fill the library's activation scratch from x (Q8 for Q8_0 weights, Q8_K otherwise)."""
+    _check(lib().rnb_hip_quantize_dev(quant, x.ptr, seq_len, cols))
+
+
+def gemv_quantized_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, seq_len: int, out: DeviceBuffer) -> None:
+    """GEMV/GEMM against the activation scratch filled by quantize_dev; does not synchronise."""
+    _check(lib().rnb_hip_gemv_quantized_dev(quant, w.ptr, rows, cols, seq_len, out.ptr))
 
 
 def moe_sparse_experts_by_token_dev(gate: DeviceBuffer, up: DeviceBuffer, down: DeviceBuffer, n_expert: int,

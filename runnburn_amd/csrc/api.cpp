@@ -59,17 +59,29 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
         *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
     }
     HIP_TRY(hipGetLastError());
+    s.act_family = quant == kQ8_0 ? kQ8_0 : kQ4K;
+    s.act_seq = seq;
+    s.act_cols = cols;
     return RNB_HIP_OK;
 }
 
 // Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
 constexpr size_t kGemmMinSeq = 16;
 
+int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
+                             float *out_dev);
+
 int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, const float *x_dev,
                    size_t seq, float *out_dev) {
     ActView act;
     int st = quantize_activations(s, quant, x_dev, seq, cols, &act);
     if (st != RNB_HIP_OK) return st;
+    return run_matmul_quantized_dev(s, quant, w_dev, rows, cols, seq, out_dev);
+}
+
+int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
+                             float *out_dev) {
+    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), quant == kQ8_0 ? nullptr : s.act_bsums.as<int16_t>()};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     if (quant == kQ4K) {
         if (seq >= kGemmMinSeq)
@@ -532,6 +544,42 @@ int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols
     Guard g;
     if (!g.state) return g.status;
     return run_matmul_dev(*g.state, quant, static_cast<const uint8_t *>(w_dev), rows, cols, x_dev, seq_len, out_dev);
+}
+
+int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    if (cols == 0 || cols % qi.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " cols must be divisible by " +
+                                                 std::to_string(qi.elems) + ", got " + std::to_string(cols));
+    if (!x_dev || (reinterpret_cast<uintptr_t>(x_dev) & 15u))
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " input must be a 16-byte aligned device pointer");
+    if (seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    ActView act;
+    return quantize_activations(*g.state, quant, x_dev, seq_len, cols, &act);
+}
+
+int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols, size_t seq_len,
+                               float *out_dev) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    if (!w_dev || !out_dev || (reinterpret_cast<uintptr_t>(w_dev) & 15u))
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " weights must be a 16-byte aligned device pointer");
+    if (rows > 0x7fffffffu || seq_len > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " shape out of range");
+    if (rows == 0 || seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint32_t family = quant == kQ8_0 ? kQ8_0 : kQ4K;
+    if (s.act_family != family || s.act_seq != seq_len || s.act_cols != cols)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    std::string(qi.label) + " activation scratch holds seq_len=" + std::to_string(s.act_seq) + " cols=" +
+                        std::to_string(s.act_cols) + " family=" + std::to_string(s.act_family) + ", requested seq_len=" +
+                        std::to_string(seq_len) + " cols=" + std::to_string(cols));
+    return run_matmul_quantized_dev(s, quant, static_cast<const uint8_t *>(w_dev), rows, cols, seq_len, out_dev);
 }
 
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev, const void *down_dev,

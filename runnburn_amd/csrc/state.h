@@ -56,6 +56,10 @@ struct State {
     PinnedBuf bounce_in, bounce_out, bounce_tables;
 
     std::map<uintptr_t, Resident> residents;  // keyed by host base address
+    // what the activation scratch currently holds (set by quantize_activations)
+    uint32_t act_family = 0;  // 8 = 32-wide Q8, 12 = Q8_K
+    size_t act_seq = 0, act_cols = 0;
+
     uint64_t resident_bytes = 0;
     uint64_t resident_budget = 0;  // bytes of unpinned + pinned residents before unpinned ones are evicted
     uint64_t epoch = 0;
