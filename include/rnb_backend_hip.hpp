@@ -1,0 +1,154 @@
+// rnb_backend_hip.hpp -- C++ host-side mirror of the reference's operator interface over the C ABI
+// in rnb_hip.h.  The reference's host code is Rust; with no Rust toolchain available this header
+// restates, name for name, the free functions a `rnb-backend-hip` crate would export:
+//
+//   q4k_gemv / q4k_gemv_into / q4k_gemv_batch   crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-238, 2283-2319
+//   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
+//   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
+//   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
+//   HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
+//
+// `Result<T, String>` becomes rnb_hip::Result<T>: either a value or the reference's error message.
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "rnb_hip.h"
+
+namespace rnb_hip {
+
+template <typename T>
+struct Result {
+    bool ok = false;
+    T value{};
+    int status = RNB_HIP_OK;  // rnb_hip_status
+    std::string error;
+    explicit operator bool() const { return ok; }
+};
+
+struct Unit {};
+
+template <typename T>
+inline Result<T> make_err(int status) {
+    Result<T> r;
+    r.status = status;
+    r.error = rnb_hip_last_error();
+    return r;
+}
+template <typename T>
+inline Result<T> make_ok(T v) {
+    Result<T> r;
+    r.ok = true;
+    r.value = std::move(v);
+    return r;
+}
+
+// borrowed byte / float ranges (the reference's &[u8] / &[f32])
+struct Bytes {
+    const uint8_t *ptr;
+    size_t len;
+};
+struct Floats {
+    const float *ptr;
+    size_t len;
+};
+
+using MatmulFn = int (*)(const uint8_t *, size_t, size_t, size_t, const float *, size_t, float *, size_t);
+
+inline Result<std::vector<float>> gemv_impl(MatmulFn fn, Bytes w, size_t rows, size_t cols, Floats x, size_t out_n) {
+    std::vector<float> out(out_n);
+    const int st = fn(w.ptr, w.len, rows, cols, x.ptr, x.len, out.data(), out.size());
+    if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
+    return make_ok(std::move(out));
+}
+inline Result<Unit> gemv_into_impl(MatmulFn fn, Bytes w, size_t rows, size_t cols, Floats x, float *out, size_t out_len) {
+    const int st = fn(w.ptr, w.len, rows, cols, x.ptr, x.len, out, out_len);
+    if (st != RNB_HIP_OK) return make_err<Unit>(st);
+    return make_ok(Unit{});
+}
+inline size_t batch_seq(Floats x, size_t cols) { return (cols != 0 && x.len % cols == 0) ? x.len / cols : 0; }
+
+inline Result<std::vector<float>> q4k_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q4k_gemv, weights, rows, cols, input, rows);
+}
+inline Result<Unit> q4k_gemv_into(Bytes weights, size_t rows, size_t cols, Floats input, float *output, size_t output_len) {
+    return gemv_into_impl(rnb_hip_q4k_gemv, weights, rows, cols, input, output, output_len);
+}
+inline Result<std::vector<float>> q4k_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q4k_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+inline Result<std::vector<float>> q6k_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q6k_gemv, weights, rows, cols, input, rows);
+}
+inline Result<Unit> q6k_gemv_into(Bytes weights, size_t rows, size_t cols, Floats input, float *output, size_t output_len) {
+    return gemv_into_impl(rnb_hip_q6k_gemv, weights, rows, cols, input, output, output_len);
+}
+inline Result<std::vector<float>> q6k_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q6k_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+inline Result<std::vector<float>> q8_0_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q8_0_gemv, weights, rows, cols, input, rows);
+}
+inline Result<std::vector<float>> q8_0_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
+    return gemv_impl(rnb_hip_q8_0_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+
+// prewarm_q4k_weights(&[&[u8]]), quant_api.rs:952
+inline Result<Unit> prewarm_weights(const std::vector<Bytes> &ranges) {
+    std::vector<const uint8_t *> ptrs;
+    std::vector<size_t> lens;
+    for (const Bytes &b : ranges) {
+        ptrs.push_back(b.ptr);
+        lens.push_back(b.len);
+    }
+    const int st = rnb_hip_prewarm(ptrs.data(), lens.data(), ptrs.size());
+    if (st != RNB_HIP_OK) return make_err<Unit>(st);
+    return make_ok(Unit{});
+}
+
+inline Result<std::vector<float>> qwen35_sparse_experts_selected_base_by_token(
+    Bytes gate_all, Bytes up_all, Bytes down_all, const std::vector<uint32_t> &expert_ids,
+    const std::vector<float> &route_weights, const std::vector<uint32_t> &token_ids, size_t token_count,
+    uint32_t down_quant, size_t n_ff, size_t n_embd, Floats input) {
+    if (route_weights.size() != expert_ids.size() || token_ids.size() != expert_ids.size()) {
+        Result<std::vector<float>> r;
+        r.status = RNB_HIP_INVALID_REQUEST;
+        r.error = "Qwen35 full-layer token-batch length mismatch: expert=" + std::to_string(expert_ids.size()) +
+                  " route=" + std::to_string(route_weights.size()) + " token=" + std::to_string(token_ids.size());
+        return r;
+    }
+    std::vector<float> out(token_count * n_embd);
+    const int st = rnb_hip_moe_sparse_experts_by_token(
+        gate_all.ptr, gate_all.len, up_all.ptr, up_all.len, down_all.ptr, down_all.len, expert_ids.data(),
+        route_weights.data(), token_ids.data(), expert_ids.size(), token_count, down_quant, n_ff, n_embd, input.ptr,
+        input.len, out.data(), out.size());
+    if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
+    return make_ok(std::move(out));
+}
+
+// trait Backend { kind, capabilities, execute }, crates/rnb-backend/api/src/lib.rs:1281-1285
+struct BackendCapabilities {
+    bool matmul, attention, gdn, moe, sampler;
+};
+class HipBackend {
+  public:
+    int kind() const { return rnb_hip_backend_kind(); }
+    BackendCapabilities capabilities() const {
+        return {rnb_hip_backend_supports(RNB_OP_MATMUL) != 0, rnb_hip_backend_supports(RNB_OP_ATTENTION) != 0,
+                rnb_hip_backend_supports(RNB_OP_GDN) != 0, rnb_hip_backend_supports(RNB_OP_MOE) != 0,
+                rnb_hip_backend_supports(RNB_OP_SAMPLER) != 0};
+    }
+    // Like CudaBackend::execute (crates/rnb-backend/cuda/src/lib.rs:193-195): requests are not executed through
+    // the trait; the operator functions above do the work.
+    Result<Unit> execute(int /*op*/) const {
+        Result<Unit> r;
+        r.status = RNB_HIP_UNSUPPORTED_OP;
+        r.error = "HipBackend::execute: requests are served by the operator functions";
+        return r;
+    }
+};
+
+}  // namespace rnb_hip

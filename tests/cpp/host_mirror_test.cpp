@@ -1,0 +1,113 @@
+// Exercises include/rnb_backend_hip.hpp (the C++ mirror of the reference's operator functions) against
+// librnb_hip.so.  Modes:
+//   host_mirror_test validate            no GPU needed: error messages, capability facade
+//   host_mirror_test run <golden_dir>    GPU: q4k/q6k/q8_0 gemv + batch on the committed raw fixtures
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <string>
+#include <vector>
+
+#include "../../include/rnb_backend_hip.hpp"
+
+using namespace rnb_hip;
+
+static int failures = 0;
+#define EXPECT(cond, what)                                    \
+    do {                                                      \
+        if (!(cond)) {                                        \
+            std::printf("FAIL: %s (%s)\n", what, #cond);      \
+            failures++;                                       \
+        }                                                     \
+    } while (0)
+
+template <typename T>
+static std::vector<T> read_file(const std::string &path) {
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    if (!f) {
+        std::printf("FAIL: cannot open %s\n", path.c_str());
+        failures++;
+        return {};
+    }
+    const size_t n = static_cast<size_t>(f.tellg());
+    std::vector<T> v(n / sizeof(T));
+    f.seekg(0);
+    f.read(reinterpret_cast<char *>(v.data()), static_cast<std::streamsize>(v.size() * sizeof(T)));
+    return v;
+}
+
+static int validate() {
+    std::vector<uint8_t> w(144, 0);
+    std::vector<float> x(256, 0.0f);
+    auto r = q4k_gemv({w.data(), w.size()}, 1, 255, {x.data(), 255});
+    EXPECT(!r && r.status == RNB_HIP_INVALID_REQUEST && r.error == "Q4_K cols must be divisible by 256, got 255", "cols message");
+    r = q4k_gemv({w.data(), 143}, 1, 256, {x.data(), 256});
+    EXPECT(!r && r.error == "Q4_K weight byte mismatch: got 143, expected 144", "weight bytes message");
+    r = q6k_gemv({w.data(), 144}, 1, 256, {x.data(), 256});
+    EXPECT(!r && r.error == "Q6_K weight byte mismatch: got 144, expected 210", "q6k weight bytes message");
+    r = q8_0_gemv_batch({w.data(), 34}, 1, 32, {x.data(), 33});
+    EXPECT(!r && r.error == "Q8_0 batch input length 33 is not divisible by cols 32", "q8_0 batch message");
+    float out1 = 0;
+    auto u = q4k_gemv_into({w.data(), 144}, 1, 256, {x.data(), 256}, &out1, 0);
+    EXPECT(!u && u.error == "Q4_K shape mismatch: input=256 output=0 expected input=256 output>=1", "into message");
+    auto m = qwen35_sparse_experts_selected_base_by_token({w.data(), 144}, {w.data(), 144}, {w.data(), 144}, {0, 1}, {1.0f}, {0}, 1, 14, 256, 256, {x.data(), 256});
+    EXPECT(!m && m.error.find("length mismatch") != std::string::npos, "moe slot arrays message");
+    HipBackend b;
+    EXPECT(b.kind() == 6, "kind ordinal");
+    const BackendCapabilities c = b.capabilities();
+    EXPECT(c.matmul && c.moe && !c.attention && !c.gdn && !c.sampler, "capabilities");
+    EXPECT(!b.execute(RNB_OP_MATMUL) && b.execute(RNB_OP_MATMUL).status == RNB_HIP_UNSUPPORTED_OP, "execute is a facade");
+    return failures;
+}
+
+static void run_case(const std::string &dir, const char *name, size_t rows, size_t cols, size_t seq,
+                     Result<std::vector<float>> (*fn)(Bytes, size_t, size_t, Floats)) {
+    const auto w = read_file<uint8_t>(dir + "/" + name + "_w.bin");
+    const auto x = read_file<float>(dir + "/" + name + "_x.bin");
+    const auto want = read_file<float>(dir + "/" + name + "_out.bin");
+    if (w.empty() || x.empty() || want.empty()) return;
+    auto r = fn({w.data(), w.size()}, rows, cols, {x.data(), x.size()});
+    if (!r) {
+        std::printf("FAIL: %s: %s\n", name, r.error.c_str());
+        failures++;
+        return;
+    }
+    EXPECT(r.value.size() == seq * rows && want.size() == seq * rows, "output size");
+    double ss = 0;
+    for (float v : want) ss += double(v) * v;
+    const double rms = std::sqrt(ss / double(want.size()));
+    double worst = 0;
+    for (size_t i = 0; i < want.size(); i++) {
+        const double diff = std::fabs(double(r.value[i]) - want[i]);
+        const double tol = std::fmax(1e-3 * rms, 1e-3 * std::fabs(want[i]));  // abs-or-rel, rel = 1e-3
+        if (!(diff <= tol)) failures++;
+        worst = std::fmax(worst, diff);
+    }
+    std::printf("%s: %zu outputs, max |diff| %.3g (rms %.3g)\n", name, want.size(), worst, rms);
+}
+
+int main(int argc, char **argv) {
+    if (argc >= 2 && std::strcmp(argv[1], "validate") == 0) {
+        const int f = validate();
+        std::printf("validate: %d failure(s)\n", f);
+        return f ? 1 : 0;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "run") == 0) {
+        if (rnb_hip_init() != RNB_HIP_OK) {
+            std::printf("SKIP: %s\n", rnb_hip_last_error());
+            return 77;
+        }
+        const std::string dir = argv[2];
+        run_case(dir, "q4k_gemv", 24, 1024, 1, q4k_gemv);
+        run_case(dir, "q6k_gemv", 20, 768, 1, q6k_gemv);
+        run_case(dir, "q8_0_gemv", 16, 544, 1, q8_0_gemv);
+        run_case(dir, "q4k_batch", 40, 512, 19, q4k_gemv_batch);
+        run_case(dir, "q6k_batch", 9, 512, 3, q6k_gemv_batch);
+        run_case(dir, "q8_0_batch", 7, 96, 4, q8_0_gemv_batch);
+        std::printf("run: %d failure(s)\n", failures);
+        return failures ? 1 : 0;
+    }
+    std::printf("usage: host_mirror_test validate | run <golden_dir>\n");
+    return 2;
+}
