@@ -159,21 +159,19 @@ class Hip:
         return float(ms.value)
 
 
-def kernel_times_ms(hip, stream, launch, n, pre=None):
-    """Mean/median duration of `launch(i)` over n launches: one event pair per launch on the stream the
-    kernel runs on.  `pre(i)` is enqueued before the start event (e.g. the activation quantiser)."""
-    starts = [hip.event() for _ in range(n)]
-    stops = [hip.event() for _ in range(n)]
+def kernel_time_ms(hip, stream, launch, n):
+    """Mean duration of `launch(i)` over n back-to-back launches: one HIP event before the first and one
+    after the last, both recorded on the stream the kernel runs on (same-stream launches serialise, so
+    elapsed / n is the kernel duration plus the inter-launch gap)."""
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, stream)
     for i in range(n):
-        if pre is not None:
-            pre(i)
-        hip.record(starts[i], stream)
         launch(i)
-        hip.record(stops[i], stream)
-    t = np.array([hip.elapsed_ms(starts[i], stops[i]) for i in range(n)])
-    for ev in starts + stops:
-        hip.rt.hipEventDestroy(ev)
-    return t
+    hip.record(e1, stream)
+    ms = hip.elapsed_ms(e0, e1)
+    hip.rt.hipEventDestroy(e0)
+    hip.rt.hipEventDestroy(e1)
+    return ms / n
 
 
 def wall_steps(rnb, step, n):
@@ -221,7 +219,8 @@ def copies_for(nbytes):
     return max(2, -(-2 * MALL_BYTES // nbytes))
 
 
-def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, name, want_graph=True):
+def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, name, want_graph=True,
+                 cache_resident=False):
     w_host = synth_weights(quant, rows, cols, seed)
     n_copies = copies_for(w_host.nbytes)
     log(f"[{name}] weights {w_host.nbytes / 1e6:.1f} MB x {n_copies} device copies")
@@ -246,16 +245,17 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
         except Exception as exc:  # keep the stream number if capture is unavailable
             log(f"[{name}] graph replay unavailable: {exc}")
     rnb.quantize_dev(quant, x_dev, seq, cols)
-    t = kernel_times_ms(hip, stream, lambda i: rnb.gemv_quantized_dev(quant, w_dev[i % n_copies], rows, cols, seq, out_dev),
-                        min(steps, 1000))
-    res["kernel_ms_mean"] = float(t.mean())
-    res["kernel_ms_median"] = float(np.median(t))
-    res["kernel_ms_p10"] = float(np.percentile(t, 10))
-    res["kernel_ms_p90"] = float(np.percentile(t, 90))
-    # cache-resident variant (one copy, weights may stay in the 256 MiB Infinity Cache): labelled, never `value`
-    t1 = kernel_times_ms(hip, stream, lambda i: rnb.gemv_quantized_dev(quant, w_dev[0], rows, cols, seq, out_dev),
-                         min(steps, 300))
-    res["kernel_ms_mean_cache_resident"] = float(t1.mean())
+    n_k = min(steps, 1000)
+    launch = lambda i: rnb.gemv_quantized_dev(quant, w_dev[i % n_copies], rows, cols, seq, out_dev)  # noqa: E731
+    for i in range(min(20, n_k)):
+        launch(i)
+    reps = [kernel_time_ms(hip, stream, launch, n_k) for _ in range(3)]
+    res["kernel_ms_mean"] = float(np.mean(reps))
+    res["kernel_ms_runs"] = [float(v) for v in reps]
+    if cache_resident:
+        # one copy only: the weights may stay in the 256 MiB Infinity Cache; labelled, never `value`
+        one = lambda i: rnb.gemv_quantized_dev(quant, w_dev[0], rows, cols, seq, out_dev)  # noqa: E731
+        res["kernel_ms_mean_cache_resident"] = kernel_time_ms(hip, stream, one, min(steps, 300))
     res["bytes"] = gemv_bytes(quant, rows, cols, seq)
     res["copies"] = n_copies
     out = out_dev.to_host(np.float32)
@@ -327,13 +327,13 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed):
 
     for i in range(10):
         step(i)
-    tms = kernel_times_ms(hip, stream, step, min(steps, 200))
+    n_k = min(steps, 200)
+    ms = float(np.mean([kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]))
     distinct = float(np.mean([len(np.unique(rt[0])) for rt in routes]))
     weight_bytes = distinct * (2 * per_gate + per_down)
     nbytes = weight_bytes + tokens * k * 292 + tokens * n_embd * 4
     for b in (gd, ud, dd, x_dev, out_dev):
         b.free()
-    ms = float(tms.mean())
     return {"workload": f"cfg5 sparse MoE 128 experts top-8, hidden 2048, ffn 768, tokens={tokens}", "ms": ms,
             "distinct_experts_mean": distinct, "bytes": nbytes, "GB/s": nbytes / ms / 1e6,
             "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "ops": 2 * tokens * k * 3 * n_ff * n_embd,
@@ -347,6 +347,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--quick", action="store_true", help="headline config only (skip the secondary configs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cache-resident", action="store_true",
+                    help="also time each kernel on ONE weight copy (may be served by the Infinity Cache)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures the single-GPU hot path only: every box in this build has one GPU, and the path "
@@ -364,7 +366,7 @@ def main() -> int:
 
     rows, cols = 14336, 4096
     main_res, w_host, x, gpu_out = bench_matmul(rnb, hip, stream, Q4_K, rows, cols, 1, args.steps, args.warmup, 20240607,
-                                                "cfg2 q4k gemv")
+                                                "cfg2 q4k gemv", cache_resident=args.cache_resident)
     nbytes = main_res["bytes"]
     step_ms = min(main_res["wall_ms_per_step"], main_res.get("graph_ms_per_step", float("inf")))
     launch = "graph" if main_res.get("graph_ms_per_step", float("inf")) <= main_res["wall_ms_per_step"] else "stream"
@@ -390,9 +392,11 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gemv_q4k_kernel",
                      "bytes_per_launch": nbytes, "kernel_ms_mean": main_res["kernel_ms_mean"],
-                     "kernel_ms_median": main_res["kernel_ms_median"],
-                     "cache_resident_GBps": nbytes / main_res["kernel_ms_mean_cache_resident"] / 1e6},
+                     "kernel_ms_runs": main_res["kernel_ms_runs"],
+                     "timing": "HIP events around back-to-back launches on the library stream, 3 runs"},
     }
+    if "kernel_ms_mean_cache_resident" in main_res:
+        result["roofline"]["cache_resident_GBps"] = nbytes / main_res["kernel_ms_mean_cache_resident"] / 1e6
     if not args.no_cpu_baseline:
         try:
             result["cpu_baseline"] = cpu_baseline_gemv(Q4_K, w_host, rows, cols, x, gpu_out)
@@ -409,11 +413,12 @@ def main() -> int:
                                       ("cfg3b_q6k_gemv_128256x4096", Q6_K, 128256, 4096, 1)):
             try:
                 res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, seq, s2 if r < 100000 else 60, 10, 7 + r, key,
-                                            want_graph=False)
+                                            want_graph=False, cache_resident=args.cache_resident)
                 gbps = res["bytes"] / res["kernel_ms_mean"] / 1e6
                 sec[key] = {"kernel_ms_mean": res["kernel_ms_mean"], "bytes": res["bytes"], "GB/s": gbps,
-                            "hbm_frac": gbps / HBM_PEAK_GBPS, "copies": res["copies"],
-                            "cache_resident_GB/s": res["bytes"] / res["kernel_ms_mean_cache_resident"] / 1e6}
+                            "hbm_frac": gbps / HBM_PEAK_GBPS, "copies": res["copies"]}
+                if "kernel_ms_mean_cache_resident" in res:
+                    sec[key]["cache_resident_GB/s"] = res["bytes"] / res["kernel_ms_mean_cache_resident"] / 1e6
             except Exception as exc:
                 sec[key] = {"error": str(exc)}
         try:

@@ -1,0 +1,111 @@
+// Wave-level activation quantisers, bit-exact with rnb-cpu: one wave64
+// quantises one 256-element span (one Q8_K block, or eight 32-wide Q8 blocks); each lane owns four
+// consecutive elements.  Single IEEE multiplies and correctly rounded divisions only
+// (-ffp-contract=off), see quantize_act.hip.
+//
+//  Q8_K: crates/rnb-cpu/src/gemm/activation_q8.rs:149-173 (quantize_q8k_block_ggml)
+//  Q8  : crates/rnb-cpu/src/gemm/activation_q8.rs:14-32   (quantize_input_q8)
+#pragma once
+
+#include "device_utils.h"
+
+namespace rnb {
+
+struct AbsMax {
+    float amax;  // max |x|
+    float val;   // the signed element that attained it first
+    int idx;     // its index within the 256-span
+};
+
+// first occurrence wins: larger |x|, or equal |x| and smaller index
+__device__ __forceinline__ AbsMax absmax_merge(AbsMax a, AbsMax b) {
+    const bool take_b = (b.amax > a.amax) || (b.amax == a.amax && b.idx < a.idx);
+    return take_b ? b : a;
+}
+
+// Quantises x_blk[0..256) to one Q8_K block: qs (256 int8, 16-byte aligned), *d_out, bsums (16 int16).
+// Must be called by all 64 lanes of the wave.
+// `v` = this lane's four consecutive elements (x_blk[4*lane .. 4*lane+4)), already loaded.
+__device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8_t *qs, float *d_out, int16_t *bsums) {
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    AbsMax m{0.0f, 0.0f, 4 * lane};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float ax = fabsf(e[i]);
+        if (ax > m.amax) {  // strict: keeps the first of equal magnitudes
+            m.amax = ax;
+            m.val = e[i];
+            m.idx = 4 * lane + i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        AbsMax o;
+        o.amax = __shfl_xor(m.amax, off, kWave);
+        o.val = __shfl_xor(m.val, off, kWave);
+        o.idx = __shfl_xor(m.idx, off, kWave);
+        m = absmax_merge(m, o);
+    }
+    float iscale = 0.0f, d = 0.0f;
+    if (m.amax != 0.0f) {
+        iscale = -127.0f / m.val;
+        d = 1.0f / iscale;
+    }
+    int part = 0;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float prod = iscale * e[i];
+        int r = __float2int_rn(prod);  // round half to even
+        r = r > 127 ? 127 : r;         // upper clamp only
+        const int q = static_cast<int>(static_cast<int8_t>(r));
+        part += q;
+        packed |= (static_cast<uint32_t>(q) & 0xffu) << (8 * i);
+    }
+    reinterpret_cast<uint32_t *>(qs)[lane] = packed;
+    const int sum16 = group_sum_i<4>(part);  // 4 lanes = 16 consecutive elements
+    if ((lane & 3) == 0) bsums[lane >> 2] = static_cast<int16_t>(sum16);
+    if (lane == 0) *d_out = d;
+}
+
+__device__ __forceinline__ void q8k_quantize_span(const float *__restrict__ x_blk, int lane, int8_t *qs, float *d_out,
+                                                  int16_t *bsums) {
+    q8k_quantize_vals(reinterpret_cast<const float4 *>(x_blk)[lane], lane, qs, d_out, bsums);
+}
+
+// Quantises x_span[0..256) to eight 32-wide Q8 blocks (8 lanes per block); lanes whose block index
+// (lane / 8) is >= live_blocks neither read nor write.
+__device__ __forceinline__ float4 q8_load_span(const float *__restrict__ x_span, int lane, int live_blocks) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if ((lane >> 3) < live_blocks) v = reinterpret_cast<const float4 *>(x_span)[lane];
+    return v;
+}
+
+__device__ __forceinline__ void q8_quantize_vals(const float4 v, int lane, int live_blocks, int8_t *qs, float *d_out) {
+    const bool live = (lane >> 3) < live_blocks;
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? 1.0f / d : 0.0f;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float prod = e[i] * id;
+        float r = roundf(prod);  // half away from zero
+        r = fminf(fmaxf(r, -128.0f), 127.0f);
+        packed |= (static_cast<uint32_t>(static_cast<int>(r)) & 0xffu) << (8 * i);
+    }
+    if (live) {
+        reinterpret_cast<uint32_t *>(qs)[lane] = packed;
+        if ((lane & 7) == 0) d_out[lane >> 3] = d;
+    }
+}
+
+__device__ __forceinline__ void q8_quantize_span(const float *__restrict__ x_span, int lane, int live_blocks, int8_t *qs,
+                                                 float *d_out) {
+    q8_quantize_vals(q8_load_span(x_span, lane, live_blocks), lane, live_blocks, qs, d_out);
+}
+
+}  // namespace rnb

@@ -2,6 +2,7 @@
 // messages, staging through pinned bounce buffers, kernel sequencing on the single stream.
 #include "../../include/rnb_hip.h"
 
+#include <algorithm>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -231,28 +232,49 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                 size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
                 const float *x_dev, float *out_dev) {
     if (token_count == 0) return RNB_HIP_OK;
-    // host tables: expert[n], token[n], route[n], tok_offsets[T+1], tok_slots[n]
-    const size_t table_words = 4 * n_slots + token_count + 1;
+    // host tables (one upload): route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] |
+    // grp_expert[G] | grp_start[G+1]; slots are grouped by expert, keeping slot order inside a group
+    std::vector<uint32_t> order(n_slots);
+    for (size_t i = 0; i < n_slots; i++) order[i] = static_cast<uint32_t>(i);
+    std::stable_sort(order.begin(), order.end(),
+                     [expert_ids](uint32_t a, uint32_t b) { return expert_ids[a] < expert_ids[b]; });
+    std::vector<uint32_t> grp_expert, grp_start;
+    for (size_t p = 0; p < n_slots; p++) {
+        if (p == 0 || expert_ids[order[p]] != expert_ids[order[p - 1]]) {
+            grp_expert.push_back(expert_ids[order[p]]);
+            grp_start.push_back(static_cast<uint32_t>(p));
+        }
+    }
+    grp_start.push_back(static_cast<uint32_t>(n_slots));
+    const size_t n_groups = grp_expert.size();
+    const size_t table_words = 4 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
     HIP_TRY(s.bounce_tables.reserve(table_words * 4));
     HIP_TRY(s.moe_tables.reserve(table_words * 4));
     uint32_t *h = s.bounce_tables.as<uint32_t>();
-    uint32_t *h_expert = h, *h_token = h + n_slots;
-    float *h_route = reinterpret_cast<float *>(h + 2 * n_slots);
-    uint32_t *h_off = h + 3 * n_slots, *h_list = h_off + token_count + 1;
+    float *h_route = reinterpret_cast<float *>(h);
+    uint32_t *h_off = h + n_slots, *h_list = h_off + token_count + 1;
+    uint32_t *h_sslot = h_list + n_slots, *h_stok = h_sslot + n_slots;
+    uint32_t *h_gexp = h_stok + n_slots, *h_gstart = h_gexp + n_groups;
     HIP_TRY(hipStreamSynchronize(s.stream));  // the previous call's table upload must have drained
-    std::memcpy(h_expert, expert_ids, n_slots * 4);
-    std::memcpy(h_token, token_ids, n_slots * 4);
     std::memcpy(h_route, route, n_slots * 4);
     std::vector<uint32_t> counts(token_count + 1, 0);
     for (size_t i = 0; i < n_slots; i++) counts[token_ids[i] + 1]++;
     for (size_t t = 0; t < token_count; t++) counts[t + 1] += counts[t];
     std::memcpy(h_off, counts.data(), (token_count + 1) * 4);
     for (size_t i = 0; i < n_slots; i++) h_list[counts[token_ids[i]]++] = static_cast<uint32_t>(i);  // slot order kept
+    for (size_t p = 0; p < n_slots; p++) {
+        h_sslot[p] = order[p];
+        h_stok[p] = token_ids[order[p]];
+    }
+    if (n_groups) std::memcpy(h_gexp, grp_expert.data(), n_groups * 4);
+    std::memcpy(h_gstart, grp_start.data(), (n_groups + 1) * 4);
     uint32_t *d = s.moe_tables.as<uint32_t>();
     HIP_TRY(hipMemcpyAsync(d, h, table_words * 4, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += table_words * 4;
-    MoeSlots slots{d, d + n_slots, reinterpret_cast<const float *>(d + 2 * n_slots), static_cast<uint32_t>(n_slots)};
-    const uint32_t *d_off = d + 3 * n_slots, *d_list = d_off + token_count + 1;
+    const float *d_route = reinterpret_cast<const float *>(d);
+    const uint32_t *d_off = d + n_slots, *d_list = d_off + token_count + 1;
+    const MoeGroups groups{d_list + 3 * n_slots, d_list + 3 * n_slots + n_groups, d_list + n_slots, d_list + 2 * n_slots,
+                           static_cast<uint32_t>(n_groups)};
 
     if (n_slots == 0) {  // nothing routed: the reduce kernel alone writes the zero rows
         launch_moe_reduce(nullptr, d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
@@ -268,13 +290,13 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     HIP_TRY(s.moe_mid_d.reserve(n_slots * sh.nb_mid * sizeof(float)));
     HIP_TRY(s.moe_mid_bsums.reserve(n_slots * sh.nb_mid * 16 * sizeof(int16_t)));
     HIP_TRY(s.moe_slot_out.reserve(n_slots * n_embd * sizeof(float)));
-    launch_moe_gate_up(gate_dev, up_dev, act, slots, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
+    launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
     launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
                         s.moe_mid_bsums.as<int16_t>(), s.stream);
     ActView mid{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>()};
-    launch_moe_down(down_dev, down_quant, mid, slots, s.moe_slot_out.as<float>(), static_cast<uint32_t>(n_embd),
-                    static_cast<uint32_t>(sh.nb_mid), s.stream);
+    launch_moe_down(down_dev, down_quant, mid, groups, d_route, s.moe_slot_out.as<float>(),
+                    static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
     launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                       static_cast<uint32_t>(n_embd), s.stream);
     HIP_TRY(hipGetLastError());

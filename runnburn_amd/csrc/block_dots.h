@@ -1,6 +1,7 @@
-// Per-lane partial dot products of one GGUF super-block against one Q8_K activation block, shared
-// by the decode GEMV and the gathered-MoE kernels.  Eight lanes cooperate on a 256-element block;
-// the caller adds the partials across lanes.
+// Per-lane partial dot products of one GGUF super-block against one Q8_K activation block, shared by
+// the decode GEMV and the gathered-MoE kernels.  FOUR lanes cooperate on a 256-element block (a wave64
+// pass covers 16 blocks); the caller adds the partials across lanes.  Activations are held in
+// registers (`Q4KAct` / `Q6KAct`) so that a wave which walks many rows loads them once.
 #pragma once
 
 #include "device_utils.h"
@@ -9,84 +10,154 @@
 namespace rnb {
 
 // ---------------------------------------------------------------------------------------------
-// Q4_K: block = {f16 d, f16 dmin, u8 scales[12], u8 qs[128]}.  Lane c (0..7) of a block group
-// owns qs[16c .. 16c+16): group g = c/2 holds elements 64g + 16(c&1) + [0,16) in the low nibbles
-// (scale 2g) and 64g + 32 + 16(c&1) + [0,16) in the high nibbles (scale 2g+1).  The mins term of
-// sub-block c goes to lane c.
+// Q4_K: block = {f16 d, f16 dmin, u8 scales[12], u8 qs[128]}.  Lane g (0..3) of a block owns group g:
+// qs[32g .. 32g+32) -> elements 64g + [0,32) in the low nibbles (scale 2g, min 2g) and
+// 64g + 32 + [0,32) in the high nibbles (scale 2g+1, min 2g+1).
+//   sumi = sc[2g]*dot(lo, a_lo) + sc[2g+1]*dot(hi, a_hi);  summ = mn[2g]*bsum32[2g] + mn[2g+1]*bsum32[2g+1]
+//   partial = d_x * (d*sumi - dmin*summ)          crates/rnb-cpu/src/gemm/neon_dot.rs:884-916
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float q4k_block_partial(const uint8_t *__restrict__ blk, const int8_t *__restrict__ aq,
-                                                   float dx, const int16_t *__restrict__ bs, int c) {
-    const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
-    const uint4 q = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * c);
-    const int g = c >> 1, half = c & 1;
-    const uint4 a_lo = *reinterpret_cast<const uint4 *>(aq + 64 * g + 16 * half);
-    const uint4 a_hi = *reinterpret_cast<const uint4 *>(aq + 64 * g + 32 + 16 * half);
-    const uint32_t bs_pair = *reinterpret_cast<const uint32_t *>(bs + 2 * c);  // bsums[2c], bsums[2c+1]
+struct Q4KAct {
+    uint4 lo0, lo1, hi0, hi1;  // 64 int8 activations of group g
+    float dx;                  // Q8_K block scale
+    int bs_lo, bs_hi;          // bsum32[2g], bsum32[2g+1]
+};
 
-    const float d = f16_bits_to_f32(hdr.x);
-    const float dmin = f16_bits_to_f32(hdr.x >> 16);
-    const Q4KScales s = unpack_q4k_scales(hdr.y, hdr.z, hdr.w);
-    const int sc0 = byte_of(s.sc_lo, s.sc_hi, 2 * g);
-    const int sc1 = byte_of(s.sc_lo, s.sc_hi, 2 * g + 1);
-    const int mn = byte_of(s.mn_lo, s.mn_hi, c);
+__device__ __forceinline__ Q4KAct q4k_load_act(const int8_t *__restrict__ aq_blk, float dx,
+                                               const int16_t *__restrict__ bs_blk, int g) {
+    Q4KAct a;
+    const int8_t *p = aq_blk + 64 * g;
+    a.lo0 = *reinterpret_cast<const uint4 *>(p);
+    a.lo1 = *reinterpret_cast<const uint4 *>(p + 16);
+    a.hi0 = *reinterpret_cast<const uint4 *>(p + 32);
+    a.hi1 = *reinterpret_cast<const uint4 *>(p + 48);
+    a.dx = dx;
+    const uint2 bp = *reinterpret_cast<const uint2 *>(bs_blk + 4 * g);  // bsums[4g .. 4g+4)
+    a.bs_lo = static_cast<int>(static_cast<int16_t>(bp.x & 0xffffu)) + (static_cast<int>(bp.x) >> 16);
+    a.bs_hi = static_cast<int>(static_cast<int16_t>(bp.y & 0xffffu)) + (static_cast<int>(bp.y) >> 16);
+    return a;
+}
 
+struct Q4KRegs {
+    uint4 h, qa, qb;  // 16-byte header, 32 bytes of packed nibbles
+};
+
+__device__ __forceinline__ Q4KRegs q4k_load_block(const uint8_t *__restrict__ blk, int g) {
+    Q4KRegs r;
+    r.h = *reinterpret_cast<const uint4 *>(blk);
+    r.qa = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * g);
+    r.qb = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * g);
+    return r;
+}
+
+__device__ __forceinline__ float q4k_partial(const Q4KRegs &r, const Q4KAct &a, int g) {
+    const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
+    const Q4KScales s = unpack_q4k_scales(r.h.y, r.h.z, r.h.w);
+    const uint32_t scw = (g & 2) ? s.sc_hi : s.sc_lo, mnw = (g & 2) ? s.mn_hi : s.mn_lo;
+    const int sh = (g & 1) * 16;
+    const int sc0 = (scw >> sh) & 0xff, sc1 = (scw >> (sh + 8)) & 0xff;
+    const int mn0 = (mnw >> sh) & 0xff, mn1 = (mnw >> (sh + 8)) & 0xff;
     int i0 = 0, i1 = 0;
-    i0 = dot4(q.x & 0x0f0f0f0fu, a_lo.x, i0);
-    i0 = dot4(q.y & 0x0f0f0f0fu, a_lo.y, i0);
-    i0 = dot4(q.z & 0x0f0f0f0fu, a_lo.z, i0);
-    i0 = dot4(q.w & 0x0f0f0f0fu, a_lo.w, i0);
-    i1 = dot4((q.x >> 4) & 0x0f0f0f0fu, a_hi.x, i1);
-    i1 = dot4((q.y >> 4) & 0x0f0f0f0fu, a_hi.y, i1);
-    i1 = dot4((q.z >> 4) & 0x0f0f0f0fu, a_hi.z, i1);
-    i1 = dot4((q.w >> 4) & 0x0f0f0f0fu, a_hi.w, i1);
+    i0 = dot4(r.qa.x & 0x0f0f0f0fu, a.lo0.x, i0);
+    i0 = dot4(r.qa.y & 0x0f0f0f0fu, a.lo0.y, i0);
+    i0 = dot4(r.qa.z & 0x0f0f0f0fu, a.lo0.z, i0);
+    i0 = dot4(r.qa.w & 0x0f0f0f0fu, a.lo0.w, i0);
+    i0 = dot4(r.qb.x & 0x0f0f0f0fu, a.lo1.x, i0);
+    i0 = dot4(r.qb.y & 0x0f0f0f0fu, a.lo1.y, i0);
+    i0 = dot4(r.qb.z & 0x0f0f0f0fu, a.lo1.z, i0);
+    i0 = dot4(r.qb.w & 0x0f0f0f0fu, a.lo1.w, i0);
+    i1 = dot4((r.qa.x >> 4) & 0x0f0f0f0fu, a.hi0.x, i1);
+    i1 = dot4((r.qa.y >> 4) & 0x0f0f0f0fu, a.hi0.y, i1);
+    i1 = dot4((r.qa.z >> 4) & 0x0f0f0f0fu, a.hi0.z, i1);
+    i1 = dot4((r.qa.w >> 4) & 0x0f0f0f0fu, a.hi0.w, i1);
+    i1 = dot4((r.qb.x >> 4) & 0x0f0f0f0fu, a.hi1.x, i1);
+    i1 = dot4((r.qb.y >> 4) & 0x0f0f0f0fu, a.hi1.y, i1);
+    i1 = dot4((r.qb.z >> 4) & 0x0f0f0f0fu, a.hi1.z, i1);
+    i1 = dot4((r.qb.w >> 4) & 0x0f0f0f0fu, a.hi1.w, i1);
     const int sumi = sc0 * i0 + sc1 * i1;
-    const int bsum32 = static_cast<int>(static_cast<int16_t>(bs_pair & 0xffffu)) + (static_cast<int>(bs_pair) >> 16);
-    const int summ = mn * bsum32;
-    return dx * (d * static_cast<float>(sumi) - dmin * static_cast<float>(summ));
+    const int summ = mn0 * a.bs_lo + mn1 * a.bs_hi;
+    return a.dx * (d * static_cast<float>(sumi) - dmin * static_cast<float>(summ));
 }
 
 // ---------------------------------------------------------------------------------------------
 // Q6_K: block = {u8 ql[128], u8 qh[64], i8 scales[16], f16 d}, 210 bytes, 2-byte aligned.
-// Lane (n = half 0/1, t = 0..3) of a block group owns l = 8t .. 8t+7 of half n: 8 bytes of
-// ql[64n + l], 8 of ql[64n + 32 + l], 8 of qh[32n + l] -> 32 six-bit values, four per activation
-// quarter 128n + 32i + l.  (q - 32) is applied as  dot(q, a) - 32 * sum(a).
+// Lane q (0..3) of a block owns half n = q>>1, l = 16*(q&1) .. +16: 16 bytes each of ql[64n+l],
+// ql[64n+32+l], qh[32n+l] -> 64 six-bit values, 16 per activation quarter 128n + 32i + l (i = 0..3),
+// scale index 8n + (q&1) + 2i.  (q6 - 32) is applied as dot(q6, a) - 32*sum(a); the activation sums
+// are part of the held activation state.                 crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ int sext8(uint32_t v, int shift) { return static_cast<int>(static_cast<int8_t>((v >> shift) & 0xffu)); }
+struct Q6KAct {
+    uint4 a0, a1, a2, a3;  // 16 int8 activations of each quarter
+    int s0, s1, s2, s3;    // their sums
+    float dx;
+};
 
-__device__ __forceinline__ float q6k_block_partial(const uint8_t *__restrict__ blk, const int8_t *__restrict__ aq,
-                                                   float dx, int sub) {
-    const int n = sub >> 2, t = sub & 3;
-    const uint2 A = ld_u2_a2(blk + 64 * n + 8 * t);
-    const uint2 B = ld_u2_a2(blk + 64 * n + 32 + 8 * t);
-    const uint2 H = ld_u2_a2(blk + 128 + 32 * n + 8 * t);
-    const uint2 S = ld_u2_a2(blk + 192 + 8 * n);
-    const float d = ld_f16(blk + 208);
-    const int8_t *a = aq + 128 * n + 8 * t;
-    const uint2 a0 = *reinterpret_cast<const uint2 *>(a);
-    const uint2 a1 = *reinterpret_cast<const uint2 *>(a + 32);
-    const uint2 a2 = *reinterpret_cast<const uint2 *>(a + 64);
-    const uint2 a3 = *reinterpret_cast<const uint2 *>(a + 96);
+__device__ __forceinline__ int sum16(const uint4 &v) {
+    int s = 0;
+    s = dot4(0x01010101u, v.x, s);
+    s = dot4(0x01010101u, v.y, s);
+    s = dot4(0x01010101u, v.z, s);
+    s = dot4(0x01010101u, v.w, s);
+    return s;
+}
 
-    const int is = (t >> 1) * 8;  // l / 16 selects scale byte 0 or 1 of each pair
-    const int s0 = sext8(S.x, is), s1 = sext8(S.x, is + 16), s2 = sext8(S.y, is), s3 = sext8(S.y, is + 16);
+__device__ __forceinline__ Q6KAct q6k_load_act(const int8_t *__restrict__ aq_blk, float dx, int q) {
+    Q6KAct a;
+    const int8_t *p = aq_blk + 128 * (q >> 1) + 16 * (q & 1);
+    a.a0 = *reinterpret_cast<const uint4 *>(p);
+    a.a1 = *reinterpret_cast<const uint4 *>(p + 32);
+    a.a2 = *reinterpret_cast<const uint4 *>(p + 64);
+    a.a3 = *reinterpret_cast<const uint4 *>(p + 96);
+    a.s0 = sum16(a.a0);
+    a.s1 = sum16(a.a1);
+    a.s2 = sum16(a.a2);
+    a.s3 = sum16(a.a3);
+    a.dx = dx;
+    return a;
+}
 
+struct Q6KRegs {
+    uint4 A, B, H;
+    uint2 S;
+    uint32_t d_bits;
+};
+
+__device__ __forceinline__ Q6KRegs q6k_load_block(const uint8_t *__restrict__ blk, int q) {
+    Q6KRegs r;
+    const int n = q >> 1, th = q & 1;
+    r.A = ld_u4_a2(blk + 64 * n + 16 * th);
+    r.B = ld_u4_a2(blk + 64 * n + 32 + 16 * th);
+    r.H = ld_u4_a2(blk + 128 + 32 * n + 16 * th);
+    r.S = ld_u2_a2(blk + 192 + 8 * n);
+    r.d_bits = *reinterpret_cast<const unsigned short *>(blk + 208);
+    return r;
+}
+
+__device__ __forceinline__ int sext8(uint32_t v, int shift) {
+    return static_cast<int>(static_cast<int8_t>((v >> shift) & 0xffu));
+}
+
+__device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, int q) {
+    const int is = (q & 1) * 8;  // l / 16 selects scale byte 0 or 1 of each pair
+    const int s0 = sext8(r.S.x, is), s1 = sext8(r.S.x, is + 16), s2 = sext8(r.S.y, is), s3 = sext8(r.S.y, is + 16);
     int p0 = 0, p1 = 0, p2 = 0, p3 = 0;
-#define RNB_Q6_STEP(Ak, Bk, Hk, a0k, a1k, a2k, a3k)                                   \
-    {                                                                                 \
-        const uint32_t u0 = ((Ak) & 0x0f0f0f0fu) | (((Hk) & 0x03030303u) << 4);       \
-        const uint32_t u1 = ((Bk) & 0x0f0f0f0fu) | (((Hk) & 0x0c0c0c0cu) << 2);       \
-        const uint32_t u2 = (((Ak) >> 4) & 0x0f0f0f0fu) | ((Hk) & 0x30303030u);       \
-        const uint32_t u3 = (((Bk) >> 4) & 0x0f0f0f0fu) | (((Hk) & 0xc0c0c0c0u) >> 2); \
-        p0 = dot4(u0, a0k, p0) - dot4(0x20202020u, a0k, 0);                           \
-        p1 = dot4(u1, a1k, p1) - dot4(0x20202020u, a1k, 0);                           \
-        p2 = dot4(u2, a2k, p2) - dot4(0x20202020u, a2k, 0);                           \
-        p3 = dot4(u3, a3k, p3) - dot4(0x20202020u, a3k, 0);                           \
+#define RNB_Q6_STEP(k)                                                                   \
+    {                                                                                    \
+        const uint32_t u0 = (r.A.k & 0x0f0f0f0fu) | ((r.H.k & 0x03030303u) << 4);        \
+        const uint32_t u1 = (r.B.k & 0x0f0f0f0fu) | ((r.H.k & 0x0c0c0c0cu) << 2);        \
+        const uint32_t u2 = ((r.A.k >> 4) & 0x0f0f0f0fu) | (r.H.k & 0x30303030u);        \
+        const uint32_t u3 = ((r.B.k >> 4) & 0x0f0f0f0fu) | ((r.H.k & 0xc0c0c0c0u) >> 2); \
+        p0 = dot4(u0, a.a0.k, p0);                                                       \
+        p1 = dot4(u1, a.a1.k, p1);                                                       \
+        p2 = dot4(u2, a.a2.k, p2);                                                       \
+        p3 = dot4(u3, a.a3.k, p3);                                                       \
     }
-    RNB_Q6_STEP(A.x, B.x, H.x, a0.x, a1.x, a2.x, a3.x)
-    RNB_Q6_STEP(A.y, B.y, H.y, a0.y, a1.y, a2.y, a3.y)
+    RNB_Q6_STEP(x)
+    RNB_Q6_STEP(y)
+    RNB_Q6_STEP(z)
+    RNB_Q6_STEP(w)
 #undef RNB_Q6_STEP
-    const int sumi = s0 * p0 + s1 * p1 + s2 * p2 + s3 * p3;
-    return (d * dx) * static_cast<float>(sumi);
+    const int sumi = s0 * (p0 - 32 * a.s0) + s1 * (p1 - 32 * a.s1) + s2 * (p2 - 32 * a.s2) + s3 * (p3 - 32 * a.s3);
+    return (f16_bits_to_f32(r.d_bits) * a.dx) * static_cast<float>(sumi);
 }
 
 }  // namespace rnb

@@ -32,20 +32,32 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
 }
 
-// sum over the 64 lanes of a wave; every lane gets the total
+// Cross-lane sums on the DPP data path (no LDS traffic).  After seg_sum<W>(v) the LAST lane of every
+// aligned W-lane segment (W = 16, 32 or 64) holds the sum over that segment.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, kRowMask, 0xf, false);
+    return v + __builtin_bit_cast(float, t);
+}
+template <int kWidth>
+__device__ __forceinline__ float seg_sum(float v) {
+    static_assert(kWidth == 16 || kWidth == 32 || kWidth == 64, "segment width");
+    v = dpp_add<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xf>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xf>(v);  // row_mirror: all 16 lanes of a row hold the row sum
+    if (kWidth >= 32) v = dpp_add<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
+    if (kWidth >= 64) v = dpp_add<0x143, 0xc>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+// sum over the 64 lanes of a wave through the LDS crossbar; every lane gets the total
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     return v;
 }
 
-// sum over aligned groups of `width` lanes (width a power of two <= 64)
-template <int width>
-__device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
 template <int width>
 __device__ __forceinline__ int group_sum_i(int v) {
 #pragma unroll

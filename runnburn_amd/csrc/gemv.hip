@@ -5,11 +5,13 @@
 //  Q8_0 x Q8   : crates/rnb-cpu/src/gemm/neon_dot.rs:376-436   (dot_q8_0_q8_neon)
 //  driver      : crates/rnb-cpu/src/gemm/quant_gemv.rs:403-536, out[s*rows + row]
 //
-// These kernels are HBM-bound: every weight byte is read exactly once, with 8- or 16-byte loads
-// per lane that tile each row contiguously.  A wave64 owns a row; groups of 8 lanes own a
-// 256-element super-block (1 lane owns a 32-element Q8_0 block).  Integer sums per lane are exact
-// (v_dot4_i32_i8); the per-block f32 scale is applied once per lane and the 64 partial sums are
-// added across the wave, so results differ from the scalar reference only by f32 summation order.
+// These kernels are HBM-bound: every weight byte is fetched once with 16-byte loads.  Four lanes own
+// a 256-element super-block, so a wave64 pass covers 16 super-blocks: one 4096-wide row, or two /
+// four shorter rows side by side (kRowsPerWave).  About 4096 waves are launched in total (16 per CU)
+// and each walks several rows, so the quantised activation of a lane's K-slice is loaded into
+// registers once per wave instead of once per row.  Integer sums per lane are exact
+// (v_dot4_i32_i8); the per-block f32 scale is applied once per lane and the partial sums are added
+// across lanes on the DPP path, so results differ from the scalar reference only by f32 summation order.
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
@@ -18,102 +20,183 @@ namespace rnb {
 
 namespace {
 
-constexpr int kRowsPerWg = 4;  // one wave per row
+constexpr int kWavesPerWg = 4;
+constexpr uint32_t kTargetWaves = 4096;  // total waves per launch: enough loads in flight, short tail
 
-__global__ void __launch_bounds__(kWave *kRowsPerWg)
-    gemv_q4k_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                    const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb) {
+// ---------------------------------------------------------------------------------------------
+// K-quant GEMV (Q4_K and Q6_K share the structure; only the block functions differ)
+// ---------------------------------------------------------------------------------------------
+template <bool kQ6, int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_kquant_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                       const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                       uint32_t row_groups) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
+    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t row = blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
     const uint32_t tok = blockIdx.y;
-    if (row >= rows) return;
-    const uint8_t *rowp = w + static_cast<size_t>(row) * nb * kQ4KBytes;
     const size_t abase = static_cast<size_t>(tok) * nb;
-    const int c = lane & 7;
-    float acc = 0.0f;
-    for (uint32_t b = lane >> 3; b < nb; b += 8) {
-        acc += q4k_block_partial(rowp + static_cast<size_t>(b) * kQ4KBytes, aq + (abase + b) * 256, ad[abase + b],
-                                 abs + (abase + b) * 16, c);
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+
+    if (nb <= kBlocksPerPass) {
+        // the whole row fits one pass: this lane's activation slice stays in registers for every row
+        const bool has_block = bslot < nb;
+        const size_t ab = abase + (has_block ? bslot : 0);
+        Q4KAct a4{};
+        Q6KAct a6{};
+        if constexpr (kQ6)
+            a6 = q6k_load_act(aq + ab * 256, ad[ab], g);
+        else
+            a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+        for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
+            const uint32_t row = grp * kRowsPerWave + rsel;
+            float acc = 0.0f;
+            if (has_block && row < rows) {
+                const uint8_t *blk = w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kBlockBytes;
+                if constexpr (kQ6)
+                    acc = q6k_partial(q6k_load_block(blk, g), a6, g);
+                else
+                    acc = q4k_partial(q4k_load_block(blk, g), a4, g);
+            }
+            acc = seg_sum<kLanesPerRow>(acc);
+            if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
+        }
+    } else {
+        for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
+            const uint32_t row = grp * kRowsPerWave + rsel;
+            float acc = 0.0f;
+            if (row < rows) {
+                const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+                for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
+                    const uint8_t *blk = rowp + static_cast<size_t>(b) * kBlockBytes;
+                    const size_t ab = abase + b;
+                    if constexpr (kQ6)
+                        acc += q6k_partial(q6k_load_block(blk, g), q6k_load_act(aq + ab * 256, ad[ab], g), g);
+                    else
+                        acc += q4k_partial(q4k_load_block(blk, g), q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g), g);
+                }
+            }
+            acc = seg_sum<kLanesPerRow>(acc);
+            if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
+        }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) out[static_cast<size_t>(tok) * rows + row] = acc;
 }
 
-__global__ void __launch_bounds__(kWave *kRowsPerWg)
-    gemv_q6k_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                    float *__restrict__ out, uint32_t rows, uint32_t nb) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t row = blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
-    const uint32_t tok = blockIdx.y;
-    if (row >= rows) return;
-    const uint8_t *rowp = w + static_cast<size_t>(row) * nb * kQ6KBytes;
-    const size_t abase = static_cast<size_t>(tok) * nb;
-    const int sub = lane & 7;
-    float acc = 0.0f;
-    for (uint32_t b = lane >> 3; b < nb; b += 8) {
-        acc += q6k_block_partial(rowp + static_cast<size_t>(b) * kQ6KBytes, aq + (abase + b) * 256, ad[abase + b], sub);
-    }
-    acc = wave_sum(acc);
-    if (lane == 0) out[static_cast<size_t>(tok) * rows + row] = acc;
+template <bool kQ6, int kRowsPerWave>
+void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                   hipStream_t stream) {
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    hipLaunchKernelGGL((gemv_kquant_kernel<kQ6, kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
+                       act.d, act.bsums, out, rows, nb, row_groups);
+}
+
+template <bool kQ6>
+void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                       hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    if (nb <= 4)
+        launch_kquant<kQ6, 4>(w, act, out, rows, nb, seq, stream);
+    else if (nb <= 8)
+        launch_kquant<kQ6, 2>(w, act, out, rows, nb, seq, stream);
+    else
+        launch_kquant<kQ6, 1>(w, act, out, rows, nb, seq, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
-// Q8_0: block = {f16 d, i8 qs[32]}, 34 bytes, 2-byte aligned.  One lane per block.
+// Q8_0: block = {f16 d, i8 qs[32]}, 34 bytes, 2-byte aligned.  One lane per block: two 16-byte loads
+// at 2-byte alignment.  Rows of up to 128 blocks (K <= 4096) keep the lane's two activation blocks
+// in registers across rows.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(kWave *kRowsPerWg)
+struct Q8Act {
+    uint4 a0, a1;
+    float dx;
+};
+
+__device__ __forceinline__ Q8Act q8_load_act(const int8_t *__restrict__ aq_blk, float dx) {
+    Q8Act a;
+    a.a0 = *reinterpret_cast<const uint4 *>(aq_blk);
+    a.a1 = *reinterpret_cast<const uint4 *>(aq_blk + 16);
+    a.dx = dx;
+    return a;
+}
+
+__device__ __forceinline__ float q8_0_partial(const uint8_t *__restrict__ blk, const Q8Act &a) {
+    const float d = ld_f16(blk);
+    const uint4 q0 = ld_u4_a2(blk + 2), q1 = ld_u4_a2(blk + 18);
+    int p = 0;
+    p = dot4(q0.x, a.a0.x, p);
+    p = dot4(q0.y, a.a0.y, p);
+    p = dot4(q0.z, a.a0.z, p);
+    p = dot4(q0.w, a.a0.w, p);
+    p = dot4(q1.x, a.a1.x, p);
+    p = dot4(q1.y, a.a1.y, p);
+    p = dot4(q1.z, a.a1.z, p);
+    p = dot4(q1.w, a.a1.w, p);
+    return (d * a.dx) * static_cast<float>(p);
+}
+
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                      float *__restrict__ out, uint32_t rows, uint32_t nb32) {
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t row = blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
     const uint32_t tok = blockIdx.y;
-    if (row >= rows) return;
-    const uint8_t *rowp = w + static_cast<size_t>(row) * nb32 * kQ8_0Bytes;
     const size_t abase = static_cast<size_t>(tok) * nb32;
-    float acc = 0.0f;
-    for (uint32_t b = lane; b < nb32; b += kWave) {
-        const uint8_t *blk = rowp + static_cast<size_t>(b) * kQ8_0Bytes;
-        const float d = ld_f16(blk);
-        const uint4 q0 = ld_u4_a2(blk + 2), q1 = ld_u4_a2(blk + 18);
-        const uint4 a0 = *reinterpret_cast<const uint4 *>(aq + (abase + b) * 32);
-        const uint4 a1 = *reinterpret_cast<const uint4 *>(aq + (abase + b) * 32 + 16);
-        int p = 0;
-        p = dot4(q0.x, a0.x, p);
-        p = dot4(q0.y, a0.y, p);
-        p = dot4(q0.z, a0.z, p);
-        p = dot4(q0.w, a0.w, p);
-        p = dot4(q1.x, a1.x, p);
-        p = dot4(q1.y, a1.y, p);
-        p = dot4(q1.z, a1.z, p);
-        p = dot4(q1.w, a1.w, p);
-        acc += (d * ad[abase + b]) * static_cast<float>(p);
+    const size_t row_bytes = static_cast<size_t>(nb32) * kQ8_0Bytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    if (nb32 <= 2 * kWave) {
+        const uint32_t b0 = lane, b1 = lane + kWave;
+        const bool has0 = b0 < nb32, has1 = b1 < nb32;
+        const Q8Act a0 = q8_load_act(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
+        const Q8Act a1 = q8_load_act(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
+        for (uint32_t row = wave_global; row < rows; row += n_waves) {
+            const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+            float acc = 0.0f;
+            if (has0) acc = q8_0_partial(rowp + static_cast<size_t>(b0) * kQ8_0Bytes, a0);
+            if (has1) acc += q8_0_partial(rowp + static_cast<size_t>(b1) * kQ8_0Bytes, a1);
+            acc = seg_sum<kWave>(acc);
+            if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
+        }
+    } else {
+        for (uint32_t row = wave_global; row < rows; row += n_waves) {
+            const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+            float acc = 0.0f;
+            for (uint32_t b = lane; b < nb32; b += kWave)
+                acc += q8_0_partial(rowp + static_cast<size_t>(b) * kQ8_0Bytes,
+                                    q8_load_act(aq + (abase + b) * 32, ad[abase + b]));
+            acc = seg_sum<kWave>(acc);
+            if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
+        }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) out[static_cast<size_t>(tok) * rows + row] = acc;
 }
-
-inline dim3 gemv_grid(uint32_t rows, uint32_t seq) { return dim3((rows + kRowsPerWg - 1) / kRowsPerWg, seq, 1); }
 
 }  // namespace
 
 void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
-    if (rows == 0 || seq == 0) return;
-    hipLaunchKernelGGL(gemv_q4k_kernel, gemv_grid(rows, seq), dim3(kWave * kRowsPerWg), 0, stream, w, act.qs, act.d,
-                       act.bsums, out, rows, nb);
+    launch_kquant_any<false>(w, act, out, rows, nb, seq, stream);
 }
 
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
-    if (rows == 0 || seq == 0) return;
-    hipLaunchKernelGGL(gemv_q6k_kernel, gemv_grid(rows, seq), dim3(kWave * kRowsPerWg), 0, stream, w, act.qs, act.d,
-                       out, rows, nb);
+    launch_kquant_any<true>(w, act, out, rows, nb, seq, stream);
 }
 
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,
                       hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
-    hipLaunchKernelGGL(gemv_q8_0_kernel, gemv_grid(rows, seq), dim3(kWave * kRowsPerWg), 0, stream, w, act.qs, act.d,
-                       out, rows, nb32);
+    const uint32_t waves = rows < kTargetWaves ? rows : kTargetWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    hipLaunchKernelGGL(gemv_q8_0_kernel, grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, act.d, out, rows, nb32);
 }
 
 }  // namespace rnb

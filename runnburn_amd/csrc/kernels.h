@@ -42,18 +42,21 @@ void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t ro
                           uint32_t seq, hipStream_t stream);
 
 // ---- gathered sparse-MoE ------------------------------------------------------------------
-struct MoeSlots {
-    const uint32_t *expert;  // [n_slots] device
-    const uint32_t *token;   // [n_slots] device
-    const float *route;      // [n_slots] device
-    uint32_t n_slots;
+// Slots grouped by expert (device arrays).  Group i covers sorted positions [start[i], start[i+1]);
+// sorted_slot[p] is the caller's slot index at sorted position p, sorted_token[p] its token.
+struct MoeGroups {
+    const uint32_t *expert;        // [n_groups]
+    const uint32_t *start;         // [n_groups + 1]
+    const uint32_t *sorted_slot;   // [n_slots]
+    const uint32_t *sorted_token;  // [n_slots]
+    uint32_t n_groups;
 };
 // mid[slot][n_ff] = silu(Wg[e] . h_tok) * (Wu[e] . h_tok); act = Q8_K(x) per token
-void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeSlots slots,
-                        float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
-// slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot]))
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeSlots slots,
-                     float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
+void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
+                        uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
+// slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])); mid_act is indexed by slot
+void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+                     const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // out[token][n_embd] = sum of slot_out over the token's slots, in list order;
 // tok_offsets [token_count+1], tok_slots [n_slots] (CSR built by the host)
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,

@@ -5,8 +5,13 @@
 // following crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:260-327
 // (compute_expert_host_from_slices), crates/rnb-cpu/src/kernels/activation.rs:73-89
 // (fused_silu_mul_inplace) and .../shared_expert_moe/prefill_cpu.rs:167-194 (ordered reduce).
-// Expert weights are never copied: a slot addresses its expert as base + e * bytes_per_expert,
-// the slicing of fanout.rs:4-22.
+//
+// Expert weights are never copied: an expert is base + e * bytes_per_expert, the slicing of
+// fanout.rs:4-22.  Slots are grouped by expert (the expert-major order of prefill_cpu.rs:113-146):
+// a workgroup owns a tile of rows of ONE expert, stages the quantised activations of that expert's
+// tokens in LDS, then every wave keeps a row's packed blocks in registers and walks the tokens, so
+// an expert's weights are streamed from HBM once however many tokens were routed to it.  A decode
+// call (one token) is the same kernel with one token per group.
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
@@ -15,63 +20,184 @@ namespace rnb {
 
 namespace {
 
-constexpr int kRowsPerWg = 4;
+constexpr int kWavesPerWg = 4;
+constexpr int kMaxChunkTokens = 8;  // tokens staged in LDS at a time
 
-__global__ void __launch_bounds__(kWave *kRowsPerWg)
+// LDS staging of `nt` quantised activation rows: qs [nt][nb*256] | d [nt][nb] | bsums [nt][nb*16]
+struct Staged {
+    const int8_t *qs;
+    const float *d;
+    const int16_t *bsums;
+};
+
+__host__ __device__ __forceinline__ size_t stage_d_offset(uint32_t tmax, uint32_t nb) {
+    return static_cast<size_t>(tmax) * nb * 256;
+}
+__host__ __device__ __forceinline__ size_t stage_bsums_offset(uint32_t tmax, uint32_t nb) {
+    return stage_d_offset(tmax, nb) + ((static_cast<size_t>(tmax) * nb * 4 + 15) & ~static_cast<size_t>(15));
+}
+__host__ __device__ __forceinline__ size_t stage_bytes(uint32_t tmax, uint32_t nb) {
+    return stage_bsums_offset(tmax, nb) + static_cast<size_t>(tmax) * nb * 32;
+}
+
+__device__ __forceinline__ Staged stage_layout(uint8_t *lds, uint32_t tmax, uint32_t nb) {
+    Staged s;
+    s.qs = reinterpret_cast<const int8_t *>(lds);
+    s.d = reinterpret_cast<const float *>(lds + stage_d_offset(tmax, nb));
+    s.bsums = reinterpret_cast<const int16_t *>(lds + stage_bsums_offset(tmax, nb));
+    return s;
+}
+
+// copies activation row `src_row` (global, SoA) into staging slot t
+__device__ __forceinline__ void stage_row(uint8_t *lds, uint32_t tmax, uint32_t nb, uint32_t t, size_t src_row,
+                                          const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                          const int16_t *__restrict__ abs) {
+    uint4 *dq = reinterpret_cast<uint4 *>(lds + static_cast<size_t>(t) * nb * 256);
+    const uint4 *sq = reinterpret_cast<const uint4 *>(aq + src_row * nb * 256);
+    for (uint32_t i = threadIdx.x; i < nb * 16; i += blockDim.x) dq[i] = sq[i];
+    float *dd = reinterpret_cast<float *>(lds + stage_d_offset(tmax, nb)) + static_cast<size_t>(t) * nb;
+    for (uint32_t i = threadIdx.x; i < nb; i += blockDim.x) dd[i] = ad[src_row * nb + i];
+    uint4 *db = reinterpret_cast<uint4 *>(lds + stage_bsums_offset(tmax, nb)) + static_cast<size_t>(t) * nb * 2;
+    const uint4 *sb = reinterpret_cast<const uint4 *>(abs + src_row * nb * 16);
+    for (uint32_t i = threadIdx.x; i < nb * 2; i += blockDim.x) db[i] = sb[i];
+}
+
+// ---------------------------------------------------------------------------------------------
+// gate + up + SiLU*up.  Grid (row tiles, expert groups).  kRowsPerWave rows side by side per wave.
+// ---------------------------------------------------------------------------------------------
+template <int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_gate_up_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
                        const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ abs,
-                       const uint32_t *__restrict__ slot_expert, const uint32_t *__restrict__ slot_token,
-                       float *__restrict__ mid, uint32_t n_ff, uint32_t nb) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t row = blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
-    const uint32_t slot = blockIdx.y;
-    if (row >= n_ff) return;
+                       const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
+                       const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
+                       float *__restrict__ mid, uint32_t n_ff, uint32_t nb, uint32_t iters, uint32_t tmax) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const uint32_t grp = blockIdx.y;
+    const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
-    const size_t off = (static_cast<size_t>(slot_expert[slot]) * n_ff + row) * row_bytes;
-    const size_t abase = static_cast<size_t>(slot_token[slot]) * nb;
-    const int c = lane & 7;
-    float gacc = 0.0f, uacc = 0.0f;
-    for (uint32_t b = lane >> 3; b < nb; b += 8) {
-        const size_t boff = off + static_cast<size_t>(b) * kQ4KBytes;
-        const int8_t *a = aq + (abase + b) * 256;
-        const int16_t *bs = abs + (abase + b) * 16;
-        const float dx = ad[abase + b];
-        gacc += q4k_block_partial(gate_all + boff, a, dx, bs, c);
-        uacc += q4k_block_partial(up_all + boff, a, dx, bs, c);
-    }
-    gacc = wave_sum(gacc);
-    uacc = wave_sum(uacc);
-    if (lane == 0) {
-        // crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up
-        const float e = expf(-gacc);
-        mid[static_cast<size_t>(slot) * n_ff + row] = (gacc / (1.0f + e)) * uacc;
+    const size_t ebase = static_cast<size_t>(expert) * n_ff * row_bytes;
+    const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
+    const Staged st = stage_layout(lds, tmax, nb);
+
+    for (uint32_t c0 = 0; c0 < count; c0 += tmax) {
+        const uint32_t nt = min(tmax, count - c0);
+        if (c0) __syncthreads();
+        for (uint32_t t = 0; t < nt; t++) stage_row(lds, tmax, nb, t, sorted_token[start + c0 + t], aq, ad, abs);
+        __syncthreads();
+        for (uint32_t it = 0; it < iters; it++) {
+            const uint32_t row = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave + rsel;
+            const bool row_ok = row < n_ff;
+            float gacc[kMaxChunkTokens], uacc[kMaxChunkTokens];
+#pragma unroll
+            for (int t = 0; t < kMaxChunkTokens; t++) gacc[t] = uacc[t] = 0.0f;
+            for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
+                if (!row_ok) break;
+                const size_t off = ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kQ4KBytes;
+                const Q4KRegs gr = q4k_load_block(gate_all + off, g);
+                const Q4KRegs ur = q4k_load_block(up_all + off, g);
+#pragma unroll
+                for (int t = 0; t < kMaxChunkTokens; t++) {
+                    if (static_cast<uint32_t>(t) < nt) {
+                        const size_t ab = static_cast<size_t>(t) * nb + b;
+                        const Q4KAct a = q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g);
+                        gacc[t] += q4k_partial(gr, a, g);
+                        uacc[t] += q4k_partial(ur, a, g);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < kMaxChunkTokens; t++) {
+                if (static_cast<uint32_t>(t) < nt) {  // nt is workgroup-uniform
+                    const float gs = seg_sum<kLanesPerRow>(gacc[t]);
+                    const float us = seg_sum<kLanesPerRow>(uacc[t]);
+                    if (sub == kLanesPerRow - 1 && row_ok) {
+                        // crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up
+                        const float e = expf(-gs);
+                        mid[static_cast<size_t>(sorted_slot[start + c0 + t]) * n_ff + row] = (gs / (1.0f + e)) * us;
+                    }
+                }
+            }
+        }
     }
 }
 
-template <bool kDownQ6>
-__global__ void __launch_bounds__(kWave *kRowsPerWg)
+// ---------------------------------------------------------------------------------------------
+// down projection of the re-quantised intermediate, scaled by the route weight.
+// ---------------------------------------------------------------------------------------------
+template <bool kQ6, int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_down_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
-                    const int16_t *__restrict__ mbs, const uint32_t *__restrict__ slot_expert,
-                    const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t row = blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
-    const uint32_t slot = blockIdx.y;
-    if (row >= n_embd) return;
-    const size_t blk_bytes = kDownQ6 ? kQ6KBytes : kQ4KBytes;
-    const size_t row_bytes = static_cast<size_t>(nb) * blk_bytes;
-    const uint8_t *rowp = down_all + (static_cast<size_t>(slot_expert[slot]) * n_embd + row) * row_bytes;
-    const size_t abase = static_cast<size_t>(slot) * nb;
-    const int sub = lane & 7;
-    float acc = 0.0f;
-    for (uint32_t b = lane >> 3; b < nb; b += 8) {
-        if (kDownQ6)
-            acc += q6k_block_partial(rowp + static_cast<size_t>(b) * blk_bytes, mq + (abase + b) * 256, md[abase + b], sub);
-        else
-            acc += q4k_block_partial(rowp + static_cast<size_t>(b) * blk_bytes, mq + (abase + b) * 256, md[abase + b],
-                               mbs + (abase + b) * 16, sub);
+                    const int16_t *__restrict__ mbs, const uint32_t *__restrict__ grp_expert,
+                    const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
+                    const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
+                    uint32_t iters, uint32_t tmax) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
+    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const uint32_t grp = blockIdx.y;
+    const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const size_t ebase = static_cast<size_t>(expert) * n_embd * row_bytes;
+    const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
+    const Staged st = stage_layout(lds, tmax, nb);
+
+    for (uint32_t c0 = 0; c0 < count; c0 += tmax) {
+        const uint32_t nt = min(tmax, count - c0);
+        if (c0) __syncthreads();
+        for (uint32_t t = 0; t < nt; t++) stage_row(lds, tmax, nb, t, sorted_slot[start + c0 + t], mq, md, mbs);
+        __syncthreads();
+        for (uint32_t it = 0; it < iters; it++) {
+            const uint32_t row = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave + rsel;
+            const bool row_ok = row < n_embd;
+            float acc[kMaxChunkTokens];
+#pragma unroll
+            for (int t = 0; t < kMaxChunkTokens; t++) acc[t] = 0.0f;
+            for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
+                if (!row_ok) break;
+                const uint8_t *blk = down_all + ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
+                Q4KRegs r4{};
+                Q6KRegs r6{};
+                if constexpr (kQ6)
+                    r6 = q6k_load_block(blk, g);
+                else
+                    r4 = q4k_load_block(blk, g);
+#pragma unroll
+                for (int t = 0; t < kMaxChunkTokens; t++) {
+                    if (static_cast<uint32_t>(t) < nt) {
+                        const size_t ab = static_cast<size_t>(t) * nb + b;
+                        if constexpr (kQ6)
+                            acc[t] += q6k_partial(r6, q6k_load_act(st.qs + ab * 256, st.d[ab], g), g);
+                        else
+                            acc[t] += q4k_partial(r4, q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g), g);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < kMaxChunkTokens; t++) {
+                if (static_cast<uint32_t>(t) < nt) {
+                    const float s = seg_sum<kLanesPerRow>(acc[t]);
+                    if (sub == kLanesPerRow - 1 && row_ok) {
+                        const uint32_t slot = sorted_slot[start + c0 + t];
+                        slot_out[static_cast<size_t>(slot) * n_embd + row] = s * slot_route[slot];  // fanout.rs:306-308
+                    }
+                }
+            }
+        }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) slot_out[static_cast<size_t>(slot) * n_embd + row] = acc * slot_route[slot];  // fanout.rs:306-308
 }
 
 __global__ void __launch_bounds__(256)
@@ -86,26 +212,69 @@ __global__ void __launch_bounds__(256)
     out[static_cast<size_t>(tok) * n_embd + i] = acc;
 }
 
-}  // namespace
+struct TilePlan {
+    uint32_t iters, tmax, tiles;
+    size_t lds_bytes;
+};
 
-void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeSlots slots, float *mid,
-                        uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
-    if (slots.n_slots == 0) return;
-    dim3 grid((n_ff + kRowsPerWg - 1) / kRowsPerWg, slots.n_slots, 1);
-    hipLaunchKernelGGL(moe_gate_up_kernel, grid, dim3(kWave * kRowsPerWg), 0, stream, gate_all, up_all, act.qs, act.d,
-                       act.bsums, slots.expert, slots.token, mid, n_ff, nb_in);
+// rows per workgroup = 4 waves * rows_per_wave * iters; keep >= ~2048 workgroups in flight when the
+// problem allows it, and at most 48 KiB of staged activations
+TilePlan plan_tiles(uint32_t rows, uint32_t nb, uint32_t n_groups, int rows_per_wave) {
+    TilePlan p;
+    const uint32_t per_pass = kWavesPerWg * static_cast<uint32_t>(rows_per_wave);
+    const uint64_t passes_total = static_cast<uint64_t>((rows + per_pass - 1) / per_pass) * n_groups;
+    uint32_t iters = static_cast<uint32_t>(passes_total / 2048);
+    p.iters = iters < 1 ? 1 : (iters > 8 ? 8 : iters);
+    const size_t per_token = static_cast<size_t>(nb) * 292;
+    uint32_t tmax = static_cast<uint32_t>((48 * 1024) / per_token);
+    p.tmax = tmax < 1 ? 1 : (tmax > kMaxChunkTokens ? kMaxChunkTokens : tmax);
+    p.lds_bytes = stage_bytes(p.tmax, nb);
+    p.tiles = (rows + per_pass * p.iters - 1) / (per_pass * p.iters);
+    return p;
 }
 
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeSlots slots, float *slot_out,
-                     uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
-    if (slots.n_slots == 0) return;
-    dim3 grid((n_embd + kRowsPerWg - 1) / kRowsPerWg, slots.n_slots, 1);
-    if (down_quant == kQ6K)
-        hipLaunchKernelGGL(moe_down_kernel<true>, grid, dim3(kWave * kRowsPerWg), 0, stream, down_all, mid_act.qs,
-                           mid_act.d, mid_act.bsums, slots.expert, slots.route, slot_out, n_embd, nb_mid);
+int rows_per_wave_for(uint32_t nb) { return nb <= 4 ? 4 : (nb <= 8 ? 2 : 1); }
+
+}  // namespace
+
+void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
+                        uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
+    if (groups.n_groups == 0) return;
+    const int rpw = rows_per_wave_for(nb_in);
+    const TilePlan p = plan_tiles(n_ff, nb_in, groups.n_groups, rpw);
+    const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
+#define RNB_LAUNCH_GU(R)                                                                                             \
+    hipLaunchKernelGGL(moe_gate_up_kernel<R>, grid, block, p.lds_bytes, stream, gate_all, up_all, act.qs, act.d,      \
+                       act.bsums, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff,   \
+                       nb_in, p.iters, p.tmax)
+    if (rpw == 4)
+        RNB_LAUNCH_GU(4);
+    else if (rpw == 2)
+        RNB_LAUNCH_GU(2);
     else
-        hipLaunchKernelGGL(moe_down_kernel<false>, grid, dim3(kWave * kRowsPerWg), 0, stream, down_all, mid_act.qs,
-                           mid_act.d, mid_act.bsums, slots.expert, slots.route, slot_out, n_embd, nb_mid);
+        RNB_LAUNCH_GU(1);
+#undef RNB_LAUNCH_GU
+}
+
+void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+                     const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
+    if (groups.n_groups == 0) return;
+    const int rpw = rows_per_wave_for(nb_mid);
+    const TilePlan p = plan_tiles(n_embd, nb_mid, groups.n_groups, rpw);
+    const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
+#define RNB_LAUNCH_DOWN(Q6, R)                                                                                       \
+    hipLaunchKernelGGL((moe_down_kernel<Q6, R>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d,   \
+                       mid_act.bsums, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, \
+                       nb_mid, p.iters, p.tmax)
+    const bool q6 = down_quant == kQ6K;
+    if (rpw == 4) {
+        if (q6) RNB_LAUNCH_DOWN(true, 4); else RNB_LAUNCH_DOWN(false, 4);
+    } else if (rpw == 2) {
+        if (q6) RNB_LAUNCH_DOWN(true, 2); else RNB_LAUNCH_DOWN(false, 2);
+    } else {
+        if (q6) RNB_LAUNCH_DOWN(true, 1); else RNB_LAUNCH_DOWN(false, 1);
+    }
+#undef RNB_LAUNCH_DOWN
 }
 
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots, float *out,

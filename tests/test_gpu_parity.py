@@ -230,6 +230,27 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
     assert rnb.q4k_gemv_batch(np.zeros(144, np.uint8), 1, 256, np.zeros(0, np.float32)).shape == (0, 1)
 
 
+@pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q4_K, 77, 2048), (Q4_K, 50, 768), (Q6_K, 300, 4096),
+                                             (Q6_K, 64, 768), (Q8_0, 200, 4096), (Q8_0, 33, 1056), (Q6_K, 40, 14336)])
+def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
+    """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
+    feed several matrices from one activation) run the same arithmetic: identical bits."""
+    w = oracle.make_weights(quant, rows, cols, 900 + rows)
+    x = oracle.fill_normal(cols, 901 + cols, 1.0)
+    wd, xd = rnb.DeviceBuffer.from_host(w), rnb.DeviceBuffer.from_host(x)
+    o1, o2 = rnb.DeviceBuffer(rows * 4), rnb.DeviceBuffer(rows * 4)
+    rnb.gemv_dev(quant, wd, rows, cols, xd, 1, o1)
+    rnb.quantize_dev(quant, xd, 1, cols)
+    rnb.gemv_quantized_dev(quant, wd, rows, cols, 1, o2)
+    rnb.sync()
+    a, b = o1.to_host(np.float32), o2.to_host(np.float32)
+    assert np.array_equal(a, b)
+    check_close(a, oracle.gemv(quant, w, rows, cols, x)[0], oracle.gemv(quant, w, rows, cols, x, gold=True)[0],
+                f"device-resident decode quant {quant} {rows}x{cols}")
+    for buf in (wd, xd, o1, o2):
+        buf.free()
+
+
 # ---- batches: seq-major layout, ragged token counts ----------------------------------------------
 
 @pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
