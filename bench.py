@@ -139,6 +139,7 @@ class Hip:
         self.rt.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
         self.rt.hipGraphExecDestroy.argtypes = [C.c_void_p]
         self.rt.hipGraphDestroy.argtypes = [C.c_void_p]
+        self.rt.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
 
     def check(self, rc, what):
         if rc != 0:
@@ -172,6 +173,29 @@ def kernel_time_ms(hip, stream, launch, n):
     hip.rt.hipEventDestroy(e0)
     hip.rt.hipEventDestroy(e1)
     return ms / n
+
+
+def calibration_copy(hip, rnb, stream, nbytes=64 << 20, reps=5):
+    """A plain device-to-device copy of known size (the runtime's copy kernel): the reference point that the
+    FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run are scaled by."""
+    src, dst = rnb.DeviceBuffer(nbytes), rnb.DeviceBuffer(nbytes)
+    for _ in range(reps):
+        hip.check(hip.rt.hipMemcpyAsync(dst.ptr, src.ptr, nbytes, 3, stream), "hipMemcpyAsync")  # 3 = device to device
+    rnb.sync()
+    src.free()
+    dst.free()
+    log(f"calibration copy: {reps} x {nbytes} bytes device-to-device")
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel`, from the committed counter summary (two rocprofv3 --pmc runs, FETCH_SIZE and
+    WRITE_SIZE, each scaled by the same counter's reading for the calibration copy); None when absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "gemv_q4k_cfg2_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel, {}).get("traffic_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
 
 
 def wall_steps(rnb, step, n):
@@ -347,6 +371,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--quick", action="store_true", help="headline config only (skip the secondary configs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a 64 MiB device-to-device copy (reference for FETCH_SIZE / WRITE_SIZE under --pmc)")
     ap.add_argument("--cache-resident", action="store_true",
                     help="also time each kernel on ONE weight copy (may be served by the Infinity Cache)")
     args = ap.parse_args()
@@ -364,6 +390,8 @@ def main() -> int:
     stream = C.c_void_p(rnb.stream_handle())
     log(f"device: {rnb.device_name()}")
 
+    if args.calibration_copy:
+        calibration_copy(hip, rnb, stream)
     rows, cols = 14336, 4096
     main_res, w_host, x, gpu_out = bench_matmul(rnb, hip, stream, Q4_K, rows, cols, 1, args.steps, args.warmup, 20240607,
                                                 "cfg2 q4k gemv", cache_resident=args.cache_resident)
@@ -390,7 +418,8 @@ def main() -> int:
                    "stream_ms_per_step": main_res["wall_ms_per_step"],
                    "graph_ms_per_step": main_res.get("graph_ms_per_step")},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "gemv_q4k_kernel",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("gemv_kquant_kernel<false,1>"),
+                     "kernel": "gemv_kquant_kernel<false,1>",
                      "bytes_per_launch": nbytes, "kernel_ms_mean": main_res["kernel_ms_mean"],
                      "kernel_ms_runs": main_res["kernel_ms_runs"],
                      "timing": "HIP events around back-to-back launches on the library stream, 3 runs"},

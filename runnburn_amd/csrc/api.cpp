@@ -232,8 +232,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                 size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
                 const float *x_dev, float *out_dev) {
     if (token_count == 0) return RNB_HIP_OK;
-    // host tables (one upload): route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] |
-    // grp_expert[G] | grp_start[G+1]; slots are grouped by expert, keeping slot order inside a group
+    // slots are grouped by expert, keeping slot order inside a group
     std::vector<uint32_t> order(n_slots);
     for (size_t i = 0; i < n_slots; i++) order[i] = static_cast<uint32_t>(i);
     std::stable_sort(order.begin(), order.end(),
@@ -247,16 +246,31 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     }
     grp_start.push_back(static_cast<uint32_t>(n_slots));
     const size_t n_groups = grp_expert.size();
+    // one table image: route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] | grp_expert[G] |
+    // grp_start[G+1]
     const size_t table_words = 4 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
-    HIP_TRY(s.bounce_tables.reserve(table_words * 4));
+    const bool inline_tables = table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
+    MoeInlineTables inl;
+    uint32_t *h = inl.words;
+    TableSlot *ring_slot = nullptr;
+    if (!inline_tables) {
+        // larger tables go through one of a ring of pinned buffers, so that a call never waits for the
+        // previous call's upload to drain
+        ring_slot = &s.table_ring[s.table_ring_next];
+        s.table_ring_next = (s.table_ring_next + 1) % State::kTableRing;
+        if (ring_slot->event == nullptr)
+            HIP_TRY(hipEventCreateWithFlags(&ring_slot->event, hipEventDisableTiming));
+        else
+            HIP_TRY(hipEventSynchronize(ring_slot->event));
+        HIP_TRY(ring_slot->host.reserve(table_words * 4));
+        h = ring_slot->host.as<uint32_t>();
+    }
     HIP_TRY(s.moe_tables.reserve(table_words * 4));
-    uint32_t *h = s.bounce_tables.as<uint32_t>();
     float *h_route = reinterpret_cast<float *>(h);
     uint32_t *h_off = h + n_slots, *h_list = h_off + token_count + 1;
     uint32_t *h_sslot = h_list + n_slots, *h_stok = h_sslot + n_slots;
     uint32_t *h_gexp = h_stok + n_slots, *h_gstart = h_gexp + n_groups;
-    HIP_TRY(hipStreamSynchronize(s.stream));  // the previous call's table upload must have drained
-    std::memcpy(h_route, route, n_slots * 4);
+    if (n_slots) std::memcpy(h_route, route, n_slots * 4);
     std::vector<uint32_t> counts(token_count + 1, 0);
     for (size_t i = 0; i < n_slots; i++) counts[token_ids[i] + 1]++;
     for (size_t t = 0; t < token_count; t++) counts[t + 1] += counts[t];
@@ -269,22 +283,40 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     if (n_groups) std::memcpy(h_gexp, grp_expert.data(), n_groups * 4);
     std::memcpy(h_gstart, grp_start.data(), (n_groups + 1) * 4);
     uint32_t *d = s.moe_tables.as<uint32_t>();
-    HIP_TRY(hipMemcpyAsync(d, h, table_words * 4, hipMemcpyHostToDevice, s.stream));
-    s.h2d_bytes += table_words * 4;
+    if (ring_slot) {
+        HIP_TRY(hipMemcpyAsync(d, h, table_words * 4, hipMemcpyHostToDevice, s.stream));
+        HIP_TRY(hipEventRecord(ring_slot->event, s.stream));
+        s.h2d_bytes += table_words * 4;
+    }
     const float *d_route = reinterpret_cast<const float *>(d);
     const uint32_t *d_off = d + n_slots, *d_list = d_off + token_count + 1;
     const MoeGroups groups{d_list + 3 * n_slots, d_list + 3 * n_slots + n_groups, d_list + n_slots, d_list + 2 * n_slots,
                            static_cast<uint32_t>(n_groups)};
 
+    ActView act;
+    if (inline_tables) {
+        // quantise x and drop the tables into device memory with the same launch
+        const size_t nq = token_count * n_embd;
+        HIP_TRY(s.act_qs.reserve(nq));
+        HIP_TRY(s.act_d.reserve(nq / 256 * sizeof(float)));
+        HIP_TRY(s.act_bsums.reserve(nq / 256 * 16 * sizeof(int16_t)));
+        launch_quantize_q8k_with_tables(x_dev, nq / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(),
+                                        s.act_bsums.as<int16_t>(), inl, static_cast<uint32_t>(table_words), d, s.stream);
+        HIP_TRY(hipGetLastError());
+        act = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
+        s.act_family = kQ4K;
+        s.act_seq = token_count;
+        s.act_cols = n_embd;
+    } else {
+        int st = quantize_activations(s, kQ4K, x_dev, token_count, n_embd, &act);
+        if (st != RNB_HIP_OK) return st;
+    }
     if (n_slots == 0) {  // nothing routed: the reduce kernel alone writes the zero rows
         launch_moe_reduce(nullptr, d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
         HIP_TRY(hipGetLastError());
         return RNB_HIP_OK;
     }
-    ActView act;
-    int st = quantize_activations(s, kQ4K, x_dev, token_count, n_embd, &act);
-    if (st != RNB_HIP_OK) return st;
     HIP_TRY(s.moe_mid.reserve(n_slots * n_ff * sizeof(float)));
     HIP_TRY(s.moe_mid_qs.reserve(n_slots * n_ff));
     HIP_TRY(s.moe_mid_d.reserve(n_slots * sh.nb_mid * sizeof(float)));

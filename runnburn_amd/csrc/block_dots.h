@@ -49,33 +49,59 @@ __device__ __forceinline__ Q4KRegs q4k_load_block(const uint8_t *__restrict__ bl
     return r;
 }
 
-__device__ __forceinline__ float q4k_partial(const Q4KRegs &r, const Q4KAct &a, int g) {
-    const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
+// A block slice decoded once (nibbles split, scales and mins picked) so that it can be dotted with
+// several tokens' activations: the batched MoE kernels keep a row in this form while walking tokens.
+struct Q4KPrep {
+    uint4 lo0, lo1, hi0, hi1;  // 32 low and 32 high nibbles, one per byte
+    float d, dmin;
+    int sc0, sc1, mn0, mn1;
+};
+
+__device__ __forceinline__ Q4KPrep q4k_prepare(const Q4KRegs &r, int g) {
+    Q4KPrep p;
+    p.d = f16_bits_to_f32(r.h.x);
+    p.dmin = f16_bits_to_f32(r.h.x >> 16);
     const Q4KScales s = unpack_q4k_scales(r.h.y, r.h.z, r.h.w);
     const uint32_t scw = (g & 2) ? s.sc_hi : s.sc_lo, mnw = (g & 2) ? s.mn_hi : s.mn_lo;
     const int sh = (g & 1) * 16;
-    const int sc0 = (scw >> sh) & 0xff, sc1 = (scw >> (sh + 8)) & 0xff;
-    const int mn0 = (mnw >> sh) & 0xff, mn1 = (mnw >> (sh + 8)) & 0xff;
+    p.sc0 = (scw >> sh) & 0xff;
+    p.sc1 = (scw >> (sh + 8)) & 0xff;
+    p.mn0 = (mnw >> sh) & 0xff;
+    p.mn1 = (mnw >> (sh + 8)) & 0xff;
+    p.lo0 = make_uint4(r.qa.x & 0x0f0f0f0fu, r.qa.y & 0x0f0f0f0fu, r.qa.z & 0x0f0f0f0fu, r.qa.w & 0x0f0f0f0fu);
+    p.lo1 = make_uint4(r.qb.x & 0x0f0f0f0fu, r.qb.y & 0x0f0f0f0fu, r.qb.z & 0x0f0f0f0fu, r.qb.w & 0x0f0f0f0fu);
+    p.hi0 = make_uint4((r.qa.x >> 4) & 0x0f0f0f0fu, (r.qa.y >> 4) & 0x0f0f0f0fu, (r.qa.z >> 4) & 0x0f0f0f0fu,
+                       (r.qa.w >> 4) & 0x0f0f0f0fu);
+    p.hi1 = make_uint4((r.qb.x >> 4) & 0x0f0f0f0fu, (r.qb.y >> 4) & 0x0f0f0f0fu, (r.qb.z >> 4) & 0x0f0f0f0fu,
+                       (r.qb.w >> 4) & 0x0f0f0f0fu);
+    return p;
+}
+
+__device__ __forceinline__ float q4k_dot(const Q4KPrep &p, const Q4KAct &a) {
     int i0 = 0, i1 = 0;
-    i0 = dot4(r.qa.x & 0x0f0f0f0fu, a.lo0.x, i0);
-    i0 = dot4(r.qa.y & 0x0f0f0f0fu, a.lo0.y, i0);
-    i0 = dot4(r.qa.z & 0x0f0f0f0fu, a.lo0.z, i0);
-    i0 = dot4(r.qa.w & 0x0f0f0f0fu, a.lo0.w, i0);
-    i0 = dot4(r.qb.x & 0x0f0f0f0fu, a.lo1.x, i0);
-    i0 = dot4(r.qb.y & 0x0f0f0f0fu, a.lo1.y, i0);
-    i0 = dot4(r.qb.z & 0x0f0f0f0fu, a.lo1.z, i0);
-    i0 = dot4(r.qb.w & 0x0f0f0f0fu, a.lo1.w, i0);
-    i1 = dot4((r.qa.x >> 4) & 0x0f0f0f0fu, a.hi0.x, i1);
-    i1 = dot4((r.qa.y >> 4) & 0x0f0f0f0fu, a.hi0.y, i1);
-    i1 = dot4((r.qa.z >> 4) & 0x0f0f0f0fu, a.hi0.z, i1);
-    i1 = dot4((r.qa.w >> 4) & 0x0f0f0f0fu, a.hi0.w, i1);
-    i1 = dot4((r.qb.x >> 4) & 0x0f0f0f0fu, a.hi1.x, i1);
-    i1 = dot4((r.qb.y >> 4) & 0x0f0f0f0fu, a.hi1.y, i1);
-    i1 = dot4((r.qb.z >> 4) & 0x0f0f0f0fu, a.hi1.z, i1);
-    i1 = dot4((r.qb.w >> 4) & 0x0f0f0f0fu, a.hi1.w, i1);
-    const int sumi = sc0 * i0 + sc1 * i1;
-    const int summ = mn0 * a.bs_lo + mn1 * a.bs_hi;
-    return a.dx * (d * static_cast<float>(sumi) - dmin * static_cast<float>(summ));
+    i0 = dot4(p.lo0.x, a.lo0.x, i0);
+    i0 = dot4(p.lo0.y, a.lo0.y, i0);
+    i0 = dot4(p.lo0.z, a.lo0.z, i0);
+    i0 = dot4(p.lo0.w, a.lo0.w, i0);
+    i0 = dot4(p.lo1.x, a.lo1.x, i0);
+    i0 = dot4(p.lo1.y, a.lo1.y, i0);
+    i0 = dot4(p.lo1.z, a.lo1.z, i0);
+    i0 = dot4(p.lo1.w, a.lo1.w, i0);
+    i1 = dot4(p.hi0.x, a.hi0.x, i1);
+    i1 = dot4(p.hi0.y, a.hi0.y, i1);
+    i1 = dot4(p.hi0.z, a.hi0.z, i1);
+    i1 = dot4(p.hi0.w, a.hi0.w, i1);
+    i1 = dot4(p.hi1.x, a.hi1.x, i1);
+    i1 = dot4(p.hi1.y, a.hi1.y, i1);
+    i1 = dot4(p.hi1.z, a.hi1.z, i1);
+    i1 = dot4(p.hi1.w, a.hi1.w, i1);
+    const int sumi = p.sc0 * i0 + p.sc1 * i1;
+    const int summ = p.mn0 * a.bs_lo + p.mn1 * a.bs_hi;
+    return a.dx * (p.d * static_cast<float>(sumi) - p.dmin * static_cast<float>(summ));
+}
+
+__device__ __forceinline__ float q4k_partial(const Q4KRegs &r, const Q4KAct &a, int g) {
+    return q4k_dot(q4k_prepare(r, g), a);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -136,28 +162,51 @@ __device__ __forceinline__ int sext8(uint32_t v, int shift) {
     return static_cast<int>(static_cast<int8_t>((v >> shift) & 0xffu));
 }
 
-__device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, int q) {
+struct Q6KPrep {
+    uint4 u0, u1, u2, u3;  // 16 six-bit values (0..63) of each activation quarter, one per byte
+    int s0, s1, s2, s3;    // their sub-block scales
+    float d;
+};
+
+__device__ __forceinline__ Q6KPrep q6k_prepare(const Q6KRegs &r, int q) {
+    Q6KPrep p;
     const int is = (q & 1) * 8;  // l / 16 selects scale byte 0 or 1 of each pair
-    const int s0 = sext8(r.S.x, is), s1 = sext8(r.S.x, is + 16), s2 = sext8(r.S.y, is), s3 = sext8(r.S.y, is + 16);
-    int p0 = 0, p1 = 0, p2 = 0, p3 = 0;
-#define RNB_Q6_STEP(k)                                                                   \
-    {                                                                                    \
-        const uint32_t u0 = (r.A.k & 0x0f0f0f0fu) | ((r.H.k & 0x03030303u) << 4);        \
-        const uint32_t u1 = (r.B.k & 0x0f0f0f0fu) | ((r.H.k & 0x0c0c0c0cu) << 2);        \
-        const uint32_t u2 = ((r.A.k >> 4) & 0x0f0f0f0fu) | (r.H.k & 0x30303030u);        \
-        const uint32_t u3 = ((r.B.k >> 4) & 0x0f0f0f0fu) | ((r.H.k & 0xc0c0c0c0u) >> 2); \
-        p0 = dot4(u0, a.a0.k, p0);                                                       \
-        p1 = dot4(u1, a.a1.k, p1);                                                       \
-        p2 = dot4(u2, a.a2.k, p2);                                                       \
-        p3 = dot4(u3, a.a3.k, p3);                                                       \
-    }
-    RNB_Q6_STEP(x)
-    RNB_Q6_STEP(y)
-    RNB_Q6_STEP(z)
-    RNB_Q6_STEP(w)
-#undef RNB_Q6_STEP
-    const int sumi = s0 * (p0 - 32 * a.s0) + s1 * (p1 - 32 * a.s1) + s2 * (p2 - 32 * a.s2) + s3 * (p3 - 32 * a.s3);
-    return (f16_bits_to_f32(r.d_bits) * a.dx) * static_cast<float>(sumi);
+    p.s0 = sext8(r.S.x, is);
+    p.s1 = sext8(r.S.x, is + 16);
+    p.s2 = sext8(r.S.y, is);
+    p.s3 = sext8(r.S.y, is + 16);
+    p.d = f16_bits_to_f32(r.d_bits);
+#define RNB_Q6_UNPACK(k)                                                          \
+    p.u0.k = (r.A.k & 0x0f0f0f0fu) | ((r.H.k & 0x03030303u) << 4);                \
+    p.u1.k = (r.B.k & 0x0f0f0f0fu) | ((r.H.k & 0x0c0c0c0cu) << 2);                \
+    p.u2.k = ((r.A.k >> 4) & 0x0f0f0f0fu) | (r.H.k & 0x30303030u);                \
+    p.u3.k = ((r.B.k >> 4) & 0x0f0f0f0fu) | ((r.H.k & 0xc0c0c0c0u) >> 2);
+    RNB_Q6_UNPACK(x)
+    RNB_Q6_UNPACK(y)
+    RNB_Q6_UNPACK(z)
+    RNB_Q6_UNPACK(w)
+#undef RNB_Q6_UNPACK
+    return p;
+}
+
+__device__ __forceinline__ int dot16(const uint4 &u, const uint4 &a) {
+    int s = 0;
+    s = dot4(u.x, a.x, s);
+    s = dot4(u.y, a.y, s);
+    s = dot4(u.z, a.z, s);
+    s = dot4(u.w, a.w, s);
+    return s;
+}
+
+__device__ __forceinline__ float q6k_dot(const Q6KPrep &p, const Q6KAct &a) {
+    const int p0 = dot16(p.u0, a.a0), p1 = dot16(p.u1, a.a1), p2 = dot16(p.u2, a.a2), p3 = dot16(p.u3, a.a3);
+    const int sumi =
+        p.s0 * (p0 - 32 * a.s0) + p.s1 * (p1 - 32 * a.s1) + p.s2 * (p2 - 32 * a.s2) + p.s3 * (p3 - 32 * a.s3);
+    return (p.d * a.dx) * static_cast<float>(sumi);
+}
+
+__device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, int q) {
+    return q6k_dot(q6k_prepare(r, q), a);
 }
 
 }  // namespace rnb

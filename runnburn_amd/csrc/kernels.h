@@ -51,6 +51,15 @@ struct MoeGroups {
     const uint32_t *sorted_token;  // [n_slots]
     uint32_t n_groups;
 };
+// Decode-sized routing tables travel as a kernel argument instead of a host-to-device copy: the
+// activation quantiser's launch also writes them to their device buffer.
+constexpr uint32_t kMoeInlineWords = 240;  // 960 bytes of kernel argument
+struct MoeInlineTables {
+    uint32_t words[kMoeInlineWords];
+};
+void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
+                                     const MoeInlineTables &tables, uint32_t n_words, uint32_t *tables_dev,
+                                     hipStream_t stream);
 // mid[slot][n_ff] = silu(Wg[e] . h_tok) * (Wu[e] . h_tok); act = Q8_K(x) per token
 void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                         uint32_t n_ff, uint32_t nb_in, hipStream_t stream);

@@ -101,15 +101,15 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
                 const size_t off = ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kQ4KBytes;
-                const Q4KRegs gr = q4k_load_block(gate_all + off, g);
-                const Q4KRegs ur = q4k_load_block(up_all + off, g);
+                const Q4KPrep gp = q4k_prepare(q4k_load_block(gate_all + off, g), g);
+                const Q4KPrep up = q4k_prepare(q4k_load_block(up_all + off, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
                         const Q4KAct a = q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g);
-                        gacc[t] += q4k_partial(gr, a, g);
-                        uacc[t] += q4k_partial(ur, a, g);
+                        gacc[t] += q4k_dot(gp, a);
+                        uacc[t] += q4k_dot(up, a);
                     }
                 }
             }
@@ -169,20 +169,20 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
                 const uint8_t *blk = down_all + ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-                Q4KRegs r4{};
-                Q6KRegs r6{};
+                Q4KPrep p4{};
+                Q6KPrep p6{};
                 if constexpr (kQ6)
-                    r6 = q6k_load_block(blk, g);
+                    p6 = q6k_prepare(q6k_load_block(blk, g), g);
                 else
-                    r4 = q4k_load_block(blk, g);
+                    p4 = q4k_prepare(q4k_load_block(blk, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
                         if constexpr (kQ6)
-                            acc[t] += q6k_partial(r6, q6k_load_act(st.qs + ab * 256, st.d[ab], g), g);
+                            acc[t] += q6k_dot(p6, q6k_load_act(st.qs + ab * 256, st.d[ab], g));
                         else
-                            acc[t] += q4k_partial(r4, q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g), g);
+                            acc[t] += q4k_dot(p4, q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g));
                     }
                 }
             }

@@ -20,6 +20,19 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     q8k_quantize_span(x + blk * 256, lane, qs + blk * 256, d_out + blk, bsums + blk * 16);
 }
 
+// Same as quantize_q8k_kernel; workgroup 0 additionally copies `n_words` routing-table words from the
+// kernel argument to device memory (n_words <= 256 = one word per thread).
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    quantize_q8k_tables_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ qs,
+                               float *__restrict__ d_out, int16_t *__restrict__ bsums, const MoeInlineTables tables,
+                               uint32_t n_words, uint32_t *__restrict__ tables_dev) {
+    if (blockIdx.x == 0 && threadIdx.x < n_words) tables_dev[threadIdx.x] = tables.words[threadIdx.x];
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t blk = static_cast<size_t>(blockIdx.x) * kWavesPerWg + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;  // wave-uniform
+    q8k_quantize_span(x + blk * 256, lane, qs + blk * 256, d_out + blk, bsums + blk * 16);
+}
+
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     quantize_q8_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ qs,
                        float *__restrict__ d_out) {
@@ -38,6 +51,14 @@ void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, 
     const unsigned grid = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
     hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(kWave * kWavesPerWg), 0, stream, x, n_blocks, qs,
                        d, bsums);
+}
+
+void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
+                                     const MoeInlineTables &tables, uint32_t n_words, uint32_t *tables_dev,
+                                     hipStream_t stream) {
+    const unsigned grid = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
+    hipLaunchKernelGGL(quantize_q8k_tables_kernel, dim3(grid ? grid : 1), dim3(kWave * kWavesPerWg), 0, stream, x,
+                       n_blocks, qs, d, bsums, tables, n_words, tables_dev);
 }
 
 void launch_quantize_q8(const float *x, size_t n_blocks, int8_t *qs, float *d, hipStream_t stream) {

@@ -41,7 +41,13 @@ struct Resident {
     bool pinned = false;  // prewarmed: never evicted, and the only kind a sub-range may resolve to
 };
 
+struct TableSlot {
+    PinnedBuf host;
+    hipEvent_t event = nullptr;  // recorded after the slot's upload was enqueued
+};
+
 struct State {
+    static constexpr int kTableRing = 8;
     int device = 0;
     hipStream_t stream = nullptr;
     std::string device_name;
@@ -53,7 +59,9 @@ struct State {
     DeviceBuf act_bsums;  // per-16 sums (Q8_K)
     DeviceBuf out_f32;    // staged outputs
     DeviceBuf moe_mid, moe_mid_qs, moe_mid_d, moe_mid_bsums, moe_slot_out, moe_tables;
-    PinnedBuf bounce_in, bounce_out, bounce_tables;
+    PinnedBuf bounce_in, bounce_out;
+    TableSlot table_ring[kTableRing];  // MoE routing tables too large for a kernel argument
+    int table_ring_next = 0;
 
     std::map<uintptr_t, Resident> residents;  // keyed by host base address
     // what the activation scratch currently holds (set by quantize_activations)
