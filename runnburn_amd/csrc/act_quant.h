@@ -26,7 +26,9 @@ __device__ __forceinline__ AbsMax absmax_merge(AbsMax a, AbsMax b) {
 // Quantises x_blk[0..256) to one Q8_K block: qs (256 int8, 16-byte aligned), *d_out, bsums (16 int16).
 // Must be called by all 64 lanes of the wave.
 // `v` = this lane's four consecutive elements (x_blk[4*lane .. 4*lane+4)), already loaded.
-__device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8_t *qs, float *d_out, int16_t *bsums) {
+// `digits` (optional, 16 bytes) receives the 32-element sums split as b0 + 64*b1: b0[0..8) then b1[0..8).
+__device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8_t *qs, float *d_out, int16_t *bsums,
+                                                  uint8_t *digits = nullptr) {
     const float e[4] = {v.x, v.y, v.z, v.w};
     AbsMax m{0.0f, 0.0f, 4 * lane};
 #pragma unroll
@@ -66,11 +68,16 @@ __device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8
     const int sum16 = group_sum_i<4>(part);  // 4 lanes = 16 consecutive elements
     if ((lane & 3) == 0) bsums[lane >> 2] = static_cast<int16_t>(sum16);
     if (lane == 0) *d_out = d;
+    if (digits != nullptr) {  // wave-uniform
+        const int sum32 = sum16 + __shfl_xor(sum16, 4, kWave);       // every lane of an 8-lane group
+        const int mine = __shfl(sum32, 8 * (lane & 7), kWave);       // lanes 0..15: sum of sub-block lane % 8
+        if (lane < 16) digits[lane] = static_cast<uint8_t>(lane < 8 ? (mine & 63) : (mine >> 6));
+    }
 }
 
 __device__ __forceinline__ void q8k_quantize_span(const float *__restrict__ x_blk, int lane, int8_t *qs, float *d_out,
-                                                  int16_t *bsums) {
-    q8k_quantize_vals(reinterpret_cast<const float4 *>(x_blk)[lane], lane, qs, d_out, bsums);
+                                                  int16_t *bsums, uint8_t *digits = nullptr) {
+    q8k_quantize_vals(reinterpret_cast<const float4 *>(x_blk)[lane], lane, qs, d_out, bsums, digits);
 }
 
 // Quantises x_span[0..256) to eight 32-wide Q8 blocks (8 lanes per block); lanes whose block index

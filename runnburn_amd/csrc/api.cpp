@@ -45,6 +45,9 @@ int hip_fail(const char *what, hipError_t e) {
     } while (0)
 
 // Quantise seq*cols staged floats on the device into the state's activation scratch.
+// Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
+constexpr size_t kGemmMinSeq = 16;
+
 int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view) {
     const size_t n = seq * cols;
     HIP_TRY(s.act_qs.reserve(n));
@@ -55,9 +58,12 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
     } else {
         HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
         HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
+        s.act_has_digits = seq >= kGemmMinSeq;
+        if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
+        uint8_t *digits = s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr;
         launch_quantize_q8k(x_dev, n / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
-                            s.stream);
-        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
+                            digits, s.stream);
+        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(), digits};
     }
     HIP_TRY(hipGetLastError());
     s.act_family = quant == kQ8_0 ? kQ8_0 : kQ4K;
@@ -65,9 +71,6 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
     s.act_cols = cols;
     return RNB_HIP_OK;
 }
-
-// Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
-constexpr size_t kGemmMinSeq = 16;
 
 int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
                              float *out_dev);
@@ -82,10 +85,12 @@ int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, 
 
 int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
                              float *out_dev) {
-    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), quant == kQ8_0 ? nullptr : s.act_bsums.as<int16_t>()};
+    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), quant == kQ8_0 ? nullptr : s.act_bsums.as<int16_t>(),
+                      quant != kQ8_0 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     if (quant == kQ4K) {
-        if (seq >= kGemmMinSeq)
+        // the GEMM fills LDS with 16-byte loads: weights at other alignments take the per-token kernel
+        if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_gemm_q4k_mfma(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
         else
             launch_gemv_q4k(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
@@ -305,6 +310,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
         HIP_TRY(hipGetLastError());
         act = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
         s.act_family = kQ4K;
+        s.act_has_digits = false;
         s.act_seq = token_count;
         s.act_cols = n_embd;
     } else {
@@ -325,7 +331,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
     launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
-                        s.moe_mid_bsums.as<int16_t>(), s.stream);
+                        s.moe_mid_bsums.as<int16_t>(), nullptr, s.stream);
     ActView mid{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>()};
     launch_moe_down(down_dev, down_quant, mid, groups, d_route, s.moe_slot_out.as<float>(),
                     static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);

@@ -15,16 +15,20 @@ constexpr size_t kQ8_0Bytes = 34, kQ4KBytes = 144, kQ6KBytes = 210;
 //   Q8_K:  qs    int8  [seq][K]          (16-byte aligned rows, K % 256 == 0)
 //          d     f32   [seq][K/256]
 //          bsums int16 [seq][K/256][16]  (sums of 16 consecutive qs)
+//          digits u8   [seq][K/256][16]  (optional; bsum32[k] = bsums[2k] + bsums[2k+1] = b0[k] + 64*b1[k]
+//                                         as int8 digits: b0[0..8) in 0..63, then b1[0..8) in -64..63)
 //   Q8:    qs    int8  [seq][K]
 //          d     f32   [seq][K/32]
 struct ActView {
     const int8_t *qs;
     const float *d;
     const int16_t *bsums;  // null for the 32-wide Q8 form
+    const uint8_t *digits = nullptr;
 };
 
 // x: f32, 16-byte aligned, n_blocks*256 values
-void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
+// digits may be null
+void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
                          hipStream_t stream);
 // x: f32, 16-byte aligned, n_blocks*32 values; n_blocks % 8 == 0 not required
 void launch_quantize_q8(const float *x, size_t n_blocks, int8_t *qs, float *d, hipStream_t stream);

@@ -13,11 +13,12 @@ constexpr int kWavesPerWg = 4;
 
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     quantize_q8k_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ qs,
-                        float *__restrict__ d_out, int16_t *__restrict__ bsums) {
+                        float *__restrict__ d_out, int16_t *__restrict__ bsums, uint8_t *__restrict__ digits) {
     const int lane = threadIdx.x & (kWave - 1);
     const size_t blk = static_cast<size_t>(blockIdx.x) * kWavesPerWg + (threadIdx.x >> 6);
     if (blk >= n_blocks) return;  // wave-uniform
-    q8k_quantize_span(x + blk * 256, lane, qs + blk * 256, d_out + blk, bsums + blk * 16);
+    q8k_quantize_span(x + blk * 256, lane, qs + blk * 256, d_out + blk, bsums + blk * 16,
+                      digits != nullptr ? digits + blk * 16 : nullptr);
 }
 
 // Same as quantize_q8k_kernel; workgroup 0 additionally copies `n_words` routing-table words from the
@@ -45,12 +46,12 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 
 }  // namespace
 
-void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
+void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
                          hipStream_t stream) {
     if (n_blocks == 0) return;
     const unsigned grid = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
     hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(kWave * kWavesPerWg), 0, stream, x, n_blocks, qs,
-                       d, bsums);
+                       d, bsums, digits);
 }
 
 void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,

@@ -57,6 +57,8 @@ struct State {
     DeviceBuf act_qs;     // quantised activations: int8
     DeviceBuf act_d;      // per-block scales
     DeviceBuf act_bsums;  // per-16 sums (Q8_K)
+    DeviceBuf act_digits; // per-32 sums as two int8 digits (Q8_K, only filled for GEMM-sized batches)
+    bool act_has_digits = false;
     DeviceBuf out_f32;    // staged outputs
     DeviceBuf moe_mid, moe_mid_qs, moe_mid_d, moe_mid_bsums, moe_slot_out, moe_tables;
     PinnedBuf bounce_in, bounce_out;
