@@ -295,16 +295,15 @@ constexpr float kMagic = 12582912.0f;
 
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-// LDS-direct global loads: 64 lanes x 16 B (or 4 B), lane i's bytes land at dst_wave + 16*i (4*i); the source is a
-// workgroup-uniform base plus a 32-bit lane offset.  Written as assembly so that the compiler does not make every
-// later LDS read wait for them: the phases below order fills and reads with wait_fills() and barriers.
-__device__ __forceinline__ void lds_fill16(const uint8_t *base, uint32_t lane_off, uint8_t *dst_wave) {
-    const uint32_t l = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)dst_wave)));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l), "v"(lane_off), "s"(base) : "memory");
+// LDS-direct global loads: 64 lanes x 16 B (or 4 B), lane i's bytes land at LDS byte address dst + 16*i (4*i); the
+// source is a wave-uniform base plus a 32-bit lane offset.  Written as assembly so that the compiler does not make
+// every later LDS read wait for them: the phases below order fills and reads with wait_fills() and barriers.
+// (m0 needs one wait state before the load reads it.)
+__device__ __forceinline__ void lds_fill16(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
 }
-__device__ __forceinline__ void lds_fill4(const uint8_t *base, uint32_t lane_off, uint8_t *dst_wave) {
-    const uint32_t l = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)dst_wave)));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(l), "v"(lane_off), "s"(base) : "memory");
+__device__ __forceinline__ void lds_fill4(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
 }
 __device__ __forceinline__ void wait_fills() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -314,8 +313,10 @@ __global__ void __launch_bounds__(kPpThreads, 1)
                              uint32_t seq) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what derives from it stays in SGPRs
     const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)lds));
     const uint32_t wg_row0 = blockIdx.x * kPpRowsPerWg;
     const uint32_t row0 = wg_row0 + wave * 32;
     const uint32_t tok0 = blockIdx.y * kPpToks;
@@ -344,23 +345,25 @@ __global__ void __launch_bounds__(kPpThreads, 1)
     const uint32_t dig_off = tok_lane * nb * 16u, dx_off = tok_lane * nb * 4u;
 
     auto issue_w = [&](uint32_t b) {
-        uint8_t *dst = lds + kPpWOff + (b & 1) * kPpWBuf;
+        const uint32_t dst = lds0 + kPpWOff + (b & 1) * kPpWBuf;
+        const uint8_t *src = w_base + b * 144u;
 #pragma unroll
         for (int k = 0; k < kPpWPerWave; k++) {
             const int i = k * kPpWaves + wave;
-            if (i < kPpWInstr) lds_fill16(w_base, w_off[k] + b * 144u, dst + i * 1024);
+            if (i < kPpWInstr) lds_fill16(src, w_off[k], dst + i * 1024);
         }
     };
     auto issue_a = [&](uint32_t b) {
-        uint8_t *dst = lds + kPpAOff + (b & 1) * kPpABuf;
+        const uint32_t dst = lds0 + kPpAOff + (b & 1) * kPpABuf;
+        const uint8_t *src = a_base + b * 256u;
 #pragma unroll
         for (int k = 0; k < kPpAPerWave; k++) {
             const int i = k * kPpWaves + wave;
-            if (i < kPpAInstr) lds_fill16(a_base, a_off[k] + b * 256u, dst + i * 1024);
+            if (i < kPpAInstr) lds_fill16(src, a_off[k], dst + i * 1024);
         }
-        uint8_t *aux = lds + kPpAuxOff + (b & 3) * kPpAuxBytes;
-        if (wave == 1) lds_fill16(dig_base, dig_off + b * 16u, aux + kPpToks * 4);
-        if (wave == 2) lds_fill4(dx_base, dx_off + b * 4u, aux);
+        const uint32_t aux = lds0 + kPpAuxOff + (b & 3) * kPpAuxBytes;
+        if (wave == 1) lds_fill16(dig_base + b * 16u, dig_off, aux + kPpToks * 4);
+        if (wave == 2) lds_fill4(dx_base + b * 4u, dx_off, aux);
     };
 
     // ---- per-wave state carried between phases -------------------------------------------------
