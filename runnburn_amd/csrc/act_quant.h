@@ -11,18 +11,6 @@
 
 namespace rnb {
 
-struct AbsMax {
-    float amax;  // max |x|
-    float val;   // the signed element that attained it first
-    int idx;     // its index within the 256-span
-};
-
-// first occurrence wins: larger |x|, or equal |x| and smaller index
-__device__ __forceinline__ AbsMax absmax_merge(AbsMax a, AbsMax b) {
-    const bool take_b = (b.amax > a.amax) || (b.amax == a.amax && b.idx < a.idx);
-    return take_b ? b : a;
-}
-
 // Quantises x_blk[0..256) to one Q8_K block: qs (256 int8, 16-byte aligned), *d_out, bsums (16 int16).
 // Must be called by all 64 lanes of the wave.
 // `v` = this lane's four consecutive elements (x_blk[4*lane .. 4*lane+4)), already loaded.
@@ -30,27 +18,25 @@ __device__ __forceinline__ AbsMax absmax_merge(AbsMax a, AbsMax b) {
 __device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8_t *qs, float *d_out, int16_t *bsums,
                                                   uint8_t *digits = nullptr) {
     const float e[4] = {v.x, v.y, v.z, v.w};
-    AbsMax m{0.0f, 0.0f, 4 * lane};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float ax = fabsf(e[i]);
-        if (ax > m.amax) {  // strict: keeps the first of equal magnitudes
-            m.amax = ax;
-            m.val = e[i];
-            m.idx = 4 * lane + i;
-        }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        AbsMax o;
-        o.amax = __shfl_xor(m.amax, off, kWave);
-        o.val = __shfl_xor(m.val, off, kWave);
-        o.idx = __shfl_xor(m.idx, off, kWave);
-        m = absmax_merge(m, o);
-    }
+    // max |x| of the span: per lane, then across the wave on the DPP path (lane 63 ends up with the maximum)
+    const float ax[4] = {fabsf(e[0]), fabsf(e[1]), fabsf(e[2]), fabsf(e[3])};
+    float lmax = fmaxf(fmaxf(ax[0], ax[1]), fmaxf(ax[2], ax[3]));
+    lmax = dpp_max<0xB1, 0xf>(lmax);   // quad_perm [1,0,3,2]
+    lmax = dpp_max<0x4E, 0xf>(lmax);   // quad_perm [2,3,0,1]
+    lmax = dpp_max<0x141, 0xf>(lmax);  // row_half_mirror
+    lmax = dpp_max<0x140, 0xf>(lmax);  // row_mirror
+    lmax = dpp_max<0x142, 0xa>(lmax);  // row_bcast15
+    lmax = dpp_max<0x143, 0xc>(lmax);  // row_bcast31
+    const float amax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lmax), 63));
+    // the element that attains it first in index order: lowest lane with a match, lowest element inside that lane
+    const bool hit[4] = {ax[0] == amax, ax[1] == amax, ax[2] == amax, ax[3] == amax};
+    const unsigned long long lanes = __builtin_amdgcn_ballot_w64(hit[0] || hit[1] || hit[2] || hit[3]);
+    const int first_lane = __builtin_ctzll(lanes);  // amax is one of the |x|, so at least one lane matches
+    const float mine = hit[0] ? e[0] : hit[1] ? e[1] : hit[2] ? e[2] : e[3];
+    const float max_val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), first_lane));
     float iscale = 0.0f, d = 0.0f;
-    if (m.amax != 0.0f) {
-        iscale = -127.0f / m.val;
+    if (amax != 0.0f) {
+        iscale = -127.0f / max_val;
         d = 1.0f / iscale;
     }
     int part = 0;
@@ -65,7 +51,9 @@ __device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8
         packed |= (static_cast<uint32_t>(q) & 0xffu) << (8 * i);
     }
     reinterpret_cast<uint32_t *>(qs)[lane] = packed;
-    const int sum16 = group_sum_i<4>(part);  // 4 lanes = 16 consecutive elements
+    // 4 lanes = 16 consecutive elements: two quad permutes leave the sum in every lane of the quad
+    int sum16 = part + __builtin_amdgcn_update_dpp(0, part, 0xB1, 0xf, 0xf, false);
+    sum16 += __builtin_amdgcn_update_dpp(0, sum16, 0x4E, 0xf, 0xf, false);
     if ((lane & 3) == 0) bsums[lane >> 2] = static_cast<int16_t>(sum16);
     if (lane == 0) *d_out = d;
     if (digits != nullptr) {  // wave-uniform

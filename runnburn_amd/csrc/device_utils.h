@@ -39,6 +39,11 @@ __device__ __forceinline__ float dpp_add(float v) {
     const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, kRowMask, 0xf, false);
     return v + __builtin_bit_cast(float, t);
 }
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_max(float v) {  // for non-negative v (lanes left out of the row mask read 0)
+    const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, kRowMask, 0xf, false);
+    return fmaxf(v, __builtin_bit_cast(float, t));
+}
 template <int kWidth>
 __device__ __forceinline__ float seg_sum(float v) {
     static_assert(kWidth == 16 || kWidth == 32 || kWidth == 64, "segment width");
