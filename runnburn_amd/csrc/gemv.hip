@@ -12,6 +12,8 @@
 // registers once per wave instead of once per row.  Integer sums per lane are exact
 // (v_dot4_i32_i8); the per-block f32 scale is applied once per lane and the partial sums are added
 // across lanes on the DPP path, so results differ from the scalar reference only by f32 summation order.
+#include <type_traits>
+
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
@@ -89,6 +91,82 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Long rows (more than 16 super-blocks): the K dimension is split across the waves of a workgroup, wave j
+// owning super-blocks [16j, 16j+16) of every row, so each lane's activation slice is loaded once and stays
+// in registers; the per-wave partial sums of kSplitRows consecutive rows meet in LDS and are added in
+// wave order.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSplitRows = 4;
+constexpr uint32_t kSplitMaxWaves = 16;  // rows of up to 256 super-blocks
+
+template <bool kQ6>
+__global__ void __launch_bounds__(kWave *kSplitMaxWaves)
+    gemv_kquant_splitk_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                              const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                              uint32_t row_chunks) {
+    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    using Regs = std::conditional_t<kQ6, Q6KRegs, Q4KRegs>;
+    __shared__ float s_part[2][kSplitRows][kSplitMaxWaves];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6, n_slices = blockDim.x >> 6;
+    const int g = lane & 3;
+    const uint32_t b = wave * 16 + (lane >> 2);
+    const bool has_block = b < nb;
+    const uint32_t tok = blockIdx.y;
+    const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? b : 0);
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    Q4KAct a4{};
+    Q6KAct a6{};
+    if constexpr (kQ6)
+        a6 = q6k_load_act(aq + ab * 256, ad[ab], g);
+    else
+        a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    uint32_t parity = 0;
+    for (uint32_t chunk = blockIdx.x; chunk < row_chunks; chunk += gridDim.x, parity ^= 1) {
+        const uint32_t row0 = chunk * kSplitRows;
+        Regs r[kSplitRows];
+#pragma unroll
+        for (int i = 0; i < kSplitRows; i++) {
+            r[i] = Regs{};  // idle lanes and rows past the end keep zeros
+            if (has_block && row0 + i < rows) {
+                const uint8_t *blk = w + static_cast<size_t>(row0 + i) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
+                if constexpr (kQ6)
+                    r[i] = q6k_load_block(blk, g);
+                else
+                    r[i] = q4k_load_block(blk, g);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kSplitRows; i++) {
+            float acc;
+            if constexpr (kQ6)
+                acc = q6k_partial(r[i], a6, g);
+            else
+                acc = q4k_partial(r[i], a4, g);
+            acc = seg_sum<kWave>(has_block ? acc : 0.0f);
+            if (lane == kWave - 1) s_part[parity][i][wave] = acc;
+        }
+        __syncthreads();  // the other parity's buffer is reused only after the next barrier
+        if (threadIdx.x < kSplitRows && row0 + threadIdx.x < rows) {
+            float sum = 0.0f;
+            for (uint32_t j = 0; j < n_slices; j++) sum += s_part[parity][threadIdx.x][j];
+            out[static_cast<size_t>(tok) * rows + row0 + threadIdx.x] = sum;
+        }
+    }
+}
+
+template <bool kQ6>
+void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream) {
+    const uint32_t n_slices = (nb + 15) / 16;
+    const uint32_t row_chunks = (rows + kSplitRows - 1) / kSplitRows;
+    const uint32_t want = kTargetWaves / n_slices;  // workgroups for about kTargetWaves waves
+    const dim3 grid(row_chunks < want ? row_chunks : want, seq, 1);
+    hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQ6>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
+                       act.bsums, out, rows, nb, row_chunks);
+}
+
 template <bool kQ6, int kRowsPerWave>
 void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                    hipStream_t stream) {
@@ -103,7 +181,9 @@ template <bool kQ6>
 void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                        hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
-    if (nb <= 4)
+    if (nb > 16 && nb <= 16 * kSplitMaxWaves)
+        launch_kquant_splitk<kQ6>(w, act, out, rows, nb, seq, stream);
+    else if (nb <= 4)
         launch_kquant<kQ6, 4>(w, act, out, rows, nb, seq, stream);
     else if (nb <= 8)
         launch_kquant<kQ6, 2>(w, act, out, rows, nb, seq, stream);
