@@ -23,7 +23,10 @@ namespace {
 constexpr int kWavesPerWg = 4;
 constexpr int kMaxChunkTokens = 8;  // tokens staged in LDS at a time
 
-// LDS staging of `nt` quantised activation rows: qs [nt][nb*256] | d [nt][nb] | bsums [nt][nb*16]
+// LDS staging of `nt` quantised activation rows: qs [nt][nb][272] | d [nt][nb] | bsums [nt][nb*16].  A block's 256
+// int8 take a 272-byte slot: the lanes of a wave read 16-byte pieces of different blocks, and a 256-byte stride
+// would put them all on the same banks.
+constexpr uint32_t kStageBlk = 272;
 struct Staged {
     const int8_t *qs;
     const float *d;
@@ -31,7 +34,7 @@ struct Staged {
 };
 
 __host__ __device__ __forceinline__ size_t stage_d_offset(uint32_t tmax, uint32_t nb) {
-    return static_cast<size_t>(tmax) * nb * 256;
+    return static_cast<size_t>(tmax) * nb * kStageBlk;
 }
 __host__ __device__ __forceinline__ size_t stage_bsums_offset(uint32_t tmax, uint32_t nb) {
     return stage_d_offset(tmax, nb) + ((static_cast<size_t>(tmax) * nb * 4 + 15) & ~static_cast<size_t>(15));
@@ -52,9 +55,10 @@ __device__ __forceinline__ Staged stage_layout(uint8_t *lds, uint32_t tmax, uint
 __device__ __forceinline__ void stage_row(uint8_t *lds, uint32_t tmax, uint32_t nb, uint32_t t, size_t src_row,
                                           const int8_t *__restrict__ aq, const float *__restrict__ ad,
                                           const int16_t *__restrict__ abs) {
-    uint4 *dq = reinterpret_cast<uint4 *>(lds + static_cast<size_t>(t) * nb * 256);
+    uint8_t *dq = lds + static_cast<size_t>(t) * nb * kStageBlk;
     const uint4 *sq = reinterpret_cast<const uint4 *>(aq + src_row * nb * 256);
-    for (uint32_t i = threadIdx.x; i < nb * 16; i += blockDim.x) dq[i] = sq[i];
+    for (uint32_t i = threadIdx.x; i < nb * 16; i += blockDim.x)
+        *reinterpret_cast<uint4 *>(dq + (i >> 4) * kStageBlk + (i & 15) * 16) = sq[i];
     float *dd = reinterpret_cast<float *>(lds + stage_d_offset(tmax, nb)) + static_cast<size_t>(t) * nb;
     for (uint32_t i = threadIdx.x; i < nb; i += blockDim.x) dd[i] = ad[src_row * nb + i];
     uint4 *db = reinterpret_cast<uint4 *>(lds + stage_bsums_offset(tmax, nb)) + static_cast<size_t>(t) * nb * 2;
@@ -107,7 +111,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
-                        const Q4KAct a = q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g);
+                        const Q4KAct a = q4k_load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g);
                         gacc[t] += q4k_dot(gp, a);
                         uacc[t] += q4k_dot(up, a);
                     }
@@ -180,9 +184,9 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
                         if constexpr (kQ6)
-                            acc[t] += q6k_dot(p6, q6k_load_act(st.qs + ab * 256, st.d[ab], g));
+                            acc[t] += q6k_dot(p6, q6k_load_act(st.qs + ab * kStageBlk, st.d[ab], g));
                         else
-                            acc[t] += q4k_dot(p4, q4k_load_act(st.qs + ab * 256, st.d[ab], st.bsums + ab * 16, g));
+                            acc[t] += q4k_dot(p4, q4k_load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
                     }
                 }
             }
@@ -225,7 +229,7 @@ TilePlan plan_tiles(uint32_t rows, uint32_t nb, uint32_t n_groups, int rows_per_
     const uint64_t passes_total = static_cast<uint64_t>((rows + per_pass - 1) / per_pass) * n_groups;
     uint32_t iters = static_cast<uint32_t>(passes_total / 2048);
     p.iters = iters < 1 ? 1 : (iters > 8 ? 8 : iters);
-    const size_t per_token = static_cast<size_t>(nb) * 292;
+    const size_t per_token = static_cast<size_t>(nb) * (kStageBlk + 36);
     uint32_t tmax = static_cast<uint32_t>((48 * 1024) / per_token);
     p.tmax = tmax < 1 ? 1 : (tmax > kMaxChunkTokens ? kMaxChunkTokens : tmax);
     p.lds_bytes = stage_bytes(p.tmax, nb);

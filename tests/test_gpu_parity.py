@@ -112,7 +112,8 @@ def test_reference_closed_forms_on_device(rnb):
 # ---- GEMV: shapes around every edge of the lane mapping ------------------------------------------
 
 @pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
-@pytest.mark.parametrize("rows,nblk", [(1, 1), (3, 2), (4, 3), (5, 5), (7, 8), (9, 9), (64, 16), (33, 17), (6, 56)])
+@pytest.mark.parametrize("rows,nblk", [(1, 1), (3, 2), (4, 3), (5, 5), (7, 8), (9, 9), (64, 16), (33, 17), (6, 56),
+                                       (5, 31), (130, 20), (9, 256), (2, 257)])
 def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
     cols = nblk * 256
     w = oracle.make_weights(quant, rows, cols, 1000 + rows * 31 + nblk)
@@ -265,7 +266,18 @@ def test_gemv_batch_small(rnb, oracle, quant, seq):
                 f"batch quant {quant} seq {seq}")
 
 
-@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33),
+@pytest.mark.parametrize("quant", [Q4_K, Q6_K])
+def test_gemv_batch_long_rows(rnb, oracle, quant):
+    """Rows longer than 16 super-blocks take the K-split kernel; several tokens ride on grid.y."""
+    rows, cols, seq = 21, 20 * 256, 3
+    w = oracle.make_weights(quant, rows, cols, 150 + quant)
+    x = oracle.fill_normal(seq * cols, 160, 1.0)
+    got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"long-row batch quant {quant}")
+
+
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
                                            (1, 1, 16), (257, 5, 40)])
 def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
     cols = nblk * 256
