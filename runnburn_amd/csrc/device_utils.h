@@ -32,6 +32,20 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
 }
 
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// LDS-direct global loads: 64 lanes x 16 B (or 4 B), lane i's bytes land at LDS byte address dst + 16*i (4*i); the
+// source is a wave-uniform base plus a 32-bit lane offset.  Written as assembly so that the compiler does not make
+// every later LDS read wait for them: callers order fills and reads themselves with waits on vmcnt and barriers.
+// (m0 needs one wait state before the load reads it.)
+__device__ __forceinline__ void lds_fill16(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_fill4(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void wait_fills() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Cross-lane sums on the DPP data path (no LDS traffic).  After seg_sum<W>(v) the LAST lane of every
 // aligned W-lane segment (W = 16, 32 or 64) holds the sum over that segment.
 template <int kCtrl, int kRowMask>

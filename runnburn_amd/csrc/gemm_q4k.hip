@@ -70,20 +70,6 @@ constexpr int kPpAPerWave = (kPpAInstr + kPpWaves - 1) / kPpWaves;  // 3
 constexpr uint32_t kMagicBits = 0x4B400000u;      // 1.5 * 2^23: int bits of 12582912.0f
 constexpr float kMagic = 12582912.0f;
 
-typedef __attribute__((address_space(3))) void *lptr_t;
-
-// LDS-direct global loads: 64 lanes x 16 B (or 4 B), lane i's bytes land at LDS byte address dst + 16*i (4*i); the
-// source is a wave-uniform base plus a 32-bit lane offset.  Written as assembly so that the compiler does not make
-// every later LDS read wait for them: the phases below order fills and reads with wait_fills() and barriers.
-// (m0 needs one wait state before the load reads it.)
-__device__ __forceinline__ void lds_fill16(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
-}
-__device__ __forceinline__ void lds_fill4(const uint8_t *base, uint32_t lane_off, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
-}
-__device__ __forceinline__ void wait_fills() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 __global__ void __launch_bounds__(kPpThreads, 1)
     gemm_q4k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                              const uint8_t *__restrict__ adig, float *__restrict__ out, uint32_t rows, uint32_t nb,
