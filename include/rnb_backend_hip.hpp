@@ -151,4 +151,92 @@ class HipBackend {
     }
 };
 
+// GGUFFile (crates/rnb-loader/src/gguf/parser.rs:16-24) over the C ABI: the handle owns the file mapping, tensors are
+// views into it.  `open` = parse + map_tensors (crates/rnb-loader/src/convert.rs:99-178).
+struct GgufTensorView {
+    std::string name;
+    std::vector<uint64_t> shape;  // row-major
+    uint32_t ggml_type = 0;
+    uint64_t file_offset = 0;
+    Bytes bytes{nullptr, 0};      // the tensor's block bytes inside the mapping
+    size_t index = 0;
+};
+
+class GgufFile {
+  public:
+    GgufFile() = default;
+    GgufFile(const GgufFile &) = delete;
+    GgufFile &operator=(const GgufFile &) = delete;
+    GgufFile(GgufFile &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    GgufFile &operator=(GgufFile &&o) noexcept {
+        if (this != &o) {
+            rnb_hip_gguf_close(h_);
+            h_ = o.h_;
+            o.h_ = nullptr;
+        }
+        return *this;
+    }
+    ~GgufFile() { rnb_hip_gguf_close(h_); }
+
+    static Result<GgufFile> open(const std::string &path) {
+        Result<GgufFile> r;
+        r.status = rnb_hip_gguf_open(path.c_str(), &r.value.h_);
+        return finish(std::move(r));
+    }
+    static Result<GgufFile> parse(Bytes data) {  // borrows `data`
+        Result<GgufFile> r;
+        r.status = rnb_hip_gguf_parse(data.ptr, data.len, &r.value.h_);
+        return finish(std::move(r));
+    }
+    uint32_t version() const { return rnb_hip_gguf_version(h_); }
+    uint64_t alignment() const { return rnb_hip_gguf_alignment(h_); }
+    uint64_t data_start() const { return rnb_hip_gguf_data_start(h_); }
+    size_t tensor_count() const { return rnb_hip_gguf_tensor_count(h_); }
+    Result<GgufTensorView> tensor(size_t index) const {
+        rnb_hip_gguf_tensor t;
+        const int st = rnb_hip_gguf_tensor_at(h_, index, &t);
+        if (st != RNB_HIP_OK) return make_err<GgufTensorView>(st);
+        GgufTensorView v;
+        v.name = t.name;
+        v.shape.assign(t.shape, t.shape + t.n_dims);
+        v.ggml_type = t.ggml_type;
+        v.file_offset = t.file_offset;
+        v.bytes = Bytes{t.data, t.data != nullptr ? static_cast<size_t>(t.n_bytes) : 0};
+        v.index = index;
+        return make_ok(std::move(v));
+    }
+    Result<GgufTensorView> tensor(const std::string &name) const {
+        for (size_t i = 0, n = tensor_count(); i < n; i++) {
+            Result<GgufTensorView> r = tensor(i);
+            if (r && r.value.name == name) return r;
+        }
+        Result<GgufTensorView> r;
+        r.status = RNB_HIP_INVALID_REQUEST;
+        r.error = "missing tensor: " + name;
+        return r;
+    }
+    std::string metadata_str(const std::string &key) const {
+        const char *s = rnb_hip_gguf_metadata_str(h_, key.c_str());
+        return s != nullptr ? s : "";
+    }
+    Result<uint64_t> metadata_u64(const std::string &key) const {
+        uint64_t v = 0;
+        const int st = rnb_hip_gguf_metadata_u64(h_, key.c_str(), &v);
+        return st == RNB_HIP_OK ? make_ok(v) : make_err<uint64_t>(st);
+    }
+    // untouched upload of one tensor, pinned in the resident table
+    Result<Unit> prewarm(size_t index) const {
+        const int st = rnb_hip_gguf_prewarm_tensor(h_, index);
+        return st == RNB_HIP_OK ? make_ok(Unit{}) : make_err<Unit>(st);
+    }
+
+  private:
+    static Result<GgufFile> finish(Result<GgufFile> r) {
+        r.ok = r.status == RNB_HIP_OK;
+        if (!r.ok) r.error = rnb_hip_last_error();
+        return r;
+    }
+    rnb_hip_gguf *h_ = nullptr;
+};
+
 }  // namespace rnb_hip

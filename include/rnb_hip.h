@@ -155,6 +155,57 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
                                             uint32_t down_quant, size_t n_ff, size_t n_embd,
                                             const float *x_dev, float *out_dev);
 
+/* ---- GGUF container: header, tensor table, untouched upload -------------------------------------
+ * The reader side of the path: crates/rnb-loader/src/gguf/parser.rs:247-407 (GGUFFile::parse; same
+ * limits, checks and message texts, reported through rnb_hip_last_error() with the Display strings of
+ * crates/rnb-loader/src/error.rs:4-16), crates/rnb-loader/src/gguf/types.rs:5-41 (ggml type ids),
+ * crates/rnb-loader/src/convert.rs:23-83 (tensor byte sizes) and :99-178 (map_tensors: every tensor
+ * inside the file).  Tensor payloads are never copied or transformed on the host: `data` points into
+ * the mapping, and rnb_hip_gguf_prewarm_tensor uploads exactly those bytes. */
+typedef struct rnb_hip_gguf rnb_hip_gguf;
+typedef struct rnb_hip_gguf_tensor {
+    const char *name;      /* owned by the rnb_hip_gguf */
+    uint32_t n_dims;       /* 0..4 */
+    uint64_t shape[4];     /* row-major (outermost first): the file stores innermost first, parser.rs:356-357 */
+    uint32_t ggml_type;    /* ggml type id: 8 = Q8_0, 12 = Q4_K, 14 = Q6_K, 0 = F32, ... */
+    uint64_t offset;       /* relative to the data section, as stored */
+    uint64_t file_offset;  /* data_start + offset */
+    uint64_t n_bytes;      /* elements / block elements * block bytes; 0 if the shape is not block-aligned */
+    const uint8_t *data;   /* mapping + file_offset, or NULL if the tensor does not lie inside the file */
+} rnb_hip_gguf_tensor;
+
+/* mmap + parse + map_tensors checks; the handle owns the mapping until rnb_hip_gguf_close */
+int rnb_hip_gguf_open(const char *path, rnb_hip_gguf **out);
+/* GGUFFile::parse over caller-owned bytes (borrowed for the handle's lifetime); payload bounds are
+ * not checked here, exactly as in the reference: call rnb_hip_gguf_map_tensors for that */
+int rnb_hip_gguf_parse(const uint8_t *data, size_t len, rnb_hip_gguf **out);
+int rnb_hip_gguf_map_tensors(const rnb_hip_gguf *g);
+void rnb_hip_gguf_close(rnb_hip_gguf *g);
+uint32_t rnb_hip_gguf_version(const rnb_hip_gguf *g);
+uint64_t rnb_hip_gguf_alignment(const rnb_hip_gguf *g);   /* general.alignment, default 32 */
+uint64_t rnb_hip_gguf_data_start(const rnb_hip_gguf *g);  /* header end rounded up to the alignment */
+size_t rnb_hip_gguf_tensor_count(const rnb_hip_gguf *g);
+int rnb_hip_gguf_tensor_at(const rnb_hip_gguf *g, size_t index, rnb_hip_gguf_tensor *out);
+int rnb_hip_gguf_find_tensor(const rnb_hip_gguf *g, const char *name, rnb_hip_gguf_tensor *out);
+/* checked_tensor_size, convert.rs:28-43 (shape row-major) */
+int rnb_hip_gguf_tensor_size(const uint64_t *shape, uint32_t n_dims, uint32_t ggml_type, uint64_t *bytes);
+/* metadata in file order; value type ids 0..12 as in the GGUF specification (8 = string, 9 = array);
+ * rnb_hip_gguf_metadata_type returns -1 for an absent key */
+size_t rnb_hip_gguf_metadata_count(const rnb_hip_gguf *g);
+const char *rnb_hip_gguf_metadata_key(const rnb_hip_gguf *g, size_t index);
+int rnb_hip_gguf_metadata_type(const rnb_hip_gguf *g, const char *key);
+int rnb_hip_gguf_metadata_u64(const rnb_hip_gguf *g, const char *key, uint64_t *out); /* any non-negative integer, bool */
+int rnb_hip_gguf_metadata_i64(const rnb_hip_gguf *g, const char *key, int64_t *out);
+int rnb_hip_gguf_metadata_f64(const rnb_hip_gguf *g, const char *key, double *out);   /* F32 or F64 */
+const char *rnb_hip_gguf_metadata_str(const rnb_hip_gguf *g, const char *key);        /* NULL unless a string */
+int rnb_hip_gguf_metadata_array(const rnb_hip_gguf *g, const char *key, uint32_t *elem_type, uint64_t *count);
+const char *rnb_hip_gguf_metadata_array_str(const rnb_hip_gguf *g, const char *key, uint64_t index);
+int rnb_hip_gguf_metadata_array_f64(const rnb_hip_gguf *g, const char *key, uint64_t index, double *out);
+/* uploads the tensor's bytes as stored (no requantisation, no repack) and pins them in the resident
+ * table (rnb_hip_prewarm): operator calls that pass `data`, or a sub-range of it such as one expert
+ * of a stacked [n_expert, rows, cols] tensor, then run from the device copy */
+int rnb_hip_gguf_prewarm_tensor(const rnb_hip_gguf *g, size_t index);
+
 #ifdef __cplusplus
 }
 #endif

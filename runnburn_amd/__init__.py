@@ -19,6 +19,9 @@ from .binding import (  # noqa: F401
     BackendError,
     HipBackend,
     DeviceBuffer,
+    GGUFFile,
+    GGUFTensor,
+    gguf_tensor_size,
     GGML_Q4_K,
     GGML_Q6_K,
     GGML_Q8_0,

@@ -49,6 +49,28 @@ SYMBOLS = [
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
+    ("rnb_hip_gguf_open", _i, [C.c_char_p, C.POINTER(_vp)]),
+    ("rnb_hip_gguf_parse", _i, [_vp, _sz, C.POINTER(_vp)]),
+    ("rnb_hip_gguf_map_tensors", _i, [_vp]),
+    ("rnb_hip_gguf_close", None, [_vp]),
+    ("rnb_hip_gguf_version", _u32, [_vp]),
+    ("rnb_hip_gguf_alignment", C.c_uint64, [_vp]),
+    ("rnb_hip_gguf_data_start", C.c_uint64, [_vp]),
+    ("rnb_hip_gguf_tensor_count", _sz, [_vp]),
+    ("rnb_hip_gguf_tensor_at", _i, [_vp, _sz, _vp]),
+    ("rnb_hip_gguf_find_tensor", _i, [_vp, C.c_char_p, _vp]),
+    ("rnb_hip_gguf_tensor_size", _i, [_u64p, _u32, _u32, _u64p]),
+    ("rnb_hip_gguf_metadata_count", _sz, [_vp]),
+    ("rnb_hip_gguf_metadata_key", C.c_char_p, [_vp, _sz]),
+    ("rnb_hip_gguf_metadata_type", _i, [_vp, C.c_char_p]),
+    ("rnb_hip_gguf_metadata_u64", _i, [_vp, C.c_char_p, _u64p]),
+    ("rnb_hip_gguf_metadata_i64", _i, [_vp, C.c_char_p, C.POINTER(C.c_int64)]),
+    ("rnb_hip_gguf_metadata_f64", _i, [_vp, C.c_char_p, C.POINTER(C.c_double)]),
+    ("rnb_hip_gguf_metadata_str", C.c_char_p, [_vp, C.c_char_p]),
+    ("rnb_hip_gguf_metadata_array", _i, [_vp, C.c_char_p, C.POINTER(_u32), _u64p]),
+    ("rnb_hip_gguf_metadata_array_str", C.c_char_p, [_vp, C.c_char_p, C.c_uint64]),
+    ("rnb_hip_gguf_metadata_array_f64", _i, [_vp, C.c_char_p, C.c_uint64, C.POINTER(C.c_double)]),
+    ("rnb_hip_gguf_prewarm_tensor", _i, [_vp, _sz]),
 ]
 
 Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
@@ -339,3 +361,164 @@ class HipBackend:
     def execute(self, request) -> None:
         raise BackendError(2, "HipBackend::execute: requests are served by the operator functions "
                               "(q4k_gemv, q6k_gemv, q8_0_gemv, *_batch, qwen35_sparse_experts_*)")
+
+
+# ---- GGUF container (crates/rnb-loader/src/gguf/parser.rs, crates/rnb-loader/src/convert.rs) ---------------------
+
+class _GGUFTensorStruct(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("shape", C.c_uint64 * 4), ("ggml_type", C.c_uint32),
+                ("offset", C.c_uint64), ("file_offset", C.c_uint64), ("n_bytes", C.c_uint64), ("data", C.c_void_p)]
+
+
+class GGUFTensor:
+    """One row of the tensor table: TensorInfo (crates/rnb-loader/src/gguf/types.rs:103-110) plus where its bytes are."""
+
+    def __init__(self, owner: "GGUFFile", index: int, st: _GGUFTensorStruct):
+        self._owner = owner  # keeps the mapping alive while `data` is in use
+        self.index = index
+        self.name = st.name.decode()
+        self.shape = [int(st.shape[i]) for i in range(st.n_dims)]
+        self.ggml_type = int(st.ggml_type)
+        self.offset = int(st.offset)
+        self.file_offset = int(st.file_offset)
+        self.n_bytes = int(st.n_bytes)
+        self._addr = st.data
+
+    @property
+    def data(self) -> np.ndarray:
+        """The tensor's bytes inside the mapping (no copy)."""
+        if not self._addr:
+            raise BackendError(1, f"tensor '{self.name}' does not lie inside the file")
+        buf = (C.c_uint8 * self.n_bytes).from_address(self._addr)
+        arr = np.frombuffer(buf, dtype=np.uint8)
+        arr.flags.writeable = False
+        return arr
+
+    def prewarm(self) -> None:
+        _check(lib().rnb_hip_gguf_prewarm_tensor(self._owner._h, self.index))
+
+
+class GGUFFile:
+    """GGUFFile::parse (+ map_tensors when opened from a path).  `GGUFFile(path)` maps the file;
+    `GGUFFile.parse(bytes)` parses caller-owned bytes without the payload bounds checks."""
+
+    def __init__(self, path: Optional[str] = None, *, _handle=None, _keep=None):
+        self._keep = _keep
+        if _handle is not None:
+            self._h = _handle
+            return
+        h = _vp()
+        _check(lib().rnb_hip_gguf_open(os.fsencode(path), C.byref(h)))
+        self._h = h
+
+    @classmethod
+    def parse(cls, data) -> "GGUFFile":
+        view = np.frombuffer(data, dtype=np.uint8) if not isinstance(data, np.ndarray) else data
+        h = _vp()
+        _check(lib().rnb_hip_gguf_parse(_ptr(view) if view.size else None, view.size, C.byref(h)))
+        return cls(_handle=h, _keep=view)
+
+    def map_tensors(self) -> None:
+        _check(lib().rnb_hip_gguf_map_tensors(self._h))
+
+    def close(self) -> None:
+        if self._h:
+            lib().rnb_hip_gguf_close(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def version(self) -> int:
+        return int(lib().rnb_hip_gguf_version(self._h))
+
+    @property
+    def alignment(self) -> int:
+        return int(lib().rnb_hip_gguf_alignment(self._h))
+
+    @property
+    def data_start(self) -> int:
+        return int(lib().rnb_hip_gguf_data_start(self._h))
+
+    def __len__(self) -> int:
+        return int(lib().rnb_hip_gguf_tensor_count(self._h))
+
+    def tensor_at(self, index: int) -> GGUFTensor:
+        st = _GGUFTensorStruct()
+        _check(lib().rnb_hip_gguf_tensor_at(self._h, index, C.byref(st)))
+        return GGUFTensor(self, index, st)
+
+    def tensors(self) -> list:
+        return [self.tensor_at(i) for i in range(len(self))]
+
+    def tensor(self, name: str) -> GGUFTensor:
+        for i in range(len(self)):
+            t = self.tensor_at(i)
+            if t.name == name:
+                return t
+        st = _GGUFTensorStruct()
+        _check(lib().rnb_hip_gguf_find_tensor(self._h, name.encode(), C.byref(st)))
+        raise AssertionError("unreachable")
+
+    def metadata_keys(self) -> list:
+        n = int(lib().rnb_hip_gguf_metadata_count(self._h))
+        return [lib().rnb_hip_gguf_metadata_key(self._h, i).decode() for i in range(n)]
+
+    def metadata_type(self, key: str) -> int:
+        return int(lib().rnb_hip_gguf_metadata_type(self._h, key.encode()))
+
+    def metadata(self, key: str):
+        """Value of a key as a Python object (int, float, bool, str or list)."""
+        k = key.encode()
+        t = self.metadata_type(key)
+        if t < 0:
+            v = C.c_uint64()
+            _check(lib().rnb_hip_gguf_metadata_u64(self._h, k, C.byref(v)))  # raises "missing metadata key"
+        if t in (0, 2, 4, 10):
+            v = C.c_uint64()
+            _check(lib().rnb_hip_gguf_metadata_u64(self._h, k, C.byref(v)))
+            return int(v.value)
+        if t in (1, 3, 5, 11):
+            v = C.c_int64()
+            _check(lib().rnb_hip_gguf_metadata_i64(self._h, k, C.byref(v)))
+            return int(v.value)
+        if t in (6, 12):
+            v = C.c_double()
+            _check(lib().rnb_hip_gguf_metadata_f64(self._h, k, C.byref(v)))
+            return float(v.value)
+        if t == 7:
+            v = C.c_uint64()
+            _check(lib().rnb_hip_gguf_metadata_u64(self._h, k, C.byref(v)))
+            return bool(v.value)
+        if t == 8:
+            return lib().rnb_hip_gguf_metadata_str(self._h, k).decode()
+        et, n = C.c_uint32(), C.c_uint64()
+        _check(lib().rnb_hip_gguf_metadata_array(self._h, k, C.byref(et), C.byref(n)))
+        if et.value == 8:
+            return [lib().rnb_hip_gguf_metadata_array_str(self._h, k, i).decode() for i in range(n.value)]
+        if et.value == 9:
+            return [None] * n.value  # nested arrays are validated but not kept
+        out = []
+        for i in range(n.value):
+            v = C.c_double()
+            _check(lib().rnb_hip_gguf_metadata_array_f64(self._h, k, i, C.byref(v)))
+            out.append(v.value if et.value in (6, 12) else (bool(v.value) if et.value == 7 else int(v.value)))
+        return out
+
+
+def gguf_tensor_size(shape: Sequence[int], ggml_type: int) -> int:
+    """checked_tensor_size, crates/rnb-loader/src/convert.rs:28-43"""
+    arr = (C.c_uint64 * max(1, len(shape)))(*shape)
+    out = C.c_uint64()
+    _check(lib().rnb_hip_gguf_tensor_size(arr, len(shape), ggml_type, C.byref(out)))
+    return int(out.value)

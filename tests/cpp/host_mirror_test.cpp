@@ -53,6 +53,25 @@ static int validate() {
     EXPECT(!u && u.error == "Q4_K shape mismatch: input=256 output=0 expected input=256 output>=1", "into message");
     auto m = qwen35_sparse_experts_selected_base_by_token({w.data(), 144}, {w.data(), 144}, {w.data(), 144}, {0, 1}, {1.0f}, {0}, 1, 14, 256, 256, {x.data(), 256});
     EXPECT(!m && m.error.find("length mismatch") != std::string::npos, "moe slot arrays message");
+    {  // GGUF header parse over the C ABI: a minimal v3 file with one key, then a wrong magic
+        std::vector<uint8_t> f = {'G', 'G', 'U', 'F', 3, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0};
+        const char key[] = "general.architecture", val[] = "llama";
+        auto put_str = [&](const char *s) {
+            const uint64_t n = std::strlen(s);
+            for (int i = 0; i < 8; i++) f.push_back(static_cast<uint8_t>(n >> (8 * i)));
+            f.insert(f.end(), s, s + n);
+        };
+        put_str(key);
+        f.insert(f.end(), {8, 0, 0, 0});
+        put_str(val);
+        auto g = GgufFile::parse({f.data(), f.size()});
+        EXPECT(g && g.value.version() == 3 && g.value.tensor_count() == 0 && g.value.alignment() == 32 &&
+                   g.value.data_start() % 32 == 0 && g.value.metadata_str(key) == val,
+               "minimal GGUF v3 header");
+        f[0] = 'X';
+        auto bad = GgufFile::parse({f.data(), f.size()});
+        EXPECT(!bad && bad.error == "invalid GGUF magic bytes", "GGUF magic message");
+    }
     HipBackend b;
     EXPECT(b.kind() == 6, "kind ordinal");
     const BackendCapabilities c = b.capabilities();

@@ -1,0 +1,310 @@
+"""GGUF reader: the product parser (librnb_hip.so, C ABI) against the Python restatement in oracle/gguf_ref.py,
+both pinned on the reference's own parser / converter tests restated as byte strings
+(crates/rnb-loader/src/gguf/parser.rs:494-717, crates/rnb-loader/src/convert.rs:186-392)."""
+import math
+import os
+
+import numpy as np
+import pytest
+
+import runnburn_amd as rnb
+from oracle import gguf_ref
+from tests import gguf_writer as gw
+
+U64_MAX = (1 << 64) - 1
+
+
+def both_parse(data):
+    """Parses with the oracle and the product and checks that they agree; returns the oracle's view."""
+    ref = gguf_ref.parse(data)
+    g = rnb.GGUFFile.parse(data)
+    assert g.version == ref["version"] and g.alignment == ref["alignment"] and g.data_start == ref["data_start"]
+    assert g.metadata_keys() == [k for k, _, _ in ref["metadata"]]
+    for key, vtype, value in ref["metadata"]:
+        assert g.metadata_type(key) == vtype
+        got = g.metadata(key)
+        if vtype == gw.T_ARR and value and isinstance(value[0], list):
+            assert len(got) == len(value)
+        elif isinstance(value, float):
+            assert got == value or (math.isnan(got) and math.isnan(value))
+        else:
+            assert got == value, (key, got, value)
+    assert len(g) == len(ref["tensors"])
+    for i, t in enumerate(ref["tensors"]):
+        pt = g.tensor_at(i)
+        assert (pt.name, pt.shape, pt.ggml_type, pt.offset) == (t["name"], t["shape"], t["ggml_type"], t["offset"])
+    g.close()
+    return ref
+
+
+def both_reject(data, fragment):
+    with pytest.raises(gguf_ref.GGUFError) as ref:
+        gguf_ref.parse(data)
+    with pytest.raises(rnb.BackendError) as got:
+        rnb.GGUFFile.parse(data)
+    assert fragment in str(ref.value), str(ref.value)
+    assert str(got.value) == str(ref.value)  # same text, offset included
+    assert got.value.kind == "InvalidRequest"
+
+
+def minimal(arch="llama"):
+    return gw.Builder(3, 0, 1).kv("general.architecture", gw.T_STR, arch).pad().build()
+
+
+def with_tensor(arch="llama"):
+    b = gw.Builder(3, 1, 1).kv("general.architecture", gw.T_STR, arch)
+    b.tensor_info("token_embd.weight", [4, 8], 0, 0).pad().raw(bytes(128))
+    return b.build()
+
+
+# ---- the reference's accepted files -----------------------------------------------------------
+
+def test_minimal_v3():
+    ref = both_parse(minimal())
+    assert ref["version"] == 3 and ref["tensors"] == []
+    assert ref["metadata"] == [("general.architecture", gw.T_STR, "llama")]
+    assert ref["data_start"] % 32 == 0
+
+
+def test_tensor_info_dimensions_are_reversed_to_row_major():
+    ref = both_parse(with_tensor())
+    assert ref["tensors"] == [{"name": "token_embd.weight", "shape": [8, 4], "ggml_type": 0, "offset": 0}]
+
+
+def test_standard_64_bit_metadata():
+    b = gw.Builder(3, 0, 3).kv("test.uint64", gw.T_U64, U64_MAX - 7).kv("test.int64", gw.T_I64, -1_234_567_890_123)
+    ref = both_parse(b.kv("test.float64", gw.T_F64, math.pi).build())
+    assert [v for _, _, v in ref["metadata"]] == [U64_MAX - 7, -1_234_567_890_123, math.pi]
+
+
+def test_every_scalar_type_and_arrays_round_trip():
+    b = gw.Builder(3, 0, 12)
+    b.kv("a.u8", gw.T_U8, 200).kv("a.i8", gw.T_I8, -100).kv("a.u16", gw.T_U16, 65000).kv("a.i16", gw.T_I16, -30000)
+    b.kv("a.u32", gw.T_U32, 4_000_000_000).kv("a.i32", gw.T_I32, -2_000_000_000).kv("a.f32", gw.T_F32, 0.5)
+    b.kv("a.bool", gw.T_BOOL, 1).kv("a.str", gw.T_STR, "héllo")
+    b.kv("a.tokens", gw.T_ARR, ["<s>", "</s>", "ÿ"], gw.T_STR).kv("a.ints", gw.T_ARR, [1, -2, 3], gw.T_I32)
+    b.kv("a.floats", gw.T_ARR, [0.25, -8.0], gw.T_F32)
+    ref = both_parse(b.build())
+    assert ref["metadata"][8][2] == "héllo" and ref["metadata"][9][2] == ["<s>", "</s>", "ÿ"]
+
+
+def test_version_2_and_custom_alignment():
+    b = gw.Builder(2, 1, 1).kv("general.alignment", gw.T_U32, 64).tensor_info("w", [32], 8, 128).pad(64)
+    ref = both_parse(b.raw(bytes(128 + 34)).build())
+    assert ref["version"] == 2 and ref["alignment"] == 64 and ref["data_start"] % 64 == 0
+
+
+# ---- the reference's rejections, message fragments from its tests ----------------------------------
+
+def test_invalid_magic():
+    both_reject(b"XXXX\x03\x00\x00\x00" + bytes(16), "invalid GGUF magic bytes")
+
+
+def test_unsupported_version():
+    both_reject(gw.Builder(1, 0, 0).build(), "unsupported GGUF version: 1")
+
+
+def test_big_endian_is_named():
+    both_reject(gw.Builder(3, 0, 0, big_endian=True).build(), "big-endian")
+
+
+@pytest.mark.parametrize("build,fragment", [
+    (lambda: gw.Builder(3, 0, 1).string("test.bool").num("I", 7).num("B", 2), "boolean"),
+    (lambda: gw.Builder(3, 0, 1).kv("general.alignment", gw.T_U32, 24), "power of two"),
+    (lambda: gw.Builder(3, 0, 1).kv("general.alignment", gw.T_U32, 12), "alignment"),
+    (lambda: gw.Builder(3, 0, 1).kv("general.alignment", gw.T_U32, 0), "power of two"),
+    (lambda: gw.Builder(3, 0, 1).kv("general.alignment", gw.T_I32, -32), "non-negative integer"),
+    (lambda: gw.Builder(3, 0, 1).kv("general.alignment", gw.T_F32, 32.0), "non-negative integer"),
+    (lambda: gw.Builder(3, 0, U64_MAX), "metadata count"),
+    (lambda: gw.Builder(3, 0, 1_000_000), "cannot fit"),
+    (lambda: gw.Builder(3, 0, 1).string("test.string").num("I", 8).num("Q", gguf_ref.MAX_STRING_LENGTH + 1),
+     "string length"),
+    (lambda: gw.Builder(3, 0, 1).string("test.array").num("I", 9).num("I", 0).num("Q", gguf_ref.MAX_ARRAY_ELEMENTS + 1),
+     "array element count"),
+    (lambda: gw.Builder(3, 0, 1).string("test.array").num("I", 9).num("I", 0).num("Q", 1000).raw(bytes(10)),
+     "remaining bytes"),
+    (lambda: gw.Builder(3, 0, 1).string("test.array").num("I", 9).num("I", 99).num("Q", 0), "unknown GGUF value type"),
+    (lambda: gw.Builder(3, 0, 1).string("test.value").num("I", 13), "unknown GGUF value type"),
+    (lambda: gw.Builder(3, 0, 2).kv("test.key", gw.T_U8, 1).kv("test.key", gw.T_U8, 2), "duplicate metadata key"),
+    (lambda: gw.Builder(3, 0, 1).kv("", gw.T_U8, 1), "metadata key must be non-empty ASCII"),
+    (lambda: gw.Builder(3, 0, 1).kv("clé", gw.T_U8, 1), "metadata key must be non-empty ASCII"),
+    (lambda: gw.Builder(3, 0, 1).string(b"\xff\xfe").num("I", 0).num("B", 1), "invalid UTF-8"),
+    (lambda: gw.Builder(3, 2, 0).tensor_info("duplicate.weight", [1], 0, 0).tensor_info("duplicate.weight", [1], 0, 32),
+     "duplicate tensor name"),
+    (lambda: gw.Builder(3, 1, 0).tensor_info("x" * 64, [1], 0, 0), "tensor name"),
+    (lambda: gw.Builder(3, 1, 0).string("five.dims").num("I", 5).raw(bytes(64)), "at most 4"),
+    (lambda: gw.Builder(3, 1, 0).tensor_info("odd.type", [1], 99, 0), "unsupported GGML type: 99"),
+    (lambda: gw.Builder(3, 1, 0).tensor_info("odd.offset", [1], 0, 16), "is not aligned to 32 bytes"),
+    (lambda: gw.Builder(3, 0, 1).string("cut.short").num("I", 10).raw(b"\x01\x02"), "need 8 bytes, only 2 remain"),
+])
+def test_rejections(build, fragment):
+    both_reject(build().build(), fragment)
+
+
+def test_nesting_limit():
+    b = gw.Builder(3, 0, 1).string("deep").num("I", 9)
+    for _ in range(70):
+        b.num("I", 9).num("Q", 1)
+    both_reject(b.raw(bytes(64)).build(), "nesting exceeds 64 levels")
+
+
+def test_name_of_63_bytes_is_accepted():
+    both_parse(gw.Builder(3, 1, 0).tensor_info("y" * 63, [1], 0, 0).pad().raw(bytes(4)).build())
+
+
+# ---- tensor sizes and payload bounds (convert.rs) ------------------------------------------------------
+
+@pytest.mark.parametrize("shape,ggml_type,expected", [
+    ([4, 4], 0, 64), ([4, 4], 26, 64), ([4, 4], 1, 32), ([256], 2, 144), ([512], 12, 288), ([8, 4], 0, 128),
+    ([256], 16, 66), ([256], 17, 74), ([256], 18, 98), ([256], 19, 50), ([256], 21, 110), ([256], 22, 82),
+    ([256], 23, 136), ([256], 29, 56), ([256], 14, 210), ([14336, 4096], 12, 33030144), ([4096, 4096], 8, 17825792),
+    ([128, 768, 2048], 12, 113246208), ([], 0, 4),
+])
+def test_tensor_sizes(shape, ggml_type, expected):
+    assert gguf_ref.tensor_size(shape, ggml_type) == expected
+    assert rnb.gguf_tensor_size(shape, ggml_type) == expected
+
+
+def test_tensor_size_errors():
+    for shape, t, frag in [([31], 2, "not divisible by block size 32"), ([3, 100], 12, "block size 256"),
+                           ([1 << 40, 1 << 40], 0, "element count overflows usize"), ([4], 99, "unsupported GGML type")]:
+        with pytest.raises(gguf_ref.GGUFError) as ref:
+            gguf_ref.tensor_size(shape, t)
+        with pytest.raises(rnb.BackendError) as got:
+            rnb.gguf_tensor_size(shape, t)
+        assert frag in str(ref.value) and str(got.value) == str(ref.value)
+
+
+def test_map_tensors_bounds(tmp_path):
+    data = with_tensor()
+    ref = gguf_ref.parse(data)
+    assert gguf_ref.map_tensors(ref, len(data)) == {"token_embd.weight": (ref["data_start"], 128)}
+    g = rnb.GGUFFile.parse(data)
+    g.map_tensors()
+    t = g.tensor_at(0)
+    assert (t.file_offset, t.n_bytes, t.data.size) == (ref["data_start"], 128, 128)
+    g.close()
+    # one byte short: the header still parses, map_tensors refuses (convert.rs:283-298)
+    cut = data[:-1]
+    ref = gguf_ref.parse(cut)
+    with pytest.raises(gguf_ref.GGUFError) as e_ref:
+        gguf_ref.map_tensors(ref, len(cut))
+    g = rnb.GGUFFile.parse(cut)
+    with pytest.raises(rnb.BackendError) as e_got:
+        g.map_tensors()
+    assert "beyond file length" in str(e_ref.value) and str(e_got.value) == str(e_ref.value)
+    with pytest.raises(rnb.BackendError):
+        g.tensor_at(0).data
+    g.close()
+    # and opening the truncated file from disk fails the same way
+    p = tmp_path / "cut.gguf"
+    p.write_bytes(cut)
+    with pytest.raises(rnb.BackendError) as e_open:
+        rnb.GGUFFile(str(p))
+    assert str(e_open.value) == str(e_ref.value)
+
+
+def test_map_tensors_rejects_row_not_divisible_by_block():
+    b = gw.Builder(3, 1, 1).kv("general.architecture", gw.T_STR, "llama").tensor_info("test.weight", [31], 2, 0)
+    data = b.pad().raw(bytes(18)).build()
+    ref = gguf_ref.parse(data)
+    with pytest.raises(gguf_ref.GGUFError) as e_ref:
+        gguf_ref.map_tensors(ref, len(data))
+    g = rnb.GGUFFile.parse(data)
+    with pytest.raises(rnb.BackendError) as e_got:
+        g.map_tensors()
+    assert "block size" in str(e_ref.value) and str(e_got.value) == str(e_ref.value)
+    g.close()
+
+
+def test_open_missing_file_and_lookup_errors(tmp_path):
+    with pytest.raises(rnb.BackendError) as e:
+        rnb.GGUFFile(str(tmp_path / "absent.gguf"))
+    assert e.value.kind == "ExecutionFailed" and str(e.value).startswith("I/O error:")
+    g = rnb.GGUFFile.parse(with_tensor())
+    with pytest.raises(rnb.BackendError) as e:
+        g.tensor("nope")
+    assert str(e.value) == "missing tensor: nope"
+    with pytest.raises(rnb.BackendError) as e:
+        g.metadata("nope")
+    assert str(e.value) == "missing metadata key: nope"
+    with pytest.raises(rnb.BackendError) as e:
+        g.tensor_at(5)
+    assert "out of range" in str(e.value)
+    g.close()
+
+
+def test_file_with_quantised_tensors_maps_untouched_bytes(tmp_path):
+    """A model-shaped file: the bytes seen through the reader are the bytes written, at the offsets the oracle computes."""
+    from oracle import oracle as o
+    rows, cols = 6, 512
+    w4 = o.make_weights(o.Q4_K, rows, cols, 1)
+    w6 = o.make_weights(o.Q6_K, rows, cols, 2)
+    w8 = o.make_weights(o.Q8_0, rows, cols, 3)
+    norm = np.arange(cols, dtype=np.float32).view(np.uint8)
+    path = str(tmp_path / "m.gguf")
+    offs = gw.write_model(path, [("general.architecture", gw.T_STR, "llama"), ("llama.block_count", gw.T_U32, 1)],
+                          [("blk.0.ffn_gate.weight", [rows, cols], 12, w4), ("blk.0.ffn_down.weight", [rows, cols], 14, w6),
+                           ("output.weight", [rows, cols], 8, w8), ("output_norm.weight", [cols], 0, norm)])
+    raw = open(path, "rb").read()
+    ref = gguf_ref.parse(raw)
+    mapped = gguf_ref.map_tensors(ref, len(raw))
+    with rnb.GGUFFile(path) as g:
+        assert g.metadata("general.architecture") == "llama" and g.metadata("llama.block_count") == 1
+        for name, src in [("blk.0.ffn_gate.weight", w4), ("blk.0.ffn_down.weight", w6), ("output.weight", w8),
+                          ("output_norm.weight", norm)]:
+            t = g.tensor(name)
+            assert (t.file_offset, t.n_bytes) == mapped[name] == (offs[name], src.size)
+            assert t.file_offset % g.alignment == 0
+            assert np.array_equal(t.data, src)
+        assert g.tensor("blk.0.ffn_gate.weight").shape == [rows, cols]
+
+
+@pytest.mark.gpu
+def test_gguf_tensors_run_from_the_untouched_upload(rnb, oracle, tmp_path):
+    """File -> reader -> prewarm (upload as stored) -> GEMV / MoE on the mapped bytes == oracle on the same bytes."""
+    o = oracle
+    rows, cols = 40, 1024
+    w4 = o.make_weights(o.Q4_K, rows, cols, 11)
+    w6 = o.make_weights(o.Q6_K, rows, cols, 12)
+    w8 = o.make_weights(o.Q8_0, rows, cols, 13)
+    n_expert, n_ff, n_embd = 4, 256, 512
+    gate = o.make_weights(o.Q4_K, n_expert * n_ff, n_embd, 21)
+    up = o.make_weights(o.Q4_K, n_expert * n_ff, n_embd, 22)
+    down = o.make_weights(o.Q6_K, n_expert * n_embd, n_ff, 23)
+    path = str(tmp_path / "model.gguf")
+    gw.write_model(path, [("general.architecture", gw.T_STR, "qwen3moe")],
+                   [("blk.0.ffn_up.weight", [rows, cols], 12, w4), ("blk.0.ffn_down.weight", [rows, cols], 14, w6),
+                    ("output.weight", [rows, cols], 8, w8),
+                    ("blk.0.ffn_gate_exps.weight", [n_expert, n_ff, n_embd], 12, gate),
+                    ("blk.0.ffn_up_exps.weight", [n_expert, n_ff, n_embd], 12, up),
+                    ("blk.0.ffn_down_exps.weight", [n_expert, n_embd, n_ff], 14, down)])
+    x = o.fill_normal(cols, 31, 1.0)
+    with rnb.GGUFFile(path) as g:
+        before = rnb.resident_bytes()[0]
+        for t in g.tensors():
+            t.prewarm()
+        assert rnb.resident_bytes()[0] - before >= sum(t.n_bytes for t in g.tensors())
+        up_before = rnb.transfer_counters()[0]
+        for name, fn, q, src in [("blk.0.ffn_up.weight", rnb.q4k_gemv, o.Q4_K, w4),
+                                 ("blk.0.ffn_down.weight", rnb.q6k_gemv, o.Q6_K, w6),
+                                 ("output.weight", rnb.q8_0_gemv, o.Q8_0, w8)]:
+            t = g.tensor(name)
+            got = fn(t.data, t.shape[0], t.shape[1], x)
+            ref = o.gemv(q, src, rows, cols, x)[0]
+            assert np.allclose(got, ref, rtol=1e-3, atol=1e-3 * np.abs(ref).max()), name
+        # the weights were already resident: only activations went up
+        assert rnb.transfer_counters()[0] - up_before < 3 * (cols * 4 + 4096)
+        # one expert of a stacked tensor = a sub-range of the pinned upload (fanout.rs:4-22 slicing)
+        tg, tu, td = (g.tensor(f"blk.0.ffn_{k}_exps.weight") for k in ("gate", "up", "down"))
+        assert tg.shape == [n_expert, n_ff, n_embd] and td.shape == [n_expert, n_embd, n_ff]
+        ids = np.array([2, 0, 3], np.uint32)
+        route = np.array([0.5, 0.3, 0.2], np.float32)
+        toks = np.zeros(3, np.uint32)
+        h = o.fill_normal(n_embd, 41, 1.0)
+        got = rnb.qwen35_sparse_experts_selected_base_by_token(tg.data, tu.data, td.data, ids, route, toks, 1, o.Q6_K,
+                                                               n_ff, n_embd, h)
+        ref = o.moe_sparse_experts_by_token(gate, up, down, n_expert, ids, route, toks, 1, o.Q6_K, n_ff, n_embd, h)
+        assert np.allclose(got, ref, rtol=1e-3, atol=1e-3 * np.abs(ref).max())
+        for t in g.tensors():
+            rnb.release(t.data)
