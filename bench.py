@@ -364,6 +364,38 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed):
             "note": "events around the whole call (table upload + quantise + gate/up + re-quantise + down + reduce)"}
 
 
+def bench_ffn(rnb, hip, stream, tokens, steps, seed):
+    """Dense SwiGLU FFN of a Llama-3-8B layer through the device-resident operator: gate/up 14336x4096 Q4_K,
+    down 4096x14336 Q6_K; the three matrices are rotated over enough copies to stream from HBM."""
+    n_ff, n_embd = 14336, 4096
+    g = synth_weights(Q4_K, n_ff, n_embd, seed)
+    u = synth_weights(Q4_K, n_ff, n_embd, seed + 1)
+    d = synth_weights(Q6_K, n_embd, n_ff, seed + 2)
+    wbytes = g.nbytes + u.nbytes + d.nbytes
+    n_copies = copies_for(wbytes)
+    sets = [tuple(rnb.DeviceBuffer.from_host(a) for a in (g, u, d)) for _ in range(n_copies)]
+    x_dev = rnb.DeviceBuffer.from_host(np.random.default_rng(seed + 3).standard_normal(tokens * n_embd).astype(np.float32))
+    out_dev = rnb.DeviceBuffer(tokens * n_embd * 4)
+
+    def step(i):
+        gd, ud, dd = sets[i % n_copies]
+        rnb.dense_q4k_silu_ffn_dev(gd, ud, dd, Q6_K, n_ff, n_embd, tokens, x_dev, out_dev)
+
+    for i in range(10):
+        step(i)
+    n_k = min(steps, 300)
+    ms = float(np.mean([kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]))
+    nbytes = wbytes + tokens * (n_embd // 256 * 292 + n_ff // 256 * 292 + n_embd * 4)
+    for trio in sets:
+        for b in trio:
+            b.free()
+    x_dev.free()
+    out_dev.free()
+    return {"workload": f"dense SwiGLU FFN 4096 -> 14336 -> 4096 (Q4_K gate/up, Q6_K down), tokens={tokens}", "ms": ms,
+            "bytes": nbytes, "GB/s": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "copies": n_copies,
+            "note": "events around the whole call (quantise + fused gate/up/SiLU + re-quantise + down)"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -464,6 +496,10 @@ def main() -> int:
                 sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens)
             except Exception as exc:
                 sec[f"cfg5_moe_tokens{tokens}"] = {"error": str(exc)}
+        try:
+            sec["ffn_llama3_8b_tokens1"] = bench_ffn(rnb, hip, stream, 1, s2, 4321)
+        except Exception as exc:
+            sec["ffn_llama3_8b_tokens1"] = {"error": str(exc)}
         result["secondary"] = sec
 
     print(json.dumps(result), flush=True)

@@ -6,6 +6,8 @@
 //   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
 //   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
 //   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
+//   dense_q4k_silu_ffn_batch                    api/dense_api.rs:297-337
+//   GgufFile                                    crates/rnb-loader/src/gguf/parser.rs:16-24, 247-407
 //   HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
 //
 // `Result<T, String>` becomes rnb_hip::Result<T>: either a value or the reference's error message.
@@ -127,6 +129,17 @@ inline Result<std::vector<float>> qwen35_sparse_experts_selected_base_by_token(
         input.len, out.data(), out.size());
     if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
     return make_ok(std::move(out));
+}
+
+// dense_q4k_silu_ffn_batch, crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337
+inline Result<std::vector<float>> dense_q4k_silu_ffn_batch(Bytes gate_weights, Bytes up_weights, Bytes down_weights,
+                                                           uint32_t down_quant, size_t n_ff, size_t n_embd,
+                                                           size_t seq_len, Floats input) {
+    std::vector<float> out(seq_len * n_embd);
+    const int st = rnb_hip_dense_q4k_silu_ffn_batch(gate_weights.ptr, gate_weights.len, up_weights.ptr, up_weights.len,
+                                                    down_weights.ptr, down_weights.len, down_quant, n_ff, n_embd, seq_len,
+                                                    input.ptr, input.len, out.data(), out.size());
+    return st == RNB_HIP_OK ? make_ok(std::move(out)) : make_err<std::vector<float>>(st);
 }
 
 // trait Backend { kind, capabilities, execute }, crates/rnb-backend/api/src/lib.rs:1281-1285

@@ -155,6 +155,22 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
                                             uint32_t down_quant, size_t n_ff, size_t n_embd,
                                             const float *x_dev, float *out_dev);
 
+/* ---- dense SwiGLU FFN: the GEMV's neighbours fused into one call -------------------------------
+ * dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq_len, input) -> Vec<f32>,
+ * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337; validation order and texts from
+ * crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765 (seq_len > 1 required, as there).
+ * out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))): gate/up are Q4_K [n_ff][n_embd],
+ * down is [n_embd][n_ff] in Q4_K (12), Q6_K (14) or Q8_0 (8); codes 7 and 13 (Q5_1, Q5_K) are valid
+ * requests that return RNB_HIP_UNSUPPORTED_OP.  Intermediates never leave the device. */
+int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
+                                     size_t out_len);
+/* device-resident form (the reference's dev-input chain, dense.rs:2189-2219); also accepts one token */
+int rnb_hip_dense_q4k_silu_ffn_dev(const void *gate_dev, const void *up_dev, const void *down_dev,
+                                   uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq_len,
+                                   const float *x_dev, float *out_dev);
+
 /* ---- GGUF container: header, tensor table, untouched upload -------------------------------------
  * The reader side of the path: crates/rnb-loader/src/gguf/parser.rs:247-407 (GGUFFile::parse; same
  * limits, checks and message texts, reported through rnb_hip_last_error() with the Display strings of

@@ -206,6 +206,16 @@ def silu_mul(gate, up) -> np.ndarray:
     return g
 
 
+def dense_silu_ffn(gate, up, down, down_quant: int, n_ff: int, n_embd: int, x) -> np.ndarray:
+    """Dense SwiGLU FFN per token, composed of pinned pieces exactly as the reference's CPU path composes them
+    (gate/up GEMV on Q8_K(x), crates/rnb-cpu/src/kernels/activation.rs:73-89 fused_silu_mul, down GEMV on the
+    re-quantised intermediate): out[seq][n_embd]."""
+    g = gemv(Q4_K, gate, n_ff, n_embd, x)
+    u = gemv(Q4_K, up, n_ff, n_embd, x)
+    mid = silu_mul(g.ravel(), u.ravel()).reshape(g.shape)
+    return gemv(down_quant, down, n_embd, n_ff, mid)
+
+
 def route_topk(logits, k: int) -> tuple[np.ndarray, np.ndarray]:
     lg = _f32(logits)
     idx = np.zeros(min(k, lg.size), dtype=np.uint32)

@@ -28,6 +28,8 @@ from .binding import (  # noqa: F401
     OP_MATMUL,
     OP_MOE,
     STATUS_NAMES,
+    dense_q4k_silu_ffn_batch,
+    dense_q4k_silu_ffn_dev,
     device_available,
     device_name,
     gemv_dev,

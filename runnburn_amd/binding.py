@@ -49,6 +49,8 @@ SYMBOLS = [
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
+    ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
+    ("rnb_hip_dense_q4k_silu_ffn_dev", _i, [_vp, _vp, _vp, _u32, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gguf_open", _i, [C.c_char_p, C.POINTER(_vp)]),
     ("rnb_hip_gguf_parse", _i, [_vp, _sz, C.POINTER(_vp)]),
     ("rnb_hip_gguf_map_tensors", _i, [_vp]),
@@ -361,6 +363,23 @@ class HipBackend:
     def execute(self, request) -> None:
         raise BackendError(2, "HipBackend::execute: requests are served by the operator functions "
                               "(q4k_gemv, q6k_gemv, q8_0_gemv, *_batch, qwen35_sparse_experts_*)")
+
+
+def dense_q4k_silu_ffn_batch(gate_weights, up_weights, down_weights, down_quant: int, n_ff: int, n_embd: int,
+                             seq_len: int, input) -> np.ndarray:  # noqa: A002
+    """api/dense_api.rs:297-337; returns out[seq_len][n_embd]."""
+    g, u, d = _bytes_view(gate_weights), _bytes_view(up_weights), _bytes_view(down_weights)
+    x = _f32(input).ravel()
+    out = np.empty((seq_len, n_embd), dtype=np.float32)
+    _check(lib().rnb_hip_dense_q4k_silu_ffn_batch(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, down_quant, n_ff,
+                                                  n_embd, seq_len, _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+def dense_q4k_silu_ffn_dev(gate: "DeviceBuffer", up: "DeviceBuffer", down: "DeviceBuffer", down_quant: int, n_ff: int,
+                           n_embd: int, seq_len: int, x: "DeviceBuffer", out: "DeviceBuffer") -> None:
+    _check(lib().rnb_hip_dense_q4k_silu_ffn_dev(gate.ptr, up.ptr, down.ptr, down_quant, n_ff, n_embd, seq_len, x.ptr,
+                                                out.ptr))
 
 
 # ---- GGUF container (crates/rnb-loader/src/gguf/parser.rs, crates/rnb-loader/src/convert.rs) ---------------------

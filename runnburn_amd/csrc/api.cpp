@@ -173,6 +173,77 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
     return RNB_HIP_OK;
 }
 
+// ---- dense SwiGLU FFN -------------------------------------------------------------------------
+// out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), the composition the reference runs per token
+// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q6_K or Q8_0.
+
+// Validation order and messages: crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765.
+int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd,
+                       size_t seq, size_t x_len, bool batch_entry) {
+    if (batch_entry && seq <= 1)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch requires seq_len > 1, got " + std::to_string(seq));
+    if (x_len != seq * n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch input length mismatch: got " + std::to_string(x_len) +
+                                                 ", expected " + std::to_string(seq * n_embd));
+    const size_t down_block = (down_quant == 7 || down_quant == 8) ? 32 : 256;
+    if (n_embd % 256 != 0 || n_ff % down_block != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch dims must align to gate/down blocks, got n_ff=" +
+                                                 std::to_string(n_ff) + " down_block=" + std::to_string(down_block) +
+                                                 " n_embd=" + std::to_string(n_embd));
+    size_t down_row_bytes = 0;
+    switch (down_quant) {
+        case 7: down_row_bytes = n_ff / 32 * 24; break;
+        case 8: down_row_bytes = n_ff / 32 * 34; break;
+        case 12: down_row_bytes = n_ff / 256 * 144; break;
+        case 13: down_row_bytes = n_ff / 256 * 176; break;
+        case 14: down_row_bytes = n_ff / 256 * 210; break;
+        default:
+            return fail(RNB_HIP_INVALID_REQUEST,
+                        "unsupported dense SiLU FFN batch down quant code " + std::to_string(down_quant));
+    }
+    const size_t gate_bytes = n_ff * (n_embd / 256) * 144;
+    if (gate_len != gate_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch gate byte mismatch: got " + std::to_string(gate_len) +
+                                                 ", expected " + std::to_string(gate_bytes));
+    if (up_len != gate_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch up byte mismatch: got " + std::to_string(up_len) +
+                                                 ", expected " + std::to_string(gate_bytes));
+    if (down_len != n_embd * down_row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch down byte mismatch: got " + std::to_string(down_len) +
+                                                 ", expected " + std::to_string(n_embd * down_row_bytes));
+    if (down_quant == 7 || down_quant == 13)  // Q5_1 / Q5_K rows are valid requests that this backend does not run
+        return fail(RNB_HIP_UNSUPPORTED_OP,
+                    "dense SiLU FFN down quant code " + std::to_string(down_quant) + " is not built in the HIP backend");
+    if (n_ff > 0x7fffffffu || n_embd > 0x7fffffffu || seq > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN shape out of range");
+    return RNB_HIP_OK;
+}
+
+int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev,
+                      uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq, const float *x_dev, float *out_dev) {
+    const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
+    HIP_TRY(s.ffn_mid.reserve(mid_bytes));
+    ActView act;
+    int st = quantize_activations(s, kQ4K, x_dev, seq, n_embd, &act);
+    if (st != RNB_HIP_OK) return st;
+    const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
+    if (seq < kGemmMinSeq && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in))) {
+        launch_gemv_q4k_gate_up(gate_dev, up_dev, act, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
+                                static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), s.stream);
+    } else {
+        HIP_TRY(s.ffn_gate.reserve(mid_bytes));
+        HIP_TRY(s.ffn_up.reserve(mid_bytes));
+        st = run_matmul_quantized_dev(s, kQ4K, gate_dev, n_ff, n_embd, seq, s.ffn_gate.as<float>());
+        if (st != RNB_HIP_OK) return st;
+        st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>());
+        if (st != RNB_HIP_OK) return st;
+        launch_silu_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, s.stream);
+    }
+    HIP_TRY(hipGetLastError());
+    // the intermediate is re-quantised in the form the down projection's rows take, then the down matmul runs
+    return run_matmul_dev(s, down_quant, down_dev, n_embd, n_ff, s.ffn_mid.as<float>(), seq, out_dev);
+}
+
 // ---- MoE ------------------------------------------------------------------------------------
 
 struct MoeShape {
@@ -586,6 +657,68 @@ int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes) {
     HIP_TRY(hipStreamSynchronize(g.state->stream));
     g.state->d2h_bytes += bytes;
     return RNB_HIP_OK;
+}
+
+int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
+                                     size_t out_len) {
+    int st = validate_dense_ffn(gate_len, up_len, down_len, down_quant, n_ff, n_embd, seq_len, x_len, true);
+    if (st != RNB_HIP_OK) return st;
+    if (out_len < seq_len * n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch output length mismatch: got " + std::to_string(out_len) +
+                                                 ", expected at least " + std::to_string(seq_len * n_embd));
+    if (!gate || !up || !down || !x || !out) return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN null pointer argument");
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *gate_dev = nullptr, *up_dev = nullptr, *down_dev = nullptr;
+    HIP_TRY(s.resident_ptr(gate, gate_len, &gate_dev));
+    HIP_TRY(s.resident_ptr(up, up_len, &up_dev));
+    HIP_TRY(s.resident_ptr(down, down_len, &down_dev));
+    const size_t io_bytes = seq_len * n_embd * sizeof(float);
+    HIP_TRY(s.bounce_in.reserve(io_bytes));
+    HIP_TRY(s.bounce_out.reserve(io_bytes));
+    HIP_TRY(s.x_f32.reserve(io_bytes));
+    HIP_TRY(s.out_f32.reserve(io_bytes));
+    std::memcpy(s.bounce_in.ptr, x, io_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, io_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += io_bytes;
+    st = run_dense_ffn_dev(s, gate_dev, up_dev, down_dev, down_quant, n_ff, n_embd, seq_len, s.x_f32.as<float>(),
+                           s.out_f32.as<float>());
+    if (st != RNB_HIP_OK) return st;
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, io_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += io_bytes;
+    std::memcpy(out, s.bounce_out.ptr, io_bytes);
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_dense_q4k_silu_ffn_dev(const void *gate_dev, const void *up_dev, const void *down_dev, uint32_t down_quant,
+                                   size_t n_ff, size_t n_embd, size_t seq_len, const float *x_dev, float *out_dev) {
+    const size_t gate_bytes = n_embd % 256 == 0 ? n_ff * (n_embd / 256) * 144 : 0;
+    size_t down_bytes = 0;
+    switch (down_quant) {
+        case 8: down_bytes = n_ff % 32 == 0 ? n_embd * (n_ff / 32) * 34 : 0; break;
+        case 12: down_bytes = n_ff % 256 == 0 ? n_embd * (n_ff / 256) * 144 : 0; break;
+        case 14: down_bytes = n_ff % 256 == 0 ? n_embd * (n_ff / 256) * 210 : 0; break;
+        case 7: down_bytes = n_ff % 32 == 0 ? n_embd * (n_ff / 32) * 24 : 0; break;
+        case 13: down_bytes = n_ff % 256 == 0 ? n_embd * (n_ff / 256) * 176 : 0; break;
+        default: break;
+    }
+    int st = validate_dense_ffn(gate_bytes, gate_bytes, down_bytes, down_quant, n_ff, n_embd, seq_len, seq_len * n_embd,
+                                false);
+    if (st != RNB_HIP_OK) return st;
+    if (!gate_dev || !up_dev || !down_dev || !x_dev || !out_dev)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN null device pointer");
+    if ((reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev) |
+         reinterpret_cast<uintptr_t>(down_dev) | reinterpret_cast<uintptr_t>(x_dev)) & 15u)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN device pointers must be 16-byte aligned");
+    if (seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    return run_dense_ffn_dev(*g.state, static_cast<const uint8_t *>(gate_dev), static_cast<const uint8_t *>(up_dev),
+                             static_cast<const uint8_t *>(down_dev), down_quant, n_ff, n_embd, seq_len, x_dev, out_dev);
 }
 
 int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols, const float *x_dev, size_t seq_len,

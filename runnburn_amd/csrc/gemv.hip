@@ -92,6 +92,68 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
+// SwiGLU front half for decode-sized batches: mid[s][r] = silu(Wg[r] . a_s) * (Wu[r] . a_s) with one launch.  Same lane
+// mapping as gemv_kquant_kernel (rows of at most 16 super-blocks); a wave fetches row r of BOTH matrices against the
+// one activation slice it holds, so the activation is loaded once and gate/up never travel through memory.
+// SiLU as crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up.
+// ---------------------------------------------------------------------------------------------
+template <int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_q4k_gate_up_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
+                            const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ abs,
+                            float *__restrict__ mid, uint32_t rows, uint32_t nb, uint32_t row_groups) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const bool has_block = bslot < nb;
+    const uint32_t tok = blockIdx.y;
+    const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const Q4KAct a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
+        const uint32_t row = grp * kRowsPerWave + rsel;
+        float gs = 0.0f, us = 0.0f;
+        if (has_block && row < rows) {
+            const size_t off = static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes;
+            const Q4KRegs rg = q4k_load_block(wg + off, g), ru = q4k_load_block(wu + off, g);
+            gs = q4k_partial(rg, a4, g);
+            us = q4k_partial(ru, a4, g);
+        }
+        gs = seg_sum<kLanesPerRow>(gs);
+        us = seg_sum<kLanesPerRow>(us);
+        if (sub == kLanesPerRow - 1 && row < rows) {
+            const float e = expf(-gs);
+            mid[static_cast<size_t>(tok) * rows + row] = (gs / (1.0f + e)) * us;
+        }
+    }
+}
+
+template <int kRowsPerWave>
+void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
+                    uint32_t seq, hipStream_t stream) {
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu, act.qs,
+                       act.d, act.bsums, mid, rows, nb, row_groups);
+}
+
+__global__ void __launch_bounds__(256) silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
+                                                      float *__restrict__ out, size_t n) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const float gs = gate[i];
+        const float e = expf(-gs);
+        out[i] = (gs / (1.0f + e)) * up[i];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Long rows (more than 16 super-blocks): the K dimension is split across the waves of a workgroup, wave j
 // owning super-blocks [16j, 16j+16) of every row, so each lane's activation slice is loaded once and stays
 // in registers; the per-wave partial sums of kSplitRows consecutive rows meet in LDS and are added in
@@ -269,6 +331,26 @@ void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
     launch_kquant_any<true>(w, act, out, rows, nb, seq, stream);
+}
+
+bool gemv_q4k_gate_up_supported(uint32_t nb) { return nb >= 1 && nb <= 16; }
+
+void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
+                             uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    if (nb <= 4)
+        launch_gate_up<4>(wg, wu, act, mid, rows, nb, seq, stream);
+    else if (nb <= 8)
+        launch_gate_up<2>(wg, wu, act, mid, rows, nb, seq, stream);
+    else
+        launch_gate_up<1>(wg, wu, act, mid, rows, nb, seq, stream);
+}
+
+void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream) {
+    if (n == 0) return;
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
+                       gate, up, out, n);
 }
 
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,

@@ -41,6 +41,13 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,
                       uint32_t seq, hipStream_t stream);
 
+// SwiGLU front half, rows of at most 16 super-blocks: mid[s*rows + r] = silu(Wg[r] . a_s) * (Wu[r] . a_s)
+bool gemv_q4k_gate_up_supported(uint32_t nb);
+void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
+                             uint32_t seq, hipStream_t stream);
+// out[i] = silu(gate[i]) * up[i]
+void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream);
+
 // Q4_K x Q8_K GEMM on int8 MFMA; same contract as launch_gemv_q4k, intended for seq >= 16
 void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);

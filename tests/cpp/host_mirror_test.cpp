@@ -53,6 +53,16 @@ static int validate() {
     EXPECT(!u && u.error == "Q4_K shape mismatch: input=256 output=0 expected input=256 output>=1", "into message");
     auto m = qwen35_sparse_experts_selected_base_by_token({w.data(), 144}, {w.data(), 144}, {w.data(), 144}, {0, 1}, {1.0f}, {0}, 1, 14, 256, 256, {x.data(), 256});
     EXPECT(!m && m.error.find("length mismatch") != std::string::npos, "moe slot arrays message");
+    {
+        std::vector<uint8_t> gw(256 * 144, 0), dw(256 * 210, 0);
+        std::vector<float> xin(512, 0.0f);
+        auto f1 = dense_q4k_silu_ffn_batch({gw.data(), gw.size()}, {gw.data(), gw.size()}, {dw.data(), dw.size()}, 14, 256,
+                                           256, 1, {xin.data(), 256});
+        EXPECT(!f1 && f1.error == "dense SiLU FFN batch requires seq_len > 1, got 1", "dense ffn seq_len message");
+        auto f2 = dense_q4k_silu_ffn_batch({gw.data(), gw.size() - 1}, {gw.data(), gw.size()}, {dw.data(), dw.size()}, 14,
+                                           256, 256, 2, {xin.data(), 512});
+        EXPECT(!f2 && f2.error == "dense SiLU FFN batch gate byte mismatch: got 36863, expected 36864", "dense ffn gate bytes");
+    }
     {  // GGUF header parse over the C ABI: a minimal v3 file with one key, then a wrong magic
         std::vector<uint8_t> f = {'G', 'G', 'U', 'F', 3, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0};
         const char key[] = "general.architecture", val[] = "llama";

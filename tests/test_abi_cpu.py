@@ -123,3 +123,28 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower().replace("test oracle", ""), f"{f} mentions the oracle"
+
+
+def test_dense_ffn_validation_messages():
+    """crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765"""
+    z = np.zeros
+    f = rnb.dense_q4k_silu_ffn_batch
+    g = z(256 * 144, np.uint8)
+    e = _err(f, g, g, z(256 * 210, np.uint8), 14, 256, 256, 1, z(256, np.float32))
+    assert (e.kind, str(e)) == ("InvalidRequest", "dense SiLU FFN batch requires seq_len > 1, got 1")
+    e = _err(f, g, g, z(256 * 210, np.uint8), 14, 256, 256, 2, z(500, np.float32))
+    assert str(e) == "dense SiLU FFN batch input length mismatch: got 500, expected 512"
+    e = _err(f, g, g, z(10, np.uint8), 14, 300, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch dims must align to gate/down blocks, got n_ff=300 down_block=256 n_embd=256"
+    e = _err(f, g, g, z(10, np.uint8), 8, 250, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch dims must align to gate/down blocks, got n_ff=250 down_block=32 n_embd=256"
+    e = _err(f, g, g, z(10, np.uint8), 2, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "unsupported dense SiLU FFN batch down quant code 2"
+    e = _err(f, g[:-1], g, z(256 * 210, np.uint8), 14, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch gate byte mismatch: got 36863, expected 36864"
+    e = _err(f, g, g[:-2], z(256 * 210, np.uint8), 14, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch up byte mismatch: got 36862, expected 36864"
+    e = _err(f, g, g, z(256 * 210 + 1, np.uint8), 14, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch down byte mismatch: got 53761, expected 53760"
+    e = _err(f, g, g, z(256 * 176, np.uint8), 13, 256, 256, 2, z(512, np.float32))
+    assert e.kind == "UnsupportedOp"

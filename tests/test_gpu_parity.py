@@ -428,3 +428,35 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
         assert np.array_equal(solo[0], got[7])
     for w in (gate, up, down):
         rnb.release(w)
+
+
+# ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
+
+@pytest.mark.parametrize("down_quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("seq,n_ff,n_embd", [(2, 256, 256), (3, 768, 512), (5, 512, 4608), (17, 512, 768), (40, 1024, 256)])
+def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
+    """Decode-sized batches take the fused gate/up GEMV, 16+ tokens the MFMA GEMM + SiLU kernel, rows longer than
+    16 super-blocks the unfused pair; all must equal the per-token composition of the oracle's pinned pieces."""
+    gate = oracle.make_weights(Q4_K, n_ff, n_embd, 300 + seq)
+    up = oracle.make_weights(Q4_K, n_ff, n_embd, 301 + seq)
+    down = oracle.make_weights(down_quant, n_embd, n_ff, 302 + seq)
+    x = oracle.fill_normal(seq * n_embd, 303 + seq, 1.0)
+    got = rnb.dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
+    ref = oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x)
+    assert got.shape == ref.shape == (seq, n_embd)
+    check_close(got, ref, None, f"dense ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
+
+
+def test_dense_silu_ffn_dev_single_token_and_residency(rnb, oracle):
+    n_ff, n_embd = 1024, 512
+    gate = oracle.make_weights(Q4_K, n_ff, n_embd, 310)
+    up = oracle.make_weights(Q4_K, n_ff, n_embd, 311)
+    down = oracle.make_weights(Q6_K, n_embd, n_ff, 312)
+    x = oracle.fill_normal(n_embd, 313, 1.0)
+    bufs = [rnb.DeviceBuffer.from_host(a) for a in (gate, up, down, x)]
+    out = rnb.DeviceBuffer(n_embd * 4)
+    rnb.dense_q4k_silu_ffn_dev(bufs[0], bufs[1], bufs[2], Q6_K, n_ff, n_embd, 1, bufs[3], out)
+    got = out.to_host(np.float32).reshape(1, n_embd)
+    check_close(got, oracle.dense_silu_ffn(gate, up, down, Q6_K, n_ff, n_embd, x), None, "dense ffn one token, device")
+    for b in bufs + [out]:
+        b.free()
