@@ -155,6 +155,12 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
                                             uint32_t down_quant, size_t n_ff, size_t n_embd,
                                             const float *x_dev, float *out_dev);
 
+/* q6k_gemv_argmax(weights, rows, cols, input) -> (u32, f32), quant_api.rs:2170-2204: the LM-head GEMV with the
+ * arg-max taken on the device (larger value wins, ties go to the lower row, as in
+ * crates/rnb-backend/cuda/cuda/kernels/quant_batch_and_ops.cuh:3286-3328); 8 bytes come back instead of rows*4. */
+int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                            uint32_t *index_out, float *value_out);
+
 /* ---- dense SwiGLU FFN: the GEMV's neighbours fused into one call -------------------------------
  * dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq_len, input) -> Vec<f32>,
  * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337; validation order and texts from

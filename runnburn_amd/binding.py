@@ -49,6 +49,7 @@ SYMBOLS = [
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
+    ("rnb_hip_q6k_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_silu_ffn_dev", _i, [_vp, _vp, _vp, _u32, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gguf_open", _i, [C.c_char_p, C.POINTER(_vp)]),
@@ -363,6 +364,14 @@ class HipBackend:
     def execute(self, request) -> None:
         raise BackendError(2, "HipBackend::execute: requests are served by the operator functions "
                               "(q4k_gemv, q6k_gemv, q8_0_gemv, *_batch, qwen35_sparse_experts_*)")
+
+
+def q6k_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A002
+    """quant_api.rs:2170-2204 -> (row index, value)"""
+    w, x = _bytes_view(weights), _f32(input).ravel()
+    idx, val = _u32(), C.c_float()
+    _check(lib().rnb_hip_q6k_gemv_argmax(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
+    return int(idx.value), float(val.value)
 
 
 def dense_q4k_silu_ffn_batch(gate_weights, up_weights, down_weights, down_quant: int, n_ff: int, n_embd: int,

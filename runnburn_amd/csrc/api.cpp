@@ -659,6 +659,47 @@ int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes) {
     return RNB_HIP_OK;
 }
 
+int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                            uint32_t *index_out, float *value_out) {
+    QuantInfo qi;
+    quant_info(kQ6K, &qi);
+    size_t seq = 0;
+    // same three checks and texts as q6k_gemv (crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:2176-2193)
+    int st = validate_matmul(qi, w_len, rows, cols, x_len, rows, false, &seq);
+    if (st != RNB_HIP_OK) return st;
+    if (!w || !x || !index_out || !value_out) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K null pointer argument");
+    if (rows == 0) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K argmax needs at least one row");
+    if (rows > 0x7fffffffu) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K shape out of range");
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *w_dev = nullptr;
+    HIP_TRY(s.resident_ptr(w, w_len, &w_dev));
+    const size_t in_bytes = cols * sizeof(float);
+    HIP_TRY(s.bounce_in.reserve(in_bytes));
+    HIP_TRY(s.bounce_out.reserve(16));
+    HIP_TRY(s.x_f32.reserve(in_bytes));
+    HIP_TRY(s.out_f32.reserve(rows * sizeof(float)));
+    HIP_TRY(s.argmax_scratch.reserve(257 * 8));
+    std::memcpy(s.bounce_in.ptr, x, in_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += in_bytes;
+    st = run_matmul_dev(s, kQ6K, w_dev, rows, cols, s.x_f32.as<float>(), 1, s.out_f32.as<float>());
+    if (st != RNB_HIP_OK) return st;
+    float *vals = s.argmax_scratch.as<float>();
+    uint32_t *idxs = reinterpret_cast<uint32_t *>(vals + 257);
+    launch_argmax(s.out_f32.as<float>(), static_cast<uint32_t>(rows), vals, idxs, vals + 256, idxs + 256, s.stream);
+    HIP_TRY(hipGetLastError());
+    // only the winner crosses the bus: 8 bytes instead of rows * 4
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, vals + 256, 4, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipMemcpyAsync(static_cast<uint8_t *>(s.bounce_out.ptr) + 4, idxs + 256, 4, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += 8;
+    std::memcpy(value_out, s.bounce_out.ptr, 4);
+    std::memcpy(index_out, static_cast<uint8_t *>(s.bounce_out.ptr) + 4, 4);
+    return RNB_HIP_OK;
+}
+
 int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
                                      const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
                                      size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,

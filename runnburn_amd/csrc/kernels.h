@@ -45,6 +45,9 @@ void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, 
 bool gemv_q4k_gate_up_supported(uint32_t nb);
 void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
                              uint32_t seq, hipStream_t stream);
+// arg-max of `len` f32 (ties to the lower index); scratch_* hold 256 entries each, the result lands in out_*[0]
+void launch_argmax(const float *values, uint32_t len, float *scratch_values, uint32_t *scratch_indices, float *out_value,
+                   uint32_t *out_index, hipStream_t stream);
 // out[i] = silu(gate[i]) * up[i]
 void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream);
 

@@ -44,7 +44,49 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     q8_quantize_span(x + span * 256, lane, left < 8 ? static_cast<int>(left) : 8, qs + span * 256, d_out + span * 8);
 }
 
+// arg-max with the reference's rule (larger value, ties to the lower index; a NaN never wins; the search starts from
+// (-FLT_MAX, 0)): crates/rnb-backend/cuda/cuda/kernels/quant_batch_and_ops.cuh:3286-3328.  Stage 1 reduces `len`
+// values to one candidate per workgroup, stage 2 (one workgroup, in = stage 1's candidates) to the result.
+struct Best {
+    float val;
+    uint32_t idx;
+};
+__device__ __forceinline__ Best better(Best a, Best b) {
+    return (b.val > a.val || (b.val == a.val && b.idx < a.idx)) ? b : a;
+}
+__global__ void __launch_bounds__(256)
+    argmax_kernel(const float *__restrict__ values, const uint32_t *__restrict__ indices, uint32_t len,
+                  float *__restrict__ out_values, uint32_t *__restrict__ out_indices) {
+    __shared__ Best s_best[4];
+    Best b{-3.4028234663852886e38f, 0u};
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < len; i += gridDim.x * blockDim.x)
+        b = better(b, Best{values[i], indices != nullptr ? indices[i] : i});
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        Best o;
+        o.val = __shfl_xor(b.val, off, kWave);
+        o.idx = __shfl_xor(b.idx, off, kWave);
+        b = better(b, o);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) s_best[threadIdx.x >> 6] = b;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        b = better(better(s_best[0], s_best[1]), better(s_best[2], s_best[3]));
+        out_values[blockIdx.x] = b.val;
+        out_indices[blockIdx.x] = b.idx;
+    }
+}
+
 }  // namespace
+
+void launch_argmax(const float *values, uint32_t len, float *scratch_values, uint32_t *scratch_indices, float *out_value,
+                   uint32_t *out_index, hipStream_t stream) {
+    const uint32_t blocks = len == 0 ? 1 : (len + 255) / 256 < 256 ? (len + 255) / 256 : 256;
+    hipLaunchKernelGGL(argmax_kernel, dim3(blocks), dim3(256), 0, stream, values, nullptr, len, scratch_values,
+                       scratch_indices);
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(256), 0, stream, scratch_values, scratch_indices, blocks, out_value,
+                       out_index);
+}
 
 void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
                          hipStream_t stream) {

@@ -57,6 +57,7 @@ struct State {
     DeviceBuf act_qs;     // quantised activations: int8
     DeviceBuf act_d;      // per-block scales
     DeviceBuf act_bsums;  // per-16 sums (Q8_K)
+    DeviceBuf argmax_scratch;             // 257 values then 257 indices
     DeviceBuf ffn_gate, ffn_up, ffn_mid;  // dense FFN intermediates, f32 [seq][n_ff]
     DeviceBuf act_digits; // per-32 sums as two int8 digits (Q8_K, only filled for GEMM-sized batches)
     bool act_has_digits = false;

@@ -460,3 +460,23 @@ def test_dense_silu_ffn_dev_single_token_and_residency(rnb, oracle):
     check_close(got, oracle.dense_silu_ffn(gate, up, down, Q6_K, n_ff, n_embd, x), None, "dense ffn one token, device")
     for b in bufs + [out]:
         b.free()
+
+
+def test_q6k_gemv_argmax_matches_gemv_and_tie_rule(rnb, oracle):
+    """quant_api.rs:2170-2204; ties go to the lower row (quant_batch_and_ops.cuh:3299)."""
+    rows, cols = 3000, 512
+    w = oracle.make_weights(Q6_K, rows, cols, 500)
+    x = oracle.fill_normal(cols, 501, 1.0)
+    full = rnb.q6k_gemv(w, rows, cols, x)
+    idx, val = rnb.q6k_gemv_argmax(w, rows, cols, x)
+    assert idx == int(np.argmax(full)) and val == full[idx]
+    ref = oracle.gemv(Q6_K, w, rows, cols, x)[0]
+    assert idx == int(np.argmax(ref))
+    # duplicate the winning row further down: the first occurrence must still win
+    w2 = w.reshape(rows, -1).copy()
+    w2[rows - 5] = w2[idx]
+    w2[idx + 1 if idx + 1 < rows - 5 else 0] = w2[idx]
+    idx2, val2 = rnb.q6k_gemv_argmax(w2.reshape(-1), rows, cols, x)
+    assert idx2 == min(idx, idx + 1 if idx + 1 < rows - 5 else 0) and val2 == val
+    one, v1 = rnb.q6k_gemv_argmax(w[:cols // 256 * 210], 1, cols, x)
+    assert one == 0 and v1 == full[0]
