@@ -290,7 +290,7 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
     return res, w_host, x, out
 
 
-def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=8.0):
+def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=10.0):
     """The CPU leg: rnb-cpu's x86 path restated in oracle/ (AVX2+FMA dots, contiguous row chunks per
     thread), timed on this host; also checks the GPU result against it (abs-or-rel 1e-3)."""
     from oracle import oracle as ora
@@ -303,19 +303,34 @@ def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=8.0):
     ref = fn()
     for _ in range(2):
         fn()
-    times, t_start = [], time.perf_counter()
-    while len(times) < 200 and time.perf_counter() - t_start < budget_s:
+    # cache-resident figure first (one copy of the weights, a few hundred passes) ...
+    hot, t_start = [], time.perf_counter()
+    while len(hot) < 200 and time.perf_counter() - t_start < 2.0:
         t0 = time.perf_counter()
         fn()
+        hot.append(time.perf_counter() - t0)
+    # ... then the figure that is reported: the weights rotate over copies totalling more than the host's last-level
+    # caches, as the GPU leg rotates over more than the Infinity Cache, for about `budget_s` seconds of CPU work
+    n_copies = max(2, -(-(1 << 30) // max(1, w_host.nbytes)))
+    copies = [w_host] + [w_host.copy() for _ in range(n_copies - 1)]
+    run = (lambda w: ora.gemv(quant, w, rows, cols, x, avx2=True, n_threads=threads)) if ora.have_avx2() else \
+        (lambda w: ora.gemv(quant, w, rows, cols, x, n_threads=threads))
+    times, t_start, i = [], time.perf_counter(), 0
+    while time.perf_counter() - t_start < budget_s:
+        t0 = time.perf_counter()
+        run(copies[i % n_copies])
         times.append(time.perf_counter() - t0)
+        i += 1
     med = float(np.median(times))
     e = np.asarray(ref, np.float64).ravel()
     g = np.asarray(gpu_out, np.float64).ravel()
     tol = np.maximum(1e-3 * np.sqrt(np.mean(e * e)), 1e-3 * np.abs(e))
     ok = bool(np.all(np.abs(g - e) <= tol))
     return {"value": gemv_bytes(quant, rows, cols, x.size // cols) / med / 1e9, "unit": "GB/s", "cores": threads,
-            "kind": "port", "sample": f"{len(times)} full passes of the same {rows}x{cols} GEMV, median",
-            "ms": med * 1e3, "isa": "avx2+fma" if ora.have_avx2() else "scalar", "gpu_matches_cpu": ok}
+            "kind": "port",
+            "sample": f"{len(times)} full passes of the same {rows}x{cols} GEMV over {n_copies} rotating weight copies "
+                      f"({n_copies * w_host.nbytes / 1e6:.0f} MB, ~{budget_s:.0f} s of wall time), median per pass",
+            "ms": med * 1e3, "cache_resident_GB/s": gemv_bytes(quant, rows, cols, x.size // cols) / float(np.median(hot)) / 1e9, "isa": "avx2+fma" if ora.have_avx2() else "scalar", "gpu_matches_cpu": ok}
 
 
 def bench_moe(rnb, hip, stream, tokens, steps, seed):
