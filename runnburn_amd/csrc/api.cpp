@@ -302,6 +302,10 @@ int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t
     return RNB_HIP_OK;
 }
 
+// Up to this many slots (the reference's decode calls pass at most 32, fanout.rs:776-790) the down projection runs
+// token-major with the reduce fused in; beyond it expert-major, so that an expert is read once for all its tokens.
+constexpr size_t kMoeTokenMajorSlots = 32;
+
 // Device-side sequence for the gathered expert path.  x_dev [token_count][n_embd], out_dev likewise.
 int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev,
                 const MoeShape &sh, const uint32_t *expert_ids, const float *route, const uint32_t *token_ids,
@@ -323,8 +327,8 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     grp_start.push_back(static_cast<uint32_t>(n_slots));
     const size_t n_groups = grp_expert.size();
     // one table image: route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] | grp_expert[G] |
-    // grp_start[G+1]
-    const size_t table_words = 4 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
+    // grp_start[G+1] | slot_expert[n]
+    const size_t table_words = 5 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
     const bool inline_tables = table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
     MoeInlineTables inl;
     uint32_t *h = inl.words;
@@ -345,8 +349,9 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     float *h_route = reinterpret_cast<float *>(h);
     uint32_t *h_off = h + n_slots, *h_list = h_off + token_count + 1;
     uint32_t *h_sslot = h_list + n_slots, *h_stok = h_sslot + n_slots;
-    uint32_t *h_gexp = h_stok + n_slots, *h_gstart = h_gexp + n_groups;
+    uint32_t *h_gexp = h_stok + n_slots, *h_gstart = h_gexp + n_groups, *h_sexp = h_gstart + n_groups + 1;
     if (n_slots) std::memcpy(h_route, route, n_slots * 4);
+    if (n_slots) std::memcpy(h_sexp, expert_ids, n_slots * 4);
     std::vector<uint32_t> counts(token_count + 1, 0);
     for (size_t i = 0; i < n_slots; i++) counts[token_ids[i] + 1]++;
     for (size_t t = 0; t < token_count; t++) counts[t + 1] += counts[t];
@@ -404,10 +409,18 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
                         s.moe_mid_bsums.as<int16_t>(), nullptr, s.stream);
     ActView mid{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>()};
-    launch_moe_down(down_dev, down_quant, mid, groups, d_route, s.moe_slot_out.as<float>(),
-                    static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
-    launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
-                      static_cast<uint32_t>(n_embd), s.stream);
+    if (n_slots <= kMoeTokenMajorSlots && sh.nb_mid <= 16) {
+        // decode: few slots, every expert is read by one token anyway; one launch does down, route and the ordered sum
+        const uint32_t *d_sexp = d_list + 3 * n_slots + n_groups + (n_groups + 1);
+        launch_moe_down_token(down_dev, down_quant, mid, d_off, d_list, d_sexp, d_route, out_dev,
+                              static_cast<uint32_t>(token_count), static_cast<uint32_t>(n_embd),
+                              static_cast<uint32_t>(sh.nb_mid), s.stream);
+    } else {
+        launch_moe_down(down_dev, down_quant, mid, groups, d_route, s.moe_slot_out.as<float>(),
+                        static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
+        launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
+                          static_cast<uint32_t>(n_embd), s.stream);
+    }
     HIP_TRY(hipGetLastError());
     return RNB_HIP_OK;
 }

@@ -80,6 +80,10 @@ void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView 
 // slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])); mid_act is indexed by slot
 void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
                      const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
+// down + route weight + ordered per-token sum in one launch (rows of at most 16 super-blocks); slot_expert [n_slots]
+void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
+                           const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
+                           uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // out[token][n_embd] = sum of slot_out over the token's slots, in list order;
 // tok_offsets [token_count+1], tok_slots [n_slots] (CSR built by the host)
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,

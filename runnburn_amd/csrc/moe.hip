@@ -204,6 +204,58 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Decode-sized calls: down projection, route weight and the per-token ordered sum in one launch, no slot_out round
+// trip.  A wave owns ONE output row of one token; its lanes are split into 64/L groups of L = 4 * (blocks a group can
+// hold) lanes, each group dotting that row of a different slot's expert against that slot's quantised intermediate.
+// The groups' sums (last lane of each group) are then added in list order, so the result is the same sequence of f32
+// additions as moe_down_kernel followed by moe_reduce_kernel.
+// ---------------------------------------------------------------------------------------------
+template <bool kQ6, int kGroups>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    moe_down_token_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq,
+                          const float *__restrict__ md, const int16_t *__restrict__ mbs,
+                          const uint32_t *__restrict__ tok_offsets, const uint32_t *__restrict__ tok_slots,
+                          const uint32_t *__restrict__ slot_expert, const float *__restrict__ slot_route,
+                          float *__restrict__ out, uint32_t n_embd, uint32_t nb) {
+    constexpr int kLanes = kWave / kGroups;  // lanes per (slot, row) pair
+    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t row = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t tok = blockIdx.y;
+    if (row >= n_embd) return;  // wave-uniform
+    const int sub = lane & (kLanes - 1);
+    const uint32_t grp = lane / kLanes;
+    const int g = sub & 3;
+    const uint32_t b = sub >> 2;
+    const bool has_block = b < nb;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t begin = tok_offsets[tok], end = tok_offsets[tok + 1];
+    float acc = 0.0f;
+    for (uint32_t k0 = begin; k0 < end; k0 += kGroups) {
+        const uint32_t k = k0 + grp;
+        float o = 0.0f;
+        if (k < end && has_block) {
+            const uint32_t slot = tok_slots[k];
+            const uint8_t *blk = down_all + (static_cast<size_t>(slot_expert[slot]) * n_embd + row) * row_bytes +
+                                 static_cast<size_t>(b) * kBlockBytes;
+            const size_t ab = static_cast<size_t>(slot) * nb + b;
+            if constexpr (kQ6)
+                o = q6k_partial(q6k_load_block(blk, g), q6k_load_act(mq + ab * 256, md[ab], g), g);
+            else
+                o = q4k_partial(q4k_load_block(blk, g), q4k_load_act(mq + ab * 256, md[ab], mbs + ab * 16, g), g);
+        }
+        o = seg_sum<kLanes>(o);
+        if (k < end) o *= slot_route[tok_slots[k]];  // fanout.rs:306-308; only the group's last lane is read below
+#pragma unroll
+        for (int j = 0; j < kGroups; j++) {
+            const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
+            if (k0 + j < end) acc += v;  // wave-uniform
+        }
+    }
+    if (lane == 0) out[static_cast<size_t>(tok) * n_embd + row] = acc;
+}
+
 __global__ void __launch_bounds__(256)
     moe_reduce_kernel(const float *__restrict__ slot_out, const uint32_t *__restrict__ tok_offsets,
                       const uint32_t *__restrict__ tok_slots, float *__restrict__ out, uint32_t n_embd) {
@@ -279,6 +331,25 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
         if (q6) RNB_LAUNCH_DOWN(true, 1); else RNB_LAUNCH_DOWN(false, 1);
     }
 #undef RNB_LAUNCH_DOWN
+}
+
+void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
+                           const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
+                           uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
+    if (token_count == 0) return;
+    const dim3 grid((n_embd + kWavesPerWg - 1) / kWavesPerWg, token_count, 1), block(kWave * kWavesPerWg);
+#define RNB_LAUNCH_DT(Q6, G)                                                                                          \
+    hipLaunchKernelGGL((moe_down_token_kernel<Q6, G>), grid, block, 0, stream, down_all, mid_act.qs, mid_act.d,       \
+                       mid_act.bsums, tok_offsets, tok_slots, slot_expert, slot_route, out, n_embd, nb_mid)
+    const bool q6 = down_quant == kQ6K;
+    if (nb_mid <= 4) {
+        if (q6) RNB_LAUNCH_DT(true, 4); else RNB_LAUNCH_DT(false, 4);
+    } else if (nb_mid <= 8) {
+        if (q6) RNB_LAUNCH_DT(true, 2); else RNB_LAUNCH_DT(false, 2);
+    } else {
+        if (q6) RNB_LAUNCH_DT(true, 1); else RNB_LAUNCH_DT(false, 1);
+    }
+#undef RNB_LAUNCH_DT
 }
 
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots, float *out,
