@@ -187,6 +187,26 @@ def calibration_copy(hip, rnb, stream, nbytes=64 << 20, reps=5):
     log(f"calibration copy: {reps} x {nbytes} bytes device-to-device")
 
 
+def copy_context(hip, rnb, stream, nbytes):
+    """Context for the roofline line: what the runtime's own device-to-device copy reaches on buffers of the size of
+    one launch's weights (it reads nbytes and writes nbytes), rotating over enough buffer pairs to miss the 256 MiB
+    Infinity Cache.  Reported as total traffic (2 * nbytes per copy) over time; informative only."""
+    pairs = max(2, -(-2 * MALL_BYTES // (2 * nbytes)))
+    bufs = [(rnb.DeviceBuffer(nbytes), rnb.DeviceBuffer(nbytes)) for _ in range(pairs)]
+
+    def one(i):
+        src, dst = bufs[i % pairs]
+        hip.check(hip.rt.hipMemcpyAsync(dst.ptr, src.ptr, nbytes, 3, stream), "hipMemcpyAsync")
+
+    for i in range(pairs):
+        one(i)
+    ms = kernel_time_ms(hip, stream, one, 200)
+    for a, b in bufs:
+        a.free()
+        b.free()
+    return {"bytes_copied": nbytes, "ms": ms, "read_plus_write_GB/s": 2 * nbytes / ms / 1e6}
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of `kernel`, from the committed counter summary (two rocprofv3 --pmc runs, FETCH_SIZE and
     WRITE_SIZE, each scaled by the same counter's reading for the calibration copy); None when absent."""
@@ -471,6 +491,10 @@ def main() -> int:
                      "kernel_ms_runs": main_res["kernel_ms_runs"],
                      "timing": "HIP events around back-to-back launches on the library stream, 3 runs"},
     }
+    try:  # what a plain device copy of the same number of bytes reaches on this box, for context
+        result["roofline"]["device_copy_same_size"] = copy_context(hip, rnb, stream, 33030144)
+    except Exception as exc:
+        log(f"copy context skipped: {exc}")
     if "kernel_ms_mean_cache_resident" in main_res:
         result["roofline"]["cache_resident_GBps"] = nbytes / main_res["kernel_ms_mean_cache_resident"] / 1e6
     if not args.no_cpu_baseline:
