@@ -47,6 +47,8 @@ int hip_fail(const char *what, hipError_t e) {
 // Quantise seq*cols staged floats on the device into the state's activation scratch.
 // Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
 constexpr size_t kGemmMinSeq = 16;
+// Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
+constexpr size_t kTokensMinSeq = 4;
 
 int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view) {
     const size_t n = seq * cols;
@@ -88,14 +90,20 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), quant == kQ8_0 ? nullptr : s.act_bsums.as<int16_t>(),
                       quant != kQ8_0 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
+    const uint32_t nb = static_cast<uint32_t>(cols / 256);
     if (quant == kQ4K) {
-        // the GEMM fills LDS with 16-byte loads: weights at other alignments take the per-token kernel
+        // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
         if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
-            launch_gemm_q4k_mfma(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+            launch_gemm_q4k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
+        else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
+            launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
         else
-            launch_gemv_q4k(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+            launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ6K) {
-        launch_gemv_q6k(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 256), q, s.stream);
+        if (seq >= kTokensMinSeq)
+            launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
+        else
+            launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else {
         launch_gemv_q8_0(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     }

@@ -51,6 +51,11 @@ void launch_argmax(const float *values, uint32_t len, float *scratch_values, uin
 // out[i] = silu(gate[i]) * up[i]
 void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream);
 
+// Multi-token matmul on the vector ALUs for Q4_K / Q6_K (weights decoded once per eight staged tokens);
+// same output contract as launch_gemv_q4k
+void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream);
+
 // Q4_K x Q8_K GEMM on int8 MFMA; same contract as launch_gemv_q4k, intended for seq >= 16
 void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);
