@@ -255,7 +255,7 @@ def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols
 # ---- batches: seq-major layout, ragged token counts ----------------------------------------------
 
 @pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
-@pytest.mark.parametrize("seq", [2, 3, 15])
+@pytest.mark.parametrize("seq", [2, 3, 4, 9, 15, 33])
 def test_gemv_batch_small(rnb, oracle, quant, seq):
     rows, cols = 37, 768
     w = oracle.make_weights(quant, rows, cols, 50 + quant)
@@ -268,13 +268,14 @@ def test_gemv_batch_small(rnb, oracle, quant, seq):
 
 @pytest.mark.parametrize("quant", [Q4_K, Q6_K])
 def test_gemv_batch_long_rows(rnb, oracle, quant):
-    """Rows longer than 16 super-blocks take the K-split kernel; several tokens ride on grid.y."""
-    rows, cols, seq = 21, 20 * 256, 3
-    w = oracle.make_weights(quant, rows, cols, 150 + quant)
-    x = oracle.fill_normal(seq * cols, 160, 1.0)
-    got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
-    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
-                f"long-row batch quant {quant}")
+    """Rows longer than 16 super-blocks: the K-split kernel with tokens on grid.y up to 3 tokens, the staged
+    multi-token kernel from 4 tokens on."""
+    for rows, cols, seq in ((21, 20 * 256, 3), (19, 20 * 256, 11), (5, 56 * 256, 6)):
+        w = oracle.make_weights(quant, rows, cols, 150 + quant)
+        x = oracle.fill_normal(seq * cols, 160, 1.0)
+        got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+        check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                    f"long-row batch quant {quant} rows {rows} seq {seq}")
 
 
 @pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
