@@ -17,6 +17,9 @@
  *   quantize_q8                 closed-form cases + numpy restatement (formula is 6 lines)
  *   dot_q4k_q8k                 reference closed forms 0 / 0 / 2560.0 (tile_q4k.rs:2019-2151),
  *                               f64 numpy dequant(W) . dequant(Q8K(x)) identity
+ *   dot_q5k_q8k                 one-hot fifth-bit vectors (each qh bit moves exactly the element the
+ *                               reference's tile_q5k.rs:944-976 statement names), f64 numpy dequant
+ *                               identity, reduction to dot_q4k_q8k when qh == 0
  *   dot_q6k_q8k                 f64 numpy dequant identity; bsums identity (avx2_dot.rs:824,880)
  *   dot_q8_0_*                  reference vector 528.0 (quant_gemv.rs:1448-1464), numpy identity
  *   gemv drivers                seq-major layout vector (quant_gemv.rs:1448-1464)
@@ -27,6 +30,8 @@
  *   quantize_row_q4_k           PARITY UNPINNED at byte level (needs the Rust original); only the
  *                               reference's round-trip property (quant.rs:766-798) is checked.
  *                               Input generation only -- GPU and oracle consume identical bytes.
+ *   quantize_row_q5_k           as quantize_row_q4_k: byte parity UNPINNED, the reference's round-trip
+ *                               property (quant.rs:732-764) is checked.  Input generation only.
  *   quantize_row_q6_k/_q8_0     not in the reference at all (ggml reference semantics); round
  *                               trip through the pinned dequantisers.  Input generation only.
  */
@@ -157,6 +162,36 @@ void rnbo_dequantize_q4_k(const uint8_t *blocks, size_t n_blocks, float *out) {
             float d2 = d * (float)sc2, m2 = dmin * (float)mn2;
             for (int l = 0; l < 32; l++) y[64 * g + l] = d1 * (float)(q[32 * g + l] & 0x0f) - m1;
             for (int l = 0; l < 32; l++) y[64 * g + 32 + l] = d2 * (float)(q[32 * g + l] >> 4) - m2;
+        }
+    }
+}
+
+/* crates/rnb-cpu/src/quantize/dequant.rs:735-770: Q4_K's walk with a fifth bit per element, bit 2g of
+ * qh[l] for the low-nibble half of group g and bit 2g+1 for the high-nibble half. */
+void rnbo_dequantize_q5_k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * RNBO_Q5_K_BLOCK_BYTES;
+        float d = rd_f16(blk);
+        float dmin = rd_f16(blk + 2);
+        const uint8_t *qh = blk + 16, *ql = blk + 48;
+        float *y = out + b * 256;
+        uint8_t u1 = 1, u2 = 2;
+        for (int g = 0; g < 4; g++) {
+            uint8_t sc1, mn1, sc2, mn2;
+            rnbo_get_scale_min_k4(2 * g, blk + 4, &sc1, &mn1);
+            rnbo_get_scale_min_k4(2 * g + 1, blk + 4, &sc2, &mn2);
+            float d1 = d * (float)sc1, m1 = dmin * (float)mn1;
+            float d2 = d * (float)sc2, m2 = dmin * (float)mn2;
+            for (int l = 0; l < 32; l++) {
+                uint8_t v = (uint8_t)((ql[32 * g + l] & 0x0f) + ((qh[l] & u1) ? 16 : 0));
+                y[64 * g + l] = d1 * (float)v - m1;
+            }
+            for (int l = 0; l < 32; l++) {
+                uint8_t v = (uint8_t)((ql[32 * g + l] >> 4) + ((qh[l] & u2) ? 16 : 0));
+                y[64 * g + 32 + l] = d2 * (float)v - m2;
+            }
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
         }
     }
 }
@@ -304,6 +339,60 @@ double rnbo_dot_q4k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_
     return acc;
 }
 
+/* integer part of one Q5_K block: crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 */
+static inline void q5k_block_ints(const uint8_t *blk, const rnbo_q8k_block *a, int32_t *sumi_out,
+                                  int32_t *summ_out) {
+    const uint8_t *qh = blk + 16, *qs = blk + 48;
+    int32_t sumi = 0, summ = 0;
+    for (int g = 0; g < 4; g++) {
+        uint8_t sc0, mn0, sc1, mn1;
+        rnbo_get_scale_min_k4(2 * g, blk + 4, &sc0, &mn0);
+        rnbo_get_scale_min_k4(2 * g + 1, blk + 4, &sc1, &mn1);
+        const uint8_t u1 = (uint8_t)(1u << (2 * g)), u2 = (uint8_t)(2u << (2 * g));
+        int32_t i0 = 0, i1 = 0;
+        for (int l = 0; l < 32; l++) {
+            int32_t w0 = (int32_t)(qs[32 * g + l] & 0x0f) + ((qh[l] & u1) ? 16 : 0);
+            int32_t w1 = (int32_t)(qs[32 * g + l] >> 4) + ((qh[l] & u2) ? 16 : 0);
+            i0 += w0 * (int32_t)a->qs[64 * g + l];
+            i1 += w1 * (int32_t)a->qs[64 * g + 32 + l];
+        }
+        sumi += (int32_t)sc0 * i0 + (int32_t)sc1 * i1;
+        summ += (int32_t)mn0 * bsum32(a, 2 * g) + (int32_t)mn1 * bsum32(a, 2 * g + 1);
+    }
+    *sumi_out = sumi;
+    *summ_out = summ;
+}
+
+/* crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 (dot_q5_k_q8k_scalar); the same per-block formula as the
+ * test oracle crates/rnb-cpu/src/gemm/tile_q5k.rs:979-1036 (q5k_q8k_exact_ref) */
+float rnbo_dot_q5k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q5_K_BLOCK_BYTES;
+        float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        int32_t sumi, summ;
+        q5k_block_ints(blk, &act[b], &sumi, &summ);
+        volatile float t0 = d * (float)sumi;
+        volatile float t1 = dmin * (float)summ;
+        volatile float t2 = t0 - t1;
+        volatile float t3 = act[b].d * t2;
+        acc += t3;
+    }
+    return acc;
+}
+
+double rnbo_dot_q5k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    double acc = 0.0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q5_K_BLOCK_BYTES;
+        double d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        int32_t sumi, summ;
+        q5k_block_ints(blk, &act[b], &sumi, &summ);
+        acc += (double)act[b].d * (d * (double)sumi - dmin * (double)summ);
+    }
+    return acc;
+}
+
 /* integer part of one Q6_K block: crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 */
 static inline int32_t q6k_block_int(const uint8_t *blk, const rnbo_q8k_block *a) {
     const uint8_t *ql = blk, *qh = blk + 128;
@@ -406,8 +495,25 @@ static size_t block_bytes_of(uint32_t quant, size_t *elems) {
     switch (quant) {
     case 8: *elems = 32; return RNBO_Q8_0_BLOCK_BYTES;
     case 12: *elems = 256; return RNBO_Q4_K_BLOCK_BYTES;
+    case 13: *elems = 256; return RNBO_Q5_K_BLOCK_BYTES;
     case 14: *elems = 256; return RNBO_Q6_K_BLOCK_BYTES;
     default: *elems = 0; return 0;
+    }
+}
+
+static float kquant_dot(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    switch (quant) {
+    case 12: return rnbo_dot_q4k_q8k(row, act, nb);
+    case 13: return rnbo_dot_q5k_q8k(row, act, nb);
+    default: return rnbo_dot_q6k_q8k(row, act, nb);
+    }
+}
+
+static double kquant_dot_f64(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    switch (quant) {
+    case 12: return rnbo_dot_q4k_q8k_f64(row, act, nb);
+    case 13: return rnbo_dot_q5k_q8k_f64(row, act, nb);
+    default: return rnbo_dot_q6k_q8k_f64(row, act, nb);
     }
 }
 
@@ -444,9 +550,7 @@ int rnbo_gemv(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const 
 #pragma omp parallel for schedule(static) num_threads(n_threads)
     for (long r = 0; r < (long)rows; r++)
         for (size_t s = 0; s < seq_len; s++)
-            out[s * rows + r] = (quant == 12)
-                                    ? rnbo_dot_q4k_q8k(w + r * row_bytes, act + s * nb, nb)
-                                    : rnbo_dot_q6k_q8k(w + r * row_bytes, act + s * nb, nb);
+            out[s * rows + r] = kquant_dot(quant, w + r * row_bytes, act + s * nb, nb);
     free(act);
     return 0;
 }
@@ -475,9 +579,7 @@ int rnbo_gemv_f64(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, co
 #pragma omp parallel for schedule(static) num_threads(n_threads)
     for (long r = 0; r < (long)rows; r++)
         for (size_t s = 0; s < seq_len; s++)
-            out[s * rows + r] = (quant == 12)
-                                    ? rnbo_dot_q4k_q8k_f64(w + r * row_bytes, act + s * nb, nb)
-                                    : rnbo_dot_q6k_q8k_f64(w + r * row_bytes, act + s * nb, nb);
+            out[s * rows + r] = kquant_dot_f64(quant, w + r * row_bytes, act + s * nb, nb);
     free(act);
     return 0;
 }
@@ -554,7 +656,7 @@ size_t rnbo_route_topk(const float *logits, size_t n_expert, size_t k, uint32_t 
 /* One slot: crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:260-327
  * (compute_expert_host_from_slices): gate/up GEMV on Q8_K(h), SiLU*up, down GEMV on the
  * re-quantised intermediate, scale by the route weight.  Gate/up are Q4_K; down is
- * Q4_K (12) or Q6_K (14).  `h_q8k` is the token's already-quantised activation. */
+ * Q4_K (12), Q5_K (13) or Q6_K (14).  `h_q8k` is the token's already-quantised activation. */
 static void moe_slot(const uint8_t *gate, const uint8_t *up, const uint8_t *down,
                      uint32_t down_quant, size_t n_ff, size_t n_embd, const rnbo_q8k_block *h_q8k,
                      float route_weight, float *gate_out, float *up_out, rnbo_q8k_block *mid_q8k,
@@ -567,10 +669,10 @@ static void moe_slot(const uint8_t *gate, const uint8_t *up, const uint8_t *down
     }
     rnbo_silu_mul_inplace(gate_out, up_out, n_ff);
     rnbo_quantize_q8k(gate_out, n_ff, mid_q8k);
-    size_t down_row = nb_mid * (down_quant == 12 ? RNBO_Q4_K_BLOCK_BYTES : RNBO_Q6_K_BLOCK_BYTES);
+    size_t elems;
+    size_t down_row = nb_mid * block_bytes_of(down_quant, &elems);
     for (size_t r = 0; r < n_embd; r++) {
-        float o = (down_quant == 12) ? rnbo_dot_q4k_q8k(down + r * down_row, mid_q8k, nb_mid)
-                                     : rnbo_dot_q6k_q8k(down + r * down_row, mid_q8k, nb_mid);
+        float o = kquant_dot(down_quant, down + r * down_row, mid_q8k, nb_mid);
         volatile float scaled = o * route_weight; /* fanout.rs:306-308 */
         expert_out[r] = scaled;
     }
@@ -588,13 +690,13 @@ int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_
                                      uint32_t down_quant, size_t n_ff, size_t n_embd,
                                      const float *x, float *out, int n_threads) {
     if (n_ff % 256 != 0 || n_embd % 256 != 0) return 1;
-    if (down_quant != 12 && down_quant != 14) return 1;
+    if (down_quant != 12 && down_quant != 13 && down_quant != 14) return 1;
     for (size_t s = 0; s < n_slots; s++)
         if (expert_ids[s] >= n_expert || token_ids[s] >= token_count) return 1;
     size_t nb_in = n_embd / 256, nb_mid = n_ff / 256;
     size_t per_gate = n_ff * nb_in * RNBO_Q4_K_BLOCK_BYTES;
-    size_t per_down =
-        n_embd * nb_mid * (down_quant == 12 ? RNBO_Q4_K_BLOCK_BYTES : RNBO_Q6_K_BLOCK_BYTES);
+    size_t down_elems;
+    size_t per_down = n_embd * nb_mid * block_bytes_of(down_quant, &down_elems);
     n_threads = resolve_threads(n_threads);
 
     rnbo_q8k_block *h_q8k = (rnbo_q8k_block *)malloc(sizeof(rnbo_q8k_block) * nb_in * token_count);
@@ -710,67 +812,102 @@ static float make_qkx2_quants(int n, int nmax, const float *x, const float *weig
     return scale;
 }
 
+/* Shared front half of the Q4_K and Q5_K quantisers (crates/rnb-cpu/src/quantize/quant.rs:312-378 and
+ * :456-545, which differ only in nmax = 15 / 31): per-sub-block fit, 6-bit packing of the sub-block
+ * scales and mins into `ys`, f16 super-block scales into hdr[0..4), then the element codes L re-derived
+ * from the rounded scales. */
+static void kquant_min_codes(const float *x, int nmax, uint8_t *hdr, uint8_t *ys, uint8_t *L) {
+    uint8_t Laux[32];
+    float mins[8], scales[8], weights[32];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 8; j++) {
+        const float *xs = x + 32 * j;
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
+        float av_x = sqrtf(sum_x2 / 32.0f);
+        for (int l = 0; l < 32; l++) weights[l] = av_x + fabsf(xs[l]);
+        float sub_min = 0.0f;
+        float s = make_qkx2_quants(32, nmax, xs, weights, L + 32 * j, &sub_min, Laux, -0.5f, 0.1f, 15);
+        scales[j] = s;
+        mins[j] = sub_min;
+        if (s > max_scale) max_scale = s;
+        if (sub_min > max_min) max_min = sub_min;
+    }
+    float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    memset(ys, 0, 12);
+    for (int j = 0; j < 8; j++) {
+        int ls = rnbo_nearest_int(inv_scale * scales[j]);
+        int lm = rnbo_nearest_int(inv_min * mins[j]);
+        ls = ls < 0 ? 0 : (ls > 63 ? 63 : ls);
+        lm = lm < 0 ? 0 : (lm > 63 ? 63 : lm);
+        if (j < 4) {
+            ys[j] = (uint8_t)ls;
+            ys[j + 4] = (uint8_t)lm;
+        } else {
+            ys[j + 4] = (uint8_t)((ls & 0x0f) | ((lm & 0x0f) << 4));
+            ys[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            ys[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    wr_f16(hdr, max_scale / 63.0f);
+    wr_f16(hdr + 2, max_min / 63.0f);
+    float d_round = rd_f16(hdr), dmin_round = rd_f16(hdr + 2);
+    for (int j = 0; j < 8; j++) {
+        uint8_t sc, mn;
+        rnbo_get_scale_min_k4(j, ys, &sc, &mn);
+        float d_sub = d_round * (float)sc;
+        if (d_sub == 0.0f) continue;
+        float dm_sub = dmin_round * (float)mn;
+        for (int ii = 0; ii < 32; ii++) {
+            int l = rnbo_nearest_int((x[32 * j + ii] + dm_sub) / d_sub);
+            L[32 * j + ii] = (uint8_t)(l < 0 ? 0 : (l > nmax ? nmax : l));
+        }
+    }
+}
+
 /* crates/rnb-cpu/src/quantize/quant.rs:289-413 (quantize_row_q4_k).
  * Byte parity with the Rust original is UNPINNED (cannot run it); input generation only. */
 void rnbo_quantize_row_q4_k(const float *input, size_t n, uint8_t *output) {
     size_t nb = n / 256;
-    uint8_t L[256], Laux[32];
-    float mins[8], scales[8], weights[32];
+    uint8_t L[256], ys[12];
     for (size_t i = 0; i < nb; i++) {
-        const float *x = input + i * 256;
-        float max_scale = 0.0f, max_min = 0.0f;
-        for (int j = 0; j < 8; j++) {
-            const float *xs = x + 32 * j;
-            float sum_x2 = 0.0f;
-            for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
-            float av_x = sqrtf(sum_x2 / 32.0f);
-            for (int l = 0; l < 32; l++) weights[l] = av_x + fabsf(xs[l]);
-            float sub_min = 0.0f;
-            float s = make_qkx2_quants(32, 15, xs, weights, L + 32 * j, &sub_min, Laux, -0.5f, 0.1f,
-                                       15);
-            scales[j] = s;
-            mins[j] = sub_min;
-            if (s > max_scale) max_scale = s;
-            if (sub_min > max_min) max_min = sub_min;
-        }
-        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
-        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
-        uint8_t ys[12];
-        memset(ys, 0, 12);
-        for (int j = 0; j < 8; j++) {
-            int ls = rnbo_nearest_int(inv_scale * scales[j]);
-            int lm = rnbo_nearest_int(inv_min * mins[j]);
-            ls = ls < 0 ? 0 : (ls > 63 ? 63 : ls);
-            lm = lm < 0 ? 0 : (lm > 63 ? 63 : lm);
-            if (j < 4) {
-                ys[j] = (uint8_t)ls;
-                ys[j + 4] = (uint8_t)lm;
-            } else {
-                ys[j + 4] = (uint8_t)((ls & 0x0f) | ((lm & 0x0f) << 4));
-                ys[j - 4] |= (uint8_t)((ls >> 4) << 6);
-                ys[j] |= (uint8_t)((lm >> 4) << 6);
-            }
-        }
         uint8_t *out = output + i * RNBO_Q4_K_BLOCK_BYTES;
-        wr_f16(out, max_scale / 63.0f);
-        wr_f16(out + 2, max_min / 63.0f);
-        float d_round = rd_f16(out), dmin_round = rd_f16(out + 2);
-        for (int j = 0; j < 8; j++) {
-            uint8_t sc, mn;
-            rnbo_get_scale_min_k4(j, ys, &sc, &mn);
-            float d_sub = d_round * (float)sc;
-            if (d_sub == 0.0f) continue;
-            float dm_sub = dmin_round * (float)mn;
-            for (int ii = 0; ii < 32; ii++) {
-                int l = rnbo_nearest_int((x[32 * j + ii] + dm_sub) / d_sub);
-                L[32 * j + ii] = (uint8_t)(l < 0 ? 0 : (l > 15 ? 15 : l));
-            }
-        }
+        kquant_min_codes(input + i * 256, 15, out, ys, L);
         memcpy(out + 4, ys, 12);
         uint8_t *qs = out + 16;
         for (int g = 0; g < 4; g++)
             for (int j = 0; j < 32; j++)
                 qs[32 * g + j] = (uint8_t)((L[64 * g + j] & 0x0f) | ((L[64 * g + j + 32] & 0x0f) << 4));
+    }
+}
+
+/* crates/rnb-cpu/src/quantize/quant.rs:433-585 (quantize_row_q5_k): 5-bit codes, the low four bits in
+ * qs as for Q4_K, the fifth in qh (bit 2g for the first half of group g, bit 2g+1 for the second).
+ * Byte parity with the Rust original is UNPINNED (cannot run it); input generation only. */
+void rnbo_quantize_row_q5_k(const float *input, size_t n, uint8_t *output) {
+    size_t nb = n / 256;
+    uint8_t L[256], ys[12];
+    for (size_t i = 0; i < nb; i++) {
+        uint8_t *out = output + i * RNBO_Q5_K_BLOCK_BYTES;
+        kquant_min_codes(input + i * 256, 31, out, ys, L);
+        memcpy(out + 4, ys, 12);
+        uint8_t *qh = out + 16, *qs = out + 48;
+        memset(qh, 0, 32);
+        for (int g = 0; g < 4; g++) {
+            for (int j = 0; j < 32; j++) {
+                int l1 = L[64 * g + j], l2 = L[64 * g + j + 32];
+                if (l1 > 15) {
+                    l1 -= 16;
+                    qh[j] |= (uint8_t)(1u << (2 * g));
+                }
+                if (l2 > 15) {
+                    l2 -= 16;
+                    qh[j] |= (uint8_t)(2u << (2 * g));
+                }
+                qs[32 * g + j] = (uint8_t)(l1 | (l2 << 4));
+            }
+        }
     }
 }
 
@@ -936,6 +1073,8 @@ int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, f
             uint8_t *dst = out + (size_t)r * row_bytes;
             if (quant == 12)
                 rnbo_quantize_row_q4_k(row, cols, dst);
+            else if (quant == 13)
+                rnbo_quantize_row_q5_k(row, cols, dst);
             else if (quant == 14)
                 rnbo_quantize_row_q6_k(row, cols, dst);
             else

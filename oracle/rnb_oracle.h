@@ -26,6 +26,7 @@ extern "C" {
 #define RNBO_QK_K 256
 #define RNBO_Q8_0_BLOCK_BYTES 34
 #define RNBO_Q4_K_BLOCK_BYTES 144
+#define RNBO_Q5_K_BLOCK_BYTES 176
 #define RNBO_Q6_K_BLOCK_BYTES 210
 
 /* Q8_K activation block, crates/rnb-cpu/src/gemm/activation_q8.rs:66-72 (repr(C), 292 B). */
@@ -50,6 +51,7 @@ int rnbo_nearest_int(float fval);
 /* ---- dequantisers (element order of the formats) -------------------------------- */
 void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out);
 void rnbo_dequantize_q4_k(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_q5_k(const uint8_t *blocks, size_t n_blocks, float *out);
 void rnbo_dequantize_q6_k(const uint8_t *blocks, size_t n_blocks, float *out);
 
 /* ---- activation quantisers (bit-exact contract) --------------------------------- */
@@ -58,16 +60,18 @@ void rnbo_quantize_q8(const float *x, size_t n, rnbo_q8_block *out);
 
 /* ---- row dots ------------------------------------------------------------------- */
 float rnbo_dot_q4k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_q5k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 float rnbo_dot_q6k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 float rnbo_dot_q8_0_q8(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
 float rnbo_dot_q8_0_f32(const uint8_t *row, const float *x, size_t n_blocks);
 /* f64-accumulated "gold" forms of the same integer arithmetic */
 double rnbo_dot_q4k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+double rnbo_dot_q5k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 double rnbo_dot_q6k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 double rnbo_dot_q8_0_q8_f64(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
 
 /* ---- GEMV / GEMM drivers: out[s*rows + row], x is [seq_len][cols] --------------- */
-/* quant: 8 = Q8_0 (Q8 x Q8_0 integer form), 12 = Q4_K, 14 = Q6_K (ggml type ids).  */
+/* quant: 8 = Q8_0 (Q8 x Q8_0 integer form), 12 = Q4_K, 13 = Q5_K, 14 = Q6_K (ggml type ids).  */
 int rnbo_gemv(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
               size_t seq_len, float *out, int n_threads);
 int rnbo_gemv_f64(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
@@ -89,6 +93,7 @@ int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_
 
 /* ---- input generation (not on the GPU path) ------------------------------------- */
 void rnbo_quantize_row_q4_k(const float *x, size_t n, uint8_t *out);
+void rnbo_quantize_row_q5_k(const float *x, size_t n, uint8_t *out);
 void rnbo_quantize_row_q6_k(const float *x, size_t n, uint8_t *out);
 void rnbo_quantize_row_q8_0(const float *x, size_t n, uint8_t *out);
 void rnbo_fill_normal(float *out, size_t n, uint64_t seed, float sigma);

@@ -24,6 +24,7 @@ bool quant_info(uint32_t quant, QuantInfo *qi) {
     switch (quant) {
     case kQ8_0: *qi = {"Q8_0", 32, kQ8_0Bytes}; return true;
     case kQ4K: *qi = {"Q4_K", 256, kQ4KBytes}; return true;
+    case kQ5K: *qi = {"Q5_K", 256, kQ5KBytes}; return true;
     case kQ6K: *qi = {"Q6_K", 256, kQ6KBytes}; return true;
     default: return false;
     }
@@ -99,6 +100,11 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);
+    } else if (quant == kQ5K) {
+        if (seq >= kTokensMinSeq)
+            launch_matmul_tokens(w_dev, kQ5K, act, out_dev, r, nb, q, s.stream);
+        else
+            launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ6K) {
         if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
@@ -183,7 +189,7 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
 
 // ---- dense SwiGLU FFN -------------------------------------------------------------------------
 // out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), the composition the reference runs per token
-// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q6_K or Q8_0.
+// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K or Q8_0.
 
 // Validation order and messages: crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765.
 int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd,
@@ -219,7 +225,7 @@ int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t
     if (down_len != n_embd * down_row_bytes)
         return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch down byte mismatch: got " + std::to_string(down_len) +
                                                  ", expected " + std::to_string(n_embd * down_row_bytes));
-    if (down_quant == 7 || down_quant == 13)  // Q5_1 / Q5_K rows are valid requests that this backend does not run
+    if (down_quant == 7)  // Q5_1 rows are a valid request that this backend does not run
         return fail(RNB_HIP_UNSUPPORTED_OP,
                     "dense SiLU FFN down quant code " + std::to_string(down_quant) + " is not built in the HIP backend");
     if (n_ff > 0x7fffffffu || n_embd > 0x7fffffffu || seq > 65535u)
@@ -275,6 +281,7 @@ int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t
     size_t down_block;
     switch (down_quant) {
     case kQ4K: down_block = kQ4KBytes; break;
+    case kQ5K: down_block = kQ5KBytes; break;
     case kQ6K: down_block = kQ6KBytes; break;
     default:
         return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported Qwen35 HIP down quant code " + std::to_string(down_quant));
@@ -442,8 +449,8 @@ int rnb_hip_backend_kind(void) { return 6; }
 int rnb_hip_backend_supports(int op) { return (op == RNB_OP_MATMUL || op == RNB_OP_MOE) ? 1 : 0; }
 
 int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
-    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || quant == kQ4K || quant == kQ6K) ? 1 : 0;
-    if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ6K) ? 1 : 0;
+    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
+    if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
     return 0;
 }
 
@@ -586,6 +593,14 @@ int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, c
 int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                            float *out, size_t out_len) {
     return matmul_host(kQ4K, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+int rnb_hip_q5k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                     float *out, size_t out_len) {
+    return matmul_host(kQ5K, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q5k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                           float *out, size_t out_len) {
+    return matmul_host(kQ5K, w, w_len, rows, cols, x, x_len, out, out_len, true);
 }
 int rnb_hip_q6k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                      float *out, size_t out_len) {
@@ -845,9 +860,10 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
     if (n_embd == 0 || n_ff == 0 || n_embd % 256 != 0 || n_ff % 256 != 0)
         return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer dims must be divisible by 256, got n_ff=" +
                                                  std::to_string(n_ff) + " n_embd=" + std::to_string(n_embd));
-    const size_t down_block = down_quant == kQ4K ? kQ4KBytes : kQ6KBytes;
-    if (down_quant != kQ4K && down_quant != kQ6K)
+    QuantInfo down_qi;
+    if ((down_quant != kQ4K && down_quant != kQ5K && down_quant != kQ6K) || !quant_info(down_quant, &down_qi))
         return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported Qwen35 HIP down quant code " + std::to_string(down_quant));
+    const size_t down_block = down_qi.bytes;
     MoeShape sh;
     sh.nb_in = n_embd / 256;
     sh.nb_mid = n_ff / 256;

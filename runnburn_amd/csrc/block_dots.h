@@ -2,6 +2,7 @@
 // the decode GEMV and the gathered-MoE kernels.  FOUR lanes cooperate on a 256-element block (a wave64
 // pass covers 16 blocks); the caller adds the partials across lanes.  Activations are held in
 // registers (`Q4KAct` / `Q6KAct`) so that a wave which walks many rows loads them once.
+// `KQuant<id>` at the end gives the kernels one interface over the three K-quant formats.
 #pragma once
 
 #include "device_utils.h"
@@ -102,6 +103,49 @@ __device__ __forceinline__ float q4k_dot(const Q4KPrep &p, const Q4KAct &a) {
 
 __device__ __forceinline__ float q4k_partial(const Q4KRegs &r, const Q4KAct &a, int g) {
     return q4k_dot(q4k_prepare(r, g), a);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q5_K: block = {f16 d, f16 dmin, u8 scales[12], u8 qh[32], u8 qs[128]}, 176 bytes.  Q4_K's element order
+// with a fifth bit: element 64g + l takes bit 2g of qh[l], element 64g + 32 + l bit 2g+1.  Lane g reads the
+// header, all of qh and its 32 bytes of qs; once the fifth bits are merged the values (0..31) sit one per
+// byte exactly as a prepared Q4_K slice does, so the activation state and the dot are Q4_K's.
+//                                                        crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800
+// ---------------------------------------------------------------------------------------------
+struct Q5KRegs {
+    uint4 h, qh0, qh1, qa, qb;
+};
+
+__device__ __forceinline__ Q5KRegs q5k_load_block(const uint8_t *__restrict__ blk, int g) {
+    Q5KRegs r;
+    r.h = *reinterpret_cast<const uint4 *>(blk);
+    r.qh0 = *reinterpret_cast<const uint4 *>(blk + 16);
+    r.qh1 = *reinterpret_cast<const uint4 *>(blk + 32);
+    r.qa = *reinterpret_cast<const uint4 *>(blk + 48 + 32 * g);
+    r.qb = *reinterpret_cast<const uint4 *>(blk + 64 + 32 * g);
+    return r;
+}
+
+__device__ __forceinline__ Q4KPrep q5k_prepare(const Q5KRegs &r, int g) {
+    Q4KRegs r4;
+    r4.h = r.h;
+    r4.qa = r.qa;
+    r4.qb = r.qb;
+    Q4KPrep p = q4k_prepare(r4, g);
+    const int s = 2 * g;  // bit s -> low-nibble half, bit s+1 -> high-nibble half; moved to bit 4 of each byte
+#define RNB_Q5_BITS(dst_lo, dst_hi, src, k)                          \
+    p.dst_lo.k |= ((r.src.k >> s) & 0x01010101u) << 4;               \
+    p.dst_hi.k |= ((r.src.k >> (s + 1)) & 0x01010101u) << 4;
+    RNB_Q5_BITS(lo0, hi0, qh0, x)
+    RNB_Q5_BITS(lo0, hi0, qh0, y)
+    RNB_Q5_BITS(lo0, hi0, qh0, z)
+    RNB_Q5_BITS(lo0, hi0, qh0, w)
+    RNB_Q5_BITS(lo1, hi1, qh1, x)
+    RNB_Q5_BITS(lo1, hi1, qh1, y)
+    RNB_Q5_BITS(lo1, hi1, qh1, z)
+    RNB_Q5_BITS(lo1, hi1, qh1, w)
+#undef RNB_Q5_BITS
+    return p;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -207,6 +251,61 @@ __device__ __forceinline__ float q6k_dot(const Q6KPrep &p, const Q6KAct &a) {
 
 __device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, int q) {
     return q6k_dot(q6k_prepare(r, q), a);
+}
+
+// ---------------------------------------------------------------------------------------------
+// One interface over the K-quant formats for the kernels that are templated on the ggml type id.
+// `bs_blk` (the activation block's 16 int16 sums) is ignored by Q6_K, whose rows have no mins.
+// ---------------------------------------------------------------------------------------------
+template <uint32_t kQuant>
+struct KQuant;
+
+template <>
+struct KQuant<kQ4K> {
+    static constexpr size_t kBytes = kQ4KBytes;
+    using Act = Q4KAct;
+    using Regs = Q4KRegs;
+    using Prep = Q4KPrep;
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *bs_blk, int g) {
+        return q4k_load_act(aq_blk, dx, bs_blk, g);
+    }
+    static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int g) { return q4k_load_block(blk, g); }
+    static __device__ __forceinline__ Prep prepare(const Regs &r, int g) { return q4k_prepare(r, g); }
+    static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q4k_dot(p, a); }
+};
+
+template <>
+struct KQuant<kQ5K> {
+    static constexpr size_t kBytes = kQ5KBytes;
+    using Act = Q4KAct;
+    using Regs = Q5KRegs;
+    using Prep = Q4KPrep;
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *bs_blk, int g) {
+        return q4k_load_act(aq_blk, dx, bs_blk, g);
+    }
+    static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int g) { return q5k_load_block(blk, g); }
+    static __device__ __forceinline__ Prep prepare(const Regs &r, int g) { return q5k_prepare(r, g); }
+    static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q4k_dot(p, a); }
+};
+
+template <>
+struct KQuant<kQ6K> {
+    static constexpr size_t kBytes = kQ6KBytes;
+    using Act = Q6KAct;
+    using Regs = Q6KRegs;
+    using Prep = Q6KPrep;
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *, int q) {
+        return q6k_load_act(aq_blk, dx, q);
+    }
+    static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q6k_load_block(blk, q); }
+    static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q6k_prepare(r, q); }
+    static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q6k_dot(p, a); }
+};
+
+template <uint32_t kQuant>
+__device__ __forceinline__ float kquant_partial(const typename KQuant<kQuant>::Regs &r,
+                                                const typename KQuant<kQuant>::Act &a, int g) {
+    return KQuant<kQuant>::dot(KQuant<kQuant>::prepare(r, g), a);
 }
 
 }  // namespace rnb

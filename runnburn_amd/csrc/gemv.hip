@@ -1,6 +1,7 @@
 // Decode GEMV kernels: one packed GGUF row x one quantised activation vector -> one f32.
 //
 //  Q4_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:884-916   (dot_q4_k_q8k_scalar)
+//  Q5_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 (dot_q5_k_q8k_scalar)
 //  Q6_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 (dot_q6_k_q8k_scalar)
 //  Q8_0 x Q8   : crates/rnb-cpu/src/gemm/neon_dot.rs:376-436   (dot_q8_0_q8_neon)
 //  driver      : crates/rnb-cpu/src/gemm/quant_gemv.rs:403-536, out[s*rows + row]
@@ -12,7 +13,6 @@
 // registers once per wave instead of once per row.  Integer sums per lane are exact
 // (v_dot4_i32_i8); the per-block f32 scale is applied once per lane and the partial sums are added
 // across lanes on the DPP path, so results differ from the scalar reference only by f32 summation order.
-#include <type_traits>
 
 #include "block_dots.h"
 #include "device_utils.h"
@@ -26,16 +26,17 @@ constexpr int kWavesPerWg = 4;
 constexpr uint32_t kTargetWaves = 4096;  // total waves per launch: enough loads in flight, short tail
 
 // ---------------------------------------------------------------------------------------------
-// K-quant GEMV (Q4_K and Q6_K share the structure; only the block functions differ)
+// K-quant GEMV (Q4_K, Q5_K and Q6_K share the structure; only the block functions differ)
 // ---------------------------------------------------------------------------------------------
-template <bool kQ6, int kRowsPerWave>
+template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_kquant_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                        const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
                        uint32_t row_groups) {
+    using Q = KQuant<kQuant>;
     constexpr int kLanesPerRow = kWave / kRowsPerWave;
     constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
-    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    constexpr size_t kBlockBytes = Q::kBytes;
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane & (kLanesPerRow - 1);
     const uint32_t rsel = lane / kLanesPerRow;
@@ -51,21 +52,13 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         // the whole row fits one pass: this lane's activation slice stays in registers for every row
         const bool has_block = bslot < nb;
         const size_t ab = abase + (has_block ? bslot : 0);
-        Q4KAct a4{};
-        Q6KAct a6{};
-        if constexpr (kQ6)
-            a6 = q6k_load_act(aq + ab * 256, ad[ab], g);
-        else
-            a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+        const typename Q::Act a = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
         for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
             const uint32_t row = grp * kRowsPerWave + rsel;
             float acc = 0.0f;
             if (has_block && row < rows) {
                 const uint8_t *blk = w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kBlockBytes;
-                if constexpr (kQ6)
-                    acc = q6k_partial(q6k_load_block(blk, g), a6, g);
-                else
-                    acc = q4k_partial(q4k_load_block(blk, g), a4, g);
+                acc = kquant_partial<kQuant>(Q::load_block(blk, g), a, g);
             }
             acc = seg_sum<kLanesPerRow>(acc);
             if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
@@ -79,10 +72,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                 for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                     const uint8_t *blk = rowp + static_cast<size_t>(b) * kBlockBytes;
                     const size_t ab = abase + b;
-                    if constexpr (kQ6)
-                        acc += q6k_partial(q6k_load_block(blk, g), q6k_load_act(aq + ab * 256, ad[ab], g), g);
-                    else
-                        acc += q4k_partial(q4k_load_block(blk, g), q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g), g);
+                    acc += kquant_partial<kQuant>(Q::load_block(blk, g),
+                                                  Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g), g);
                 }
             }
             acc = seg_sum<kLanesPerRow>(acc);
@@ -162,13 +153,14 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const float *__restrict__
 constexpr int kSplitRows = 4;
 constexpr uint32_t kSplitMaxWaves = 16;  // rows of up to 256 super-blocks
 
-template <bool kQ6>
+template <uint32_t kQuant>
 __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     gemv_kquant_splitk_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                               const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
                               uint32_t row_chunks) {
-    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
-    using Regs = std::conditional_t<kQ6, Q6KRegs, Q4KRegs>;
+    using Q = KQuant<kQuant>;
+    using Regs = typename Q::Regs;
+    constexpr size_t kBlockBytes = Q::kBytes;
     __shared__ float s_part[2][kSplitRows][kSplitMaxWaves];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = threadIdx.x >> 6, n_slices = blockDim.x >> 6;
@@ -178,12 +170,7 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     const uint32_t tok = blockIdx.y;
     const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? b : 0);
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    Q4KAct a4{};
-    Q6KAct a6{};
-    if constexpr (kQ6)
-        a6 = q6k_load_act(aq + ab * 256, ad[ab], g);
-    else
-        a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    const typename Q::Act a = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
     uint32_t parity = 0;
     for (uint32_t chunk = blockIdx.x; chunk < row_chunks; chunk += gridDim.x, parity ^= 1) {
         const uint32_t row0 = chunk * kSplitRows;
@@ -193,19 +180,12 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
             r[i] = Regs{};  // idle lanes and rows past the end keep zeros
             if (has_block && row0 + i < rows) {
                 const uint8_t *blk = w + static_cast<size_t>(row0 + i) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-                if constexpr (kQ6)
-                    r[i] = q6k_load_block(blk, g);
-                else
-                    r[i] = q4k_load_block(blk, g);
+                r[i] = Q::load_block(blk, g);
             }
         }
 #pragma unroll
         for (int i = 0; i < kSplitRows; i++) {
-            float acc;
-            if constexpr (kQ6)
-                acc = q6k_partial(r[i], a6, g);
-            else
-                acc = q4k_partial(r[i], a4, g);
+            float acc = kquant_partial<kQuant>(r[i], a, g);
             acc = seg_sum<kWave>(has_block ? acc : 0.0f);
             if (lane == kWave - 1) s_part[parity][i][wave] = acc;
         }
@@ -218,39 +198,39 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     }
 }
 
-template <bool kQ6>
+template <uint32_t kQuant>
 void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                           hipStream_t stream) {
     const uint32_t n_slices = (nb + 15) / 16;
     const uint32_t row_chunks = (rows + kSplitRows - 1) / kSplitRows;
     const uint32_t want = kTargetWaves / n_slices;  // workgroups for about kTargetWaves waves
     const dim3 grid(row_chunks < want ? row_chunks : want, seq, 1);
-    hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQ6>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
+    hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
                        act.bsums, out, rows, nb, row_chunks);
 }
 
-template <bool kQ6, int kRowsPerWave>
+template <uint32_t kQuant, int kRowsPerWave>
 void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                    hipStream_t stream) {
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
-    hipLaunchKernelGGL((gemv_kquant_kernel<kQ6, kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
+    hipLaunchKernelGGL((gemv_kquant_kernel<kQuant, kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
                        act.d, act.bsums, out, rows, nb, row_groups);
 }
 
-template <bool kQ6>
+template <uint32_t kQuant>
 void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                        hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
     if (nb > 16 && nb <= 16 * kSplitMaxWaves)
-        launch_kquant_splitk<kQ6>(w, act, out, rows, nb, seq, stream);
+        launch_kquant_splitk<kQuant>(w, act, out, rows, nb, seq, stream);
     else if (nb <= 4)
-        launch_kquant<kQ6, 4>(w, act, out, rows, nb, seq, stream);
+        launch_kquant<kQuant, 4>(w, act, out, rows, nb, seq, stream);
     else if (nb <= 8)
-        launch_kquant<kQ6, 2>(w, act, out, rows, nb, seq, stream);
+        launch_kquant<kQuant, 2>(w, act, out, rows, nb, seq, stream);
     else
-        launch_kquant<kQ6, 1>(w, act, out, rows, nb, seq, stream);
+        launch_kquant<kQuant, 1>(w, act, out, rows, nb, seq, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -325,12 +305,17 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 
 void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
-    launch_kquant_any<false>(w, act, out, rows, nb, seq, stream);
+    launch_kquant_any<kQ4K>(w, act, out, rows, nb, seq, stream);
+}
+
+void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                     hipStream_t stream) {
+    launch_kquant_any<kQ5K>(w, act, out, rows, nb, seq, stream);
 }
 
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
-    launch_kquant_any<true>(w, act, out, rows, nb, seq, stream);
+    launch_kquant_any<kQ6K>(w, act, out, rows, nb, seq, stream);
 }
 
 bool gemv_q4k_gate_up_supported(uint32_t nb) { return nb >= 1 && nb <= 16; }

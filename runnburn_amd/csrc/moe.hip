@@ -136,7 +136,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // ---------------------------------------------------------------------------------------------
 // down projection of the re-quantised intermediate, scaled by the route weight.
 // ---------------------------------------------------------------------------------------------
-template <bool kQ6, int kRowsPerWave>
+template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_down_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
                     const int16_t *__restrict__ mbs, const uint32_t *__restrict__ grp_expert,
@@ -146,7 +146,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kLanesPerRow = kWave / kRowsPerWave;
     constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
-    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    using Q = KQuant<kQuant>;
+    constexpr size_t kBlockBytes = Q::kBytes;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int sub = lane & (kLanesPerRow - 1);
     const uint32_t rsel = lane / kLanesPerRow;
@@ -173,20 +174,12 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
                 const uint8_t *blk = down_all + ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-                Q4KPrep p4{};
-                Q6KPrep p6{};
-                if constexpr (kQ6)
-                    p6 = q6k_prepare(q6k_load_block(blk, g), g);
-                else
-                    p4 = q4k_prepare(q4k_load_block(blk, g), g);
+                const typename Q::Prep p = Q::prepare(Q::load_block(blk, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
-                        if constexpr (kQ6)
-                            acc[t] += q6k_dot(p6, q6k_load_act(st.qs + ab * kStageBlk, st.d[ab], g));
-                        else
-                            acc[t] += q4k_dot(p4, q4k_load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
+                        acc[t] += Q::dot(p, Q::load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
                     }
                 }
             }
@@ -205,11 +198,11 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Dense multi-token matmul on the vector ALUs (Q6_K at any batch size, Q4_K below the MFMA GEMM's minimum): the same
+// Dense multi-token matmul on the vector ALUs (Q5_K and Q6_K at any batch size, Q4_K below the MFMA GEMM's minimum): the same
 // "stage up to eight tokens in LDS, decode a weight block once, dot it per token" walk as the expert kernels, over
 // one weight matrix and consecutive tokens.  out[token * rows + row].
 // ---------------------------------------------------------------------------------------------
-template <bool kQ6, int kRowsPerWave>
+template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     matmul_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                          const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
@@ -217,7 +210,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int kLanesPerRow = kWave / kRowsPerWave;
     constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
-    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    using Q = KQuant<kQuant>;
+    constexpr size_t kBlockBytes = Q::kBytes;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int sub = lane & (kLanesPerRow - 1);
     const uint32_t rsel = lane / kLanesPerRow;
@@ -243,20 +237,12 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
                 const uint8_t *blk = w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-                Q4KPrep p4{};
-                Q6KPrep p6{};
-                if constexpr (kQ6)
-                    p6 = q6k_prepare(q6k_load_block(blk, g), g);
-                else
-                    p4 = q4k_prepare(q4k_load_block(blk, g), g);
+                const typename Q::Prep p = Q::prepare(Q::load_block(blk, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
                         const size_t ab = static_cast<size_t>(t) * nb + b;
-                        if constexpr (kQ6)
-                            acc[t] += q6k_dot(p6, q6k_load_act(st.qs + ab * kStageBlk, st.d[ab], g));
-                        else
-                            acc[t] += q4k_dot(p4, q4k_load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
+                        acc[t] += Q::dot(p, Q::load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
                     }
                 }
             }
@@ -278,7 +264,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // The groups' sums (last lane of each group) are then added in list order, so the result is the same sequence of f32
 // additions as moe_down_kernel followed by moe_reduce_kernel.
 // ---------------------------------------------------------------------------------------------
-template <bool kQ6, int kGroups>
+template <uint32_t kQuant, int kGroups>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_down_token_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq,
                           const float *__restrict__ md, const int16_t *__restrict__ mbs,
@@ -286,7 +272,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                           const uint32_t *__restrict__ slot_expert, const float *__restrict__ slot_route,
                           float *__restrict__ out, uint32_t n_embd, uint32_t nb) {
     constexpr int kLanes = kWave / kGroups;  // lanes per (slot, row) pair
-    constexpr size_t kBlockBytes = kQ6 ? kQ6KBytes : kQ4KBytes;
+    using Q = KQuant<kQuant>;
+    constexpr size_t kBlockBytes = Q::kBytes;
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t row = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     const uint32_t tok = blockIdx.y;
@@ -307,10 +294,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             const uint8_t *blk = down_all + (static_cast<size_t>(slot_expert[slot]) * n_embd + row) * row_bytes +
                                  static_cast<size_t>(b) * kBlockBytes;
             const size_t ab = static_cast<size_t>(slot) * nb + b;
-            if constexpr (kQ6)
-                o = q6k_partial(q6k_load_block(blk, g), q6k_load_act(mq + ab * 256, md[ab], g), g);
-            else
-                o = q4k_partial(q4k_load_block(blk, g), q4k_load_act(mq + ab * 256, md[ab], mbs + ab * 16, g), g);
+            o = kquant_partial<kQuant>(Q::load_block(blk, g), Q::load_act(mq + ab * 256, md[ab], mbs + ab * 16, g), g);
         }
         o = seg_sum<kLanes>(o);
         if (k < end) o *= slot_route[tok_slots[k]];  // fanout.rs:306-308; only the group's last lane is read below
@@ -358,6 +342,27 @@ TilePlan plan_tiles(uint32_t rows, uint32_t nb, uint32_t n_groups, int rows_per_
 
 int rows_per_wave_for(uint32_t nb) { return nb <= 4 ? 4 : (nb <= 8 ? 2 : 1); }
 
+// LAUNCH(format id, rows or slots per wave) for a run-time K-quant id (Q4_K, Q5_K or Q6_K; callers have
+// validated it) and a run-time 4 / 2 / 1 split
+#define RNB_DISPATCH_KQUANT_R(Q, rpw, LAUNCH) \
+    do {                                      \
+        if ((rpw) == 4)                       \
+            LAUNCH(Q, 4);                     \
+        else if ((rpw) == 2)                  \
+            LAUNCH(Q, 2);                     \
+        else                                  \
+            LAUNCH(Q, 1);                     \
+    } while (0)
+#define RNB_DISPATCH_KQUANT(quant, rpw, LAUNCH)          \
+    do {                                                 \
+        if ((quant) == kQ6K)                             \
+            RNB_DISPATCH_KQUANT_R(kQ6K, rpw, LAUNCH);    \
+        else if ((quant) == kQ5K)                        \
+            RNB_DISPATCH_KQUANT_R(kQ5K, rpw, LAUNCH);    \
+        else                                             \
+            RNB_DISPATCH_KQUANT_R(kQ4K, rpw, LAUNCH);    \
+    } while (0)
+
 }  // namespace
 
 void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
@@ -385,18 +390,11 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
     const int rpw = rows_per_wave_for(nb_mid);
     const TilePlan p = plan_tiles(n_embd, nb_mid, groups.n_groups, rpw);
     const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
-#define RNB_LAUNCH_DOWN(Q6, R)                                                                                       \
-    hipLaunchKernelGGL((moe_down_kernel<Q6, R>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d,   \
+#define RNB_LAUNCH_DOWN(Q, R)                                                                                        \
+    hipLaunchKernelGGL((moe_down_kernel<Q, R>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d,    \
                        mid_act.bsums, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, \
                        nb_mid, p.iters, p.tmax)
-    const bool q6 = down_quant == kQ6K;
-    if (rpw == 4) {
-        if (q6) RNB_LAUNCH_DOWN(true, 4); else RNB_LAUNCH_DOWN(false, 4);
-    } else if (rpw == 2) {
-        if (q6) RNB_LAUNCH_DOWN(true, 2); else RNB_LAUNCH_DOWN(false, 2);
-    } else {
-        if (q6) RNB_LAUNCH_DOWN(true, 1); else RNB_LAUNCH_DOWN(false, 1);
-    }
+    RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN);
 #undef RNB_LAUNCH_DOWN
 }
 
@@ -411,17 +409,10 @@ void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *
     while (p.tiles * ysplit < 1024 && ysplit < chunks) ysplit *= 2;
     const uint32_t chunks_per_wg = (chunks + ysplit - 1) / ysplit;
     const dim3 grid(p.tiles, (chunks + chunks_per_wg - 1) / chunks_per_wg, 1), block(kWave * kWavesPerWg);
-#define RNB_LAUNCH_MT(Q6, R)                                                                                          \
-    hipLaunchKernelGGL((matmul_tokens_kernel<Q6, R>), grid, block, p.lds_bytes, stream, w, act.qs, act.d, act.bsums,  \
+#define RNB_LAUNCH_MT(Q, R)                                                                                           \
+    hipLaunchKernelGGL((matmul_tokens_kernel<Q, R>), grid, block, p.lds_bytes, stream, w, act.qs, act.d, act.bsums,   \
                        out, rows, nb, seq, p.iters, p.tmax, chunks_per_wg)
-    const bool q6 = quant == kQ6K;
-    if (rpw == 4) {
-        if (q6) RNB_LAUNCH_MT(true, 4); else RNB_LAUNCH_MT(false, 4);
-    } else if (rpw == 2) {
-        if (q6) RNB_LAUNCH_MT(true, 2); else RNB_LAUNCH_MT(false, 2);
-    } else {
-        if (q6) RNB_LAUNCH_MT(true, 1); else RNB_LAUNCH_MT(false, 1);
-    }
+    RNB_DISPATCH_KQUANT(quant, rpw, RNB_LAUNCH_MT);
 #undef RNB_LAUNCH_MT
 }
 
@@ -430,17 +421,10 @@ void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView
                            uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (token_count == 0) return;
     const dim3 grid((n_embd + kWavesPerWg - 1) / kWavesPerWg, token_count, 1), block(kWave * kWavesPerWg);
-#define RNB_LAUNCH_DT(Q6, G)                                                                                          \
-    hipLaunchKernelGGL((moe_down_token_kernel<Q6, G>), grid, block, 0, stream, down_all, mid_act.qs, mid_act.d,       \
+#define RNB_LAUNCH_DT(Q, G)                                                                                           \
+    hipLaunchKernelGGL((moe_down_token_kernel<Q, G>), grid, block, 0, stream, down_all, mid_act.qs, mid_act.d,        \
                        mid_act.bsums, tok_offsets, tok_slots, slot_expert, slot_route, out, n_embd, nb_mid)
-    const bool q6 = down_quant == kQ6K;
-    if (nb_mid <= 4) {
-        if (q6) RNB_LAUNCH_DT(true, 4); else RNB_LAUNCH_DT(false, 4);
-    } else if (nb_mid <= 8) {
-        if (q6) RNB_LAUNCH_DT(true, 2); else RNB_LAUNCH_DT(false, 2);
-    } else {
-        if (q6) RNB_LAUNCH_DT(true, 1); else RNB_LAUNCH_DT(false, 1);
-    }
+    RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DT);
 #undef RNB_LAUNCH_DT
 }
 

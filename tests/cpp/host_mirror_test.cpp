@@ -46,6 +46,8 @@ static int validate() {
     EXPECT(!r && r.error == "Q4_K weight byte mismatch: got 143, expected 144", "weight bytes message");
     r = q6k_gemv({w.data(), 144}, 1, 256, {x.data(), 256});
     EXPECT(!r && r.error == "Q6_K weight byte mismatch: got 144, expected 210", "q6k weight bytes message");
+    r = q5k_gemv({w.data(), 144}, 1, 256, {x.data(), 256});
+    EXPECT(!r && r.error == "Q5_K weight byte mismatch: got 144, expected 176", "q5k weight bytes message");
     r = q8_0_gemv_batch({w.data(), 34}, 1, 32, {x.data(), 33});
     EXPECT(!r && r.error == "Q8_0 batch input length 33 is not divisible by cols 32", "q8_0 batch message");
     float out1 = 0;
@@ -134,6 +136,8 @@ int main(int argc, char **argv) {
         run_case(dir, "q4k_batch", 40, 512, 19, q4k_gemv_batch);
         run_case(dir, "q6k_batch", 9, 512, 3, q6k_gemv_batch);
         run_case(dir, "q8_0_batch", 7, 96, 4, q8_0_gemv_batch);
+        run_case(dir, "q5k_gemv", 22, 1280, 1, q5k_gemv);
+        run_case(dir, "q5k_batch", 13, 512, 5, q5k_gemv_batch);
         std::printf("run: %d failure(s)\n", failures);
         return failures ? 1 : 0;
     }

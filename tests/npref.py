@@ -49,6 +49,44 @@ def dequant_q4k_f64(blocks) -> np.ndarray:
     return (scale * nib - minv).reshape(-1)
 
 
+# ---- Q5_K ---------------------------------------------------------------------------
+
+def make_q5k_block(d, dmin, sc, mn, values) -> np.ndarray:
+    """values: 256 five-bit values 0..31 in element order.  Layout {f16 d, f16 dmin, scales[12], qh[32], qs[128]}:
+    element 64g + 32h + l keeps its low four bits in nibble h of qs[32g + l] and its fifth bit in bit 2g + h of
+    qh[l]."""
+    v = np.asarray(values, dtype=np.uint8).reshape(4, 2, 32)  # group, lo/hi half, l
+    qs = ((v[:, 0, :] & 15) | ((v[:, 1, :] & 15) << 4)).reshape(128)
+    qh = np.zeros(32, dtype=np.uint8)
+    for g in range(4):
+        for h in range(2):
+            qh |= ((v[g, h, :] >> 4) & 1) << (2 * g + h)
+    return np.concatenate([
+        np.frombuffer(f16_bytes(d), dtype=np.uint8), np.frombuffer(f16_bytes(dmin), dtype=np.uint8),
+        pack_scales_k4(sc, mn), qh, qs]).astype(np.uint8)
+
+
+def split_q5k(blocks: np.ndarray):
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, 176)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float64).reshape(-1)
+    dmin = b[:, 2:4].copy().view(np.float16).astype(np.float64).reshape(-1)
+    s = b[:, 4:16].astype(np.int64)
+    sc = np.concatenate([s[:, 0:4] & 63, (s[:, 8:12] & 15) | ((s[:, 0:4] >> 6) << 4)], axis=1)
+    mn = np.concatenate([s[:, 4:8] & 63, (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)], axis=1)
+    qh = b[:, 16:48].astype(np.int64)                       # [n, l]
+    qs = b[:, 48:176].reshape(-1, 4, 32).astype(np.int64)   # [n, group, l]
+    bits = (qh[:, None, :] >> np.arange(8)[None, :, None]) & 1          # [n, bit, l], bit = 2*group + half
+    low = np.stack([qs & 15, qs >> 4], axis=2).reshape(-1, 8, 32)       # [n, 2*group + half, l]
+    return d, dmin, sc, mn, (low + 16 * bits).reshape(-1, 256)
+
+
+def dequant_q5k_f64(blocks) -> np.ndarray:
+    d, dmin, sc, mn, val = split_q5k(blocks)
+    scale = np.repeat(sc, 32, axis=1) * d[:, None]
+    minv = np.repeat(mn, 32, axis=1) * dmin[:, None]
+    return (scale * val - minv).reshape(-1)
+
+
 # ---- Q6_K ---------------------------------------------------------------------------
 
 def make_q6k_block(d, scales, q6) -> np.ndarray:

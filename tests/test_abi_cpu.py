@@ -35,7 +35,8 @@ def test_trait_facade():
     caps = b.capabilities()
     assert caps == {"MatMul": True, "Attention": False, "Gdn": False, "MoE": True, "Sampler": False}
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q4_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q8_0)
-    assert not b.supports_quant(rnb.OP_MATMUL, 13)  # Q5_K is not on this path
+    assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q5_K) and b.supports_quant(rnb.OP_MOE, rnb.GGML_Q5_K)
+    assert not b.supports_quant(rnb.OP_MATMUL, 10) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # Q2_K; Q8_0 down
     with pytest.raises(rnb.BackendError) as ei:
         b.execute(object())
     assert ei.value.kind == "UnsupportedOp"
@@ -61,6 +62,17 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q4_K shape mismatch: input=256 output=1 expected input=256 output>=2"
     e = _err(rnb.q4k_gemv_batch, z(144, np.uint8), 1, 256, z(300, np.float32))
     assert str(e) == "Q4_K batch input length 300 is not divisible by cols 256"
+    # crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:2207-2281, 3957-3993
+    e = _err(rnb.q5k_gemv, z(176, np.uint8), 1, 100, z(100, np.float32))
+    assert str(e) == "Q5_K cols must be divisible by 256, got 100"
+    e = _err(rnb.q5k_gemv, z(175, np.uint8), 1, 256, z(256, np.float32))
+    assert str(e) == "Q5_K weight byte mismatch: got 175, expected 176"
+    e = _err(rnb.q5k_gemv, z(176, np.uint8), 1, 256, z(255, np.float32))
+    assert str(e) == "Q5_K input length mismatch: got 255, expected 256"
+    e = _err(rnb.q5k_gemv_into, z(352, np.uint8), 2, 256, z(256, np.float32), out)
+    assert str(e) == "Q5_K shape mismatch: input=256 output=1 expected input=256 output>=2"
+    e = _err(rnb.q5k_gemv_batch, z(176, np.uint8), 1, 256, z(300, np.float32))
+    assert str(e) == "Q5_K batch input length 300 is not divisible by cols 256"
     e = _err(rnb.q6k_gemv, z(210, np.uint8), 1, 100, z(100, np.float32))
     assert str(e) == "Q6_K cols must be divisible by 256, got 100"
     e = _err(rnb.q6k_gemv, z(200, np.uint8), 1, 256, z(256, np.float32))
@@ -89,8 +101,10 @@ def test_moe_validation_messages():
     assert str(e) == "Qwen35 full-layer dims must be divisible by 256, got n_ff=100 n_embd=256"
     e = _err(call, g, u, d, [0], [1.0], [1], 1, 14, n_ff, n_embd, x)
     assert str(e) == "Qwen35 full-layer token id out of range"
-    e = _err(call, g, u, d, [0], [1.0], [0], 1, 13, n_ff, n_embd, x)
-    assert e.kind == "UnsupportedOp" and "down quant code 13" in str(e)
+    e = _err(call, g, u, d, [0], [1.0], [0], 1, 10, n_ff, n_embd, x)
+    assert e.kind == "UnsupportedOp" and "down quant code 10" in str(e)
+    e = _err(call, g, u, d, [0], [1.0], [0], 1, 13, n_ff, n_embd, x)  # Q5_K down: 176-byte blocks expected
+    assert str(e) == "Qwen35 selected-base down length mismatch: len=107520 expected=90112"
     e = _err(call, g[:-1], u, d, [0], [1.0], [0], 1, 14, n_ff, n_embd, x)
     assert str(e).startswith("Qwen35 selected-base gate length is not expert-aligned")
     e = _err(call, g, u[:per_gate], d, [0], [1.0], [0], 1, 14, n_ff, n_embd, x)
@@ -146,5 +160,7 @@ def test_dense_ffn_validation_messages():
     assert str(e) == "dense SiLU FFN batch up byte mismatch: got 36862, expected 36864"
     e = _err(f, g, g, z(256 * 210 + 1, np.uint8), 14, 256, 256, 2, z(512, np.float32))
     assert str(e) == "dense SiLU FFN batch down byte mismatch: got 53761, expected 53760"
-    e = _err(f, g, g, z(256 * 176, np.uint8), 13, 256, 256, 2, z(512, np.float32))
+    e = _err(f, g, g, z(256 * 176 - 1, np.uint8), 13, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "dense SiLU FFN batch down byte mismatch: got 45055, expected 45056"
+    e = _err(f, g, g, z(256 * 8 * 24, np.uint8), 7, 256, 256, 2, z(512, np.float32))  # Q5_1: valid, not built
     assert e.kind == "UnsupportedOp"

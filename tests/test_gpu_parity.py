@@ -10,7 +10,7 @@ from tests import npref
 
 pytestmark = pytest.mark.gpu
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 REL = 1e-3          # tolerance named by the task: max relative error 1e-3 per row
 TIGHT = 2e-5        # what f32 summation-order differences actually allow, relative to rms
 
@@ -27,8 +27,9 @@ def check_close(got, ref, gold=None, label=""):
 
 
 def gemv_fn(rnb, quant, batch=False):
-    table = {(Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q6_K, False): rnb.q6k_gemv,
-             (Q6_K, True): rnb.q6k_gemv_batch, (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
+    table = {(Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q5_K, False): rnb.q5k_gemv,
+             (Q5_K, True): rnb.q5k_gemv_batch, (Q6_K, False): rnb.q6k_gemv, (Q6_K, True): rnb.q6k_gemv_batch,
+             (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
     return table[(quant, batch)]
 
 
@@ -111,7 +112,7 @@ def test_reference_closed_forms_on_device(rnb):
 
 # ---- GEMV: shapes around every edge of the lane mapping ------------------------------------------
 
-@pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("rows,nblk", [(1, 1), (3, 2), (4, 3), (5, 5), (7, 8), (9, 9), (64, 16), (33, 17), (6, 56),
                                        (5, 31), (130, 20), (9, 256), (2, 257)])
 def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
@@ -151,6 +152,15 @@ def test_gemv_extreme_blocks(rnb, oracle):
     blocks = []
     for r in range(rows):
         for b in range(nblk):
+            d = [1.0, 0.0, 6e-8, 2.0 ** -14][(r + b) % 4]
+            vals = [np.full(256, 31), rng.integers(0, 32, 256), np.tile([16, 15], 128), np.zeros(256)][(r + 2 * b) % 4]
+            blocks.append(npref.make_q5k_block(d, [0.5, 6e-8, 0.0, 1.0][(r + b) % 4], np.full(8, 63), np.full(8, 63), vals))
+    w = np.concatenate(blocks)
+    check_close(rnb.q5k_gemv(w, rows, nblk * 256, x), oracle.gemv(Q5_K, w, rows, nblk * 256, x)[0],
+                oracle.gemv(Q5_K, w, rows, nblk * 256, x, gold=True)[0], "q5k extremes")
+    blocks = []
+    for r in range(rows):
+        for b in range(nblk):
             d = [1.0, -0.5, 6e-8, 0.0][(r + b) % 4]
             scales = np.full(16, -128) if b == 0 else rng.integers(-128, 128, 16)
             q = np.full(256, 63) if b == 1 else (np.zeros(256) if b == 2 else rng.integers(0, 64, 256))
@@ -169,7 +179,7 @@ def test_unaligned_host_weights_and_subrange_residency(rnb, oracle):
     """Rows at odd host byte offsets must give identical results (crates/rnb-cpu/src/gemm/quant_gemv.rs:1257-1296);
     a sub-range of a resident parent resolves to parent + offset (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:722-741)."""
     rows, cols = 16, 1024
-    for quant in (Q4_K, Q6_K, Q8_0):
+    for quant in (Q4_K, Q5_K, Q6_K, Q8_0):
         w = oracle.make_weights(quant, rows, cols, 42 + quant)
         x = oracle.fill_normal(cols, 43, 1.0)
         base = gemv_fn(rnb, quant)(w, rows, cols, x)
@@ -232,7 +242,8 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
 
 
 @pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q4_K, 77, 2048), (Q4_K, 50, 768), (Q6_K, 300, 4096),
-                                             (Q6_K, 64, 768), (Q8_0, 200, 4096), (Q8_0, 33, 1056), (Q6_K, 40, 14336)])
+                                             (Q6_K, 64, 768), (Q8_0, 200, 4096), (Q8_0, 33, 1056), (Q6_K, 40, 14336),
+                                             (Q5_K, 300, 4096), (Q5_K, 41, 1280), (Q5_K, 24, 14336)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
     feed several matrices from one activation) run the same arithmetic: identical bits."""
@@ -254,7 +265,7 @@ def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols
 
 # ---- batches: seq-major layout, ragged token counts ----------------------------------------------
 
-@pytest.mark.parametrize("quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("seq", [2, 3, 4, 9, 15, 33])
 def test_gemv_batch_small(rnb, oracle, quant, seq):
     rows, cols = 37, 768
@@ -266,7 +277,7 @@ def test_gemv_batch_small(rnb, oracle, quant, seq):
                 f"batch quant {quant} seq {seq}")
 
 
-@pytest.mark.parametrize("quant", [Q4_K, Q6_K])
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K])
 def test_gemv_batch_long_rows(rnb, oracle, quant):
     """Rows longer than 16 super-blocks: the K-split kernel with tokens on grid.y up to 3 tokens, the staged
     multi-token kernel from 4 tokens on."""
@@ -342,6 +353,27 @@ def test_config3b_q6k_gemv_lm_head_128256x4096(rnb, oracle):
     _full_gemv(rnb, oracle, Q6_K, 128256, 4096, "cfg3b")
 
 
+def test_q5k_gemv_full_size_14336x4096_and_4096x14336(rnb, oracle):
+    """Q5_K at the up- and down-projection shapes of the Q4_K / Q6_K configurations."""
+    _full_gemv(rnb, oracle, Q5_K, 14336, 4096, "q5k_up")
+    _full_gemv(rnb, oracle, Q5_K, 4096, 14336, "q5k_down")
+
+
+def test_q5k_fifth_bit_vectors_on_device(rnb):
+    """The hand-built vectors that pin the oracle's Q5_K dot (one qh bit set in every byte, d = 1, dmin = 0,
+    sub-block scales 1..8), through the device: 16 * (bit + 1) * sum of that sub-block's activations."""
+    hdr = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(0.0), np.uint8),
+                          npref.pack_scales_k4(np.arange(1, 9), np.zeros(8))])
+    x = np.zeros(256, np.float32)
+    x[0] = 127.0                                   # Q8_K scale exactly 1: x == its quantised form
+    x[1:] = (np.arange(1, 256) % 7 - 3).astype(np.float32)
+    w = np.concatenate([np.concatenate([hdr, np.full(32, 1 << bit, np.uint8), np.zeros(128, np.uint8)])
+                        for bit in range(8)])
+    got = rnb.q5k_gemv(w, 8, 256, x)
+    want = [16.0 * (bit + 1) * float(x[32 * bit:32 * bit + 32].sum()) for bit in range(8)]
+    assert np.allclose(got, want, rtol=1e-6, atol=0), (got, want)
+
+
 def test_config4_q4k_gemm_512x4096_to_14336(rnb, oracle):
     rows, cols, seq = 14336, 4096, 512
     w = oracle.make_weights(Q4_K, rows, cols, oracle.tensor_seed("cfg2", "weight"))
@@ -383,7 +415,7 @@ def _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, seed, down_quant=Q6_K):
     return gate, up, down, x, np.array(eids, np.uint32), np.array(route, np.float32), np.array(tids, np.uint32)
 
 
-@pytest.mark.parametrize("tokens,down_quant", [(1, Q6_K), (3, Q6_K), (2, Q4_K)])
+@pytest.mark.parametrize("tokens,down_quant", [(1, Q6_K), (3, Q6_K), (2, Q4_K), (1, Q5_K), (5, Q5_K), (40, Q5_K)])
 def test_moe_small(rnb, oracle, tokens, down_quant):
     n_expert, n_ff, n_embd, k = 8, 512, 768, 3
     gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 1, down_quant)
@@ -433,7 +465,7 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
 
 # ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
 
-@pytest.mark.parametrize("down_quant", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("seq,n_ff,n_embd", [(2, 256, 256), (3, 768, 512), (5, 512, 4608), (17, 512, 768), (40, 1024, 256)])
 def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
     """Decode-sized batches take the fused gate/up GEMV, 16+ tokens the MFMA GEMM + SiLU kernel, rows longer than

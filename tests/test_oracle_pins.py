@@ -9,7 +9,7 @@ import pytest
 
 from tests import npref
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 
 
 # ---- f16 ----------------------------------------------------------------------------
@@ -81,6 +81,15 @@ def _random_q4k(rng, n):
     return np.concatenate(blocks)
 
 
+def _random_q5k(rng, n):
+    blocks = []
+    for _ in range(n):
+        blocks.append(npref.make_q5k_block(rng.uniform(1e-4, 5e-3), rng.uniform(1e-4, 5e-3),
+                                           rng.integers(0, 64, 8), rng.integers(0, 64, 8),
+                                           rng.integers(0, 32, 256)))
+    return np.concatenate(blocks)
+
+
 def _random_q6k(rng, n):
     blocks = []
     for _ in range(n):
@@ -109,6 +118,43 @@ def test_dequantize_q4k_places_each_nibble(oracle):
     got = oracle.dequantize(Q4_K, blocks).astype(np.float64)
     want = npref.dequant_q4k_f64(blocks)
     assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
+
+
+def test_dequantize_q5k_zero_block(oracle):
+    """crates/rnb-cpu/src/quantize/dequant.rs:1036-1047 (test_dequant_q5_k_zero)."""
+    assert np.all(oracle.dequantize(Q5_K, np.zeros(176, np.uint8)) == 0.0)
+
+
+def test_dequantize_q5k_places_each_bit(oracle):
+    """Hand-built bytes (no packer): one qh bit set -> exactly the element 64*(bit//2) + 32*(bit%2) + l gains 16
+    (the placement crates/rnb-cpu/src/gemm/tile_q5k.rs:944-976 states: bit 2g of qh[l] for l < 32 of group g,
+    bit 2g+1 for the upper half); one nibble set -> as for Q4_K, 48 bytes further into the block."""
+    hdr = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(0.0), np.uint8),
+                          npref.pack_scales_k4(np.arange(1, 9), np.zeros(8))])
+    for l in (0, 5, 31):
+        for bit in range(8):
+            blk = np.concatenate([hdr, np.zeros(32 + 128, np.uint8)])
+            blk[16 + l] = 1 << bit
+            y = oracle.dequantize(Q5_K, blk)
+            want = np.zeros(256, np.float32)
+            want[64 * (bit // 2) + 32 * (bit % 2) + l] = 16.0 * (bit + 1)  # scale of sub-block `bit` is bit + 1
+            assert np.array_equal(y, want), (l, bit)
+    for g, l in ((0, 0), (1, 7), (3, 31)):
+        blk = np.concatenate([hdr, np.zeros(32 + 128, np.uint8)])
+        blk[48 + 32 * g + l] = 0x93  # low nibble 3, high nibble 9
+        y = oracle.dequantize(Q5_K, blk)
+        want = np.zeros(256, np.float32)
+        want[64 * g + l] = 3.0 * (2 * g + 1)
+        want[64 * g + 32 + l] = 9.0 * (2 * g + 2)
+        assert np.array_equal(y, want), (g, l)
+    rng = np.random.default_rng(31)
+    blocks = _random_q5k(rng, 64)
+    got = oracle.dequantize(Q5_K, blocks).astype(np.float64)
+    want = npref.dequant_q5k_f64(blocks)
+    assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
+    # packer and splitter are inverse on the five-bit values
+    vals = rng.integers(0, 32, 256)
+    assert np.array_equal(npref.split_q5k(npref.make_q5k_block(1.0, 1.0, np.zeros(8), np.zeros(8), vals))[4][0], vals)
 
 
 def test_dequantize_q6k_places_each_value(oracle):
@@ -263,6 +309,46 @@ def test_q4k_mins_use_32_wide_bsums(oracle):
     assert oracle.dot(Q4_K, blk, act, avx2=True) == -2.0 * summ
 
 
+# ---- Q5_K x Q8_K dot ------------------------------------------------------------------
+
+def test_q5k_dot_fifth_bit_vectors(oracle):
+    """Known answers for crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 built by hand: d = 1, dmin = 0, sub-block
+    scales 1..8, every nibble 0, one qh bit set in every byte -> the 32 elements of sub-block `bit` are 16, so the
+    dot is 16 * (bit + 1) * sum of that sub-block's activations."""
+    hdr = np.concatenate([np.frombuffer(npref.f16_bytes(1.0), np.uint8), np.frombuffer(npref.f16_bytes(0.0), np.uint8),
+                          npref.pack_scales_k4(np.arange(1, 9), np.zeros(8))])
+    q = (np.arange(256) % 7 - 3).astype(np.int8)
+    act = _act_from_parts(0.5, q)
+    for bit in range(8):
+        blk = np.concatenate([hdr, np.full(32, 1 << bit, np.uint8), np.zeros(128, np.uint8)])
+        want = 0.5 * 16.0 * (bit + 1) * float(q[32 * bit:32 * bit + 32].astype(np.int64).sum())
+        assert oracle.dot(Q5_K, blk, act) == want, bit
+    # with qh == 0 a Q5_K block is the Q4_K block with 32 zero bytes inserted
+    rng = np.random.default_rng(32)
+    row4 = _random_q4k(rng, 3).reshape(3, 144)
+    row5 = np.concatenate([row4[:, :16], np.zeros((3, 32), np.uint8), row4[:, 16:]], axis=1).reshape(-1)
+    act3 = oracle.quantize_q8k(rng.standard_normal(3 * 256).astype(np.float32))
+    assert oracle.dot(Q5_K, row5, act3) == oracle.dot(Q4_K, row4.reshape(-1), act3)
+    # dmin term: values 0, mins 1..8 -> summ over 32-wide bsums, as for Q4_K
+    blk = npref.make_q5k_block(0.0, 1.0, np.zeros(8), np.arange(1, 9), np.zeros(256))
+    bs = np.arange(1, 17, dtype=np.int16).reshape(1, 16)
+    summ = sum((k + 1) * (bs[0, 2 * k] + bs[0, 2 * k + 1]) for k in range(8))
+    assert oracle.dot(Q5_K, blk, _act_from_parts(2.0, np.zeros(256, np.int8), bsums=bs)) == -2.0 * summ
+
+
+def test_q5k_dot_equals_f64_dequant_identity(oracle):
+    rng = np.random.default_rng(33)
+    for nb in (1, 2, 7, 16):
+        row = _random_q5k(rng, nb)
+        x = rng.standard_normal(nb * 256).astype(np.float32)
+        act = oracle.quantize_q8k(x)
+        want = float(np.dot(npref.dequant_q5k_f64(row), npref.deq_act_q8k_f64(act)))
+        gold = oracle.dot(Q5_K, row, act, gold=True)
+        assert gold == pytest.approx(want, rel=1e-11, abs=1e-12)
+        scale = float(np.sum(np.abs(npref.dequant_q5k_f64(row) * npref.deq_act_q8k_f64(act))))
+        assert abs(oracle.dot(Q5_K, row, act) - want) <= 4e-7 * scale
+
+
 # ---- Q6_K x Q8_K dot ------------------------------------------------------------------
 
 def test_q6k_dot_equals_f64_dequant_identity(oracle):
@@ -340,7 +426,7 @@ def test_q8_0_q8_equals_f64_identity(oracle):
 
 # ---- drivers --------------------------------------------------------------------------
 
-@pytest.mark.parametrize("quant,maker", [(Q4_K, _random_q4k), (Q6_K, _random_q6k)])
+@pytest.mark.parametrize("quant,maker", [(Q4_K, _random_q4k), (Q5_K, _random_q5k), (Q6_K, _random_q6k)])
 def test_gemv_driver_layout_and_row_independence(oracle, quant, maker):
     rng = np.random.default_rng(12)
     rows, nb, seq = 5, 2, 3
@@ -354,8 +440,9 @@ def test_gemv_driver_layout_and_row_independence(oracle, quant, maker):
             assert out[s, r] == np.float32(oracle.dot(quant, w[r * rb:(r + 1) * rb], act))
     gold = oracle.gemv(quant, w, rows, nb * 256, x, gold=True)
     assert np.allclose(out, gold, rtol=1e-4, atol=1e-6)
-    fast = oracle.gemv(quant, w, rows, nb * 256, x, avx2=True)
-    assert np.allclose(fast, gold, rtol=1e-4, atol=1e-6)
+    if quant != Q5_K:  # the vectorised baseline covers the benchmarked formats only
+        fast = oracle.gemv(quant, w, rows, nb * 256, x, avx2=True)
+        assert np.allclose(fast, gold, rtol=1e-4, atol=1e-6)
     # 1 thread == many threads, bitwise (rows are independent)
     assert np.array_equal(oracle.gemv(quant, w, rows, nb * 256, x, n_threads=1), out)
 
@@ -446,6 +533,23 @@ def test_q4k_quantiser_roundtrip_property(oracle):
     cos = float(np.dot(x, y) / (np.linalg.norm(x) * np.linalg.norm(y)))
     assert cos >= 0.97
     assert np.sqrt(np.mean((x - y) ** 2)) / np.sqrt(np.mean(x ** 2)) < 0.1
+
+
+def test_q5k_quantiser_roundtrip_property(oracle):
+    """crates/rnb-cpu/src/quantize/quant.rs:732-764: the reference's own input and bound (cosine >= 0.98).  Byte
+    parity with the Rust quantiser is UNPINNED (cannot run it); GPU and oracle consume identical bytes."""
+    t = np.arange(1024, dtype=np.float32) * np.float32(0.019)
+    x = (np.sin(t) * (1.0 + 0.3 * np.cos(t * np.float32(0.7)))).astype(np.float32)
+    q = oracle.quantize_row(Q5_K, x)
+    assert q.size == 4 * 176
+    y = oracle.dequantize(Q5_K, q)
+    assert float(np.dot(x, y) / (np.linalg.norm(x) * np.linalg.norm(y) + 1e-10)) >= 0.98
+    xn = oracle.fill_normal(256 * 40, 23, 0.02)
+    qn = oracle.quantize_row(Q5_K, xn)
+    yn = oracle.dequantize(Q5_K, qn)
+    assert np.sqrt(np.mean((xn - yn) ** 2)) / np.sqrt(np.mean(xn ** 2)) < 0.05
+    d, dmin, sc, mn, val = npref.split_q5k(qn)
+    assert sc.max() == 63 and val.max() == 31 and val.min() == 0
 
 
 def test_q6k_q8_0_generators_roundtrip(oracle):
