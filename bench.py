@@ -30,9 +30,9 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA, POP/s -> TOP/s
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256}
 MALL_BYTES = 256 << 20
 
 
@@ -59,12 +59,14 @@ def synth_q8_0(rng, rows, cols):
     return out.reshape(-1)
 
 
-def synth_q4_k(rng, rows, cols):
+def _synth_kquant_min(rng, rows, cols, qmax):
+    """Shared fit of the Q4_K / Q5_K synthetic generators: header bytes (d, dmin, 12 packed 6-bit scales and mins) and
+    the per-element codes 0..qmax as [rows][nb][4 groups][2 halves][32]."""
     nb = cols // 256
     x = rng.standard_normal((rows, nb, 8, 32), dtype=np.float32) * np.float32(0.02)
     lo = np.minimum(x.min(axis=3), 0.0)
     hi = x.max(axis=3)
-    scale = (hi - lo) / 15.0
+    scale = (hi - lo) / float(qmax)
     mins = -lo
     d = (scale.max(axis=2) / 63.0).astype(np.float16)
     dmin = (mins.max(axis=2) / 63.0).astype(np.float16)
@@ -73,15 +75,36 @@ def synth_q4_k(rng, rows, cols):
     sc = np.clip(np.rint(scale / df), 0, 63).astype(np.uint8)
     mn = np.clip(np.rint(mins / dmf), 0, 63).astype(np.uint8)
     step = np.maximum(df * sc, 1e-12)[..., None]
-    q = np.clip(np.rint((x + (dmf * mn)[..., None]) / step), 0, 15).astype(np.uint8)
+    q = np.clip(np.rint((x + (dmf * mn)[..., None]) / step), 0, qmax).astype(np.uint8)
+    hdr = np.empty((rows, nb, 16), np.uint8)
+    hdr[..., 0:2] = d.view(np.uint8).reshape(rows, nb, 2)
+    hdr[..., 2:4] = dmin.view(np.uint8).reshape(rows, nb, 2)
+    hdr[..., 4:8] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
+    hdr[..., 8:12] = (mn[..., 0:4] & 63) | ((mn[..., 4:8] >> 4) << 6)
+    hdr[..., 12:16] = (sc[..., 4:8] & 15) | ((mn[..., 4:8] & 15) << 4)
+    return hdr, q.reshape(rows, nb, 4, 2, 32)
+
+
+def synth_q4_k(rng, rows, cols):
+    nb = cols // 256
+    hdr, qg = _synth_kquant_min(rng, rows, cols, 15)
     out = np.empty((rows, nb, 144), np.uint8)
-    out[..., 0:2] = d.view(np.uint8).reshape(rows, nb, 2)
-    out[..., 2:4] = dmin.view(np.uint8).reshape(rows, nb, 2)
-    out[..., 4:8] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
-    out[..., 8:12] = (mn[..., 0:4] & 63) | ((mn[..., 4:8] >> 4) << 6)
-    out[..., 12:16] = (sc[..., 4:8] & 15) | ((mn[..., 4:8] & 15) << 4)
-    qg = q.reshape(rows, nb, 4, 2, 32)
+    out[..., 0:16] = hdr
     out[..., 16:] = (qg[:, :, :, 0, :] | (qg[:, :, :, 1, :] << 4)).reshape(rows, nb, 128)
+    return out.reshape(-1)
+
+
+def synth_q5_k(rng, rows, cols):
+    nb = cols // 256
+    hdr, qg = _synth_kquant_min(rng, rows, cols, 31)
+    out = np.empty((rows, nb, 176), np.uint8)
+    out[..., 0:16] = hdr
+    qh = np.zeros((rows, nb, 32), np.uint8)
+    for g in range(4):
+        for h in range(2):
+            qh |= (qg[:, :, g, h, :] >> 4) << (2 * g + h)
+    out[..., 16:48] = qh
+    out[..., 48:] = ((qg[:, :, :, 0, :] & 15) | ((qg[:, :, :, 1, :] & 15) << 4)).reshape(rows, nb, 128)
     return out.reshape(-1)
 
 
@@ -106,7 +129,7 @@ def synth_q6_k(rng, rows, cols):
     return out.reshape(-1)
 
 
-SYNTH = {Q8_0: synth_q8_0, Q4_K: synth_q4_k, Q6_K: synth_q6_k}
+SYNTH = {Q8_0: synth_q8_0, Q4_K: synth_q4_k, Q5_K: synth_q5_k, Q6_K: synth_q6_k}
 
 
 def synth_weights(quant, rows, cols, seed, distinct_rows=16384):
@@ -510,7 +533,8 @@ def main() -> int:
         s2 = max(50, min(args.steps, 500))
         for key, quant, r, c, seq in (("cfg1_q8_0_gemv_4096x4096", Q8_0, 4096, 4096, 1),
                                       ("cfg3a_q6k_gemv_4096x14336", Q6_K, 4096, 14336, 1),
-                                      ("cfg3b_q6k_gemv_128256x4096", Q6_K, 128256, 4096, 1)):
+                                      ("cfg3b_q6k_gemv_128256x4096", Q6_K, 128256, 4096, 1),
+                                      ("q5k_gemv_14336x4096", Q5_K, 14336, 4096, 1)):
             try:
                 res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, seq, s2 if r < 100000 else 60, 10, 7 + r, key,
                                             want_graph=False, cache_resident=args.cache_resident)
