@@ -96,8 +96,9 @@ __device__ __forceinline__ float q4k_dot(const Q4KPrep &p, const Q4KAct &a) {
     i1 = dot4(p.hi1.y, a.hi1.y, i1);
     i1 = dot4(p.hi1.z, a.hi1.z, i1);
     i1 = dot4(p.hi1.w, a.hi1.w, i1);
-    const int sumi = p.sc0 * i0 + p.sc1 * i1;
-    const int summ = p.mn0 * a.bs_lo + p.mn1 * a.bs_hi;
+    // |i| <= 32 * 31 * 127 and |bsum32| <= 32 * 127 against 6-bit scales: every product fits 24 bits
+    const int sumi = mul24(p.sc0, i0) + mul24(p.sc1, i1);
+    const int summ = mul24(p.mn0, a.bs_lo) + mul24(p.mn1, a.bs_hi);
     return a.dx * (p.d * static_cast<float>(sumi) - p.dmin * static_cast<float>(summ));
 }
 
@@ -161,26 +162,22 @@ struct Q6KAct {
     float dx;
 };
 
-__device__ __forceinline__ int sum16(const uint4 &v) {
-    int s = 0;
-    s = dot4(0x01010101u, v.x, s);
-    s = dot4(0x01010101u, v.y, s);
-    s = dot4(0x01010101u, v.z, s);
-    s = dot4(0x01010101u, v.w, s);
-    return s;
-}
-
-__device__ __forceinline__ Q6KAct q6k_load_act(const int8_t *__restrict__ aq_blk, float dx, int q) {
+// The sum of the 16 activations starting at element 16*j is the Q8_K block's bsums[j]: quarter i of lane q starts
+// at element 128n + 32i + 16(q&1), so its sum is bsums[8n + 2i + (q&1)].
+__device__ __forceinline__ Q6KAct q6k_load_act(const int8_t *__restrict__ aq_blk, float dx,
+                                               const int16_t *__restrict__ bs_blk, int q) {
     Q6KAct a;
     const int8_t *p = aq_blk + 128 * (q >> 1) + 16 * (q & 1);
     a.a0 = *reinterpret_cast<const uint4 *>(p);
     a.a1 = *reinterpret_cast<const uint4 *>(p + 32);
     a.a2 = *reinterpret_cast<const uint4 *>(p + 64);
     a.a3 = *reinterpret_cast<const uint4 *>(p + 96);
-    a.s0 = sum16(a.a0);
-    a.s1 = sum16(a.a1);
-    a.s2 = sum16(a.a2);
-    a.s3 = sum16(a.a3);
+    const uint4 bs = *reinterpret_cast<const uint4 *>(bs_blk + 8 * (q >> 1));  // bsums[8n .. 8n+8)
+    const int sh = 16 * (q & 1);                                               // even or odd entry of each pair
+    a.s0 = static_cast<int>(bs.x << (16 - sh)) >> 16;
+    a.s1 = static_cast<int>(bs.y << (16 - sh)) >> 16;
+    a.s2 = static_cast<int>(bs.z << (16 - sh)) >> 16;
+    a.s3 = static_cast<int>(bs.w << (16 - sh)) >> 16;
     a.dx = dx;
     return a;
 }
@@ -244,8 +241,9 @@ __device__ __forceinline__ int dot16(const uint4 &u, const uint4 &a) {
 
 __device__ __forceinline__ float q6k_dot(const Q6KPrep &p, const Q6KAct &a) {
     const int p0 = dot16(p.u0, a.a0), p1 = dot16(p.u1, a.a1), p2 = dot16(p.u2, a.a2), p3 = dot16(p.u3, a.a3);
-    const int sumi =
-        p.s0 * (p0 - 32 * a.s0) + p.s1 * (p1 - 32 * a.s1) + p.s2 * (p2 - 32 * a.s2) + p.s3 * (p3 - 32 * a.s3);
+    // |p - 32 s| <= 16 * 63 * 127 + 32 * 16 * 127 against int8 scales: every product fits 24 bits
+    const int sumi = mul24(p.s0, p0 - 32 * a.s0) + mul24(p.s1, p1 - 32 * a.s1) + mul24(p.s2, p2 - 32 * a.s2) +
+                     mul24(p.s3, p3 - 32 * a.s3);
     return (p.d * a.dx) * static_cast<float>(sumi);
 }
 
@@ -255,7 +253,7 @@ __device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, 
 
 // ---------------------------------------------------------------------------------------------
 // One interface over the K-quant formats for the kernels that are templated on the ggml type id.
-// `bs_blk` (the activation block's 16 int16 sums) is ignored by Q6_K, whose rows have no mins.
+// `bs_blk` points at the activation block's 16 int16 sums.
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant>
 struct KQuant;
@@ -294,8 +292,8 @@ struct KQuant<kQ6K> {
     using Act = Q6KAct;
     using Regs = Q6KRegs;
     using Prep = Q6KPrep;
-    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *, int q) {
-        return q6k_load_act(aq_blk, dx, q);
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *bs_blk, int q) {
+        return q6k_load_act(aq_blk, dx, bs_blk, q);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q6k_load_block(blk, q); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q6k_prepare(r, q); }

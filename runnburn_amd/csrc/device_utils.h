@@ -28,6 +28,10 @@ __device__ __forceinline__ float ld_f16(const uint8_t *p) {
     return f16_bits_to_f32(*reinterpret_cast<const unsigned short *>(p));
 }
 
+// a * b for operands known to fit 24 signed bits (block sums times 6- or 8-bit scales): one full-rate multiply
+// where the 32-bit form takes a quarter-rate one
+__device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
+
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
 }
