@@ -90,6 +90,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     const size_t ebase = static_cast<size_t>(expert) * n_ff * row_bytes;
     const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
     const Staged st = stage_layout(lds, tmax, nb);
+    float2 *xch = reinterpret_cast<float2 *>(lds + stage_bytes(tmax, nb)) + wave * (kMaxChunkTokens * kRowsPerWave);
 
     for (uint32_t c0 = 0; c0 < count; c0 += tmax) {
         const uint32_t nt = min(tmax, count - c0);
@@ -97,7 +98,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         for (uint32_t t = 0; t < nt; t++) stage_row(lds, tmax, nb, t, sorted_token[start + c0 + t], aq, ad, abs);
         __syncthreads();
         for (uint32_t it = 0; it < iters; it++) {
-            const uint32_t row = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave + rsel;
+            const uint32_t row0_it = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave;
+            const uint32_t row = row0_it + rsel;
             const bool row_ok = row < n_ff;
             float gacc[kMaxChunkTokens], uacc[kMaxChunkTokens];
 #pragma unroll
@@ -117,18 +119,30 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                     }
                 }
             }
+            // The row sums land in the last lane of each row segment.  SiLU on them lane by lane would spend a full
+            // instruction stream per token on one or two useful lanes, so the (gate, up) pairs of all staged tokens go
+            // through a per-wave LDS slot and lane t * kRowsPerWave + r finishes token t of row r: one SiLU pass per
+            // row iteration.  LDS operations of one wave complete in order; the fence only pins the compiler's order.
 #pragma unroll
             for (int t = 0; t < kMaxChunkTokens; t++) {
                 if (static_cast<uint32_t>(t) < nt) {  // nt is workgroup-uniform
                     const float gs = seg_sum<kLanesPerRow>(gacc[t]);
                     const float us = seg_sum<kLanesPerRow>(uacc[t]);
-                    if (sub == kLanesPerRow - 1 && row_ok) {
-                        // crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up
-                        const float e = expf(-gs);
-                        mid[static_cast<size_t>(sorted_slot[start + c0 + t]) * n_ff + row] = (gs / (1.0f + e)) * us;
-                    }
+                    if (sub == kLanesPerRow - 1) xch[t * kRowsPerWave + rsel] = make_float2(gs, us);
                 }
             }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            if (static_cast<uint32_t>(lane) < nt * kRowsPerWave) {
+                const uint32_t t = lane / kRowsPerWave;
+                const uint32_t r2 = row0_it + lane % kRowsPerWave;
+                const float2 v = xch[lane];
+                if (r2 < n_ff) {
+                    // crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up
+                    const float e = expf(-v.x);
+                    mid[static_cast<size_t>(sorted_slot[start + c0 + t]) * n_ff + r2] = (v.x / (1.0f + e)) * v.y;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
     }
 }
@@ -371,8 +385,10 @@ void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView 
     const int rpw = rows_per_wave_for(nb_in);
     const TilePlan p = plan_tiles(n_ff, nb_in, groups.n_groups, rpw);
     const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
+    // staged activations, then one (gate, up) exchange slot per wave, staged token and row
+    const size_t lds_bytes = p.lds_bytes + kWavesPerWg * kMaxChunkTokens * 4 * sizeof(float2);
 #define RNB_LAUNCH_GU(R)                                                                                             \
-    hipLaunchKernelGGL(moe_gate_up_kernel<R>, grid, block, p.lds_bytes, stream, gate_all, up_all, act.qs, act.d,      \
+    hipLaunchKernelGGL(moe_gate_up_kernel<R>, grid, block, lds_bytes, stream, gate_all, up_all, act.qs, act.d,        \
                        act.bsums, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff,   \
                        nb_in, p.iters, p.tmax)
     if (rpw == 4)
