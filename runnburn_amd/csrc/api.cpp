@@ -147,9 +147,9 @@ int validate_matmul(const QuantInfo &qi, size_t w_len, size_t rows, size_t cols,
         return fail(RNB_HIP_INVALID_REQUEST, label + " shape mismatch: input=" + std::to_string(x_len) +
                                                  " output=" + std::to_string(out_len) + " expected output>=" +
                                                  std::to_string(seq * rows));
-    if (rows > 0x7fffffffu || seq > 65535u)
-        return fail(RNB_HIP_INVALID_REQUEST, label + " shape out of range: rows=" + std::to_string(rows) +
-                                                 " seq_len=" + std::to_string(seq));
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu || seq > 65535u)  // the kernels index with 32 bits
+        return fail(RNB_HIP_INVALID_REQUEST, label + " shape out of range: rows=" + std::to_string(rows) + " cols=" +
+                                                 std::to_string(cols) + " seq_len=" + std::to_string(seq));
     *seq_out = seq;
     return RNB_HIP_OK;
 }
@@ -313,6 +313,8 @@ int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t
                                                  std::to_string(token_count * n_embd));
     if (n_slots > 0x0fffffffu || token_count > 0x0fffffffu)
         return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer slot count out of range");
+    if (n_ff > 0x00ffffffu || n_embd > 0x00ffffffu)  // the kernels index with 32 bits
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 full-layer dims out of range");
     *shape = sh;
     return RNB_HIP_OK;
 }
@@ -808,7 +810,7 @@ int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols
     if (!w_dev || !x_dev || !out_dev) return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " null device pointer");
     if ((reinterpret_cast<uintptr_t>(w_dev) | reinterpret_cast<uintptr_t>(x_dev)) & 15u)
         return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " device pointers must be 16-byte aligned");
-    if (rows > 0x7fffffffu || seq_len > 65535u)
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu || seq_len > 65535u)
         return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " shape out of range");
     if (rows == 0 || seq_len == 0) return RNB_HIP_OK;
     Guard g;
@@ -824,6 +826,8 @@ int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, siz
                                                  std::to_string(qi.elems) + ", got " + std::to_string(cols));
     if (!x_dev || (reinterpret_cast<uintptr_t>(x_dev) & 15u))
         return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " input must be a 16-byte aligned device pointer");
+    if (cols > 0x7fffffffu || seq_len > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " shape out of range");
     if (seq_len == 0) return RNB_HIP_OK;
     Guard g;
     if (!g.state) return g.status;

@@ -87,6 +87,17 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q8_0 input length mismatch: got 33, expected 32"
 
 
+def test_shapes_beyond_32_bit_indexing_are_refused():
+    z = np.zeros
+    e = _err(rnb.q4k_gemv_batch, z(0, np.uint8), 0, 1 << 32, z(0, np.float32))
+    assert str(e) == "Q4_K shape out of range: rows=0 cols=4294967296 seq_len=0"
+    e = _err(rnb.q8_0_gemv_batch, z(0, np.uint8), 0, 1 << 31, z(0, np.float32))
+    assert "shape out of range" in str(e)
+    e = _err(rnb.qwen35_sparse_experts_selected_base_by_token, z(0, np.uint8), z(0, np.uint8), z(0, np.uint8), [], [], [],
+             0, 14, 1 << 24, 256, z(0, np.float32))
+    assert str(e) == "Qwen35 full-layer dims out of range"
+
+
 def test_moe_validation_messages():
     """crates/rnb-backend/cuda/src/runtime/helpers.rs:1570-1600, 2747-2800"""
     z = np.zeros
