@@ -14,9 +14,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "librnb_oracle.so")
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14  # ggml type ids (crates/rnb-loader/src/gguf/types.rs:5-41)
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256}
+Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14  # ggml type ids (crates/rnb-loader/src/gguf/types.rs:5-41)
+BLOCK_BYTES = {Q8_0: 34, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q2_K: 256, Q3_K: 256, Q4_K: 256, Q5_K: 256, Q6_K: 256}
 
 Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
 Q8_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (32,))])
@@ -47,17 +47,19 @@ def lib() -> C.CDLL:
         L.rnbo_nearest_int.argtypes = [f32]
         L.rnbo_get_scale_min_k4.restype = None
         L.rnbo_get_scale_min_k4.argtypes = [i32, vp, vp, vp]
-        for name in ("rnbo_dequantize_q8_0", "rnbo_dequantize_q4_k", "rnbo_dequantize_q5_k", "rnbo_dequantize_q6_k"):
+        for name in ("rnbo_dequantize_q8_0", "rnbo_dequantize_q2_k", "rnbo_dequantize_q3_k", "rnbo_dequantize_q4_k",
+                     "rnbo_dequantize_q5_k", "rnbo_dequantize_q6_k"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, sz, vp]
         for name in ("rnbo_quantize_q8k", "rnbo_quantize_q8"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, sz, vp]
-        for name in ("rnbo_dot_q4k_q8k", "rnbo_dot_q5k_q8k", "rnbo_dot_q6k_q8k", "rnbo_dot_q8_0_q8", "rnbo_dot_q8_0_f32",
+        for name in ("rnbo_dot_q2k_q8k", "rnbo_dot_q3k_q8k", "rnbo_dot_q4k_q8k", "rnbo_dot_q5k_q8k", "rnbo_dot_q6k_q8k", "rnbo_dot_q8_0_q8", "rnbo_dot_q8_0_f32",
                      "rnbo_dot_q4k_q8k_avx2", "rnbo_dot_q6k_q8k_avx2"):
             getattr(L, name).restype = f32
             getattr(L, name).argtypes = [vp, vp, sz]
-        for name in ("rnbo_dot_q4k_q8k_f64", "rnbo_dot_q5k_q8k_f64", "rnbo_dot_q6k_q8k_f64", "rnbo_dot_q8_0_q8_f64"):
+        for name in ("rnbo_dot_q2k_q8k_f64", "rnbo_dot_q3k_q8k_f64", "rnbo_dot_q4k_q8k_f64", "rnbo_dot_q5k_q8k_f64",
+                     "rnbo_dot_q6k_q8k_f64", "rnbo_dot_q8_0_q8_f64"):
             getattr(L, name).restype = C.c_double
             getattr(L, name).argtypes = [vp, vp, sz]
         for name in ("rnbo_gemv", "rnbo_gemv_f64", "rnbo_gemv_avx2"):
@@ -72,7 +74,8 @@ def lib() -> C.CDLL:
         L.rnbo_moe_sparse_experts_by_token.restype = i32
         L.rnbo_moe_sparse_experts_by_token.argtypes = [vp, vp, vp, sz, vp, vp, vp, sz, sz, u32, sz, sz,
                                                        vp, vp, i32]
-        for name in ("rnbo_quantize_row_q4_k", "rnbo_quantize_row_q5_k", "rnbo_quantize_row_q6_k", "rnbo_quantize_row_q8_0"):
+        for name in ("rnbo_quantize_row_q2_k", "rnbo_quantize_row_q3_k", "rnbo_quantize_row_q4_k", "rnbo_quantize_row_q5_k",
+                     "rnbo_quantize_row_q6_k", "rnbo_quantize_row_q8_0"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, sz, vp]
         L.rnbo_fill_normal.restype = None
@@ -128,8 +131,8 @@ def dequantize(quant: int, blocks) -> np.ndarray:
     n = b.size // BLOCK_BYTES[quant]
     assert n * BLOCK_BYTES[quant] == b.size
     out = np.empty(n * BLOCK_ELEMS[quant], dtype=np.float32)
-    fn = {Q8_0: "rnbo_dequantize_q8_0", Q4_K: "rnbo_dequantize_q4_k", Q5_K: "rnbo_dequantize_q5_k",
-          Q6_K: "rnbo_dequantize_q6_k"}[quant]
+    fn = {Q8_0: "rnbo_dequantize_q8_0", Q2_K: "rnbo_dequantize_q2_k", Q3_K: "rnbo_dequantize_q3_k",
+          Q4_K: "rnbo_dequantize_q4_k", Q5_K: "rnbo_dequantize_q5_k", Q6_K: "rnbo_dequantize_q6_k"}[quant]
     getattr(lib(), fn)(_p(b), n, _p(out))
     return out
 
@@ -158,8 +161,8 @@ def dot(quant: int, row, act: np.ndarray, gold: bool = False, avx2: bool = False
     r = _u8(row)
     nb = r.size // BLOCK_BYTES[quant]
     assert act.size == nb
-    base = {Q8_0: "rnbo_dot_q8_0_q8", Q4_K: "rnbo_dot_q4k_q8k", Q5_K: "rnbo_dot_q5k_q8k",
-            Q6_K: "rnbo_dot_q6k_q8k"}[quant]
+    base = {Q8_0: "rnbo_dot_q8_0_q8", Q2_K: "rnbo_dot_q2k_q8k", Q3_K: "rnbo_dot_q3k_q8k", Q4_K: "rnbo_dot_q4k_q8k",
+            Q5_K: "rnbo_dot_q5k_q8k", Q6_K: "rnbo_dot_q6k_q8k"}[quant]
     if gold:
         base += "_f64"
     elif avx2:
@@ -250,8 +253,8 @@ def quantize_row(quant: int, x) -> np.ndarray:
     x = _f32(x).ravel()
     assert x.size % BLOCK_ELEMS[quant] == 0
     out = np.zeros(x.size // BLOCK_ELEMS[quant] * BLOCK_BYTES[quant], dtype=np.uint8)
-    fn = {Q8_0: "rnbo_quantize_row_q8_0", Q4_K: "rnbo_quantize_row_q4_k", Q5_K: "rnbo_quantize_row_q5_k",
-          Q6_K: "rnbo_quantize_row_q6_k"}[quant]
+    fn = {Q8_0: "rnbo_quantize_row_q8_0", Q2_K: "rnbo_quantize_row_q2_k", Q3_K: "rnbo_quantize_row_q3_k",
+          Q4_K: "rnbo_quantize_row_q4_k", Q5_K: "rnbo_quantize_row_q5_k", Q6_K: "rnbo_quantize_row_q6_k"}[quant]
     getattr(lib(), fn)(_p(x), x.size, _p(out))
     return out
 

@@ -17,6 +17,11 @@
  *   quantize_q8                 closed-form cases + numpy restatement (formula is 6 lines)
  *   dot_q4k_q8k                 reference closed forms 0 / 0 / 2560.0 (tile_q4k.rs:2019-2151),
  *                               f64 numpy dequant(W) . dequant(Q8K(x)) identity
+ *   dequantize_q2_k/_q3_k       the reference's own vectors (dequant.rs:898-927, 1009-1019: zero blocks, qs[1] = 3 ->
+ *                               out[1] = 3) + one-hot placement of every field + independent numpy statements
+ *   dot_q2k_q8k, dot_q3k_q8k    hand-built vectors per sub-block scale / min / high bit, f64 numpy dequant
+ *                               identity (the reference's AVX2 kernels are checked the same way, loosely:
+ *                               avx2_dot.rs tests)
  *   dot_q5k_q8k                 one-hot fifth-bit vectors (each qh bit moves exactly the element the
  *                               reference's tile_q5k.rs:944-976 statement names), f64 numpy dequant
  *                               identity, reduction to dot_q4k_q8k when qh == 0
@@ -32,6 +37,9 @@
  *                               Input generation only -- GPU and oracle consume identical bytes.
  *   quantize_row_q5_k           as quantize_row_q4_k: byte parity UNPINNED, the reference's round-trip
  *                               property (quant.rs:732-764) is checked.  Input generation only.
+ *   quantize_row_q2_k           restates quant.rs:44-160; byte parity UNPINNED (cannot run the original), the
+ *                               reference's round-trip bound (cosine >= 0.90) is checked.  Input generation only.
+ *   quantize_row_q3_k           not in the reference (plain symmetric fit).  Input generation only.
  *   quantize_row_q6_k/_q8_0     not in the reference at all (ggml reference semantics); round
  *                               trip through the pinned dequantisers.  Input generation only.
  */
@@ -143,6 +151,65 @@ void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out) {
         const uint8_t *blk = blocks + b * RNBO_Q8_0_BLOCK_BYTES;
         float d = rd_f16(blk);
         for (int i = 0; i < 32; i++) out[b * 32 + i] = (float)(int8_t)blk[2 + i] * d;
+    }
+}
+
+/* crates/rnb-cpu/src/quantize/dequant.rs:66-86.  Block = {u8 scales[16] (scale | min << 4), u8 qs[64], f16 d,
+ * f16 dmin}; sub-block j (16 elements) lives in half j/8, bytes 16*(j%2).. of that half's 32, bit pair (j%8)/2. */
+void rnbo_dequantize_q2_k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * RNBO_Q2_K_BLOCK_BYTES;
+        const uint8_t *qs = blk + 16;
+        float d = rd_f16(blk + 80), dmin = rd_f16(blk + 82);
+        float *y = out + b * 256;
+        for (int j = 0; j < 16; j++) {
+            float scale = d * (float)(blk[j] & 0x0f);
+            float min = dmin * (float)(blk[j] >> 4);
+            int q_base = (j / 8) * 32 + (j % 2) * 16, shift = ((j % 8) / 2) * 2;
+            for (int l = 0; l < 16; l++) {
+                float q = (float)((qs[q_base + l] >> shift) & 3);
+                y[16 * j + l] = q * scale - min;
+            }
+        }
+    }
+}
+
+/* The sixteen 6-bit scales of a Q3_K block: crates/rnb-cpu/src/quantize/dequant.rs:240-263.  Scale k keeps its
+ * low four bits in nibble k/8 of byte k%8 and its high two in bit pair k/4 of byte 8 + k%4. */
+static void q3k_scales(const uint8_t *sb, int8_t *scales) {
+    for (int k = 0; k < 16; k++) {
+        int lo = (k < 8) ? (sb[k] & 0x0f) : (sb[k - 8] >> 4);
+        int hi = (sb[8 + (k % 4)] >> (2 * (k / 4))) & 3;
+        scales[k] = (int8_t)(lo | (hi << 4));
+    }
+}
+
+/* crates/rnb-cpu/src/quantize/dequant.rs:237-297.  Block = {u8 hmask[32], u8 qs[64], u8 scales[12], f16 d}; the
+ * value is the 2-bit field minus 4 unless its hmask bit is set; qs is laid out as for Q2_K and the 32-element
+ * group g = 4*half + bit-pair uses bit g of hmask[l]. */
+void rnbo_dequantize_q3_k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * RNBO_Q3_K_BLOCK_BYTES;
+        const uint8_t *hm = blk, *q = blk + 32;
+        float d_all = rd_f16(blk + 108);
+        int8_t scales[16];
+        q3k_scales(blk + 96, scales);
+        float *y = out + b * 256;
+        int is = 0;
+        uint8_t m = 1;
+        for (int n = 0; n < 2; n++) {
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int h = 0; h < 2; h++) {
+                    float dl = d_all * ((float)scales[is++] - 32.0f);
+                    for (int l = 0; l < 16; l++) {
+                        int qv = (q[32 * n + 16 * h + l] >> shift) & 3;
+                        int hv = (hm[16 * h + l] & m) ? 0 : 4;
+                        *y++ = dl * (float)(qv - hv);
+                    }
+                }
+                m = (uint8_t)(m << 1);
+            }
+        }
     }
 }
 
@@ -339,6 +406,95 @@ double rnbo_dot_q4k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_
     return acc;
 }
 
+/* integer parts of one Q2_K block: crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242 (sub-block scales times 16-element
+ * dots; mins times the Q8_K block's 16-element sums) */
+static inline void q2k_block_ints(const uint8_t *blk, const rnbo_q8k_block *a, int32_t *sumi_out,
+                                  int32_t *summ_out) {
+    const uint8_t *qs = blk + 16;
+    int32_t sumi = 0, summ = 0;
+    for (int j = 0; j < 16; j++) {
+        int q_base = (j / 8) * 32 + (j % 2) * 16, shift = ((j % 8) / 2) * 2;
+        int32_t p = 0;
+        for (int l = 0; l < 16; l++) p += (int32_t)((qs[q_base + l] >> shift) & 3) * (int32_t)a->qs[16 * j + l];
+        sumi += (int32_t)(blk[j] & 0x0f) * p;
+        summ += (int32_t)(blk[j] >> 4) * (int32_t)a->bsums[j];
+    }
+    *sumi_out = sumi;
+    *summ_out = summ;
+}
+
+/* crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242 (dot_q2k_q8k_avx2): per block acc += (-d_x * dmin) * summ, then
+ * acc += (d_x * d) * sumi.  The reference keeps eight f32 lanes and adds them at the end; this form adds in block
+ * order -- the difference is f32 summation order only. */
+float rnbo_dot_q2k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q2_K_BLOCK_BYTES;
+        int32_t sumi, summ;
+        q2k_block_ints(blk, &act[b], &sumi, &summ);
+        volatile float d = act[b].d * rd_f16(blk + 80);
+        volatile float dmin = act[b].d * rd_f16(blk + 82);
+        volatile float t1 = dmin * (float)summ;
+        volatile float t0 = d * (float)sumi;
+        acc -= t1;
+        acc += t0;
+    }
+    return acc;
+}
+
+double rnbo_dot_q2k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    double acc = 0.0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q2_K_BLOCK_BYTES;
+        int32_t sumi, summ;
+        q2k_block_ints(blk, &act[b], &sumi, &summ);
+        acc += (double)act[b].d * ((double)rd_f16(blk + 80) * (double)sumi - (double)rd_f16(blk + 82) * (double)summ);
+    }
+    return acc;
+}
+
+/* integer part of one Q3_K block: crates/rnb-cpu/src/gemm/avx2_dot.rs:247-375 */
+static inline int32_t q3k_block_int(const uint8_t *blk, const rnbo_q8k_block *a) {
+    const uint8_t *hm = blk, *q = blk + 32;
+    int8_t scales[16];
+    q3k_scales(blk + 96, scales);
+    int32_t sumi = 0;
+    for (int j = 0; j < 16; j++) {
+        int n = j / 8, pair = (j % 8) / 2, h = j % 2;
+        uint8_t m = (uint8_t)(1u << (4 * n + pair));
+        int32_t p = 0;
+        for (int l = 0; l < 16; l++) {
+            int qv = (q[32 * n + 16 * h + l] >> (2 * pair)) & 3;
+            int hv = (hm[16 * h + l] & m) ? 0 : 4;
+            p += (int32_t)(qv - hv) * (int32_t)a->qs[16 * j + l];
+        }
+        sumi += ((int32_t)scales[j] - 32) * p;
+    }
+    return sumi;
+}
+
+/* crates/rnb-cpu/src/gemm/avx2_dot.rs:247-375 (dot_q3k_q8k_avx2): acc += (d_x * d) * sumi per block */
+float rnbo_dot_q3k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q3_K_BLOCK_BYTES;
+        int32_t sumi = q3k_block_int(blk, &act[b]);
+        volatile float d = act[b].d * rd_f16(blk + 108);
+        volatile float t = d * (float)sumi;
+        acc += t;
+    }
+    return acc;
+}
+
+double rnbo_dot_q3k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
+    double acc = 0.0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * RNBO_Q3_K_BLOCK_BYTES;
+        acc += (double)act[b].d * (double)rd_f16(blk + 108) * (double)q3k_block_int(blk, &act[b]);
+    }
+    return acc;
+}
+
 /* integer part of one Q5_K block: crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 */
 static inline void q5k_block_ints(const uint8_t *blk, const rnbo_q8k_block *a, int32_t *sumi_out,
                                   int32_t *summ_out) {
@@ -494,6 +650,8 @@ float rnbo_dot_q8_0_f32(const uint8_t *row, const float *x, size_t nb) {
 static size_t block_bytes_of(uint32_t quant, size_t *elems) {
     switch (quant) {
     case 8: *elems = 32; return RNBO_Q8_0_BLOCK_BYTES;
+    case 10: *elems = 256; return RNBO_Q2_K_BLOCK_BYTES;
+    case 11: *elems = 256; return RNBO_Q3_K_BLOCK_BYTES;
     case 12: *elems = 256; return RNBO_Q4_K_BLOCK_BYTES;
     case 13: *elems = 256; return RNBO_Q5_K_BLOCK_BYTES;
     case 14: *elems = 256; return RNBO_Q6_K_BLOCK_BYTES;
@@ -503,6 +661,8 @@ static size_t block_bytes_of(uint32_t quant, size_t *elems) {
 
 static float kquant_dot(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
     switch (quant) {
+    case 10: return rnbo_dot_q2k_q8k(row, act, nb);
+    case 11: return rnbo_dot_q3k_q8k(row, act, nb);
     case 12: return rnbo_dot_q4k_q8k(row, act, nb);
     case 13: return rnbo_dot_q5k_q8k(row, act, nb);
     default: return rnbo_dot_q6k_q8k(row, act, nb);
@@ -511,6 +671,8 @@ static float kquant_dot(uint32_t quant, const uint8_t *row, const rnbo_q8k_block
 
 static double kquant_dot_f64(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t nb) {
     switch (quant) {
+    case 10: return rnbo_dot_q2k_q8k_f64(row, act, nb);
+    case 11: return rnbo_dot_q3k_q8k_f64(row, act, nb);
     case 12: return rnbo_dot_q4k_q8k_f64(row, act, nb);
     case 13: return rnbo_dot_q5k_q8k_f64(row, act, nb);
     default: return rnbo_dot_q6k_q8k_f64(row, act, nb);
@@ -911,6 +1073,92 @@ void rnbo_quantize_row_q5_k(const float *input, size_t n, uint8_t *output) {
     }
 }
 
+/* crates/rnb-cpu/src/quantize/quant.rs:44-160 (quantize_row_q2_k): min/max fit per 16 elements, 4-bit scale and min
+ * codes against d = max scale / 15 and dmin = max min / 15.  Byte parity with the Rust original is UNPINNED
+ * (cannot run it); input generation only. */
+void rnbo_quantize_row_q2_k(const float *input, size_t n, uint8_t *output) {
+    const float eps = 1e-10f;
+    for (size_t sb = 0; sb < n / 256; sb++) {
+        const float *x = input + sb * 256;
+        uint8_t *out = output + sb * RNBO_Q2_K_BLOCK_BYTES;
+        float sub_scale[16], sub_min[16];
+        uint8_t q[256];
+        memset(q, 0, sizeof q);
+        for (int j = 0; j < 16; j++) {
+            const float *xs = x + 16 * j;
+            float lo = xs[0], hi = xs[0];
+            for (int l = 1; l < 16; l++) {
+                if (xs[l] < lo) lo = xs[l];
+                if (xs[l] > hi) hi = xs[l];
+            }
+            float base = lo <= 0.0f ? lo : 0.0f;
+            float range = hi - base;
+            sub_scale[j] = range > eps ? range / 3.0f : 0.0f;
+            sub_min[j] = -base;
+            if (sub_scale[j] > eps)
+                for (int l = 0; l < 16; l++) {
+                    float r = roundf((xs[l] - base) / sub_scale[j]);
+                    q[16 * j + l] = (uint8_t)(r < 0.0f ? 0.0f : (r > 3.0f ? 3.0f : r));
+                }
+        }
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 16; j++) {
+            if (sub_scale[j] > max_scale) max_scale = sub_scale[j];
+            if (sub_min[j] > max_min) max_min = sub_min[j];
+        }
+        float d = max_scale > eps ? max_scale / 15.0f : 0.0f, dmin = max_min > eps ? max_min / 15.0f : 0.0f;
+        for (int j = 0; j < 16; j++) {
+            float sc = d > eps ? roundf(sub_scale[j] / d) : 0.0f, mn = dmin > eps ? roundf(sub_min[j] / dmin) : 0.0f;
+            sc = sc < 0.0f ? 0.0f : (sc > 15.0f ? 15.0f : sc);
+            mn = mn < 0.0f ? 0.0f : (mn > 15.0f ? 15.0f : mn);
+            out[j] = (uint8_t)(((uint8_t)mn << 4) | ((uint8_t)sc & 0x0f));
+        }
+        memset(out + 16, 0, 64);
+        for (int i = 0; i < 256; i++)
+            out[16 + (i / 128) * 32 + i % 32] |= (uint8_t)((q[i] & 3) << (((i % 128) / 32) * 2));
+        wr_f16(out + 80, d);
+        wr_f16(out + 82, dmin);
+    }
+}
+
+/* Q3_K generator: NOT in the reference repository.  Symmetric fit per 16 elements (scale = max |x| / 4), 6-bit scale
+ * codes 32 + round(scale / d) against d = max scale / 31, values round(x / (d * code)) in -4..3. */
+void rnbo_quantize_row_q3_k(const float *input, size_t n, uint8_t *output) {
+    for (size_t sb = 0; sb < n / 256; sb++) {
+        const float *x = input + sb * 256;
+        uint8_t *out = output + sb * RNBO_Q3_K_BLOCK_BYTES;
+        float sub_scale[16], max_scale = 0.0f;
+        for (int j = 0; j < 16; j++) {
+            float amax = 0.0f;
+            for (int l = 0; l < 16; l++) amax = fmaxf(amax, fabsf(x[16 * j + l]));
+            sub_scale[j] = amax / 4.0f;
+            max_scale = fmaxf(max_scale, sub_scale[j]);
+        }
+        memset(out, 0, RNBO_Q3_K_BLOCK_BYTES);
+        wr_f16(out + 108, max_scale / 31.0f);
+        float d = rd_f16(out + 108);
+        for (int j = 0; j < 16; j++) {
+            int code = d > 0.0f ? (int)roundf(sub_scale[j] / d) : 0;
+            code = code < 0 ? 0 : (code > 31 ? 31 : code);
+            int stored = code + 32; /* 6 bits: low four in byte j%8 (nibble j/8), high two in byte 8 + j%4 */
+            if (j < 8)
+                out[96 + j] |= (uint8_t)(stored & 0x0f);
+            else
+                out[96 + j - 8] |= (uint8_t)((stored & 0x0f) << 4);
+            out[96 + 8 + (j % 4)] |= (uint8_t)(((stored >> 4) & 3) << (2 * (j / 4)));
+            float step = d * (float)code;
+            int n_half = j / 8, pair = (j % 8) / 2, h = j % 2;
+            for (int l = 0; l < 16; l++) {
+                int v = step > 0.0f ? (int)roundf(x[16 * j + l] / step) : 0;
+                v = v < -4 ? -4 : (v > 3 ? 3 : v);
+                int u = v + 4; /* 0..7: low two bits in qs, the third bit set in hmask */
+                out[32 + 32 * n_half + 16 * h + l] |= (uint8_t)((u & 3) << (2 * pair));
+                if (u & 4) out[16 * h + l] |= (uint8_t)(1u << (4 * n_half + pair));
+            }
+        }
+    }
+}
+
 /* Symmetric fit used by the Q6_K generator (ggml reference `make_qx_quants`, rmse_type 1,
  * no external quant weights: w = x^2).  NOT in the reference repository. */
 static float make_qx_quants(int n, int nmax, const float *x, int8_t *L) {
@@ -1071,7 +1319,11 @@ int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, f
         for (long r = 0; r < (long)rows; r++) {
             for (size_t c = 0; c < cols; c++) row[c] = normal_at(seed, (uint64_t)r * cols + c, sigma);
             uint8_t *dst = out + (size_t)r * row_bytes;
-            if (quant == 12)
+            if (quant == 10)
+                rnbo_quantize_row_q2_k(row, cols, dst);
+            else if (quant == 11)
+                rnbo_quantize_row_q3_k(row, cols, dst);
+            else if (quant == 12)
                 rnbo_quantize_row_q4_k(row, cols, dst);
             else if (quant == 13)
                 rnbo_quantize_row_q5_k(row, cols, dst);

@@ -23,6 +23,8 @@ struct QuantInfo {
 bool quant_info(uint32_t quant, QuantInfo *qi) {
     switch (quant) {
     case kQ8_0: *qi = {"Q8_0", 32, kQ8_0Bytes}; return true;
+    case kQ2K: *qi = {"Q2_K", 256, kQ2KBytes}; return true;
+    case kQ3K: *qi = {"Q3_K", 256, kQ3KBytes}; return true;
     case kQ4K: *qi = {"Q4_K", 256, kQ4KBytes}; return true;
     case kQ5K: *qi = {"Q5_K", 256, kQ5KBytes}; return true;
     case kQ6K: *qi = {"Q6_K", 256, kQ6KBytes}; return true;
@@ -100,6 +102,11 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);
+    } else if (quant == kQ2K || quant == kQ3K) {
+        if (seq >= kTokensMinSeq)
+            launch_matmul_tokens(w_dev, quant, act, out_dev, r, nb, q, s.stream);
+        else
+            launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ5K) {
         if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ5K, act, out_dev, r, nb, q, s.stream);
@@ -451,7 +458,7 @@ int rnb_hip_backend_kind(void) { return 6; }
 int rnb_hip_backend_supports(int op) { return (op == RNB_OP_MATMUL || op == RNB_OP_MOE) ? 1 : 0; }
 
 int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
-    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
+    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || (quant >= kQ2K && quant <= kQ6K)) ? 1 : 0;
     if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
     return 0;
 }
@@ -595,6 +602,22 @@ int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, c
 int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                            float *out, size_t out_len) {
     return matmul_host(kQ4K, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+int rnb_hip_q2k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                     float *out, size_t out_len) {
+    return matmul_host(kQ2K, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q2k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                           float *out, size_t out_len) {
+    return matmul_host(kQ2K, w, w_len, rows, cols, x, x_len, out, out_len, true);
+}
+int rnb_hip_q3k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                     float *out, size_t out_len) {
+    return matmul_host(kQ3K, w, w_len, rows, cols, x, x_len, out, out_len, false);
+}
+int rnb_hip_q3k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                           float *out, size_t out_len) {
+    return matmul_host(kQ3K, w, w_len, rows, cols, x, x_len, out, out_len, true);
 }
 int rnb_hip_q5k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                      float *out, size_t out_len) {

@@ -2,7 +2,7 @@
 // the decode GEMV and the gathered-MoE kernels.  FOUR lanes cooperate on a 256-element block (a wave64
 // pass covers 16 blocks); the caller adds the partials across lanes.  Activations are held in
 // registers (`Q4KAct` / `Q6KAct`) so that a wave which walks many rows loads them once.
-// `KQuant<id>` at the end gives the kernels one interface over the three K-quant formats.
+// `KQuant<id>` at the end gives the kernels one interface over the K-quant formats.
 #pragma once
 
 #include "device_utils.h"
@@ -252,11 +252,157 @@ __device__ __forceinline__ float q6k_partial(const Q6KRegs &r, const Q6KAct &a, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Q2_K: block = {u8 scales[16] (scale | min << 4), u8 qs[64], f16 d, f16 dmin}, 84 bytes, 4-byte aligned.
+// Q3_K: block = {u8 hmask[32], u8 qs[64], u8 scales[12], f16 d}, 110 bytes, 2-byte aligned.
+// Both keep sixteen 16-element sub-blocks and lay qs out alike: byte 32n + l holds elements 128n + 32i + l in bit
+// pair i.  Lane q owns half n = q>>1, l = 16*(q&1) .. +16, i.e. one 16-byte piece of qs and, as for Q6_K, the four
+// activation quarters 128n + 32i + 16*(q&1) with sub-block index 8n + 2i + (q&1): activation state is Q6KAct.
+//   Q2_K: sum_i sc_i * dot(u_i, a_i) and sum_i mn_i * bsums_i           crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242
+//   Q3_K: value = u - 4 + 4 * hbit (bit 4n + i of hmask[l]), signed scale = 6-bit code - 32; (u + 4 hbit - 4) is applied
+//         as dot(u | hbit << 2, a) - 4 * sum(a)                          crates/rnb-cpu/src/gemm/avx2_dot.rs:247-375
+// ---------------------------------------------------------------------------------------------
+struct Q2KRegs {
+    uint4 q;        // 16 bytes of packed 2-bit values
+    uint2 s;        // scale bytes 8n .. 8n+8
+    uint32_t dd;    // f16 d | f16 dmin << 16
+};
+
+__device__ __forceinline__ Q2KRegs q2k_load_block(const uint8_t *__restrict__ blk, int q) {
+    Q2KRegs r;
+    r.q = ld_u4_a2(blk + 16 + 32 * (q >> 1) + 16 * (q & 1));
+    r.s = ld_u2_a2(blk + 8 * (q >> 1));
+    r.dd = ld_u32_a2(blk + 80);
+    return r;
+}
+
+struct Q2KPrep {
+    uint4 u0, u1, u2, u3;  // 16 two-bit (Q3_K: three-bit) values of each activation quarter, one per byte
+    int s0, s1, s2, s3;    // sub-block scales
+    int m0, m1, m2, m3;    // sub-block mins (Q2_K only)
+    float d, dmin;
+};
+
+__device__ __forceinline__ Q2KPrep q2k_prepare(const Q2KRegs &r, int q) {
+    Q2KPrep p;
+    const int sh = 8 * (q & 1);  // sub-block 8n + 2i + (q&1): byte (q&1) of each 16-bit pair
+    const uint32_t b0 = (r.s.x >> sh) & 0xffu, b1 = (r.s.x >> (16 + sh)) & 0xffu;
+    const uint32_t b2 = (r.s.y >> sh) & 0xffu, b3 = (r.s.y >> (16 + sh)) & 0xffu;
+    p.s0 = b0 & 15; p.m0 = b0 >> 4;
+    p.s1 = b1 & 15; p.m1 = b1 >> 4;
+    p.s2 = b2 & 15; p.m2 = b2 >> 4;
+    p.s3 = b3 & 15; p.m3 = b3 >> 4;
+    p.d = f16_bits_to_f32(r.dd);
+    p.dmin = f16_bits_to_f32(r.dd >> 16);
+#define RNB_Q2_UNPACK(k)                      \
+    p.u0.k = r.q.k & 0x03030303u;             \
+    p.u1.k = (r.q.k >> 2) & 0x03030303u;      \
+    p.u2.k = (r.q.k >> 4) & 0x03030303u;      \
+    p.u3.k = (r.q.k >> 6) & 0x03030303u;
+    RNB_Q2_UNPACK(x)
+    RNB_Q2_UNPACK(y)
+    RNB_Q2_UNPACK(z)
+    RNB_Q2_UNPACK(w)
+#undef RNB_Q2_UNPACK
+    return p;
+}
+
+__device__ __forceinline__ float q2k_dot(const Q2KPrep &p, const Q6KAct &a) {
+    const int sumi = mul24(p.s0, dot16(p.u0, a.a0)) + mul24(p.s1, dot16(p.u1, a.a1)) + mul24(p.s2, dot16(p.u2, a.a2)) +
+                     mul24(p.s3, dot16(p.u3, a.a3));
+    const int summ = mul24(p.m0, a.s0) + mul24(p.m1, a.s1) + mul24(p.m2, a.s2) + mul24(p.m3, a.s3);
+    return (a.dx * p.d) * static_cast<float>(sumi) - (a.dx * p.dmin) * static_cast<float>(summ);
+}
+
+struct Q3KRegs {
+    uint4 q, hm;       // 16 bytes of packed low bits, the 16 hmask bytes of the same l range
+    uint2 s01;         // scale bytes 0..7 (low nibbles of codes 0..7, high nibbles of codes 8..15)
+    uint32_t s2;       // scale bytes 8..11 (two high bits of every code)
+    uint32_t d_bits;
+};
+
+__device__ __forceinline__ Q3KRegs q3k_load_block(const uint8_t *__restrict__ blk, int q) {
+    Q3KRegs r;
+    r.hm = ld_u4_a2(blk + 16 * (q & 1));
+    r.q = ld_u4_a2(blk + 32 + 32 * (q >> 1) + 16 * (q & 1));
+    r.s01 = ld_u2_a2(blk + 96);
+    r.s2 = ld_u32_a2(blk + 104);
+    r.d_bits = *reinterpret_cast<const unsigned short *>(blk + 108);
+    return r;
+}
+
+// code k = 8n + 2i + h: low nibble from nibble n of byte k%8 = 2i + h, high bits from bit pair k/4 = 2n + i/2 of
+// byte 8 + k%4 = 8 + 2(i%2) + h
+__device__ __forceinline__ int q3k_code(const Q3KRegs &r, int n, int i, int h) {
+    const uint32_t lo_word = (i < 2) ? r.s01.x : r.s01.y;
+    const uint32_t lo = (lo_word >> (8 * (2 * (i & 1) + h) + 4 * n)) & 15u;
+    const uint32_t hi = (r.s2 >> (8 * (2 * (i & 1) + h) + 2 * (2 * n + (i >> 1)))) & 3u;
+    return static_cast<int>(lo | (hi << 4)) - 32;
+}
+
+__device__ __forceinline__ Q2KPrep q3k_prepare(const Q3KRegs &r, int q) {
+    Q2KPrep p;
+    const int n = q >> 1, h = q & 1;
+    p.s0 = q3k_code(r, n, 0, h);
+    p.s1 = q3k_code(r, n, 1, h);
+    p.s2 = q3k_code(r, n, 2, h);
+    p.s3 = q3k_code(r, n, 3, h);
+    p.m0 = p.m1 = p.m2 = p.m3 = 0;
+    p.d = f16_bits_to_f32(r.d_bits);
+    p.dmin = 0.0f;
+    const int hb = 4 * n;  // hmask bit of quarter i is 4n + i
+#define RNB_Q3_UNPACK(k)                                                               \
+    p.u0.k = (r.q.k & 0x03030303u) | (((r.hm.k >> hb) & 0x01010101u) << 2);            \
+    p.u1.k = ((r.q.k >> 2) & 0x03030303u) | (((r.hm.k >> (hb + 1)) & 0x01010101u) << 2); \
+    p.u2.k = ((r.q.k >> 4) & 0x03030303u) | (((r.hm.k >> (hb + 2)) & 0x01010101u) << 2); \
+    p.u3.k = ((r.q.k >> 6) & 0x03030303u) | (((r.hm.k >> (hb + 3)) & 0x01010101u) << 2);
+    RNB_Q3_UNPACK(x)
+    RNB_Q3_UNPACK(y)
+    RNB_Q3_UNPACK(z)
+    RNB_Q3_UNPACK(w)
+#undef RNB_Q3_UNPACK
+    return p;
+}
+
+__device__ __forceinline__ float q3k_dot(const Q2KPrep &p, const Q6KAct &a) {
+    const int sumi = mul24(p.s0, dot16(p.u0, a.a0) - 4 * a.s0) + mul24(p.s1, dot16(p.u1, a.a1) - 4 * a.s1) +
+                     mul24(p.s2, dot16(p.u2, a.a2) - 4 * a.s2) + mul24(p.s3, dot16(p.u3, a.a3) - 4 * a.s3);
+    return (a.dx * p.d) * static_cast<float>(sumi);
+}
+
+// ---------------------------------------------------------------------------------------------
 // One interface over the K-quant formats for the kernels that are templated on the ggml type id.
 // `bs_blk` points at the activation block's 16 int16 sums.
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant>
 struct KQuant;
+
+template <>
+struct KQuant<kQ2K> {
+    static constexpr size_t kBytes = kQ2KBytes;
+    using Act = Q6KAct;
+    using Regs = Q2KRegs;
+    using Prep = Q2KPrep;
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *bs_blk, int q) {
+        return q6k_load_act(aq_blk, dx, bs_blk, q);
+    }
+    static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q2k_load_block(blk, q); }
+    static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q2k_prepare(r, q); }
+    static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q2k_dot(p, a); }
+};
+
+template <>
+struct KQuant<kQ3K> {
+    static constexpr size_t kBytes = kQ3KBytes;
+    using Act = Q6KAct;
+    using Regs = Q3KRegs;
+    using Prep = Q2KPrep;
+    static __device__ __forceinline__ Act load_act(const int8_t *aq_blk, float dx, const int16_t *bs_blk, int q) {
+        return q6k_load_act(aq_blk, dx, bs_blk, q);
+    }
+    static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q3k_load_block(blk, q); }
+    static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q3k_prepare(r, q); }
+    static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q3k_dot(p, a); }
+};
 
 template <>
 struct KQuant<kQ4K> {

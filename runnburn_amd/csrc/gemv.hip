@@ -1,5 +1,7 @@
 // Decode GEMV kernels: one packed GGUF row x one quantised activation vector -> one f32.
 //
+//  Q2_K x Q8_K : crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242   (dot_q2k_q8k_avx2)
+//  Q3_K x Q8_K : crates/rnb-cpu/src/gemm/avx2_dot.rs:247-375   (dot_q3k_q8k_avx2)
 //  Q4_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:884-916   (dot_q4_k_q8k_scalar)
 //  Q5_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 (dot_q5_k_q8k_scalar)
 //  Q6_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 (dot_q6_k_q8k_scalar)
@@ -26,7 +28,7 @@ constexpr int kWavesPerWg = 4;
 constexpr uint32_t kTargetWaves = 4096;  // total waves per launch: enough loads in flight, short tail
 
 // ---------------------------------------------------------------------------------------------
-// K-quant GEMV (Q4_K, Q5_K and Q6_K share the structure; only the block functions differ)
+// K-quant GEMV (Q2_K ... Q6_K share the structure; only the block functions differ)
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
@@ -311,6 +313,14 @@ void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
     launch_kquant_any<kQ5K>(w, act, out, rows, nb, seq, stream);
+}
+
+void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
+                         uint32_t seq, hipStream_t stream) {
+    if (quant == kQ2K)
+        launch_kquant_any<kQ2K>(w, act, out, rows, nb, seq, stream);
+    else
+        launch_kquant_any<kQ3K>(w, act, out, rows, nb, seq, stream);
 }
 
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,

@@ -8,8 +8,8 @@
 
 namespace rnb {
 
-constexpr uint32_t kQ8_0 = 8, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
-constexpr size_t kQ8_0Bytes = 34, kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210;
+constexpr uint32_t kQ8_0 = 8, kQ2K = 10, kQ3K = 11, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
+constexpr size_t kQ8_0Bytes = 34, kQ2KBytes = 84, kQ3KBytes = 110, kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210;
 
 // Device layout of quantised activations (structure of arrays, one set per call):
 //   Q8_K:  qs    int8  [seq][K]          (16-byte aligned rows, K % 256 == 0)
@@ -38,6 +38,9 @@ void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                      uint32_t seq, hipStream_t stream);
+// Q2_K / Q3_K rows (84 / 110-byte blocks at 4- / 2-byte alignment); quant is kQ2K or kQ3K
+void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
+                         uint32_t seq, hipStream_t stream);
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,
@@ -53,7 +56,7 @@ void launch_argmax(const float *values, uint32_t len, float *scratch_values, uin
 // out[i] = silu(gate[i]) * up[i]
 void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream);
 
-// Multi-token matmul on the vector ALUs for Q4_K / Q5_K / Q6_K (weights decoded once per eight staged tokens);
+// Multi-token matmul on the vector ALUs for Q2_K ... Q6_K (weights decoded once per eight staged tokens);
 // same output contract as launch_gemv_q4k
 void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);

@@ -428,7 +428,12 @@ void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *
 #define RNB_LAUNCH_MT(Q, R)                                                                                           \
     hipLaunchKernelGGL((matmul_tokens_kernel<Q, R>), grid, block, p.lds_bytes, stream, w, act.qs, act.d, act.bsums,   \
                        out, rows, nb, seq, p.iters, p.tmax, chunks_per_wg)
-    RNB_DISPATCH_KQUANT(quant, rpw, RNB_LAUNCH_MT);
+    if (quant == kQ2K)
+        RNB_DISPATCH_KQUANT_R(kQ2K, rpw, RNB_LAUNCH_MT);
+    else if (quant == kQ3K)
+        RNB_DISPATCH_KQUANT_R(kQ3K, rpw, RNB_LAUNCH_MT);
+    else
+        RNB_DISPATCH_KQUANT(quant, rpw, RNB_LAUNCH_MT);
 #undef RNB_LAUNCH_MT
 }
 

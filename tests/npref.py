@@ -8,6 +8,69 @@ def f16_bytes(v) -> bytes:
     return np.array([v], dtype=np.float16).tobytes()
 
 
+# ---- Q2_K ---------------------------------------------------------------------------
+
+def make_q2k_block(d, dmin, sc, mn, values) -> np.ndarray:
+    """values: 256 two-bit values in element order; sc, mn: sixteen 4-bit codes.  Layout {scales[16], qs[64], f16 d,
+    f16 dmin}: element 128h + 32p + l keeps its two bits at bit 2p of qs[32h + l]; its sub-block is (128h + 32p + l) / 16."""
+    v = np.asarray(values, dtype=np.uint8).reshape(2, 4, 32)  # half, bit pair, l
+    qs = np.zeros((2, 32), dtype=np.uint8)
+    for p in range(4):
+        qs |= (v[:, p, :] & 3) << (2 * p)
+    scales = (np.asarray(sc, dtype=np.uint8) & 15) | ((np.asarray(mn, dtype=np.uint8) & 15) << 4)
+    return np.concatenate([scales, qs.reshape(64), np.frombuffer(f16_bytes(d), dtype=np.uint8),
+                           np.frombuffer(f16_bytes(dmin), dtype=np.uint8)]).astype(np.uint8)
+
+
+def dequant_q2k_f64(blocks) -> np.ndarray:
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, 84)
+    sc = (b[:, 0:16] & 15).astype(np.float64)
+    mn = (b[:, 0:16] >> 4).astype(np.float64)
+    d = b[:, 80:82].copy().view(np.float16).astype(np.float64).reshape(-1, 1)
+    dmin = b[:, 82:84].copy().view(np.float16).astype(np.float64).reshape(-1, 1)
+    qs = b[:, 16:80].reshape(-1, 2, 1, 32).astype(np.int64)
+    val = ((qs >> (2 * np.arange(4)).reshape(1, 1, 4, 1)) & 3).reshape(-1, 256)  # half, pair, l == element order
+    return (np.repeat(sc * d, 16, axis=1) * val - np.repeat(mn * dmin, 16, axis=1)).reshape(-1)
+
+
+# ---- Q3_K ---------------------------------------------------------------------------
+
+def make_q3k_block(d, codes, values) -> np.ndarray:
+    """values: 256 signed values -4..3 in element order; codes: sixteen signed sub-block scales -32..31.  Layout
+    {hmask[32], qs[64], scales[12], f16 d}: the stored value v + 4 keeps its low two bits as for Q2_K and its third bit
+    in bit 4h + p of hmask[l]; the stored scale code + 32 keeps its low four bits in nibble k/8 of byte k%8 and its
+    high two in bit pair k/4 of byte 8 + k%4."""
+    u = (np.asarray(values, dtype=np.int64) + 4).astype(np.uint8).reshape(2, 4, 32)
+    qs = np.zeros((2, 32), dtype=np.uint8)
+    hm = np.zeros(32, dtype=np.uint8)
+    for h in range(2):
+        for p in range(4):
+            qs[h] |= (u[h, p] & 3) << (2 * p)
+            hm |= ((u[h, p] >> 2) & 1) << (4 * h + p)
+    st = (np.asarray(codes, dtype=np.int64) + 32).astype(np.uint8)
+    sb = np.zeros(12, dtype=np.uint8)
+    sb[0:8] = (st[0:8] & 15) | ((st[8:16] & 15) << 4)
+    for k in range(16):
+        sb[8 + k % 4] |= ((st[k] >> 4) & 3) << (2 * (k // 4))
+    return np.concatenate([hm, qs.reshape(64), sb, np.frombuffer(f16_bytes(d), dtype=np.uint8)]).astype(np.uint8)
+
+
+def dequant_q3k_f64(blocks) -> np.ndarray:
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, 110)
+    hm = b[:, 0:32].astype(np.int64)
+    qs = b[:, 32:96].reshape(-1, 2, 1, 32).astype(np.int64)
+    sb = b[:, 96:108].astype(np.int64)
+    d = b[:, 108:110].copy().view(np.float16).astype(np.float64).reshape(-1, 1)
+    low = (qs >> (2 * np.arange(4)).reshape(1, 1, 4, 1)) & 3                        # [n, half, pair, l]
+    bit = (hm[:, None, :] >> np.arange(8)[None, :, None]) & 1                        # [n, 4*half + pair, l]
+    val = (low + 4 * bit.reshape(-1, 2, 4, 32) - 4).reshape(-1, 256)
+    k = np.arange(16)
+    lo4 = np.where(k < 8, sb[:, k % 8] & 15, sb[:, k % 8] >> 4)
+    hi2 = (sb[:, 8 + k % 4] >> (2 * (k // 4))) & 3
+    code = (lo4 | (hi2 << 4)) - 32
+    return (np.repeat(code * d, 16, axis=1) * val).reshape(-1)
+
+
 # ---- Q4_K ---------------------------------------------------------------------------
 
 def pack_scales_k4(sc, mn) -> np.ndarray:

@@ -36,7 +36,8 @@ def test_trait_facade():
     assert caps == {"MatMul": True, "Attention": False, "Gdn": False, "MoE": True, "Sampler": False}
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q4_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q8_0)
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q5_K) and b.supports_quant(rnb.OP_MOE, rnb.GGML_Q5_K)
-    assert not b.supports_quant(rnb.OP_MATMUL, 10) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # Q2_K; Q8_0 down
+    assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q2_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q3_K)
+    assert not b.supports_quant(rnb.OP_MATMUL, 2) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # Q4_0; Q8_0 down
     with pytest.raises(rnb.BackendError) as ei:
         b.execute(object())
     assert ei.value.kind == "UnsupportedOp"
@@ -62,6 +63,15 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q4_K shape mismatch: input=256 output=1 expected input=256 output>=2"
     e = _err(rnb.q4k_gemv_batch, z(144, np.uint8), 1, 256, z(300, np.float32))
     assert str(e) == "Q4_K batch input length 300 is not divisible by cols 256"
+    # crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:73-181
+    e = _err(rnb.q2k_gemv, z(84, np.uint8), 1, 100, z(100, np.float32))
+    assert str(e) == "Q2_K cols must be divisible by 256, got 100"
+    e = _err(rnb.q2k_gemv, z(85, np.uint8), 1, 256, z(256, np.float32))
+    assert str(e) == "Q2_K weight byte mismatch: got 85, expected 84"
+    e = _err(rnb.q3k_gemv, z(110, np.uint8), 1, 256, z(255, np.float32))
+    assert str(e) == "Q3_K input length mismatch: got 255, expected 256"
+    e = _err(rnb.q3k_gemv_batch, z(110, np.uint8), 1, 256, z(300, np.float32))
+    assert str(e) == "Q3_K batch input length 300 is not divisible by cols 256"
     # crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:2207-2281, 3957-3993
     e = _err(rnb.q5k_gemv, z(176, np.uint8), 1, 100, z(100, np.float32))
     assert str(e) == "Q5_K cols must be divisible by 256, got 100"

@@ -10,7 +10,7 @@ from tests import npref
 
 pytestmark = pytest.mark.gpu
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 REL = 1e-3          # tolerance named by the task: max relative error 1e-3 per row
 TIGHT = 2e-5        # what f32 summation-order differences actually allow, relative to rms
 
@@ -27,7 +27,8 @@ def check_close(got, ref, gold=None, label=""):
 
 
 def gemv_fn(rnb, quant, batch=False):
-    table = {(Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q5_K, False): rnb.q5k_gemv,
+    table = {(Q2_K, False): rnb.q2k_gemv, (Q2_K, True): rnb.q2k_gemv_batch, (Q3_K, False): rnb.q3k_gemv,
+             (Q3_K, True): rnb.q3k_gemv_batch, (Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q5_K, False): rnb.q5k_gemv,
              (Q5_K, True): rnb.q5k_gemv_batch, (Q6_K, False): rnb.q6k_gemv, (Q6_K, True): rnb.q6k_gemv_batch,
              (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
     return table[(quant, batch)]
@@ -112,7 +113,7 @@ def test_reference_closed_forms_on_device(rnb):
 
 # ---- GEMV: shapes around every edge of the lane mapping ------------------------------------------
 
-@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("rows,nblk", [(1, 1), (3, 2), (4, 3), (5, 5), (7, 8), (9, 9), (64, 16), (33, 17), (6, 56),
                                        (5, 31), (130, 20), (9, 256), (2, 257)])
 def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
@@ -179,7 +180,7 @@ def test_unaligned_host_weights_and_subrange_residency(rnb, oracle):
     """Rows at odd host byte offsets must give identical results (crates/rnb-cpu/src/gemm/quant_gemv.rs:1257-1296);
     a sub-range of a resident parent resolves to parent + offset (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:722-741)."""
     rows, cols = 16, 1024
-    for quant in (Q4_K, Q5_K, Q6_K, Q8_0):
+    for quant in (Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0):
         w = oracle.make_weights(quant, rows, cols, 42 + quant)
         x = oracle.fill_normal(cols, 43, 1.0)
         base = gemv_fn(rnb, quant)(w, rows, cols, x)
@@ -243,7 +244,8 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
 
 @pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q4_K, 77, 2048), (Q4_K, 50, 768), (Q6_K, 300, 4096),
                                              (Q6_K, 64, 768), (Q8_0, 200, 4096), (Q8_0, 33, 1056), (Q6_K, 40, 14336),
-                                             (Q5_K, 300, 4096), (Q5_K, 41, 1280), (Q5_K, 24, 14336)])
+                                             (Q5_K, 300, 4096), (Q5_K, 41, 1280), (Q5_K, 24, 14336),
+                                             (Q2_K, 300, 4096), (Q2_K, 24, 14336), (Q3_K, 300, 4096), (Q3_K, 24, 14336)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
     feed several matrices from one activation) run the same arithmetic: identical bits."""
@@ -265,7 +267,7 @@ def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols
 
 # ---- batches: seq-major layout, ragged token counts ----------------------------------------------
 
-@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("seq", [2, 3, 4, 9, 15, 33])
 def test_gemv_batch_small(rnb, oracle, quant, seq):
     rows, cols = 37, 768
@@ -277,7 +279,7 @@ def test_gemv_batch_small(rnb, oracle, quant, seq):
                 f"batch quant {quant} seq {seq}")
 
 
-@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_gemv_batch_long_rows(rnb, oracle, quant):
     """Rows longer than 16 super-blocks: the K-split kernel with tokens on grid.y up to 3 tokens, the staged
     multi-token kernel from 4 tokens on."""
@@ -357,6 +359,30 @@ def test_q5k_gemv_full_size_14336x4096_and_4096x14336(rnb, oracle):
     """Q5_K at the up- and down-projection shapes of the Q4_K / Q6_K configurations."""
     _full_gemv(rnb, oracle, Q5_K, 14336, 4096, "q5k_up")
     _full_gemv(rnb, oracle, Q5_K, 4096, 14336, "q5k_down")
+
+
+def test_q2k_q3k_gemv_full_size_and_extremes(rnb, oracle):
+    """Q2_K and Q3_K at the 14336x4096 shape of the Q4_K configuration, then blocks at the ends of every field's range
+    (all-max and all-min values, scale codes -32 and 31, zero and subnormal f16 scales, a zero activation block)."""
+    _full_gemv(rnb, oracle, Q2_K, 14336, 4096, "q2k_up")
+    _full_gemv(rnb, oracle, Q3_K, 14336, 4096, "q3k_up")
+    rng = np.random.default_rng(27)
+    nblk, rows = 4, 8
+    x = oracle.fill_normal(nblk * 256, 28, 1.0)
+    x[512:768] = 0.0
+    b2, b3 = [], []
+    for r in range(rows):
+        for b in range(nblk):
+            d = [1.0, 0.0, 6e-8, 2.0 ** -14][(r + b) % 4]
+            b2.append(npref.make_q2k_block(d, [0.5, 6e-8, 0.0, 1.0][(r + b) % 4], np.full(16, 15), np.full(16, 15),
+                                           [np.full(256, 3), rng.integers(0, 4, 256), np.zeros(256)][(r + b) % 3]))
+            b3.append(npref.make_q3k_block([1.0, -0.5, 6e-8, 0.0][(r + b) % 4],
+                                           [np.full(16, -32), np.full(16, 31), rng.integers(-32, 32, 16)][(r + 2 * b) % 3],
+                                           [np.full(256, -4), np.full(256, 3), rng.integers(-4, 4, 256)][(r + b) % 3]))
+    for quant, blocks in ((Q2_K, b2), (Q3_K, b3)):
+        w = np.concatenate(blocks)
+        check_close(gemv_fn(rnb, quant)(w, rows, nblk * 256, x), oracle.gemv(quant, w, rows, nblk * 256, x)[0],
+                    oracle.gemv(quant, w, rows, nblk * 256, x, gold=True)[0], f"quant {quant} extremes")
 
 
 def test_q5k_fifth_bit_vectors_on_device(rnb):

@@ -9,7 +9,7 @@ import pytest
 
 from tests import npref
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 
 
 # ---- f16 ----------------------------------------------------------------------------
@@ -81,6 +81,16 @@ def _random_q4k(rng, n):
     return np.concatenate(blocks)
 
 
+def _random_q2k(rng, n):
+    return np.concatenate([npref.make_q2k_block(rng.uniform(1e-4, 5e-3), rng.uniform(1e-4, 5e-3), rng.integers(0, 16, 16),
+                                                rng.integers(0, 16, 16), rng.integers(0, 4, 256)) for _ in range(n)])
+
+
+def _random_q3k(rng, n):
+    return np.concatenate([npref.make_q3k_block(rng.uniform(-5e-3, 5e-3), rng.integers(-32, 32, 16),
+                                                rng.integers(-4, 4, 256)) for _ in range(n)])
+
+
 def _random_q5k(rng, n):
     blocks = []
     for _ in range(n):
@@ -118,6 +128,65 @@ def test_dequantize_q4k_places_each_nibble(oracle):
     got = oracle.dequantize(Q4_K, blocks).astype(np.float64)
     want = npref.dequant_q4k_f64(blocks)
     assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
+
+
+def test_dequantize_q2k_reference_vectors_and_placement(oracle):
+    """crates/rnb-cpu/src/quantize/dequant.rs:898-927: the zero block, and qs[1] = 3 with all scales 1, d = 1,
+    dmin = 0 -> out[1] = 3, out[4] = 0, out[33] = 0 (hand-built bytes); then every element one at a time."""
+    assert np.all(oracle.dequantize(Q2_K, np.zeros(84, np.uint8)) == 0.0)
+    blk = np.zeros(84, np.uint8)
+    blk[0:16] = 1
+    blk[16 + 1] = 3
+    blk[80:82] = np.frombuffer(npref.f16_bytes(1.0), np.uint8)
+    y = oracle.dequantize(Q2_K, blk)
+    assert y[1] == 3.0 and y[4] == 0.0 and y[33] == 0.0 and np.count_nonzero(y) == 1
+    for elem in (0, 15, 16, 31, 32, 47, 100, 127, 128, 200, 255):
+        v = np.zeros(256, np.uint8)
+        v[elem] = 2
+        y = oracle.dequantize(Q2_K, npref.make_q2k_block(1.0, 0.0, np.arange(16) % 15 + 1, np.zeros(16), v))
+        want = np.zeros(256, np.float32)
+        want[elem] = 2.0 * ((elem // 16) % 15 + 1)
+        assert np.array_equal(y, want), elem
+    # mins: values 0 -> every element of sub-block j is -dmin * mn[j]
+    y = oracle.dequantize(Q2_K, npref.make_q2k_block(0.0, 0.5, np.zeros(16), np.arange(16), np.zeros(256)))
+    assert np.array_equal(y, np.repeat(-0.5 * np.arange(16), 16).astype(np.float32))
+    rng = np.random.default_rng(41)
+    blocks = _random_q2k(rng, 64)
+    got = oracle.dequantize(Q2_K, blocks).astype(np.float64)
+    want = npref.dequant_q2k_f64(blocks)
+    assert np.allclose(got, want, rtol=0, atol=4e-7 * np.abs(want).max())
+
+
+def test_dequantize_q3k_zero_block_and_placement(oracle):
+    """crates/rnb-cpu/src/quantize/dequant.rs:1009-1019 (zero block); hand-built bytes for each field: with every
+    stored scale 33 (signed 1), d = 1, qs = hmask = 0 every value is -4; setting one hmask bit lifts one element to 0;
+    one 2-bit field adds its value."""
+    assert np.all(oracle.dequantize(Q3_K, np.zeros(110, np.uint8)) == 0.0)
+    base = np.zeros(110, np.uint8)
+    base[96:104] = 0x11       # low nibbles of all sixteen codes: 1
+    base[104:108] = 0xAA      # high two bits of all sixteen codes: 2 -> stored 33, signed 1
+    base[108:110] = np.frombuffer(npref.f16_bytes(1.0), np.uint8)
+    assert np.all(oracle.dequantize(Q3_K, base) == -4.0)
+    for l, bit in ((0, 0), (5, 3), (31, 7), (16, 4)):
+        blk = base.copy()
+        blk[l] = 1 << bit
+        want = np.full(256, -4.0, np.float32)
+        want[128 * (bit // 4) + 32 * (bit % 4) + l] = 0.0
+        assert np.array_equal(oracle.dequantize(Q3_K, blk), want), (l, bit)
+    blk = base.copy()
+    blk[32 + 32 + 7] = 0b10_01_11_00  # half 1, l = 7: pairs 0..3 hold 0, 3, 1, 2
+    want = np.full(256, -4.0, np.float32)
+    want[128 + 32 * np.arange(4) + 7] = np.array([0, 3, 1, 2], np.float32) - 4.0
+    assert np.array_equal(oracle.dequantize(Q3_K, blk), want)
+    # scales: each code on its own sub-block
+    codes = np.arange(-8, 8) * 4
+    y = oracle.dequantize(Q3_K, npref.make_q3k_block(0.5, codes, np.full(256, 3)))
+    assert np.array_equal(y, np.repeat(0.5 * codes * 3, 16).astype(np.float32))
+    rng = np.random.default_rng(42)
+    blocks = _random_q3k(rng, 64)
+    got = oracle.dequantize(Q3_K, blocks).astype(np.float64)
+    want = npref.dequant_q3k_f64(blocks)
+    assert np.allclose(got, want, rtol=0, atol=4e-7 * np.abs(want).max())
 
 
 def test_dequantize_q5k_zero_block(oracle):
@@ -309,6 +378,43 @@ def test_q4k_mins_use_32_wide_bsums(oracle):
     assert oracle.dot(Q4_K, blk, act, avx2=True) == -2.0 * summ
 
 
+# ---- Q2_K / Q3_K x Q8_K dots ------------------------------------------------------------
+
+def test_q2k_q3k_dot_known_vectors(oracle):
+    """Hand-built blocks for crates/rnb-cpu/src/gemm/avx2_dot.rs:169-375: all values 1, one non-zero sub-block scale ->
+    scale * (sum of that sub-block's 16 activations); mins against the 16-wide bsums; Q3_K's signed scales."""
+    q = (np.arange(256) % 11 - 5).astype(np.int8)
+    act = _act_from_parts(0.25, q)
+    for j in range(16):
+        sc = np.zeros(16, np.int64)
+        sc[j] = 7
+        blk = npref.make_q2k_block(2.0, 0.0, sc, np.zeros(16), np.ones(256))
+        assert oracle.dot(Q2_K, blk, act) == 0.25 * 2.0 * 7 * float(q[16 * j:16 * j + 16].astype(np.int64).sum()), j
+        codes = np.zeros(16, np.int64)
+        codes[j] = -9
+        blk3 = npref.make_q3k_block(2.0, codes, np.full(256, 3))
+        assert oracle.dot(Q3_K, blk3, act) == 0.25 * 2.0 * -9 * 3 * float(q[16 * j:16 * j + 16].astype(np.int64).sum()), j
+    blk = npref.make_q2k_block(0.0, 1.0, np.zeros(16), np.arange(16), np.zeros(256))
+    bs = (np.arange(16, dtype=np.int16) * 3 - 20).reshape(1, 16)
+    summ = int((np.arange(16) * bs[0].astype(np.int64)).sum())
+    assert oracle.dot(Q2_K, blk, _act_from_parts(2.0, np.zeros(256, np.int8), bsums=bs)) == -2.0 * summ
+
+
+@pytest.mark.parametrize("quant,maker,deq", [(Q2_K, _random_q2k, npref.dequant_q2k_f64),
+                                             (Q3_K, _random_q3k, npref.dequant_q3k_f64)])
+def test_q2k_q3k_dot_equals_f64_dequant_identity(oracle, quant, maker, deq):
+    rng = np.random.default_rng(43 + quant)
+    for nb in (1, 2, 7, 16):
+        row = maker(rng, nb)
+        x = rng.standard_normal(nb * 256).astype(np.float32)
+        act = oracle.quantize_q8k(x)
+        want = float(np.dot(deq(row), npref.deq_act_q8k_f64(act)))
+        gold = oracle.dot(quant, row, act, gold=True)
+        assert gold == pytest.approx(want, rel=1e-11, abs=1e-12)
+        scale = float(np.sum(np.abs(deq(row) * npref.deq_act_q8k_f64(act))))
+        assert abs(oracle.dot(quant, row, act) - want) <= 4e-7 * scale
+
+
 # ---- Q5_K x Q8_K dot ------------------------------------------------------------------
 
 def test_q5k_dot_fifth_bit_vectors(oracle):
@@ -426,7 +532,8 @@ def test_q8_0_q8_equals_f64_identity(oracle):
 
 # ---- drivers --------------------------------------------------------------------------
 
-@pytest.mark.parametrize("quant,maker", [(Q4_K, _random_q4k), (Q5_K, _random_q5k), (Q6_K, _random_q6k)])
+@pytest.mark.parametrize("quant,maker", [(Q2_K, _random_q2k), (Q3_K, _random_q3k), (Q4_K, _random_q4k),
+                                         (Q5_K, _random_q5k), (Q6_K, _random_q6k)])
 def test_gemv_driver_layout_and_row_independence(oracle, quant, maker):
     rng = np.random.default_rng(12)
     rows, nb, seq = 5, 2, 3
@@ -440,7 +547,7 @@ def test_gemv_driver_layout_and_row_independence(oracle, quant, maker):
             assert out[s, r] == np.float32(oracle.dot(quant, w[r * rb:(r + 1) * rb], act))
     gold = oracle.gemv(quant, w, rows, nb * 256, x, gold=True)
     assert np.allclose(out, gold, rtol=1e-4, atol=1e-6)
-    if quant != Q5_K:  # the vectorised baseline covers the benchmarked formats only
+    if quant in (Q4_K, Q6_K):  # the vectorised baseline covers the benchmarked formats only
         fast = oracle.gemv(quant, w, rows, nb * 256, x, avx2=True)
         assert np.allclose(fast, gold, rtol=1e-4, atol=1e-6)
     # 1 thread == many threads, bitwise (rows are independent)
@@ -550,6 +657,22 @@ def test_q5k_quantiser_roundtrip_property(oracle):
     assert np.sqrt(np.mean((xn - yn) ** 2)) / np.sqrt(np.mean(xn ** 2)) < 0.05
     d, dmin, sc, mn, val = npref.split_q5k(qn)
     assert sc.max() == 63 and val.max() == 31 and val.min() == 0
+
+
+def test_q2k_q3k_generators_roundtrip(oracle):
+    """crates/rnb-cpu/src/quantize/quant.rs (q2k round-trip test: cosine > 0.90 on its sine input); the Q3_K
+    generator is not the reference's.  Input generation only."""
+    t = np.arange(1024, dtype=np.float32) * np.float32(0.013)
+    x = (np.sin(t) * (1.0 + 0.2 * np.cos(t * np.float32(0.5)))).astype(np.float32)
+    y = oracle.dequantize(Q2_K, oracle.quantize_row(Q2_K, x))
+    assert float(np.dot(x, y) / (np.linalg.norm(x) * np.linalg.norm(y))) > 0.90
+    xn = oracle.fill_normal(256 * 40, 24, 0.02)
+    y2 = oracle.dequantize(Q2_K, oracle.quantize_row(Q2_K, xn))
+    y3 = oracle.dequantize(Q3_K, oracle.quantize_row(Q3_K, xn))
+    assert float(np.dot(xn, y2) / (np.linalg.norm(xn) * np.linalg.norm(y2))) > 0.90
+    assert np.sqrt(np.mean((xn - y3) ** 2)) / np.sqrt(np.mean(xn ** 2)) < 0.25
+    b3 = oracle.quantize_row(Q3_K, xn).reshape(-1, 110)
+    assert b3[:, 0:32].any() and b3[:, 32:96].any()  # both bit planes in use
 
 
 def test_q6k_q8_0_generators_roundtrip(oracle):
