@@ -7,8 +7,8 @@
  *
  * Semantics are those of the reference's rnb-cpu crate: activations are quantised on the
  * device to Q8_K (256-wide, crates/rnb-cpu/src/gemm/activation_q8.rs:149-173) for the K-quant
- * weights (Q2_K ... Q6_K) and to the 32-wide f32-scale Q8 block (:14-32) for Q8_0 weights; weight blocks are
- * consumed exactly as stored in GGUF (34 / 84 / 110 / 144 / 176 / 210 bytes, no repack, no requantisation).
+ * weights (Q2_K ... Q6_K) and to the 32-wide f32-scale Q8 block (:14-32) for the 32-element formats; weight blocks are
+ * consumed exactly as stored in GGUF (18 ... 34 / 84 / 110 / 144 / 176 / 210 bytes, no repack, no requantisation).
  *
  * Threading model (crates/rnb-backend/cuda/src/runtime.rs:9): one process-global state behind
  * a mutex, opened lazily on first use, one device, one stream.  Host-pointer entry points
@@ -36,6 +36,10 @@ typedef enum {
 } rnb_hip_status;
 
 /* ggml type ids, crates/rnb-loader/src/gguf/types.rs:5-41 */
+#define RNB_GGML_Q4_0 2u
+#define RNB_GGML_Q4_1 3u
+#define RNB_GGML_Q5_0 6u
+#define RNB_GGML_Q5_1 7u
 #define RNB_GGML_Q8_0 8u
 #define RNB_GGML_Q2_K 10u
 #define RNB_GGML_Q3_K 11u
@@ -56,7 +60,7 @@ typedef enum {
 int rnb_hip_backend_kind(void);
 /* capabilities(): 1 when `op` (RNB_OP_*) executes on this backend, else 0. */
 int rnb_hip_backend_supports(int op);
-/* 1 when (op, ggml quant id) is supported: MatMul x {Q8_0,Q2_K,Q3_K,Q4_K,Q5_K,Q6_K}; MoE x gate/up Q4_K with
+/* 1 when (op, ggml quant id) is supported: MatMul x {Q4_0,Q4_1,Q5_0,Q5_1,Q8_0,Q2_K..Q6_K}; MoE x gate/up Q4_K with
  * down Q4_K|Q5_K|Q6_K (pass the down quant). */
 int rnb_hip_backend_supports_quant(int op, uint32_t quant);
 
@@ -99,6 +103,25 @@ int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, c
  * out_len >= seq_len*rows.  seq_len >= 16 takes the int8-MFMA GEMM. */
 int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                            const float *x, size_t x_len, float *out, size_t out_len);
+/* q4_0_gemv, q4_1_gemv, q5_0_gemv, q5_1_gemv and their batch forms, quant_api.rs:374-496 (checks and texts of
+ * q5_basic_gemv(_batch), :1983-2075): 18 / 20 / 22 / 24-byte blocks of 32 x the 32-wide Q8 activation, the integer
+ * dots of crates/rnb-cpu/src/gemm/neon_dot.rs:83-214 and neon_quant.rs:88-158 */
+int rnb_hip_q4_0_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+int rnb_hip_q4_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_q4_1_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+int rnb_hip_q4_1_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_q5_0_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+int rnb_hip_q5_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_q5_1_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+int rnb_hip_q5_1_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
 /* q2k_gemv / q3k_gemv and their batch forms, quant_api.rs:73-181 (same three checks and texts): Q2_K (84-byte) and
  * Q3_K (110-byte) rows x Q8_K(x), the block dots of crates/rnb-cpu/src/gemm/avx2_dot.rs:169-375 */
 int rnb_hip_q2k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
@@ -161,7 +184,7 @@ int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols
  * rnb_q4k_gate_up_gemv_* in crates/rnb-backend/cuda/cuda/kernels/quant_gemv.cuh:700-1267).
  * rnb_hip_quantize_dev fills the library's activation scratch from x_dev [seq_len][cols];
  * rnb_hip_gemv_quantized_dev multiplies a weight matrix with whatever the scratch holds and must
- * be given the same quant family (Q8_0 -> 32-wide Q8, K-quants -> Q8_K), cols and seq_len. */
+ * be given the same quant family (32-element formats -> 32-wide Q8, K-quants -> Q8_K), cols and seq_len. */
 int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols);
 int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
                                size_t seq_len, float *out_dev);
@@ -186,8 +209,7 @@ int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t 
  * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337; validation order and texts from
  * crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765 (seq_len > 1 required, as there).
  * out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))): gate/up are Q4_K [n_ff][n_embd],
- * down is [n_embd][n_ff] in Q4_K (12), Q5_K (13), Q6_K (14) or Q8_0 (8); code 7 (Q5_1) is a valid
- * request that returns RNB_HIP_UNSUPPORTED_OP.  Intermediates never leave the device. */
+ * down is [n_embd][n_ff] in Q4_K (12), Q5_K (13), Q6_K (14), Q8_0 (8) or Q5_1 (7), the reference's five codes.  Intermediates never leave the device. */
 int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
                                      const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
                                      size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
@@ -209,7 +231,7 @@ typedef struct rnb_hip_gguf_tensor {
     const char *name;      /* owned by the rnb_hip_gguf */
     uint32_t n_dims;       /* 0..4 */
     uint64_t shape[4];     /* row-major (outermost first): the file stores innermost first, parser.rs:356-357 */
-    uint32_t ggml_type;    /* ggml type id: 8 = Q8_0, 10..14 = Q2_K..Q6_K, 0 = F32, ... */
+    uint32_t ggml_type;    /* ggml type id: 2/3/6/7/8 = Q4_0/Q4_1/Q5_0/Q5_1/Q8_0, 10..14 = Q2_K..Q6_K, 0 = F32, ... */
     uint64_t offset;       /* relative to the data section, as stored */
     uint64_t file_offset;  /* data_start + offset */
     uint64_t n_bytes;      /* elements / block elements * block bytes; 0 if the shape is not block-aligned */

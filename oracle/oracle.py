@@ -14,9 +14,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "librnb_oracle.so")
 
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)  # 32-element blocks with 4- or 5-bit codes, dotted against 32-wide Q8 activations
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14  # ggml type ids (crates/rnb-loader/src/gguf/types.rs:5-41)
-BLOCK_BYTES = {Q8_0: 34, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210}
-BLOCK_ELEMS = {Q8_0: 32, Q2_K: 256, Q3_K: 256, Q4_K: 256, Q5_K: 256, Q6_K: 256}
+BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210}
+BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q2_K: 256, Q3_K: 256, Q4_K: 256, Q5_K: 256, Q6_K: 256}
 
 Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
 Q8_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (32,))])
@@ -78,6 +80,14 @@ def lib() -> C.CDLL:
                      "rnbo_quantize_row_q6_k", "rnbo_quantize_row_q8_0"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, sz, vp]
+        L.rnbo_dequantize_legacy.restype = i32
+        L.rnbo_dequantize_legacy.argtypes = [u32, vp, sz, vp]
+        L.rnbo_dot_legacy_q8.restype = f32
+        L.rnbo_dot_legacy_q8.argtypes = [u32, vp, vp, sz]
+        L.rnbo_dot_legacy_q8_f64.restype = C.c_double
+        L.rnbo_dot_legacy_q8_f64.argtypes = [u32, vp, vp, sz]
+        L.rnbo_quantize_row_legacy.restype = i32
+        L.rnbo_quantize_row_legacy.argtypes = [u32, vp, sz, vp]
         L.rnbo_fill_normal.restype = None
         L.rnbo_fill_normal.argtypes = [vp, sz, u64, f32]
         L.rnbo_make_weights.restype = i32
@@ -131,6 +141,9 @@ def dequantize(quant: int, blocks) -> np.ndarray:
     n = b.size // BLOCK_BYTES[quant]
     assert n * BLOCK_BYTES[quant] == b.size
     out = np.empty(n * BLOCK_ELEMS[quant], dtype=np.float32)
+    if quant in LEGACY:
+        assert lib().rnbo_dequantize_legacy(quant, _p(b), n, _p(out)) == 0
+        return out
     fn = {Q8_0: "rnbo_dequantize_q8_0", Q2_K: "rnbo_dequantize_q2_k", Q3_K: "rnbo_dequantize_q3_k",
           Q4_K: "rnbo_dequantize_q4_k", Q5_K: "rnbo_dequantize_q5_k", Q6_K: "rnbo_dequantize_q6_k"}[quant]
     getattr(lib(), fn)(_p(b), n, _p(out))
@@ -161,6 +174,11 @@ def dot(quant: int, row, act: np.ndarray, gold: bool = False, avx2: bool = False
     r = _u8(row)
     nb = r.size // BLOCK_BYTES[quant]
     assert act.size == nb
+    if quant in LEGACY:
+        assert not avx2
+        act = np.ascontiguousarray(act)
+        fn = lib().rnbo_dot_legacy_q8_f64 if gold else lib().rnbo_dot_legacy_q8
+        return float(fn(quant, _p(r), _p(act), nb))
     base = {Q8_0: "rnbo_dot_q8_0_q8", Q2_K: "rnbo_dot_q2k_q8k", Q3_K: "rnbo_dot_q3k_q8k", Q4_K: "rnbo_dot_q4k_q8k",
             Q5_K: "rnbo_dot_q5k_q8k", Q6_K: "rnbo_dot_q6k_q8k"}[quant]
     if gold:
@@ -253,6 +271,9 @@ def quantize_row(quant: int, x) -> np.ndarray:
     x = _f32(x).ravel()
     assert x.size % BLOCK_ELEMS[quant] == 0
     out = np.zeros(x.size // BLOCK_ELEMS[quant] * BLOCK_BYTES[quant], dtype=np.uint8)
+    if quant in LEGACY:
+        assert lib().rnbo_quantize_row_legacy(quant, _p(x), x.size, _p(out)) == 0
+        return out
     fn = {Q8_0: "rnbo_quantize_row_q8_0", Q2_K: "rnbo_quantize_row_q2_k", Q3_K: "rnbo_quantize_row_q3_k",
           Q4_K: "rnbo_quantize_row_q4_k", Q5_K: "rnbo_quantize_row_q5_k", Q6_K: "rnbo_quantize_row_q6_k"}[quant]
     getattr(lib(), fn)(_p(x), x.size, _p(out))

@@ -17,6 +17,9 @@
  *   quantize_q8                 closed-form cases + numpy restatement (formula is 6 lines)
  *   dot_q4k_q8k                 reference closed forms 0 / 0 / 2560.0 (tile_q4k.rs:2019-2151),
  *                               f64 numpy dequant(W) . dequant(Q8K(x)) identity
+ *   dequantize_q4_0 .. _q5_1    one-hot placement of every nibble and high bit + independent numpy statements
+ *   dot_q4_0/_q4_1/_q5_0/_q5_1  hand-built vectors (offset 8 / 16, min term against the activation sum, high bits),
+ *   (x Q8)                      f64 numpy dequant identity
  *   dequantize_q2_k/_q3_k       the reference's own vectors (dequant.rs:898-927, 1009-1019: zero blocks, qs[1] = 3 ->
  *                               out[1] = 3) + one-hot placement of every field + independent numpy statements
  *   dot_q2k_q8k, dot_q3k_q8k    hand-built vectors per sub-block scale / min / high bit, f64 numpy dequant
@@ -40,6 +43,7 @@
  *   quantize_row_q2_k           restates quant.rs:44-160; byte parity UNPINNED (cannot run the original), the
  *                               reference's round-trip bound (cosine >= 0.90) is checked.  Input generation only.
  *   quantize_row_q3_k           not in the reference (plain symmetric fit).  Input generation only.
+ *   quantize_row_q4_0 .. _q5_1  not in the reference (ggml reference semantics).  Input generation only.
  *   quantize_row_q6_k/_q8_0     not in the reference at all (ggml reference semantics); round
  *                               trip through the pinned dequantisers.  Input generation only.
  */
@@ -152,6 +156,49 @@ void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out) {
         float d = rd_f16(blk);
         for (int i = 0; i < 32; i++) out[b * 32 + i] = (float)(int8_t)blk[2 + i] * d;
     }
+}
+
+/* The 32-element formats with 4- or 5-bit codes: crates/rnb-cpu/src/quantize/dequant.rs:7-53.
+ *   Q4_0 {f16 d, qs[16]}                 (code - 8) * d        Q4_1 {f16 d, f16 m, qs[16]}          code * d + m
+ *   Q5_0 {f16 d, qh[4], qs[16]}          (code - 16) * d       Q5_1 {f16 d, f16 m, qh[4], qs[16]}   code * d + m
+ * Element i < 16 is the low nibble of qs[i], element 16 + i the high nibble; the fifth bit of element e is bit e of
+ * the little-endian 32-bit qh. */
+typedef struct {
+    int bytes, qs_off, qh_off, has_min, offset; /* qh_off < 0: no fifth bit */
+} legacy_fmt;
+
+static int legacy_format(uint32_t quant, legacy_fmt *f) {
+    switch (quant) {
+    case 2: *f = (legacy_fmt){RNBO_Q4_0_BLOCK_BYTES, 2, -1, 0, 8}; return 1;
+    case 3: *f = (legacy_fmt){RNBO_Q4_1_BLOCK_BYTES, 4, -1, 1, 0}; return 1;
+    case 6: *f = (legacy_fmt){RNBO_Q5_0_BLOCK_BYTES, 6, 2, 0, 16}; return 1;
+    case 7: *f = (legacy_fmt){RNBO_Q5_1_BLOCK_BYTES, 8, 4, 1, 0}; return 1;
+    default: return 0;
+    }
+}
+
+static inline int legacy_code(const legacy_fmt *f, const uint8_t *blk, int e) {
+    int nib = e < 16 ? (blk[f->qs_off + e] & 0x0f) : (blk[f->qs_off + e - 16] >> 4);
+    if (f->qh_off >= 0) {
+        uint32_t qh = (uint32_t)blk[f->qh_off] | ((uint32_t)blk[f->qh_off + 1] << 8) |
+                      ((uint32_t)blk[f->qh_off + 2] << 16) | ((uint32_t)blk[f->qh_off + 3] << 24);
+        nib |= (int)((qh >> e) & 1u) << 4;
+    }
+    return nib;
+}
+
+int rnbo_dequantize_legacy(uint32_t quant, const uint8_t *blocks, size_t n_blocks, float *out) {
+    legacy_fmt f;
+    if (!legacy_format(quant, &f)) return 1;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * (size_t)f.bytes;
+        float d = rd_f16(blk), m = f.has_min ? rd_f16(blk + 2) : 0.0f;
+        for (int e = 0; e < 32; e++) {
+            int code = legacy_code(&f, blk, e);
+            out[b * 32 + e] = f.has_min ? (float)code * d + m : ((float)code - (float)f.offset) * d;
+        }
+    }
+    return 0;
 }
 
 /* crates/rnb-cpu/src/quantize/dequant.rs:66-86.  Block = {u8 scales[16] (scale | min << 4), u8 qs[64], f16 d,
@@ -625,6 +672,58 @@ double rnbo_dot_q8_0_q8_f64(const uint8_t *row, const rnbo_q8_block *act, size_t
     return acc;
 }
 
+/* Q4_0 / Q5_0 x Q8: crates/rnb-cpu/src/gemm/neon_dot.rs:83-137, 163-214: acc += (f32)sum((code - offset) * q) *
+ * (d * d_x).  Q4_1 / Q5_1 x Q8: crates/rnb-cpu/src/gemm/neon_quant.rs:88-158: acc += d_x * (d * (f32)sum(code * q) +
+ * m * (f32)sum(q)).  Integer sums exact; the two-accumulator NEON forms differ by f32 add order only. */
+static inline void legacy_block_ints(const legacy_fmt *f, const uint8_t *blk, const rnbo_q8_block *a, int32_t *dot,
+                                     int32_t *sum) {
+    int32_t p = 0, sq = 0;
+    for (int e = 0; e < 32; e++) {
+        p += (int32_t)(legacy_code(f, blk, e) - f->offset) * (int32_t)a->qs[e];
+        sq += (int32_t)a->qs[e];
+    }
+    *dot = p;
+    *sum = sq;
+}
+
+float rnbo_dot_legacy_q8(uint32_t quant, const uint8_t *row, const rnbo_q8_block *act, size_t nb) {
+    legacy_fmt f;
+    if (!legacy_format(quant, &f)) return NAN;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * (size_t)f.bytes;
+        int32_t p, sq;
+        legacy_block_ints(&f, blk, &act[b], &p, &sq);
+        float d = rd_f16(blk);
+        if (f.has_min) {
+            volatile float t0 = d * (float)p;
+            volatile float t1 = rd_f16(blk + 2) * (float)sq;
+            volatile float t2 = t0 + t1;
+            volatile float t3 = act[b].d * t2;
+            acc += t3;
+        } else {
+            volatile float sc = d * act[b].d;
+            volatile float t = (float)p * sc;
+            acc += t;
+        }
+    }
+    return acc;
+}
+
+double rnbo_dot_legacy_q8_f64(uint32_t quant, const uint8_t *row, const rnbo_q8_block *act, size_t nb) {
+    legacy_fmt f;
+    if (!legacy_format(quant, &f)) return NAN;
+    double acc = 0.0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * (size_t)f.bytes;
+        int32_t p, sq;
+        legacy_block_ints(&f, blk, &act[b], &p, &sq);
+        double m = f.has_min ? (double)rd_f16(blk + 2) : 0.0;
+        acc += (double)act[b].d * ((double)rd_f16(blk) * (double)p + m * (double)sq);
+    }
+    return acc;
+}
+
 /* crates/rnb-cpu/src/gemm/quant_gemv.rs:127-141 (dot_q8_0_row): f32 activations */
 float rnbo_dot_q8_0_f32(const uint8_t *row, const float *x, size_t nb) {
     float acc = 0.0f;
@@ -649,6 +748,10 @@ float rnbo_dot_q8_0_f32(const uint8_t *row, const float *x, size_t nb) {
 
 static size_t block_bytes_of(uint32_t quant, size_t *elems) {
     switch (quant) {
+    case 2: *elems = 32; return RNBO_Q4_0_BLOCK_BYTES;
+    case 3: *elems = 32; return RNBO_Q4_1_BLOCK_BYTES;
+    case 6: *elems = 32; return RNBO_Q5_0_BLOCK_BYTES;
+    case 7: *elems = 32; return RNBO_Q5_1_BLOCK_BYTES;
     case 8: *elems = 32; return RNBO_Q8_0_BLOCK_BYTES;
     case 10: *elems = 256; return RNBO_Q2_K_BLOCK_BYTES;
     case 11: *elems = 256; return RNBO_Q3_K_BLOCK_BYTES;
@@ -695,14 +798,15 @@ int rnbo_gemv(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const 
     if (bb == 0 || cols % elems != 0) return 1;
     size_t nb = cols / elems, row_bytes = nb * bb;
     n_threads = resolve_threads(n_threads);
-    if (quant == 8) {
+    if (elems == 32) {
         rnbo_q8_block *act = (rnbo_q8_block *)malloc(sizeof(rnbo_q8_block) * nb * seq_len);
         if (!act) return 2;
         for (size_t s = 0; s < seq_len; s++) rnbo_quantize_q8(x + s * cols, cols, act + s * nb);
 #pragma omp parallel for schedule(static) num_threads(n_threads)
         for (long r = 0; r < (long)rows; r++)
             for (size_t s = 0; s < seq_len; s++)
-                out[s * rows + r] = rnbo_dot_q8_0_q8(w + r * row_bytes, act + s * nb, nb);
+                out[s * rows + r] = quant == 8 ? rnbo_dot_q8_0_q8(w + r * row_bytes, act + s * nb, nb)
+                                               : rnbo_dot_legacy_q8(quant, w + r * row_bytes, act + s * nb, nb);
         free(act);
         return 0;
     }
@@ -724,14 +828,15 @@ int rnbo_gemv_f64(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, co
     if (bb == 0 || cols % elems != 0) return 1;
     size_t nb = cols / elems, row_bytes = nb * bb;
     n_threads = resolve_threads(n_threads);
-    if (quant == 8) {
+    if (elems == 32) {
         rnbo_q8_block *act = (rnbo_q8_block *)malloc(sizeof(rnbo_q8_block) * nb * seq_len);
         if (!act) return 2;
         for (size_t s = 0; s < seq_len; s++) rnbo_quantize_q8(x + s * cols, cols, act + s * nb);
 #pragma omp parallel for schedule(static) num_threads(n_threads)
         for (long r = 0; r < (long)rows; r++)
             for (size_t s = 0; s < seq_len; s++)
-                out[s * rows + r] = rnbo_dot_q8_0_q8_f64(w + r * row_bytes, act + s * nb, nb);
+                out[s * rows + r] = quant == 8 ? rnbo_dot_q8_0_q8_f64(w + r * row_bytes, act + s * nb, nb)
+                                               : rnbo_dot_legacy_q8_f64(quant, w + r * row_bytes, act + s * nb, nb);
         free(act);
         return 0;
     }
@@ -1264,6 +1369,56 @@ void rnbo_quantize_row_q6_k(const float *input, size_t n, uint8_t *output) {
     }
 }
 
+/* Generators for the 4- and 5-bit 32-element formats: ggml reference semantics (quantize_row_q4_0_ref and
+ * siblings: d = signed max / -2^(bits-1) for the _0 formats, (max - min) / (2^bits - 1) with m = min for the _1
+ * formats); the reference repository has none.  Input generation only. */
+int rnbo_quantize_row_legacy(uint32_t quant, const float *input, size_t n, uint8_t *output) {
+    legacy_fmt f;
+    if (!legacy_format(quant, &f)) return 1;
+    const int top = f.qh_off >= 0 ? 31 : 15;
+    for (size_t b = 0; b < n / 32; b++) {
+        const float *x = input + b * 32;
+        uint8_t *out = output + b * (size_t)f.bytes;
+        memset(out, 0, (size_t)f.bytes);
+        float d, base;
+        if (f.has_min) {
+            float lo = x[0], hi = x[0];
+            for (int i = 1; i < 32; i++) {
+                if (x[i] < lo) lo = x[i];
+                if (x[i] > hi) hi = x[i];
+            }
+            d = (hi - lo) / (float)top;
+            base = lo;
+            wr_f16(out + 2, lo);
+        } else {
+            float amax = 0.0f, vmax = 0.0f;
+            for (int i = 0; i < 32; i++)
+                if (fabsf(x[i]) > amax) {
+                    amax = fabsf(x[i]);
+                    vmax = x[i];
+                }
+            d = vmax / -(float)f.offset;
+            base = 0.0f;
+        }
+        wr_f16(out, d);
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        uint32_t qh = 0;
+        for (int e = 0; e < 32; e++) {
+            float v = f.has_min ? (x[e] - base) * id + 0.5f : x[e] * id + (float)f.offset + 0.5f;
+            int code = (int)v;
+            code = code < 0 ? 0 : (code > top ? top : code);
+            if (e < 16)
+                out[f.qs_off + e] |= (uint8_t)(code & 0x0f);
+            else
+                out[f.qs_off + e - 16] |= (uint8_t)((code & 0x0f) << 4);
+            qh |= (uint32_t)((code >> 4) & 1) << e;
+        }
+        if (f.qh_off >= 0)
+            for (int k = 0; k < 4; k++) out[f.qh_off + k] = (uint8_t)(qh >> (8 * k));
+    }
+    return 0;
+}
+
 /* Q8_0 weight generator: ggml reference semantics (quantize_row_q8_0_ref); the reference
  * repository has no Q8_0 weight quantiser. */
 void rnbo_quantize_row_q8_0(const float *input, size_t n, uint8_t *output) {
@@ -1319,7 +1474,9 @@ int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, f
         for (long r = 0; r < (long)rows; r++) {
             for (size_t c = 0; c < cols; c++) row[c] = normal_at(seed, (uint64_t)r * cols + c, sigma);
             uint8_t *dst = out + (size_t)r * row_bytes;
-            if (quant == 10)
+            if (quant == 2 || quant == 3 || quant == 6 || quant == 7)
+                rnbo_quantize_row_legacy(quant, row, cols, dst);
+            else if (quant == 10)
                 rnbo_quantize_row_q2_k(row, cols, dst);
             else if (quant == 11)
                 rnbo_quantize_row_q3_k(row, cols, dst);

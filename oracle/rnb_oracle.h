@@ -25,6 +25,10 @@ extern "C" {
 
 #define RNBO_QK_K 256
 #define RNBO_Q8_0_BLOCK_BYTES 34
+#define RNBO_Q4_0_BLOCK_BYTES 18
+#define RNBO_Q4_1_BLOCK_BYTES 20
+#define RNBO_Q5_0_BLOCK_BYTES 22
+#define RNBO_Q5_1_BLOCK_BYTES 24
 #define RNBO_Q2_K_BLOCK_BYTES 84
 #define RNBO_Q3_K_BLOCK_BYTES 110
 #define RNBO_Q4_K_BLOCK_BYTES 144
@@ -52,6 +56,8 @@ int rnbo_nearest_int(float fval);
 
 /* ---- dequantisers (element order of the formats) -------------------------------- */
 void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out);
+/* quant: 2 = Q4_0, 3 = Q4_1, 6 = Q5_0, 7 = Q5_1 (32-element blocks); non-zero return: unknown id */
+int rnbo_dequantize_legacy(uint32_t quant, const uint8_t *blocks, size_t n_blocks, float *out);
 void rnbo_dequantize_q2_k(const uint8_t *blocks, size_t n_blocks, float *out);
 void rnbo_dequantize_q3_k(const uint8_t *blocks, size_t n_blocks, float *out);
 void rnbo_dequantize_q4_k(const uint8_t *blocks, size_t n_blocks, float *out);
@@ -63,6 +69,8 @@ void rnbo_quantize_q8k(const float *x, size_t n, rnbo_q8k_block *out);
 void rnbo_quantize_q8(const float *x, size_t n, rnbo_q8_block *out);
 
 /* ---- row dots ------------------------------------------------------------------- */
+float rnbo_dot_legacy_q8(uint32_t quant, const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
+double rnbo_dot_legacy_q8_f64(uint32_t quant, const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
 float rnbo_dot_q2k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 float rnbo_dot_q3k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 float rnbo_dot_q4k_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
@@ -79,7 +87,7 @@ double rnbo_dot_q6k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_
 double rnbo_dot_q8_0_q8_f64(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
 
 /* ---- GEMV / GEMM drivers: out[s*rows + row], x is [seq_len][cols] --------------- */
-/* quant: 8 = Q8_0 (Q8 x Q8_0 integer form), 10 = Q2_K, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K (ggml type ids).  */
+/* quant: 2 = Q4_0, 3 = Q4_1, 6 = Q5_0, 7 = Q5_1, 8 = Q8_0 (all against 32-wide Q8 activations), 10 = Q2_K, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K (ggml type ids).  */
 int rnbo_gemv(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
               size_t seq_len, float *out, int n_threads);
 int rnbo_gemv_f64(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
@@ -100,6 +108,7 @@ int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_
                                      const float *x, float *out, int n_threads);
 
 /* ---- input generation (not on the GPU path) ------------------------------------- */
+int rnbo_quantize_row_legacy(uint32_t quant, const float *x, size_t n, uint8_t *out);
 void rnbo_quantize_row_q2_k(const float *x, size_t n, uint8_t *out);
 void rnbo_quantize_row_q3_k(const float *x, size_t n, uint8_t *out);
 void rnbo_quantize_row_q4_k(const float *x, size_t n, uint8_t *out);

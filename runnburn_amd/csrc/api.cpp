@@ -22,6 +22,10 @@ struct QuantInfo {
 
 bool quant_info(uint32_t quant, QuantInfo *qi) {
     switch (quant) {
+    case kQ4_0: *qi = {"Q4_0", 32, kQ4_0Bytes}; return true;
+    case kQ4_1: *qi = {"Q4_1", 32, kQ4_1Bytes}; return true;
+    case kQ5_0: *qi = {"Q5_0", 32, kQ5_0Bytes}; return true;
+    case kQ5_1: *qi = {"Q5_1", 32, kQ5_1Bytes}; return true;
     case kQ8_0: *qi = {"Q8_0", 32, kQ8_0Bytes}; return true;
     case kQ2K: *qi = {"Q2_K", 256, kQ2KBytes}; return true;
     case kQ3K: *qi = {"Q3_K", 256, kQ3KBytes}; return true;
@@ -30,6 +34,11 @@ bool quant_info(uint32_t quant, QuantInfo *qi) {
     case kQ6K: *qi = {"Q6_K", 256, kQ6KBytes}; return true;
     default: return false;
     }
+}
+
+// the 32-element formats take 32-wide Q8 activations, the K-quants 256-wide Q8_K
+bool is_block32(uint32_t quant) {
+    return quant == kQ8_0 || quant == kQ4_0 || quant == kQ4_1 || quant == kQ5_0 || quant == kQ5_1;
 }
 
 int fail(int status, const std::string &msg) {
@@ -56,7 +65,7 @@ constexpr size_t kTokensMinSeq = 4;
 int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view) {
     const size_t n = seq * cols;
     HIP_TRY(s.act_qs.reserve(n));
-    if (quant == kQ8_0) {
+    if (is_block32(quant)) {
         HIP_TRY(s.act_d.reserve(n / 32 * sizeof(float)));
         launch_quantize_q8(x_dev, n / 32, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.stream);
         *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), nullptr};
@@ -71,7 +80,7 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
         *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(), digits};
     }
     HIP_TRY(hipGetLastError());
-    s.act_family = quant == kQ8_0 ? kQ8_0 : kQ4K;
+    s.act_family = is_block32(quant) ? kQ8_0 : kQ4K;
     s.act_seq = seq;
     s.act_cols = cols;
     return RNB_HIP_OK;
@@ -90,8 +99,9 @@ int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, 
 
 int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
                              float *out_dev) {
-    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), quant == kQ8_0 ? nullptr : s.act_bsums.as<int16_t>(),
-                      quant != kQ8_0 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
+    const bool b32 = is_block32(quant);
+    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), b32 ? nullptr : s.act_bsums.as<int16_t>(),
+                      !b32 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     const uint32_t nb = static_cast<uint32_t>(cols / 256);
     if (quant == kQ4K) {
@@ -118,7 +128,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else {
-        launch_gemv_q8_0(w_dev, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
+        launch_gemv_block32(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     }
     HIP_TRY(hipGetLastError());
     return RNB_HIP_OK;
@@ -196,7 +206,7 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
 
 // ---- dense SwiGLU FFN -------------------------------------------------------------------------
 // out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), the composition the reference runs per token
-// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K or Q8_0.
+// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K, Q8_0 or Q5_1.
 
 // Validation order and messages: crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765.
 int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd,
@@ -232,9 +242,6 @@ int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t
     if (down_len != n_embd * down_row_bytes)
         return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch down byte mismatch: got " + std::to_string(down_len) +
                                                  ", expected " + std::to_string(n_embd * down_row_bytes));
-    if (down_quant == 7)  // Q5_1 rows are a valid request that this backend does not run
-        return fail(RNB_HIP_UNSUPPORTED_OP,
-                    "dense SiLU FFN down quant code " + std::to_string(down_quant) + " is not built in the HIP backend");
     if (n_ff > 0x7fffffffu || n_embd > 0x7fffffffu || seq > 65535u)
         return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN shape out of range");
     return RNB_HIP_OK;
@@ -458,7 +465,7 @@ int rnb_hip_backend_kind(void) { return 6; }
 int rnb_hip_backend_supports(int op) { return (op == RNB_OP_MATMUL || op == RNB_OP_MOE) ? 1 : 0; }
 
 int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
-    if (op == RNB_OP_MATMUL) return (quant == kQ8_0 || (quant >= kQ2K && quant <= kQ6K)) ? 1 : 0;
+    if (op == RNB_OP_MATMUL) return (is_block32(quant) || (quant >= kQ2K && quant <= kQ6K)) ? 1 : 0;
     if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
     return 0;
 }
@@ -603,6 +610,21 @@ int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t c
                            float *out, size_t out_len) {
     return matmul_host(kQ4K, w, w_len, rows, cols, x, x_len, out, out_len, true);
 }
+#define RNB_BLOCK32_ENTRY(name, quant)                                                                                \
+    int rnb_hip_##name##_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,  \
+                              float *out, size_t out_len) {                                                            \
+        return matmul_host(quant, w, w_len, rows, cols, x, x_len, out, out_len, false);                                \
+    }                                                                                                                  \
+    int rnb_hip_##name##_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,          \
+                                    size_t x_len, float *out, size_t out_len) {                                        \
+        return matmul_host(quant, w, w_len, rows, cols, x, x_len, out, out_len, true);                                 \
+    }
+RNB_BLOCK32_ENTRY(q4_0, kQ4_0)
+RNB_BLOCK32_ENTRY(q4_1, kQ4_1)
+RNB_BLOCK32_ENTRY(q5_0, kQ5_0)
+RNB_BLOCK32_ENTRY(q5_1, kQ5_1)
+#undef RNB_BLOCK32_ENTRY
+
 int rnb_hip_q2k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                      float *out, size_t out_len) {
     return matmul_host(kQ2K, w, w_len, rows, cols, x, x_len, out, out_len, false);
@@ -870,7 +892,7 @@ int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, s
     Guard g;
     if (!g.state) return g.status;
     State &s = *g.state;
-    const uint32_t family = quant == kQ8_0 ? kQ8_0 : kQ4K;
+    const uint32_t family = is_block32(quant) ? kQ8_0 : kQ4K;
     if (s.act_family != family || s.act_seq != seq_len || s.act_cols != cols)
         return fail(RNB_HIP_INVALID_REQUEST,
                     std::string(qi.label) + " activation scratch holds seq_len=" + std::to_string(s.act_seq) + " cols=" +

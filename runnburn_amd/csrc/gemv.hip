@@ -5,7 +5,7 @@
 //  Q4_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:884-916   (dot_q4_k_q8k_scalar)
 //  Q5_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 (dot_q5_k_q8k_scalar)
 //  Q6_K x Q8_K : crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 (dot_q6_k_q8k_scalar)
-//  Q8_0 x Q8   : crates/rnb-cpu/src/gemm/neon_dot.rs:376-436   (dot_q8_0_q8_neon)
+//  Q8_0 x Q8   : crates/rnb-cpu/src/gemm/neon_dot.rs:376-436   (dot_q8_0_q8_neon); Q4_0, Q4_1, Q5_0, Q5_1 x Q8 below
 //  driver      : crates/rnb-cpu/src/gemm/quant_gemv.rs:403-536, out[s*rows + row]
 //
 // These kernels are HBM-bound: every weight byte is fetched once with 16-byte loads.  Four lanes own
@@ -236,57 +236,136 @@ void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Q8_0: block = {f16 d, i8 qs[32]}, 34 bytes, 2-byte aligned.  One lane per block: two 16-byte loads
-// at 2-byte alignment.  Rows of up to 128 blocks (K <= 4096) keep the lane's two activation blocks
-// in registers across rows.
+// The 32-element formats against 32-wide Q8 activations, one lane per block (blocks are 2-byte aligned: 16-byte loads
+// at 2-byte alignment).  Rows of up to 128 blocks (K <= 4096) keep the lane's two activation blocks in registers.
+//   Q8_0 {f16 d, i8 qs[32]}                 (d * d_x) * sum(w * q)                   neon_dot.rs:376-436
+//   Q4_0 {f16 d, qs[16]}                    (d * d_x) * sum((code - 8) * q)          neon_dot.rs:83-137
+//   Q5_0 {f16 d, u32 qh, qs[16]}            (d * d_x) * sum((code - 16) * q)         neon_dot.rs:163-214
+//   Q4_1 {f16 d, f16 m, qs[16]}             d_x * (d * sum(code * q) + m * sum(q))   neon_quant.rs:88-108
+//   Q5_1 {f16 d, f16 m, u32 qh, qs[16]}     likewise                                 neon_quant.rs:130-158
+// (all under crates/rnb-cpu/src/gemm/).  Element i < 16 is the low nibble of qs[i], element 16 + i the high nibble; the
+// fifth bit of element e is bit e of qh.  (code - offset) is applied as dot(code, q) - offset * sum(q).
 // ---------------------------------------------------------------------------------------------
 struct Q8Act {
     uint4 a0, a1;
     float dx;
+    int sum;  // of the 32 activations (unused by Q8_0)
 };
 
+template <bool kWithSum>
 __device__ __forceinline__ Q8Act q8_load_act(const int8_t *__restrict__ aq_blk, float dx) {
     Q8Act a;
     a.a0 = *reinterpret_cast<const uint4 *>(aq_blk);
     a.a1 = *reinterpret_cast<const uint4 *>(aq_blk + 16);
     a.dx = dx;
+    a.sum = 0;
+    if constexpr (kWithSum) {
+        int s = 0;
+        s = dot4(0x01010101u, a.a0.x, s);
+        s = dot4(0x01010101u, a.a0.y, s);
+        s = dot4(0x01010101u, a.a0.z, s);
+        s = dot4(0x01010101u, a.a0.w, s);
+        s = dot4(0x01010101u, a.a1.x, s);
+        s = dot4(0x01010101u, a.a1.y, s);
+        s = dot4(0x01010101u, a.a1.z, s);
+        s = dot4(0x01010101u, a.a1.w, s);
+        a.sum = s;
+    }
     return a;
 }
 
-__device__ __forceinline__ float q8_0_partial(const uint8_t *__restrict__ blk, const Q8Act &a) {
-    const float d = ld_f16(blk);
-    const uint4 q0 = ld_u4_a2(blk + 2), q1 = ld_u4_a2(blk + 18);
-    int p = 0;
-    p = dot4(q0.x, a.a0.x, p);
-    p = dot4(q0.y, a.a0.y, p);
-    p = dot4(q0.z, a.a0.z, p);
-    p = dot4(q0.w, a.a0.w, p);
-    p = dot4(q1.x, a.a1.x, p);
-    p = dot4(q1.y, a.a1.y, p);
-    p = dot4(q1.z, a.a1.z, p);
-    p = dot4(q1.w, a.a1.w, p);
-    return (d * a.dx) * static_cast<float>(p);
+struct Block32Layout {
+    int bytes, qs, qh, offset;  // block size, offsets of qs and qh (qh < 0: no fifth bit), code offset
+    bool min;                   // f16 m follows d
+};
+template <uint32_t kQuant>
+constexpr Block32Layout block32_layout() {
+    switch (kQuant) {
+    case kQ4_0: return {static_cast<int>(kQ4_0Bytes), 2, -1, 8, false};
+    case kQ4_1: return {static_cast<int>(kQ4_1Bytes), 4, -1, 0, true};
+    case kQ5_0: return {static_cast<int>(kQ5_0Bytes), 6, 2, 16, false};
+    case kQ5_1: return {static_cast<int>(kQ5_1Bytes), 8, 4, 0, true};
+    default: return {static_cast<int>(kQ8_0Bytes), 2, -1, 0, false};
+    }
 }
 
+// four bits -> bit 4 of four bytes (bit j of x lands in byte j)
+__device__ __forceinline__ uint32_t spread_fifth_bits(uint32_t x) {
+    return ((__umul24(x & 15u, 0x00204081u)) & 0x01010101u) << 4;
+}
+
+template <uint32_t kQuant>
+__device__ __forceinline__ float block32_partial(const uint8_t *__restrict__ blk, const Q8Act &a) {
+    constexpr Block32Layout F = block32_layout<kQuant>();
+    const float d = ld_f16(blk);
+    if constexpr (kQuant == kQ8_0) {
+        const uint4 q0 = ld_u4_a2(blk + 2), q1 = ld_u4_a2(blk + 18);
+        int p = 0;
+        p = dot4(q0.x, a.a0.x, p);
+        p = dot4(q0.y, a.a0.y, p);
+        p = dot4(q0.z, a.a0.z, p);
+        p = dot4(q0.w, a.a0.w, p);
+        p = dot4(q1.x, a.a1.x, p);
+        p = dot4(q1.y, a.a1.y, p);
+        p = dot4(q1.z, a.a1.z, p);
+        p = dot4(q1.w, a.a1.w, p);
+        return (d * a.dx) * static_cast<float>(p);
+    } else {
+        const uint4 qs = ld_u4_a2(blk + F.qs);
+        uint4 lo = make_uint4(qs.x & 0x0f0f0f0fu, qs.y & 0x0f0f0f0fu, qs.z & 0x0f0f0f0fu, qs.w & 0x0f0f0f0fu);
+        uint4 hi = make_uint4((qs.x >> 4) & 0x0f0f0f0fu, (qs.y >> 4) & 0x0f0f0f0fu, (qs.z >> 4) & 0x0f0f0f0fu,
+                              (qs.w >> 4) & 0x0f0f0f0fu);
+        if constexpr (F.qh >= 0) {
+            const uint32_t qh = ld_u32_a2(blk + F.qh);
+            lo.x |= spread_fifth_bits(qh);
+            lo.y |= spread_fifth_bits(qh >> 4);
+            lo.z |= spread_fifth_bits(qh >> 8);
+            lo.w |= spread_fifth_bits(qh >> 12);
+            hi.x |= spread_fifth_bits(qh >> 16);
+            hi.y |= spread_fifth_bits(qh >> 20);
+            hi.z |= spread_fifth_bits(qh >> 24);
+            hi.w |= spread_fifth_bits(qh >> 28);
+        }
+        int p = 0;
+        p = dot4(lo.x, a.a0.x, p);
+        p = dot4(lo.y, a.a0.y, p);
+        p = dot4(lo.z, a.a0.z, p);
+        p = dot4(lo.w, a.a0.w, p);
+        p = dot4(hi.x, a.a1.x, p);
+        p = dot4(hi.y, a.a1.y, p);
+        p = dot4(hi.z, a.a1.z, p);
+        p = dot4(hi.w, a.a1.w, p);
+        if constexpr (F.min) {
+            const float m = ld_f16(blk + 2);
+            return a.dx * (d * static_cast<float>(p) + m * static_cast<float>(a.sum));
+        } else {
+            return (d * a.dx) * static_cast<float>(p - F.offset * a.sum);
+        }
+    }
+}
+
+template <uint32_t kQuant>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
-    gemv_q8_0_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                     float *__restrict__ out, uint32_t rows, uint32_t nb32) {
+    gemv_block32_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                        float *__restrict__ out, uint32_t rows, uint32_t nb32) {
+    constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
+    constexpr bool kSum = kQuant != kQ8_0;
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t tok = blockIdx.y;
     const size_t abase = static_cast<size_t>(tok) * nb32;
-    const size_t row_bytes = static_cast<size_t>(nb32) * kQ8_0Bytes;
+    const size_t row_bytes = static_cast<size_t>(nb32) * kBlockBytes;
     const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     const uint32_t n_waves = gridDim.x * kWavesPerWg;
     if (nb32 <= 2 * kWave) {
         const uint32_t b0 = lane, b1 = lane + kWave;
         const bool has0 = b0 < nb32, has1 = b1 < nb32;
-        const Q8Act a0 = q8_load_act(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
-        const Q8Act a1 = q8_load_act(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
+        const Q8Act a0 = q8_load_act<kSum>(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
+        const Q8Act a1 = q8_load_act<kSum>(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
         for (uint32_t row = wave_global; row < rows; row += n_waves) {
             const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
             float acc = 0.0f;
-            if (has0) acc = q8_0_partial(rowp + static_cast<size_t>(b0) * kQ8_0Bytes, a0);
-            if (has1) acc += q8_0_partial(rowp + static_cast<size_t>(b1) * kQ8_0Bytes, a1);
+            if (has0) acc = block32_partial<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes, a0);
+            if (has1) acc += block32_partial<kQuant>(rowp + static_cast<size_t>(b1) * kBlockBytes, a1);
             acc = seg_sum<kWave>(acc);
             if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
         }
@@ -295,12 +374,21 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
             float acc = 0.0f;
             for (uint32_t b = lane; b < nb32; b += kWave)
-                acc += q8_0_partial(rowp + static_cast<size_t>(b) * kQ8_0Bytes,
-                                    q8_load_act(aq + (abase + b) * 32, ad[abase + b]));
+                acc += block32_partial<kQuant>(rowp + static_cast<size_t>(b) * kBlockBytes,
+                                               q8_load_act<kSum>(aq + (abase + b) * 32, ad[abase + b]));
             acc = seg_sum<kWave>(acc);
             if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
         }
     }
+}
+
+template <uint32_t kQuant>
+void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,
+                    hipStream_t stream) {
+    const uint32_t waves = rows < kTargetWaves ? rows : kTargetWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    hipLaunchKernelGGL(gemv_block32_kernel<kQuant>, grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, act.d, out, rows,
+                       nb32);
 }
 
 }  // namespace
@@ -351,9 +439,19 @@ void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, h
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,
                       hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
-    const uint32_t waves = rows < kTargetWaves ? rows : kTargetWaves;
-    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
-    hipLaunchKernelGGL(gemv_q8_0_kernel, grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, act.d, out, rows, nb32);
+    launch_block32<kQ8_0>(w, act, out, rows, nb32, seq, stream);
+}
+
+void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
+                         uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    switch (quant) {
+    case kQ4_0: launch_block32<kQ4_0>(w, act, out, rows, nb32, seq, stream); break;
+    case kQ4_1: launch_block32<kQ4_1>(w, act, out, rows, nb32, seq, stream); break;
+    case kQ5_0: launch_block32<kQ5_0>(w, act, out, rows, nb32, seq, stream); break;
+    case kQ5_1: launch_block32<kQ5_1>(w, act, out, rows, nb32, seq, stream); break;
+    default: launch_block32<kQ8_0>(w, act, out, rows, nb32, seq, stream); break;
+    }
 }
 
 }  // namespace rnb

@@ -140,6 +140,8 @@ int main(int argc, char **argv) {
         run_case(dir, "q5k_batch", 13, 512, 5, q5k_gemv_batch);
         run_case(dir, "q2k_gemv", 18, 768, 1, q2k_gemv);
         run_case(dir, "q3k_batch", 11, 512, 6, q3k_gemv_batch);
+        run_case(dir, "q4_0_gemv", 21, 608, 1, q4_0_gemv);
+        run_case(dir, "q5_1_batch", 10, 160, 3, q5_1_gemv_batch);
         std::printf("run: %d failure(s)\n", failures);
         return failures ? 1 : 0;
     }

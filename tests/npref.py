@@ -8,6 +8,48 @@ def f16_bytes(v) -> bytes:
     return np.array([v], dtype=np.float16).tobytes()
 
 
+# ---- Q4_0 / Q4_1 / Q5_0 / Q5_1 (32-element blocks) ------------------------------------
+
+LEGACY_LAYOUT = {2: (18, False, False), 3: (20, True, False), 6: (22, False, True), 7: (24, True, True)}  # bytes, min, qh
+
+
+def make_legacy_block(quant, d, m, codes) -> np.ndarray:
+    """codes: 32 unsigned codes (0..15, or 0..31 for the 5-bit formats) in element order.  Layout: f16 d, [f16 m],
+    [u32 qh], qs[16]; element i < 16 in the low nibble of qs[i], element 16 + i in its high nibble, fifth bit of
+    element e in bit e of qh."""
+    _, has_min, has_qh = LEGACY_LAYOUT[quant]
+    c = np.asarray(codes, dtype=np.uint32)
+    parts = [np.frombuffer(f16_bytes(d), dtype=np.uint8)]
+    if has_min:
+        parts.append(np.frombuffer(f16_bytes(m), dtype=np.uint8))
+    if has_qh:
+        qh = int((((c >> 4) & 1) << np.arange(32, dtype=np.uint32)).sum())
+        parts.append(np.frombuffer(np.array([qh], dtype="<u4").tobytes(), dtype=np.uint8))
+    parts.append(((c[:16] & 15) | ((c[16:] & 15) << 4)).astype(np.uint8))
+    return np.concatenate(parts).astype(np.uint8)
+
+
+def dequant_legacy_f64(quant, blocks) -> np.ndarray:
+    nbytes, has_min, has_qh = LEGACY_LAYOUT[quant]
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, nbytes)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float64)
+    off = 2
+    m = np.zeros_like(d)
+    if has_min:
+        m = b[:, 2:4].copy().view(np.float16).astype(np.float64)
+        off = 4
+    code = np.zeros((b.shape[0], 32), dtype=np.int64)
+    if has_qh:
+        qh = b[:, off:off + 4].copy().view("<u4").astype(np.int64)
+        code += ((qh >> np.arange(32)) & 1) << 4
+        off += 4
+    qs = b[:, off:off + 16].astype(np.int64)
+    code += np.concatenate([qs & 15, qs >> 4], axis=1)
+    if has_min:
+        return (code * d + m).reshape(-1)
+    return ((code - (16 if has_qh else 8)) * d).reshape(-1)
+
+
 # ---- Q2_K ---------------------------------------------------------------------------
 
 def make_q2k_block(d, dmin, sc, mn, values) -> np.ndarray:

@@ -10,6 +10,8 @@ from tests import npref
 
 pytestmark = pytest.mark.gpu
 
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 REL = 1e-3          # tolerance named by the task: max relative error 1e-3 per row
 TIGHT = 2e-5        # what f32 summation-order differences actually allow, relative to rms
@@ -27,7 +29,9 @@ def check_close(got, ref, gold=None, label=""):
 
 
 def gemv_fn(rnb, quant, batch=False):
-    table = {(Q2_K, False): rnb.q2k_gemv, (Q2_K, True): rnb.q2k_gemv_batch, (Q3_K, False): rnb.q3k_gemv,
+    table = {(Q4_0, False): rnb.q4_0_gemv, (Q4_0, True): rnb.q4_0_gemv_batch, (Q4_1, False): rnb.q4_1_gemv,
+             (Q4_1, True): rnb.q4_1_gemv_batch, (Q5_0, False): rnb.q5_0_gemv, (Q5_0, True): rnb.q5_0_gemv_batch,
+             (Q5_1, False): rnb.q5_1_gemv, (Q5_1, True): rnb.q5_1_gemv_batch, (Q2_K, False): rnb.q2k_gemv, (Q2_K, True): rnb.q2k_gemv_batch, (Q3_K, False): rnb.q3k_gemv,
              (Q3_K, True): rnb.q3k_gemv_batch, (Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q5_K, False): rnb.q5k_gemv,
              (Q5_K, True): rnb.q5k_gemv_batch, (Q6_K, False): rnb.q6k_gemv, (Q6_K, True): rnb.q6k_gemv_batch,
              (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
@@ -126,13 +130,47 @@ def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
     check_close(got, ref, gold, f"quant {quant} rows {rows} nblk {nblk}")
 
 
-@pytest.mark.parametrize("quant,cols", [(Q8_0, 32), (Q8_0, 96), (Q8_0, 32 * 65), (Q8_0, 32 * 129)])
-def test_q8_0_gemv_block_counts_off_the_wave_size(rnb, oracle, quant, cols):
+@pytest.mark.parametrize("quant", (Q8_0,) + LEGACY)
+@pytest.mark.parametrize("cols", [32, 96, 32 * 65, 32 * 129])
+def test_block32_gemv_block_counts_off_the_wave_size(rnb, oracle, quant, cols):
     rows = 6
     w = oracle.make_weights(quant, rows, cols, 3000 + cols)
     x = oracle.fill_normal(cols, 3001 + cols, 1.0)
-    check_close(rnb.q8_0_gemv(w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x)[0],
-                oracle.gemv(quant, w, rows, cols, x, gold=True)[0], f"q8_0 cols {cols}")
+    check_close(gemv_fn(rnb, quant)(w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x)[0],
+                oracle.gemv(quant, w, rows, cols, x, gold=True)[0], f"quant {quant} cols {cols}")
+
+
+@pytest.mark.parametrize("quant", LEGACY)
+def test_legacy_formats_shapes_batches_and_extremes(rnb, oracle, quant):
+    """Q4_0 / Q4_1 / Q5_0 / Q5_1: decode shapes up to 4096x4096, small batches, and blocks at the ends of every field's
+    range (all-max and all-zero codes, every fifth bit set, negative / zero / subnormal f16 scales and mins)."""
+    for rows, cols in ((1, 32), (7, 1056), (300, 4096), (4096, 4096), (33, 11008)):
+        w = oracle.make_weights(quant, rows, cols, 4000 + rows + quant)
+        x = oracle.fill_normal(cols, 4001 + cols, 1.0)
+        check_close(gemv_fn(rnb, quant)(w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x)[0],
+                    oracle.gemv(quant, w, rows, cols, x, gold=True)[0], f"quant {quant} {rows}x{cols}")
+        rnb.release(w)
+    for seq in (2, 5, 17):
+        rows, cols = 37, 768
+        w = oracle.make_weights(quant, rows, cols, 4100 + quant)
+        x = oracle.fill_normal(seq * cols, 4101 + seq, 1.0)
+        got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+        assert got.shape == (seq, rows)
+        check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                    f"quant {quant} batch {seq}")
+    rng = np.random.default_rng(29 + quant)
+    top = 31 if quant in (Q5_0, Q5_1) else 15
+    rows, nb32 = 8, 16
+    x = oracle.fill_normal(nb32 * 32, 30, 1.0)
+    x[64:96] = 0.0
+    blocks = []
+    for i in range(rows * nb32):
+        codes = [np.full(32, top), np.zeros(32), rng.integers(0, top + 1, 32), np.full(32, 16 if top == 31 else 8)][i % 4]
+        blocks.append(npref.make_legacy_block(quant, [1.0, -0.5, 6e-8, 0.0, 2.0 ** -14][i % 5], [0.25, -1.0, 0.0, 6e-8][i % 4],
+                                              codes))
+    w = np.concatenate(blocks)
+    check_close(gemv_fn(rnb, quant)(w, rows, nb32 * 32, x), oracle.gemv(quant, w, rows, nb32 * 32, x)[0],
+                oracle.gemv(quant, w, rows, nb32 * 32, x, gold=True)[0], f"quant {quant} extremes")
 
 
 def test_gemv_extreme_blocks(rnb, oracle):
@@ -491,7 +529,7 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
 
 # ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
 
-@pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q5_1])
 @pytest.mark.parametrize("seq,n_ff,n_embd", [(2, 256, 256), (3, 768, 512), (5, 512, 4608), (17, 512, 768), (40, 1024, 256)])
 def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
     """Decode-sized batches take the fused gate/up GEMV, 16+ tokens the MFMA GEMM + SiLU kernel, rows longer than

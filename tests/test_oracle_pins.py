@@ -9,6 +9,8 @@ import pytest
 
 from tests import npref
 
+Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 
 
@@ -81,6 +83,12 @@ def _random_q4k(rng, n):
     return np.concatenate(blocks)
 
 
+def _random_legacy(quant, rng, n):
+    top = 32 if quant in (Q5_0, Q5_1) else 16
+    return np.concatenate([npref.make_legacy_block(quant, rng.uniform(-1e-2, 1e-2), rng.uniform(-0.1, 0.1),
+                                                   rng.integers(0, top, 32)) for _ in range(n)])
+
+
 def _random_q2k(rng, n):
     return np.concatenate([npref.make_q2k_block(rng.uniform(1e-4, 5e-3), rng.uniform(1e-4, 5e-3), rng.integers(0, 16, 16),
                                                 rng.integers(0, 16, 16), rng.integers(0, 4, 256)) for _ in range(n)])
@@ -128,6 +136,38 @@ def test_dequantize_q4k_places_each_nibble(oracle):
     got = oracle.dequantize(Q4_K, blocks).astype(np.float64)
     want = npref.dequant_q4k_f64(blocks)
     assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
+
+
+@pytest.mark.parametrize("quant", LEGACY)
+def test_dequantize_legacy_formats_place_every_field(oracle, quant):
+    """crates/rnb-cpu/src/quantize/dequant.rs:7-53 against hand-built bytes: one nibble, one high bit at a time."""
+    nbytes, has_min, has_qh = npref.LEGACY_LAYOUT[quant]
+    qs_off = 2 + (2 if has_min else 0) + (4 if has_qh else 0)
+    offset = 0 if has_min else (16 if has_qh else 8)
+    base = np.zeros(nbytes, np.uint8)
+    base[0:2] = np.frombuffer(npref.f16_bytes(2.0), np.uint8)
+    if has_min:
+        base[2:4] = np.frombuffer(npref.f16_bytes(0.5), np.uint8)
+    background = 0.5 if has_min else -2.0 * offset
+    for i in (0, 7, 15):
+        blk = base.copy()
+        blk[qs_off + i] = 0xA3  # low nibble 3 -> element i, high nibble 10 -> element 16 + i
+        want = np.full(32, background, np.float32)
+        want[i] += 2.0 * 3
+        want[16 + i] += 2.0 * 10
+        assert np.array_equal(oracle.dequantize(quant, blk), want), i
+    if has_qh:
+        for e in (0, 9, 16, 31):
+            blk = base.copy()
+            blk[qs_off - 4 + e // 8] = 1 << (e % 8)
+            want = np.full(32, background, np.float32)
+            want[e] += 2.0 * 16
+            assert np.array_equal(oracle.dequantize(quant, blk), want), e
+    rng = np.random.default_rng(50 + quant)
+    blocks = _random_legacy(quant, rng, 200)
+    got = oracle.dequantize(quant, blocks).astype(np.float64)
+    want = npref.dequant_legacy_f64(quant, blocks)
+    assert np.allclose(got, want, rtol=0, atol=4e-7 * np.abs(want).max())
 
 
 def test_dequantize_q2k_reference_vectors_and_placement(oracle):
@@ -376,6 +416,47 @@ def test_q4k_mins_use_32_wide_bsums(oracle):
     summ = sum((k + 1) * (bs[0, 2 * k] + bs[0, 2 * k + 1]) for k in range(8))
     assert oracle.dot(Q4_K, blk, act) == -2.0 * summ
     assert oracle.dot(Q4_K, blk, act, avx2=True) == -2.0 * summ
+
+
+# ---- Q4_0 / Q4_1 / Q5_0 / Q5_1 x Q8 dots -------------------------------------------------
+
+def _q8_act(d, q):
+    a = np.zeros(1, dtype=np.dtype([("d", "<f4"), ("qs", "i1", (32,))]))
+    a["d"] = d
+    a["qs"] = np.asarray(q, np.int8)
+    return a
+
+
+@pytest.mark.parametrize("quant", LEGACY)
+def test_legacy_dot_known_vectors_and_identity(oracle, quant):
+    """crates/rnb-cpu/src/gemm/neon_dot.rs:83-214 and neon_quant.rs:88-158 on hand vectors: all codes equal ->
+    (code - offset) * sum(q) * d * d_x for the _0 formats, d_x * (d * code + m) * sum(q) for the _1 formats; then the
+    f64 identity against an independent dequantiser."""
+    _, has_min, has_qh = npref.LEGACY_LAYOUT[quant]
+    q = (np.arange(32) % 9 - 4).astype(np.int8)
+    sq = float(q.astype(np.int64).sum())
+    code = 19 if has_qh else 11
+    blk = npref.make_legacy_block(quant, 2.0, 0.25, np.full(32, code))
+    got = oracle.dot(quant, blk, _q8_act(0.5, q))
+    if has_min:
+        assert got == 0.5 * (2.0 * code * sq + 0.25 * sq)
+    else:
+        assert got == (code - (16 if has_qh else 8)) * sq * (2.0 * 0.5)
+    # one code differs: only that element's activation enters the difference
+    codes = np.full(32, code)
+    codes[21] += 3
+    got2 = oracle.dot(quant, npref.make_legacy_block(quant, 2.0, 0.25, codes), _q8_act(0.5, q))
+    assert got2 - got == 3 * float(q[21]) * 2.0 * 0.5
+    rng = np.random.default_rng(60 + quant)
+    for nb in (1, 3, 128):
+        row = _random_legacy(quant, rng, nb)
+        x = rng.standard_normal(nb * 32).astype(np.float32)
+        act = oracle.quantize_q8(x)
+        xq = (act["d"].astype(np.float64)[:, None] * act["qs"].astype(np.float64)).reshape(-1)
+        want = float(np.dot(npref.dequant_legacy_f64(quant, row), xq))
+        assert oracle.dot(quant, row, act, gold=True) == pytest.approx(want, rel=1e-11, abs=1e-12)
+        scale = float(np.sum(np.abs(npref.dequant_legacy_f64(quant, row) * xq)))
+        assert abs(oracle.dot(quant, row, act) - want) <= 4e-7 * scale
 
 
 # ---- Q2_K / Q3_K x Q8_K dots ------------------------------------------------------------
@@ -657,6 +738,24 @@ def test_q5k_quantiser_roundtrip_property(oracle):
     assert np.sqrt(np.mean((xn - yn) ** 2)) / np.sqrt(np.mean(xn ** 2)) < 0.05
     d, dmin, sc, mn, val = npref.split_q5k(qn)
     assert sc.max() == 63 and val.max() == 31 and val.min() == 0
+
+
+@pytest.mark.parametrize("quant,bound", [(Q4_0, 0.12), (Q4_1, 0.12), (Q5_0, 0.06), (Q5_1, 0.06)])
+def test_legacy_generators_roundtrip(oracle, quant, bound):
+    x = oracle.fill_normal(32 * 300, 25, 0.02)
+    w = oracle.quantize_row(quant, x)
+    y = oracle.dequantize(quant, w)
+    assert np.sqrt(np.mean((x - y) ** 2)) / np.sqrt(np.mean(x ** 2)) < bound
+    # the driver: out[s][r] == dot(row r, Q8(x_s)), seq-major
+    rows, cols = 3, 96
+    wm = oracle.make_weights(quant, rows, cols, 7)
+    xs = oracle.fill_normal(2 * cols, 8, 1.0).reshape(2, cols)
+    out = oracle.gemv(quant, wm, rows, cols, xs)
+    rb = wm.size // rows
+    for si in range(2):
+        act = oracle.quantize_q8(xs[si])
+        for r in range(rows):
+            assert out[si, r] == np.float32(oracle.dot(quant, wm[r * rb:(r + 1) * rb], act))
 
 
 def test_q2k_q3k_generators_roundtrip(oracle):
