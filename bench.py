@@ -508,8 +508,8 @@ def main() -> int:
                    "stream_ms_per_step": main_res["wall_ms_per_step"],
                    "graph_ms_per_step": main_res.get("graph_ms_per_step")},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("gemv_kquant_kernel<false,1>"),
-                     "kernel": "gemv_kquant_kernel<false,1>",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("gemv_kquant_kernel<12,1>"),
+                     "kernel": "gemv_kquant_kernel<12,1>",
                      "bytes_per_launch": nbytes, "kernel_ms_mean": main_res["kernel_ms_mean"],
                      "kernel_ms_runs": main_res["kernel_ms_runs"],
                      "timing": "HIP events around back-to-back launches on the library stream, 3 runs"},
