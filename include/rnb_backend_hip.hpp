@@ -8,6 +8,7 @@
 //   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
 //   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
 //   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
+//   q6k_gemv_argmax / q8_0_gemv_argmax          quant_api.rs:2170-2204, 733-768
 //   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
 //   dense_q4k_silu_ffn_batch                    api/dense_api.rs:297-337
 //   GgufFile                                    crates/rnb-loader/src/gguf/parser.rs:16-24, 247-407
@@ -84,6 +85,19 @@ inline Result<Unit> q4k_gemv_into(Bytes weights, size_t rows, size_t cols, Float
 }
 inline Result<std::vector<float>> q4k_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
     return gemv_impl(rnb_hip_q4k_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+// q6k_gemv_argmax / q8_0_gemv_argmax -> (row index, value), quant_api.rs:2170-2204, 733-768
+inline Result<std::pair<uint32_t, float>> q6k_gemv_argmax(Bytes weights, size_t rows, size_t cols, Floats input) {
+    std::pair<uint32_t, float> best{0, 0.0f};
+    const int st = rnb_hip_q6k_gemv_argmax(weights.ptr, weights.len, rows, cols, input.ptr, input.len, &best.first, &best.second);
+    if (st != RNB_HIP_OK) return make_err<std::pair<uint32_t, float>>(st);
+    return make_ok(best);
+}
+inline Result<std::pair<uint32_t, float>> q8_0_gemv_argmax(Bytes weights, size_t rows, size_t cols, Floats input) {
+    std::pair<uint32_t, float> best{0, 0.0f};
+    const int st = rnb_hip_q8_0_gemv_argmax(weights.ptr, weights.len, rows, cols, input.ptr, input.len, &best.first, &best.second);
+    if (st != RNB_HIP_OK) return make_err<std::pair<uint32_t, float>>(st);
+    return make_ok(best);
 }
 #define RNB_HIP_BLOCK32_MIRROR(name)                                                                               \
     inline Result<std::vector<float>> name##_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {         \

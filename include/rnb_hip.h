@@ -203,6 +203,9 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
  * crates/rnb-backend/cuda/cuda/kernels/quant_batch_and_ops.cuh:3286-3328); 8 bytes come back instead of rows*4. */
 int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                             uint32_t *index_out, float *value_out);
+/* q8_0_gemv_argmax, quant_api.rs:733-768: the same for a Q8_0 head (Q8 x Q8_0 integer dot) */
+int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                             uint32_t *index_out, float *value_out);
 
 /* ---- dense SwiGLU FFN: the GEMV's neighbours fused into one call -------------------------------
  * dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq_len, input) -> Vec<f32>,

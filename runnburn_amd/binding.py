@@ -65,6 +65,7 @@ SYMBOLS = [
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
     ("rnb_hip_q6k_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
+    ("rnb_hip_q8_0_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_silu_ffn_dev", _i, [_vp, _vp, _vp, _u32, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gguf_open", _i, [C.c_char_p, C.POINTER(_vp)]),
@@ -446,6 +447,14 @@ def q6k_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A00
     w, x = _bytes_view(weights), _f32(input).ravel()
     idx, val = _u32(), C.c_float()
     _check(lib().rnb_hip_q6k_gemv_argmax(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
+    return int(idx.value), float(val.value)
+
+
+def q8_0_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A002
+    """quant_api.rs:733-768 -> (row index, value)"""
+    w, x = _bytes_view(weights), _f32(input).ravel()
+    idx, val = _u32(), C.c_float()
+    _check(lib().rnb_hip_q8_0_gemv_argmax(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
     return int(idx.value), float(val.value)
 
 

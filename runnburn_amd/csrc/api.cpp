@@ -742,17 +742,22 @@ int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes) {
     return RNB_HIP_OK;
 }
 
-int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
-                            uint32_t *index_out, float *value_out) {
+}  // extern "C"
+
+namespace {
+
+// LM-head GEMV with the arg-max taken on the device.  The same three checks and texts as the format's plain GEMV
+// (crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:2176-2193 for Q6_K, :739-756 for Q8_0).
+int gemv_argmax_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                     size_t x_len, uint32_t *index_out, float *value_out) {
     QuantInfo qi;
-    quant_info(kQ6K, &qi);
+    quant_info(quant, &qi);
+    const std::string label = qi.label;
     size_t seq = 0;
-    // same three checks and texts as q6k_gemv (crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:2176-2193)
     int st = validate_matmul(qi, w_len, rows, cols, x_len, rows, false, &seq);
     if (st != RNB_HIP_OK) return st;
-    if (!w || !x || !index_out || !value_out) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K null pointer argument");
-    if (rows == 0) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K argmax needs at least one row");
-    if (rows > 0x7fffffffu) return fail(RNB_HIP_INVALID_REQUEST, "Q6_K shape out of range");
+    if (!w || !x || !index_out || !value_out) return fail(RNB_HIP_INVALID_REQUEST, label + " null pointer argument");
+    if (rows == 0) return fail(RNB_HIP_INVALID_REQUEST, label + " argmax needs at least one row");
     Guard g;
     if (!g.state) return g.status;
     State &s = *g.state;
@@ -767,7 +772,7 @@ int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t 
     std::memcpy(s.bounce_in.ptr, x, in_bytes);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += in_bytes;
-    st = run_matmul_dev(s, kQ6K, w_dev, rows, cols, s.x_f32.as<float>(), 1, s.out_f32.as<float>());
+    st = run_matmul_dev(s, quant, w_dev, rows, cols, s.x_f32.as<float>(), 1, s.out_f32.as<float>());
     if (st != RNB_HIP_OK) return st;
     float *vals = s.argmax_scratch.as<float>();
     uint32_t *idxs = reinterpret_cast<uint32_t *>(vals + 257);
@@ -781,6 +786,20 @@ int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t 
     std::memcpy(value_out, s.bounce_out.ptr, 4);
     std::memcpy(index_out, static_cast<uint8_t *>(s.bounce_out.ptr) + 4, 4);
     return RNB_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                            uint32_t *index_out, float *value_out) {
+    return gemv_argmax_host(kQ6K, w, w_len, rows, cols, x, x_len, index_out, value_out);
+}
+
+int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                             uint32_t *index_out, float *value_out) {
+    return gemv_argmax_host(kQ8_0, w, w_len, rows, cols, x, x_len, index_out, value_out);
 }
 
 int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,

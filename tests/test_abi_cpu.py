@@ -109,6 +109,18 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q8_0 input length mismatch: got 33, expected 32"
 
 
+def test_argmax_entry_points_validate_like_their_gemv():
+    z = np.zeros
+    e = _err(rnb.q8_0_gemv_argmax, z(34, np.uint8), 1, 31, z(31, np.float32))
+    assert str(e) == "Q8_0 cols must be divisible by 32, got 31"
+    e = _err(rnb.q8_0_gemv_argmax, z(35, np.uint8), 1, 32, z(32, np.float32))
+    assert str(e) == "Q8_0 weight byte mismatch: got 35, expected 34"
+    e = _err(rnb.q6k_gemv_argmax, z(210, np.uint8), 1, 256, z(255, np.float32))
+    assert str(e) == "Q6_K input length mismatch: got 255, expected 256"
+    e = _err(rnb.q8_0_gemv_argmax, z(0, np.uint8), 0, 32, z(32, np.float32))
+    assert str(e) == "Q8_0 argmax needs at least one row"
+
+
 def test_shapes_beyond_32_bit_indexing_are_refused():
     z = np.zeros
     e = _err(rnb.q4k_gemv_batch, z(0, np.uint8), 0, 1 << 32, z(0, np.float32))

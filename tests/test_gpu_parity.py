@@ -527,6 +527,22 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
         rnb.release(w)
 
 
+def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
+    rows, cols = 3001, 1024
+    w = oracle.make_weights(Q8_0, rows, cols, 510)
+    x = oracle.fill_normal(cols, 511, 1.0)
+    full = rnb.q8_0_gemv(w, rows, cols, x)
+    idx, val = rnb.q8_0_gemv_argmax(w, rows, cols, x)
+    assert idx == int(np.argmax(full)) and val == full[idx]
+    # two identical rows that win: the lower index is reported
+    rb = cols // 32 * 34
+    w2 = w.copy().reshape(rows, rb)
+    w2[2500] = w2[idx]
+    w2[17] = w2[idx]
+    idx2, val2 = rnb.q8_0_gemv_argmax(w2.reshape(-1), rows, cols, x)
+    assert idx2 == min(17, idx) and val2 == val
+
+
 # ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
 
 @pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q5_1])
