@@ -11,6 +11,7 @@
 //   q6k_gemv_argmax / q8_0_gemv_argmax          quant_api.rs:2170-2204, 733-768
 //   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
 //   dense_q4k_silu_ffn_batch                    api/dense_api.rs:297-337
+//   dense_q4k_attention_qkv                     api/dense_api.rs:916-985
 //   GgufFile                                    crates/rnb-loader/src/gguf/parser.rs:16-24, 247-407
 //   HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
 //
@@ -85,6 +86,16 @@ inline Result<Unit> q4k_gemv_into(Bytes weights, size_t rows, size_t cols, Float
 }
 inline Result<std::vector<float>> q4k_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
     return gemv_impl(rnb_hip_q4k_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+// dense_q4k_attention_qkv(q_weights, k_weights, v_weights, q_rows, kv_rows, n_embd, input, q, k, v), api/dense_api.rs:916-985
+inline Result<Unit> dense_q4k_attention_qkv(Bytes q_weights, Bytes k_weights, Bytes v_weights, size_t q_rows, size_t kv_rows,
+                                            size_t n_embd, Floats input, float *q, size_t q_len, float *k, size_t k_len,
+                                            float *v, size_t v_len) {
+    const int st = rnb_hip_dense_q4k_attention_qkv(q_weights.ptr, q_weights.len, k_weights.ptr, k_weights.len, v_weights.ptr,
+                                                   v_weights.len, q_rows, kv_rows, n_embd, input.ptr, input.len, q, q_len, k,
+                                                   k_len, v, v_len);
+    if (st != RNB_HIP_OK) return make_err<Unit>(st);
+    return make_ok(Unit{});
 }
 // q6k_gemv_argmax / q8_0_gemv_argmax -> (row index, value), quant_api.rs:2170-2204, 733-768
 inline Result<std::pair<uint32_t, float>> q6k_gemv_argmax(Bytes weights, size_t rows, size_t cols, Floats input) {

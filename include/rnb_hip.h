@@ -207,6 +207,15 @@ int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t 
 int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                              uint32_t *index_out, float *value_out);
 
+/* dense_q4k_attention_qkv(q_weights, k_weights, v_weights, q_rows, kv_rows, n_embd, input, q, k, v),
+ * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:916-985 (validation order and texts :928-968): the three Q4_K
+ * projections of one decode token.  x is quantised once and the rows of the three matrices run as ONE launch;
+ * q[0..q_rows), k[0..kv_rows), v[0..kv_rows) are written (capacities may be larger). */
+int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint8_t *k_w, size_t k_len,
+                                    const uint8_t *v_w, size_t v_len, size_t q_rows, size_t kv_rows,
+                                    size_t n_embd, const float *x, size_t x_len, float *q, size_t q_cap,
+                                    float *k, size_t k_cap, float *v, size_t v_cap);
+
 /* ---- dense SwiGLU FFN: the GEMV's neighbours fused into one call -------------------------------
  * dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq_len, input) -> Vec<f32>,
  * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337; validation order and texts from

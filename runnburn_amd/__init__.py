@@ -72,6 +72,7 @@ from .binding import (  # noqa: F401
     q6k_gemv_batch,
     q6k_gemv_into,
     q6k_gemv_argmax,
+    dense_q4k_attention_qkv,
     q8_0_gemv_argmax,
     q8_0_gemv,
     q8_0_gemv_batch,

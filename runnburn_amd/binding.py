@@ -65,6 +65,7 @@ SYMBOLS = [
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
     ("rnb_hip_q6k_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
+    ("rnb_hip_dense_q4k_attention_qkv", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_q8_0_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_silu_ffn_dev", _i, [_vp, _vp, _vp, _u32, _sz, _sz, _sz, _vp, _vp]),
@@ -448,6 +449,18 @@ def q6k_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A00
     idx, val = _u32(), C.c_float()
     _check(lib().rnb_hip_q6k_gemv_argmax(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
     return int(idx.value), float(val.value)
+
+
+def dense_q4k_attention_qkv(q_weights, k_weights, v_weights, q_rows: int, kv_rows: int, n_embd: int, input,  # noqa: A002
+                            q: np.ndarray, k: np.ndarray, v: np.ndarray) -> None:
+    """api/dense_api.rs:916-985: writes q[:q_rows], k[:kv_rows], v[:kv_rows] (f32, C-contiguous, may be longer)."""
+    qw, kw, vw = _bytes_view(q_weights), _bytes_view(k_weights), _bytes_view(v_weights)
+    x = _f32(input).ravel()
+    for name, a in (("q", q), ("k", k), ("v", v)):
+        if a.dtype != np.float32 or not a.flags["C_CONTIGUOUS"]:
+            raise TypeError(f"{name} must be a C-contiguous float32 array")
+    _check(lib().rnb_hip_dense_q4k_attention_qkv(_ptr(qw), qw.size, _ptr(kw), kw.size, _ptr(vw), vw.size, q_rows, kv_rows,
+                                                 n_embd, _ptr(x), x.size, _ptr(q), q.size, _ptr(k), k.size, _ptr(v), v.size))
 
 
 def q8_0_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A002

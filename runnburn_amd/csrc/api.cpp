@@ -802,6 +802,66 @@ int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t
     return gemv_argmax_host(kQ8_0, w, w_len, rows, cols, x, x_len, index_out, value_out);
 }
 
+int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint8_t *k_w, size_t k_len, const uint8_t *v_w,
+                                    size_t v_len, size_t q_rows, size_t kv_rows, size_t n_embd, const float *x, size_t x_len,
+                                    float *q, size_t q_cap, float *k, size_t k_cap, float *v, size_t v_cap) {
+    // validation order and texts: crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:928-968
+    if (x_len != n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    "dense QKV input length mismatch: got " + std::to_string(x_len) + ", expected " + std::to_string(n_embd));
+    if (n_embd % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV cols must be divisible by 256, got " + std::to_string(n_embd));
+    if (q_cap < q_rows || k_cap < kv_rows || v_cap < kv_rows)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV output length mismatch: q=" + std::to_string(q_cap) + " k=" +
+                                                 std::to_string(k_cap) + " v=" + std::to_string(v_cap) + " expected q>=" +
+                                                 std::to_string(q_rows) + " k/v>=" + std::to_string(kv_rows));
+    const size_t row_bytes = n_embd / 256 * kQ4KBytes;
+    if (q_len != q_rows * row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV q byte mismatch: got " + std::to_string(q_len) + ", expected " +
+                                                 std::to_string(q_rows * row_bytes));
+    if (k_len != kv_rows * row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV k byte mismatch: got " + std::to_string(k_len) + ", expected " +
+                                                 std::to_string(kv_rows * row_bytes));
+    if (v_len != kv_rows * row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV v byte mismatch: got " + std::to_string(v_len) + ", expected " +
+                                                 std::to_string(kv_rows * row_bytes));
+    if (q_rows > 0x3fffffffu || kv_rows > 0x1fffffffu || n_embd > 0x7fffffffu)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV shape out of range");
+    if ((q_len && !q_w) || (k_len && !k_w) || (v_len && !v_w) || (x_len && !x) || (q_rows && !q) || (kv_rows && (!k || !v)))
+        return fail(RNB_HIP_INVALID_REQUEST, "dense QKV null pointer argument");
+    const size_t total = q_rows + 2 * kv_rows;
+    if (total == 0 || n_embd == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *w_dev[3] = {nullptr, nullptr, nullptr};
+    if (q_len) HIP_TRY(s.resident_ptr(q_w, q_len, &w_dev[0]));
+    if (k_len) HIP_TRY(s.resident_ptr(k_w, k_len, &w_dev[1]));
+    if (v_len) HIP_TRY(s.resident_ptr(v_w, v_len, &w_dev[2]));
+    const size_t in_bytes = n_embd * sizeof(float), out_bytes = total * sizeof(float);
+    HIP_TRY(s.bounce_in.reserve(in_bytes));
+    HIP_TRY(s.bounce_out.reserve(out_bytes));
+    HIP_TRY(s.x_f32.reserve(in_bytes));
+    HIP_TRY(s.out_f32.reserve(out_bytes));
+    std::memcpy(s.bounce_in.ptr, x, in_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += in_bytes;
+    ActView act;
+    int st = quantize_activations(s, kQ4K, s.x_f32.as<float>(), 1, n_embd, &act);  // once for the three projections
+    if (st != RNB_HIP_OK) return st;
+    const uint32_t rows[3] = {static_cast<uint32_t>(q_rows), static_cast<uint32_t>(kv_rows), static_cast<uint32_t>(kv_rows)};
+    launch_gemv_q4k_multi(w_dev, rows, act, s.out_f32.as<float>(), static_cast<uint32_t>(n_embd / 256), s.stream);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += out_bytes;
+    const float *res = static_cast<const float *>(s.bounce_out.ptr);
+    std::memcpy(q, res, q_rows * sizeof(float));
+    std::memcpy(k, res + q_rows, kv_rows * sizeof(float));
+    std::memcpy(v, res + q_rows + kv_rows, kv_rows * sizeof(float));
+    return RNB_HIP_OK;
+}
+
 int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
                                      const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
                                      size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,

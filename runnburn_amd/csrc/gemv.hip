@@ -136,6 +136,59 @@ void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mi
                        act.d, act.bsums, mid, rows, nb, row_groups);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Several Q4_K matrices against ONE quantised activation in one launch (the Q, K and V projections of a decode step:
+// crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:916-985): the rows of the matrices are numbered through, a
+// lane segment finds its row's matrix by comparing against the running row counts, results go to one contiguous
+// vector [rows of matrix 0 | rows of matrix 1 | rows of matrix 2].
+// ---------------------------------------------------------------------------------------------
+struct MultiMat {
+    const uint8_t *w[3];
+    uint32_t end[3];  // running row counts: rows of matrices 0..i
+};
+
+template <int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_q4k_multi_kernel(MultiMat mats, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                          const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t nb, uint32_t row_groups) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const uint32_t rows = mats.end[2];
+    for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
+        const uint32_t row = grp * kRowsPerWave + rsel;
+        float acc = 0.0f;
+        if (row < rows) {
+            const int m = row < mats.end[0] ? 0 : (row < mats.end[1] ? 1 : 2);
+            const uint32_t local = row - (m == 0 ? 0u : mats.end[m - 1]);
+            const uint8_t *rowp = mats.w[m] + static_cast<size_t>(local) * row_bytes;
+            for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
+                const uint8_t *blk = rowp + static_cast<size_t>(b) * kQ4KBytes;
+                acc += q4k_partial(q4k_load_block(blk, g), q4k_load_act(aq + static_cast<size_t>(b) * 256, ad[b], abs + b * 16, g), g);
+            }
+        }
+        acc = seg_sum<kLanesPerRow>(acc);
+        if (sub == kLanesPerRow - 1 && row < rows) out[row] = acc;
+    }
+}
+
+template <int kRowsPerWave>
+void launch_multi(const MultiMat &mats, ActView act, float *out, uint32_t nb, hipStream_t stream) {
+    const uint32_t rows = mats.end[2];
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, 1, 1);
+    hipLaunchKernelGGL((gemv_q4k_multi_kernel<kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, mats, act.qs, act.d,
+                       act.bsums, out, nb, row_groups);
+}
+
 __global__ void __launch_bounds__(256) silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
                                                       float *__restrict__ out, size_t n) {
     for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
@@ -427,6 +480,24 @@ void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, 
         launch_gate_up<2>(wg, wu, act, mid, rows, nb, seq, stream);
     else
         launch_gate_up<1>(wg, wu, act, mid, rows, nb, seq, stream);
+}
+
+void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], ActView act, float *out, uint32_t nb,
+                           hipStream_t stream) {
+    MultiMat mats;
+    uint32_t total = 0;
+    for (int i = 0; i < 3; i++) {
+        mats.w[i] = w[i];
+        total += rows[i];
+        mats.end[i] = total;
+    }
+    if (total == 0) return;
+    if (nb <= 4)
+        launch_multi<4>(mats, act, out, nb, stream);
+    else if (nb <= 8)
+        launch_multi<2>(mats, act, out, nb, stream);
+    else
+        launch_multi<1>(mats, act, out, nb, stream);
 }
 
 void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream) {

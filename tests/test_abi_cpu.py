@@ -109,6 +109,26 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q8_0 input length mismatch: got 33, expected 32"
 
 
+def test_dense_qkv_validation_messages():
+    """crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:928-968"""
+    z = np.zeros
+    f = rnb.dense_q4k_attention_qkv
+    w2, w1 = z(2 * 144, np.uint8), z(144, np.uint8)
+    q, k, v = z(2, np.float32), z(1, np.float32), z(1, np.float32)
+    e = _err(f, w2, w1, w1, 2, 1, 256, z(255, np.float32), q, k, v)
+    assert str(e) == "dense QKV input length mismatch: got 255, expected 256"
+    e = _err(f, w2, w1, w1, 2, 1, 100, z(100, np.float32), q, k, v)
+    assert str(e) == "dense QKV cols must be divisible by 256, got 100"
+    e = _err(f, w2, w1, w1, 2, 1, 256, z(256, np.float32), q[:1], k, v)
+    assert str(e) == "dense QKV output length mismatch: q=1 k=1 v=1 expected q>=2 k/v>=1"
+    e = _err(f, w2[:-1], w1, w1, 2, 1, 256, z(256, np.float32), q, k, v)
+    assert str(e) == "dense QKV q byte mismatch: got 287, expected 288"
+    e = _err(f, w2, w2, w1, 2, 1, 256, z(256, np.float32), q, k, v)
+    assert str(e) == "dense QKV k byte mismatch: got 288, expected 144"
+    e = _err(f, w2, w1, w2, 2, 1, 256, z(256, np.float32), q, k, v)
+    assert str(e) == "dense QKV v byte mismatch: got 288, expected 144"
+
+
 def test_argmax_entry_points_validate_like_their_gemv():
     z = np.zeros
     e = _err(rnb.q8_0_gemv_argmax, z(34, np.uint8), 1, 31, z(31, np.float32))

@@ -527,6 +527,30 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
         rnb.release(w)
 
 
+@pytest.mark.parametrize("q_rows,kv_rows,n_embd", [(4096, 1024, 4096), (5, 3, 512), (7, 2, 1280), (64, 0, 2048),
+                                                     (0, 9, 768), (33, 33, 5120)])
+def test_dense_q4k_attention_qkv_one_launch(rnb, oracle, q_rows, kv_rows, n_embd):
+    """crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:916-985: three projections of one token from one quantised
+    activation; for rows of up to 16 super-blocks each output equals the plain GEMV of its matrix bit for bit."""
+    wq = oracle.make_weights(Q4_K, q_rows, n_embd, 600 + q_rows)
+    wk = oracle.make_weights(Q4_K, kv_rows, n_embd, 601 + kv_rows)
+    wv = oracle.make_weights(Q4_K, kv_rows, n_embd, 602 + kv_rows)
+    x = oracle.fill_normal(n_embd, 603, 1.0)
+    q = np.full(q_rows + 2, -3.0, np.float32)
+    k = np.full(kv_rows + 1, -3.0, np.float32)
+    v = np.full(kv_rows, -3.0, np.float32)
+    rnb.dense_q4k_attention_qkv(wq, wk, wv, q_rows, kv_rows, n_embd, x, q, k, v)
+    assert np.all(q[q_rows:] == -3.0) and np.all(k[kv_rows:] == -3.0)
+    for got, w, rows, name in ((q[:q_rows], wq, q_rows, "q"), (k[:kv_rows], wk, kv_rows, "k"), (v, wv, kv_rows, "v")):
+        if rows == 0:
+            continue
+        check_close(got, oracle.gemv(Q4_K, w, rows, n_embd, x)[0], oracle.gemv(Q4_K, w, rows, n_embd, x, gold=True)[0],
+                    f"qkv {name} {rows}x{n_embd}")
+        if n_embd <= 4096:  # longer rows: the plain GEMV splits K across waves, another f32 summation order
+            assert np.array_equal(got, rnb.q4k_gemv(w, rows, n_embd, x)), name
+        rnb.release(w)
+
+
 def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
     rows, cols = 3001, 1024
     w = oracle.make_weights(Q8_0, rows, cols, 510)
