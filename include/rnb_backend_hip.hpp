@@ -11,6 +11,7 @@
 //   q6k_gemv_argmax / q8_0_gemv_argmax          quant_api.rs:2170-2204, 733-768
 //   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
 //   dense_q4k_silu_ffn_batch                    api/dense_api.rs:297-337
+//   dense_q4k_gelu_ffn / dense_q4k_gelu_ffn_batch  api/dense_api.rs:182-293
 //   dense_q4k_attention_qkv                     api/dense_api.rs:916-985
 //   GgufFile                                    crates/rnb-loader/src/gguf/parser.rs:16-24, 247-407
 //   HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
@@ -201,6 +202,24 @@ inline Result<std::vector<float>> dense_q4k_silu_ffn_batch(Bytes gate_weights, B
                                                     down_weights.ptr, down_weights.len, down_quant, n_ff, n_embd, seq_len,
                                                     input.ptr, input.len, out.data(), out.size());
     return st == RNB_HIP_OK ? make_ok(std::move(out)) : make_err<std::vector<float>>(st);
+}
+inline Result<std::vector<float>> dense_q4k_gelu_ffn_batch(Bytes gate_weights, Bytes up_weights, Bytes down_weights,
+                                                           uint32_t down_quant, size_t n_ff, size_t n_embd,
+                                                           size_t seq_len, Floats input) {
+    std::vector<float> out(seq_len * n_embd);
+    const int st = rnb_hip_dense_q4k_gelu_ffn_batch(gate_weights.ptr, gate_weights.len, up_weights.ptr, up_weights.len,
+                                                    down_weights.ptr, down_weights.len, down_quant, n_ff, n_embd, seq_len,
+                                                    input.ptr, input.len, out.data(), out.size());
+    return st == RNB_HIP_OK ? make_ok(std::move(out)) : make_err<std::vector<float>>(st);
+}
+inline Result<std::vector<float>> dense_q4k_gelu_ffn(Bytes gate_weights, Bytes up_weights, Bytes down_weights, uint32_t down_quant,
+                                                    size_t n_ff, size_t n_embd, Floats input) {
+    std::vector<float> out(n_embd);
+    const int st = rnb_hip_dense_q4k_gelu_ffn(gate_weights.ptr, gate_weights.len, up_weights.ptr, up_weights.len,
+                                              down_weights.ptr, down_weights.len, down_quant, n_ff, n_embd, input.ptr,
+                                              input.len, out.data(), out.size());
+    if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
+    return make_ok(std::move(out));
 }
 
 // trait Backend { kind, capabilities, execute }, crates/rnb-backend/api/src/lib.rs:1281-1285

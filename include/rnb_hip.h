@@ -226,6 +226,18 @@ int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const
                                      const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
                                      size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
                                      size_t out_len);
+/* dense_q4k_gelu_ffn_batch, dense_api.rs:256-293: the same with the tanh form of GELU between the halves
+ * (crates/rnb-cpu/src/kernels/activation.rs:91-98); validation shared with the SiLU form (dense.rs:1712-1765, texts
+ * say "GELU") */
+int rnb_hip_dense_q4k_gelu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
+                                     size_t out_len);
+/* dense_q4k_gelu_ffn(gate, up, down, down_quant, n_ff, n_embd, input) -> Vec<f32>, dense_api.rs:182-254: one token;
+ * down in Q4_K, Q5_K or Q6_K (validation order and texts :191-232) */
+int rnb_hip_dense_q4k_gelu_ffn(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                               const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                               size_t n_embd, const float *x, size_t x_len, float *out, size_t out_len);
 /* device-resident form (the reference's dev-input chain, dense.rs:2189-2219); also accepts one token */
 int rnb_hip_dense_q4k_silu_ffn_dev(const void *gate_dev, const void *up_dev, const void *down_dev,
                                    uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq_len,

@@ -69,8 +69,9 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes = [u32, vp, sz, sz, vp, sz, vp, i32]
         L.rnbo_gemv_q8_0_f32act.restype = i32
         L.rnbo_gemv_q8_0_f32act.argtypes = [vp, sz, sz, vp, sz, vp, i32]
-        L.rnbo_silu_mul_inplace.restype = None
-        L.rnbo_silu_mul_inplace.argtypes = [vp, vp, sz]
+        for name in ("rnbo_silu_mul_inplace", "rnbo_gelu_mul_inplace"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [vp, vp, sz]
         L.rnbo_route_topk.restype = sz
         L.rnbo_route_topk.argtypes = [vp, sz, sz, vp, vp]
         L.rnbo_moe_sparse_experts_by_token.restype = i32
@@ -227,6 +228,20 @@ def silu_mul(gate, up) -> np.ndarray:
     g, u = _f32(gate).copy(), _f32(up)
     lib().rnbo_silu_mul_inplace(_p(g), _p(u), g.size)
     return g
+
+
+def gelu_mul(gate, up) -> np.ndarray:
+    g, u = _f32(gate).copy(), _f32(up)
+    lib().rnbo_gelu_mul_inplace(_p(g), _p(u), g.size)
+    return g
+
+
+def dense_gelu_ffn(gate, up, down, down_quant: int, n_ff: int, n_embd: int, x) -> np.ndarray:
+    """As dense_silu_ffn with crates/rnb-cpu/src/kernels/activation.rs:91-98 (fused_gelu_mul) between the halves."""
+    g = gemv(Q4_K, gate, n_ff, n_embd, x)
+    u = gemv(Q4_K, up, n_ff, n_embd, x)
+    mid = gelu_mul(g.ravel(), u.ravel()).reshape(g.shape)
+    return gemv(down_quant, down, n_embd, n_ff, mid)
 
 
 def dense_silu_ffn(gate, up, down, down_quant: int, n_ff: int, n_embd: int, x) -> np.ndarray:

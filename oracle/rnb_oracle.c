@@ -31,6 +31,8 @@
  *   dot_q6k_q8k                 f64 numpy dequant identity; bsums identity (avx2_dot.rs:824,880)
  *   dot_q8_0_*                  reference vector 528.0 (quant_gemv.rs:1448-1464), numpy identity
  *   gemv drivers                seq-major layout vector (quant_gemv.rs:1448-1464)
+ *   gelu_mul_inplace            reference vector (activation.rs:166-173: gate [1, -1], up [2, 3] -> 1.6824, -0.4764)
+ *                               + f64 numpy statement of the tanh form
  *   route_topk                  reference vectors (routing.rs:272-318)
  *   moe_sparse_experts_by_token f32-dequant statement of the reference's CUDA test oracle
  *                               (cuda tests.rs:29561-29584) to activation-quant noise; composition
@@ -876,6 +878,26 @@ void rnbo_silu_mul_inplace(float *gate, const float *up, size_t n) {
         volatile float den = 1.0f + e;
         volatile float s = g / den;
         volatile float r = s * up[i];
+        gate[i] = r;
+    }
+}
+
+/* crates/rnb-cpu/src/kernels/activation.rs:91-98 (fused_gelu_mul_inplace): tanh form,
+ * 0.5 * g * (1 + tanh(sqrt(2/pi) * (g + 0.044715 * g^3))) * up, every step rounded to f32 */
+void rnbo_gelu_mul_inplace(float *gate, const float *up, size_t n) {
+    const float sqrt_2_over_pi = sqrtf(2.0f / 3.14159265358979323846f);
+    for (size_t i = 0; i < n; i++) {
+        float g = gate[i];
+        volatile float g2 = g * g;
+        volatile float g3 = g2 * g;
+        volatile float c = 0.044715f * g3;
+        volatile float inner = g + c;
+        volatile float arg = sqrt_2_over_pi * inner;
+        volatile float t = tanhf(arg);
+        volatile float one = 1.0f + t;
+        volatile float half = 0.5f * g;
+        volatile float act = half * one;
+        volatile float r = act * up[i];
         gate[i] = r;
     }
 }

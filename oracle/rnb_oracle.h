@@ -98,6 +98,7 @@ int rnbo_gemv_q8_0_f32act(const uint8_t *w, size_t rows, size_t cols, const floa
 
 /* ---- MoE ------------------------------------------------------------------------ */
 void rnbo_silu_mul_inplace(float *gate, const float *up, size_t n);
+void rnbo_gelu_mul_inplace(float *gate, const float *up, size_t n);
 size_t rnbo_route_topk(const float *logits, size_t n_expert, size_t k, uint32_t *idx_out,
                        float *weights_out);
 int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_all,

@@ -73,6 +73,8 @@ from .binding import (  # noqa: F401
     q6k_gemv_into,
     q6k_gemv_argmax,
     dense_q4k_attention_qkv,
+    dense_q4k_gelu_ffn,
+    dense_q4k_gelu_ffn_batch,
     q8_0_gemv_argmax,
     q8_0_gemv,
     q8_0_gemv_batch,

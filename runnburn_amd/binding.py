@@ -68,6 +68,8 @@ SYMBOLS = [
     ("rnb_hip_dense_q4k_attention_qkv", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_q8_0_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
+    ("rnb_hip_dense_q4k_gelu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
+    ("rnb_hip_dense_q4k_gelu_ffn", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_silu_ffn_dev", _i, [_vp, _vp, _vp, _u32, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gguf_open", _i, [C.c_char_p, C.POINTER(_vp)]),
     ("rnb_hip_gguf_parse", _i, [_vp, _sz, C.POINTER(_vp)]),
@@ -479,6 +481,28 @@ def dense_q4k_silu_ffn_batch(gate_weights, up_weights, down_weights, down_quant:
     out = np.empty((seq_len, n_embd), dtype=np.float32)
     _check(lib().rnb_hip_dense_q4k_silu_ffn_batch(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, down_quant, n_ff,
                                                   n_embd, seq_len, _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+def dense_q4k_gelu_ffn_batch(gate_weights, up_weights, down_weights, down_quant: int, n_ff: int, n_embd: int,
+                             seq_len: int, input) -> np.ndarray:  # noqa: A002
+    """api/dense_api.rs:256-293; returns out[seq_len][n_embd]."""
+    g, u, d = _bytes_view(gate_weights), _bytes_view(up_weights), _bytes_view(down_weights)
+    x = _f32(input).ravel()
+    out = np.empty((seq_len, n_embd), dtype=np.float32)
+    _check(lib().rnb_hip_dense_q4k_gelu_ffn_batch(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, down_quant, n_ff,
+                                                  n_embd, seq_len, _ptr(x), x.size, _ptr(out), out.size))
+    return out
+
+
+def dense_q4k_gelu_ffn(gate_weights, up_weights, down_weights, down_quant: int, n_ff: int, n_embd: int,
+                       input) -> np.ndarray:  # noqa: A002
+    """api/dense_api.rs:182-254: one token; returns out[n_embd]."""
+    g, u, d = _bytes_view(gate_weights), _bytes_view(up_weights), _bytes_view(down_weights)
+    x = _f32(input).ravel()
+    out = np.empty(n_embd, dtype=np.float32)
+    _check(lib().rnb_hip_dense_q4k_gelu_ffn(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, down_quant, n_ff, n_embd,
+                                            _ptr(x), x.size, _ptr(out), out.size))
     return out
 
 

@@ -204,21 +204,22 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
     return RNB_HIP_OK;
 }
 
-// ---- dense SwiGLU FFN -------------------------------------------------------------------------
-// out[s] = W_down . Q(silu(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), the composition the reference runs per token
-// on the CPU (gate/up GEMV, fused_silu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K, Q8_0 or Q5_1.
+// ---- dense gated FFN --------------------------------------------------------------------------
+// out[s] = W_down . Q(act(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), act = SiLU or GELU: the composition the reference
+// runs per token on the CPU (gate/up GEMV, fused_silu_mul / fused_gelu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K, Q8_0 or Q5_1.
 
 // Validation order and messages: crates/rnb-backend/cuda/src/runtime/dense.rs:1712-1765.
 int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd,
-                       size_t seq, size_t x_len, bool batch_entry) {
+                       size_t seq, size_t x_len, bool batch_entry, bool gelu = false) {
+    const std::string name = gelu ? "dense GELU FFN" : "dense SiLU FFN";
     if (batch_entry && seq <= 1)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch requires seq_len > 1, got " + std::to_string(seq));
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch requires seq_len > 1, got " + std::to_string(seq));
     if (x_len != seq * n_embd)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch input length mismatch: got " + std::to_string(x_len) +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch input length mismatch: got " + std::to_string(x_len) +
                                                  ", expected " + std::to_string(seq * n_embd));
     const size_t down_block = (down_quant == 7 || down_quant == 8) ? 32 : 256;
     if (n_embd % 256 != 0 || n_ff % down_block != 0)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch dims must align to gate/down blocks, got n_ff=" +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch dims must align to gate/down blocks, got n_ff=" +
                                                  std::to_string(n_ff) + " down_block=" + std::to_string(down_block) +
                                                  " n_embd=" + std::to_string(n_embd));
     size_t down_row_bytes = 0;
@@ -230,25 +231,26 @@ int validate_dense_ffn(size_t gate_len, size_t up_len, size_t down_len, uint32_t
         case 14: down_row_bytes = n_ff / 256 * 210; break;
         default:
             return fail(RNB_HIP_INVALID_REQUEST,
-                        "unsupported dense SiLU FFN batch down quant code " + std::to_string(down_quant));
+                        "unsupported " + name + " batch down quant code " + std::to_string(down_quant));
     }
     const size_t gate_bytes = n_ff * (n_embd / 256) * 144;
     if (gate_len != gate_bytes)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch gate byte mismatch: got " + std::to_string(gate_len) +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch gate byte mismatch: got " + std::to_string(gate_len) +
                                                  ", expected " + std::to_string(gate_bytes));
     if (up_len != gate_bytes)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch up byte mismatch: got " + std::to_string(up_len) +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch up byte mismatch: got " + std::to_string(up_len) +
                                                  ", expected " + std::to_string(gate_bytes));
     if (down_len != n_embd * down_row_bytes)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch down byte mismatch: got " + std::to_string(down_len) +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch down byte mismatch: got " + std::to_string(down_len) +
                                                  ", expected " + std::to_string(n_embd * down_row_bytes));
     if (n_ff > 0x7fffffffu || n_embd > 0x7fffffffu || seq > 65535u)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN shape out of range");
+        return fail(RNB_HIP_INVALID_REQUEST, name + " shape out of range");
     return RNB_HIP_OK;
 }
 
 int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev,
-                      uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq, const float *x_dev, float *out_dev) {
+                      uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq, const float *x_dev, float *out_dev,
+                      bool gelu = false) {
     const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
     HIP_TRY(s.ffn_mid.reserve(mid_bytes));
     ActView act;
@@ -257,7 +259,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
     const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
     if (seq < kGemmMinSeq && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in))) {
         launch_gemv_q4k_gate_up(gate_dev, up_dev, act, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
-                                static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), s.stream);
+                                static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), gelu, s.stream);
     } else {
         HIP_TRY(s.ffn_gate.reserve(mid_bytes));
         HIP_TRY(s.ffn_up.reserve(mid_bytes));
@@ -265,7 +267,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         if (st != RNB_HIP_OK) return st;
         st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>());
         if (st != RNB_HIP_OK) return st;
-        launch_silu_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, s.stream);
+        launch_act_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, gelu, s.stream);
     }
     HIP_TRY(hipGetLastError());
     // the intermediate is re-quantised in the form the down projection's rows take, then the down matmul runs
@@ -862,16 +864,19 @@ int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint
     return RNB_HIP_OK;
 }
 
-int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
-                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
-                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
-                                     size_t out_len) {
-    int st = validate_dense_ffn(gate_len, up_len, down_len, down_quant, n_ff, n_embd, seq_len, x_len, true);
-    if (st != RNB_HIP_OK) return st;
+}  // extern "C"
+
+namespace {
+
+// host-pointer gated FFN after validation: residency, staging, the device sequence, the copy back
+int dense_ffn_host(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len, const uint8_t *down,
+                   size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq_len, const float *x,
+                   float *out, size_t out_len, bool gelu) {
+    const std::string name = gelu ? "dense GELU FFN" : "dense SiLU FFN";
     if (out_len < seq_len * n_embd)
-        return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN batch output length mismatch: got " + std::to_string(out_len) +
+        return fail(RNB_HIP_INVALID_REQUEST, name + " batch output length mismatch: got " + std::to_string(out_len) +
                                                  ", expected at least " + std::to_string(seq_len * n_embd));
-    if (!gate || !up || !down || !x || !out) return fail(RNB_HIP_INVALID_REQUEST, "dense SiLU FFN null pointer argument");
+    if (!gate || !up || !down || !x || !out) return fail(RNB_HIP_INVALID_REQUEST, name + " null pointer argument");
     Guard g;
     if (!g.state) return g.status;
     State &s = *g.state;
@@ -887,14 +892,71 @@ int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const
     std::memcpy(s.bounce_in.ptr, x, io_bytes);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, io_bytes, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += io_bytes;
-    st = run_dense_ffn_dev(s, gate_dev, up_dev, down_dev, down_quant, n_ff, n_embd, seq_len, s.x_f32.as<float>(),
-                           s.out_f32.as<float>());
+    int st = run_dense_ffn_dev(s, gate_dev, up_dev, down_dev, down_quant, n_ff, n_embd, seq_len, s.x_f32.as<float>(),
+                               s.out_f32.as<float>(), gelu);
     if (st != RNB_HIP_OK) return st;
     HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, io_bytes, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipStreamSynchronize(s.stream));
     s.d2h_bytes += io_bytes;
     std::memcpy(out, s.bounce_out.ptr, io_bytes);
     return RNB_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rnb_hip_dense_q4k_silu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
+                                     size_t out_len) {
+    int st = validate_dense_ffn(gate_len, up_len, down_len, down_quant, n_ff, n_embd, seq_len, x_len, true);
+    if (st != RNB_HIP_OK) return st;
+    return dense_ffn_host(gate, gate_len, up, up_len, down, down_len, down_quant, n_ff, n_embd, seq_len, x, out, out_len,
+                          false);
+}
+
+int rnb_hip_dense_q4k_gelu_ffn_batch(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len,
+                                     const uint8_t *down, size_t down_len, uint32_t down_quant, size_t n_ff,
+                                     size_t n_embd, size_t seq_len, const float *x, size_t x_len, float *out,
+                                     size_t out_len) {
+    int st = validate_dense_ffn(gate_len, up_len, down_len, down_quant, n_ff, n_embd, seq_len, x_len, true, true);
+    if (st != RNB_HIP_OK) return st;
+    return dense_ffn_host(gate, gate_len, up, up_len, down, down_len, down_quant, n_ff, n_embd, seq_len, x, out, out_len,
+                          true);
+}
+
+int rnb_hip_dense_q4k_gelu_ffn(const uint8_t *gate, size_t gate_len, const uint8_t *up, size_t up_len, const uint8_t *down,
+                               size_t down_len, uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x,
+                               size_t x_len, float *out, size_t out_len) {
+    // validation order and texts: crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:191-232
+    if (x_len != n_embd)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN input length mismatch: got " + std::to_string(x_len) +
+                                                 ", expected " + std::to_string(n_embd));
+    if (n_embd % 256 != 0 || n_ff % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN dims must be divisible by 256, got n_ff=" +
+                                                 std::to_string(n_ff) + " n_embd=" + std::to_string(n_embd));
+    size_t down_row_bytes = 0;
+    switch (down_quant) {
+        case 12: down_row_bytes = n_ff / 256 * 144; break;
+        case 13: down_row_bytes = n_ff / 256 * 176; break;
+        case 14: down_row_bytes = n_ff / 256 * 210; break;
+        default:
+            return fail(RNB_HIP_INVALID_REQUEST, "unsupported dense GELU FFN down quant code " + std::to_string(down_quant));
+    }
+    const size_t gate_bytes = n_ff * (n_embd / 256) * 144;
+    if (gate_len != gate_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN gate byte mismatch: got " + std::to_string(gate_len) +
+                                                 ", expected " + std::to_string(gate_bytes));
+    if (up_len != gate_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN up byte mismatch: got " + std::to_string(up_len) +
+                                                 ", expected " + std::to_string(gate_bytes));
+    if (down_len != n_embd * down_row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN down byte mismatch: got " + std::to_string(down_len) +
+                                                 ", expected " + std::to_string(n_embd * down_row_bytes));
+    if (n_ff > 0x7fffffffu || n_embd > 0x7fffffffu) return fail(RNB_HIP_INVALID_REQUEST, "dense GELU FFN shape out of range");
+    if (n_embd == 0) return RNB_HIP_OK;
+    return dense_ffn_host(gate, gate_len, up, up_len, down, down_len, down_quant, n_ff, n_embd, 1, x, out, out_len, true);
 }
 
 int rnb_hip_dense_q4k_silu_ffn_dev(const void *gate_dev, const void *up_dev, const void *down_dev, uint32_t down_quant,

@@ -50,6 +50,19 @@ __device__ __forceinline__ void lds_fill4(const uint8_t *base, uint32_t lane_off
 }
 __device__ __forceinline__ void wait_fills() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// gate activation times up, as crates/rnb-cpu/src/kernels/activation.rs:73-98: SiLU g / (1 + exp(-g)) or the tanh form
+// of GELU, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+template <bool kGelu>
+__device__ __forceinline__ float act_mul(float g, float up) {
+    if constexpr (kGelu) {
+        const float inner = g + 0.044715f * (g * g * g);
+        return (0.5f * g) * (1.0f + tanhf(0.7978845608028654f * inner)) * up;
+    } else {
+        const float e = expf(-g);
+        return (g / (1.0f + e)) * up;
+    }
+}
+
 // Cross-lane sums on the DPP data path (no LDS traffic).  After seg_sum<W>(v) the LAST lane of every
 // aligned W-lane segment (W = 16, 32 or 64) holds the sum over that segment.
 template <int kCtrl, int kRowMask>

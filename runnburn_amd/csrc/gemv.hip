@@ -85,12 +85,11 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
-// SwiGLU front half for decode-sized batches: mid[s][r] = silu(Wg[r] . a_s) * (Wu[r] . a_s) with one launch.  Same lane
+// Gated-FFN front half for decode-sized batches: mid[s][r] = act(Wg[r] . a_s) * (Wu[r] . a_s) with one launch (act = SiLU or GELU).  Same lane
 // mapping as gemv_kquant_kernel (rows of at most 16 super-blocks); a wave fetches row r of BOTH matrices against the
 // one activation slice it holds, so the activation is loaded once and gate/up never travel through memory.
-// SiLU as crates/rnb-cpu/src/kernels/activation.rs:73-89: (g / (1 + exp(-g))) * up.
 // ---------------------------------------------------------------------------------------------
-template <int kRowsPerWave>
+template <int kRowsPerWave, bool kGelu>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_q4k_gate_up_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ abs,
@@ -119,21 +118,22 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         }
         gs = seg_sum<kLanesPerRow>(gs);
         us = seg_sum<kLanesPerRow>(us);
-        if (sub == kLanesPerRow - 1 && row < rows) {
-            const float e = expf(-gs);
-            mid[static_cast<size_t>(tok) * rows + row] = (gs / (1.0f + e)) * us;
-        }
+        if (sub == kLanesPerRow - 1 && row < rows) mid[static_cast<size_t>(tok) * rows + row] = act_mul<kGelu>(gs, us);
     }
 }
 
 template <int kRowsPerWave>
 void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
-                    uint32_t seq, hipStream_t stream) {
+                    uint32_t seq, bool gelu, hipStream_t stream) {
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
-    hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu, act.qs,
-                       act.d, act.bsums, mid, rows, nb, row_groups);
+    if (gelu)
+        hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, true>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu,
+                           act.qs, act.d, act.bsums, mid, rows, nb, row_groups);
+    else
+        hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, false>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu,
+                           act.qs, act.d, act.bsums, mid, rows, nb, row_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -189,14 +189,12 @@ void launch_multi(const MultiMat &mats, ActView act, float *out, uint32_t nb, hi
                        act.bsums, out, nb, row_groups);
 }
 
-__global__ void __launch_bounds__(256) silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
-                                                      float *__restrict__ out, size_t n) {
+template <bool kGelu>
+__global__ void __launch_bounds__(256) act_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up,
+                                                     float *__restrict__ out, size_t n) {
     for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
-         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
-        const float gs = gate[i];
-        const float e = expf(-gs);
-        out[i] = (gs / (1.0f + e)) * up[i];
-    }
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        out[i] = act_mul<kGelu>(gate[i], up[i]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -472,14 +470,14 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 bool gemv_q4k_gate_up_supported(uint32_t nb) { return nb >= 1 && nb <= 16; }
 
 void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
-                             uint32_t seq, hipStream_t stream) {
+                             uint32_t seq, bool gelu, hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
     if (nb <= 4)
-        launch_gate_up<4>(wg, wu, act, mid, rows, nb, seq, stream);
+        launch_gate_up<4>(wg, wu, act, mid, rows, nb, seq, gelu, stream);
     else if (nb <= 8)
-        launch_gate_up<2>(wg, wu, act, mid, rows, nb, seq, stream);
+        launch_gate_up<2>(wg, wu, act, mid, rows, nb, seq, gelu, stream);
     else
-        launch_gate_up<1>(wg, wu, act, mid, rows, nb, seq, stream);
+        launch_gate_up<1>(wg, wu, act, mid, rows, nb, seq, gelu, stream);
 }
 
 void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], ActView act, float *out, uint32_t nb,
@@ -500,11 +498,14 @@ void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], Ac
         launch_multi<1>(mats, act, out, nb, stream);
 }
 
-void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream) {
+void launch_act_mul(const float *gate, const float *up, float *out, size_t n, bool gelu, hipStream_t stream) {
     if (n == 0) return;
     const size_t blocks = (n + 255) / 256;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
-                       gate, up, out, n);
+    const dim3 grid(static_cast<unsigned>(blocks < 4096 ? blocks : 4096));
+    if (gelu)
+        hipLaunchKernelGGL(act_mul_kernel<true>, grid, dim3(256), 0, stream, gate, up, out, n);
+    else
+        hipLaunchKernelGGL(act_mul_kernel<false>, grid, dim3(256), 0, stream, gate, up, out, n);
 }
 
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,

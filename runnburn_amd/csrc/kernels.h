@@ -49,10 +49,11 @@ void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, 
 void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
                          uint32_t seq, hipStream_t stream);
 
-// SwiGLU front half, rows of at most 16 super-blocks: mid[s*rows + r] = silu(Wg[r] . a_s) * (Wu[r] . a_s)
+// gated-FFN front half, rows of at most 16 super-blocks: mid[s*rows + r] = act(Wg[r] . a_s) * (Wu[r] . a_s),
+// act = SiLU or (gelu) the tanh form of GELU
 bool gemv_q4k_gate_up_supported(uint32_t nb);
 void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mid, uint32_t rows, uint32_t nb,
-                             uint32_t seq, hipStream_t stream);
+                             uint32_t seq, bool gelu, hipStream_t stream);
 // up to three Q4_K matrices of nb super-blocks per row against one activation (token 0 of `act`), one launch;
 // out = [rows[0] results | rows[1] results | rows[2] results]
 void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], ActView act, float *out, uint32_t nb,
@@ -60,8 +61,8 @@ void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], Ac
 // arg-max of `len` f32 (ties to the lower index); scratch_* hold 256 entries each, the result lands in out_*[0]
 void launch_argmax(const float *values, uint32_t len, float *scratch_values, uint32_t *scratch_indices, float *out_value,
                    uint32_t *out_index, hipStream_t stream);
-// out[i] = silu(gate[i]) * up[i]
-void launch_silu_mul(const float *gate, const float *up, float *out, size_t n, hipStream_t stream);
+// out[i] = act(gate[i]) * up[i]
+void launch_act_mul(const float *gate, const float *up, float *out, size_t n, bool gelu, hipStream_t stream);
 
 // Multi-token matmul on the vector ALUs for Q2_K ... Q6_K (weights decoded once per eight staged tokens);
 // same output contract as launch_gemv_q4k

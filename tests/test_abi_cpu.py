@@ -109,6 +109,30 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q8_0 input length mismatch: got 33, expected 32"
 
 
+def test_dense_gelu_ffn_validation_messages():
+    """crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:191-232 (one token) and dense.rs:1712-1765 with "GELU"."""
+    z = np.zeros
+    g = z(256 * 144, np.uint8)
+    f = rnb.dense_q4k_gelu_ffn
+    e = _err(f, g, g, z(256 * 210, np.uint8), 14, 256, 256, z(255, np.float32))
+    assert str(e) == "dense GELU FFN input length mismatch: got 255, expected 256"
+    e = _err(f, g, g, z(256 * 210, np.uint8), 14, 250, 256, z(256, np.float32))
+    assert str(e) == "dense GELU FFN dims must be divisible by 256, got n_ff=250 n_embd=256"
+    e = _err(f, g, g, z(256 * 8 * 34, np.uint8), 8, 256, 256, z(256, np.float32))
+    assert str(e) == "unsupported dense GELU FFN down quant code 8"
+    e = _err(f, g[:-1], g, z(256 * 210, np.uint8), 14, 256, 256, z(256, np.float32))
+    assert str(e) == "dense GELU FFN gate byte mismatch: got 36863, expected 36864"
+    e = _err(f, g, g, z(256 * 176 + 2, np.uint8), 13, 256, 256, z(256, np.float32))
+    assert str(e) == "dense GELU FFN down byte mismatch: got 45058, expected 45056"
+    fb = rnb.dense_q4k_gelu_ffn_batch
+    e = _err(fb, g, g, z(256 * 210, np.uint8), 14, 256, 256, 1, z(256, np.float32))
+    assert str(e) == "dense GELU FFN batch requires seq_len > 1, got 1"
+    e = _err(fb, g, g, z(10, np.uint8), 2, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "unsupported dense GELU FFN batch down quant code 2"
+    e = _err(fb, g, g[:-2], z(256 * 210, np.uint8), 14, 256, 256, 2, z(512, np.float32))
+    assert str(e) == "dense GELU FFN batch up byte mismatch: got 36862, expected 36864"
+
+
 def test_dense_qkv_validation_messages():
     """crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:928-968"""
     z = np.zeros

@@ -584,6 +584,25 @@ def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
     check_close(got, ref, None, f"dense ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
 
 
+@pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("seq,n_ff,n_embd", [(1, 512, 256), (1, 1024, 4608), (3, 768, 512), (17, 512, 768)])
+def test_dense_gelu_ffn(rnb, oracle, down_quant, seq, n_ff, n_embd):
+    """crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:182-293: the tanh-form GELU between the halves; one token
+    through dense_q4k_gelu_ffn, more through the batch form (fused gate/up GEMV, long-row pair, MFMA GEMM routes)."""
+    gate = oracle.make_weights(Q4_K, n_ff, n_embd, 320 + seq)
+    up = oracle.make_weights(Q4_K, n_ff, n_embd, 321 + seq)
+    down = oracle.make_weights(down_quant, n_embd, n_ff, 322 + seq)
+    x = oracle.fill_normal(seq * n_embd, 323 + seq, 1.0)
+    ref = oracle.dense_gelu_ffn(gate, up, down, down_quant, n_ff, n_embd, x)
+    if seq == 1:
+        got = rnb.dense_q4k_gelu_ffn(gate, up, down, down_quant, n_ff, n_embd, x).reshape(1, n_embd)
+    else:
+        got = rnb.dense_q4k_gelu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
+    check_close(got, ref, None, f"gelu ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
+    # and it is not the SiLU result
+    assert not np.allclose(got, oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x), rtol=1e-3, atol=0)
+
+
 def test_dense_silu_ffn_dev_single_token_and_residency(rnb, oracle):
     n_ff, n_embd = 1024, 512
     gate = oracle.make_weights(Q4_K, n_ff, n_embd, 310)

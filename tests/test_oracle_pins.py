@@ -670,6 +670,18 @@ def test_silu_mul(oracle):
 
 # ---- MoE ------------------------------------------------------------------------------
 
+def test_gelu_mul_reference_vector_and_formula(oracle):
+    """crates/rnb-cpu/src/kernels/activation.rs:166-173: gate [1, -1], up [2, 3] -> 1.6824, -0.4764 (1e-3)."""
+    got = oracle.gelu_mul(np.array([1.0, -1.0], np.float32), np.array([2.0, 3.0], np.float32))
+    assert abs(got[0] - 1.6824) < 1e-3 and abs(got[1] + 0.4764) < 1e-3
+    g = (np.arange(2048) % 257).astype(np.float32) / np.float32(32.0) - np.float32(4.0)   # the inputs of activation.rs:181-186
+    u = (np.arange(2048) % 113).astype(np.float32) / np.float32(64.0) - np.float32(0.75)
+    g64 = g.astype(np.float64)
+    want = 0.5 * g64 * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (g64 + 0.044715 * g64 ** 3))) * u
+    assert np.allclose(oracle.gelu_mul(g, u), want, rtol=2e-6, atol=1e-7)
+    assert oracle.gelu_mul(np.zeros(3, np.float32), np.ones(3, np.float32)).tolist() == [0.0, 0.0, 0.0]
+
+
 def test_moe_matches_f32_dequant_statement(oracle):
     """The reference's CUDA-test oracle (crates/rnb-backend/cuda/src/runtime/tests.rs:29561-29584) is an
     f32-dequant statement of gate/up -> SiLU*up -> Q6_K down -> route-weighted sum; the integer path agrees
