@@ -16,6 +16,7 @@
 // (v_dot4_i32_i8); the per-block f32 scale is applied once per lane and the partial sums are added
 // across lanes on the DPP path, so results differ from the scalar reference only by f32 summation order.
 
+#include "act_quant.h"
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
@@ -82,6 +83,107 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// K-quant GEMV of ONE f32 token: the workgroup quantises the token to Q8_K itself into LDS (the same wave-level
+// quantiser as the stand-alone kernel, so the same bits), then runs the row loop of gemv_kquant_kernel against it.
+// Rows of at most 16 super-blocks.  Each lane requests its first rows' weight blocks before the quantisation starts,
+// so the weight stream is already in flight while the activation is prepared; the separate quantise launch and the
+// gap behind it disappear from a decode step.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFusedWaves = 8;   // waves per workgroup: each quantises 16 / 8 = 2 blocks of the token
+constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (more measured slower)
+constexpr uint32_t kFusedTargetWaves = 4096;
+
+template <uint32_t kQuant, int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kFusedWaves)
+    gemv_kquant_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
+                           uint32_t rows, uint32_t nb, uint32_t row_groups) {
+    using Q = KQuant<kQuant>;
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr size_t kBlockBytes = Q::kBytes;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[16 * 256];
+    __shared__ float s_d[16];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[16 * 16];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const bool has_block = bslot < nb;
+    const uint32_t tok = blockIdx.y;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t n_waves = gridDim.x * kFusedWaves;
+    uint32_t grp = blockIdx.x * kFusedWaves + wave;
+    uint32_t row = grp * kRowsPerWave + rsel;
+    // the activation is requested first: loads return in order, and the quantiser must not wait for weights
+    constexpr int kSpans = 16 / kFusedWaves;  // Q8_K blocks a wave quantises
+    float4 xv[kSpans];
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t blk = wave + i * kFusedWaves;
+        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x + (static_cast<size_t>(tok) * nb + blk) * 256)[lane];
+    }
+    // kDepth rows in flight per lane segment, the first ones requested before the quantisation starts
+    typename Q::Regs regs[kDepth];
+    bool live[kDepth];
+    auto fetch = [&](uint32_t group, bool *ok) {
+        const uint32_t r = group * kRowsPerWave + rsel;
+        *ok = has_block && group < row_groups && r < rows;
+        const size_t off = *ok ? static_cast<size_t>(r) * row_bytes + static_cast<size_t>(bslot) * kBlockBytes : 0;
+        return Q::load_block(w + off, g);  // rows >= 1 and nb >= 1: offset 0 is readable
+    };
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) regs[i] = fetch(grp + i * n_waves, &live[i]);
+
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t blk = wave + i * kFusedWaves;
+        if (blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+    }
+    __syncthreads();
+    const uint32_t ab = has_block ? bslot : 0;
+    const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
+
+    for (; grp < row_groups; grp += n_waves) {
+        row = grp * kRowsPerWave + rsel;
+        bool far_live;
+        const typename Q::Regs far = fetch(grp + kDepth * n_waves, &far_live);
+        float acc = live[0] ? kquant_partial<kQuant>(regs[0], a, g) : 0.0f;
+        acc = seg_sum<kLanesPerRow>(acc);
+        if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
+#pragma unroll
+        for (int i = 0; i + 1 < kDepth; i++) {
+            regs[i] = regs[i + 1];
+            live[i] = live[i + 1];
+        }
+        regs[kDepth - 1] = far;
+        live[kDepth - 1] = far_live;
+    }
+}
+
+template <uint32_t kQuant, int kRowsPerWave>
+void launch_kquant_f32(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                       hipStream_t stream) {
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kFusedTargetWaves ? row_groups : kFusedTargetWaves;
+    const dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, seq, 1);
+    hipLaunchKernelGGL((gemv_kquant_f32_kernel<kQuant, kRowsPerWave>), grid, dim3(kWave * kFusedWaves), 0, stream, w, x, out,
+                       rows, nb, row_groups);
+}
+
+template <uint32_t kQuant>
+void launch_kquant_f32_any(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                           hipStream_t stream) {
+    if (nb <= 4)
+        launch_kquant_f32<kQuant, 4>(w, x, out, rows, nb, seq, stream);
+    else if (nb <= 8)
+        launch_kquant_f32<kQuant, 2>(w, x, out, rows, nb, seq, stream);
+    else
+        launch_kquant_f32<kQuant, 1>(w, x, out, rows, nb, seq, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -465,6 +567,23 @@ void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *o
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                      hipStream_t stream) {
     launch_kquant_any<kQ6K>(w, act, out, rows, nb, seq, stream);
+}
+
+bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
+    const bool kq = quant == kQ2K || quant == kQ3K || quant == kQ4K || quant == kQ5K || quant == kQ6K;
+    return kq && nb >= 1 && nb <= 16 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
+                            uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    switch (quant) {
+    case kQ2K: launch_kquant_f32_any<kQ2K>(w, x, out, rows, nb, seq, stream); break;
+    case kQ3K: launch_kquant_f32_any<kQ3K>(w, x, out, rows, nb, seq, stream); break;
+    case kQ4K: launch_kquant_f32_any<kQ4K>(w, x, out, rows, nb, seq, stream); break;
+    case kQ5K: launch_kquant_f32_any<kQ5K>(w, x, out, rows, nb, seq, stream); break;
+    default: launch_kquant_f32_any<kQ6K>(w, x, out, rows, nb, seq, stream); break;
+    }
 }
 
 bool gemv_q4k_gate_up_supported(uint32_t nb) { return nb >= 1 && nb <= 16; }

@@ -41,6 +41,11 @@ void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 // Q2_K / Q3_K rows (84 / 110-byte blocks at 4- / 2-byte alignment); quant is kQ2K or kQ3K
 void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                          uint32_t seq, hipStream_t stream);
+// K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 16
+// super-blocks, x 16-byte aligned; same output contract as launch_gemv_q4k
+bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x);
+void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
+                            uint32_t seq, hipStream_t stream);
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,

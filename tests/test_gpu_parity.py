@@ -283,10 +283,14 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
 @pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q4_K, 77, 2048), (Q4_K, 50, 768), (Q6_K, 300, 4096),
                                              (Q6_K, 64, 768), (Q8_0, 200, 4096), (Q8_0, 33, 1056), (Q6_K, 40, 14336),
                                              (Q5_K, 300, 4096), (Q5_K, 41, 1280), (Q5_K, 24, 14336),
-                                             (Q2_K, 300, 4096), (Q2_K, 24, 14336), (Q3_K, 300, 4096), (Q3_K, 24, 14336)])
+                                             (Q2_K, 300, 4096), (Q2_K, 24, 14336), (Q3_K, 300, 4096), (Q3_K, 24, 14336),
+                                             (Q4_K, 5, 256), (Q4_K, 20001, 256), (Q6_K, 9001, 1024), (Q5_K, 4099, 4096),
+                                             (Q3_K, 8200, 2304)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
-    feed several matrices from one activation) run the same arithmetic: identical bits."""
+    feed several matrices from one activation) run the same arithmetic: identical bits.  For K-quant rows of at most
+    16 super-blocks gemv_dev is the one-launch kernel whose workgroups quantise the token themselves; the shapes cover
+    1, 2 and 4 rows per wave, row counts that are no multiple of those, and more row groups than waves."""
     w = oracle.make_weights(quant, rows, cols, 900 + rows)
     x = oracle.fill_normal(cols, 901 + cols, 1.0)
     wd, xd = rnb.DeviceBuffer.from_host(w), rnb.DeviceBuffer.from_host(x)
