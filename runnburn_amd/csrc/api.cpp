@@ -260,11 +260,21 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
                       bool gelu = false) {
     const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
     HIP_TRY(s.ffn_mid.reserve(mid_bytes));
-    ActView act;
-    int st = quantize_activations(s, kQ4K, x_dev, seq, n_embd, &act);
-    if (st != RNB_HIP_OK) return st;
     const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
-    if (seq < kGemmMinSeq && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in))) {
+    const bool small = seq < kGemmMinSeq && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
+    ActView act;
+    int st = RNB_HIP_OK;
+    if (small && seq == 1 && reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) {
+        // one token: one launch quantises it (per workgroup, in LDS) and makes act(gate) * up; with more tokens the
+        // repeated quantisation costs more than the launch it saves (measured)
+        launch_gemv_q4k_gate_up_f32(gate_dev, up_dev, x_dev, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
+                                    static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), gelu, s.stream);
+        HIP_TRY(hipGetLastError());
+        return run_matmul_dev(s, down_quant, down_dev, n_embd, n_ff, s.ffn_mid.as<float>(), seq, out_dev);
+    }
+    st = quantize_activations(s, kQ4K, x_dev, seq, n_embd, &act);
+    if (st != RNB_HIP_OK) return st;
+    if (small) {
         launch_gemv_q4k_gate_up(gate_dev, up_dev, act, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
                                 static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), gelu, s.stream);
     } else {
@@ -855,11 +865,16 @@ int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint
     std::memcpy(s.bounce_in.ptr, x, in_bytes);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += in_bytes;
-    ActView act;
-    int st = quantize_activations(s, kQ4K, s.x_f32.as<float>(), 1, n_embd, &act);  // once for the three projections
-    if (st != RNB_HIP_OK) return st;
     const uint32_t rows[3] = {static_cast<uint32_t>(q_rows), static_cast<uint32_t>(kv_rows), static_cast<uint32_t>(kv_rows)};
-    launch_gemv_q4k_multi(w_dev, rows, act, s.out_f32.as<float>(), static_cast<uint32_t>(n_embd / 256), s.stream);
+    if (n_embd / 256 <= 16) {  // the workgroups quantise the token themselves: one launch for the three projections
+        launch_gemv_q4k_multi_f32(w_dev, rows, s.x_f32.as<float>(), s.out_f32.as<float>(), static_cast<uint32_t>(n_embd / 256),
+                                  s.stream);
+    } else {
+        ActView act;
+        int st = quantize_activations(s, kQ4K, s.x_f32.as<float>(), 1, n_embd, &act);  // once for the three projections
+        if (st != RNB_HIP_OK) return st;
+        launch_gemv_q4k_multi(w_dev, rows, act, s.out_f32.as<float>(), static_cast<uint32_t>(n_embd / 256), s.stream);
+    }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipStreamSynchronize(s.stream));

@@ -95,6 +95,30 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 constexpr int kFusedWaves = 8;   // waves per workgroup: each quantises 16 / 8 = 2 blocks of the token
 constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (more measured slower)
 constexpr uint32_t kFusedTargetWaves = 4096;
+constexpr int kFusedSpans = 16 / kFusedWaves;  // Q8_K blocks of the token a wave quantises
+
+struct TokenSpans {
+    float4 v[kFusedSpans];
+};
+// wave `wave` of the workgroup requests blocks wave, wave + 8, ... of the token (four consecutive floats per lane)
+__device__ __forceinline__ void token_load(const float *__restrict__ x_tok, uint32_t nb, uint32_t wave, int lane,
+                                           TokenSpans &xv) {
+#pragma unroll
+    for (int i = 0; i < kFusedSpans; i++) {
+        const uint32_t blk = wave + i * kFusedWaves;
+        xv.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (blk < nb) xv.v[i] = reinterpret_cast<const float4 *>(x_tok + static_cast<size_t>(blk) * 256)[lane];
+    }
+}
+// ... and quantises them into the workgroup's LDS copy of the Q8_K token (qs[nb][256], d[nb], bsums[nb][16])
+__device__ __forceinline__ void token_quantize(const TokenSpans &xv, uint32_t nb, uint32_t wave, int lane, int8_t *s_qs,
+                                               float *s_d, int16_t *s_bsums) {
+#pragma unroll
+    for (int i = 0; i < kFusedSpans; i++) {
+        const uint32_t blk = wave + i * kFusedWaves;
+        if (blk < nb) q8k_quantize_vals(xv.v[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+    }
+}
 
 template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kFusedWaves)
@@ -119,14 +143,8 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     uint32_t grp = blockIdx.x * kFusedWaves + wave;
     uint32_t row = grp * kRowsPerWave + rsel;
     // the activation is requested first: loads return in order, and the quantiser must not wait for weights
-    constexpr int kSpans = 16 / kFusedWaves;  // Q8_K blocks a wave quantises
-    float4 xv[kSpans];
-#pragma unroll
-    for (int i = 0; i < kSpans; i++) {
-        const uint32_t blk = wave + i * kFusedWaves;
-        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x + (static_cast<size_t>(tok) * nb + blk) * 256)[lane];
-    }
+    TokenSpans xv;
+    token_load(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
     // kDepth rows in flight per lane segment, the first ones requested before the quantisation starts
     typename Q::Regs regs[kDepth];
     bool live[kDepth];
@@ -139,11 +157,7 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
 #pragma unroll
     for (int i = 0; i < kDepth; i++) regs[i] = fetch(grp + i * n_waves, &live[i]);
 
-#pragma unroll
-    for (int i = 0; i < kSpans; i++) {
-        const uint32_t blk = wave + i * kFusedWaves;
-        if (blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
-    }
+    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
     __syncthreads();
     const uint32_t ab = has_block ? bslot : 0;
     const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
@@ -238,6 +252,78 @@ void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mi
                            act.qs, act.d, act.bsums, mid, rows, nb, row_groups);
 }
 
+// The same front half straight from f32 tokens: the workgroup quantises token blockIdx.y to Q8_K in LDS as
+// gemv_kquant_f32_kernel does, with the first rows of both matrices already requested.
+template <int kRowsPerWave, bool kGelu>
+__global__ void __launch_bounds__(kWave *kFusedWaves)
+    gemv_q4k_gate_up_f32_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu, const float *__restrict__ x,
+                                float *__restrict__ mid, uint32_t rows, uint32_t nb, uint32_t row_groups) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[16 * 256];
+    __shared__ float s_d[16];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[16 * 16];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const bool has_block = bslot < nb;
+    const uint32_t tok = blockIdx.y;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    const uint32_t n_waves = gridDim.x * kFusedWaves;
+    uint32_t grp = blockIdx.x * kFusedWaves + wave;
+    TokenSpans xv;
+    token_load(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
+    auto offset_of = [&](uint32_t group, bool *ok) {
+        const uint32_t r = group * kRowsPerWave + rsel;
+        *ok = has_block && group < row_groups && r < rows;
+        return *ok ? static_cast<size_t>(r) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0;  // 0 is readable
+    };
+    bool live, next_live;
+    size_t off = offset_of(grp, &live);
+    Q4KRegs rg = q4k_load_block(wg + off, g), ru = q4k_load_block(wu + off, g);
+    off = offset_of(grp + n_waves, &next_live);
+    Q4KRegs ng = q4k_load_block(wg + off, g), nu = q4k_load_block(wu + off, g);
+
+    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    __syncthreads();
+    const uint32_t ab = has_block ? bslot : 0;
+    const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
+
+    for (; grp < row_groups; grp += n_waves) {
+        const uint32_t row = grp * kRowsPerWave + rsel;
+        bool far_live;
+        off = offset_of(grp + 2 * n_waves, &far_live);
+        const Q4KRegs fg = q4k_load_block(wg + off, g), fu = q4k_load_block(wu + off, g);
+        float gs = live ? q4k_partial(rg, a4, g) : 0.0f;
+        float us = live ? q4k_partial(ru, a4, g) : 0.0f;
+        gs = seg_sum<kLanesPerRow>(gs);
+        us = seg_sum<kLanesPerRow>(us);
+        if (sub == kLanesPerRow - 1 && row < rows) mid[static_cast<size_t>(tok) * rows + row] = act_mul<kGelu>(gs, us);
+        rg = ng;
+        ru = nu;
+        live = next_live;
+        ng = fg;
+        nu = fu;
+        next_live = far_live;
+    }
+}
+
+template <int kRowsPerWave>
+void launch_gate_up_f32(const uint8_t *wg, const uint8_t *wu, const float *x, float *mid, uint32_t rows, uint32_t nb,
+                        uint32_t seq, bool gelu, hipStream_t stream) {
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kFusedTargetWaves ? row_groups : kFusedTargetWaves;
+    const dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, seq, 1);
+    if (gelu)
+        hipLaunchKernelGGL((gemv_q4k_gate_up_f32_kernel<kRowsPerWave, true>), grid, dim3(kWave * kFusedWaves), 0, stream, wg,
+                           wu, x, mid, rows, nb, row_groups);
+    else
+        hipLaunchKernelGGL((gemv_q4k_gate_up_f32_kernel<kRowsPerWave, false>), grid, dim3(kWave * kFusedWaves), 0, stream, wg,
+                           wu, x, mid, rows, nb, row_groups);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Several Q4_K matrices against ONE quantised activation in one launch (the Q, K and V projections of a decode step:
 // crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:916-985): the rows of the matrices are numbered through, a
@@ -289,6 +375,71 @@ void launch_multi(const MultiMat &mats, ActView act, float *out, uint32_t nb, hi
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, 1, 1);
     hipLaunchKernelGGL((gemv_q4k_multi_kernel<kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, mats, act.qs, act.d,
                        act.bsums, out, nb, row_groups);
+}
+
+// The same straight from the f32 token (rows of at most 16 super-blocks): quantised by the workgroup in LDS.
+template <int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kFusedWaves)
+    gemv_q4k_multi_f32_kernel(MultiMat mats, const float *__restrict__ x, float *__restrict__ out, uint32_t nb,
+                              uint32_t row_groups) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[16 * 256];
+    __shared__ float s_d[16];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[16 * 16];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const bool has_block = bslot < nb;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    const uint32_t n_waves = gridDim.x * kFusedWaves;
+    const uint32_t rows = mats.end[2];
+    uint32_t grp = blockIdx.x * kFusedWaves + wave;
+    TokenSpans xv;
+    token_load(x, nb, wave, lane, xv);
+    auto fetch = [&](uint32_t group, bool *ok) {
+        const uint32_t r = group * kRowsPerWave + rsel;
+        *ok = has_block && group < row_groups && r < rows;
+        const int m = r < mats.end[0] ? 0 : (r < mats.end[1] ? 1 : 2);
+        const uint32_t local = r - (m == 0 ? 0u : mats.end[m - 1]);
+        // a dead lane reads the first block of the first matrix that has rows
+        const uint8_t *blk = *ok ? mats.w[m] + static_cast<size_t>(local) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes
+                                 : mats.w[mats.end[0] > 0 ? 0 : (mats.end[1] > mats.end[0] ? 1 : 2)];
+        return q4k_load_block(blk, g);
+    };
+    bool live, next_live;
+    Q4KRegs cur = fetch(grp, &live);
+    Q4KRegs nxt = fetch(grp + n_waves, &next_live);
+
+    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    __syncthreads();
+    const uint32_t ab = has_block ? bslot : 0;
+    const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
+
+    for (; grp < row_groups; grp += n_waves) {
+        const uint32_t row = grp * kRowsPerWave + rsel;
+        bool far_live;
+        const Q4KRegs far = fetch(grp + 2 * n_waves, &far_live);
+        float acc = live ? q4k_partial(cur, a4, g) : 0.0f;
+        acc = seg_sum<kLanesPerRow>(acc);
+        if (sub == kLanesPerRow - 1 && row < rows) out[row] = acc;
+        cur = nxt;
+        live = next_live;
+        nxt = far;
+        next_live = far_live;
+    }
+}
+
+template <int kRowsPerWave>
+void launch_multi_f32(const MultiMat &mats, const float *x, float *out, uint32_t nb, hipStream_t stream) {
+    const uint32_t rows = mats.end[2];
+    const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
+    const uint32_t waves = row_groups < kFusedTargetWaves ? row_groups : kFusedTargetWaves;
+    const dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, 1, 1);
+    hipLaunchKernelGGL((gemv_q4k_multi_f32_kernel<kRowsPerWave>), grid, dim3(kWave * kFusedWaves), 0, stream, mats, x, out, nb,
+                       row_groups);
 }
 
 template <bool kGelu>
@@ -597,6 +748,35 @@ void launch_gemv_q4k_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, 
         launch_gate_up<2>(wg, wu, act, mid, rows, nb, seq, gelu, stream);
     else
         launch_gate_up<1>(wg, wu, act, mid, rows, nb, seq, gelu, stream);
+}
+
+void launch_gemv_q4k_gate_up_f32(const uint8_t *wg, const uint8_t *wu, const float *x, float *mid, uint32_t rows,
+                                 uint32_t nb, uint32_t seq, bool gelu, hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    if (nb <= 4)
+        launch_gate_up_f32<4>(wg, wu, x, mid, rows, nb, seq, gelu, stream);
+    else if (nb <= 8)
+        launch_gate_up_f32<2>(wg, wu, x, mid, rows, nb, seq, gelu, stream);
+    else
+        launch_gate_up_f32<1>(wg, wu, x, mid, rows, nb, seq, gelu, stream);
+}
+
+void launch_gemv_q4k_multi_f32(const uint8_t *const w[3], const uint32_t rows[3], const float *x, float *out, uint32_t nb,
+                               hipStream_t stream) {
+    MultiMat mats;
+    uint32_t total = 0;
+    for (int i = 0; i < 3; i++) {
+        mats.w[i] = w[i];
+        total += rows[i];
+        mats.end[i] = total;
+    }
+    if (total == 0) return;
+    if (nb <= 4)
+        launch_multi_f32<4>(mats, x, out, nb, stream);
+    else if (nb <= 8)
+        launch_multi_f32<2>(mats, x, out, nb, stream);
+    else
+        launch_multi_f32<1>(mats, x, out, nb, stream);
 }
 
 void launch_gemv_q4k_multi(const uint8_t *const w[3], const uint32_t rows[3], ActView act, float *out, uint32_t nb,
