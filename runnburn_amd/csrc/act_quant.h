@@ -68,6 +68,33 @@ __device__ __forceinline__ void q8k_quantize_span(const float *__restrict__ x_bl
     q8k_quantize_vals(reinterpret_cast<const float4 *>(x_blk)[lane], lane, qs, d_out, bsums, digits);
 }
 
+// A workgroup of kWaves waves quantises one token of at most 16 Q8_K blocks into its LDS (qs[nb][256], d[nb],
+// bsums[nb][16]): wave `wave` takes blocks wave, wave + kWaves, ...  The loads are a call of their own so that a
+// kernel can request the token before its first weights and quantise after them.
+template <int kWaves>
+struct TokenSpans {
+    float4 v[16 / kWaves];
+};
+template <int kWaves>
+__device__ __forceinline__ void token_load(const float *__restrict__ x_tok, uint32_t nb, uint32_t wave, int lane,
+                                           TokenSpans<kWaves> &xv) {
+#pragma unroll
+    for (int i = 0; i < 16 / kWaves; i++) {
+        const uint32_t blk = wave + i * kWaves;
+        xv.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (blk < nb) xv.v[i] = reinterpret_cast<const float4 *>(x_tok + static_cast<size_t>(blk) * 256)[lane];
+    }
+}
+template <int kWaves>
+__device__ __forceinline__ void token_quantize(const TokenSpans<kWaves> &xv, uint32_t nb, uint32_t wave, int lane,
+                                               int8_t *s_qs, float *s_d, int16_t *s_bsums) {
+#pragma unroll
+    for (int i = 0; i < 16 / kWaves; i++) {
+        const uint32_t blk = wave + i * kWaves;
+        if (blk < nb) q8k_quantize_vals(xv.v[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+    }
+}
+
 // Quantises x_span[0..256) to eight 32-wide Q8 blocks (8 lanes per block); lanes whose block index
 // (lane / 8) is >= live_blocks neither read nor write.
 __device__ __forceinline__ float4 q8_load_span(const float *__restrict__ x_span, int lane, int live_blocks) {

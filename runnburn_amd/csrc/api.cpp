@@ -362,6 +362,21 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                 size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
                 const float *x_dev, float *out_dev) {
     if (token_count == 0) return RNB_HIP_OK;
+    if (token_count == 1 && moe_decode_supported(n_slots, sh.nb_in, sh.nb_mid, x_dev)) {
+        // decode: no host-side tables, two launches
+        MoeDecodeTable table;
+        table.n_slots = static_cast<uint32_t>(n_slots);
+        for (size_t i = 0; i < kMoeDecodeMaxSlots; i++) {
+            table.expert[i] = i < n_slots ? expert_ids[i] : 0;
+            table.route[i] = i < n_slots ? route[i] : 0.0f;
+        }
+        HIP_TRY(s.moe_mid.reserve(n_slots * n_ff * sizeof(float)));
+        launch_moe_decode(gate_dev, up_dev, down_dev, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
+                          static_cast<uint32_t>(n_ff), static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_in),
+                          static_cast<uint32_t>(sh.nb_mid), s.stream);
+        HIP_TRY(hipGetLastError());
+        return RNB_HIP_OK;
+    }
     // slots are grouped by expert, keeping slot order inside a group
     std::vector<uint32_t> order(n_slots);
     for (size_t i = 0; i < n_slots; i++) order[i] = static_cast<uint32_t>(i);

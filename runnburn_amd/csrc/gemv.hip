@@ -95,31 +95,6 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 constexpr int kFusedWaves = 8;   // waves per workgroup: each quantises 16 / 8 = 2 blocks of the token
 constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (more measured slower)
 constexpr uint32_t kFusedTargetWaves = 4096;
-constexpr int kFusedSpans = 16 / kFusedWaves;  // Q8_K blocks of the token a wave quantises
-
-struct TokenSpans {
-    float4 v[kFusedSpans];
-};
-// wave `wave` of the workgroup requests blocks wave, wave + 8, ... of the token (four consecutive floats per lane)
-__device__ __forceinline__ void token_load(const float *__restrict__ x_tok, uint32_t nb, uint32_t wave, int lane,
-                                           TokenSpans &xv) {
-#pragma unroll
-    for (int i = 0; i < kFusedSpans; i++) {
-        const uint32_t blk = wave + i * kFusedWaves;
-        xv.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (blk < nb) xv.v[i] = reinterpret_cast<const float4 *>(x_tok + static_cast<size_t>(blk) * 256)[lane];
-    }
-}
-// ... and quantises them into the workgroup's LDS copy of the Q8_K token (qs[nb][256], d[nb], bsums[nb][16])
-__device__ __forceinline__ void token_quantize(const TokenSpans &xv, uint32_t nb, uint32_t wave, int lane, int8_t *s_qs,
-                                               float *s_d, int16_t *s_bsums) {
-#pragma unroll
-    for (int i = 0; i < kFusedSpans; i++) {
-        const uint32_t blk = wave + i * kFusedWaves;
-        if (blk < nb) q8k_quantize_vals(xv.v[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
-    }
-}
-
 template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kFusedWaves)
     gemv_kquant_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
@@ -143,8 +118,8 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     uint32_t grp = blockIdx.x * kFusedWaves + wave;
     uint32_t row = grp * kRowsPerWave + rsel;
     // the activation is requested first: loads return in order, and the quantiser must not wait for weights
-    TokenSpans xv;
-    token_load(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
+    TokenSpans<kFusedWaves> xv;
+    token_load<kFusedWaves>(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
     // kDepth rows in flight per lane segment, the first ones requested before the quantisation starts
     typename Q::Regs regs[kDepth];
     bool live[kDepth];
@@ -157,7 +132,7 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
 #pragma unroll
     for (int i = 0; i < kDepth; i++) regs[i] = fetch(grp + i * n_waves, &live[i]);
 
-    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    token_quantize<kFusedWaves>(xv, nb, wave, lane, s_qs, s_d, s_bsums);
     __syncthreads();
     const uint32_t ab = has_block ? bslot : 0;
     const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
@@ -273,8 +248,8 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
     const uint32_t n_waves = gridDim.x * kFusedWaves;
     uint32_t grp = blockIdx.x * kFusedWaves + wave;
-    TokenSpans xv;
-    token_load(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
+    TokenSpans<kFusedWaves> xv;
+    token_load<kFusedWaves>(x + static_cast<size_t>(tok) * nb * 256, nb, wave, lane, xv);
     auto offset_of = [&](uint32_t group, bool *ok) {
         const uint32_t r = group * kRowsPerWave + rsel;
         *ok = has_block && group < row_groups && r < rows;
@@ -286,7 +261,7 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     off = offset_of(grp + n_waves, &next_live);
     Q4KRegs ng = q4k_load_block(wg + off, g), nu = q4k_load_block(wu + off, g);
 
-    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    token_quantize<kFusedWaves>(xv, nb, wave, lane, s_qs, s_d, s_bsums);
     __syncthreads();
     const uint32_t ab = has_block ? bslot : 0;
     const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
@@ -397,8 +372,8 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     const uint32_t n_waves = gridDim.x * kFusedWaves;
     const uint32_t rows = mats.end[2];
     uint32_t grp = blockIdx.x * kFusedWaves + wave;
-    TokenSpans xv;
-    token_load(x, nb, wave, lane, xv);
+    TokenSpans<kFusedWaves> xv;
+    token_load<kFusedWaves>(x, nb, wave, lane, xv);
     auto fetch = [&](uint32_t group, bool *ok) {
         const uint32_t r = group * kRowsPerWave + rsel;
         *ok = has_block && group < row_groups && r < rows;
@@ -413,7 +388,7 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     Q4KRegs cur = fetch(grp, &live);
     Q4KRegs nxt = fetch(grp + n_waves, &next_live);
 
-    token_quantize(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    token_quantize<kFusedWaves>(xv, nb, wave, lane, s_qs, s_d, s_bsums);
     __syncthreads();
     const uint32_t ab = has_block ? bslot : 0;
     const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);

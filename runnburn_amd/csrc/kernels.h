@@ -113,6 +113,18 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
 void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
                            const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
                            uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
+// One token, at most 16 slots: the whole expert step in two launches, the routing table as a kernel argument (x f32
+// [n_embd] 16-byte aligned, mid scratch [n_slots][n_ff], out [n_embd]); the same bits as the general sequence
+constexpr uint32_t kMoeDecodeMaxSlots = 16;
+struct MoeDecodeTable {
+    uint32_t n_slots;
+    uint32_t expert[kMoeDecodeMaxSlots];
+    float route[kMoeDecodeMaxSlots];
+};
+bool moe_decode_supported(size_t n_slots, size_t nb_in, size_t nb_mid, const void *x);
+void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
+                       const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
+                       uint32_t nb_in, uint32_t nb_mid, hipStream_t stream);
 // out[token][n_embd] = sum of slot_out over the token's slots, in list order;
 // tok_offsets [token_count+1], tok_slots [n_slots] (CSR built by the host)
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,

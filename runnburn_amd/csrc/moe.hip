@@ -12,6 +12,7 @@
 // tokens in LDS, then every wave keeps a row's packed blocks in registers and walks the tokens, so
 // an expert's weights are streamed from HBM once however many tokens were routed to it.  A decode
 // call (one token) is the same kernel with one token per group.
+#include "act_quant.h"
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
@@ -321,6 +322,122 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     if (lane == 0) out[static_cast<size_t>(tok) * n_embd + row] = acc;
 }
 
+// ---------------------------------------------------------------------------------------------
+// One token (decode): two launches for the whole expert step, the routing table riding in the kernel arguments.
+//   moe_decode_gate_up_kernel   grid (row groups / 8, slots): the workgroup quantises the token to Q8_K in LDS (as
+//                               gemv_kquant_f32_kernel does), every wave makes one group of rows of its slot's expert
+//   moe_decode_down_kernel      the workgroup quantises the slots' intermediates (n_slots * nb_mid <= 64 blocks) in
+//                               LDS, then moe_down_token_kernel's row scheme: down, route weight, ordered sum
+// Same quantiser, dots and order of additions as the general path, so the same bits.
+// ---------------------------------------------------------------------------------------------
+constexpr int kDecodeWaves = 8;
+
+template <int kRowsPerWave>
+__global__ void __launch_bounds__(kWave *kDecodeWaves)
+    moe_decode_gate_up_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
+                              const float *__restrict__ x, const MoeDecodeTable table, float *__restrict__ mid,
+                              uint32_t n_ff, uint32_t nb) {
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[16 * 256];
+    __shared__ float s_d[16];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[16 * 16];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const uint32_t slot = blockIdx.y;
+    const uint32_t row = (blockIdx.x * kDecodeWaves + wave) * kRowsPerWave + rsel;
+    const bool live = bslot < nb && row < n_ff;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    TokenSpans<kDecodeWaves> xv;
+    token_load<kDecodeWaves>(x, nb, wave, lane, xv);
+    // dead lanes read the expert's first block
+    const size_t off = static_cast<size_t>(table.expert[slot]) * n_ff * row_bytes +
+                       (live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0);
+    const Q4KRegs rg = q4k_load_block(gate_all + off, g), ru = q4k_load_block(up_all + off, g);
+    token_quantize<kDecodeWaves>(xv, nb, wave, lane, s_qs, s_d, s_bsums);
+    __syncthreads();
+    const uint32_t ab = bslot < nb ? bslot : 0;
+    const Q4KAct a = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
+    float gs = 0.0f, us = 0.0f;
+    if (live) {
+        gs = q4k_dot(q4k_prepare(rg, g), a);
+        us = q4k_dot(q4k_prepare(ru, g), a);
+    }
+    gs = seg_sum<kLanesPerRow>(gs);
+    us = seg_sum<kLanesPerRow>(us);
+    // crates/rnb-cpu/src/kernels/activation.rs:73-89
+    if (sub == kLanesPerRow - 1 && row < n_ff) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(gs, us);
+}
+
+template <uint32_t kQuant, int kGroups>
+__global__ void __launch_bounds__(kWave *kDecodeWaves)
+    moe_decode_down_kernel(const uint8_t *__restrict__ down_all, const float *__restrict__ mid, const MoeDecodeTable table,
+                           float *__restrict__ out, uint32_t n_embd, uint32_t nb) {
+    constexpr int kLanes = kWave / kGroups;  // lanes per (slot, row) pair
+    constexpr int kSpans = 64 / kDecodeWaves;
+    using Q = KQuant<kQuant>;
+    constexpr size_t kBlockBytes = Q::kBytes;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[64 * 256];
+    __shared__ float s_d[64];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[64 * 16];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * kDecodeWaves + wave;
+    const int sub = lane & (kLanes - 1);
+    const uint32_t grp = lane / kLanes;
+    const int g = sub & 3;
+    const uint32_t b = sub >> 2;
+    const uint32_t n_slots = table.n_slots, n_blocks = n_slots * nb;
+    const bool lane_ok = b < nb && row < n_embd;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    // the intermediates first, then the weights of the first kGroups slots, then the quantisation
+    float4 mv[kSpans];
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t blk = wave + i * kDecodeWaves;
+        mv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (blk < n_blocks) mv[i] = reinterpret_cast<const float4 *>(mid + static_cast<size_t>(blk) * 256)[lane];
+    }
+    auto fetch = [&](uint32_t k, bool *ok) {
+        *ok = lane_ok && k < n_slots;
+        const size_t off = *ok ? (static_cast<size_t>(table.expert[k]) * n_embd + row) * row_bytes + static_cast<size_t>(b) * kBlockBytes
+                               : 0;  // dead lanes read the first block of the tensor
+        return Q::load_block(down_all + off, g);
+    };
+    bool cur_ok;
+    typename Q::Regs cur = fetch(grp, &cur_ok);
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t blk = wave + i * kDecodeWaves;
+        if (blk < n_blocks) q8k_quantize_vals(mv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+    }
+    __syncthreads();
+    float acc = 0.0f;
+    for (uint32_t k0 = 0; k0 < n_slots; k0 += kGroups) {
+        const uint32_t k = k0 + grp;
+        bool nxt_ok;
+        const typename Q::Regs nxt = fetch(k + kGroups, &nxt_ok);
+        float o = 0.0f;
+        if (cur_ok) {
+            const uint32_t ab = k * nb + b;
+            o = kquant_partial<kQuant>(cur, Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g), g);
+        }
+        o = seg_sum<kLanes>(o);
+        if (k < n_slots) o *= table.route[k];  // fanout.rs:306-308; only the group's last lane is read below
+#pragma unroll
+        for (int j = 0; j < kGroups; j++) {
+            const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
+            if (k0 + j < n_slots) acc += v;  // wave-uniform
+        }
+        cur = nxt;
+        cur_ok = nxt_ok;
+    }
+    if (lane == 0 && row < n_embd) out[row] = acc;
+}
+
 __global__ void __launch_bounds__(256)
     moe_reduce_kernel(const float *__restrict__ slot_out, const uint32_t *__restrict__ tok_offsets,
                       const uint32_t *__restrict__ tok_slots, float *__restrict__ out, uint32_t n_embd) {
@@ -447,6 +564,31 @@ void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView
                        mid_act.bsums, tok_offsets, tok_slots, slot_expert, slot_route, out, n_embd, nb_mid)
     RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DT);
 #undef RNB_LAUNCH_DT
+}
+
+bool moe_decode_supported(size_t n_slots, size_t nb_in, size_t nb_mid, const void *x) {
+    return n_slots >= 1 && n_slots <= kMoeDecodeMaxSlots && nb_in >= 1 && nb_in <= 16 && nb_mid >= 1 && nb_mid <= 16 &&
+           n_slots * nb_mid <= 64 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
+                       const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
+                       uint32_t nb_in, uint32_t nb_mid, hipStream_t stream) {
+    const dim3 block(kWave * kDecodeWaves);
+    {
+        const int rpw = rows_per_wave_for(nb_in);
+        const uint32_t row_groups = (n_ff + rpw - 1) / rpw;
+        const dim3 grid((row_groups + kDecodeWaves - 1) / kDecodeWaves, table.n_slots, 1);
+#define RNB_LAUNCH_DGU(Q, R) \
+    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
+        RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU);
+#undef RNB_LAUNCH_DGU
+    }
+    const dim3 grid((n_embd + kDecodeWaves - 1) / kDecodeWaves, 1, 1);
+#define RNB_LAUNCH_DD(Q, G) \
+    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
+    RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD);
+#undef RNB_LAUNCH_DD
 }
 
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots, float *out,

@@ -494,6 +494,31 @@ def test_moe_small(rnb, oracle, tokens, down_quant):
         rnb.release(w)
 
 
+@pytest.mark.parametrize("n_ff,n_embd,k,down_quant", [(768, 2048, 8, Q6_K), (256, 512, 1, Q4_K), (512, 1280, 16, Q5_K),
+                                                     (1024, 4096, 16, Q6_K), (256, 768, 17, Q6_K), (2304, 512, 8, Q4_K),
+                                                     (512, 256, 5, Q5_K)])
+def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant):
+    """One token takes the two-launch decode path (token and intermediates quantised inside the kernels, routing table
+    in the kernel arguments) when it has at most 16 slots and 64 intermediate blocks; otherwise, and for batches, the
+    general sequence.  Same arithmetic: the token alone equals its row in a two-token batch bit for bit, with an
+    expert repeated in the slot list, and both agree with the oracle."""
+    n_expert = 20
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, 1, k, 77 + k, down_quant)
+    if k >= 3:
+        e[2] = e[0]  # the same expert twice in one token's list
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, 1, down_quant, n_ff, n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, 1, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"moe decode n_ff {n_ff} n_embd {n_embd} k {k}")
+    x2 = np.concatenate([oracle.fill_normal(n_embd, 5, 1.0), x])
+    m = min(2, e.size)
+    e2, r2 = np.concatenate([e[:m], e]), np.concatenate([r[:m], r])
+    t2 = np.concatenate([np.zeros(m, np.uint32), np.ones(e.size, np.uint32)])
+    both = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e2, r2, t2, 2, down_quant, n_ff, n_embd, x2)
+    assert np.array_equal(both[1], got[0])
+    for w in (gate, up, down):
+        rnb.release(w)
+
+
 def test_moe_unrouted_token_and_empty_slot_list(rnb, oracle):
     n_expert, n_ff, n_embd = 4, 256, 256
     gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, 3, 2, 2)
