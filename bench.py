@@ -320,7 +320,8 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
     # One token against K-quant rows of at most 16 super-blocks is ONE launch in the library (the GEMV's workgroups
     # quantise the token themselves): that kernel is the step, so it is the one the roofline is quoted on; the GEMV
     # over an already quantised token is kept beside it.
-    res["one_launch_step"] = seq == 1 and quant in (10, 11, Q4_K, Q5_K, Q6_K) and cols // 256 <= 16
+    res["one_launch_step"] = seq == 1 and ((quant in (10, 11, Q4_K, Q5_K, Q6_K) and cols // 256 <= 16) or
+                                           (quant in (2, 3, 6, 7, Q8_0) and cols // 32 <= 128 and rows * (cols // 32) >= 1 << 18))
     if res["one_launch_step"]:
         res["prequantised_kernel_ms_mean"] = float(np.mean(reps))
         reps = [kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]

@@ -98,6 +98,12 @@ int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, 
         HIP_TRY(hipGetLastError());
         return RNB_HIP_OK;
     }
+    if (seq == 1 && is_block32(quant) && gemv_block32_f32_supported(static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 32), x_dev)) {
+        launch_gemv_block32_f32(w_dev, quant, x_dev, out_dev, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 32), 1,
+                                s.stream);
+        HIP_TRY(hipGetLastError());
+        return RNB_HIP_OK;
+    }
     ActView act;
     int st = quantize_activations(s, quant, x_dev, seq, cols, &act);
     if (st != RNB_HIP_OK) return st;

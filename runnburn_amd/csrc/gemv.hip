@@ -573,29 +573,51 @@ __device__ __forceinline__ uint32_t spread_fifth_bits(uint32_t x) {
     return ((__umul24(x & 15u, 0x00204081u)) & 0x01010101u) << 4;
 }
 
+// one weight block in registers: loads and arithmetic are separate calls so that a kernel can request a block early
+struct Block32Regs {
+    uint4 q0, q1;  // Q8_0: the 32 codes; others: q0 = the 16 bytes of nibbles
+    uint32_t qh;
+    float d, m;
+};
 template <uint32_t kQuant>
-__device__ __forceinline__ float block32_partial(const uint8_t *__restrict__ blk, const Q8Act &a) {
+__device__ __forceinline__ Block32Regs block32_load(const uint8_t *__restrict__ blk) {
     constexpr Block32Layout F = block32_layout<kQuant>();
-    const float d = ld_f16(blk);
+    Block32Regs r;
+    r.d = ld_f16(blk);
+    r.m = 0.0f;
+    r.qh = 0;
+    r.q1 = make_uint4(0, 0, 0, 0);
     if constexpr (kQuant == kQ8_0) {
-        const uint4 q0 = ld_u4_a2(blk + 2), q1 = ld_u4_a2(blk + 18);
-        int p = 0;
-        p = dot4(q0.x, a.a0.x, p);
-        p = dot4(q0.y, a.a0.y, p);
-        p = dot4(q0.z, a.a0.z, p);
-        p = dot4(q0.w, a.a0.w, p);
-        p = dot4(q1.x, a.a1.x, p);
-        p = dot4(q1.y, a.a1.y, p);
-        p = dot4(q1.z, a.a1.z, p);
-        p = dot4(q1.w, a.a1.w, p);
-        return (d * a.dx) * static_cast<float>(p);
+        r.q0 = ld_u4_a2(blk + 2);
+        r.q1 = ld_u4_a2(blk + 18);
     } else {
-        const uint4 qs = ld_u4_a2(blk + F.qs);
+        r.q0 = ld_u4_a2(blk + F.qs);
+        if constexpr (F.qh >= 0) r.qh = ld_u32_a2(blk + F.qh);
+        if constexpr (F.min) r.m = ld_f16(blk + 2);
+    }
+    return r;
+}
+template <uint32_t kQuant>
+__device__ __forceinline__ float block32_dot(const Block32Regs &r, const Q8Act &a) {
+    constexpr Block32Layout F = block32_layout<kQuant>();
+    if constexpr (kQuant == kQ8_0) {
+        int p = 0;
+        p = dot4(r.q0.x, a.a0.x, p);
+        p = dot4(r.q0.y, a.a0.y, p);
+        p = dot4(r.q0.z, a.a0.z, p);
+        p = dot4(r.q0.w, a.a0.w, p);
+        p = dot4(r.q1.x, a.a1.x, p);
+        p = dot4(r.q1.y, a.a1.y, p);
+        p = dot4(r.q1.z, a.a1.z, p);
+        p = dot4(r.q1.w, a.a1.w, p);
+        return (r.d * a.dx) * static_cast<float>(p);
+    } else {
+        const uint4 qs = r.q0;
         uint4 lo = make_uint4(qs.x & 0x0f0f0f0fu, qs.y & 0x0f0f0f0fu, qs.z & 0x0f0f0f0fu, qs.w & 0x0f0f0f0fu);
         uint4 hi = make_uint4((qs.x >> 4) & 0x0f0f0f0fu, (qs.y >> 4) & 0x0f0f0f0fu, (qs.z >> 4) & 0x0f0f0f0fu,
                               (qs.w >> 4) & 0x0f0f0f0fu);
         if constexpr (F.qh >= 0) {
-            const uint32_t qh = ld_u32_a2(blk + F.qh);
+            const uint32_t qh = r.qh;
             lo.x |= spread_fifth_bits(qh);
             lo.y |= spread_fifth_bits(qh >> 4);
             lo.z |= spread_fifth_bits(qh >> 8);
@@ -615,12 +637,15 @@ __device__ __forceinline__ float block32_partial(const uint8_t *__restrict__ blk
         p = dot4(hi.z, a.a1.z, p);
         p = dot4(hi.w, a.a1.w, p);
         if constexpr (F.min) {
-            const float m = ld_f16(blk + 2);
-            return a.dx * (d * static_cast<float>(p) + m * static_cast<float>(a.sum));
+            return a.dx * (r.d * static_cast<float>(p) + r.m * static_cast<float>(a.sum));
         } else {
-            return (d * a.dx) * static_cast<float>(p - F.offset * a.sum);
+            return (r.d * a.dx) * static_cast<float>(p - F.offset * a.sum);
         }
     }
+}
+template <uint32_t kQuant>
+__device__ __forceinline__ float block32_partial(const uint8_t *__restrict__ blk, const Q8Act &a) {
+    return block32_dot<kQuant>(block32_load<kQuant>(blk), a);
 }
 
 template <uint32_t kQuant>
@@ -668,6 +693,69 @@ void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, ui
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
     hipLaunchKernelGGL(gemv_block32_kernel<kQuant>, grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, act.d, out, rows,
                        nb32);
+}
+
+// One f32 token against rows of at most 128 blocks: the workgroup quantises the token to 32-wide Q8 in LDS itself
+// (the wave-level quantiser of quantize_q8_kernel, so the same bits), as gemv_kquant_f32_kernel does for Q8_K; each
+// lane's first row blocks are requested before the quantisation (a second row in flight measured slower here).
+template <uint32_t kQuant>
+__global__ void __launch_bounds__(kWave *kFusedWaves)
+    gemv_block32_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, uint32_t rows,
+                            uint32_t nb32) {
+    constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
+    constexpr bool kSum = kQuant != kQ8_0;
+    constexpr int kSpans = 16 / kFusedWaves;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[128 * 32];
+    __shared__ float s_d[128];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t tok = blockIdx.y;
+    const float *x_tok = x + static_cast<size_t>(tok) * nb32 * 32;
+    const size_t row_bytes = static_cast<size_t>(nb32) * kBlockBytes;
+    const uint32_t n_waves = gridDim.x * kFusedWaves;
+    uint32_t row = blockIdx.x * kFusedWaves + wave;
+    const uint32_t b0 = lane, b1 = lane + kWave;
+    const bool has0 = b0 < nb32, has1 = b1 < nb32;
+    // the token first (span = 256 elements = 8 blocks; the last span may be partial), then the first rows' blocks
+    float4 xv[kSpans];
+    int live[kSpans];
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t span = wave + i * kFusedWaves;
+        const int left = static_cast<int>(nb32) - static_cast<int>(span) * 8;
+        live[i] = left < 0 ? 0 : (left > 8 ? 8 : left);
+        xv[i] = q8_load_span(x_tok + static_cast<size_t>(span) * 256, lane, live[i]);
+    }
+    auto fetch = [&](uint32_t r, bool has, uint32_t b) {
+        const size_t off = (has && r < rows) ? static_cast<size_t>(r) * row_bytes + static_cast<size_t>(b) * kBlockBytes : 0;
+        return block32_load<kQuant>(w + off);  // rows >= 1 and nb32 >= 1: offset 0 is readable
+    };
+    Block32Regs c0 = fetch(row, has0, b0), c1 = fetch(row, has1, b1);
+#pragma unroll
+    for (int i = 0; i < kSpans; i++) {
+        const uint32_t span = wave + i * kFusedWaves;
+        q8_quantize_vals(xv[i], lane, live[i], s_qs + span * 256, s_d + span * 8);
+    }
+    __syncthreads();
+    const Q8Act a0 = q8_load_act<kSum>(s_qs + (has0 ? b0 : 0) * 32, s_d[has0 ? b0 : 0]);
+    const Q8Act a1 = q8_load_act<kSum>(s_qs + (has1 ? b1 : 0) * 32, s_d[has1 ? b1 : 0]);
+    for (; row < rows; row += n_waves) {
+        float acc = 0.0f;
+        if (has0) acc = block32_dot<kQuant>(c0, a0);
+        if (has1) acc += block32_dot<kQuant>(c1, a1);
+        acc = seg_sum<kWave>(acc);
+        if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
+        c0 = fetch(row + n_waves, has0, b0);
+        c1 = fetch(row + n_waves, has1, b1);
+    }
+}
+
+template <uint32_t kQuant>
+void launch_block32_f32(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,
+                        hipStream_t stream) {
+    const uint32_t waves = rows < kFusedTargetWaves ? rows : kFusedTargetWaves;
+    const dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, seq, 1);
+    hipLaunchKernelGGL(gemv_block32_f32_kernel<kQuant>, grid, dim3(kWave * kFusedWaves), 0, stream, w, x, out, rows, nb32);
 }
 
 }  // namespace
@@ -797,6 +885,24 @@ void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *o
     case kQ5_0: launch_block32<kQ5_0>(w, act, out, rows, nb32, seq, stream); break;
     case kQ5_1: launch_block32<kQ5_1>(w, act, out, rows, nb32, seq, stream); break;
     default: launch_block32<kQ8_0>(w, act, out, rows, nb32, seq, stream); break;
+    }
+}
+
+bool gemv_block32_f32_supported(uint32_t rows, uint32_t nb32, const void *x) {
+    // measured: the saved launch outweighs the per-workgroup quantisation from about 4096 x 2048 upwards
+    return nb32 >= 1 && nb32 <= 128 && static_cast<uint64_t>(rows) * nb32 >= (1u << 18) &&
+           reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+void launch_gemv_block32_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb32,
+                             uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0) return;
+    switch (quant) {
+    case kQ4_0: launch_block32_f32<kQ4_0>(w, x, out, rows, nb32, seq, stream); break;
+    case kQ4_1: launch_block32_f32<kQ4_1>(w, x, out, rows, nb32, seq, stream); break;
+    case kQ5_0: launch_block32_f32<kQ5_0>(w, x, out, rows, nb32, seq, stream); break;
+    case kQ5_1: launch_block32_f32<kQ5_1>(w, x, out, rows, nb32, seq, stream); break;
+    default: launch_block32_f32<kQ8_0>(w, x, out, rows, nb32, seq, stream); break;
     }
 }
 

@@ -41,6 +41,11 @@ void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 // Q2_K / Q3_K rows (84 / 110-byte blocks at 4- / 2-byte alignment); quant is kQ2K or kQ3K
 void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                          uint32_t seq, hipStream_t stream);
+// 32-element formats straight from an f32 token (the workgroup quantises it to 32-wide Q8 in LDS): rows of at most
+// 128 blocks, x 16-byte aligned; same output contract as launch_gemv_block32
+bool gemv_block32_f32_supported(uint32_t rows, uint32_t nb32, const void *x);  // false below the size where it pays
+void launch_gemv_block32_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb32,
+                             uint32_t seq, hipStream_t stream);
 // the f32-token forms of launch_gemv_q4k_gate_up and launch_gemv_q4k_multi (same limits as gemv_kquant_f32_supported:
 // rows of at most 16 super-blocks, x 16-byte aligned; weights 16-byte aligned as for the quantised forms)
 void launch_gemv_q4k_gate_up_f32(const uint8_t *wg, const uint8_t *wu, const float *x, float *mid, uint32_t rows,
