@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // ---------------------------------------------------------------------------------------------
 constexpr int kFusedWaves = 8;   // waves per workgroup: each quantises 16 / 8 = 2 blocks of the token
 constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (more measured slower)
-constexpr uint32_t kFusedTargetWaves = 4096;
+constexpr uint32_t kFusedTargetWaves = 4096;  // 3584, 4784 and 7168 (whole rows per wave for 14336 rows) measured slower
 template <uint32_t kQuant, int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kFusedWaves)
     gemv_kquant_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
