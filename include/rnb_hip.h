@@ -40,6 +40,7 @@ typedef enum {
 #define RNB_GGML_Q4_1 3u
 #define RNB_GGML_Q5_0 6u
 #define RNB_GGML_Q5_1 7u
+#define RNB_GGML_Q8_1 9u
 #define RNB_GGML_Q8_0 8u
 #define RNB_GGML_Q2_K 10u
 #define RNB_GGML_Q3_K 11u
@@ -60,7 +61,7 @@ typedef enum {
 int rnb_hip_backend_kind(void);
 /* capabilities(): 1 when `op` (RNB_OP_*) executes on this backend, else 0. */
 int rnb_hip_backend_supports(int op);
-/* 1 when (op, ggml quant id) is supported: MatMul x {Q4_0,Q4_1,Q5_0,Q5_1,Q8_0,Q2_K..Q6_K}; MoE x gate/up Q4_K with
+/* 1 when (op, ggml quant id) is supported: MatMul x {Q4_0,Q4_1,Q5_0,Q5_1,Q8_0,Q8_1,Q2_K..Q6_K}; MoE x gate/up Q4_K with
  * down Q4_K|Q5_K|Q6_K (pass the down quant). */
 int rnb_hip_backend_supports_quant(int op, uint32_t quant);
 
@@ -121,6 +122,13 @@ int rnb_hip_q5_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t 
 int rnb_hip_q5_1_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
                       size_t x_len, float *out, size_t out_len);
 int rnb_hip_q5_1_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                            const float *x, size_t x_len, float *out, size_t out_len);
+/* q8_1_gemv / q8_1_gemv_batch, quant_api.rs:507-541 (checks and texts of quant_block_gemv(_batch), :1680-1775):
+ * 36-byte blocks {f16 d, f16 s, i8 qs[32]} x the 32-wide Q8 activation; the stored sum s is not read
+ * (crates/rnb-cpu/src/gemm/neon_quant.rs:236-253) */
+int rnb_hip_q8_1_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                      size_t x_len, float *out, size_t out_len);
+int rnb_hip_q8_1_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                             const float *x, size_t x_len, float *out, size_t out_len);
 /* q2k_gemv / q3k_gemv and their batch forms, quant_api.rs:73-181 (same three checks and texts): Q2_K (84-byte) and
  * Q3_K (110-byte) rows x Q8_K(x), the block dots of crates/rnb-cpu/src/gemm/avx2_dot.rs:169-375 */
@@ -255,7 +263,7 @@ typedef struct rnb_hip_gguf_tensor {
     const char *name;      /* owned by the rnb_hip_gguf */
     uint32_t n_dims;       /* 0..4 */
     uint64_t shape[4];     /* row-major (outermost first): the file stores innermost first, parser.rs:356-357 */
-    uint32_t ggml_type;    /* ggml type id: 2/3/6/7/8 = Q4_0/Q4_1/Q5_0/Q5_1/Q8_0, 10..14 = Q2_K..Q6_K, 0 = F32, ... */
+    uint32_t ggml_type;    /* ggml type id: 2/3/6/7/8/9 = Q4_0/Q4_1/Q5_0/Q5_1/Q8_0/Q8_1, 10..14 = Q2_K..Q6_K, 0 = F32, ... */
     uint64_t offset;       /* relative to the data section, as stored */
     uint64_t file_offset;  /* data_start + offset */
     uint64_t n_bytes;      /* elements / block elements * block bytes; 0 if the shape is not block-aligned */

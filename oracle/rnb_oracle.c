@@ -30,6 +30,9 @@
  *                               identity, reduction to dot_q4k_q8k when qh == 0
  *   dot_q6k_q8k                 f64 numpy dequant identity; bsums identity (avx2_dot.rs:824,880)
  *   dot_q8_0_*                  reference vector 528.0 (quant_gemv.rs:1448-1464), numpy identity
+ *   Q8_1 dequant / dot          the reference holds no known-answer test for Q8_1: hand-built bytes (every
+ *                               element position, the stored sum ignored), closed form on constant vectors,
+ *                               f64 numpy dequant identity
  *   gemv drivers                seq-major layout vector (quant_gemv.rs:1448-1464)
  *   gelu_mul_inplace            reference vector (activation.rs:166-173: gate [1, -1], up [2, 3] -> 1.6824, -0.4764)
  *                               + f64 numpy statement of the tanh form
@@ -45,7 +48,7 @@
  *   quantize_row_q2_k           restates quant.rs:44-160; byte parity UNPINNED (cannot run the original), the
  *                               reference's round-trip bound (cosine >= 0.90) is checked.  Input generation only.
  *   quantize_row_q3_k           not in the reference (plain symmetric fit).  Input generation only.
- *   quantize_row_q4_0 .. _q5_1  not in the reference (ggml reference semantics).  Input generation only.
+ *   quantize_row_q4_0 .. _q5_1, _q8_1  not in the reference (ggml reference semantics).  Input generation only.
  *   quantize_row_q6_k/_q8_0     not in the reference at all (ggml reference semantics); round
  *                               trip through the pinned dequantisers.  Input generation only.
  */
@@ -164,22 +167,27 @@ void rnbo_dequantize_q8_0(const uint8_t *blocks, size_t n_blocks, float *out) {
  *   Q4_0 {f16 d, qs[16]}                 (code - 8) * d        Q4_1 {f16 d, f16 m, qs[16]}          code * d + m
  *   Q5_0 {f16 d, qh[4], qs[16]}          (code - 16) * d       Q5_1 {f16 d, f16 m, qh[4], qs[16]}   code * d + m
  * Element i < 16 is the low nibble of qs[i], element 16 + i the high nibble; the fifth bit of element e is bit e of
- * the little-endian 32-bit qh. */
+ * the little-endian 32-bit qh.
+ *   Q8_1 {f16 d, f16 s, i8 qs[32]}       code * d  (whole-byte codes; s = d * sum(qs) is stored for other back ends and
+ *                                        not used: crates/rnb-cpu/src/gemm/quant_gemv.rs:210-216, neon_quant.rs:236-253) */
 typedef struct {
     int bytes, qs_off, qh_off, has_min, offset; /* qh_off < 0: no fifth bit */
+    int byte_codes;                             /* codes are the 32 signed bytes at qs_off */
 } legacy_fmt;
 
 static int legacy_format(uint32_t quant, legacy_fmt *f) {
     switch (quant) {
-    case 2: *f = (legacy_fmt){RNBO_Q4_0_BLOCK_BYTES, 2, -1, 0, 8}; return 1;
-    case 3: *f = (legacy_fmt){RNBO_Q4_1_BLOCK_BYTES, 4, -1, 1, 0}; return 1;
-    case 6: *f = (legacy_fmt){RNBO_Q5_0_BLOCK_BYTES, 6, 2, 0, 16}; return 1;
-    case 7: *f = (legacy_fmt){RNBO_Q5_1_BLOCK_BYTES, 8, 4, 1, 0}; return 1;
+    case 2: *f = (legacy_fmt){RNBO_Q4_0_BLOCK_BYTES, 2, -1, 0, 8, 0}; return 1;
+    case 3: *f = (legacy_fmt){RNBO_Q4_1_BLOCK_BYTES, 4, -1, 1, 0, 0}; return 1;
+    case 6: *f = (legacy_fmt){RNBO_Q5_0_BLOCK_BYTES, 6, 2, 0, 16, 0}; return 1;
+    case 7: *f = (legacy_fmt){RNBO_Q5_1_BLOCK_BYTES, 8, 4, 1, 0, 0}; return 1;
+    case 9: *f = (legacy_fmt){RNBO_Q8_1_BLOCK_BYTES, 4, -1, 0, 0, 1}; return 1;
     default: return 0;
     }
 }
 
 static inline int legacy_code(const legacy_fmt *f, const uint8_t *blk, int e) {
+    if (f->byte_codes) return (int)(int8_t)blk[f->qs_off + e];
     int nib = e < 16 ? (blk[f->qs_off + e] & 0x0f) : (blk[f->qs_off + e - 16] >> 4);
     if (f->qh_off >= 0) {
         uint32_t qh = (uint32_t)blk[f->qh_off] | ((uint32_t)blk[f->qh_off + 1] << 8) |
@@ -755,6 +763,7 @@ static size_t block_bytes_of(uint32_t quant, size_t *elems) {
     case 6: *elems = 32; return RNBO_Q5_0_BLOCK_BYTES;
     case 7: *elems = 32; return RNBO_Q5_1_BLOCK_BYTES;
     case 8: *elems = 32; return RNBO_Q8_0_BLOCK_BYTES;
+    case 9: *elems = 32; return RNBO_Q8_1_BLOCK_BYTES;
     case 10: *elems = 256; return RNBO_Q2_K_BLOCK_BYTES;
     case 11: *elems = 256; return RNBO_Q3_K_BLOCK_BYTES;
     case 12: *elems = 256; return RNBO_Q4_K_BLOCK_BYTES;
@@ -1402,6 +1411,21 @@ int rnbo_quantize_row_legacy(uint32_t quant, const float *input, size_t n, uint8
         const float *x = input + b * 32;
         uint8_t *out = output + b * (size_t)f.bytes;
         memset(out, 0, (size_t)f.bytes);
+        if (f.byte_codes) { /* Q8_1, ggml reference semantics: d = amax / 127, q = round(x / d), s = d * sum(q) */
+            float amax = 0.0f;
+            for (int i = 0; i < 32; i++)
+                if (fabsf(x[i]) > amax) amax = fabsf(x[i]);
+            float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+            int sum = 0;
+            for (int i = 0; i < 32; i++) {
+                int q = (int)roundf(x[i] * id);
+                out[f.qs_off + i] = (uint8_t)(int8_t)q;
+                sum += q;
+            }
+            wr_f16(out, d);
+            wr_f16(out + 2, d * (float)sum);
+            continue;
+        }
         float d, base;
         if (f.has_min) {
             float lo = x[0], hi = x[0];
@@ -1496,7 +1520,7 @@ int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, f
         for (long r = 0; r < (long)rows; r++) {
             for (size_t c = 0; c < cols; c++) row[c] = normal_at(seed, (uint64_t)r * cols + c, sigma);
             uint8_t *dst = out + (size_t)r * row_bytes;
-            if (quant == 2 || quant == 3 || quant == 6 || quant == 7)
+            if (quant == 2 || quant == 3 || quant == 6 || quant == 7 || quant == 9)
                 rnbo_quantize_row_legacy(quant, row, cols, dst);
             else if (quant == 10)
                 rnbo_quantize_row_q2_k(row, cols, dst);

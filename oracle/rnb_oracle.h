@@ -29,6 +29,7 @@ extern "C" {
 #define RNBO_Q4_1_BLOCK_BYTES 20
 #define RNBO_Q5_0_BLOCK_BYTES 22
 #define RNBO_Q5_1_BLOCK_BYTES 24
+#define RNBO_Q8_1_BLOCK_BYTES 36
 #define RNBO_Q2_K_BLOCK_BYTES 84
 #define RNBO_Q3_K_BLOCK_BYTES 110
 #define RNBO_Q4_K_BLOCK_BYTES 144

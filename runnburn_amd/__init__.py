@@ -6,6 +6,7 @@ functions keep the reference's names, argument meaning and error behaviour:
 
   q4k_gemv / q4k_gemv_into / q4k_gemv_batch   crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-238, 2283-2319
   q4_0 / q4_1 / q5_0 / q5_1 _gemv (+ _batch)  quant_api.rs:374-496
+  q8_1_gemv (+ _batch)                         quant_api.rs:507-541
   q2k_gemv / q3k_gemv (+ _batch)              quant_api.rs:73-181
   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
@@ -29,6 +30,7 @@ from .binding import (  # noqa: F401
     GGML_Q4_1,
     GGML_Q5_0,
     GGML_Q5_1,
+    GGML_Q8_1,
     GGML_Q2_K,
     GGML_Q3_K,
     GGML_Q4_K,
@@ -61,6 +63,8 @@ from .binding import (  # noqa: F401
     q5_0_gemv_batch,
     q5_1_gemv,
     q5_1_gemv_batch,
+    q8_1_gemv,
+    q8_1_gemv_batch,
     q2k_gemv,
     q2k_gemv_batch,
     q3k_gemv,

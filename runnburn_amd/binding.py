@@ -10,7 +10,7 @@ import numpy as np
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_PKG, "librnb_hip.so")
 
-GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1 = 2, 3, 6, 7
+GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1, GGML_Q8_1 = 2, 3, 6, 7, 9
 GGML_Q8_0, GGML_Q2_K, GGML_Q3_K, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 10, 11, 12, 13, 14
 OP_MATMUL, OP_ATTENTION, OP_GDN, OP_MOE, OP_SAMPLER = 0, 1, 2, 3, 4
 STATUS_NAMES = {0: "Ok", 1: "InvalidRequest", 2: "UnsupportedOp", 3: "ExecutionFailed", 4: "NoDevice"}
@@ -43,6 +43,8 @@ SYMBOLS = [
     ("rnb_hip_q5_0_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q5_1_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q5_1_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_q8_1_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_q8_1_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q2k_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q2k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q3k_gemv", _i, _MATMUL_ARGS),
@@ -287,6 +289,15 @@ def q5_1_gemv(weights, rows, cols, input):  # noqa: A002
 
 def q5_1_gemv_batch(weights, rows, cols, input):  # noqa: A002
     return _gemv_batch("rnb_hip_q5_1_gemv_batch", weights, rows, cols, input)
+
+
+def q8_1_gemv(weights, rows, cols, input):  # noqa: A002
+    """crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:507-523."""
+    return _gemv("rnb_hip_q8_1_gemv", weights, rows, cols, input)
+
+
+def q8_1_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_q8_1_gemv_batch", weights, rows, cols, input)
 
 
 def q2k_gemv(weights, rows, cols, input):  # noqa: A002

@@ -26,6 +26,7 @@ bool quant_info(uint32_t quant, QuantInfo *qi) {
     case kQ4_1: *qi = {"Q4_1", 32, kQ4_1Bytes}; return true;
     case kQ5_0: *qi = {"Q5_0", 32, kQ5_0Bytes}; return true;
     case kQ5_1: *qi = {"Q5_1", 32, kQ5_1Bytes}; return true;
+    case kQ8_1: *qi = {"Q8_1", 32, kQ8_1Bytes}; return true;
     case kQ8_0: *qi = {"Q8_0", 32, kQ8_0Bytes}; return true;
     case kQ2K: *qi = {"Q2_K", 256, kQ2KBytes}; return true;
     case kQ3K: *qi = {"Q3_K", 256, kQ3KBytes}; return true;
@@ -38,7 +39,7 @@ bool quant_info(uint32_t quant, QuantInfo *qi) {
 
 // the 32-element formats take 32-wide Q8 activations, the K-quants 256-wide Q8_K
 bool is_block32(uint32_t quant) {
-    return quant == kQ8_0 || quant == kQ4_0 || quant == kQ4_1 || quant == kQ5_0 || quant == kQ5_1;
+    return quant == kQ8_0 || quant == kQ4_0 || quant == kQ4_1 || quant == kQ5_0 || quant == kQ5_1 || quant == kQ8_1;
 }
 
 int fail(int status, const std::string &msg) {
@@ -663,6 +664,7 @@ RNB_BLOCK32_ENTRY(q4_0, kQ4_0)
 RNB_BLOCK32_ENTRY(q4_1, kQ4_1)
 RNB_BLOCK32_ENTRY(q5_0, kQ5_0)
 RNB_BLOCK32_ENTRY(q5_1, kQ5_1)
+RNB_BLOCK32_ENTRY(q8_1, kQ8_1)
 #undef RNB_BLOCK32_ENTRY
 
 int rnb_hip_q2k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,

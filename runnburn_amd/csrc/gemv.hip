@@ -522,6 +522,7 @@ void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows,
 //   Q5_0 {f16 d, u32 qh, qs[16]}            (d * d_x) * sum((code - 16) * q)         neon_dot.rs:163-214
 //   Q4_1 {f16 d, f16 m, qs[16]}             d_x * (d * sum(code * q) + m * sum(q))   neon_quant.rs:88-108
 //   Q5_1 {f16 d, f16 m, u32 qh, qs[16]}     likewise                                 neon_quant.rs:130-158
+//   Q8_1 {f16 d, f16 s, i8 qs[32]}          (d * d_x) * sum(w * q), s is not read      neon_quant.rs:236-253
 // (all under crates/rnb-cpu/src/gemm/).  Element i < 16 is the low nibble of qs[i], element 16 + i the high nibble; the
 // fifth bit of element e is bit e of qh.  (code - offset) is applied as dot(code, q) - offset * sum(q).
 // ---------------------------------------------------------------------------------------------
@@ -564,6 +565,7 @@ constexpr Block32Layout block32_layout() {
     case kQ4_1: return {static_cast<int>(kQ4_1Bytes), 4, -1, 0, true};
     case kQ5_0: return {static_cast<int>(kQ5_0Bytes), 6, 2, 16, false};
     case kQ5_1: return {static_cast<int>(kQ5_1Bytes), 8, 4, 0, true};
+    case kQ8_1: return {static_cast<int>(kQ8_1Bytes), 4, -1, 0, false};
     default: return {static_cast<int>(kQ8_0Bytes), 2, -1, 0, false};
     }
 }
@@ -587,9 +589,9 @@ __device__ __forceinline__ Block32Regs block32_load(const uint8_t *__restrict__ 
     r.m = 0.0f;
     r.qh = 0;
     r.q1 = make_uint4(0, 0, 0, 0);
-    if constexpr (kQuant == kQ8_0) {
-        r.q0 = ld_u4_a2(blk + 2);
-        r.q1 = ld_u4_a2(blk + 18);
+    if constexpr (kQuant == kQ8_0 || kQuant == kQ8_1) {  // whole-byte codes
+        r.q0 = ld_u4_a2(blk + F.qs);
+        r.q1 = ld_u4_a2(blk + F.qs + 16);
     } else {
         r.q0 = ld_u4_a2(blk + F.qs);
         if constexpr (F.qh >= 0) r.qh = ld_u32_a2(blk + F.qh);
@@ -600,7 +602,7 @@ __device__ __forceinline__ Block32Regs block32_load(const uint8_t *__restrict__ 
 template <uint32_t kQuant>
 __device__ __forceinline__ float block32_dot(const Block32Regs &r, const Q8Act &a) {
     constexpr Block32Layout F = block32_layout<kQuant>();
-    if constexpr (kQuant == kQ8_0) {
+    if constexpr (kQuant == kQ8_0 || kQuant == kQ8_1) {
         int p = 0;
         p = dot4(r.q0.x, a.a0.x, p);
         p = dot4(r.q0.y, a.a0.y, p);
@@ -653,7 +655,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_block32_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                         float *__restrict__ out, uint32_t rows, uint32_t nb32) {
     constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
-    constexpr bool kSum = kQuant != kQ8_0;
+    constexpr bool kSum = kQuant != kQ8_0 && kQuant != kQ8_1;
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t tok = blockIdx.y;
     const size_t abase = static_cast<size_t>(tok) * nb32;
@@ -703,7 +705,7 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     gemv_block32_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, uint32_t rows,
                             uint32_t nb32) {
     constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
-    constexpr bool kSum = kQuant != kQ8_0;
+    constexpr bool kSum = kQuant != kQ8_0 && kQuant != kQ8_1;
     constexpr int kSpans = 16 / kFusedWaves;
     __shared__ __attribute__((aligned(16))) int8_t s_qs[128 * 32];
     __shared__ float s_d[128];
@@ -884,6 +886,7 @@ void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *o
     case kQ4_1: launch_block32<kQ4_1>(w, act, out, rows, nb32, seq, stream); break;
     case kQ5_0: launch_block32<kQ5_0>(w, act, out, rows, nb32, seq, stream); break;
     case kQ5_1: launch_block32<kQ5_1>(w, act, out, rows, nb32, seq, stream); break;
+    case kQ8_1: launch_block32<kQ8_1>(w, act, out, rows, nb32, seq, stream); break;
     default: launch_block32<kQ8_0>(w, act, out, rows, nb32, seq, stream); break;
     }
 }
@@ -902,6 +905,7 @@ void launch_gemv_block32_f32(const uint8_t *w, uint32_t quant, const float *x, f
     case kQ4_1: launch_block32_f32<kQ4_1>(w, x, out, rows, nb32, seq, stream); break;
     case kQ5_0: launch_block32_f32<kQ5_0>(w, x, out, rows, nb32, seq, stream); break;
     case kQ5_1: launch_block32_f32<kQ5_1>(w, x, out, rows, nb32, seq, stream); break;
+    case kQ8_1: launch_block32_f32<kQ8_1>(w, x, out, rows, nb32, seq, stream); break;
     default: launch_block32_f32<kQ8_0>(w, x, out, rows, nb32, seq, stream); break;
     }
 }

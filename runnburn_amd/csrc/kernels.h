@@ -8,8 +8,8 @@
 
 namespace rnb {
 
-constexpr uint32_t kQ4_0 = 2, kQ4_1 = 3, kQ5_0 = 6, kQ5_1 = 7, kQ8_0 = 8, kQ2K = 10, kQ3K = 11, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
-constexpr size_t kQ4_0Bytes = 18, kQ4_1Bytes = 20, kQ5_0Bytes = 22, kQ5_1Bytes = 24, kQ8_0Bytes = 34, kQ2KBytes = 84, kQ3KBytes = 110, kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210;
+constexpr uint32_t kQ4_0 = 2, kQ4_1 = 3, kQ5_0 = 6, kQ5_1 = 7, kQ8_0 = 8, kQ8_1 = 9, kQ2K = 10, kQ3K = 11, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
+constexpr size_t kQ4_0Bytes = 18, kQ4_1Bytes = 20, kQ5_0Bytes = 22, kQ5_1Bytes = 24, kQ8_0Bytes = 34, kQ8_1Bytes = 36, kQ2KBytes = 84, kQ3KBytes = 110, kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210;
 
 // Device layout of quantised activations (structure of arrays, one set per call):
 //   Q8_K:  qs    int8  [seq][K]          (16-byte aligned rows, K % 256 == 0)
@@ -61,7 +61,7 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,
                       uint32_t seq, hipStream_t stream);
-// any 32-element format (kQ4_0, kQ4_1, kQ5_0, kQ5_1, kQ8_0) against 32-wide Q8 activations
+// any 32-element format (kQ4_0, kQ4_1, kQ5_0, kQ5_1, kQ8_0, kQ8_1) against 32-wide Q8 activations
 void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
                          uint32_t seq, hipStream_t stream);
 

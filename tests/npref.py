@@ -29,6 +29,18 @@ def make_legacy_block(quant, d, m, codes) -> np.ndarray:
     return np.concatenate(parts).astype(np.uint8)
 
 
+def make_q8_1_block(d, s, values) -> np.ndarray:
+    """Q8_1 {f16 d, f16 s, i8 qs[32]} (crates/rnb-cpu/src/quantize/blocks.rs:54-59); s is carried, never read."""
+    return np.concatenate([np.frombuffer(f16_bytes(d), dtype=np.uint8), np.frombuffer(f16_bytes(s), dtype=np.uint8),
+                           np.asarray(values, dtype=np.int8).view(np.uint8)]).astype(np.uint8)
+
+
+def dequant_q8_1_f64(blocks) -> np.ndarray:
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, 36)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float64)
+    return (b[:, 4:36].copy().view(np.int8).astype(np.float64) * d).reshape(-1)
+
+
 def dequant_legacy_f64(quant, blocks) -> np.ndarray:
     nbytes, has_min, has_qh = LEGACY_LAYOUT[quant]
     b = np.asarray(blocks, dtype=np.uint8).reshape(-1, nbytes)

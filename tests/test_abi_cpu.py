@@ -38,6 +38,7 @@ def test_trait_facade():
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q5_K) and b.supports_quant(rnb.OP_MOE, rnb.GGML_Q5_K)
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q2_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q3_K)
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q4_0) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q5_1)
+    assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q8_1)
     assert not b.supports_quant(rnb.OP_MATMUL, 16) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # IQ2_XXS; Q8_0 down
     with pytest.raises(rnb.BackendError) as ei:
         b.execute(object())
@@ -66,7 +67,7 @@ def test_matmul_validation_messages_match_reference():
     assert str(e) == "Q4_K batch input length 300 is not divisible by cols 256"
     # crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:374-496, 1983-2075
     for fn, label, nbytes in ((rnb.q4_0_gemv, "Q4_0", 18), (rnb.q4_1_gemv, "Q4_1", 20), (rnb.q5_0_gemv, "Q5_0", 22),
-                              (rnb.q5_1_gemv, "Q5_1", 24)):
+                              (rnb.q5_1_gemv, "Q5_1", 24), (rnb.q8_1_gemv, "Q8_1", 36)):
         e = _err(fn, z(nbytes, np.uint8), 1, 33, z(33, np.float32))
         assert str(e) == f"{label} cols must be divisible by 32, got 33"
         e = _err(fn, z(nbytes + 1, np.uint8), 1, 32, z(32, np.float32))
@@ -75,6 +76,8 @@ def test_matmul_validation_messages_match_reference():
         assert str(e) == f"{label} input length mismatch: got 31, expected 32"
     e = _err(rnb.q5_1_gemv_batch, z(24, np.uint8), 1, 32, z(40, np.float32))
     assert str(e) == "Q5_1 batch input length 40 is not divisible by cols 32"
+    e = _err(rnb.q8_1_gemv_batch, z(36, np.uint8), 1, 32, z(40, np.float32))  # quant_api.rs:1737-1742
+    assert str(e) == "Q8_1 batch input length 40 is not divisible by cols 32"
     # crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:73-181
     e = _err(rnb.q2k_gemv, z(84, np.uint8), 1, 100, z(100, np.float32))
     assert str(e) == "Q2_K cols must be divisible by 256, got 100"

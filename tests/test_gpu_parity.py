@@ -10,7 +10,7 @@ from tests import npref
 
 pytestmark = pytest.mark.gpu
 
-Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_1 = 2, 3, 6, 7, 9
 LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 REL = 1e-3          # tolerance named by the task: max relative error 1e-3 per row
@@ -34,7 +34,8 @@ def gemv_fn(rnb, quant, batch=False):
              (Q5_1, False): rnb.q5_1_gemv, (Q5_1, True): rnb.q5_1_gemv_batch, (Q2_K, False): rnb.q2k_gemv, (Q2_K, True): rnb.q2k_gemv_batch, (Q3_K, False): rnb.q3k_gemv,
              (Q3_K, True): rnb.q3k_gemv_batch, (Q4_K, False): rnb.q4k_gemv, (Q4_K, True): rnb.q4k_gemv_batch, (Q5_K, False): rnb.q5k_gemv,
              (Q5_K, True): rnb.q5k_gemv_batch, (Q6_K, False): rnb.q6k_gemv, (Q6_K, True): rnb.q6k_gemv_batch,
-             (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch}
+             (Q8_0, False): rnb.q8_0_gemv, (Q8_0, True): rnb.q8_0_gemv_batch,
+             (Q8_1, False): rnb.q8_1_gemv, (Q8_1, True): rnb.q8_1_gemv_batch}
     return table[(quant, batch)]
 
 
@@ -130,7 +131,7 @@ def test_gemv_small_shapes(rnb, oracle, quant, rows, nblk):
     check_close(got, ref, gold, f"quant {quant} rows {rows} nblk {nblk}")
 
 
-@pytest.mark.parametrize("quant", (Q8_0,) + LEGACY)
+@pytest.mark.parametrize("quant", (Q8_0, Q8_1) + LEGACY)
 @pytest.mark.parametrize("cols", [32, 96, 32 * 65, 32 * 129])
 def test_block32_gemv_block_counts_off_the_wave_size(rnb, oracle, quant, cols):
     rows = 6
@@ -171,6 +172,36 @@ def test_legacy_formats_shapes_batches_and_extremes(rnb, oracle, quant):
     w = np.concatenate(blocks)
     check_close(gemv_fn(rnb, quant)(w, rows, nb32 * 32, x), oracle.gemv(quant, w, rows, nb32 * 32, x)[0],
                 oracle.gemv(quant, w, rows, nb32 * 32, x, gold=True)[0], f"quant {quant} extremes")
+
+
+def test_q8_1_shapes_batches_and_extremes(rnb, oracle):
+    """Q8_1 weights (crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:507-541): decode shapes (the large ones take the
+    one-launch kernel), batches, and hand-built blocks with -128 / 127 codes, negative, zero and subnormal scales and an
+    arbitrary stored sum (it must not be read)."""
+    for rows, cols in ((1, 32), (7, 1056), (300, 4096), (4096, 4096), (33, 11008)):
+        w = oracle.make_weights(Q8_1, rows, cols, 4200 + rows)
+        x = oracle.fill_normal(cols, 4201 + cols, 1.0)
+        check_close(rnb.q8_1_gemv(w, rows, cols, x), oracle.gemv(Q8_1, w, rows, cols, x)[0],
+                    oracle.gemv(Q8_1, w, rows, cols, x, gold=True)[0], f"q8_1 {rows}x{cols}")
+        rnb.release(w)
+    for seq in (2, 5, 17):
+        rows, cols = 37, 768
+        w = oracle.make_weights(Q8_1, rows, cols, 4300)
+        x = oracle.fill_normal(seq * cols, 4301 + seq, 1.0)
+        got = rnb.q8_1_gemv_batch(w, rows, cols, x)
+        assert got.shape == (seq, rows)
+        check_close(got, oracle.gemv(Q8_1, w, rows, cols, x), oracle.gemv(Q8_1, w, rows, cols, x, gold=True), f"q8_1 batch {seq}")
+    rng = np.random.default_rng(31)
+    rows, nb32 = 8, 16
+    x = oracle.fill_normal(nb32 * 32, 30, 1.0)
+    x[64:96] = 0.0
+    blocks = []
+    for i in range(rows * nb32):
+        codes = [np.full(32, 127), np.full(32, -128), rng.integers(-128, 128, 32), np.zeros(32)][i % 4]
+        blocks.append(npref.make_q8_1_block([1.0, -0.5, 6e-8, 0.0, 2.0 ** -14][i % 5], [1e4, -3.0, 0.0][i % 3], codes))
+    w = np.concatenate(blocks)
+    check_close(rnb.q8_1_gemv(w, rows, nb32 * 32, x), oracle.gemv(Q8_1, w, rows, nb32 * 32, x)[0],
+                oracle.gemv(Q8_1, w, rows, nb32 * 32, x, gold=True)[0], "q8_1 extremes")
 
 
 def test_gemv_extreme_blocks(rnb, oracle):
@@ -286,7 +317,7 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
                                              (Q2_K, 300, 4096), (Q2_K, 24, 14336), (Q3_K, 300, 4096), (Q3_K, 24, 14336),
                                              (Q4_K, 5, 256), (Q4_K, 20001, 256), (Q6_K, 9001, 1024), (Q5_K, 4099, 4096),
                                              (Q3_K, 8200, 2304), (Q8_0, 4100, 2048), (Q8_0, 5000, 2080), (2, 2100, 4096), (3, 8200, 1056),
-                                             (6, 4100, 4096), (7, 90000, 96)])
+                                             (6, 4100, 4096), (7, 90000, 96), (9, 4100, 2048), (9, 50, 96)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
     feed several matrices from one activation) run the same arithmetic: identical bits.  For K-quant rows of at most

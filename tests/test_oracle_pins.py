@@ -9,8 +9,9 @@ import pytest
 
 from tests import npref
 
-Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
-LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1)
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_1 = 2, 3, 6, 7, 9
+NIBBLE_FORMATS = (Q4_0, Q4_1, Q5_0, Q5_1)
+LEGACY = NIBBLE_FORMATS
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 
 
@@ -138,7 +139,56 @@ def test_dequantize_q4k_places_each_nibble(oracle):
     assert np.allclose(got, want, rtol=0, atol=1e-7 * np.abs(want).max() * 4)
 
 
-@pytest.mark.parametrize("quant", LEGACY)
+def test_q8_1_dequant_and_dot(oracle):
+    """Q8_1 {f16 d, f16 s, i8 qs[32]}: crates/rnb-cpu/src/gemm/quant_gemv.rs:210-216 (element = d * q) and
+    neon_quant.rs:236-253 (dot = d * d_x * sum(q * a); "the stored Q8_1 sum is not needed").  The reference holds no
+    known-answer test for this format; pinned by hand-built bytes (every element position, s ignored), the closed
+    form on constant vectors and the f64 identity against an independent numpy dequantiser."""
+    q = (np.arange(32) * 7 % 255 - 127).astype(np.int8)
+    blk = npref.make_q8_1_block(0.5, 123.0, q)
+    assert blk.size == 36
+    assert np.array_equal(oracle.dequantize(Q8_1, blk), q.astype(np.float32) * np.float32(0.5))
+    assert np.array_equal(oracle.dequantize(Q8_1, npref.make_q8_1_block(0.5, -7.0, q)), oracle.dequantize(Q8_1, blk))
+    for e in (0, 1, 15, 16, 31):
+        one = np.zeros(32, np.int8)
+        one[e] = -128
+        want = np.zeros(32, np.float32)
+        want[e] = -256.0
+        assert np.array_equal(oracle.dequantize(Q8_1, npref.make_q8_1_block(2.0, 0.0, one)), want), e
+    a = (np.arange(32) % 9 - 4).astype(np.int8)
+    act = _q8_act(0.25, a)
+    assert oracle.dot(Q8_1, npref.make_q8_1_block(2.0, 99.0, np.full(32, 3)), act) == 2.0 * 0.25 * 3 * float(a.astype(np.int64).sum())
+    assert oracle.dot(Q8_1, blk, act) == 0.5 * 0.25 * float(np.dot(q.astype(np.int64), a.astype(np.int64)))
+    rng = np.random.default_rng(69)
+    for nb in (1, 3, 128):
+        row = np.concatenate([npref.make_q8_1_block(rng.uniform(-1e-2, 1e-2), rng.uniform(-1, 1), rng.integers(-128, 128, 32))
+                              for _ in range(nb)])
+        x = rng.standard_normal(nb * 32).astype(np.float32)
+        xa = oracle.quantize_q8(x)
+        xq = (xa["d"].astype(np.float64)[:, None] * xa["qs"].astype(np.float64)).reshape(-1)
+        want = float(np.dot(npref.dequant_q8_1_f64(row), xq))
+        assert oracle.dot(Q8_1, row, xa, gold=True) == pytest.approx(want, rel=1e-11, abs=1e-12)
+        assert abs(oracle.dot(Q8_1, row, xa) - want) <= 4e-7 * float(np.sum(np.abs(npref.dequant_q8_1_f64(row) * xq)))
+    # the generator (ggml semantics, input generation only): round trip and the stored sum
+    xw = oracle.fill_normal(32 * 200, 26, 0.02)
+    w = oracle.quantize_row(Q8_1, xw)
+    y = oracle.dequantize(Q8_1, w)
+    assert np.sqrt(np.mean((xw - y) ** 2)) / np.sqrt(np.mean(xw ** 2)) < 0.01
+    b = w.reshape(-1, 36)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    ssum = b[:, 4:].copy().view(np.int8).astype(np.int64).sum(axis=1)
+    assert np.allclose(b[:, 2:4].copy().view(np.float16).astype(np.float32).reshape(-1), d * ssum, rtol=2e-3, atol=1e-6)
+    rows, cols = 3, 96
+    wm = oracle.make_weights(Q8_1, rows, cols, 7)
+    xs = oracle.fill_normal(2 * cols, 8, 1.0).reshape(2, cols)
+    out = oracle.gemv(Q8_1, wm, rows, cols, xs)
+    for si in range(2):
+        xa = oracle.quantize_q8(xs[si])
+        for r in range(rows):
+            assert out[si, r] == np.float32(oracle.dot(Q8_1, wm[r * 108:(r + 1) * 108], xa))
+
+
+@pytest.mark.parametrize("quant", NIBBLE_FORMATS)
 def test_dequantize_legacy_formats_place_every_field(oracle, quant):
     """crates/rnb-cpu/src/quantize/dequant.rs:7-53 against hand-built bytes: one nibble, one high bit at a time."""
     nbytes, has_min, has_qh = npref.LEGACY_LAYOUT[quant]
@@ -427,7 +477,7 @@ def _q8_act(d, q):
     return a
 
 
-@pytest.mark.parametrize("quant", LEGACY)
+@pytest.mark.parametrize("quant", NIBBLE_FORMATS)
 def test_legacy_dot_known_vectors_and_identity(oracle, quant):
     """crates/rnb-cpu/src/gemm/neon_dot.rs:83-214 and neon_quant.rs:88-158 on hand vectors: all codes equal ->
     (code - offset) * sum(q) * d * d_x for the _0 formats, d_x * (d * code + m) * sum(q) for the _1 formats; then the
