@@ -568,6 +568,15 @@ def main() -> int:
                                                       "mfma_frac": tops / INT8_PEAK_TOPS}
         except Exception as exc:
             sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"error": str(exc)}
+        # prefill on the formats whose scales cannot ride on an int8 operand (scale groups applied on the vector units)
+        for key, quant, r, c in (("q6k_gemm_512x14336_to_4096", Q6_K, 4096, 14336), ("q8_0_gemm_512x4096_to_4096", Q8_0, 4096, 4096)):
+            try:
+                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, 512, 20, 3, 101, key, want_graph=False)
+                ops = 2 * 512 * r * c
+                tops = ops / res["kernel_ms_mean"] / 1e9
+                sec[key] = {"kernel_ms_mean": res["kernel_ms_mean"], "ops": ops, "TOP/s": tops, "mfma_frac": tops / INT8_PEAK_TOPS}
+            except Exception as exc:
+                sec[key] = {"error": str(exc)}
         for tokens in (1, 64):
             try:
                 sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens)

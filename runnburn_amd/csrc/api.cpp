@@ -137,10 +137,14 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ6K) {
-        if (seq >= kTokensMinSeq)
+        if (seq >= kGemmMinSeq)
+            launch_gemm_q6k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
+        else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
+    } else if (seq >= kGemmMinSeq && gemm_q8_mfma_supported(quant, static_cast<uint32_t>(cols / 32))) {
+        launch_gemm_q8_mfma(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     } else {
         launch_gemv_block32(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     }

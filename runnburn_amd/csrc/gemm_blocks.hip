@@ -1,0 +1,409 @@
+// Prefill GEMM for the formats whose scales do not fold onto an int8 operand: Q6_K (int8 scale per 16 elements) and
+// the 32-element byte formats Q8_0 / Q8_1 (f16 scale per 32 elements).  out[seq][rows], same contract as the GEMVs.
+//
+// The matrix cores do the integer part of one scale group per instruction and the vector units apply the group's scale
+// to the 16 results a lane holds:
+//   Q6_K   v_mfma_i32_32x32x16_i8 per 16-element sub-block: I_sb = sum (q - 32) * a  (exact), tot += sc[r][sb] * I_sb
+//          in 24-bit integer multiplies, and once per super-block out += (d[r] * d_x[s]) * float(tot): the arithmetic of
+//          crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 (dot_q6_k_q8k_scalar).
+//   Q8_0   v_mfma_i32_32x32x32_i8 per 32-element block: out += (d[r][b] * d_x[s][b]) * float(I_b),
+//   Q8_1   crates/rnb-cpu/src/gemm/neon_dot.rs:376-436, neon_quant.rs:236-253.
+// That is 16 (Q6_K) or 48 (Q8) vector instructions per matrix instruction, so these kernels are bound by the vector
+// port, not the matrix pipe; they replace one GEMV pass per token (Q8) or the integer-dot multi-token kernel (Q6_K),
+// which are 20 to 100 times slower at 512 tokens.
+//
+// Tiling: workgroup = 4 waves = 128 weight rows x kTT*32 tokens; a wave owns 32 rows and all the workgroup's tokens.
+// MFMA "M" = token, "N" = weight row: a lane's 16 results belong to ONE row (lane % 32), so that row's scales are
+// per-lane scalars; both operands take their K bytes per lane from the same K positions (8 or 16 times lane / 32 + j),
+// so the contraction does not depend on how the hardware orders K inside the instruction.  Weights go from global
+// memory straight to the registers of the lane that owns the row (one scale group ahead of use is the next
+// super-block / block pair, requested before the current one is multiplied); the quantised activations of the
+// workgroup's tokens are staged in LDS, double-buffered, one barrier per step.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace rnb {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kGbWaves = 4;
+constexpr int kGbThreads = kWave * kGbWaves;
+constexpr int kGbRows = 32 * kGbWaves;  // 128 rows per workgroup
+constexpr int kGbStride64 = 264;   // bytes per staged token row for 64-bit operand reads (256 + 8): bank-conflict free
+constexpr int kGbStride128 = 272;  // ... and for 128-bit operand reads (256 + 16, keeps them 16-byte aligned)
+
+// ---------------------------------------------------------------------------------------------
+// Q6_K: block = {ql[128], qh[64], i8 scales[16], f16 d}, 210 bytes, 2-byte aligned.  Element 128h + 32p + l
+// (h = half, p = quarter, l < 32) = ((ql[64h + 32(p&1) + l] >> 4(p>>1)) & 15 | ((qh[32h + l] >> 2p) & 3) << 4) - 32, its
+// 16-element sub-block is 8h + 2p + l/16.  The lane of K-half k takes l = 16(sb&1) + 8k .. +8 of every sub-block.
+// ---------------------------------------------------------------------------------------------
+struct Q6Half {
+    uint2 ql[2][2];  // [p & 1][l / 16]
+    uint2 qh[2];     // [l / 16]
+};
+struct Q6Row {
+    Q6Half h[2];
+    uint4 scales;
+    float d;
+};
+
+__device__ __forceinline__ Q6Row q6_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q6Row r;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int lh = 0; lh < 2; lh++) r.h[h].ql[a][lh] = ld_u2_a2(blk + 64 * h + 32 * a + 16 * lh + 8 * khalf);
+#pragma unroll
+        for (int lh = 0; lh < 2; lh++) r.h[h].qh[lh] = ld_u2_a2(blk + 128 + 32 * h + 16 * lh + 8 * khalf);
+    }
+    r.scales = ld_u4_a2(blk + 192);
+    r.d = ld_f16(blk + 208);
+    return r;
+}
+
+// four 6-bit values (low 4 bits in `nib`, high 2 bits already at bit 4 in `two`) minus 32, as signed bytes: the sum
+// v + 0x60 never carries between bytes (v <= 63), and flipping bit 7 of v + 96 gives v - 32 modulo 256
+__device__ __forceinline__ uint32_t q6_signed(uint32_t nib, uint32_t two) {
+    return ((nib | two) + 0x60606060u) ^ 0x80808080u;
+}
+
+template <int kSb>
+__device__ __forceinline__ long q6_operand(const Q6Row &r) {
+    constexpr int h = kSb >> 3, p = (kSb >> 1) & 3, lh = kSb & 1;
+    const uint2 ql = r.h[h].ql[p & 1][lh], qh = r.h[h].qh[lh];
+    uint32_t n0, n1, t0, t1;
+    if constexpr ((p >> 1) == 0) {
+        n0 = ql.x & 0x0f0f0f0fu;
+        n1 = ql.y & 0x0f0f0f0fu;
+    } else {
+        n0 = (ql.x >> 4) & 0x0f0f0f0fu;
+        n1 = (ql.y >> 4) & 0x0f0f0f0fu;
+    }
+    if constexpr (p == 0) {
+        t0 = (qh.x << 4) & 0x30303030u;
+        t1 = (qh.y << 4) & 0x30303030u;
+    } else if constexpr (p == 1) {
+        t0 = (qh.x << 2) & 0x30303030u;
+        t1 = (qh.y << 2) & 0x30303030u;
+    } else if constexpr (p == 2) {
+        t0 = qh.x & 0x30303030u;
+        t1 = qh.y & 0x30303030u;
+    } else {
+        t0 = (qh.x >> 2) & 0x30303030u;
+        t1 = (qh.y >> 2) & 0x30303030u;
+    }
+    const uint32_t lo = q6_signed(n0, t0), hi = q6_signed(n1, t1);
+    return static_cast<long>(static_cast<unsigned long>(lo) | (static_cast<unsigned long>(hi) << 32));
+}
+
+template <int kSb>
+__device__ __forceinline__ int q6_scale(const Q6Row &r) {
+    const uint32_t word = kSb < 4 ? r.scales.x : (kSb < 8 ? r.scales.y : (kSb < 12 ? r.scales.z : r.scales.w));
+    return static_cast<int>(__builtin_amdgcn_sbfe(static_cast<int>(word), 8 * (kSb & 3), 8));
+}
+
+// cooperative copy of the workgroup's tokens' quantised activations of one 256-element block into LDS
+template <int kToks>
+struct Stage {
+    static constexpr int kChunks = kToks * 32 / kGbThreads;  // 8-byte chunks per thread
+    uint2 v[kChunks];
+    float dx;
+};
+
+template <int kToks>
+__device__ __forceinline__ void stage_load(Stage<kToks> &st, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                           uint32_t tok0, uint32_t last_tok, size_t blocks_per_tok, size_t b, int tid) {
+#pragma unroll
+    for (int i = 0; i < Stage<kToks>::kChunks; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        const uint32_t t = min(tok0 + (c >> 5), last_tok);
+        st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(t) * blocks_per_tok + b) * 256 + (c & 31) * 8);
+    }
+    st.dx = 0.0f;
+    if (tid < kToks) st.dx = ad[static_cast<size_t>(min(tok0 + tid, last_tok)) * blocks_per_tok + b];
+}
+
+template <int kToks>
+__device__ __forceinline__ void stage_store(const Stage<kToks> &st, uint8_t *abuf, float *dxbuf, int tid) {
+#pragma unroll
+    for (int i = 0; i < Stage<kToks>::kChunks; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kGbStride64 + (c & 31) * 8) = st.v[i];
+    }
+    if (tid < kToks) dxbuf[tid] = st.dx;
+}
+
+template <int kTT>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    gemm_q6k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                         float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq) {
+    constexpr int kToks = 32 * kTT;
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride64];
+    __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kQ6KBytes;
+
+    float accf[kTT][16];
+    int tot[kTT][16];
+#pragma unroll
+    for (int t = 0; t < kTT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            accf[t][i] = 0.0f;
+            tot[t][i] = 0;
+        }
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    Stage<kToks> st;
+    stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, 0, tid);
+    Q6Row cur = q6_load_row(wrow, khalf);
+    stage_store<kToks>(st, s_a[0], s_dx[0], tid);
+    __syncthreads();
+
+    for (uint32_t b = 0; b < nb; b++) {
+        const int buf = b & 1;
+        const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
+        stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, bn, tid);
+        const Q6Row nxt = q6_load_row(wrow + static_cast<size_t>(bn) * kQ6KBytes, khalf);
+        const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
+
+        // one 16-element sub-block: operand from the packed row, one matrix instruction per token tile, the sub-block's
+        // scale applied to the 16 results.  The empty asm and the scheduling barrier keep the sub-blocks in order: left
+        // alone the compiler turns each result's sixteen additions into a tree and keeps all 256 products alive.
+#define RNB_Q6_SUB_BLOCK(SB)                                                                                           \
+    {                                                                                                                  \
+        const long bop = q6_operand<SB>(cur);                                                                          \
+        const int sc = q6_scale<SB>(cur);                                                                              \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
+            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
+            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 32 * 127 */                                          \
+                asm volatile("" : "+v"(tot[t][i])); /* no re-association of the sixteen sums into a tree */            \
+            }                                                                                                          \
+        }                                                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                                             \
+    }
+        RNB_Q6_SUB_BLOCK(0)
+        RNB_Q6_SUB_BLOCK(1)
+        RNB_Q6_SUB_BLOCK(2)
+        RNB_Q6_SUB_BLOCK(3)
+        RNB_Q6_SUB_BLOCK(4)
+        RNB_Q6_SUB_BLOCK(5)
+        RNB_Q6_SUB_BLOCK(6)
+        RNB_Q6_SUB_BLOCK(7)
+        RNB_Q6_SUB_BLOCK(8)
+        RNB_Q6_SUB_BLOCK(9)
+        RNB_Q6_SUB_BLOCK(10)
+        RNB_Q6_SUB_BLOCK(11)
+        RNB_Q6_SUB_BLOCK(12)
+        RNB_Q6_SUB_BLOCK(13)
+        RNB_Q6_SUB_BLOCK(14)
+        RNB_Q6_SUB_BLOCK(15)
+#undef RNB_Q6_SUB_BLOCK
+
+        // out += (d * d_x) * float(sum): result i of a tile is token 8 * (i / 4) + 4 * khalf + i % 4
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
+                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = 4 * j + i;
+                    accf[t][r] += (cur.d * dx[i]) * static_cast<float>(tot[t][r]);
+                    tot[t][r] = 0;
+                }
+            }
+        stage_store<kToks>(st, s_a[buf ^ 1], s_dx[buf ^ 1], tid);
+        cur = nxt;
+        __syncthreads();
+    }
+
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
+                if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q8_0 {f16 d, i8 qs[32]} (34 bytes) and Q8_1 {f16 d, f16 s, i8 qs[32]} (36 bytes) against 32-wide Q8 activations
+// (one f32 scale per 32 elements).  A step covers 8 blocks = 256 elements, staged exactly like a Q8_K block.
+// ---------------------------------------------------------------------------------------------
+struct Q8Blocks {
+    uint4 q[8];  // the lane's 16 codes (K-half) of each of the 8 blocks
+    float d[8];
+};
+
+template <int kBlockBytes, int kQsOff>
+__device__ __forceinline__ Q8Blocks q8_load_blocks(const uint8_t *__restrict__ rowp, uint32_t blk0, uint32_t nb32, int khalf) {
+    Q8Blocks r;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const uint32_t b = min(blk0 + k, nb32 - 1);  // a partial last step repeats the last block; its results are dropped
+        const uint8_t *blk = rowp + static_cast<size_t>(b) * kBlockBytes;
+        r.q[k] = ld_u4_a2(blk + kQsOff + 16 * khalf);
+        r.d[k] = ld_f16(blk);
+    }
+    return r;
+}
+
+template <int kTT, int kBlockBytes, int kQsOff>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    gemm_q8_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                        float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq) {
+    constexpr int kToks = 32 * kTT;
+    constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride128];
+    __shared__ __attribute__((aligned(16))) float s_dx[2][8][kToks];  // [block of the step][token]
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb32 * kBlockBytes;
+    const uint32_t steps = (nb32 + 7) / 8;
+    const size_t tok_bytes = static_cast<size_t>(nb32) * 32;
+
+    float accf[kTT][16];
+#pragma unroll
+    for (int t = 0; t < kTT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) accf[t][i] = 0.0f;
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    uint2 sv[kToks * 32 / kGbThreads];
+    float sdx[kDxPerThread];
+    auto stage_load8 = [&](uint32_t step) {
+#pragma unroll
+        for (int i = 0; i < kToks * 32 / kGbThreads; i++) {
+            const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+            const uint32_t t = min(tok0 + (c >> 5), last_tok);
+            // 8-byte chunk (c & 31) of the step; chunks past the end of the row re-read the row's last 8 bytes
+            const size_t off = min(static_cast<size_t>(step) * 256 + (c & 31) * 8, tok_bytes - 8);
+            sv[i] = *reinterpret_cast<const uint2 *>(aq + static_cast<size_t>(t) * tok_bytes + off);
+        }
+#pragma unroll
+        for (int i = 0; i < kDxPerThread; i++) {
+            const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;  // c = block-in-step * kToks + token
+            const uint32_t t = min(tok0 + c % kToks, last_tok);
+            const uint32_t blk = min(step * 8 + c / kToks, nb32 - 1);
+            sdx[i] = ad[static_cast<size_t>(t) * nb32 + blk];
+        }
+    };
+    auto stage_store8 = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kToks * 32 / kGbThreads; i++) {
+            const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+            *reinterpret_cast<uint2 *>(s_a[buf] + (c >> 5) * kGbStride128 + (c & 31) * 8) = sv[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kDxPerThread; i++) {
+            const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+            s_dx[buf][c / kToks][c % kToks] = sdx[i];
+        }
+    };
+
+    stage_load8(0);
+    Q8Blocks cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, 0, nb32, khalf);
+    stage_store8(0);
+    __syncthreads();
+
+    for (uint32_t step = 0; step < steps; step++) {
+        const int buf = step & 1;
+        const uint32_t sn = step + 1 < steps ? step + 1 : step;
+        stage_load8(sn);
+        const Q8Blocks nxt = q8_load_blocks<kBlockBytes, kQsOff>(wrow, sn * 8, nb32, khalf);
+        const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
+        const uint32_t live = min(8u, nb32 - step * 8);  // blocks of this step that exist (workgroup-uniform)
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (static_cast<uint32_t>(k) < live) {
+                const v4i bop = {static_cast<int>(cur.q[k].x), static_cast<int>(cur.q[k].y), static_cast<int>(cur.q[k].z),
+                                 static_cast<int>(cur.q[k].w)};
+#pragma unroll
+                for (int t = 0; t < kTT; t++) {
+                    const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * k);
+                    const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf][k])[8 * t + 2 * j + khalf];
+                        const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            accf[t][4 * j + i] += (cur.d[k] * dx[i]) * static_cast<float>(acc[4 * j + i]);
+                    }
+                }
+            }
+        }
+        stage_store8(buf ^ 1);
+        cur = nxt;
+        __syncthreads();
+    }
+
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
+                if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
+            }
+    }
+}
+
+}  // namespace
+
+void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb == 0) return;
+    const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    if (seq > 32) {
+        const dim3 grid(row_tiles, (seq + 63) / 64, 1);
+        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, out, rows, nb, seq);
+    } else {
+        const dim3 grid(row_tiles, 1, 1);
+        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, out, rows, nb, seq);
+    }
+}
+
+bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32) { return (quant == kQ8_0 || quant == kQ8_1) && nb32 >= 1; }
+
+void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
+                         uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb32 == 0) return;
+    const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    const bool wide = seq > 32;
+    const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, 1), block(kGbThreads);
+#define RNB_LAUNCH_Q8(TT, BYTES, OFF) \
+    hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF>), grid, block, 0, stream, w, act.qs, act.d, out, rows, nb32, seq)
+    if (quant == kQ8_0) {
+        if (wide)
+            RNB_LAUNCH_Q8(2, 34, 2);
+        else
+            RNB_LAUNCH_Q8(1, 34, 2);
+    } else {
+        if (wide)
+            RNB_LAUNCH_Q8(2, 36, 4);
+        else
+            RNB_LAUNCH_Q8(1, 36, 4);
+    }
+#undef RNB_LAUNCH_Q8
+}
+
+}  // namespace rnb

@@ -377,6 +377,56 @@ def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
                 f"gemm rows {rows} nblk {nblk} seq {seq}")
 
 
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
+                                           (1, 1, 16), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
+def test_q6k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
+    """16 or more tokens on Q6_K take the matrix-core GEMM (one K=16 instruction per sub-block, sub-block scales on
+    the vector units): row and token counts off the 128 x 32 / 64 tile, one token tile and two."""
+    cols = nblk * 256
+    w = oracle.make_weights(Q6_K, rows, cols, 170 + rows)
+    x = oracle.fill_normal(seq * cols, 180 + seq, 1.0)
+    got = rnb.q6k_gemv_batch(w, rows, cols, x)
+    check_close(got, oracle.gemv(Q6_K, w, rows, cols, x), oracle.gemv(Q6_K, w, rows, cols, x, gold=True),
+                f"q6k gemm rows {rows} nblk {nblk} seq {seq}")
+    # a token's row does not depend on the batch around it: the same bits with the tokens reversed
+    rev = rnb.q6k_gemv_batch(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
+def test_q6k_gemm_extreme_blocks(rnb, oracle):
+    """every 6-bit code at both ends of its range, scales -128 / 127 / 0, zero and subnormal d, zero activations"""
+    rng = np.random.default_rng(19)
+    rows, nblk, seq = 40, 3, 24
+    blocks = []
+    for i in range(rows * nblk):
+        q = [np.full(256, 63), np.zeros(256), rng.integers(0, 64, 256), np.tile([0, 63], 128)][i % 4]
+        sc = [np.full(16, 127), np.full(16, -128), rng.integers(-128, 128, 16), np.zeros(16)][(i // 4) % 4]
+        blocks.append(npref.make_q6k_block([1.0, 6e-8, 0.0, 2.0 ** -14, -0.5][i % 5], sc, q))
+    w = np.concatenate(blocks)
+    x = oracle.fill_normal(seq * nblk * 256, 18, 1.0).reshape(seq, -1)
+    x[3, 256:512] = 0.0
+    x[5] = 0.0
+    got = rnb.q6k_gemv_batch(w, rows, nblk * 256, x)
+    assert np.all(got[5] == 0.0)
+    check_close(got, oracle.gemv(Q6_K, w, rows, nblk * 256, x), oracle.gemv(Q6_K, w, rows, nblk * 256, x, gold=True),
+                "q6k gemm extremes")
+
+
+@pytest.mark.parametrize("quant", [Q8_0, Q8_1])
+@pytest.mark.parametrize("rows,cols,seq", [(32, 32, 16), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
+                                           (1, 4096, 16), (300, 288, 100)])
+def test_q8_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, cols, seq):
+    """16 or more tokens on Q8_0 / Q8_1 take the matrix-core GEMM (one K=32 instruction per block, the two f32 scales on
+    the vector units): block counts off the 8-block step, rows and tokens off the tile."""
+    w = oracle.make_weights(quant, rows, cols, 270 + rows)
+    x = oracle.fill_normal(seq * cols, 280 + seq, 1.0)
+    got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"q8 gemm quant {quant} rows {rows} cols {cols} seq {seq}")
+    rev = gemv_fn(rnb, quant, True)(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
 def test_q4k_gemm_extreme_blocks(rnb, oracle):
     rng = np.random.default_rng(17)
     rows, nblk, seq = 40, 3, 24
