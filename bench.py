@@ -569,7 +569,8 @@ def main() -> int:
         except Exception as exc:
             sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"error": str(exc)}
         # prefill on the formats whose scales cannot ride on an int8 operand (scale groups applied on the vector units)
-        for key, quant, r, c in (("q6k_gemm_512x14336_to_4096", Q6_K, 4096, 14336), ("q8_0_gemm_512x4096_to_4096", Q8_0, 4096, 4096)):
+        for key, quant, r, c in (("q6k_gemm_512x14336_to_4096", Q6_K, 4096, 14336), ("q5k_gemm_512x4096_to_14336", Q5_K, 14336, 4096),
+                                 ("q8_0_gemm_512x4096_to_4096", Q8_0, 4096, 4096)):
             try:
                 res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, 512, 20, 3, 101, key, want_graph=False)
                 ops = 2 * 512 * r * c

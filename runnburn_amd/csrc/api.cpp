@@ -132,7 +132,9 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ5K) {
-        if (seq >= kTokensMinSeq)
+        if (seq >= kGemmMinSeq && act.digits != nullptr)
+            launch_gemm_q5k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
+        else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ5K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);

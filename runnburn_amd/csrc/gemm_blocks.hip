@@ -1,11 +1,14 @@
-// Prefill GEMM for the formats whose scales do not fold onto an int8 operand: Q6_K (int8 scale per 16 elements) and
-// the 32-element byte formats Q8_0 / Q8_1 (f16 scale per 32 elements).  out[seq][rows], same contract as the GEMVs.
+// Prefill GEMM for the formats whose scales do not fold onto an int8 operand: Q6_K (int8 scale per 16 elements), Q5_K
+// (6-bit scale per 32 five-bit codes: scale times code needs 11 bits) and the 32-element byte formats Q8_0 / Q8_1 (f16
+// scale per 32 elements).  out[seq][rows], same contract as the GEMVs.
 //
 // The matrix cores do the integer part of one scale group per instruction and the vector units apply the group's scale
 // to the 16 results a lane holds:
 //   Q6_K   v_mfma_i32_32x32x16_i8 per 16-element sub-block: I_sb = sum (q - 32) * a  (exact), tot += sc[r][sb] * I_sb
 //          in 24-bit integer multiplies, and once per super-block out += (d[r] * d_x[s]) * float(tot): the arithmetic of
 //          crates/rnb-cpu/src/gemm/neon_dot.rs:2240-2288 (dot_q6_k_q8k_scalar).
+//   Q5_K   v_mfma_i32_32x32x32_i8 per 32-element sub-block, tot += sc * I_sb, the mins through two K=16 instructions on
+//          the quantiser's digits, out += d_x * (d * float(tot) - dmin * float(S)) per super-block.
 //   Q8_0   v_mfma_i32_32x32x32_i8 per 32-element block: out += (d[r][b] * d_x[s][b]) * float(I_b),
 //   Q8_1   crates/rnb-cpu/src/gemm/neon_dot.rs:376-436, neon_quant.rs:236-253.
 // That is 16 (Q6_K) or 48 (Q8) vector instructions per matrix instruction, so these kernels are bound by the vector
@@ -242,6 +245,159 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 }
 
 // ---------------------------------------------------------------------------------------------
+// Q5_K: block = {f16 d, f16 dmin, scales[12] (eight 6-bit scales and mins), qh[32], qs[128]}, 176 bytes.  Element
+// 64g + 32h + l = nibble h of qs[32g + l] | bit (2g + h) of qh[l] << 4 (0..31), sub-block 2g + h.  One K=32 matrix
+// instruction per sub-block, tot += sc * I_sb; the mins term S = sum mn * bsum32 rides on the matrix cores through the
+// quantiser's digits (bsum32 = b0 + 64 * b1): two K=16 instructions with eight live K slots per token tile.
+// Per super-block out += d_x * (d * float(tot) - dmin * float(S)): crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800.
+// ---------------------------------------------------------------------------------------------
+struct Q5Row {
+    uint4 hdr, qh;
+    uint4 qs[4];
+};
+
+__device__ __forceinline__ Q5Row q5_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q5Row r;
+    r.hdr = ld_u4_a2(blk);
+    r.qh = ld_u4_a2(blk + 16 + 16 * khalf);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + 48 + 32 * g + 16 * khalf);
+    return r;
+}
+
+template <int kSb>
+__device__ __forceinline__ uint32_t q5_codes(uint32_t qs, uint32_t qh) {
+    const uint32_t nib = (kSb & 1) ? (qs >> 4) & 0x0f0f0f0fu : qs & 0x0f0f0f0fu;
+    const uint32_t fifth = kSb <= 4 ? (qh << (4 - kSb)) & 0x10101010u : (qh >> (kSb - 4)) & 0x10101010u;
+    return nib | fifth;
+}
+
+template <int kTT>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    gemm_q5k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                         const uint8_t *__restrict__ adig, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                         uint32_t seq) {
+    constexpr int kToks = 32 * kTT;
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride128];
+    __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
+    __shared__ __attribute__((aligned(16))) uint4 s_dig[2][kToks];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kQ5KBytes;
+
+    float accf[kTT][16];
+    int tot[kTT][16];
+#pragma unroll
+    for (int t = 0; t < kTT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            accf[t][i] = 0.0f;
+            tot[t][i] = 0;
+        }
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    Stage<kToks> st;
+    uint4 sdig = make_uint4(0, 0, 0, 0);
+    auto stage_load5 = [&](uint32_t b) {
+        stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, b, tid);
+        if (tid < kToks)
+            sdig = *reinterpret_cast<const uint4 *>(adig + (static_cast<size_t>(min(tok0 + tid, last_tok)) * nb + b) * 16);
+    };
+    auto stage_store5 = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < Stage<kToks>::kChunks; i++) {
+            const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+            *reinterpret_cast<uint2 *>(s_a[buf] + (c >> 5) * kGbStride128 + (c & 31) * 8) = st.v[i];
+        }
+        if (tid < kToks) {
+            s_dx[buf][tid] = st.dx;
+            s_dig[buf][tid] = sdig;
+        }
+    };
+    stage_load5(0);
+    Q5Row cur = q5_load_row(wrow, khalf);
+    stage_store5(0);
+    __syncthreads();
+
+    for (uint32_t b = 0; b < nb; b++) {
+        const int buf = b & 1;
+        const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
+        stage_load5(bn);
+        const Q5Row nxt = q5_load_row(wrow + static_cast<size_t>(bn) * kQ5KBytes, khalf);
+        const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
+        const Q4KScales sc8 = unpack_q4k_scales(cur.hdr.y, cur.hdr.z, cur.hdr.w);
+
+#define RNB_Q5_SUB_BLOCK(SB)                                                                                           \
+    {                                                                                                                  \
+        const uint4 qs = cur.qs[(SB) >> 1];                                                                            \
+        const v4i bop = {static_cast<int>(q5_codes<SB>(qs.x, cur.qh.x)), static_cast<int>(q5_codes<SB>(qs.y, cur.qh.y)), \
+                         static_cast<int>(q5_codes<SB>(qs.z, cur.qh.z)), static_cast<int>(q5_codes<SB>(qs.w, cur.qh.w))}; \
+        const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                              \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * (SB));                 \
+            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);                         \
+            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 32 * 31 * 127 */                                          \
+                asm volatile("" : "+v"(tot[t][i])); /* no re-association of the eight sums into a tree */              \
+            }                                                                                                          \
+        }                                                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                                             \
+    }
+        RNB_Q5_SUB_BLOCK(0)
+        RNB_Q5_SUB_BLOCK(1)
+        RNB_Q5_SUB_BLOCK(2)
+        RNB_Q5_SUB_BLOCK(3)
+        RNB_Q5_SUB_BLOCK(4)
+        RNB_Q5_SUB_BLOCK(5)
+        RNB_Q5_SUB_BLOCK(6)
+        RNB_Q5_SUB_BLOCK(7)
+#undef RNB_Q5_SUB_BLOCK
+
+        // mins: K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
+        const float d = f16_bits_to_f32(cur.hdr.x), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+        const long mnop = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(sc8.mn_lo) |
+                                                         (static_cast<unsigned long>(sc8.mn_hi) << 32))
+                                     : 0L;
+#pragma unroll
+        for (int t = 0; t < kTT; t++) {
+            const uint4 dig = s_dig[buf][32 * t + lrow];
+            const long op0 = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(dig.x) | (static_cast<unsigned long>(dig.y) << 32)) : 0L;
+            const long op1 = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(dig.z) | (static_cast<unsigned long>(dig.w) << 32)) : 0L;
+            const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op0, mnop, zero16, 0, 0, 0);
+            const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op1, mnop, zero16, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
+                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = 4 * j + i;
+                    const int smin = c0[r] + 64 * c1[r];
+                    accf[t][r] += dx[i] * (d * static_cast<float>(tot[t][r]) - dmin * static_cast<float>(smin));
+                    tot[t][r] = 0;
+                }
+            }
+        }
+        stage_store5(buf ^ 1);
+        cur = nxt;
+        __syncthreads();
+    }
+
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
+                if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Q8_0 {f16 d, i8 qs[32]} (34 bytes) and Q8_1 {f16 d, f16 s, i8 qs[32]} (36 bytes) against 32-wide Q8 activations
 // (one f32 scale per 32 elements).  A step covers 8 blocks = 256 elements, staged exactly like a Q8_K block.
 // ---------------------------------------------------------------------------------------------
@@ -379,6 +535,21 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t ro
     } else {
         const dim3 grid(row_tiles, 1, 1);
         hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, out, rows, nb, seq);
+    }
+}
+
+void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb == 0) return;
+    const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    if (seq > 32) {
+        const dim3 grid(row_tiles, (seq + 63) / 64, 1);
+        hipLaunchKernelGGL(gemm_q5k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits, out, rows,
+                           nb, seq);
+    } else {
+        const dim3 grid(row_tiles, 1, 1);
+        hipLaunchKernelGGL(gemm_q5k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits, out, rows,
+                           nb, seq);
     }
 }
 

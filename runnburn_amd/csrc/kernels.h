@@ -85,9 +85,12 @@ void launch_act_mul(const float *gate, const float *up, float *out, size_t n, bo
 void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);
 
-// Q6_K x Q8_K and Q8_0 / Q8_1 x Q8 GEMMs on int8 MFMA (scale groups applied on the vector units); same contracts as
+// Q6_K / Q5_K x Q8_K and Q8_0 / Q8_1 x Q8 GEMMs on int8 MFMA (scale groups applied on the vector units); same contracts as
 // launch_gemv_q6k / launch_gemv_block32, intended for seq >= 16
 void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream);
+// Q5_K needs act.digits (the quantiser writes them for 16+ tokens)
+void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                           hipStream_t stream);
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32);
 void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,

@@ -412,6 +412,44 @@ def test_q6k_gemm_extreme_blocks(rnb, oracle):
                 "q6k gemm extremes")
 
 
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
+                                           (1, 1, 16), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
+def test_q5k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
+    """16 or more tokens on Q5_K: one K=32 matrix instruction per sub-block, 6-bit scales on the vector units, the mins
+    term through the quantiser's digits."""
+    cols = nblk * 256
+    w = oracle.make_weights(Q5_K, rows, cols, 470 + rows)
+    x = oracle.fill_normal(seq * cols, 480 + seq, 1.0)
+    got = rnb.q5k_gemv_batch(w, rows, cols, x)
+    check_close(got, oracle.gemv(Q5_K, w, rows, cols, x), oracle.gemv(Q5_K, w, rows, cols, x, gold=True),
+                f"q5k gemm rows {rows} nblk {nblk} seq {seq}")
+    rev = rnb.q5k_gemv_batch(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
+def test_q5k_gemm_extreme_blocks(rnb, oracle):
+    """all-31 and all-0 codes, alternating 16 / 15 (fifth bit on and off), scales and mins 63, zero / subnormal d and
+    dmin, activations whose 32-element sums reach the digits' ends (all 127, all -127 -> rounds to -127), a zero token"""
+    rng = np.random.default_rng(23)
+    rows, nblk, seq = 40, 3, 24
+    blocks = []
+    for i in range(rows * nblk):
+        vals = [np.full(256, 31), rng.integers(0, 32, 256), np.tile([16, 15], 128), np.zeros(256)][i % 4]
+        blocks.append(npref.make_q5k_block([1.0, 0.0, 6e-8, 2.0 ** -14][i % 4], [0.5, 6e-8, 0.0, 1.0][(i // 2) % 4],
+                                           np.full(8, 63) if i % 3 else rng.integers(0, 64, 8),
+                                           np.full(8, 63) if i % 5 else rng.integers(0, 64, 8), vals))
+    w = np.concatenate(blocks)
+    x = oracle.fill_normal(seq * nblk * 256, 18, 1.0).reshape(seq, -1)
+    x[3, 256:512] = 0.0
+    x[5] = 0.0
+    x[7] = 3.0       # every quantised value 127... the sign rule makes them -127: sums at the negative end
+    x[8] = -3.0
+    got = rnb.q5k_gemv_batch(w, rows, nblk * 256, x)
+    assert np.all(got[5] == 0.0)
+    check_close(got, oracle.gemv(Q5_K, w, rows, nblk * 256, x), oracle.gemv(Q5_K, w, rows, nblk * 256, x, gold=True),
+                "q5k gemm extremes")
+
+
 @pytest.mark.parametrize("quant", [Q8_0, Q8_1])
 @pytest.mark.parametrize("rows,cols,seq", [(32, 32, 16), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
                                            (1, 4096, 16), (300, 288, 100)])
