@@ -407,7 +407,12 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     // one table image: route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] | grp_expert[G] |
     // grp_start[G+1] | slot_expert[n]
     const size_t table_words = 5 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
-    const bool inline_tables = table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
+    // Batches with at least four slots per routed expert on average: the expert GEMMs run on the matrix cores (a
+    // 32-token tile costs the same whatever its number of live tokens, the integer-dot kernels cost per token; measured
+    // crossover on 128 experts x top-8: 64 tokens) and need the quantiser's digits
+    const bool mfma = token_count >= kGemmMinSeq && n_slots >= 4 * n_groups &&
+                      moe_mfma_supported(static_cast<uint32_t>(sh.nb_in), static_cast<uint32_t>(sh.nb_mid), down_quant);
+    const bool inline_tables = !mfma && table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
     MoeInlineTables inl;
     uint32_t *h = inl.words;
     TableSlot *ring_slot = nullptr;
@@ -482,6 +487,25 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     HIP_TRY(s.moe_mid_d.reserve(n_slots * sh.nb_mid * sizeof(float)));
     HIP_TRY(s.moe_mid_bsums.reserve(n_slots * sh.nb_mid * 16 * sizeof(int16_t)));
     HIP_TRY(s.moe_slot_out.reserve(n_slots * n_embd * sizeof(float)));
+    if (mfma && act.digits != nullptr) {
+        // prefill: grouped GEMMs, 32-token tiles per expert
+        uint8_t *mid_digits = nullptr;
+        if (down_quant != kQ6K) {  // Q4_K / Q5_K mins need the 32-element sums' digits
+            HIP_TRY(s.moe_mid_digits.reserve(n_slots * sh.nb_mid * 16));
+            mid_digits = s.moe_mid_digits.as<uint8_t>();
+        }
+        launch_moe_gate_up_mfma(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
+                                static_cast<uint32_t>(sh.nb_in), s.stream);
+        launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
+                            s.moe_mid_bsums.as<int16_t>(), mid_digits, s.stream);
+        const ActView mid_act{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>(), mid_digits};
+        launch_moe_down_mfma(down_dev, down_quant, mid_act, groups, d_route, s.moe_slot_out.as<float>(),
+                             static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
+        launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
+                          static_cast<uint32_t>(n_embd), s.stream);
+        HIP_TRY(hipGetLastError());
+        return RNB_HIP_OK;
+    }
     launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
     launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),

@@ -1,0 +1,149 @@
+// Pieces shared by the matrix-core kernels for the formats whose scale groups are applied on the vector units
+// (gemm_blocks.hip: dense prefill GEMMs; moe_mfma.hip: the grouped expert GEMMs): how a lane that owns a weight row
+// loads its share of a block, turns a scale group into an int8 MFMA operand, and how a workgroup stages its tokens'
+// quantised activations in LDS.  Lane = (row lane % 32, K-half lane / 32).
+#pragma once
+
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace rnb {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kGbWaves = 4;
+constexpr int kGbThreads = kWave * kGbWaves;
+constexpr int kGbRows = 32 * kGbWaves;  // 128 rows per workgroup
+constexpr int kGbStride64 = 264;   // bytes per staged token row for 64-bit operand reads (256 + 8): bank-conflict free
+constexpr int kGbStride128 = 272;  // ... and for 128-bit operand reads (256 + 16, keeps them 16-byte aligned)
+
+// ---------------------------------------------------------------------------------------------
+// Q6_K: block = {ql[128], qh[64], i8 scales[16], f16 d}, 210 bytes, 2-byte aligned.  Element 128h + 32p + l
+// (h = half, p = quarter, l < 32) = ((ql[64h + 32(p&1) + l] >> 4(p>>1)) & 15 | ((qh[32h + l] >> 2p) & 3) << 4) - 32, its
+// 16-element sub-block is 8h + 2p + l/16.  The lane of K-half k takes l = 16(sb&1) + 8k .. +8 of every sub-block.
+// ---------------------------------------------------------------------------------------------
+struct Q6Half {
+    uint2 ql[2][2];  // [p & 1][l / 16]
+    uint2 qh[2];     // [l / 16]
+};
+struct Q6Row {
+    Q6Half h[2];
+    uint4 scales;
+    float d;
+};
+
+__device__ __forceinline__ Q6Row q6_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q6Row r;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int lh = 0; lh < 2; lh++) r.h[h].ql[a][lh] = ld_u2_a2(blk + 64 * h + 32 * a + 16 * lh + 8 * khalf);
+#pragma unroll
+        for (int lh = 0; lh < 2; lh++) r.h[h].qh[lh] = ld_u2_a2(blk + 128 + 32 * h + 16 * lh + 8 * khalf);
+    }
+    r.scales = ld_u4_a2(blk + 192);
+    r.d = ld_f16(blk + 208);
+    return r;
+}
+
+// four 6-bit values (low 4 bits in `nib`, high 2 bits already at bit 4 in `two`) minus 32, as signed bytes: the sum
+// v + 0x60 never carries between bytes (v <= 63), and flipping bit 7 of v + 96 gives v - 32 modulo 256
+__device__ __forceinline__ uint32_t q6_signed(uint32_t nib, uint32_t two) {
+    return ((nib | two) + 0x60606060u) ^ 0x80808080u;
+}
+
+template <int kSb>
+__device__ __forceinline__ long q6_operand(const Q6Row &r) {
+    constexpr int h = kSb >> 3, p = (kSb >> 1) & 3, lh = kSb & 1;
+    const uint2 ql = r.h[h].ql[p & 1][lh], qh = r.h[h].qh[lh];
+    uint32_t n0, n1, t0, t1;
+    if constexpr ((p >> 1) == 0) {
+        n0 = ql.x & 0x0f0f0f0fu;
+        n1 = ql.y & 0x0f0f0f0fu;
+    } else {
+        n0 = (ql.x >> 4) & 0x0f0f0f0fu;
+        n1 = (ql.y >> 4) & 0x0f0f0f0fu;
+    }
+    if constexpr (p == 0) {
+        t0 = (qh.x << 4) & 0x30303030u;
+        t1 = (qh.y << 4) & 0x30303030u;
+    } else if constexpr (p == 1) {
+        t0 = (qh.x << 2) & 0x30303030u;
+        t1 = (qh.y << 2) & 0x30303030u;
+    } else if constexpr (p == 2) {
+        t0 = qh.x & 0x30303030u;
+        t1 = qh.y & 0x30303030u;
+    } else {
+        t0 = (qh.x >> 2) & 0x30303030u;
+        t1 = (qh.y >> 2) & 0x30303030u;
+    }
+    const uint32_t lo = q6_signed(n0, t0), hi = q6_signed(n1, t1);
+    return static_cast<long>(static_cast<unsigned long>(lo) | (static_cast<unsigned long>(hi) << 32));
+}
+
+template <int kSb>
+__device__ __forceinline__ int q6_scale(const Q6Row &r) {
+    const uint32_t word = kSb < 4 ? r.scales.x : (kSb < 8 ? r.scales.y : (kSb < 12 ? r.scales.z : r.scales.w));
+    return static_cast<int>(__builtin_amdgcn_sbfe(static_cast<int>(word), 8 * (kSb & 3), 8));
+}
+
+// cooperative copy of the workgroup's tokens' quantised activations of one 256-element block into LDS
+template <int kToks>
+struct Stage {
+    static constexpr int kChunks = kToks * 32 / kGbThreads;  // 8-byte chunks per thread
+    uint2 v[kChunks];
+    float dx;
+};
+
+template <int kToks>
+__device__ __forceinline__ void stage_load(Stage<kToks> &st, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                           uint32_t tok0, uint32_t last_tok, size_t blocks_per_tok, size_t b, int tid) {
+#pragma unroll
+    for (int i = 0; i < Stage<kToks>::kChunks; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        const uint32_t t = min(tok0 + (c >> 5), last_tok);
+        st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(t) * blocks_per_tok + b) * 256 + (c & 31) * 8);
+    }
+    st.dx = 0.0f;
+    if (tid < kToks) st.dx = ad[static_cast<size_t>(min(tok0 + tid, last_tok)) * blocks_per_tok + b];
+}
+
+template <int kToks>
+__device__ __forceinline__ void stage_store(const Stage<kToks> &st, uint8_t *abuf, float *dxbuf, int tid) {
+#pragma unroll
+    for (int i = 0; i < Stage<kToks>::kChunks; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kGbStride64 + (c & 31) * 8) = st.v[i];
+    }
+    if (tid < kToks) dxbuf[tid] = st.dx;
+}
+
+struct Q5Row {
+    uint4 hdr, qh;
+    uint4 qs[4];
+};
+
+__device__ __forceinline__ Q5Row q5_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q5Row r;
+    r.hdr = ld_u4_a2(blk);
+    r.qh = ld_u4_a2(blk + 16 + 16 * khalf);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + 48 + 32 * g + 16 * khalf);
+    return r;
+}
+
+template <int kSb>
+__device__ __forceinline__ uint32_t q5_codes(uint32_t qs, uint32_t qh) {
+    const uint32_t nib = (kSb & 1) ? (qs >> 4) & 0x0f0f0f0fu : qs & 0x0f0f0f0fu;
+    const uint32_t fifth = kSb <= 4 ? (qh << (4 - kSb)) & 0x10101010u : (qh >> (kSb - 4)) & 0x10101010u;
+    return nib | fifth;
+}
+
+}  // namespace
+
+}  // namespace rnb

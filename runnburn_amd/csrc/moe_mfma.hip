@@ -1,0 +1,401 @@
+// Gathered sparse-MoE experts for batches (prefill) on the matrix cores: the grouped form of gemm_blocks.hip.
+// Slots are sorted by expert on the host (api.cpp); workgroup (row tile, expert group) walks the group's slots in tiles
+// of 32 tokens: the tokens' quantised activations are gathered into LDS by the sorted lists, the expert's weight rows go
+// from global memory to the registers of the lane that owns the row, one int8 matrix instruction per scale group, the
+// group's scale on the vector units (see gemm_blocks.hip).  With a handful of tokens per expert most of a 32-token tile
+// is padding, which costs nothing extra: the vector work per tile is the same whatever the number of live tokens, and
+// it is a third of what the integer-dot kernels of moe.hip spend per token.
+//   gate/up   mid[slot][n_ff] = silu(Wg[e] . a_tok) * (Wu[e] . a_tok), both Q4_K: the two matrices share the activation
+//             operand of every instruction                        fanout.rs:260-327, activation.rs:73-89
+//   down      slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])), Q4_K, Q5_K or Q6_K
+// (crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs, crates/rnb-cpu/src/kernels/activation.rs)
+#include "device_utils.h"
+#include "kernels.h"
+#include "mfma_blocks.h"
+
+namespace rnb {
+
+namespace {
+
+constexpr int kMmToks = 32;  // tokens per tile
+
+// the tile's list entries: activation row, output row (0xffffffff past the end of the group) and output scale
+struct TileMap {
+    uint32_t act_row[kMmToks];
+    uint32_t out_row[kMmToks];
+    float scale[kMmToks];
+};
+
+__device__ __forceinline__ void tile_map_fill(TileMap &m, const uint32_t *__restrict__ act_idx, const uint32_t *__restrict__ out_idx,
+                                              const float *__restrict__ out_scale, uint32_t first, uint32_t left, int tid) {
+    if (tid < kMmToks) {
+        const bool live = static_cast<uint32_t>(tid) < left;
+        const uint32_t p = first + (live ? static_cast<uint32_t>(tid) : left - 1);  // padding repeats the last entry
+        m.act_row[tid] = act_idx[p];
+        const uint32_t o = out_idx[p];
+        m.out_row[tid] = live ? o : 0xffffffffu;
+        m.scale[tid] = out_scale != nullptr ? out_scale[o] : 1.0f;
+    }
+}
+
+// the tile's quantised activations of block b (256 int8 per token, 8-byte chunks), scale and digits
+struct TileStage {
+    uint2 v[kMmToks * 32 / kGbThreads];  // 4 chunks per thread
+    float dx;
+    uint4 dig;
+};
+
+template <bool kDigits>
+__device__ __forceinline__ void tile_stage_load(TileStage &st, const TileMap &m, const int8_t *__restrict__ aq,
+                                                const float *__restrict__ ad, const uint8_t *__restrict__ adig, size_t nb,
+                                                size_t b, int tid) {
+#pragma unroll
+    for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(m.act_row[c >> 5]) * nb + b) * 256 + (c & 31) * 8);
+    }
+    st.dx = 0.0f;
+    st.dig = make_uint4(0, 0, 0, 0);
+    if (tid < kMmToks) {
+        const size_t blk = static_cast<size_t>(m.act_row[tid]) * nb + b;
+        st.dx = ad[blk];
+        if constexpr (kDigits) st.dig = *reinterpret_cast<const uint4 *>(adig + blk * 16);
+    }
+}
+
+template <int kStride, bool kDigits>
+__device__ __forceinline__ void tile_stage_store(const TileStage &st, uint8_t *abuf, float *dxbuf, uint4 *digbuf, int tid) {
+#pragma unroll
+    for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+        *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kStride + (c & 31) * 8) = st.v[i];
+    }
+    if (tid < kMmToks) {
+        dxbuf[tid] = st.dx;
+        if constexpr (kDigits) digbuf[tid] = st.dig;
+    }
+}
+
+// Q4_K / Q5_K row share of a block: header, (fifth bits,) the K-half's 16 bytes of every 32-byte nibble group
+template <bool kFifth>
+__device__ __forceinline__ Q5Row q45_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q5Row r;
+    r.hdr = ld_u4_a2(blk);
+    r.qh = make_uint4(0, 0, 0, 0);
+    if constexpr (kFifth) r.qh = ld_u4_a2(blk + 16 + 16 * khalf);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + (kFifth ? 48 : 16) + 32 * g + 16 * khalf);
+    return r;
+}
+
+template <int kSb, bool kFifth>
+__device__ __forceinline__ v4i q45_operand(const Q5Row &r) {
+    const uint4 qs = r.qs[kSb >> 1];
+    if constexpr (kFifth) {
+        return v4i{static_cast<int>(q5_codes<kSb>(qs.x, r.qh.x)), static_cast<int>(q5_codes<kSb>(qs.y, r.qh.y)),
+                   static_cast<int>(q5_codes<kSb>(qs.z, r.qh.z)), static_cast<int>(q5_codes<kSb>(qs.w, r.qh.w))};
+    } else {
+        constexpr int sh = (kSb & 1) * 4;
+        return v4i{static_cast<int>((qs.x >> sh) & 0x0f0f0f0fu), static_cast<int>((qs.y >> sh) & 0x0f0f0f0fu),
+                   static_cast<int>((qs.z >> sh) & 0x0f0f0f0fu), static_cast<int>((qs.w >> sh) & 0x0f0f0f0fu)};
+    }
+}
+
+// One super-block of one 32-token tile against one Q4_K / Q5_K row share: I = sum_sb sc * (codes . a) and the mins sum
+// S = sum_sb mn * bsum32 (through the digits); returns d * I - dmin * S per result in `val`.
+#define RNB_Q45_SUB_BLOCK(SB, ROW, TOT)                                                                  \
+    {                                                                                                    \
+        const v4i bop = q45_operand<SB, kFifth>(ROW);                                                    \
+        const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                \
+        const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * (SB));                               \
+        const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);               \
+        _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                 \
+            TOT[i] += mul24(acc[i], sc);                                                                 \
+            asm volatile("" : "+v"(TOT[i])); /* keep the eight additions a chain, not a tree */          \
+        }                                                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+    }
+
+template <bool kFifth>
+__device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *abase, const uint4 dig, int khalf,
+                                               float (&val)[16]) {
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const Q4KScales sc8 = unpack_q4k_scales(row.hdr.y, row.hdr.z, row.hdr.w);
+    int tot[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) tot[i] = 0;
+    RNB_Q45_SUB_BLOCK(0, row, tot)
+    RNB_Q45_SUB_BLOCK(1, row, tot)
+    RNB_Q45_SUB_BLOCK(2, row, tot)
+    RNB_Q45_SUB_BLOCK(3, row, tot)
+    RNB_Q45_SUB_BLOCK(4, row, tot)
+    RNB_Q45_SUB_BLOCK(5, row, tot)
+    RNB_Q45_SUB_BLOCK(6, row, tot)
+    RNB_Q45_SUB_BLOCK(7, row, tot)
+    const float d = f16_bits_to_f32(row.hdr.x), dmin = f16_bits_to_f32(row.hdr.x >> 16);
+    // K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
+    const long mnop = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(sc8.mn_lo) | (static_cast<unsigned long>(sc8.mn_hi) << 32)) : 0L;
+    const long op0 = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(dig.x) | (static_cast<unsigned long>(dig.y) << 32)) : 0L;
+    const long op1 = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(dig.z) | (static_cast<unsigned long>(dig.w) << 32)) : 0L;
+    const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op0, mnop, zero16, 0, 0, 0);
+    const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op1, mnop, zero16, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) val[i] = d * static_cast<float>(tot[i]) - dmin * static_cast<float>(c0[i] + 64 * c1[i]);
+}
+#undef RNB_Q45_SUB_BLOCK
+
+// ... and against one Q6_K row share: returns d * sum_sb sc * ((q - 32) . a)
+#define RNB_Q6_TILE_SUB_BLOCK(SB)                                                                        \
+    {                                                                                                    \
+        const long bop = q6_operand<SB>(row);                                                            \
+        const int sc = q6_scale<SB>(row);                                                                \
+        const long aop = *reinterpret_cast<const long *>(abase + 16 * (SB));                             \
+        const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);               \
+        _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                 \
+            tot[i] += mul24(acc[i], sc);                                                                 \
+            asm volatile("" : "+v"(tot[i]));                                                             \
+        }                                                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+    }
+__device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *abase, float (&val)[16]) {
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    int tot[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) tot[i] = 0;
+    RNB_Q6_TILE_SUB_BLOCK(0)
+    RNB_Q6_TILE_SUB_BLOCK(1)
+    RNB_Q6_TILE_SUB_BLOCK(2)
+    RNB_Q6_TILE_SUB_BLOCK(3)
+    RNB_Q6_TILE_SUB_BLOCK(4)
+    RNB_Q6_TILE_SUB_BLOCK(5)
+    RNB_Q6_TILE_SUB_BLOCK(6)
+    RNB_Q6_TILE_SUB_BLOCK(7)
+    RNB_Q6_TILE_SUB_BLOCK(8)
+    RNB_Q6_TILE_SUB_BLOCK(9)
+    RNB_Q6_TILE_SUB_BLOCK(10)
+    RNB_Q6_TILE_SUB_BLOCK(11)
+    RNB_Q6_TILE_SUB_BLOCK(12)
+    RNB_Q6_TILE_SUB_BLOCK(13)
+    RNB_Q6_TILE_SUB_BLOCK(14)
+    RNB_Q6_TILE_SUB_BLOCK(15)
+#pragma unroll
+    for (int i = 0; i < 16; i++) val[i] = row.d * static_cast<float>(tot[i]);
+}
+#undef RNB_Q6_TILE_SUB_BLOCK
+
+// accf[r] += d_x[token of result r] * val[r]; result r of a tile is token 8 * (r / 4) + 4 * khalf + r % 4
+__device__ __forceinline__ void tile_scale_add(const float *dxbuf, int khalf, const float (&val)[16], float (&accf)[16]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float4 dx4 = reinterpret_cast<const float4 *>(dxbuf)[2 * j + khalf];
+        const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) accf[4 * j + i] += dx[i] * val[4 * j + i];
+    }
+}
+
+// LDS image of one tile: every 256-element block of the tile's tokens, staged once and then only read
+//   act[nb][32 tokens][kStride] | d_x[nb][32] | digits[nb][32] (16 bytes each; absent for Q6_K weights)
+template <int kStride, bool kDigits>
+struct TileImage {
+    static __host__ __device__ size_t act_bytes(uint32_t nb) { return static_cast<size_t>(nb) * kMmToks * kStride; }
+    static __host__ __device__ size_t bytes(uint32_t nb) {
+        return act_bytes(nb) + static_cast<size_t>(nb) * kMmToks * (4 + (kDigits ? 16 : 0));
+    }
+    uint8_t *base;
+    uint32_t nb;
+    __device__ uint8_t *act(uint32_t b) const { return base + static_cast<size_t>(b) * kMmToks * kStride; }
+    __device__ float *dx(uint32_t b) const { return reinterpret_cast<float *>(base + act_bytes(nb)) + b * kMmToks; }
+    __device__ uint4 *dig(uint32_t b) const {
+        return reinterpret_cast<uint4 *>(base + act_bytes(nb) + static_cast<size_t>(nb) * kMmToks * 4) + b * kMmToks;
+    }
+};
+
+template <int kStride, bool kDigits>
+__device__ __forceinline__ void tile_image_fill(const TileImage<kStride, kDigits> &img, const TileMap &m,
+                                                const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                                const uint8_t *__restrict__ adig, int tid) {
+    const uint32_t nb = img.nb;
+    for (uint32_t b = 0; b < nb; b += 2) {  // two blocks' loads in flight before their stores
+        TileStage st0, st1;
+        const uint32_t b1 = b + 1 < nb ? b + 1 : b;
+        tile_stage_load<kDigits>(st0, m, aq, ad, adig, nb, b, tid);
+        tile_stage_load<kDigits>(st1, m, aq, ad, adig, nb, b1, tid);
+        tile_stage_store<kStride, kDigits>(st0, img.act(b), img.dx(b), img.dig(b), tid);
+        tile_stage_store<kStride, kDigits>(st1, img.act(b1), img.dx(b1), img.dig(b1), tid);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// gate + up + SiLU * up.  Grid (row tiles of 128, expert groups).  The tile's activations are staged once, all blocks;
+// after that the waves run without barriers, each streaming its 32 rows of both matrices one block ahead.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(kGbThreads, 2)
+    moe_gate_up_mfma_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
+                            const int8_t *__restrict__ aq, const float *__restrict__ ad, const uint8_t *__restrict__ adig,
+                            const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
+                            const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
+                            float *__restrict__ mid, uint32_t n_ff, uint32_t nb) {
+    constexpr bool kFifth = false;
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
+    __shared__ TileMap s_map;
+    const TileImage<kGbStride128, true> img{s_dyn, nb};
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t grp = blockIdx.y;
+    const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
+    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
+    const size_t woff = (static_cast<size_t>(expert) * n_ff + min(row, n_ff - 1)) * row_bytes;
+    const uint8_t *grow = gate_all + woff, *urow = up_all + woff;
+
+    for (uint32_t tile0 = 0; tile0 < count; tile0 += kMmToks) {
+        // the first weight blocks do not depend on the token lists: requested before them
+        Q5Row cg = q45_load_row<kFifth>(grow, khalf), cu = q45_load_row<kFifth>(urow, khalf);
+        if (tile0) __syncthreads();  // the previous tile's readers of the map and the image are done
+        tile_map_fill(s_map, sorted_token, sorted_slot, nullptr, start + tile0, count - tile0, tid);
+        __syncthreads();
+        tile_image_fill(img, s_map, aq, ad, adig, tid);
+        __syncthreads();
+        float accg[16], accu[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) accg[i] = accu[i] = 0.0f;
+        for (uint32_t b = 0; b < nb; b++) {
+            const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
+            const Q5Row ng = q45_load_row<kFifth>(grow + static_cast<size_t>(bn) * kQ4KBytes, khalf);
+            const Q5Row nu = q45_load_row<kFifth>(urow + static_cast<size_t>(bn) * kQ4KBytes, khalf);
+            const uint8_t *abase = img.act(b) + lrow * kGbStride128 + 16 * khalf;
+            const uint4 dig = img.dig(b)[lrow];
+            float val[16];
+            q45_block_tile<kFifth>(cg, abase, dig, khalf, val);
+            tile_scale_add(img.dx(b), khalf, val, accg);
+            q45_block_tile<kFifth>(cu, abase, dig, khalf, val);
+            tile_scale_add(img.dx(b), khalf, val, accu);
+            cg = ng;
+            cu = nu;
+        }
+        if (row < n_ff) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
+                if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// down projection of the re-quantised intermediate, scaled by the route weight.  Grid (row tiles of 128, expert groups).
+// ---------------------------------------------------------------------------------------------
+template <uint32_t kQuant>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
+                         const uint8_t *__restrict__ mdig, const uint32_t *__restrict__ grp_expert,
+                         const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
+                         const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb) {
+    constexpr bool kSix = kQuant == kQ6K;
+    constexpr bool kFifth = kQuant == kQ5K;
+    constexpr int kStride = kSix ? kGbStride64 : kGbStride128;
+    constexpr size_t kBlockBytes = kSix ? kQ6KBytes : (kFifth ? kQ5KBytes : kQ4KBytes);
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
+    __shared__ TileMap s_map;
+    const TileImage<kStride, !kSix> img{s_dyn, nb};
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t grp = blockIdx.y;
+    const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint8_t *wrow = down_all + (static_cast<size_t>(expert) * n_embd + min(row, n_embd - 1)) * row_bytes;
+
+    for (uint32_t tile0 = 0; tile0 < count; tile0 += kMmToks) {
+        Q6Row c6{};
+        Q5Row c5{};
+        if constexpr (kSix)
+            c6 = q6_load_row(wrow, khalf);
+        else
+            c5 = q45_load_row<kFifth>(wrow, khalf);
+        if (tile0) __syncthreads();
+        tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, count - tile0, tid);
+        __syncthreads();
+        tile_image_fill(img, s_map, mq, md, mdig, tid);
+        __syncthreads();
+        float accf[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) accf[i] = 0.0f;
+        for (uint32_t b = 0; b < nb; b++) {
+            const uint32_t bn = b + 1 < nb ? b + 1 : b;
+            Q6Row n6{};
+            Q5Row n5{};
+            float val[16];
+            if constexpr (kSix) {
+                n6 = q6_load_row(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+                q6_block_tile(c6, img.act(b) + lrow * kStride + 8 * khalf, val);
+            } else {
+                n5 = q45_load_row<kFifth>(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+                q45_block_tile<kFifth>(c5, img.act(b) + lrow * kStride + 16 * khalf, img.dig(b)[lrow], khalf, val);
+            }
+            tile_scale_add(img.dx(b), khalf, val, accf);
+            c6 = n6;
+            c5 = n5;
+        }
+        if (row < n_embd) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int t = 8 * (r >> 2) + 4 * khalf + (r & 3);
+                const uint32_t slot = s_map.out_row[t];
+                // fanout.rs:306-308: the expert's output times the slot's route weight
+                if (slot != 0xffffffffu) slot_out[static_cast<size_t>(slot) * n_embd + row] = accf[r] * s_map.scale[t];
+            }
+        }
+    }
+}
+
+template <typename K>
+void allow_lds(K kernel, size_t bytes) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(bytes));
+}
+
+}  // namespace
+
+// the tile image (all blocks of 32 tokens) must fit the LDS of a compute unit beside the small static arrays
+constexpr size_t kMmLdsLimit = 150 * 1024;
+
+bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
+    const size_t gu = TileImage<kGbStride128, true>::bytes(nb_in);
+    const size_t dn = down_quant == kQ6K ? TileImage<kGbStride64, false>::bytes(nb_mid) : TileImage<kGbStride128, true>::bytes(nb_mid);
+    return nb_in >= 1 && nb_mid >= 1 && gu <= kMmLdsLimit && dn <= kMmLdsLimit;
+}
+
+void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
+                             uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
+    if (groups.n_groups == 0 || n_ff == 0) return;
+    const size_t lds = TileImage<kGbStride128, true>::bytes(nb_in);
+    allow_lds(moe_gate_up_mfma_kernel, kMmLdsLimit);
+    const dim3 grid((n_ff + kGbRows - 1) / kGbRows, groups.n_groups, 1);
+    hipLaunchKernelGGL(moe_gate_up_mfma_kernel, grid, dim3(kGbThreads), lds, stream, gate_all, up_all, act.qs, act.d, act.digits,
+                       groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in);
+}
+
+void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+                          const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
+    if (groups.n_groups == 0 || n_embd == 0) return;
+    const dim3 grid((n_embd + kGbRows - 1) / kGbRows, groups.n_groups, 1), block(kGbThreads);
+#define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
+    allow_lds(moe_down_mfma_kernel<Q>, kMmLdsLimit);                                                                  \
+    hipLaunchKernelGGL((moe_down_mfma_kernel<Q>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
+                       groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid)
+    if (down_quant == kQ6K) {
+        RNB_LAUNCH_DM(kQ6K, (TileImage<kGbStride64, false>::bytes(nb_mid)));
+    } else if (down_quant == kQ5K) {
+        RNB_LAUNCH_DM(kQ5K, (TileImage<kGbStride128, true>::bytes(nb_mid)));
+    } else {
+        RNB_LAUNCH_DM(kQ4K, (TileImage<kGbStride128, true>::bytes(nb_mid)));
+    }
+#undef RNB_LAUNCH_DM
+}
+
+}  // namespace rnb

@@ -640,6 +640,26 @@ def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant
         rnb.release(w)
 
 
+@pytest.mark.parametrize("tokens,n_expert,k,n_ff,n_embd,down_quant", [(16, 8, 2, 256, 256, Q6_K), (64, 3, 2, 512, 768, Q4_K),
+                                                                     (100, 2, 2, 768, 512, Q5_K), (33, 20, 4, 300 * 0 + 512, 1280, Q6_K),
+                                                                     (40, 5, 3, 1024, 256, Q4_K), (20, 64, 3, 256, 512, Q6_K)])
+def test_moe_prefill_matrix_core_path(rnb, oracle, tokens, n_expert, k, n_ff, n_embd, down_quant):
+    """16 or more tokens and at least four slots per routed expert on average: the grouped expert GEMMs on the matrix
+    cores (32-token tiles per expert; experts with more than 32 tokens take several tiles, experts with few run mostly
+    padding); the last case stays below that average and keeps the integer-dot kernels.  Against the oracle, and a token's row must
+    not depend on the batch: the same bits with the tokens in reverse order."""
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 90 + tokens, down_quant)
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"moe prefill tokens {tokens} experts {n_expert} down {down_quant}")
+    xr = x.reshape(tokens, n_embd)[::-1].copy()
+    tr = (tokens - 1 - t).astype(np.uint32)
+    rev = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, tr, tokens, down_quant, n_ff, n_embd, xr)
+    assert np.array_equal(rev[::-1], got)
+    for w in (gate, up, down):
+        rnb.release(w)
+
+
 def test_moe_unrouted_token_and_empty_slot_list(rnb, oracle):
     n_expert, n_ff, n_embd = 4, 256, 256
     gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, 3, 2, 2)
@@ -668,11 +688,12 @@ def test_config5_moe_qwen3_30b_a3b(rnb, oracle, tokens):
     ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
     check_close(got, ref, None, f"cfg5 tokens {tokens}")
     if tokens > 1:
-        # a (token, expert) result does not depend on batching: token 7 alone == row 7 of the batch
+        # a (token, expert) result does not depend on batching: token 7 alone (the decode kernels: per-lane f32 partial
+        # sums) against row 7 of the batch (the matrix-core kernels: exact integer sums per block) agree to f32 rounding
         sel = t == 7
         solo = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e[sel], r[sel], np.zeros(sel.sum(), np.uint32),
                                                                 1, Q6_K, n_ff, n_embd, x[7 * n_embd:8 * n_embd])
-        assert np.array_equal(solo[0], got[7])
+        assert np.abs(solo[0] - got[7]).max() <= 2e-5 * float(np.sqrt(np.mean(got[7].astype(np.float64) ** 2)))
     for w in (gate, up, down):
         rnb.release(w)
 
