@@ -12,8 +12,8 @@
 //   Q8_0   v_mfma_i32_32x32x32_i8 per 32-element block: out += (d[r][b] * d_x[s][b]) * float(I_b),
 //   Q8_1   crates/rnb-cpu/src/gemm/neon_dot.rs:376-436, neon_quant.rs:236-253.
 // That is 16 (Q6_K) or 48 (Q8) vector instructions per matrix instruction, so these kernels are bound by the vector
-// port, not the matrix pipe; they replace one GEMV pass per token (Q8) or the integer-dot multi-token kernel (Q6_K),
-// which are 20 to 100 times slower at 512 tokens.
+// port, not the matrix pipe; they replace one GEMV pass per token (Q8) or the integer-dot multi-token kernel (Q5_K,
+// Q6_K), which measured 9 to 17 times slower at 512 tokens.
 //
 // Tiling: workgroup = 4 waves = 128 weight rows x kTT*32 tokens; a wave owns 32 rows and all the workgroup's tokens.
 // MFMA "M" = token, "N" = weight row: a lane's 16 results belong to ONE row (lane % 32), so that row's scales are

@@ -3,8 +3,8 @@
 // of 32 tokens: the tokens' quantised activations are gathered into LDS by the sorted lists, the expert's weight rows go
 // from global memory to the registers of the lane that owns the row, one int8 matrix instruction per scale group, the
 // group's scale on the vector units (see gemm_blocks.hip).  With a handful of tokens per expert most of a 32-token tile
-// is padding, which costs nothing extra: the vector work per tile is the same whatever the number of live tokens, and
-// it is a third of what the integer-dot kernels of moe.hip spend per token.
+// is padding, which costs nothing extra: the work per tile is the same whatever the number of live tokens, where the
+// integer-dot kernels of moe.hip cost per token (measured crossover on 128 experts x top-8: 64 tokens).
 //   gate/up   mid[slot][n_ff] = silu(Wg[e] . a_tok) * (Wu[e] . a_tok), both Q4_K: the two matrices share the activation
 //             operand of every instruction                        fanout.rs:260-327, activation.rs:73-89
 //   down      slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])), Q4_K, Q5_K or Q6_K
