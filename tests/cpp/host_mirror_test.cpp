@@ -142,6 +142,10 @@ int main(int argc, char **argv) {
         run_case(dir, "q3k_batch", 11, 512, 6, q3k_gemv_batch);
         run_case(dir, "q4_0_gemv", 21, 608, 1, q4_0_gemv);
         run_case(dir, "q5_1_batch", 10, 160, 3, q5_1_gemv_batch);
+        run_case(dir, "q8_1_gemv", 19, 160, 1, q8_1_gemv);
+        run_case(dir, "q6k_gemm", 33, 512, 20, q6k_gemv_batch);
+        run_case(dir, "q5k_gemm", 40, 256, 17, q5k_gemv_batch);
+        run_case(dir, "q8_0_gemm", 35, 96, 18, q8_0_gemv_batch);
         std::printf("run: %d failure(s)\n", failures);
         return failures ? 1 : 0;
     }

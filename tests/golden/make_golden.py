@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 from oracle import oracle as ora  # noqa: E402
 
-Q4_0, Q5_1 = 2, 7
+Q4_0, Q5_1, Q8_1 = 2, 7, 9
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
 
 
@@ -41,7 +41,10 @@ def main():
                                          ("q6k_batch", Q6_K, 9, 512, 3), ("q8_0_batch", Q8_0, 7, 96, 4),
                                          ("q5k_gemv", Q5_K, 22, 1280, 1), ("q5k_batch", Q5_K, 13, 512, 5),
                                          ("q2k_gemv", Q2_K, 18, 768, 1), ("q3k_batch", Q3_K, 11, 512, 6),
-                                         ("q4_0_gemv", Q4_0, 21, 608, 1), ("q5_1_batch", Q5_1, 10, 160, 3)):
+                                         ("q4_0_gemv", Q4_0, 21, 608, 1), ("q5_1_batch", Q5_1, 10, 160, 3),
+                                         # 16+ tokens: the matrix-core GEMMs of the formats other than Q4_K
+                                         ("q8_1_gemv", Q8_1, 19, 160, 1), ("q6k_gemm", Q6_K, 33, 512, 20),
+                                         ("q5k_gemm", Q5_K, 40, 256, 17), ("q8_0_gemm", Q8_0, 35, 96, 18)):
         w = ora.make_weights(quant, rows, cols, ora.tensor_seed(name, "w"))
         xin = ora.fill_normal(seq * cols, ora.tensor_seed(name, "x"), 1.0)
         ref = ora.gemv(quant, w, rows, cols, xin)
