@@ -297,6 +297,23 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         if (st != RNB_HIP_OK) return st;
         st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>());
         if (st != RNB_HIP_OK) return st;
+        if (!is_block32(down_quant)) {
+            // K-quant down projection: act(gate) * up is quantised to Q8_K as it is made, no f32 intermediate in memory
+            const size_t n = seq * n_ff;
+            HIP_TRY(s.act_qs.reserve(n));
+            HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
+            HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
+            s.act_has_digits = seq >= kGemmMinSeq;
+            if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
+            launch_quantize_q8k_gated(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), n / 256, gelu, s.act_qs.as<int8_t>(),
+                                      s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
+                                      s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr, s.stream);
+            HIP_TRY(hipGetLastError());
+            s.act_family = kQ4K;
+            s.act_seq = seq;
+            s.act_cols = n_ff;
+            return run_matmul_quantized_dev(s, down_quant, down_dev, n_embd, n_ff, seq, out_dev);
+        }
         launch_act_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, gelu, s.stream);
     }
     HIP_TRY(hipGetLastError());

@@ -109,6 +109,9 @@ struct MoeGroups {
     const uint32_t *sorted_token;  // [n_slots]
     uint32_t n_groups;
 };
+// Q8_K of act(gate[i]) * up[i] (SiLU, or the tanh form of GELU): the gated FFN's intermediate quantised as it is made
+void launch_quantize_q8k_gated(const float *gate, const float *up, size_t n_blocks, bool gelu, int8_t *qs, float *d,
+                               int16_t *bsums, uint8_t *digits, hipStream_t stream);
 // Decode-sized routing tables travel as a kernel argument instead of a host-to-device copy: the
 // activation quantiser's launch also writes them to their device buffer.
 constexpr uint32_t kMoeInlineWords = 240;  // 960 bytes of kernel argument

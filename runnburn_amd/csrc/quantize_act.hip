@@ -21,6 +21,23 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                       digits != nullptr ? digits + blk * 16 : nullptr);
 }
 
+// The gated-FFN intermediate quantised as it is made: x = act(gate) * up element by element (SiLU or the tanh form of
+// GELU, device_utils.h::act_mul), then quantize_q8k_kernel's routine; the f32 intermediate never travels through memory.
+template <bool kGelu>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    quantize_q8k_gated_kernel(const float *__restrict__ gate, const float *__restrict__ up, size_t n_blocks,
+                              int8_t *__restrict__ qs, float *__restrict__ d_out, int16_t *__restrict__ bsums,
+                              uint8_t *__restrict__ digits) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t blk = static_cast<size_t>(blockIdx.x) * kWavesPerWg + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;  // wave-uniform
+    const float4 g = reinterpret_cast<const float4 *>(gate + blk * 256)[lane];
+    const float4 u = reinterpret_cast<const float4 *>(up + blk * 256)[lane];
+    const float4 v = make_float4(act_mul<kGelu>(g.x, u.x), act_mul<kGelu>(g.y, u.y), act_mul<kGelu>(g.z, u.z),
+                                 act_mul<kGelu>(g.w, u.w));
+    q8k_quantize_vals(v, lane, qs + blk * 256, d_out + blk, bsums + blk * 16, digits != nullptr ? digits + blk * 16 : nullptr);
+}
+
 // Same as quantize_q8k_kernel; workgroup 0 additionally copies `n_words` routing-table words from the
 // kernel argument to device memory (n_words <= 256 = one word per thread).
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
@@ -94,6 +111,16 @@ void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, 
     const unsigned grid = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
     hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(kWave * kWavesPerWg), 0, stream, x, n_blocks, qs,
                        d, bsums, digits);
+}
+
+void launch_quantize_q8k_gated(const float *gate, const float *up, size_t n_blocks, bool gelu, int8_t *qs, float *d,
+                               int16_t *bsums, uint8_t *digits, hipStream_t stream) {
+    if (n_blocks == 0) return;
+    const dim3 grid(static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg)), block(kWave * kWavesPerWg);
+    if (gelu)
+        hipLaunchKernelGGL(quantize_q8k_gated_kernel<true>, grid, block, 0, stream, gate, up, n_blocks, qs, d, bsums, digits);
+    else
+        hipLaunchKernelGGL(quantize_q8k_gated_kernel<false>, grid, block, 0, stream, gate, up, n_blocks, qs, d, bsums, digits);
 }
 
 void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
