@@ -60,6 +60,8 @@ int hip_fail(const char *what, hipError_t e) {
 // Quantise seq*cols staged floats on the device into the state's activation scratch.
 // Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
 constexpr size_t kGemmMinSeq = 16;
+// Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
+constexpr uint64_t kGemmBigTilesMin = 128;
 // Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
 constexpr size_t kTokensMinSeq = 4;
 
@@ -120,7 +122,13 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     const uint32_t nb = static_cast<uint32_t>(cols / 256);
     if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
-        if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
+        // gemm_q4k.hip's 256-row x 64-token workgroups need about half the compute units' worth of tiles to pay off; below
+        // that the 128 x 32 / 64 kernel of gemm_blocks.hip wins (4096 x 4096 x 64 tokens: 26 vs 34 us; 14336 x 4096 x 64:
+        // 28 vs 40 us; at 14336 x 4096 x 512 the big tiles win, 93 vs 116 us)
+        const uint64_t big_tiles = static_cast<uint64_t>((rows + 255) / 256) * ((seq + 63) / 64);
+        if (seq >= kGemmMinSeq && act.digits != nullptr && big_tiles < kGemmBigTilesMin)
+            launch_gemm_q4k_small(w_dev, act, out_dev, r, nb, q, s.stream);
+        else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_gemm_q4k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
         else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);

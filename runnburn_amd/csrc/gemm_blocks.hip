@@ -140,9 +140,9 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 // quantiser's digits (bsum32 = b0 + 64 * b1): two K=16 instructions with eight live K slots per token tile.
 // Per super-block out += d_x * (d * float(tot) - dmin * float(S)): crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800.
 // ---------------------------------------------------------------------------------------------
-template <int kTT>
+template <int kTT, bool kFifth>
 __global__ void __launch_bounds__(kGbThreads, 2)
-    gemm_q5k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+    gemm_q45k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                          const uint8_t *__restrict__ adig, float *__restrict__ out, uint32_t rows, uint32_t nb,
                          uint32_t seq) {
     constexpr int kToks = 32 * kTT;
@@ -154,7 +154,8 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const int lrow = lane & 31, khalf = lane >> 5;
     const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
     const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
-    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kQ5KBytes;
+    constexpr size_t kBlockBytes = kFifth ? kQ5KBytes : kQ4KBytes;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kBlockBytes;
 
     float accf[kTT][16];
     int tot[kTT][16];
@@ -186,7 +187,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }
     };
     stage_load5(0);
-    Q5Row cur = q5_load_row(wrow, khalf);
+    Q5Row cur = q45_load_row<kFifth>(wrow, khalf);
     stage_store5(0);
     __syncthreads();
 
@@ -194,15 +195,13 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const int buf = b & 1;
         const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
         stage_load5(bn);
-        const Q5Row nxt = q5_load_row(wrow + static_cast<size_t>(bn) * kQ5KBytes, khalf);
+        const Q5Row nxt = q45_load_row<kFifth>(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
         const Q4KScales sc8 = unpack_q4k_scales(cur.hdr.y, cur.hdr.z, cur.hdr.w);
 
 #define RNB_Q5_SUB_BLOCK(SB)                                                                                           \
     {                                                                                                                  \
-        const uint4 qs = cur.qs[(SB) >> 1];                                                                            \
-        const v4i bop = {static_cast<int>(q5_codes<SB>(qs.x, cur.qh.x)), static_cast<int>(q5_codes<SB>(qs.y, cur.qh.y)), \
-                         static_cast<int>(q5_codes<SB>(qs.z, cur.qh.z)), static_cast<int>(q5_codes<SB>(qs.w, cur.qh.w))}; \
+        const v4i bop = q45_operand<SB, kFifth>(cur);                                                                  \
         const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                              \
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * (SB));                 \
@@ -413,19 +412,30 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t ro
     }
 }
 
-void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                          hipStream_t stream) {
+template <bool kFifth>
+static void launch_gemm_q45k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                             hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
     if (wide_tiles(row_tiles, seq)) {
         const dim3 grid(row_tiles, (seq + 63) / 64, 1);
-        hipLaunchKernelGGL(gemm_q5k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits, out, rows,
-                           nb, seq);
+        hipLaunchKernelGGL((gemm_q45k_mfma_kernel<2, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
+                           out, rows, nb, seq);
     } else {
         const dim3 grid(row_tiles, (seq + 31) / 32, 1);
-        hipLaunchKernelGGL(gemm_q5k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits, out, rows,
-                           nb, seq);
+        hipLaunchKernelGGL((gemm_q45k_mfma_kernel<1, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
+                           out, rows, nb, seq);
     }
+}
+
+void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream) {
+    launch_gemm_q45k<true>(w, act, out, rows, nb, seq, stream);
+}
+
+void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                           hipStream_t stream) {
+    launch_gemm_q45k<false>(w, act, out, rows, nb, seq, stream);
 }
 
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32) { return (quant == kQ8_0 || quant == kQ8_1) && nb32 >= 1; }

@@ -92,6 +92,10 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t ro
 // Q5_K needs act.digits (the quantiser writes them for 16+ tokens)
 void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                           hipStream_t stream);
+// Q4_K through the same kernel (scales on the vector units): for shapes that give gemm_q4k.hip's 256 x 64 tiles too few
+// workgroups to fill the chip
+void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                           hipStream_t stream);
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32);
 void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
                          uint32_t seq, hipStream_t stream);

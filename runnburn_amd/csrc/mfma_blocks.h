@@ -128,20 +128,36 @@ struct Q5Row {
     uint4 qs[4];
 };
 
-__device__ __forceinline__ Q5Row q5_load_row(const uint8_t *__restrict__ blk, int khalf) {
-    Q5Row r;
-    r.hdr = ld_u4_a2(blk);
-    r.qh = ld_u4_a2(blk + 16 + 16 * khalf);
-#pragma unroll
-    for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + 48 + 32 * g + 16 * khalf);
-    return r;
-}
-
 template <int kSb>
 __device__ __forceinline__ uint32_t q5_codes(uint32_t qs, uint32_t qh) {
     const uint32_t nib = (kSb & 1) ? (qs >> 4) & 0x0f0f0f0fu : qs & 0x0f0f0f0fu;
     const uint32_t fifth = kSb <= 4 ? (qh << (4 - kSb)) & 0x10101010u : (qh >> (kSb - 4)) & 0x10101010u;
     return nib | fifth;
+}
+
+// Q4_K / Q5_K row share of a block: header, (fifth bits,) the K-half's 16 bytes of every 32-byte nibble group
+template <bool kFifth>
+__device__ __forceinline__ Q5Row q45_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q5Row r;
+    r.hdr = ld_u4_a2(blk);
+    r.qh = make_uint4(0, 0, 0, 0);
+    if constexpr (kFifth) r.qh = ld_u4_a2(blk + 16 + 16 * khalf);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + (kFifth ? 48 : 16) + 32 * g + 16 * khalf);
+    return r;
+}
+
+template <int kSb, bool kFifth>
+__device__ __forceinline__ v4i q45_operand(const Q5Row &r) {
+    const uint4 qs = r.qs[kSb >> 1];
+    if constexpr (kFifth) {
+        return v4i{static_cast<int>(q5_codes<kSb>(qs.x, r.qh.x)), static_cast<int>(q5_codes<kSb>(qs.y, r.qh.y)),
+                   static_cast<int>(q5_codes<kSb>(qs.z, r.qh.z)), static_cast<int>(q5_codes<kSb>(qs.w, r.qh.w))};
+    } else {
+        constexpr int sh = (kSb & 1) * 4;
+        return v4i{static_cast<int>((qs.x >> sh) & 0x0f0f0f0fu), static_cast<int>((qs.y >> sh) & 0x0f0f0f0fu),
+                   static_cast<int>((qs.z >> sh) & 0x0f0f0f0fu), static_cast<int>((qs.w >> sh) & 0x0f0f0f0fu)};
+    }
 }
 
 }  // namespace
