@@ -123,8 +123,8 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
         // gemm_q4k.hip's 256-row x 64-token workgroups need about half the compute units' worth of tiles to pay off; below
-        // that the 128 x 32 / 64 kernel of gemm_blocks.hip wins (4096 x 4096 x 64 tokens: 26 vs 34 us; 14336 x 4096 x 64:
-        // 28 vs 40 us; at 14336 x 4096 x 512 the big tiles win, 93 vs 116 us)
+        // that the 128 x 32 / 64 kernel of gemm_blocks.hip wins (4096 x 4096 x 64 tokens: 20 vs 34 us; 14336 x 4096 x 64:
+        // 25 vs 40 us; at 14336 x 4096 x 512 the big tiles win, 93 vs 132 us)
         const uint64_t big_tiles = static_cast<uint64_t>((rows + 255) / 256) * ((seq + 63) / 64);
         if (seq >= kGemmMinSeq && act.digits != nullptr && big_tiles < kGemmBigTilesMin)
             launch_gemm_q4k_small(w_dev, act, out_dev, r, nb, q, s.stream);

@@ -199,6 +199,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
         const Q4KScales sc8 = unpack_q4k_scales(cur.hdr.y, cur.hdr.z, cur.hdr.w);
 
+        if constexpr (kFifth) {
 #define RNB_Q5_SUB_BLOCK(SB)                                                                                           \
     {                                                                                                                  \
         const v4i bop = q45_operand<SB, kFifth>(cur);                                                                  \
@@ -213,15 +214,50 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }                                                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                                                             \
     }
-        RNB_Q5_SUB_BLOCK(0)
-        RNB_Q5_SUB_BLOCK(1)
-        RNB_Q5_SUB_BLOCK(2)
-        RNB_Q5_SUB_BLOCK(3)
-        RNB_Q5_SUB_BLOCK(4)
-        RNB_Q5_SUB_BLOCK(5)
-        RNB_Q5_SUB_BLOCK(6)
-        RNB_Q5_SUB_BLOCK(7)
+            RNB_Q5_SUB_BLOCK(0)
+            RNB_Q5_SUB_BLOCK(1)
+            RNB_Q5_SUB_BLOCK(2)
+            RNB_Q5_SUB_BLOCK(3)
+            RNB_Q5_SUB_BLOCK(4)
+            RNB_Q5_SUB_BLOCK(5)
+            RNB_Q5_SUB_BLOCK(6)
+            RNB_Q5_SUB_BLOCK(7)
 #undef RNB_Q5_SUB_BLOCK
+        } else {
+            // Q4_K: the 6-bit scale is folded into the weight operand as in gemm_q4k.hip (sc = lo + 8 * hi, lo * nib and
+            // hi * nib <= 105 are int8 values made with one packed 16-bit multiply per four weights), two accumulator
+            // chains over the whole super-block and I = I_lo + 8 * I_hi: no multiply-add per result and sub-block
+            const uint32_t dlo[2] = {sc8.sc_lo & 0x07070707u, sc8.sc_hi & 0x07070707u};
+            const uint32_t dhi[2] = {(sc8.sc_lo >> 3) & 0x07070707u, (sc8.sc_hi >> 3) & 0x07070707u};
+            v16i acc_lo[kTT], acc_hi[kTT];
+#define RNB_Q4_SUB_BLOCK(SB)                                                                                           \
+    {                                                                                                                  \
+        const v4i nib = q45_operand<SB, false>(cur);                                                                   \
+        constexpr uint32_t sel = 0x0c000c00u | (((SB) & 3) << 16) | ((SB) & 3);                                        \
+        const uint32_t slo = __builtin_amdgcn_perm(0u, dlo[(SB) >> 2], sel);                                           \
+        const uint32_t shi = __builtin_amdgcn_perm(0u, dhi[(SB) >> 2], sel);                                           \
+        const v4i wlo = {pk_scale(nib[0], slo), pk_scale(nib[1], slo), pk_scale(nib[2], slo), pk_scale(nib[3], slo)};  \
+        const v4i whi = {pk_scale(nib[0], shi), pk_scale(nib[1], shi), pk_scale(nib[2], shi), pk_scale(nib[3], shi)};  \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * (SB));                 \
+            acc_lo[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, wlo, (SB) == 0 ? zero16 : acc_lo[t], 0, 0, 0);      \
+            acc_hi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, whi, (SB) == 0 ? zero16 : acc_hi[t], 0, 0, 0);      \
+        }                                                                                                              \
+    }
+            RNB_Q4_SUB_BLOCK(0)
+            RNB_Q4_SUB_BLOCK(1)
+            RNB_Q4_SUB_BLOCK(2)
+            RNB_Q4_SUB_BLOCK(3)
+            RNB_Q4_SUB_BLOCK(4)
+            RNB_Q4_SUB_BLOCK(5)
+            RNB_Q4_SUB_BLOCK(6)
+            RNB_Q4_SUB_BLOCK(7)
+#undef RNB_Q4_SUB_BLOCK
+#pragma unroll
+            for (int t = 0; t < kTT; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) tot[t][i] = acc_lo[t][i] + 8 * acc_hi[t][i];
+        }
 
         // mins: K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
         const float d = f16_bits_to_f32(cur.hdr.x), dmin = f16_bits_to_f32(cur.hdr.x >> 16);

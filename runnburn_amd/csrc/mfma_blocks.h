@@ -135,6 +135,13 @@ __device__ __forceinline__ uint32_t q5_codes(uint32_t qs, uint32_t qh) {
     return nib | fifth;
 }
 
+// four bytes (each <= 15) times a scalar <= 7 held in both 16-bit halves of `s2`: no carry between bytes
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int pk_scale(uint32_t nib4, uint32_t s2) {
+    const u16x2_t a = __builtin_bit_cast(u16x2_t, nib4), b = __builtin_bit_cast(u16x2_t, s2);
+    return __builtin_bit_cast(int, static_cast<u16x2_t>(a * b));
+}
+
 // Q4_K / Q5_K row share of a block: header, (fifth bits,) the K-half's 16 bytes of every 32-byte nibble group
 template <bool kFifth>
 __device__ __forceinline__ Q5Row q45_load_row(const uint8_t *__restrict__ blk, int khalf) {
