@@ -97,16 +97,46 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const Q4KScales sc8 = unpack_q4k_scales(row.hdr.y, row.hdr.z, row.hdr.w);
     int tot[16];
+    if constexpr (kFifth) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) tot[i] = 0;
-    RNB_Q45_SUB_BLOCK(0, row, tot)
-    RNB_Q45_SUB_BLOCK(1, row, tot)
-    RNB_Q45_SUB_BLOCK(2, row, tot)
-    RNB_Q45_SUB_BLOCK(3, row, tot)
-    RNB_Q45_SUB_BLOCK(4, row, tot)
-    RNB_Q45_SUB_BLOCK(5, row, tot)
-    RNB_Q45_SUB_BLOCK(6, row, tot)
-    RNB_Q45_SUB_BLOCK(7, row, tot)
+        for (int i = 0; i < 16; i++) tot[i] = 0;
+        RNB_Q45_SUB_BLOCK(0, row, tot)
+        RNB_Q45_SUB_BLOCK(1, row, tot)
+        RNB_Q45_SUB_BLOCK(2, row, tot)
+        RNB_Q45_SUB_BLOCK(3, row, tot)
+        RNB_Q45_SUB_BLOCK(4, row, tot)
+        RNB_Q45_SUB_BLOCK(5, row, tot)
+        RNB_Q45_SUB_BLOCK(6, row, tot)
+        RNB_Q45_SUB_BLOCK(7, row, tot)
+    } else {
+        // Q4_K: the scale folded into the operand (sc = lo + 8 * hi, two accumulator chains), as in gemm_blocks.hip
+        const uint32_t dlo[2] = {sc8.sc_lo & 0x07070707u, sc8.sc_hi & 0x07070707u};
+        const uint32_t dhi[2] = {(sc8.sc_lo >> 3) & 0x07070707u, (sc8.sc_hi >> 3) & 0x07070707u};
+        v16i acc_lo = zero16, acc_hi = zero16;
+#define RNB_Q4_FOLD_SUB_BLOCK(SB)                                                                        \
+    {                                                                                                    \
+        const v4i nib = q45_operand<SB, false>(row);                                                     \
+        constexpr uint32_t sel = 0x0c000c00u | (((SB) & 3) << 16) | ((SB) & 3);                          \
+        const uint32_t slo = __builtin_amdgcn_perm(0u, dlo[(SB) >> 2], sel);                             \
+        const uint32_t shi = __builtin_amdgcn_perm(0u, dhi[(SB) >> 2], sel);                             \
+        const v4i wlo = {pk_scale(nib[0], slo), pk_scale(nib[1], slo), pk_scale(nib[2], slo), pk_scale(nib[3], slo)}; \
+        const v4i whi = {pk_scale(nib[0], shi), pk_scale(nib[1], shi), pk_scale(nib[2], shi), pk_scale(nib[3], shi)}; \
+        const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * (SB));                               \
+        acc_lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, wlo, acc_lo, 0, 0, 0);                       \
+        acc_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, whi, acc_hi, 0, 0, 0);                       \
+    }
+        RNB_Q4_FOLD_SUB_BLOCK(0)
+        RNB_Q4_FOLD_SUB_BLOCK(1)
+        RNB_Q4_FOLD_SUB_BLOCK(2)
+        RNB_Q4_FOLD_SUB_BLOCK(3)
+        RNB_Q4_FOLD_SUB_BLOCK(4)
+        RNB_Q4_FOLD_SUB_BLOCK(5)
+        RNB_Q4_FOLD_SUB_BLOCK(6)
+        RNB_Q4_FOLD_SUB_BLOCK(7)
+#undef RNB_Q4_FOLD_SUB_BLOCK
+#pragma unroll
+        for (int i = 0; i < 16; i++) tot[i] = acc_lo[i] + 8 * acc_hi[i];
+    }
     const float d = f16_bits_to_f32(row.hdr.x), dmin = f16_bits_to_f32(row.hdr.x >> 16);
     // K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
     const long mnop = khalf == 0 ? static_cast<long>(static_cast<unsigned long>(sc8.mn_lo) | (static_cast<unsigned long>(sc8.mn_hi) << 32)) : 0L;
