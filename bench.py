@@ -458,9 +458,16 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
             b.free()
     x_dev.free()
     out_dev.free()
-    return {"workload": f"dense SwiGLU FFN 4096 -> 14336 -> 4096 (Q4_K gate/up, Q6_K down), tokens={tokens}", "ms": ms,
-            "bytes": nbytes, "GB/s": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "copies": n_copies,
-            "note": "events around the whole call (quantise + fused gate/up/SiLU + re-quantise + down)"}
+    res = {"workload": f"dense SwiGLU FFN 4096 -> 14336 -> 4096 (Q4_K gate/up, Q6_K down), tokens={tokens}", "ms": ms,
+           "copies": n_copies}
+    if tokens < 16:  # decode: weight streaming
+        res.update({"bytes": nbytes, "GB/s": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS,
+                    "note": "events around the whole call (token quantisation + gate/up/SiLU in one launch, re-quantise, down)"})
+    else:  # prefill: matrix-core GEMMs
+        ops = 2 * tokens * 3 * n_ff * n_embd
+        res.update({"ops": ops, "TOP/s": ops / ms / 1e9, "mfma_frac": ops / ms / 1e9 / INT8_PEAK_TOPS,
+                    "note": "events around the whole call (quantise, two Q4_K GEMMs, SiLU*up quantised as it is made, Q6_K GEMM)"})
+    return res
 
 
 def main() -> int:
@@ -583,10 +590,11 @@ def main() -> int:
                 sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens)
             except Exception as exc:
                 sec[f"cfg5_moe_tokens{tokens}"] = {"error": str(exc)}
-        try:
-            sec["ffn_llama3_8b_tokens1"] = bench_ffn(rnb, hip, stream, 1, s2, 4321)
-        except Exception as exc:
-            sec["ffn_llama3_8b_tokens1"] = {"error": str(exc)}
+        for tokens, n in ((1, s2), (512, 20)):
+            try:
+                sec[f"ffn_llama3_8b_tokens{tokens}"] = bench_ffn(rnb, hip, stream, tokens, n, 4321)
+            except Exception as exc:
+                sec[f"ffn_llama3_8b_tokens{tokens}"] = {"error": str(exc)}
         result["secondary"] = sec
 
     print(json.dumps(result), flush=True)
