@@ -36,6 +36,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                          float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq) {
     constexpr int kToks = 32 * kTT;
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride64];
+    __shared__ __attribute__((aligned(16))) uint8_t s_w[kGbWaves][32 * kQ6StripStride];
     __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid >> 6;
@@ -55,9 +56,20 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
+    // the wave's 32 rows come in by whole cache lines and reach their lanes through the wave's strip of LDS
+    const uint32_t wrow0 = min(blockIdx.x * kGbRows + wave * 32, rows - 1);
+    const uint8_t *wbase = w + static_cast<size_t>(wrow0) * nb * kQ6KBytes;
+    uint8_t *strip = s_w[wave];
+    RowRoute<kQ6Pieces> rt;
+    route_setup<kQ6Pieces, kQ6StripStride>(rt, rows - wrow0, static_cast<size_t>(nb) * kQ6KBytes, lane);
+
     Stage<kToks> st;
     stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, 0, tid);
-    Q6Row cur = q6_load_row(wrow, khalf);
+    route_load(rt, wbase);
+    Q6Row cur;
+    cur.d = ld_f16(wrow + 208);
+    route_store(rt, strip, lane);
+    q6_row_from_strip(cur, strip + lrow * kQ6StripStride, khalf);
     stage_store<kToks>(st, s_a[0], s_dx[0], tid);
     __syncthreads();
 
@@ -65,7 +77,9 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const int buf = b & 1;
         const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
         stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, bn, tid);
-        const Q6Row nxt = q6_load_row(wrow + static_cast<size_t>(bn) * kQ6KBytes, khalf);
+        route_load(rt, wbase + static_cast<size_t>(bn) * kQ6KBytes);
+        const float d_next = ld_f16(wrow + static_cast<size_t>(bn) * kQ6KBytes + 208);
+        const float d_cur = cur.d;
         const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
 
         // one 16-element sub-block: operand from the packed row, one matrix instruction per token tile, the sub-block's
@@ -113,12 +127,14 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int r = 4 * j + i;
-                    accf[t][r] += (cur.d * dx[i]) * static_cast<float>(tot[t][r]);
+                    accf[t][r] += (d_cur * dx[i]) * static_cast<float>(tot[t][r]);
                     tot[t][r] = 0;
                 }
             }
         stage_store<kToks>(st, s_a[buf ^ 1], s_dx[buf ^ 1], tid);
-        cur = nxt;
+        route_store(rt, strip, lane);
+        q6_row_from_strip(cur, strip + lrow * kQ6StripStride, khalf);
+        cur.d = d_next;
         __syncthreads();
     }
 
@@ -322,14 +338,72 @@ __device__ __forceinline__ Q8Blocks q8_load_blocks(const uint8_t *__restrict__ r
     return r;
 }
 
-template <int kTT, int kBlockBytes, int kQsOff>
+// Route of a wave's 32 rows of one step (8 blocks) to the lanes that own them, by whole cache lines (see RowRoute):
+// lane takes the 16-byte half j % 2 of block j / 2 (j = lane % 16) of rows lane / 16 + 4 i, and the scale of block
+// lane % 8 of rows lane / 8 + 8 i.  In the strip a row is its 256 codes (rows kGbStride128 bytes apart), followed by
+// the 32 rows' scales (8 f16 each).  Only for rows whose block count is a multiple of 8, where every step is whole.
+constexpr int kQ8StripBytes = 32 * kGbStride128 + 32 * 16;
+
+struct Q8Route {
+    uint32_t qoff[8], doff[4];  // byte offsets from the wave's first row (rows past the end: the last row)
+    uint4 q[8];
+    uint16_t d[4];
+};
+
+template <int kBlockBytes, int kQsOff>
+__device__ __forceinline__ void q8_route_setup(Q8Route &rt, uint32_t rows_left, size_t row_bytes, int lane) {
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        rt.qoff[i] = static_cast<uint32_t>(min(static_cast<uint32_t>(lane >> 4) + 4 * i, rows_left - 1) * row_bytes) +
+                     ((lane & 15) >> 1) * kBlockBytes + kQsOff + 16 * (lane & 1);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        rt.doff[i] = static_cast<uint32_t>(min(static_cast<uint32_t>(lane >> 3) + 8 * i, rows_left - 1) * row_bytes) +
+                     (lane & 7) * kBlockBytes;
+}
+
+__device__ __forceinline__ void q8_route_load(Q8Route &rt, const uint8_t *__restrict__ base) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) rt.q[i] = ld_u4_a2(base + rt.qoff[i]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) rt.d[i] = *reinterpret_cast<const uint16_t *>(base + rt.doff[i]);
+}
+
+__device__ __forceinline__ void q8_route_store(const Q8Route &rt, uint8_t *strip, int lane) {
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        *reinterpret_cast<uint4 *>(strip + ((lane >> 4) + 4 * i) * kGbStride128 + 16 * (lane & 15)) = rt.q[i];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        *reinterpret_cast<uint16_t *>(strip + 32 * kGbStride128 + ((lane >> 3) + 8 * i) * 16 + 2 * (lane & 7)) = rt.d[i];
+}
+
+__device__ __forceinline__ Q8Blocks q8_blocks_from_strip(const uint8_t *strip, int lrow, int khalf) {
+    Q8Blocks r;
+#pragma unroll
+    for (int k = 0; k < 8; k++)
+        r.q[k] = *reinterpret_cast<const uint4 *>(strip + lrow * kGbStride128 + 32 * k + 16 * khalf);
+    const uint4 d8 = *reinterpret_cast<const uint4 *>(strip + 32 * kGbStride128 + lrow * 16);
+    const uint32_t dw[4] = {d8.x, d8.y, d8.z, d8.w};
+#pragma unroll
+    for (int k = 0; k < 8; k++) r.d[k] = f16_bits_to_f32(dw[k >> 1] >> (16 * (k & 1)));
+    return r;
+}
+
+template <int kTT>
+constexpr size_t q8_lds_bytes(bool routed) {
+    return 2 * (32 * kTT) * kGbStride128 + 2 * 8 * (32 * kTT) * sizeof(float) + (routed ? kGbWaves * kQ8StripBytes : 0);
+}
+
+template <int kTT, int kBlockBytes, int kQsOff, bool kRouted>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q8_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                         float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq) {
     constexpr int kToks = 32 * kTT;
     constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
-    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride128];
-    __shared__ __attribute__((aligned(16))) float s_dx[2][8][kToks];  // [block of the step][token]
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
+    uint8_t(*s_a)[kToks * kGbStride128] = reinterpret_cast<uint8_t(*)[kToks * kGbStride128]>(s_dyn);
+    float(*s_dx)[8][kToks] = reinterpret_cast<float(*)[8][kToks]>(s_dyn + 2 * kToks * kGbStride128);  // [block][token]
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid >> 6;
     const int lrow = lane & 31, khalf = lane >> 5;
@@ -378,8 +452,20 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }
     };
 
+    const uint32_t wrow0 = min(blockIdx.x * kGbRows + wave * 32, rows - 1);
+    const uint8_t *wbase = w + static_cast<size_t>(wrow0) * nb32 * kBlockBytes;
+    uint8_t *strip = s_dyn + q8_lds_bytes<kTT>(false) + wave * kQ8StripBytes;
+    Q8Route rt;
+    Q8Blocks cur, nxt;
     stage_load8(0);
-    Q8Blocks cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, 0, nb32, khalf);
+    if constexpr (kRouted) {
+        q8_route_setup<kBlockBytes, kQsOff>(rt, rows - wrow0, static_cast<size_t>(nb32) * kBlockBytes, lane);
+        q8_route_load(rt, wbase);
+        q8_route_store(rt, strip, lane);
+        cur = q8_blocks_from_strip(strip, lrow, khalf);
+    } else {
+        cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, 0, nb32, khalf);
+    }
     stage_store8(0);
     __syncthreads();
 
@@ -387,7 +473,10 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const int buf = step & 1;
         const uint32_t sn = step + 1 < steps ? step + 1 : step;
         stage_load8(sn);
-        const Q8Blocks nxt = q8_load_blocks<kBlockBytes, kQsOff>(wrow, sn * 8, nb32, khalf);
+        if constexpr (kRouted)
+            q8_route_load(rt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
+        else
+            nxt = q8_load_blocks<kBlockBytes, kQsOff>(wrow, sn * 8, nb32, khalf);
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
         const uint32_t live = min(8u, nb32 - step * 8);  // blocks of this step that exist (workgroup-uniform)
 #pragma unroll
@@ -411,7 +500,12 @@ __global__ void __launch_bounds__(kGbThreads, 2)
             }
         }
         stage_store8(buf ^ 1);
-        cur = nxt;
+        if constexpr (kRouted) {
+            q8_route_store(rt, strip, lane);
+            cur = q8_blocks_from_strip(strip, lrow, khalf);
+        } else {
+            cur = nxt;
+        }
         __syncthreads();
     }
 
@@ -482,19 +576,35 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
     const bool wide = seq > 32;  // measured: the 64-token tile wins here even on a small grid (4096 x 4096 x 512: 100 vs 123 us)
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, 1), block(kGbThreads);
-#define RNB_LAUNCH_Q8(TT, BYTES, OFF) \
-    hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF>), grid, block, 0, stream, w, act.qs, act.d, out, rows, nb32, seq)
-    if (quant == kQ8_0) {
-        if (wide)
-            RNB_LAUNCH_Q8(2, 34, 2);
-        else
-            RNB_LAUNCH_Q8(1, 34, 2);
-    } else {
-        if (wide)
-            RNB_LAUNCH_Q8(2, 36, 4);
-        else
-            RNB_LAUNCH_Q8(1, 36, 4);
+    const bool routed = nb32 % 8 == 0;  // whole steps only: a partial step's 16-byte pieces would leave the last row
+#define RNB_LAUNCH_Q8R(TT, BYTES, OFF, R)                                                                              \
+    {                                                                                                                  \
+        constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
+        static bool configured = false;                                                                                \
+        if (!configured) { /* above the default 64 KB of dynamic LDS in the routed 64-token form */                    \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, BYTES, OFF, R>),          \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));              \
+            configured = true;                                                                                         \
+        }                                                                                                              \
+        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF, R>), grid, block, lds, stream, w, act.qs, act.d, out,  \
+                           rows, nb32, seq);                                                                           \
     }
+#define RNB_LAUNCH_Q8(TT, BYTES, OFF)                                                                                  \
+    if (routed) RNB_LAUNCH_Q8R(TT, BYTES, OFF, true) else RNB_LAUNCH_Q8R(TT, BYTES, OFF, false)
+    if (quant == kQ8_0) {
+        if (wide) {
+            RNB_LAUNCH_Q8(2, 34, 2);
+        } else {
+            RNB_LAUNCH_Q8(1, 34, 2);
+        }
+    } else {
+        if (wide) {
+            RNB_LAUNCH_Q8(2, 36, 4);
+        } else {
+            RNB_LAUNCH_Q8(1, 36, 4);
+        }
+    }
+#undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8
 }
 

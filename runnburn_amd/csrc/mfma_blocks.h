@@ -92,6 +92,71 @@ __device__ __forceinline__ int q6_scale(const Q6Row &r) {
     return static_cast<int>(__builtin_amdgcn_sbfe(static_cast<int>(word), 8 * (kSb & 3), 8));
 }
 
+// ---------------------------------------------------------------------------------------------
+// Route of a wave's 32 weight rows from global memory to the lanes that own them.  A lane that reads its own row
+// directly makes every load instruction touch 64 cache lines, and the vector cache, which looks up one line a cycle,
+// becomes the limit long before the matrix cores.  Here consecutive lanes take consecutive 16-byte pieces of a row
+// (kPieces per row step, so one instruction covers whole lines), the pieces go to a strip of LDS private to the wave
+// with rows kStride bytes apart, and each lane reads its row back from there.  Only the wave itself touches the strip:
+// LDS accesses of one wave execute in order, so no barrier is involved.
+// ---------------------------------------------------------------------------------------------
+template <int kPieces>
+struct RowRoute {
+    static constexpr int kN = (32 * kPieces + kWave - 1) / kWave;  // load instructions per row step
+    uint32_t goff[kN];  // byte offset of this lane's piece from the wave's first row (rows past the end: the last row)
+    uint32_t loff[kN];  // where it goes in the strip
+    uint4 v[kN];
+};
+
+template <int kPieces, int kStride>
+__device__ __forceinline__ void route_setup(RowRoute<kPieces> &rt, uint32_t rows_left, size_t row_bytes, int lane) {
+#pragma unroll
+    for (int i = 0; i < RowRoute<kPieces>::kN; i++) {
+        const uint32_t c = min(static_cast<uint32_t>(lane) + i * kWave, 32u * kPieces - 1);
+        const uint32_t r = c / kPieces, j = c - r * kPieces;
+        rt.goff[i] = static_cast<uint32_t>(min(r, rows_left - 1) * row_bytes) + 16 * j;
+        rt.loff[i] = r * kStride + 16 * j;
+    }
+}
+
+template <int kPieces>
+__device__ __forceinline__ void route_load(RowRoute<kPieces> &rt, const uint8_t *__restrict__ base) {
+#pragma unroll
+    for (int i = 0; i < RowRoute<kPieces>::kN; i++) rt.v[i] = ld_u4_a2(base + rt.goff[i]);
+}
+
+// 64-bit stores: the strip's row stride is a multiple of 8, not of 16, to keep the per-row reads off each other's banks
+template <int kPieces>
+__device__ __forceinline__ void route_store(const RowRoute<kPieces> &rt, uint8_t *strip, int lane) {
+#pragma unroll
+    for (int i = 0; i < RowRoute<kPieces>::kN; i++) {
+        if ((i + 1) * kWave <= 32 * kPieces || lane + i * kWave < 32 * kPieces) {
+            *reinterpret_cast<uint2 *>(strip + rt.loff[i]) = make_uint2(rt.v[i].x, rt.v[i].y);
+            *reinterpret_cast<uint2 *>(strip + rt.loff[i] + 8) = make_uint2(rt.v[i].z, rt.v[i].w);
+        }
+    }
+}
+
+constexpr int kQ6Pieces = 13;        // ql, qh and scales: 208 bytes; d is read by the row's lanes themselves
+constexpr int kQ6StripStride = 216;  // 54 dwords: the 32 rows' 64-bit reads fall on 32 different bank pairs
+
+// a lane's share of a Q6_K block from the wave's strip (same pieces as q6_load_row, without d)
+__device__ __forceinline__ void q6_row_from_strip(Q6Row &r, const uint8_t *row, int khalf) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int lh = 0; lh < 2; lh++)
+                r.h[h].ql[a][lh] = *reinterpret_cast<const uint2 *>(row + 64 * h + 32 * a + 16 * lh + 8 * khalf);
+#pragma unroll
+        for (int lh = 0; lh < 2; lh++)
+            r.h[h].qh[lh] = *reinterpret_cast<const uint2 *>(row + 128 + 32 * h + 16 * lh + 8 * khalf);
+    }
+    const uint2 s0 = *reinterpret_cast<const uint2 *>(row + 192), s1 = *reinterpret_cast<const uint2 *>(row + 200);
+    r.scales = make_uint4(s0.x, s0.y, s1.x, s1.y);
+}
+
 // cooperative copy of the workgroup's tokens' quantised activations of one 256-element block into LDS
 template <int kToks>
 struct Stage {
