@@ -120,15 +120,26 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
                       !b32 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     const uint32_t nb = static_cast<uint32_t>(cols / 256);
+    // workspace of the GEMMs that cut K into slices on small grids (null: none needed)
+    auto slice_ws = [&](uint32_t k_steps, float **ws) -> int {
+        *ws = nullptr;
+        const size_t floats = gemm_blocks_slice_floats(quant, r, k_steps, q);
+        if (floats == 0) return RNB_HIP_OK;
+        HIP_TRY(s.gemm_slices.reserve(floats * sizeof(float)));
+        *ws = s.gemm_slices.as<float>();
+        return RNB_HIP_OK;
+    };
+    float *ws = nullptr;
     if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
         // gemm_q4k.hip's 256-row x 64-token workgroups need about half the compute units' worth of tiles to pay off; below
         // that the 128 x 32 / 64 kernel of gemm_blocks.hip wins (4096 x 4096 x 64 tokens: 20 vs 34 us; 14336 x 4096 x 64:
         // 25 vs 40 us; at 14336 x 4096 x 512 the big tiles win, 93 vs 132 us)
         const uint64_t big_tiles = static_cast<uint64_t>((rows + 255) / 256) * ((seq + 63) / 64);
-        if (seq >= kGemmMinSeq && act.digits != nullptr && big_tiles < kGemmBigTilesMin)
-            launch_gemm_q4k_small(w_dev, act, out_dev, r, nb, q, s.stream);
-        else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
+        if (seq >= kGemmMinSeq && act.digits != nullptr && big_tiles < kGemmBigTilesMin) {
+            if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
+            launch_gemm_q4k_small(w_dev, act, out_dev, ws, r, nb, q, s.stream);
+        } else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_gemm_q4k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
         else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
@@ -140,21 +151,25 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ5K) {
-        if (seq >= kGemmMinSeq && act.digits != nullptr)
-            launch_gemm_q5k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
-        else if (seq >= kTokensMinSeq)
+        if (seq >= kGemmMinSeq && act.digits != nullptr) {
+            if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
+            launch_gemm_q5k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
+        } else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ5K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ6K) {
-        if (seq >= kGemmMinSeq)
-            launch_gemm_q6k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
-        else if (seq >= kTokensMinSeq)
+        if (seq >= kGemmMinSeq) {
+            if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
+            launch_gemm_q6k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
+        } else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (seq >= kGemmMinSeq && gemm_q8_mfma_supported(quant, static_cast<uint32_t>(cols / 32))) {
-        launch_gemm_q8_mfma(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
+        const uint32_t nb32 = static_cast<uint32_t>(cols / 32);
+        if (int st = slice_ws((nb32 + 7) / 8, &ws); st != RNB_HIP_OK) return st;
+        launch_gemm_q8_mfma(w_dev, quant, act, out_dev, ws, r, nb32, q, s.stream);
     } else {
         launch_gemv_block32(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     }

@@ -24,6 +24,8 @@
 // workgroup's tokens are staged in LDS, double-buffered, one barrier per step.
 #include "device_utils.h"
 #include "kernels.h"
+#include <algorithm>
+
 #include "mfma_blocks.h"
 
 namespace rnb {
@@ -33,7 +35,7 @@ namespace {
 template <int kTT>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q6k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                         float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq) {
+                         float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq, uint32_t nb_slice) {
     constexpr int kToks = 32 * kTT;
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride64];
     __shared__ __attribute__((aligned(16))) uint8_t s_w[kGbWaves][32 * kQ6StripStride];
@@ -63,19 +65,23 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     RowRoute<kQ6Pieces> rt;
     route_setup<kQ6Pieces, kQ6StripStride>(rt, rows - wrow0, static_cast<size_t>(nb) * kQ6KBytes, lane);
 
+    // K slice of this workgroup (blockIdx.z): blocks b0 .. b1, its sums go to the slice's own copy of the output
+    const uint32_t b0 = blockIdx.z * nb_slice, b1 = min(nb, b0 + nb_slice);
+    out += static_cast<size_t>(blockIdx.z) * seq * rows;
+
     Stage<kToks> st;
-    stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, 0, tid);
-    route_load(rt, wbase);
+    stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, b0, tid);
+    route_load(rt, wbase + static_cast<size_t>(b0) * kQ6KBytes);
     Q6Row cur;
-    cur.d = ld_f16(wrow + 208);
+    cur.d = ld_f16(wrow + static_cast<size_t>(b0) * kQ6KBytes + 208);
     route_store(rt, strip, lane);
     q6_row_from_strip(cur, strip + lrow * kQ6StripStride, khalf);
     stage_store<kToks>(st, s_a[0], s_dx[0], tid);
     __syncthreads();
 
-    for (uint32_t b = 0; b < nb; b++) {
-        const int buf = b & 1;
-        const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
+    for (uint32_t b = b0; b < b1; b++) {
+        const int buf = (b - b0) & 1;
+        const uint32_t bn = b + 1 < b1 ? b + 1 : b;  // the last step reloads its own block, unused
         stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, bn, tid);
         route_load(rt, wbase + static_cast<size_t>(bn) * kQ6KBytes);
         const float d_next = ld_f16(wrow + static_cast<size_t>(bn) * kQ6KBytes + 208);
@@ -160,7 +166,7 @@ template <int kTT, bool kFifth>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q45k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                          const uint8_t *__restrict__ adig, float *__restrict__ out, uint32_t rows, uint32_t nb,
-                         uint32_t seq) {
+                         uint32_t seq, uint32_t nb_slice) {
     constexpr int kToks = 32 * kTT;
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride128];
     __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
@@ -202,14 +208,17 @@ __global__ void __launch_bounds__(kGbThreads, 2)
             s_dig[buf][tid] = sdig;
         }
     };
-    stage_load5(0);
-    Q5Row cur = q45_load_row<kFifth>(wrow, khalf);
+    // K slice of this workgroup (blockIdx.z): blocks b0 .. b1, its sums go to the slice's own copy of the output
+    const uint32_t b0 = blockIdx.z * nb_slice, b1 = min(nb, b0 + nb_slice);
+    out += static_cast<size_t>(blockIdx.z) * seq * rows;
+    stage_load5(b0);
+    Q5Row cur = q45_load_row<kFifth>(wrow + static_cast<size_t>(b0) * kBlockBytes, khalf);
     stage_store5(0);
     __syncthreads();
 
-    for (uint32_t b = 0; b < nb; b++) {
-        const int buf = b & 1;
-        const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
+    for (uint32_t b = b0; b < b1; b++) {
+        const int buf = (b - b0) & 1;
+        const uint32_t bn = b + 1 < b1 ? b + 1 : b;  // the last step reloads its own block, unused
         stage_load5(bn);
         const Q5Row nxt = q45_load_row<kFifth>(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
@@ -398,7 +407,7 @@ constexpr size_t q8_lds_bytes(bool routed) {
 template <int kTT, int kBlockBytes, int kQsOff, bool kRouted>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q8_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                        float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq) {
+                        float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq, uint32_t steps_slice) {
     constexpr int kToks = 32 * kTT;
     constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
@@ -410,7 +419,9 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
     const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
     const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb32 * kBlockBytes;
-    const uint32_t steps = (nb32 + 7) / 8;
+    // K slice of this workgroup (blockIdx.z): steps s0 .. s1, its sums go to the slice's own copy of the output
+    const uint32_t s0 = blockIdx.z * steps_slice, s1 = min((nb32 + 7) / 8, s0 + steps_slice);
+    out += static_cast<size_t>(blockIdx.z) * seq * rows;
     const size_t tok_bytes = static_cast<size_t>(nb32) * 32;
 
     float accf[kTT][16];
@@ -457,21 +468,21 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     uint8_t *strip = s_dyn + q8_lds_bytes<kTT>(false) + wave * kQ8StripBytes;
     Q8Route rt;
     Q8Blocks cur, nxt;
-    stage_load8(0);
+    stage_load8(s0);
     if constexpr (kRouted) {
         q8_route_setup<kBlockBytes, kQsOff>(rt, rows - wrow0, static_cast<size_t>(nb32) * kBlockBytes, lane);
-        q8_route_load(rt, wbase);
+        q8_route_load(rt, wbase + static_cast<size_t>(s0) * 8 * kBlockBytes);
         q8_route_store(rt, strip, lane);
         cur = q8_blocks_from_strip(strip, lrow, khalf);
     } else {
-        cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, 0, nb32, khalf);
+        cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, s0 * 8, nb32, khalf);
     }
     stage_store8(0);
     __syncthreads();
 
-    for (uint32_t step = 0; step < steps; step++) {
-        const int buf = step & 1;
-        const uint32_t sn = step + 1 < steps ? step + 1 : step;
+    for (uint32_t step = s0; step < s1; step++) {
+        const int buf = (step - s0) & 1;
+        const uint32_t sn = step + 1 < s1 ? step + 1 : step;
         stage_load8(sn);
         if constexpr (kRouted)
             q8_route_load(rt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
@@ -529,53 +540,116 @@ static bool wide_tiles(uint32_t row_tiles, uint32_t seq) {
     return seq > 32 && static_cast<uint64_t>(row_tiles) * ((seq + 63) / 64) >= 512;
 }
 
-void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                          hipStream_t stream) {
+// ---------------------------------------------------------------------------------------------
+// K slices.  A grid of rows / 128 x tokens / 32 workgroups leaves most of the 256 compute units idle when both are
+// small (a 4096-row projection of 64 tokens: 64 workgroups, each walking the whole row): then the blocks of a row are
+// dealt out to blockIdx.z, every slice writes its own copy of the output and a second small kernel adds the copies in
+// slice order, so the result does not depend on which slice finishes first.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kSliceTargetWgs = 512;  // slices are added until the grid has this many workgroups
+constexpr uint32_t kSliceMax = 16;
+
+// measured on 4096 x 4096 and 4096 x 14336 at 16 .. 256 tokens: up to 5x faster where the unsliced grid has at most 128
+// workgroups; at 256 workgroups only Q6_K and Q8 (the slowest per block) still gain, hence split_at_256; a slice keeps
+// four 256-element steps, two on the smallest grids
+static uint32_t k_slices(uint64_t wgs, uint32_t k_steps, bool split_at_256) {
+    if (wgs > 256 || (wgs == 256 && !split_at_256)) return 1;
+    const uint64_t want = (kSliceTargetWgs + wgs - 1) / wgs;
+    const uint32_t min_steps = wgs <= 32 ? 2 : 4;
+    return static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>({want, k_steps / min_steps, kSliceMax})));
+}
+
+static uint64_t tile_grid(uint32_t rows, uint32_t seq, bool wide) {
+    return static_cast<uint64_t>((rows + kGbRows - 1) / kGbRows) * (wide ? (seq + 63) / 64 : (seq + 31) / 32);
+}
+
+namespace {
+__global__ void __launch_bounds__(256) sum_slices_kernel(const float *__restrict__ parts, float *__restrict__ out, size_t n,
+                                                         uint32_t slices) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n) return;
+    float acc = parts[i];
+    for (uint32_t z = 1; z < slices; z++) acc += parts[z * n + i];
+    out[i] = acc;
+}
+}  // namespace
+
+static void sum_slices(const float *parts, float *out, size_t n, uint32_t slices, hipStream_t stream) {
+    hipLaunchKernelGGL(sum_slices_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, stream, parts, out, n,
+                       slices);
+}
+
+size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps, uint32_t seq) {
+    if (rows == 0 || seq == 0 || k_steps == 0) return 0;
+    const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    const bool wide = (quant == kQ8_0 || quant == kQ8_1) ? seq > 32 : wide_tiles(row_tiles, seq);
+    const uint32_t slices = k_slices(tile_grid(rows, seq, wide), k_steps, quant != kQ4K && quant != kQ5K);
+    return slices > 1 ? static_cast<size_t>(slices) * seq * rows : 0;
+}
+
+void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
-    if (wide_tiles(row_tiles, seq)) {
-        const dim3 grid(row_tiles, (seq + 63) / 64, 1);
-        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, out, rows, nb, seq);
+    const bool wide = wide_tiles(row_tiles, seq);
+    const uint32_t slices = slice_out ? k_slices(tile_grid(rows, seq, wide), nb, true) : 1;
+    const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
+    float *dst = nz > 1 ? slice_out : out;
+    if (wide) {
+        const dim3 grid(row_tiles, (seq + 63) / 64, nz);
+        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
+                           nb_slice);
     } else {
-        const dim3 grid(row_tiles, (seq + 31) / 32, 1);
-        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, out, rows, nb, seq);
+        const dim3 grid(row_tiles, (seq + 31) / 32, nz);
+        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
+                           nb_slice);
     }
+    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
 template <bool kFifth>
-static void launch_gemm_q45k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                             hipStream_t stream) {
+static void launch_gemm_q45k(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                             uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
-    if (wide_tiles(row_tiles, seq)) {
-        const dim3 grid(row_tiles, (seq + 63) / 64, 1);
+    const bool wide = wide_tiles(row_tiles, seq);
+    const uint32_t slices = slice_out ? k_slices(tile_grid(rows, seq, wide), nb, false) : 1;
+    const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
+    float *dst = nz > 1 ? slice_out : out;
+    if (wide) {
+        const dim3 grid(row_tiles, (seq + 63) / 64, nz);
         hipLaunchKernelGGL((gemm_q45k_mfma_kernel<2, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
-                           out, rows, nb, seq);
+                           dst, rows, nb, seq, nb_slice);
     } else {
-        const dim3 grid(row_tiles, (seq + 31) / 32, 1);
+        const dim3 grid(row_tiles, (seq + 31) / 32, nz);
         hipLaunchKernelGGL((gemm_q45k_mfma_kernel<1, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
-                           out, rows, nb, seq);
+                           dst, rows, nb, seq, nb_slice);
     }
+    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
-void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                          hipStream_t stream) {
-    launch_gemm_q45k<true>(w, act, out, rows, nb, seq, stream);
+void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream) {
+    launch_gemm_q45k<true>(w, act, out, slice_out, rows, nb, seq, stream);
 }
 
-void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                           hipStream_t stream) {
-    launch_gemm_q45k<false>(w, act, out, rows, nb, seq, stream);
+void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                           uint32_t seq, hipStream_t stream) {
+    launch_gemm_q45k<false>(w, act, out, slice_out, rows, nb, seq, stream);
 }
 
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32) { return (quant == kQ8_0 || quant == kQ8_1) && nb32 >= 1; }
 
-void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
-                         uint32_t seq, hipStream_t stream) {
+void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
+                         uint32_t nb32, uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb32 == 0) return;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
     const bool wide = seq > 32;  // measured: the 64-token tile wins here even on a small grid (4096 x 4096 x 512: 100 vs 123 us)
-    const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, 1), block(kGbThreads);
+    const uint32_t steps = (nb32 + 7) / 8;
+    const uint32_t slices = slice_out ? k_slices(tile_grid(rows, seq, wide), steps, true) : 1;
+    const uint32_t steps_slice = (steps + slices - 1) / slices, nz = (steps + steps_slice - 1) / steps_slice;
+    float *dst = nz > 1 ? slice_out : out;
+    const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, nz), block(kGbThreads);
     const bool routed = nb32 % 8 == 0;  // whole steps only: a partial step's 16-byte pieces would leave the last row
 #define RNB_LAUNCH_Q8R(TT, BYTES, OFF, R)                                                                              \
     {                                                                                                                  \
@@ -586,8 +660,8 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));              \
             configured = true;                                                                                         \
         }                                                                                                              \
-        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF, R>), grid, block, lds, stream, w, act.qs, act.d, out,  \
-                           rows, nb32, seq);                                                                           \
+        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF, R>), grid, block, lds, stream, w, act.qs, act.d, dst,  \
+                           rows, nb32, seq, steps_slice);                                                              \
     }
 #define RNB_LAUNCH_Q8(TT, BYTES, OFF)                                                                                  \
     if (routed) RNB_LAUNCH_Q8R(TT, BYTES, OFF, true) else RNB_LAUNCH_Q8R(TT, BYTES, OFF, false)
@@ -606,6 +680,7 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     }
 #undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8
+    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
 }  // namespace rnb

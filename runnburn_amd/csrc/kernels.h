@@ -86,19 +86,23 @@ void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *
                           uint32_t seq, hipStream_t stream);
 
 // Q6_K / Q5_K x Q8_K and Q8_0 / Q8_1 x Q8 GEMMs on int8 MFMA (scale groups applied on the vector units); same contracts as
-// launch_gemv_q6k / launch_gemv_block32, intended for seq >= 16
-void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                          hipStream_t stream);
+// launch_gemv_q6k / launch_gemv_block32, intended for seq >= 16.  Small grids are cut into K slices that are summed by
+// a second kernel: slice_out is the workspace for that, gemm_blocks_slice_floats(quant, rows, k_steps, seq) floats
+// (k_steps = 256-element steps per row: blocks, or ceil(32-element blocks / 8)); when that is 0, or slice_out is null,
+// the kernel writes out directly.
+size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps, uint32_t seq);
+void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream);
 // Q5_K needs act.digits (the quantiser writes them for 16+ tokens)
-void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                          hipStream_t stream);
+void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, hipStream_t stream);
 // Q4_K through the same kernel (scales on the vector units): for shapes that give gemm_q4k.hip's 256 x 64 tiles too few
 // workgroups to fill the chip
-void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                           hipStream_t stream);
+void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                           uint32_t seq, hipStream_t stream);
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32);
-void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
-                         uint32_t seq, hipStream_t stream);
+void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
+                         uint32_t nb32, uint32_t seq, hipStream_t stream);
 // Q4_K x Q8_K GEMM on int8 MFMA; same contract as launch_gemv_q4k, intended for seq >= 16
 void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);

@@ -454,6 +454,22 @@ def test_q5k_gemm_extreme_blocks(rnb, oracle):
                 "q5k gemm extremes")
 
 
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1])
+@pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 16), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
+def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
+    """Grids too small for the chip are cut along K (blockIdx.z) and the slices' outputs added by a second kernel in
+    slice order: 13 slices of 3 blocks and one of 1 (the cap of 16 slices asked for), slices of unequal length, and the
+    two shapes where every slice has whole steps.  The sum does not depend on the batch around a token."""
+    cols = nblk * 256
+    w = oracle.make_weights(quant, rows, cols, 900 + rows)
+    x = oracle.fill_normal(seq * cols, 910 + seq, 1.0)
+    got = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"k slices quant {quant} rows {rows} nblk {nblk} seq {seq}")
+    rev = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
 @pytest.mark.parametrize("quant", [Q8_0, Q8_1])
 @pytest.mark.parametrize("rows,cols,seq", [(32, 32, 16), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
                                            (1, 4096, 16), (300, 288, 100)])
