@@ -61,7 +61,7 @@ int hip_fail(const char *what, hipError_t e) {
 // Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
 constexpr size_t kGemmMinSeq = 16;
 // Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
-constexpr uint64_t kGemmBigTilesMin = 128;
+constexpr uint64_t kGemmBigTilesMin = 32;
 // Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
 constexpr size_t kTokensMinSeq = 4;
 
@@ -132,16 +132,21 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     float *ws = nullptr;
     if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
-        // gemm_q4k.hip's 256-row x 64-token workgroups need about half the compute units' worth of tiles to pay off; below
-        // that the 128 x 32 / 64 kernel of gemm_blocks.hip wins (4096 x 4096 x 64 tokens: 20 vs 34 us; 14336 x 4096 x 64:
-        // 25 vs 40 us; at 14336 x 4096 x 512 the big tiles win, 93 vs 132 us)
+        // gemm_q4k.hip's 256-row x 64-token workgroups (K cut into slices up to 128 tiles) win from 32 tiles on when the
+        // token tile is more than half full; below that the 128 x 32 kernel of gemm_blocks.hip, sliced as well, does
+        // (4096 x 4096 x 64 tokens, 16 tiles: 11.7 vs 14.8 us; 14336 x 4096 x 32: 18.1 vs 20.6 us; 14336 x 4096 x 64,
+        // 56 tiles: 28.3 vs 24.0 us; 4096 x 14336 x 128, 32 tiles: 43.2 vs 32.9 us)
         const uint64_t big_tiles = static_cast<uint64_t>((rows + 255) / 256) * ((seq + 63) / 64);
-        if (seq >= kGemmMinSeq && act.digits != nullptr && big_tiles < kGemmBigTilesMin) {
+        if (seq >= kGemmMinSeq && act.digits != nullptr && (big_tiles < kGemmBigTilesMin || seq <= 32)) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q4k_small(w_dev, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
-            launch_gemm_q4k_mfma(w_dev, act, out_dev, r, nb, q, s.stream);
-        else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
+        } else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0) {
+            if (const size_t floats = gemm_q4k_slice_floats(r, nb, q)) {
+                HIP_TRY(s.gemm_slices.reserve(floats * sizeof(float)));
+                ws = s.gemm_slices.as<float>();
+            }
+            launch_gemm_q4k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
+        } else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);

@@ -574,7 +574,7 @@ __global__ void __launch_bounds__(256) sum_slices_kernel(const float *__restrict
 }
 }  // namespace
 
-static void sum_slices(const float *parts, float *out, size_t n, uint32_t slices, hipStream_t stream) {
+void launch_sum_slices(const float *parts, float *out, size_t n, uint32_t slices, hipStream_t stream) {
     hipLaunchKernelGGL(sum_slices_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, stream, parts, out, n,
                        slices);
 }
@@ -604,7 +604,7 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slic
         hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
                            nb_slice);
     }
-    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
+    if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
 template <bool kFifth>
@@ -625,7 +625,7 @@ static void launch_gemm_q45k(const uint8_t *w, ActView act, float *out, float *s
         hipLaunchKernelGGL((gemm_q45k_mfma_kernel<1, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
                            dst, rows, nb, seq, nb_slice);
     }
-    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
+    if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
 void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
@@ -680,7 +680,7 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     }
 #undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8
-    if (nz > 1) sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
+    if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 
 }  // namespace rnb

@@ -104,8 +104,12 @@ bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32);
 void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
                          uint32_t nb32, uint32_t seq, hipStream_t stream);
 // Q4_K x Q8_K GEMM on int8 MFMA; same contract as launch_gemv_q4k, intended for seq >= 16
-void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
+// Up to 128 tiles the K range is cut into slices (workspace: gemm_q4k_slice_floats floats, as for the kernels above)
+size_t gemm_q4k_slice_floats(uint32_t rows, uint32_t nb, uint32_t seq);
+void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream);
+// out[i] = parts[0][i] + parts[1][i] + ... in that order (n floats per slice)
+void launch_sum_slices(const float *parts, float *out, size_t n, uint32_t slices, hipStream_t stream);
 
 // ---- gathered sparse-MoE ------------------------------------------------------------------
 // Slots grouped by expert (device arrays).  Group i covers sorted positions [start[i], start[i+1]);

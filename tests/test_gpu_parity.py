@@ -369,10 +369,12 @@ def test_gemv_batch_long_rows(rnb, oracle, quant):
 
 
 @pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
-                                           (1, 1, 16), (257, 5, 40), (4097, 1, 513), (8200, 2, 260)])
+                                           (1, 1, 16), (257, 5, 40), (4097, 1, 513), (8200, 2, 260), (2050, 9, 260),
+                                           (8192, 8, 65)])
 def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
-    """Q4_K with 16+ tokens: shapes with fewer than 128 tiles of 256 rows x 64 tokens take the 128 x 32 / 64 kernel of
-    gemm_blocks.hip, the last two (153 and 165 tiles, both dimensions off the tile) the ping-pong kernel of gemm_q4k.hip."""
+    """Q4_K with 16+ tokens: shapes with fewer than 32 tiles of 256 rows x 64 tokens take the 128 x 32 / 64 kernel of
+    gemm_blocks.hip, the last four the ping-pong kernel of gemm_q4k.hip: 153 and 165 tiles, both dimensions off the
+    tile, then 45 and 64 tiles, where K is cut into two slices (5 + 4 blocks, 4 + 4) that a second kernel adds."""
     cols = nblk * 256
     w = oracle.make_weights(Q4_K, rows, cols, 70 + rows)
     x = oracle.fill_normal(seq * cols, 80 + seq, 1.0)
