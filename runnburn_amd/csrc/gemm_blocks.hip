@@ -579,10 +579,20 @@ void launch_sum_slices(const float *parts, float *out, size_t n, uint32_t slices
                        slices);
 }
 
+// Q6_K spends the most vector work per tile, and the 64-token form saves the most of it: it also wins where its
+// workgroups fill the 256 compute units just once (4096 rows x 512 tokens x 14336: 164 vs 189 us; with 224 or 320
+// workgroups the 32-token form is level or ahead)
+static bool q6_wide_tiles(uint32_t row_tiles, uint32_t seq) {
+    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * ((seq + 63) / 64);
+    return seq > 32 && (tiles >= 512 || (tiles > 224 && tiles <= 256));
+}
+
 size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps, uint32_t seq) {
     if (rows == 0 || seq == 0 || k_steps == 0) return 0;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
-    const bool wide = (quant == kQ8_0 || quant == kQ8_1) ? seq > 32 : wide_tiles(row_tiles, seq);
+    const bool wide = (quant == kQ8_0 || quant == kQ8_1) ? seq > 32
+                      : quant == kQ6K                    ? q6_wide_tiles(row_tiles, seq)
+                                                         : wide_tiles(row_tiles, seq);
     const uint32_t slices = k_slices(tile_grid(rows, seq, wide), k_steps, quant != kQ4K && quant != kQ5K);
     return slices > 1 ? static_cast<size_t>(slices) * seq * rows : 0;
 }
@@ -591,7 +601,7 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slic
                           uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
-    const bool wide = wide_tiles(row_tiles, seq);
+    const bool wide = q6_wide_tiles(row_tiles, seq);
     const uint32_t slices = slice_out ? k_slices(tile_grid(rows, seq, wide), nb, true) : 1;
     const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
     float *dst = nz > 1 ? slice_out : out;
