@@ -58,8 +58,20 @@ int hip_fail(const char *what, hipError_t e) {
     } while (0)
 
 // Quantise seq*cols staged floats on the device into the state's activation scratch.
-// Minimum tokens for which the MFMA GEMM replaces one GEMV launch per token.
-constexpr size_t kGemmMinSeq = 16;
+// Minimum tokens for which the MFMA GEMMs replace the vector-unit kernels, whose time grows with every token while a
+// GEMM's 32-token tile costs the same from 1 to 32.  Measured crossovers: Q6_K 4096 x 14336 (48 MB) 4 tokens (26.9 us
+// either way; 8 tokens 47 vs 27), Q4_K 14336 x 4096 (33 MB) 4 (21 vs 16 us), Q8_0 4096 x 14336 (62 MB) 3, Q8_0
+// 4096 x 4096 (18 MB) 5, Q4_K and Q5_K 4096 x 4096 (9 and 12 MB) 8 (10.4 vs 9.8 us).
+constexpr size_t kGemmMinSeqLarge = 4, kGemmMinSeqSmall = 8, kGemmLargeBytes = size_t(16) << 20;
+size_t gemm_min_seq(uint32_t quant, size_t rows, size_t cols) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return kGemmMinSeqSmall;
+    return rows * (cols / qi.elems) * qi.bytes >= kGemmLargeBytes ? kGemmMinSeqLarge : kGemmMinSeqSmall;
+}
+// The Q8_K quantiser adds the per-32 sums as two digits (the Q4_K / Q5_K GEMMs' mins term) from this many tokens on.
+constexpr size_t kDigitsMinSeq = kGemmMinSeqLarge < kGemmMinSeqSmall ? kGemmMinSeqLarge : kGemmMinSeqSmall;
+// Minimum tokens for which the grouped MoE GEMMs on the matrix cores are considered.
+constexpr size_t kMoeMfmaMinTokens = 16;
 // Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
 constexpr uint64_t kGemmBigTilesMin = 32;
 // Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
@@ -75,7 +87,7 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
     } else {
         HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
         HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
-        s.act_has_digits = seq >= kGemmMinSeq;
+        s.act_has_digits = seq >= kDigitsMinSeq;
         if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
         uint8_t *digits = s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr;
         launch_quantize_q8k(x_dev, n / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
@@ -120,6 +132,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
                       !b32 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     const uint32_t nb = static_cast<uint32_t>(cols / 256);
+    const size_t min_gemm_seq = gemm_min_seq(quant, rows, cols);
     // workspace of the GEMMs that cut K into slices on small grids (null: none needed)
     auto slice_ws = [&](uint32_t k_steps, float **ws) -> int {
         *ws = nullptr;
@@ -137,10 +150,10 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         // (4096 x 4096 x 64 tokens, 16 tiles: 11.7 vs 14.8 us; 14336 x 4096 x 32: 18.1 vs 20.6 us; 14336 x 4096 x 64,
         // 56 tiles: 28.3 vs 24.0 us; 4096 x 14336 x 128, 32 tiles: 43.2 vs 32.9 us)
         const uint64_t big_tiles = static_cast<uint64_t>((rows + 255) / 256) * ((seq + 63) / 64);
-        if (seq >= kGemmMinSeq && act.digits != nullptr && (big_tiles < kGemmBigTilesMin || seq <= 32)) {
+        if (seq >= min_gemm_seq && act.digits != nullptr && (big_tiles < kGemmBigTilesMin || seq <= 32)) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q4k_small(w_dev, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kGemmMinSeq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0) {
+        } else if (seq >= min_gemm_seq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0) {
             if (const size_t floats = gemm_q4k_slice_floats(r, nb, q)) {
                 HIP_TRY(s.gemm_slices.reserve(floats * sizeof(float)));
                 ws = s.gemm_slices.as<float>();
@@ -156,7 +169,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ5K) {
-        if (seq >= kGemmMinSeq && act.digits != nullptr) {
+        if (seq >= min_gemm_seq && act.digits != nullptr) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q5k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
         } else if (seq >= kTokensMinSeq)
@@ -164,14 +177,14 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ6K) {
-        if (seq >= kGemmMinSeq) {
+        if (seq >= min_gemm_seq) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q6k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
         } else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
-    } else if (seq >= kGemmMinSeq && gemm_q8_mfma_supported(quant, static_cast<uint32_t>(cols / 32))) {
+    } else if (seq >= min_gemm_seq && gemm_q8_mfma_supported(quant, static_cast<uint32_t>(cols / 32))) {
         const uint32_t nb32 = static_cast<uint32_t>(cols / 32);
         if (int st = slice_ws((nb32 + 7) / 8, &ws); st != RNB_HIP_OK) return st;
         launch_gemm_q8_mfma(w_dev, quant, act, out_dev, ws, r, nb32, q, s.stream);
@@ -302,7 +315,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
     const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
     HIP_TRY(s.ffn_mid.reserve(mid_bytes));
     const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
-    const bool small = seq < kGemmMinSeq && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
+    const bool small = seq < gemm_min_seq(kQ4K, n_ff, n_embd) && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
     ActView act;
     int st = RNB_HIP_OK;
     if (small && seq == 1 && reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) {
@@ -331,7 +344,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
             HIP_TRY(s.act_qs.reserve(n));
             HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
             HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
-            s.act_has_digits = seq >= kGemmMinSeq;
+            s.act_has_digits = seq >= kDigitsMinSeq;
             if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
             launch_quantize_q8k_gated(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), n / 256, gelu, s.act_qs.as<int8_t>(),
                                       s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
@@ -455,7 +468,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     // Batches with at least four slots per routed expert on average: the expert GEMMs run on the matrix cores (a
     // 32-token tile costs the same whatever its number of live tokens, the integer-dot kernels cost per token; measured
     // crossover on 128 experts x top-8: 64 tokens) and need the quantiser's digits
-    const bool mfma = token_count >= kGemmMinSeq && n_slots >= 4 * n_groups &&
+    const bool mfma = token_count >= kMoeMfmaMinTokens && n_slots >= 4 * n_groups &&
                       moe_mfma_supported(static_cast<uint32_t>(sh.nb_in), static_cast<uint32_t>(sh.nb_mid), down_quant);
     const bool inline_tables = !mfma && table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
     MoeInlineTables inl;

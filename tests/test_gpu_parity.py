@@ -456,6 +456,21 @@ def test_q5k_gemm_extreme_blocks(rnb, oracle):
                 "q5k gemm extremes")
 
 
+@pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 8192, 4096, 4), (Q4_K, 8192, 4096, 7), (Q5_K, 6144, 4096, 6),
+                                                 (Q6_K, 4096, 5120, 5), (Q8_0, 4096, 4096, 4), (Q8_1, 4096, 4096, 15),
+                                                 (Q4_K, 4096, 4096, 8), (Q6_K, 2048, 4096, 11)])
+def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
+    """Matrices of 16 MB and more go to the matrix-core GEMMs from 4 tokens on, smaller ones from 8 (a 32-token tile
+    mostly empty: loads of the missing tokens repeat the last one, their results are not stored)."""
+    w = oracle.make_weights(quant, rows, cols, 1200 + seq)
+    x = oracle.fill_normal(seq * cols, 1210 + seq, 1.0)
+    got = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"few tokens quant {quant} rows {rows} cols {cols} seq {seq}")
+    rev = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
 @pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1])
 @pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 16), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
 def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
