@@ -298,7 +298,8 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
                          const uint8_t *__restrict__ mdig, const uint32_t *__restrict__ grp_expert,
                          const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
-                         const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb) {
+                         const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
+                         uint32_t tiles_per_wg) {
     constexpr bool kSix = kQuant == kQ6K;
     constexpr bool kFifth = kQuant == kQ5K;
     constexpr int kStride = kSix ? kGbStride64 : kGbStride128;
@@ -309,51 +310,96 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid >> 6;
     const int lrow = lane & 31, khalf = lane >> 5;
-    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    const uint8_t *wrow = down_all + (static_cast<size_t>(expert) * n_embd + min(row, n_embd - 1)) * row_bytes;
+    // The workgroup walks tiles_per_wg row tiles of 128 against one staged token tile: map and image are made once,
+    // and the weight blocks of the whole walk form one stream that is requested one block ahead across row tiles.
+    const uint32_t row_tiles = (n_embd + kGbRows - 1) / kGbRows;
+    const uint32_t rt0 = blockIdx.x * tiles_per_wg, rt_n = min(tiles_per_wg, row_tiles - rt0);
+    const uint32_t steps = rt_n * nb;
+    auto row_of = [&](uint32_t rt) { return (rt0 + rt) * kGbRows + wave * 32 + lrow; };
+    auto block_ptr = [&](uint32_t rt, uint32_t b) {
+        return down_all + (static_cast<size_t>(expert) * n_embd + min(row_of(rt), n_embd - 1)) * row_bytes + b * kBlockBytes;
+    };
+    // Q6_K rows come in by whole cache lines through the wave's strip of LDS (RowRoute: the lane-owns-row loads of
+    // q6_load_row touch 64 lines per instruction); the other formats' 16-byte loads go straight to the lane
+    __shared__ __attribute__((aligned(16))) uint8_t s_w[kSix ? kGbWaves : 1][kSix ? 32 * kQ6StripStride : 16];
+    uint8_t *strip = s_w[kSix ? wave : 0];
+    RowRoute<kQ6Pieces> route;
+    float d_next = 0.0f;
+    auto q6_request = [&](uint32_t rt, uint32_t b) {  // block b of row tile rt: pieces into route.v, d into d_next
+        const uint32_t first = min((rt0 + rt) * kGbRows + wave * 32, n_embd - 1);  // the wave's first row
+        // offsets of rows past the end were clamped to the last row at set-up for the first row tile's distance to the
+        // end; row tiles further down are never short of rows unless they are the last one, which set-up cannot know,
+        // so the clamp is redone per request
+        route_setup<kQ6Pieces, kQ6StripStride>(route, n_embd - first, row_bytes, lane);
+        route_load(route, down_all + (static_cast<size_t>(expert) * n_embd + first) * row_bytes + b * kBlockBytes);
+        d_next = ld_f16(block_ptr(rt, b) + 208);
+    };
+    auto q6_take = [&](Q6Row &r) {
+        route_store(route, strip, lane);
+        q6_row_from_strip(r, strip + lrow * kQ6StripStride, khalf);
+        r.d = d_next;
+    };
 
     for (uint32_t tile0 = 0; tile0 < count; tile0 += kMmToks) {
         Q6Row c6{};
         Q5Row c5{};
+        // the first weight block does not depend on the token lists: requested before them
         if constexpr (kSix)
-            c6 = q6_load_row(wrow, khalf);
+            q6_request(0, 0);
         else
-            c5 = q45_load_row<kFifth>(wrow, khalf);
+            c5 = q45_load_row<kFifth>(block_ptr(0, 0), khalf);
         if (tile0) __syncthreads();
         tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, count - tile0, tid);
         __syncthreads();
         tile_image_fill(img, s_map, mq, md, mdig, tid);
+        if constexpr (kSix) q6_take(c6);
         __syncthreads();
         float accf[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) accf[i] = 0.0f;
-        for (uint32_t b = 0; b < nb; b++) {
-            const uint32_t bn = b + 1 < nb ? b + 1 : b;
-            Q6Row n6{};
+        uint32_t rt = 0, b = 0;
+        for (uint32_t s = 0; s < steps; s++) {
+            uint32_t rtn = rt, bn = b + 1;  // the step after this one; the last step reloads its own block, unused
+            if (bn == nb) {
+                bn = 0;
+                rtn = rt + 1;
+            }
+            if (s + 1 == steps) {
+                rtn = rt;
+                bn = b;
+            }
             Q5Row n5{};
             float val[16];
             if constexpr (kSix) {
-                n6 = q6_load_row(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+                q6_request(rtn, bn);
                 q6_block_tile(c6, img.act(b) + lrow * kStride + 8 * khalf, val);
             } else {
-                n5 = q45_load_row<kFifth>(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+                n5 = q45_load_row<kFifth>(block_ptr(rtn, bn), khalf);
                 q45_block_tile<kFifth>(c5, img.act(b) + lrow * kStride + 16 * khalf, img.dig(b)[lrow], khalf, val);
             }
             tile_scale_add(img.dx(b), khalf, val, accf);
-            c6 = n6;
+            if constexpr (kSix) q6_take(c6);
             c5 = n5;
-        }
-        if (row < n_embd) {
+            if (b + 1 == nb) {  // the row tile is complete
+                const uint32_t row = row_of(rt);
+                if (row < n_embd) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int t = 8 * (r >> 2) + 4 * khalf + (r & 3);
-                const uint32_t slot = s_map.out_row[t];
-                // fanout.rs:306-308: the expert's output times the slot's route weight
-                if (slot != 0xffffffffu) slot_out[static_cast<size_t>(slot) * n_embd + row] = accf[r] * s_map.scale[t];
+                    for (int r = 0; r < 16; r++) {
+                        const int t = 8 * (r >> 2) + 4 * khalf + (r & 3);
+                        const uint32_t slot = s_map.out_row[t];
+                        // fanout.rs:306-308: the expert's output times the slot's route weight
+                        if (slot != 0xffffffffu)
+                            slot_out[static_cast<size_t>(slot) * n_embd + row] = accf[r] * s_map.scale[t];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 16; i++) accf[i] = 0.0f;
             }
+            rt = rtn;
+            b = bn;
         }
     }
 }
@@ -373,11 +419,12 @@ void allow_lds(K kernel, size_t bytes) {
 
 // the tile image (all blocks of 32 tokens) must fit the LDS of a compute unit beside the small static arrays
 constexpr size_t kMmLdsLimit = 150 * 1024;
+constexpr size_t kMmQ6DownLdsLimit = kMmLdsLimit - kGbWaves * 32 * kQ6StripStride;  // beside the four waves' strips
 
 bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
     const size_t gu = TileImage<kGbStride128, true>::bytes(nb_in);
     const size_t dn = down_quant == kQ6K ? TileImage<kGbStride64, false>::bytes(nb_mid) : TileImage<kGbStride128, true>::bytes(nb_mid);
-    return nb_in >= 1 && nb_mid >= 1 && gu <= kMmLdsLimit && dn <= kMmLdsLimit;
+    return nb_in >= 1 && nb_mid >= 1 && gu <= kMmLdsLimit && dn <= (down_quant == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit);
 }
 
 void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
@@ -393,11 +440,18 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
 void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
                           const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (groups.n_groups == 0 || n_embd == 0) return;
-    const dim3 grid((n_embd + kGbRows - 1) / kGbRows, groups.n_groups, 1), block(kGbThreads);
+    // A workgroup's setup (group, map, image: a chain of dependent loads) costs more than a row tile's few blocks, and
+    // about three workgroups fit a compute unit: row tiles are merged (up to 4 per workgroup) until the grid fits them at
+    // once (cfg5's shape, 16 row tiles x 126 groups, 64 tokens: 1 / 2 / 4 / 8 tiles per workgroup 72 / 62 / 59 / 62 us)
+    const uint32_t row_tiles = (n_embd + kGbRows - 1) / kGbRows;
+    uint32_t tiles_per_wg = 1;
+    while (tiles_per_wg < 4 && static_cast<uint64_t>((row_tiles + tiles_per_wg - 1) / tiles_per_wg) * groups.n_groups > 768)
+        tiles_per_wg *= 2;
+    const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1), block(kGbThreads);
 #define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
-    allow_lds<static_cast<int>(Q)>(moe_down_mfma_kernel<Q>, kMmLdsLimit);                                             \
+    allow_lds<static_cast<int>(Q)>(moe_down_mfma_kernel<Q>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit);                                           \
     hipLaunchKernelGGL((moe_down_mfma_kernel<Q>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
-                       groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid)
+                       groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg)
     if (down_quant == kQ6K) {
         RNB_LAUNCH_DM(kQ6K, (TileImage<kGbStride64, false>::bytes(nb_mid)));
     } else if (down_quant == kQ5K) {

@@ -679,11 +679,14 @@ def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant
 
 @pytest.mark.parametrize("tokens,n_expert,k,n_ff,n_embd,down_quant", [(16, 8, 2, 256, 256, Q6_K), (64, 3, 2, 512, 768, Q4_K),
                                                                      (100, 2, 2, 768, 512, Q5_K), (33, 20, 4, 300 * 0 + 512, 1280, Q6_K),
-                                                                     (40, 5, 3, 1024, 256, Q4_K), (20, 64, 3, 256, 512, Q6_K)])
+                                                                     (40, 5, 3, 1024, 256, Q4_K), (20, 64, 3, 256, 512, Q6_K),
+                                                                     (64, 128, 8, 256, 1792, Q6_K), (48, 96, 8, 256, 1792, Q4_K)])
 def test_moe_prefill_matrix_core_path(rnb, oracle, tokens, n_expert, k, n_ff, n_embd, down_quant):
     """16 or more tokens and at least four slots per routed expert on average: the grouped expert GEMMs on the matrix
     cores (32-token tiles per expert; experts with more than 32 tokens take several tiles, experts with few run mostly
-    padding); the last case stays below that average and keeps the integer-dot kernels.  Against the oracle, and a token's row must
+    padding); the sixth case stays below that average and keeps the integer-dot kernels; in the last two the down
+    kernel's workgroups walk four row tiles each (14 row tiles x ~100 expert groups: the last workgroup of a group gets two).
+    Against the oracle, and a token's row must
     not depend on the batch: the same bits with the tokens in reverse order."""
     gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 90 + tokens, down_quant)
     got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x)
