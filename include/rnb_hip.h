@@ -101,7 +101,7 @@ int rnb_hip_quantize_q8(const float *x, size_t n, void *out_blocks, size_t out_b
 int rnb_hip_q4k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
                      size_t x_len, float *out, size_t out_len);
 /* q4k_gemv_batch, quant_api.rs:2283-2319: seq_len = x_len / cols, out[s*rows + row],
- * out_len >= seq_len*rows.  seq_len >= 16 takes the int8-MFMA GEMM. */
+ * out_len >= seq_len*rows.  seq_len >= 4 (matrices of 16 MB and more) or >= 8 takes the int8-MFMA GEMM. */
 int rnb_hip_q4k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                            const float *x, size_t x_len, float *out, size_t out_len);
 /* q4_0_gemv, q4_1_gemv, q5_0_gemv, q5_1_gemv and their batch forms, quant_api.rs:374-496 (checks and texts of
