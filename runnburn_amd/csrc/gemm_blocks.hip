@@ -326,25 +326,62 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Q8_0 {f16 d, i8 qs[32]} (34 bytes) and Q8_1 {f16 d, f16 s, i8 qs[32]} (36 bytes) against 32-wide Q8 activations
-// (one f32 scale per 32 elements).  A step covers 8 blocks = 256 elements, staged exactly like a Q8_K block.
+// The 32-element formats against 32-wide Q8 activations (one f32 scale per 32 elements): Q8_0 {f16 d, i8 qs[32]} (34
+// bytes), Q8_1 {f16 d, f16 s, i8 qs[32]} (36), and the nibble formats Q4_0 {d, 16 bytes} (18; element j < 16 = low nibble
+// of byte j, j + 16 the high one; value d (n - 8)), Q4_1 {d, m, 16 bytes} (20; d n + m), Q5_0 {d, u32 qh, 16 bytes} (22;
+// fifth bit of element j = bit j of qh; d (n - 16)), Q5_1 {d, m, qh, 16 bytes} (24; d n + m).  A step covers 8 blocks
+// = 256 elements, staged exactly like a Q8_K block.  The K-half of a lane is elements 16 khalf .. + 16 of a block: for
+// the nibble formats the low (khalf 0) or high nibbles of the same 16 bytes.
 // ---------------------------------------------------------------------------------------------
-struct Q8Blocks {
-    uint4 q[8];  // the lane's 16 codes (K-half) of each of the 8 blocks
-    float d[8];
+template <uint32_t kFmt>
+struct B32 {
+    static constexpr bool kNibbles = kFmt == kQ4_0 || kFmt == kQ4_1 || kFmt == kQ5_0 || kFmt == kQ5_1;
+    static constexpr bool kFifth = kFmt == kQ5_0 || kFmt == kQ5_1;
+    static constexpr bool kMin = kFmt == kQ4_1 || kFmt == kQ5_1;  // value = d * code + m
+    static constexpr int kBytes = kFmt == kQ8_0 ? 34 : kFmt == kQ8_1 ? 36 : kFmt == kQ4_0 ? 18 : kFmt == kQ4_1 ? 20 : kFmt == kQ5_0 ? 22 : 24;
+    static constexpr int kQhOff = kMin ? 4 : 2;
+    static constexpr int kQsOff = kFmt == kQ8_0 ? 2 : kFmt == kQ8_1 ? 4 : kBytes - 16;
 };
 
-template <int kBlockBytes, int kQsOff>
+struct Q8Blocks {
+    uint4 q[8];       // Q8: the lane's 16 codes (K-half) of each of the 8 blocks; nibble formats: the block's 16 bytes
+    uint32_t qh[8];   // fifth bits (Q5_0, Q5_1)
+    float d[8], m[8];
+};
+
+template <uint32_t kFmt>
 __device__ __forceinline__ Q8Blocks q8_load_blocks(const uint8_t *__restrict__ rowp, uint32_t blk0, uint32_t nb32, int khalf) {
     Q8Blocks r;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const uint32_t b = min(blk0 + k, nb32 - 1);  // a partial last step repeats the last block; its results are dropped
-        const uint8_t *blk = rowp + static_cast<size_t>(b) * kBlockBytes;
-        r.q[k] = ld_u4_a2(blk + kQsOff + 16 * khalf);
+        const uint8_t *blk = rowp + static_cast<size_t>(b) * B32<kFmt>::kBytes;
+        r.q[k] = ld_u4_a2(blk + B32<kFmt>::kQsOff + (B32<kFmt>::kNibbles ? 0 : 16 * khalf));
         r.d[k] = ld_f16(blk);
+        r.qh[k] = 0;
+        r.m[k] = 0.0f;
+        if constexpr (B32<kFmt>::kFifth) r.qh[k] = ld_u32_a2(blk + B32<kFmt>::kQhOff);
+        if constexpr (B32<kFmt>::kMin) r.m[k] = ld_f16(blk + 2);
     }
     return r;
+}
+
+// the lane's 16 codes of a block as signed bytes: Q8 as stored; nibbles split by K-half, fifth bits spread with one
+// multiply per four (bit j of a 4-bit group to bit 8 j), the symmetric formats' offset (8, 16) taken in packed bytes
+template <uint32_t kFmt>
+__device__ __forceinline__ v4i b32_operand(uint4 q, uint32_t qh, int khalf) {
+    uint32_t v[4] = {q.x, q.y, q.z, q.w};
+    if constexpr (B32<kFmt>::kNibbles) {
+        const uint32_t bits = khalf ? qh >> 16 : qh & 0xffffu;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[i] = khalf ? (v[i] >> 4) & 0x0f0f0f0fu : v[i] & 0x0f0f0f0fu;
+            if constexpr (B32<kFmt>::kFifth) v[i] |= ((((bits >> (4 * i)) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+            if constexpr (kFmt == kQ4_0) v[i] = (v[i] + 0x78787878u) ^ 0x80808080u;  // n - 8 per byte, no carries
+            if constexpr (kFmt == kQ5_0) v[i] = (v[i] + 0x70707070u) ^ 0x80808080u;  // n - 16
+        }
+    }
+    return v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
 }
 
 // Route of a wave's 32 rows of one step (8 blocks) to the lanes that own them, by whole cache lines (see RowRoute):
@@ -404,12 +441,14 @@ constexpr size_t q8_lds_bytes(bool routed) {
     return 2 * (32 * kTT) * kGbStride128 + 2 * 8 * (32 * kTT) * sizeof(float) + (routed ? kGbWaves * kQ8StripBytes : 0);
 }
 
-template <int kTT, int kBlockBytes, int kQsOff, bool kRouted>
+template <int kTT, uint32_t kFmt, bool kRouted>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q8_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                         float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq, uint32_t steps_slice) {
     constexpr int kToks = 32 * kTT;
     constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
+    constexpr int kBlockBytes = B32<kFmt>::kBytes, kQsOff = B32<kFmt>::kQsOff;
+    static_assert(!kRouted || !B32<kFmt>::kNibbles, "the strip route is laid out for Q8_0 / Q8_1");
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t(*s_a)[kToks * kGbStride128] = reinterpret_cast<uint8_t(*)[kToks * kGbStride128]>(s_dyn);
     float(*s_dx)[8][kToks] = reinterpret_cast<float(*)[8][kToks]>(s_dyn + 2 * kToks * kGbStride128);  // [block][token]
@@ -475,7 +514,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         q8_route_store(rt, strip, lane);
         cur = q8_blocks_from_strip(strip, lrow, khalf);
     } else {
-        cur = q8_load_blocks<kBlockBytes, kQsOff>(wrow, s0 * 8, nb32, khalf);
+        cur = q8_load_blocks<kFmt>(wrow, s0 * 8, nb32, khalf);
     }
     stage_store8(0);
     __syncthreads();
@@ -487,25 +526,32 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         if constexpr (kRouted)
             q8_route_load(rt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
         else
-            nxt = q8_load_blocks<kBlockBytes, kQsOff>(wrow, sn * 8, nb32, khalf);
+            nxt = q8_load_blocks<kFmt>(wrow, sn * 8, nb32, khalf);
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
         const uint32_t live = min(8u, nb32 - step * 8);  // blocks of this step that exist (workgroup-uniform)
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             if (static_cast<uint32_t>(k) < live) {
-                const v4i bop = {static_cast<int>(cur.q[k].x), static_cast<int>(cur.q[k].y), static_cast<int>(cur.q[k].z),
-                                 static_cast<int>(cur.q[k].w)};
+                const v4i bop = b32_operand<kFmt>(cur.q[k], cur.qh[k], khalf);
 #pragma unroll
                 for (int t = 0; t < kTT; t++) {
                     const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * k);
                     const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);
+                    v16i sum = zero16;  // d n + m formats: the block's sum of activations, from a row of ones
+                    if constexpr (B32<kFmt>::kMin) {
+                        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+                        sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, ones, zero16, 0, 0, 0);
+                    }
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf][k])[8 * t + 2 * j + khalf];
                         const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
-                        for (int i = 0; i < 4; i++)
+                        for (int i = 0; i < 4; i++) {
                             accf[t][4 * j + i] += (cur.d[k] * dx[i]) * static_cast<float>(acc[4 * j + i]);
+                            if constexpr (B32<kFmt>::kMin)
+                                accf[t][4 * j + i] += (cur.m[k] * dx[i]) * static_cast<float>(sum[4 * j + i]);
+                        }
                     }
                 }
             }
@@ -579,6 +625,10 @@ void launch_sum_slices(const float *parts, float *out, size_t n, uint32_t slices
                        slices);
 }
 
+static bool is_b32(uint32_t quant) {
+    return quant == kQ8_0 || quant == kQ8_1 || quant == kQ4_0 || quant == kQ4_1 || quant == kQ5_0 || quant == kQ5_1;
+}
+
 // Q6_K spends the most vector work per tile, and the 64-token form saves the most of it: it also wins where its
 // workgroups fill the 256 compute units just once (4096 rows x 512 tokens x 14336: 164 vs 189 us; with 224 or 320
 // workgroups the 32-token form is level or ahead)
@@ -590,7 +640,7 @@ static bool q6_wide_tiles(uint32_t row_tiles, uint32_t seq) {
 size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps, uint32_t seq) {
     if (rows == 0 || seq == 0 || k_steps == 0) return 0;
     const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
-    const bool wide = (quant == kQ8_0 || quant == kQ8_1) ? seq > 32
+    const bool wide = is_b32(quant) ? seq > 32
                       : quant == kQ6K                    ? q6_wide_tiles(row_tiles, seq)
                                                          : wide_tiles(row_tiles, seq);
     const uint32_t slices = k_slices(tile_grid(rows, seq, wide), k_steps, quant != kQ4K && quant != kQ5K);
@@ -648,7 +698,7 @@ void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, float *sli
     launch_gemm_q45k<false>(w, act, out, slice_out, rows, nb, seq, stream);
 }
 
-bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32) { return (quant == kQ8_0 || quant == kQ8_1) && nb32 >= 1; }
+bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32) { return is_b32(quant) && nb32 >= 1; }
 
 void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
                          uint32_t nb32, uint32_t seq, hipStream_t stream) {
@@ -660,33 +710,37 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     const uint32_t steps_slice = (steps + slices - 1) / slices, nz = (steps + steps_slice - 1) / steps_slice;
     float *dst = nz > 1 ? slice_out : out;
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, nz), block(kGbThreads);
-    const bool routed = nb32 % 8 == 0;  // whole steps only: a partial step's 16-byte pieces would leave the last row
-#define RNB_LAUNCH_Q8R(TT, BYTES, OFF, R)                                                                              \
+    // the strip route: Q8_0 / Q8_1, whole steps only (a partial step's 16-byte pieces would leave the last row)
+    const bool routed = nb32 % 8 == 0 && (quant == kQ8_0 || quant == kQ8_1);
+#define RNB_LAUNCH_Q8R(TT, FMT, R)                                                                                     \
     {                                                                                                                  \
         constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
         static bool configured = false;                                                                                \
         if (!configured) { /* above the default 64 KB of dynamic LDS in the routed 64-token form */                    \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, BYTES, OFF, R>),          \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, FMT, R>),                 \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));              \
             configured = true;                                                                                         \
         }                                                                                                              \
-        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, BYTES, OFF, R>), grid, block, lds, stream, w, act.qs, act.d, dst,  \
-                           rows, nb32, seq, steps_slice);                                                              \
+        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, FMT, R>), grid, block, lds, stream, w, act.qs, act.d, dst, rows,   \
+                           nb32, seq, steps_slice);                                                                    \
     }
-#define RNB_LAUNCH_Q8(TT, BYTES, OFF)                                                                                  \
-    if (routed) RNB_LAUNCH_Q8R(TT, BYTES, OFF, true) else RNB_LAUNCH_Q8R(TT, BYTES, OFF, false)
-    if (quant == kQ8_0) {
-        if (wide) {
-            RNB_LAUNCH_Q8(2, 34, 2);
-        } else {
-            RNB_LAUNCH_Q8(1, 34, 2);
-        }
-    } else {
-        if (wide) {
-            RNB_LAUNCH_Q8(2, 36, 4);
-        } else {
-            RNB_LAUNCH_Q8(1, 36, 4);
-        }
+#define RNB_LAUNCH_Q8(FMT, ROUTABLE)                                                                                   \
+    if constexpr (ROUTABLE) {                                                                                          \
+        if (routed && wide) RNB_LAUNCH_Q8R(2, FMT, true)                                                               \
+        else if (routed) RNB_LAUNCH_Q8R(1, FMT, true)                                                                  \
+        else if (wide) RNB_LAUNCH_Q8R(2, FMT, false)                                                                   \
+        else RNB_LAUNCH_Q8R(1, FMT, false)                                                                             \
+    } else {                                                                                                           \
+        if (wide) RNB_LAUNCH_Q8R(2, FMT, false)                                                                        \
+        else RNB_LAUNCH_Q8R(1, FMT, false)                                                                             \
+    }
+    switch (quant) {
+    case kQ8_0: RNB_LAUNCH_Q8(kQ8_0, true) break;
+    case kQ8_1: RNB_LAUNCH_Q8(kQ8_1, true) break;
+    case kQ4_0: RNB_LAUNCH_Q8(kQ4_0, false) break;
+    case kQ4_1: RNB_LAUNCH_Q8(kQ4_1, false) break;
+    case kQ5_0: RNB_LAUNCH_Q8(kQ5_0, false) break;
+    default: RNB_LAUNCH_Q8(kQ5_1, false) break;
     }
 #undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8

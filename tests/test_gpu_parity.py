@@ -471,7 +471,7 @@ def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
     assert np.array_equal(rev[::-1], got)
 
 
-@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1])
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1])
 @pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 16), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
 def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
     """Grids too small for the chip are cut along K (blockIdx.z) and the slices' outputs added by a second kernel in
@@ -487,12 +487,14 @@ def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
     assert np.array_equal(rev[::-1], got)
 
 
-@pytest.mark.parametrize("quant", [Q8_0, Q8_1])
+@pytest.mark.parametrize("quant", [Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1])
 @pytest.mark.parametrize("rows,cols,seq", [(32, 32, 16), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
                                            (1, 4096, 16), (300, 288, 100)])
 def test_q8_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, cols, seq):
-    """16 or more tokens on Q8_0 / Q8_1 take the matrix-core GEMM (one K=32 instruction per block, the two f32 scales on
-    the vector units): block counts off the 8-block step, rows and tokens off the tile."""
+    """Batches on the 32-element formats take the matrix-core GEMM (one K=32 instruction per block, the two f32 scales
+    on the vector units; the nibble formats' codes are split, given their fifth bit and offset in packed bytes, the
+    d n + m formats add m times the block's sum of activations from a second instruction against ones): block counts off
+    the 8-block step, rows and tokens off the tile."""
     w = oracle.make_weights(quant, rows, cols, 270 + rows)
     x = oracle.fill_normal(seq * cols, 280 + seq, 1.0)
     got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
