@@ -164,7 +164,10 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         else
             launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);
     } else if (quant == kQ2K || quant == kQ3K) {
-        if (seq >= kTokensMinSeq)
+        if (seq >= min_gemm_seq) {
+            if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
+            launch_gemm_q23k_mfma(w_dev, quant, act, out_dev, ws, r, nb, q, s.stream);
+        } else if (seq >= kTokensMinSeq)
             launch_matmul_tokens(w_dev, quant, act, out_dev, r, nb, q, s.stream);
         else
             launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);

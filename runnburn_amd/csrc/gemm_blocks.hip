@@ -1,6 +1,7 @@
 // Prefill GEMM for the formats whose scales do not fold onto an int8 operand: Q6_K (int8 scale per 16 elements), Q5_K
-// (6-bit scale per 32 five-bit codes: scale times code needs 11 bits) and the 32-element byte formats Q8_0 / Q8_1 (f16
-// scale per 32 elements).  out[seq][rows], same contract as the GEMVs.
+// (6-bit scale per 32 five-bit codes: scale times code needs 11 bits), Q2_K / Q3_K (sixteen sub-blocks like Q6_K) and
+// the 32-element formats Q8_0 / Q8_1 / Q4_0 / Q4_1 / Q5_0 / Q5_1 (f16 scale per 32 elements).  out[seq][rows], same
+// contract as the GEMVs.  Small grids are cut along K into slices whose outputs a second kernel adds in slice order.
 //
 // The matrix cores do the integer part of one scale group per instruction and the vector units apply the group's scale
 // to the 16 results a lane holds:
@@ -11,6 +12,10 @@
 //          the quantiser's digits, out += d_x * (d * float(tot) - dmin * float(S)) per super-block.
 //   Q8_0   v_mfma_i32_32x32x32_i8 per 32-element block: out += (d[r][b] * d_x[s][b]) * float(I_b),
 //   Q8_1   crates/rnb-cpu/src/gemm/neon_dot.rs:376-436, neon_quant.rs:236-253.
+//   Q4_0 Q4_1 Q5_0 Q5_1   the same with the block's nibbles (and fifth bits) made into signed bytes when consumed; the
+//          d n + m formats add (m * d_x) * sum(a) from a second instruction against a row of ones.
+//   Q2_K Q3_K   Q6_K's scheme; Q2_K's mins term through two K=16 instructions over the sub-block sums' digits:
+//          crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242 (Q2_K), :247-375 (Q3_K).
 // That is 16 (Q6_K) or 48 (Q8) vector instructions per matrix instruction, so these kernels are bound by the vector
 // port, not the matrix pipe; they replace one GEMV pass per token (Q8) or the integer-dot multi-token kernel (Q5_K,
 // Q6_K), which measured 9 to 17 times slower at 512 tokens.
@@ -141,6 +146,224 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         route_store(rt, strip, lane);
         q6_row_from_strip(cur, strip + lrow * kQ6StripStride, khalf);
         cur.d = d_next;
+        __syncthreads();
+    }
+
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
+                if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q2_K {u8 scales[16] (scale | min << 4), u8 qs[64], f16 d, f16 dmin} (84 bytes) and Q3_K {u8 hmask[32], u8 qs[64],
+// u8 scales[12], f16 d} (110 bytes): sixteen 16-element sub-blocks like Q6_K, so the same scheme: one K=16 matrix
+// instruction per sub-block and the sub-block's scale on its 16 results.  Byte 32n + l of qs holds elements
+// 128n + 32j + l in bit pair j; sub-block 8n + 2j + l/16 is elements 16 sb .. + 16, of which the lane of K-half k takes
+// l%16 = 8k .. + 8.  Q3_K: code | hbit << 2 (bit 4n + j of hmask[l]) minus 4 in packed bytes, scale = 6-bit code - 32.
+// Q2_K: unsigned codes, 4-bit scales; its mins term sum_sb mn_sb * bsum16_sb is itself a K=16 contraction over the
+// sub-blocks: the activations' 16-element sums are staged as two int8 digits (bsum = lo + 64 hi, lo = bsum & 63) and
+// two more matrix instructions per block and token tile deliver it in the result layout.
+// ---------------------------------------------------------------------------------------------
+struct Q23Row {
+    uint2 qs[2][2];  // [n][l / 16]: the lane's 8 bytes
+    uint2 hm[2];     // [l / 16] (Q3_K)
+    uint4 sc;        // Q2_K: scales[16]; Q3_K: scales[12] in x, y, z
+    float d, dmin;
+};
+
+template <bool kThree>
+__device__ __forceinline__ Q23Row q23_load_row(const uint8_t *__restrict__ blk, int khalf) {
+    Q23Row r;
+    constexpr int kQsOff = kThree ? 32 : 16;
+#pragma unroll
+    for (int n = 0; n < 2; n++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) r.qs[n][h] = ld_u2_a2(blk + kQsOff + 32 * n + 16 * h + 8 * khalf);
+    if constexpr (kThree) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) r.hm[h] = ld_u2_a2(blk + 16 * h + 8 * khalf);
+        const uint2 s01 = ld_u2_a2(blk + 96);
+        r.sc = make_uint4(s01.x, s01.y, ld_u32_a2(blk + 104), 0);
+        r.d = ld_f16(blk + 108);
+        r.dmin = 0.0f;
+    } else {
+        r.hm[0] = r.hm[1] = make_uint2(0, 0);
+        r.sc = ld_u4_a2(blk);
+        const uint32_t dd = ld_u32_a2(blk + 80);
+        r.d = f16_bits_to_f32(dd);
+        r.dmin = f16_bits_to_f32(dd >> 16);
+    }
+    return r;
+}
+
+template <int kSb, bool kThree>
+__device__ __forceinline__ long q23_operand(const Q23Row &r) {
+    constexpr int g = kSb >> 1, n = g >> 2, j = g & 3, h = kSb & 1;
+    uint32_t v0 = (r.qs[n][h].x >> (2 * j)) & 0x03030303u, v1 = (r.qs[n][h].y >> (2 * j)) & 0x03030303u;
+    if constexpr (kThree) {
+        v0 |= ((r.hm[h].x >> g) & 0x01010101u) << 2;
+        v1 |= ((r.hm[h].y >> g) & 0x01010101u) << 2;
+        v0 = (v0 + 0x7c7c7c7cu) ^ 0x80808080u;  // v - 4 per byte: v + 0x7c never carries, flipping bit 7 finishes it
+        v1 = (v1 + 0x7c7c7c7cu) ^ 0x80808080u;
+    }
+    return static_cast<long>(static_cast<unsigned long>(v0) | (static_cast<unsigned long>(v1) << 32));
+}
+
+template <int kSb, bool kThree>
+__device__ __forceinline__ int q23_scale(const Q23Row &r) {
+    const uint32_t w[4] = {r.sc.x, r.sc.y, r.sc.z, r.sc.w};
+    if constexpr (kThree) {
+        // code k: low nibble = nibble k / 8 of byte k % 8, high two bits = bit pair k / 4 of byte 8 + k % 4
+        const uint32_t lo = (w[(kSb & 7) >> 2] >> (8 * (kSb & 3) + 4 * (kSb >> 3))) & 15u;
+        const uint32_t hi = (w[2] >> (8 * (kSb & 3) + 2 * (kSb >> 2))) & 3u;
+        return static_cast<int>(lo | (hi << 4)) - 32;
+    } else {
+        return static_cast<int>((w[kSb >> 2] >> (8 * (kSb & 3))) & 15u);
+    }
+}
+
+template <int kTT, bool kThree>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    gemm_q23k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                          const int16_t *__restrict__ abs16, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                          uint32_t seq, uint32_t nb_slice) {
+    constexpr int kToks = 32 * kTT;
+    constexpr int kBlockBytes = kThree ? kQ3KBytes : kQ2KBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride64];
+    __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
+    __shared__ __attribute__((aligned(16))) uint4 s_bd[2][kToks][2];  // Q2_K: digits lo, hi of the 16 sub-block sums
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kBlockBytes;
+
+    float accf[kTT][16];
+    int tot[kTT][16];
+#pragma unroll
+    for (int t = 0; t < kTT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            accf[t][i] = 0.0f;
+            tot[t][i] = 0;
+        }
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    Stage<kToks> st;
+    uint4 bd_lo = make_uint4(0, 0, 0, 0), bd_hi = make_uint4(0, 0, 0, 0);
+    auto stage_load2 = [&](uint32_t b) {
+        stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, b, tid);
+        if constexpr (!kThree) {
+            if (tid < kToks) {
+                const int16_t *bs = abs16 + (static_cast<size_t>(min(tok0 + tid, last_tok)) * nb + b) * 16;
+                const uint4 s0 = *reinterpret_cast<const uint4 *>(bs), s1 = *reinterpret_cast<const uint4 *>(bs + 8);
+                const uint32_t pr[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};  // two sums per dword
+                uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int v = static_cast<int16_t>(pr[i >> 1] >> (16 * (i & 1)));
+                    lo[i >> 2] |= static_cast<uint32_t>(v & 63) << (8 * (i & 3));
+                    hi[i >> 2] |= (static_cast<uint32_t>(v >> 6) & 0xffu) << (8 * (i & 3));  // |sum| <= 2048: -32 .. 31
+                }
+                bd_lo = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                bd_hi = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            }
+        }
+    };
+    auto stage_store2 = [&](int buf) {
+        stage_store<kToks>(st, s_a[buf], s_dx[buf], tid);
+        if constexpr (!kThree) {
+            if (tid < kToks) {
+                s_bd[buf][tid][0] = bd_lo;
+                s_bd[buf][tid][1] = bd_hi;
+            }
+        }
+    };
+
+    // K slice of this workgroup (blockIdx.z): blocks b0 .. b1, its sums go to the slice's own copy of the output
+    const uint32_t b0 = blockIdx.z * nb_slice, b1 = min(nb, b0 + nb_slice);
+    out += static_cast<size_t>(blockIdx.z) * seq * rows;
+    stage_load2(b0);
+    Q23Row cur = q23_load_row<kThree>(wrow + static_cast<size_t>(b0) * kBlockBytes, khalf);
+    stage_store2(0);
+    __syncthreads();
+
+    for (uint32_t b = b0; b < b1; b++) {
+        const int buf = (b - b0) & 1;
+        const uint32_t bn = b + 1 < b1 ? b + 1 : b;  // the last step reloads its own block, unused
+        stage_load2(bn);
+        const Q23Row nxt = q23_load_row<kThree>(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+        const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
+
+        // as in the Q6_K kernel: the empty asm and the scheduling barrier keep the sixteen sub-blocks a chain
+#define RNB_Q23_SUB_BLOCK(SB)                                                                                          \
+    {                                                                                                                  \
+        const long bop = q23_operand<SB, kThree>(cur);                                                                 \
+        const int sc = q23_scale<SB, kThree>(cur);                                                                     \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
+            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
+            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 4 * 127 */                                           \
+                asm volatile("" : "+v"(tot[t][i]));                                                                    \
+            }                                                                                                          \
+        }                                                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                                             \
+    }
+        RNB_Q23_SUB_BLOCK(0)
+        RNB_Q23_SUB_BLOCK(1)
+        RNB_Q23_SUB_BLOCK(2)
+        RNB_Q23_SUB_BLOCK(3)
+        RNB_Q23_SUB_BLOCK(4)
+        RNB_Q23_SUB_BLOCK(5)
+        RNB_Q23_SUB_BLOCK(6)
+        RNB_Q23_SUB_BLOCK(7)
+        RNB_Q23_SUB_BLOCK(8)
+        RNB_Q23_SUB_BLOCK(9)
+        RNB_Q23_SUB_BLOCK(10)
+        RNB_Q23_SUB_BLOCK(11)
+        RNB_Q23_SUB_BLOCK(12)
+        RNB_Q23_SUB_BLOCK(13)
+        RNB_Q23_SUB_BLOCK(14)
+        RNB_Q23_SUB_BLOCK(15)
+#undef RNB_Q23_SUB_BLOCK
+
+        // Q2_K mins: K slot i of the lane's K-half is sub-block 8 khalf + i on both sides
+        const uint32_t mn0 = ((khalf ? cur.sc.z : cur.sc.x) >> 4) & 0x0f0f0f0fu, mn1 = ((khalf ? cur.sc.w : cur.sc.y) >> 4) & 0x0f0f0f0fu;
+        const long mnop = static_cast<long>(static_cast<unsigned long>(mn0) | (static_cast<unsigned long>(mn1) << 32));
+#pragma unroll
+        for (int t = 0; t < kTT; t++) {
+            v16i mins = zero16;
+            if constexpr (!kThree) {
+                const uint8_t *dg = reinterpret_cast<const uint8_t *>(&s_bd[buf][32 * t + lrow][0]) + 8 * khalf;
+                const long lo = *reinterpret_cast<const long *>(dg), hi = *reinterpret_cast<const long *>(dg + 16);
+                const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(lo, mnop, zero16, 0, 0, 0);
+                const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(hi, mnop, zero16, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; i++) mins[i] = c0[i] + 64 * c1[i];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
+                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = 4 * j + i;
+                    accf[t][r] += (cur.d * dx[i]) * static_cast<float>(tot[t][r]);
+                    if constexpr (!kThree) accf[t][r] -= (cur.dmin * dx[i]) * static_cast<float>(mins[r]);
+                    tot[t][r] = 0;
+                }
+            }
+        }
+        stage_store2(buf ^ 1);
+        cur = nxt;
         __syncthreads();
     }
 
@@ -643,7 +866,7 @@ size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps,
     const bool wide = is_b32(quant) ? seq > 32
                       : quant == kQ6K                    ? q6_wide_tiles(row_tiles, seq)
                                                          : wide_tiles(row_tiles, seq);
-    const uint32_t slices = k_slices(tile_grid(rows, seq, wide), k_steps, quant != kQ4K && quant != kQ5K);
+    const uint32_t slices = k_slices(tile_grid(rows, seq, wide), k_steps, quant != kQ4K && quant != kQ5K);  // as the launchers
     return slices > 1 ? static_cast<size_t>(slices) * seq * rows : 0;
 }
 
@@ -664,6 +887,33 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slic
         hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
                            nb_slice);
     }
+    if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
+}
+
+void launch_gemm_q23k_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
+                           uint32_t nb, uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb == 0) return;
+    const uint32_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    const bool wide = wide_tiles(row_tiles, seq);
+    const uint32_t slices = slice_out ? k_slices(tile_grid(rows, seq, wide), nb, true) : 1;
+    const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
+    float *dst = nz > 1 ? slice_out : out;
+    const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : (seq + 31) / 32, nz), block(kGbThreads);
+#define RNB_LAUNCH_Q23(TT, THREE)                                                                                      \
+    hipLaunchKernelGGL((gemm_q23k_mfma_kernel<TT, THREE>), grid, block, 0, stream, w, act.qs, act.d, act.bsums, dst, rows, nb, \
+                       seq, nb_slice)
+    if (quant == kQ3K) {
+        if (wide)
+            RNB_LAUNCH_Q23(2, true);
+        else
+            RNB_LAUNCH_Q23(1, true);
+    } else {
+        if (wide)
+            RNB_LAUNCH_Q23(2, false);
+        else
+            RNB_LAUNCH_Q23(1, false);
+    }
+#undef RNB_LAUNCH_Q23
     if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
 

@@ -100,6 +100,9 @@ void launch_gemm_q5k_mfma(const uint8_t *w, ActView act, float *out, float *slic
 // workgroups to fill the chip
 void launch_gemm_q4k_small(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
                            uint32_t seq, hipStream_t stream);
+// Q2_K / Q3_K (needs act.bsums, which the Q8_K quantiser always writes)
+void launch_gemm_q23k_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
+                           uint32_t nb, uint32_t seq, hipStream_t stream);
 bool gemm_q8_mfma_supported(uint32_t quant, uint32_t nb32);
 void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows,
                          uint32_t nb32, uint32_t seq, hipStream_t stream);

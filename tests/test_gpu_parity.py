@@ -471,7 +471,7 @@ def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
     assert np.array_equal(rev[::-1], got)
 
 
-@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1])
+@pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
 @pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 16), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
 def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
     """Grids too small for the chip are cut along K (blockIdx.z) and the slices' outputs added by a second kernel in
@@ -484,6 +484,23 @@ def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
     check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
                 f"k slices quant {quant} rows {rows} nblk {nblk} seq {seq}")
     rev = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
+    assert np.array_equal(rev[::-1], got)
+
+
+@pytest.mark.parametrize("quant", [Q2_K, Q3_K])
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (1, 1, 8),
+                                           (257, 5, 40), (129, 1, 65), (640, 3, 600)])
+def test_q2k_q3k_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, nblk, seq):
+    """Batches on Q2_K / Q3_K take the matrix-core GEMM (one K=16 instruction per 16-element sub-block, its scale on the
+    vector units; Q2_K's mins through the activations' 16-element sums as two int8 digits): rows and tokens off the
+    128 x 32 / 64 tile, one token tile and several, the last shape with 64-token workgroups."""
+    cols = nblk * 256
+    w = oracle.make_weights(quant, rows, cols, 370 + rows)
+    x = oracle.fill_normal(seq * cols, 380 + seq, 1.0)
+    got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"q2k/q3k gemm quant {quant} rows {rows} nblk {nblk} seq {seq}")
+    rev = gemv_fn(rnb, quant, True)(w, rows, cols, x.reshape(seq, cols)[::-1].copy())
     assert np.array_equal(rev[::-1], got)
 
 
