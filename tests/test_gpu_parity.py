@@ -866,3 +866,48 @@ def test_q6k_gemv_argmax_matches_gemv_and_tie_rule(rnb, oracle):
     assert idx2 == min(idx, idx + 1 if idx + 1 < rows - 5 else 0) and val2 == val
     one, v1 = rnb.q6k_gemv_argmax(w[:cols // 256 * 210], 1, cols, x)
     assert one == 0 and v1 == full[0]
+
+
+# ---- HIP graph replay of the device-resident entry points --------------------------------------
+
+@pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 512, 1024, 1), (Q6_K, 256, 2048, 24), (Q8_0, 300, 1024, 40),
+                                                 (Q4_K, 2304, 2048, 260)])
+def test_graph_replay_matches_eager(rnb, quant, rows, cols, seq):
+    """The `_dev` entry points only enqueue on the library's stream, so a caller may capture them (after one eager call
+    of the shape, which sizes the grow-only scratch): a decode GEMV in one launch, GEMMs cut into K slices plus their
+    summing kernel, and the ping-pong GEMM with two slices.  Three replays with the input changed between them by eager
+    uploads and synchronisations, each compared bit for bit with the eager result on the same input."""
+    import ctypes as C
+    import bench
+    hip = bench.Hip()
+    lib = rnb.lib()
+    stream = C.c_void_p(rnb.stream_handle())
+    rng = np.random.default_rng(4000 + rows)
+    w = rnb.DeviceBuffer.from_host(bench.synth_weights(quant, rows, cols, 4100 + seq))
+    xs = [rng.standard_normal(seq * cols).astype(np.float32) for _ in range(3)]
+    x_dev = rnb.DeviceBuffer.from_host(xs[0])
+    out_dev = rnb.DeviceBuffer(seq * rows * 4)
+    eager = []
+    for x in xs:
+        assert lib.rnb_hip_dev_upload(x_dev.ptr, x.ctypes.data_as(C.c_void_p), x.nbytes) == 0
+        rnb.gemv_dev(quant, w, rows, cols, x_dev, seq, out_dev)
+        eager.append(out_dev.to_host(np.float32))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.check(hip.rt.hipStreamBeginCapture(stream, 2), "hipStreamBeginCapture")
+    try:
+        rnb.gemv_dev(quant, w, rows, cols, x_dev, seq, out_dev)
+    finally:
+        rc = hip.rt.hipStreamEndCapture(stream, C.byref(graph))
+    hip.check(rc, "hipStreamEndCapture")
+    hip.check(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0), "hipGraphInstantiate")
+    try:
+        for x, want in zip(xs, eager):
+            assert lib.rnb_hip_dev_upload(x_dev.ptr, x.ctypes.data_as(C.c_void_p), x.nbytes) == 0
+            hip.check(hip.rt.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            rnb.sync()
+            assert np.array_equal(out_dev.to_host(np.float32), want)
+    finally:
+        hip.rt.hipGraphExecDestroy(gexec)
+        hip.rt.hipGraphDestroy(graph)
+        for b in (w, x_dev, out_dev):
+            b.free()
