@@ -659,6 +659,63 @@ __device__ __forceinline__ Q8Blocks q8_blocks_from_strip(const uint8_t *strip, i
     return r;
 }
 
+// The same route for Q4_0 / Q4_1, whose block has one 16-byte piece (the nibbles; both K-halves read it) and two or
+// four header bytes: lane takes block lane % 8 of rows lane / 8 + 8 i.  In the strip a row is its eight pieces (144
+// bytes apart: conflict-free 128-bit reads) and, after the 32 rows, eight dwords of d | m << 16.  The strip is no
+// larger than the Q8 one, so both share the LDS layout.
+struct N4Route {
+    uint32_t off[4];  // byte offset of the lane's block from the wave's first row (rows past the end: the last row)
+    uint4 q[4];
+    uint32_t dm[4];
+};
+constexpr int kN4RowStride = 144;
+static_assert(32 * kN4RowStride + 32 * 32 <= kQ8StripBytes, "the nibble strip fits the Q8 strip");
+
+template <uint32_t kFmt>
+__device__ __forceinline__ void n4_route_setup(N4Route &rt, uint32_t rows_left, size_t row_bytes, int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        rt.off[i] = static_cast<uint32_t>(min(static_cast<uint32_t>(lane >> 3) + 8 * i, rows_left - 1) * row_bytes) +
+                    (lane & 7) * B32<kFmt>::kBytes;
+}
+
+template <uint32_t kFmt>
+__device__ __forceinline__ void n4_route_load(N4Route &rt, const uint8_t *__restrict__ base) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        rt.q[i] = ld_u4_a2(base + rt.off[i] + B32<kFmt>::kQsOff);
+        if constexpr (B32<kFmt>::kMin)
+            rt.dm[i] = ld_u32_a2(base + rt.off[i]);
+        else
+            rt.dm[i] = *reinterpret_cast<const uint16_t *>(base + rt.off[i]);
+    }
+}
+
+__device__ __forceinline__ void n4_route_store(const N4Route &rt, uint8_t *strip, int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (lane >> 3) + 8 * i;
+        *reinterpret_cast<uint4 *>(strip + r * kN4RowStride + 16 * (lane & 7)) = rt.q[i];
+        *reinterpret_cast<uint32_t *>(strip + 32 * kN4RowStride + r * 32 + 4 * (lane & 7)) = rt.dm[i];
+    }
+}
+
+__device__ __forceinline__ Q8Blocks n4_blocks_from_strip(const uint8_t *strip, int lrow) {
+    Q8Blocks r;
+#pragma unroll
+    for (int k = 0; k < 8; k++) r.q[k] = *reinterpret_cast<const uint4 *>(strip + lrow * kN4RowStride + 16 * k);
+    const uint4 h0 = *reinterpret_cast<const uint4 *>(strip + 32 * kN4RowStride + lrow * 32);
+    const uint4 h1 = *reinterpret_cast<const uint4 *>(strip + 32 * kN4RowStride + lrow * 32 + 16);
+    const uint32_t dm[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        r.d[k] = f16_bits_to_f32(dm[k]);
+        r.m[k] = f16_bits_to_f32(dm[k] >> 16);
+        r.qh[k] = 0;
+    }
+    return r;
+}
+
 template <int kTT>
 constexpr size_t q8_lds_bytes(bool routed) {
     return 2 * (32 * kTT) * kGbStride128 + 2 * 8 * (32 * kTT) * sizeof(float) + (routed ? kGbWaves * kQ8StripBytes : 0);
@@ -671,7 +728,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     constexpr int kToks = 32 * kTT;
     constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
     constexpr int kBlockBytes = B32<kFmt>::kBytes, kQsOff = B32<kFmt>::kQsOff;
-    static_assert(!kRouted || !B32<kFmt>::kNibbles, "the strip route is laid out for Q8_0 / Q8_1");
+    static_assert(!kRouted || !B32<kFmt>::kFifth, "the strip routes are laid out for Q8_0 / Q8_1 and Q4_0 / Q4_1");
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t(*s_a)[kToks * kGbStride128] = reinterpret_cast<uint8_t(*)[kToks * kGbStride128]>(s_dyn);
     float(*s_dx)[8][kToks] = reinterpret_cast<float(*)[8][kToks]>(s_dyn + 2 * kToks * kGbStride128);  // [block][token]
@@ -729,13 +786,21 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const uint8_t *wbase = w + static_cast<size_t>(wrow0) * nb32 * kBlockBytes;
     uint8_t *strip = s_dyn + q8_lds_bytes<kTT>(false) + wave * kQ8StripBytes;
     Q8Route rt;
+    N4Route nrt;
     Q8Blocks cur, nxt;
     stage_load8(s0);
     if constexpr (kRouted) {
-        q8_route_setup<kBlockBytes, kQsOff>(rt, rows - wrow0, static_cast<size_t>(nb32) * kBlockBytes, lane);
-        q8_route_load(rt, wbase + static_cast<size_t>(s0) * 8 * kBlockBytes);
-        q8_route_store(rt, strip, lane);
-        cur = q8_blocks_from_strip(strip, lrow, khalf);
+        if constexpr (B32<kFmt>::kNibbles) {
+            n4_route_setup<kFmt>(nrt, rows - wrow0, static_cast<size_t>(nb32) * kBlockBytes, lane);
+            n4_route_load<kFmt>(nrt, wbase + static_cast<size_t>(s0) * 8 * kBlockBytes);
+            n4_route_store(nrt, strip, lane);
+            cur = n4_blocks_from_strip(strip, lrow);
+        } else {
+            q8_route_setup<kBlockBytes, kQsOff>(rt, rows - wrow0, static_cast<size_t>(nb32) * kBlockBytes, lane);
+            q8_route_load(rt, wbase + static_cast<size_t>(s0) * 8 * kBlockBytes);
+            q8_route_store(rt, strip, lane);
+            cur = q8_blocks_from_strip(strip, lrow, khalf);
+        }
     } else {
         cur = q8_load_blocks<kFmt>(wrow, s0 * 8, nb32, khalf);
     }
@@ -747,7 +812,10 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const uint32_t sn = step + 1 < s1 ? step + 1 : step;
         stage_load8(sn);
         if constexpr (kRouted)
-            q8_route_load(rt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
+            if constexpr (B32<kFmt>::kNibbles)
+                n4_route_load<kFmt>(nrt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
+            else
+                q8_route_load(rt, wbase + static_cast<size_t>(sn) * 8 * kBlockBytes);
         else
             nxt = q8_load_blocks<kFmt>(wrow, sn * 8, nb32, khalf);
         const uint8_t *abase = s_a[buf] + lrow * kGbStride128 + 16 * khalf;
@@ -781,8 +849,13 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }
         stage_store8(buf ^ 1);
         if constexpr (kRouted) {
-            q8_route_store(rt, strip, lane);
-            cur = q8_blocks_from_strip(strip, lrow, khalf);
+            if constexpr (B32<kFmt>::kNibbles) {
+                n4_route_store(nrt, strip, lane);
+                cur = n4_blocks_from_strip(strip, lrow);
+            } else {
+                q8_route_store(rt, strip, lane);
+                cur = q8_blocks_from_strip(strip, lrow, khalf);
+            }
         } else {
             cur = nxt;
         }
@@ -960,8 +1033,8 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     const uint32_t steps_slice = (steps + slices - 1) / slices, nz = (steps + steps_slice - 1) / steps_slice;
     float *dst = nz > 1 ? slice_out : out;
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, nz), block(kGbThreads);
-    // the strip route: Q8_0 / Q8_1, whole steps only (a partial step's 16-byte pieces would leave the last row)
-    const bool routed = nb32 % 8 == 0 && (quant == kQ8_0 || quant == kQ8_1);
+    // the strip routes: Q8_0 / Q8_1 and Q4_0 / Q4_1, whole steps only (a partial step's pieces would leave the last row)
+    const bool routed = nb32 % 8 == 0 && quant != kQ5_0 && quant != kQ5_1;
 #define RNB_LAUNCH_Q8R(TT, FMT, R)                                                                                     \
     {                                                                                                                  \
         constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
@@ -987,8 +1060,8 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     switch (quant) {
     case kQ8_0: RNB_LAUNCH_Q8(kQ8_0, true) break;
     case kQ8_1: RNB_LAUNCH_Q8(kQ8_1, true) break;
-    case kQ4_0: RNB_LAUNCH_Q8(kQ4_0, false) break;
-    case kQ4_1: RNB_LAUNCH_Q8(kQ4_1, false) break;
+    case kQ4_0: RNB_LAUNCH_Q8(kQ4_0, true) break;
+    case kQ4_1: RNB_LAUNCH_Q8(kQ4_1, true) break;
     case kQ5_0: RNB_LAUNCH_Q8(kQ5_0, false) break;
     default: RNB_LAUNCH_Q8(kQ5_1, false) break;
     }
