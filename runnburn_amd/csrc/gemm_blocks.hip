@@ -659,17 +659,17 @@ __device__ __forceinline__ Q8Blocks q8_blocks_from_strip(const uint8_t *strip, i
     return r;
 }
 
-// The same route for Q4_0 / Q4_1, whose block has one 16-byte piece (the nibbles; both K-halves read it) and two or
-// four header bytes: lane takes block lane % 8 of rows lane / 8 + 8 i.  In the strip a row is its eight pieces (144
-// bytes apart: conflict-free 128-bit reads) and, after the 32 rows, eight dwords of d | m << 16.  The strip is no
+// The same route for the nibble formats, whose block has one 16-byte piece (the nibbles; both K-halves read it) and a
+// header of two to eight bytes: lane takes block lane % 8 of rows lane / 8 + 8 i.  In the strip a row is its eight pieces
+// (144 bytes apart: conflict-free 128-bit reads) and, after the 32 rows, eight pairs {d | m << 16, qh} per row.  The strip is no
 // larger than the Q8 one, so both share the LDS layout.
 struct N4Route {
     uint32_t off[4];  // byte offset of the lane's block from the wave's first row (rows past the end: the last row)
     uint4 q[4];
-    uint32_t dm[4];
+    uint32_t dm[4], qh[4];
 };
 constexpr int kN4RowStride = 144;
-static_assert(32 * kN4RowStride + 32 * 32 <= kQ8StripBytes, "the nibble strip fits the Q8 strip");
+static_assert(32 * kN4RowStride + 32 * 64 <= kQ8StripBytes, "the nibble strip fits the Q8 strip");
 
 template <uint32_t kFmt>
 __device__ __forceinline__ void n4_route_setup(N4Route &rt, uint32_t rows_left, size_t row_bytes, int lane) {
@@ -688,6 +688,8 @@ __device__ __forceinline__ void n4_route_load(N4Route &rt, const uint8_t *__rest
             rt.dm[i] = ld_u32_a2(base + rt.off[i]);
         else
             rt.dm[i] = *reinterpret_cast<const uint16_t *>(base + rt.off[i]);
+        rt.qh[i] = 0;
+        if constexpr (B32<kFmt>::kFifth) rt.qh[i] = ld_u32_a2(base + rt.off[i] + B32<kFmt>::kQhOff);
     }
 }
 
@@ -696,7 +698,7 @@ __device__ __forceinline__ void n4_route_store(const N4Route &rt, uint8_t *strip
     for (int i = 0; i < 4; i++) {
         const int r = (lane >> 3) + 8 * i;
         *reinterpret_cast<uint4 *>(strip + r * kN4RowStride + 16 * (lane & 7)) = rt.q[i];
-        *reinterpret_cast<uint32_t *>(strip + 32 * kN4RowStride + r * 32 + 4 * (lane & 7)) = rt.dm[i];
+        *reinterpret_cast<uint2 *>(strip + 32 * kN4RowStride + r * 64 + 8 * (lane & 7)) = make_uint2(rt.dm[i], rt.qh[i]);
     }
 }
 
@@ -704,14 +706,15 @@ __device__ __forceinline__ Q8Blocks n4_blocks_from_strip(const uint8_t *strip, i
     Q8Blocks r;
 #pragma unroll
     for (int k = 0; k < 8; k++) r.q[k] = *reinterpret_cast<const uint4 *>(strip + lrow * kN4RowStride + 16 * k);
-    const uint4 h0 = *reinterpret_cast<const uint4 *>(strip + 32 * kN4RowStride + lrow * 32);
-    const uint4 h1 = *reinterpret_cast<const uint4 *>(strip + 32 * kN4RowStride + lrow * 32 + 16);
-    const uint32_t dm[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
 #pragma unroll
-    for (int k = 0; k < 8; k++) {
-        r.d[k] = f16_bits_to_f32(dm[k]);
-        r.m[k] = f16_bits_to_f32(dm[k] >> 16);
-        r.qh[k] = 0;
+    for (int p = 0; p < 4; p++) {  // two blocks' {d | m << 16, qh} per 128-bit read
+        const uint4 h = *reinterpret_cast<const uint4 *>(strip + 32 * kN4RowStride + lrow * 64 + 16 * p);
+        r.d[2 * p] = f16_bits_to_f32(h.x);
+        r.m[2 * p] = f16_bits_to_f32(h.x >> 16);
+        r.qh[2 * p] = h.y;
+        r.d[2 * p + 1] = f16_bits_to_f32(h.z);
+        r.m[2 * p + 1] = f16_bits_to_f32(h.z >> 16);
+        r.qh[2 * p + 1] = h.w;
     }
     return r;
 }
@@ -728,7 +731,6 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     constexpr int kToks = 32 * kTT;
     constexpr int kDxPerThread = kToks * 8 / kGbThreads;  // 1 (32 tokens) or 2 (64 tokens)
     constexpr int kBlockBytes = B32<kFmt>::kBytes, kQsOff = B32<kFmt>::kQsOff;
-    static_assert(!kRouted || !B32<kFmt>::kFifth, "the strip routes are laid out for Q8_0 / Q8_1 and Q4_0 / Q4_1");
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t(*s_a)[kToks * kGbStride128] = reinterpret_cast<uint8_t(*)[kToks * kGbStride128]>(s_dyn);
     float(*s_dx)[8][kToks] = reinterpret_cast<float(*)[8][kToks]>(s_dyn + 2 * kToks * kGbStride128);  // [block][token]
@@ -1033,8 +1035,8 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     const uint32_t steps_slice = (steps + slices - 1) / slices, nz = (steps + steps_slice - 1) / steps_slice;
     float *dst = nz > 1 ? slice_out : out;
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, nz), block(kGbThreads);
-    // the strip routes: Q8_0 / Q8_1 and Q4_0 / Q4_1, whole steps only (a partial step's pieces would leave the last row)
-    const bool routed = nb32 % 8 == 0 && quant != kQ5_0 && quant != kQ5_1;
+    // the strip routes: whole steps only (a partial step's pieces would leave the last row)
+    const bool routed = nb32 % 8 == 0;
 #define RNB_LAUNCH_Q8R(TT, FMT, R)                                                                                     \
     {                                                                                                                  \
         constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
@@ -1062,8 +1064,8 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     case kQ8_1: RNB_LAUNCH_Q8(kQ8_1, true) break;
     case kQ4_0: RNB_LAUNCH_Q8(kQ4_0, true) break;
     case kQ4_1: RNB_LAUNCH_Q8(kQ4_1, true) break;
-    case kQ5_0: RNB_LAUNCH_Q8(kQ5_0, false) break;
-    default: RNB_LAUNCH_Q8(kQ5_1, false) break;
+    case kQ5_0: RNB_LAUNCH_Q8(kQ5_0, true) break;
+    default: RNB_LAUNCH_Q8(kQ5_1, true) break;
     }
 #undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8
