@@ -802,8 +802,9 @@ def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
 @pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q5_1])
 @pytest.mark.parametrize("seq,n_ff,n_embd", [(2, 256, 256), (3, 768, 512), (5, 512, 4608), (17, 512, 768), (40, 1024, 256)])
 def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
-    """Decode-sized batches take the fused gate/up GEMV, 16+ tokens the MFMA GEMM + SiLU kernel, rows longer than
-    16 super-blocks the unfused pair; all must equal the per-token composition of the oracle's pinned pieces."""
+    """Decode-sized batches take the fused gate/up GEMV, 8+ tokens (these matrices are small) the MFMA GEMMs and the gated
+    quantiser, rows longer than 16 super-blocks the unfused pair; all must equal the per-token composition of the
+    oracle's pinned pieces."""
     gate = oracle.make_weights(Q4_K, n_ff, n_embd, 300 + seq)
     up = oracle.make_weights(Q4_K, n_ff, n_embd, 301 + seq)
     down = oracle.make_weights(down_quant, n_embd, n_ff, 302 + seq)
@@ -831,6 +832,20 @@ def test_dense_gelu_ffn(rnb, oracle, down_quant, seq, n_ff, n_embd):
     check_close(got, ref, None, f"gelu ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
     # and it is not the SiLU result
     assert not np.allclose(got, oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x), rtol=1e-3, atol=0)
+
+
+@pytest.mark.parametrize("seq,down_quant", [(5, Q6_K), (9, Q4_K)])
+def test_dense_silu_ffn_few_tokens_large_matrices(rnb, oracle, seq, down_quant):
+    """Gate / up matrices of 16 MB and more (8192 x 4096 Q4_K) leave the fused gate/up GEMV for the GEMMs from 4 tokens
+    on: gate and up GEMMs, SiLU * up quantised as it is made, down GEMM (K slices on these small grids)."""
+    n_ff, n_embd = 8192, 4096
+    gate = oracle.make_weights(Q4_K, n_ff, n_embd, 340 + seq)
+    up = oracle.make_weights(Q4_K, n_ff, n_embd, 341 + seq)
+    down = oracle.make_weights(down_quant, n_embd, n_ff, 342 + seq)
+    x = oracle.fill_normal(seq * n_embd, 343 + seq, 1.0)
+    got = rnb.dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
+    ref = oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"dense ffn, large matrices, seq {seq} down {down_quant}")
 
 
 def test_dense_silu_ffn_dev_single_token_and_residency(rnb, oracle):
