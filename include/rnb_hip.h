@@ -187,6 +187,17 @@ int rnb_hip_dev_download(void *dst_host, const void *src_dev, size_t bytes);
 /* quant: RNB_GGML_*; x_dev [seq_len][cols] f32 (16-byte aligned); out_dev [seq_len][rows] f32 */
 int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
                      const float *x_dev, size_t seq_len, float *out_dev);
+/* rnb_hip_gemv_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments, arithmetic and results as
+ * rnb_hip_gemv_dev, but the quantised activations and the K-slice partial sums live in a fixed array inside the
+ * library's code object (rnb_hip_gemv_dev_noalloc_scratch_bytes() bytes per GPU, held until the process ends) instead
+ * of the grow-only scratch, so the call never allocates or frees device memory.  Shapes that need more scratch than
+ * that are rejected with RNB_HIP_INVALID_REQUEST (about 1.32 bytes per activation element, seq_len * cols, plus
+ * slices * seq_len * rows * 4 for the small-grid GEMMs).  The array keeps the previous call's contents and every call
+ * on a GPU shares it: calls that overlap on one GPU race, and it does not feed rnb_hip_gemv_quantized_dev. */
+size_t rnb_hip_gemv_dev_noalloc_scratch_bytes(void);
+int rnb_hip_gemv_dev_noalloc(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
+                             const float *x_dev, size_t seq_len, float *out_dev);
 /* The two halves of rnb_hip_gemv_dev, for callers that feed several weight matrices from one
  * activation (the reference quantises once for gate+up / QKV: rnb_quantize_q8_1_by_32 followed by
  * rnb_q4k_gate_up_gemv_* in crates/rnb-backend/cuda/cuda/kernels/quant_gemv.cuh:700-1267).

@@ -45,6 +45,8 @@ from .binding import (  # noqa: F401
     device_available,
     device_name,
     gemv_dev,
+    gemv_dev_noalloc,
+    gemv_dev_noalloc_scratch_bytes,
     gemv_quantized_dev,
     quantize_dev,
     last_error,

@@ -62,6 +62,8 @@ SYMBOLS = [
     ("rnb_hip_dev_upload", _i, [_vp, _vp, _sz]),
     ("rnb_hip_dev_download", _i, [_vp, _vp, _sz]),
     ("rnb_hip_gemv_dev", _i, [_u32, _vp, _sz, _sz, _vp, _sz, _vp]),
+    ("rnb_hip_gemv_dev_noalloc", _i, [_u32, _vp, _sz, _sz, _vp, _sz, _vp]),
+    ("rnb_hip_gemv_dev_noalloc_scratch_bytes", _sz, []),
     ("rnb_hip_quantize_dev", _i, [_u32, _vp, _sz, _sz]),
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
@@ -408,6 +410,16 @@ def gemv_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, x: DeviceBuffer,
              out: DeviceBuffer) -> None:
     """Enqueue activation quantisation + GEMV/GEMM on the library stream; does not synchronise."""
     _check(lib().rnb_hip_gemv_dev(quant, w.ptr, rows, cols, x.ptr, seq_len, out.ptr))
+
+
+def gemv_dev_noalloc(quant: int, w: DeviceBuffer, rows: int, cols: int, x: DeviceBuffer, seq_len: int,
+                     out: DeviceBuffer) -> None:
+    """gemv_dev with its scratch in the library's fixed device array: never allocates; does not synchronise."""
+    _check(lib().rnb_hip_gemv_dev_noalloc(quant, w.ptr, rows, cols, x.ptr, seq_len, out.ptr))
+
+
+def gemv_dev_noalloc_scratch_bytes() -> int:
+    return int(lib().rnb_hip_gemv_dev_noalloc_scratch_bytes())
 
 
 def quantize_dev(quant: int, x: DeviceBuffer, seq_len: int, cols: int) -> None:

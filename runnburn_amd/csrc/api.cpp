@@ -57,7 +57,6 @@ int hip_fail(const char *what, hipError_t e) {
         if (_e != hipSuccess) return hip_fail(#expr, _e);  \
     } while (0)
 
-// Quantise seq*cols staged floats on the device into the state's activation scratch.
 // Minimum tokens for which the MFMA GEMMs replace the vector-unit kernels, whose time grows with every token while a
 // GEMM's 32-token tile costs the same from 1 to 32.  Measured crossovers: Q6_K 4096 x 14336 (48 MB) 4 tokens (26.9 us
 // either way; 8 tokens 47 vs 27), Q4_K 14336 x 4096 (33 MB) 4 (21 vs 16 us), Q8_0 4096 x 14336 (62 MB) 3, Q8_0
@@ -77,35 +76,85 @@ constexpr uint64_t kGemmBigTilesMin = 32;
 // Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
 constexpr size_t kTokensMinSeq = 4;
 
-int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view) {
-    const size_t n = seq * cols;
-    HIP_TRY(s.act_qs.reserve(n));
-    if (is_block32(quant)) {
-        HIP_TRY(s.act_d.reserve(n / 32 * sizeof(float)));
-        launch_quantize_q8(x_dev, n / 32, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.stream);
-        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), nullptr};
-    } else {
-        HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
-        HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
-        s.act_has_digits = seq >= kDigitsMinSeq;
-        if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
-        uint8_t *digits = s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr;
-        launch_quantize_q8k(x_dev, n / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
-                            digits, s.stream);
-        *view = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>(), digits};
+// A fixed span of device memory that a call carves its scratch from instead of the state's grow-only buffers: the
+// entry point that must not allocate passes one over its static array.
+struct Arena {
+    uint8_t *base = nullptr;
+    size_t cap = 0, used = 0;
+    const char *who = "";
+};
+
+// `bytes` of scratch: from the arena when there is one (256-byte aligned pieces, an error when it is full), else the
+// state's buffer `slot`, grown if needed.
+int take_scratch(DeviceBuf &slot, Arena *arena, size_t bytes, void **out) {
+    if (arena) {
+        const size_t at = (arena->used + 255) / 256 * 256;
+        if (at + bytes > arena->cap)
+            return fail(RNB_HIP_INVALID_REQUEST, std::string(arena->who) + " needs more than the " +
+                                                     std::to_string(arena->cap) + " bytes of static scratch (" +
+                                                     std::to_string(at + bytes) + " so far)");
+        *out = arena->base + at;
+        arena->used = at + bytes;
+        return RNB_HIP_OK;
     }
-    HIP_TRY(hipGetLastError());
-    s.act_family = is_block32(quant) ? kQ8_0 : kQ4K;
-    s.act_seq = seq;
-    s.act_cols = cols;
+    HIP_TRY(slot.reserve(bytes));
+    *out = slot.ptr;
     return RNB_HIP_OK;
 }
 
+#define SCRATCH_TRY(slot, bytes, type, var)                                                         \
+    type *var = nullptr;                                                                            \
+    do {                                                                                            \
+        void *_p = nullptr;                                                                         \
+        if (int _st = take_scratch(slot, arena, bytes, &_p); _st != RNB_HIP_OK) return _st;         \
+        var = static_cast<type *>(_p);                                                              \
+    } while (0)
+
+// Quantise seq*cols f32 values on the device into activation scratch (the state's, which then remembers what it holds,
+// or the arena's).
+int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view,
+                         Arena *arena = nullptr) {
+    const size_t n = seq * cols;
+    SCRATCH_TRY(s.act_qs, n, int8_t, qs);
+    bool has_digits = false;
+    if (is_block32(quant)) {
+        SCRATCH_TRY(s.act_d, n / 32 * sizeof(float), float, d);
+        launch_quantize_q8(x_dev, n / 32, qs, d, s.stream);
+        *view = {qs, d, nullptr};
+    } else {
+        SCRATCH_TRY(s.act_d, n / 256 * sizeof(float), float, d);
+        SCRATCH_TRY(s.act_bsums, n / 256 * 16 * sizeof(int16_t), int16_t, bsums);
+        has_digits = seq >= kDigitsMinSeq;
+        uint8_t *digits = nullptr;
+        if (has_digits) {
+            SCRATCH_TRY(s.act_digits, n / 256 * 16, uint8_t, dg);
+            digits = dg;
+        }
+        launch_quantize_q8k(x_dev, n / 256, qs, d, bsums, digits, s.stream);
+        *view = {qs, d, bsums, digits};
+    }
+    HIP_TRY(hipGetLastError());
+    if (!arena) {
+        s.act_has_digits = has_digits;
+        s.act_family = is_block32(quant) ? kQ8_0 : kQ4K;
+        s.act_seq = seq;
+        s.act_cols = cols;
+    }
+    return RNB_HIP_OK;
+}
+
+// what the state's activation scratch holds, as the kernels take it
+ActView state_act_view(const State &s, uint32_t quant) {
+    const bool b32 = is_block32(quant);
+    return ActView{s.act_qs.as<int8_t>(), s.act_d.as<float>(), b32 ? nullptr : s.act_bsums.as<int16_t>(),
+                   !b32 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
+}
+
 int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
-                             float *out_dev);
+                             float *out_dev, const ActView &act, Arena *arena = nullptr);
 
 int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, const float *x_dev,
-                   size_t seq, float *out_dev) {
+                   size_t seq, float *out_dev, Arena *arena = nullptr) {
     // one token against rows of at most 16 super-blocks: the GEMV's workgroups quantise the token themselves
     if (seq == 1 && !is_block32(quant) && gemv_kquant_f32_supported(quant, static_cast<uint32_t>(cols / 256), x_dev)) {
         launch_gemv_kquant_f32(w_dev, quant, x_dev, out_dev, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 256),
@@ -120,27 +169,26 @@ int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, 
         return RNB_HIP_OK;
     }
     ActView act;
-    int st = quantize_activations(s, quant, x_dev, seq, cols, &act);
+    int st = quantize_activations(s, quant, x_dev, seq, cols, &act, arena);
     if (st != RNB_HIP_OK) return st;
-    return run_matmul_quantized_dev(s, quant, w_dev, rows, cols, seq, out_dev);
+    return run_matmul_quantized_dev(s, quant, w_dev, rows, cols, seq, out_dev, act, arena);
 }
 
 int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, size_t seq,
-                             float *out_dev) {
-    const bool b32 = is_block32(quant);
-    const ActView act{s.act_qs.as<int8_t>(), s.act_d.as<float>(), b32 ? nullptr : s.act_bsums.as<int16_t>(),
-                      !b32 && s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr};
+                             float *out_dev, const ActView &act, Arena *arena) {
     const uint32_t r = static_cast<uint32_t>(rows), q = static_cast<uint32_t>(seq);
     const uint32_t nb = static_cast<uint32_t>(cols / 256);
     const size_t min_gemm_seq = gemm_min_seq(quant, rows, cols);
     // workspace of the GEMMs that cut K into slices on small grids (null: none needed)
-    auto slice_ws = [&](uint32_t k_steps, float **ws) -> int {
+    auto slice_floats = [&](size_t floats, float **ws) -> int {
         *ws = nullptr;
-        const size_t floats = gemm_blocks_slice_floats(quant, r, k_steps, q);
         if (floats == 0) return RNB_HIP_OK;
-        HIP_TRY(s.gemm_slices.reserve(floats * sizeof(float)));
-        *ws = s.gemm_slices.as<float>();
+        SCRATCH_TRY(s.gemm_slices, floats * sizeof(float), float, p);
+        *ws = p;
         return RNB_HIP_OK;
+    };
+    auto slice_ws = [&](uint32_t k_steps, float **ws) -> int {
+        return slice_floats(gemm_blocks_slice_floats(quant, r, k_steps, q), ws);
     };
     float *ws = nullptr;
     if (quant == kQ4K) {
@@ -154,10 +202,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q4k_small(w_dev, act, out_dev, ws, r, nb, q, s.stream);
         } else if (seq >= min_gemm_seq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0) {
-            if (const size_t floats = gemm_q4k_slice_floats(r, nb, q)) {
-                HIP_TRY(s.gemm_slices.reserve(floats * sizeof(float)));
-                ws = s.gemm_slices.as<float>();
-            }
+            if (int st = slice_floats(gemm_q4k_slice_floats(r, nb, q), &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q4k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
         } else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
             launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
@@ -337,9 +382,9 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
     } else {
         HIP_TRY(s.ffn_gate.reserve(mid_bytes));
         HIP_TRY(s.ffn_up.reserve(mid_bytes));
-        st = run_matmul_quantized_dev(s, kQ4K, gate_dev, n_ff, n_embd, seq, s.ffn_gate.as<float>());
+        st = run_matmul_quantized_dev(s, kQ4K, gate_dev, n_ff, n_embd, seq, s.ffn_gate.as<float>(), act);
         if (st != RNB_HIP_OK) return st;
-        st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>());
+        st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>(), act);
         if (st != RNB_HIP_OK) return st;
         if (!is_block32(down_quant)) {
             // K-quant down projection: act(gate) * up is quantised to Q8_K as it is made, no f32 intermediate in memory
@@ -356,7 +401,8 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
             s.act_family = kQ4K;
             s.act_seq = seq;
             s.act_cols = n_ff;
-            return run_matmul_quantized_dev(s, down_quant, down_dev, n_embd, n_ff, seq, out_dev);
+            return run_matmul_quantized_dev(s, down_quant, down_dev, n_embd, n_ff, seq, out_dev,
+                                            state_act_view(s, down_quant));
         }
         launch_act_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, gelu, s.stream);
     }
@@ -588,6 +634,8 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     return RNB_HIP_OK;
 }
 
+int static_scratch_ptr(State &s, uint8_t **out);
+
 }  // namespace
 
 extern "C" {
@@ -604,7 +652,9 @@ int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
 
 int rnb_hip_init(void) {
     Guard g;
-    return g.state ? RNB_HIP_OK : g.status;
+    if (!g.state) return g.status;
+    uint8_t *unused = nullptr;  // the no-allocation entry point's scratch address is looked up here, once per device
+    return static_scratch_ptr(*g.state, &unused);
 }
 
 const char *rnb_hip_last_error(void) { return last_error_cstr(); }
@@ -1140,6 +1190,69 @@ int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols
     return run_matmul_dev(*g.state, quant, static_cast<const uint8_t *>(w_dev), rows, cols, x_dev, seq_len, out_dev);
 }
 
+}  // extern "C"
+
+namespace {
+
+// Scratch of rnb_hip_gemv_dev_noalloc: part of the code object, so every GPU that loads the library holds its own copy
+// until the process ends.  Host code never uses the array's name as an address; it asks the runtime for the device
+// address once per device and passes that to the kernels.
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
+constexpr int kStaticScratchMaxDevices = 64;
+uint8_t *g_static_scratch[kStaticScratchMaxDevices] = {};
+
+// device address of `scratch` on the state's device (the Guard has made it current)
+int static_scratch_ptr(State &s, uint8_t **out) {
+    if (s.device < 0 || s.device >= kStaticScratchMaxDevices)
+        return fail(RNB_HIP_EXECUTION_FAILED, "static scratch: device ordinal " + std::to_string(s.device) + " out of range");
+    if (g_static_scratch[s.device] == nullptr) {
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(RNB_HIP_EXECUTION_FAILED, "static scratch: hipGetSymbolAddress returned null");
+        g_static_scratch[s.device] = static_cast<uint8_t *>(p);
+    }
+    *out = g_static_scratch[s.device];
+    return RNB_HIP_OK;
+}
+
+// argument checks shared by rnb_hip_gemv_dev and rnb_hip_gemv_dev_noalloc
+int validate_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols, const float *x_dev, size_t seq_len,
+                      const float *out_dev) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    if (cols == 0 || cols % qi.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " cols must be divisible by " +
+                                                 std::to_string(qi.elems) + ", got " + std::to_string(cols));
+    if (!w_dev || !x_dev || !out_dev) return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " null device pointer");
+    if ((reinterpret_cast<uintptr_t>(w_dev) | reinterpret_cast<uintptr_t>(x_dev)) & 15u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " device pointers must be 16-byte aligned");
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu || seq_len > 65535u)
+        return fail(RNB_HIP_INVALID_REQUEST, std::string(qi.label) + " shape out of range");
+    return RNB_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t rnb_hip_gemv_dev_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int rnb_hip_gemv_dev_noalloc(uint32_t quant, const void *w_dev, size_t rows, size_t cols, const float *x_dev,
+                             size_t seq_len, float *out_dev) {
+    int st = validate_gemv_dev(quant, w_dev, rows, cols, x_dev, seq_len, out_dev);
+    if (st != RNB_HIP_OK) return st;
+    if (rows == 0 || seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    Arena arena;
+    arena.cap = kStaticScratchBytes;
+    arena.who = "rnb_hip_gemv_dev_noalloc";
+    st = static_scratch_ptr(*g.state, &arena.base);
+    if (st != RNB_HIP_OK) return st;
+    return run_matmul_dev(*g.state, quant, static_cast<const uint8_t *>(w_dev), rows, cols, x_dev, seq_len, out_dev, &arena);
+}
+
 int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols) {
     QuantInfo qi;
     if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
@@ -1175,7 +1288,8 @@ int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, s
                     std::string(qi.label) + " activation scratch holds seq_len=" + std::to_string(s.act_seq) + " cols=" +
                         std::to_string(s.act_cols) + " family=" + std::to_string(s.act_family) + ", requested seq_len=" +
                         std::to_string(seq_len) + " cols=" + std::to_string(cols));
-    return run_matmul_quantized_dev(s, quant, static_cast<const uint8_t *>(w_dev), rows, cols, seq_len, out_dev);
+    return run_matmul_quantized_dev(s, quant, static_cast<const uint8_t *>(w_dev), rows, cols, seq_len, out_dev,
+                                    state_act_view(s, quant));
 }
 
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev, const void *down_dev,
