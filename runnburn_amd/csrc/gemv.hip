@@ -27,6 +27,9 @@ namespace {
 
 constexpr int kWavesPerWg = 4;
 constexpr uint32_t kTargetWaves = 4096;  // total waves per launch: enough loads in flight, short tail
+// Matrices from this size on take gemv_kquant_chunks_kernel (measured crossover on Q4_K rows of 16 super-blocks: 33 MB
+// 7.5 us either way, 66 MB 12.4 against 13.0 us, 132 MB 22.1 against 24.1 us).
+constexpr uint64_t kGemvChunkMinBytes = uint64_t(48) << 20;
 
 // ---------------------------------------------------------------------------------------------
 // K-quant GEMV (Q2_K ... Q6_K share the structure; only the block functions differ)
@@ -82,6 +85,53 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             acc = seg_sum<kLanesPerRow>(acc);
             if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same GEMV for matrices far larger than what the chip holds in flight (rows of 9 to 16 super-blocks): every wave
+// takes kRows CONSECUTIVE rows, requests all of them at once and retires; with one wave per chunk the hardware
+// dispatcher keeps the CUs supplied with fresh waves, so the window of outstanding requests sweeps the matrix in
+// address order.  Measured on 264 MB of Q4_K: 41.5 us against 46.4 us for the grid-stride kernel above (80 % against
+// 71 % of 8 TB/s); on 33 MB the two are equal, so the launcher keeps the kernel above for small matrices.
+// The per-row arithmetic and the cross-lane sum are those of gemv_kquant_kernel: same bits.
+// ---------------------------------------------------------------------------------------------
+template <uint32_t kQuant, int kRows>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_kquant_chunks_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                              const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                              uint32_t n_chunks) {
+    using Q = KQuant<kQuant>;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int g = lane & 3;
+    const uint32_t bslot = lane >> 2;
+    const bool has_block = bslot < nb;
+    const uint32_t tok = blockIdx.y;
+    const size_t row_bytes = static_cast<size_t>(nb) * Q::kBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+    const typename Q::Act a = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    for (uint32_t c = wave_global; c < n_chunks; c += n_waves) {
+        typename Q::Regs r[kRows];
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t row = c * kRows + k;
+            const bool ok = has_block && row < rows;  // rows >= 1 and nb >= 1: offset 0 is readable
+            r[k] = Q::load_block(w + (ok ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * Q::kBytes : 0), g);
+        }
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t row = c * kRows + k;
+            float acc = (has_block && row < rows) ? kquant_partial<kQuant>(r[k], a, g) : 0.0f;
+            acc = seg_sum<kWave>(acc);
+            // lane 63 - k keeps row k's sum, so that one store instruction writes the chunk
+            const float t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), kWave - 1));
+            v = (lane == kWave - 1 - k) ? t : v;
+        }
+        const uint32_t row = c * kRows + (kWave - 1 - lane);
+        if (lane >= kWave - kRows && row < rows) out[static_cast<size_t>(tok) * rows + row] = v;
     }
 }
 
@@ -500,11 +550,29 @@ void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uin
                        act.d, act.bsums, out, rows, nb, row_groups);
 }
 
+// one wave per chunk of kRows rows (at most kChunkMaxWaves waves; beyond that the waves loop)
+constexpr uint32_t kChunkMaxWaves = 1u << 20;
+template <uint32_t kQuant, int kRows>
+void launch_kquant_chunks(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                          hipStream_t stream) {
+    const uint32_t n_chunks = (rows + kRows - 1) / kRows;
+    const uint32_t waves = n_chunks < kChunkMaxWaves ? n_chunks : kChunkMaxWaves;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    hipLaunchKernelGGL((gemv_kquant_chunks_kernel<kQuant, kRows>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
+                       act.d, act.bsums, out, rows, nb, n_chunks);
+}
+
 template <uint32_t kQuant>
 void launch_kquant_any(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                        hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
-    if (nb > 16 && nb <= 16 * kSplitMaxWaves)
+    if (nb > 8 && nb <= 16 && static_cast<uint64_t>(rows) * nb * KQuant<kQuant>::kBytes >= kGemvChunkMinBytes) {
+        // Q6_K measured best with four rows per wave (431 MB: 71.7 against 77.0 us with two), Q4_K with two
+        if (kQuant == kQ6K)
+            launch_kquant_chunks<kQuant, 4>(w, act, out, rows, nb, seq, stream);
+        else
+            launch_kquant_chunks<kQuant, 2>(w, act, out, rows, nb, seq, stream);
+    } else if (nb > 16 && nb <= 16 * kSplitMaxWaves)
         launch_kquant_splitk<kQuant>(w, act, out, rows, nb, seq, stream);
     else if (nb <= 4)
         launch_kquant<kQuant, 4>(w, act, out, rows, nb, seq, stream);
@@ -788,6 +856,20 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
     const bool kq = quant == kQ2K || quant == kQ3K || quant == kQ4K || quant == kQ5K || quant == kQ6K;
     return kq && nb >= 1 && nb <= 16 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
+    // From about 190 MB on, the separate quantiser launch (2.5 us) costs less than what the chunked kernel gains over
+    // the one-launch kernel, whose workgroups loop (264 MB of Q4_K: 41.5 + 2.5 against 48.0 us).
+    size_t bytes = 0;
+    switch (quant) {
+    case kQ2K: bytes = kQ2KBytes; break;
+    case kQ3K: bytes = kQ3KBytes; break;
+    case kQ4K: bytes = kQ4KBytes; break;
+    case kQ5K: bytes = kQ5KBytes; break;
+    default: bytes = kQ6KBytes; break;
+    }
+    return nb <= 8 || static_cast<uint64_t>(rows) * nb * bytes < (uint64_t(190) << 20);
 }
 
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,

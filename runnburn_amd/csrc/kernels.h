@@ -55,6 +55,8 @@ void launch_gemv_q4k_multi_f32(const uint8_t *const w[3], const uint32_t rows[3]
 // K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 16
 // super-blocks, x 16-byte aligned; same output contract as launch_gemv_q4k
 bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x);
+// false for matrices so large that quantising with a launch of its own and running the chunked GEMV is faster
+bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb);
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
                             uint32_t seq, hipStream_t stream);
 void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,

@@ -574,6 +574,27 @@ def test_config3b_q6k_gemv_lm_head_128256x4096(rnb, oracle):
     _full_gemv(rnb, oracle, Q6_K, 128256, 4096, "cfg3b")
 
 
+@pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 21001, 4096, 1), (Q6_K, 15003, 4096, 1), (Q5_K, 17921, 4096, 3),
+                                                 (Q4_K, 38839, 2304, 2), (Q2_K, 40001, 4096, 1), (Q3_K, 30001, 4096, 1)])
+def test_gemv_chunked_rows_kernel_large_matrices(rnb, oracle, quant, rows, cols, seq):
+    """Matrices of 48 MB and more with rows of 9 to 16 super-blocks take the kernel whose waves each reduce a chunk of
+    consecutive rows (two, four for Q6_K): row counts that are no multiple of the chunk, 9 super-blocks per row (idle
+    lanes), and two or three tokens (one grid row per token).  The arithmetic per row is the grid-stride kernel's, so
+    the first 4096 rows alone, a matrix small enough for that kernel, give the same bits."""
+    w = oracle.make_weights(quant, rows, cols, 7000 + rows)
+    x = oracle.fill_normal(seq * cols, 7001 + rows, 1.0)
+    fn = gemv_fn(rnb, quant, batch=seq > 1)
+    got = fn(w, rows, cols, x).reshape(seq, rows)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"chunked GEMV quant {quant} {rows}x{cols} seq {seq}")
+    rb = w.size // rows
+    head = w[:4096 * rb].copy()
+    small = fn(head, 4096, cols, x).reshape(seq, 4096)
+    assert np.array_equal(small.view(np.uint32), got[:, :4096].view(np.uint32))
+    rnb.release(head)
+    rnb.release(w)
+
+
 def test_q5k_gemv_full_size_14336x4096_and_4096x14336(rnb, oracle):
     """Q5_K at the up- and down-projection shapes of the Q4_K / Q6_K configurations."""
     _full_gemv(rnb, oracle, Q5_K, 14336, 4096, "q5k_up")
