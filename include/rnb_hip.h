@@ -86,6 +86,20 @@ int rnb_hip_prewarm(const uint8_t *const *ptrs, const size_t *lens, size_t n);
 /* drop a resident range (call before unmapping the host bytes) */
 int rnb_hip_release(const uint8_t *ptr, size_t len);
 int rnb_hip_resident_bytes(uint64_t *bytes, uint64_t *entries);
+/* Residency policy (crates/rnb-memory/src/byte_lru.rs:32-91, sparse_expert_cache.rs:221-250 and :272-395,
+ * crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:1055-1079, :1263-1459): host ranges that are not prewarmed
+ * stay resident least-recently-used inside a byte budget (85 % of the HBM free at open, RNB_HIP_RESIDENT_BUDGET_MB, or
+ * rnb_hip_set_resident_budget).  A missing range that fits only by evicting others is kept when
+ * bytes * (decayed earlier lookups + 1) > bytes + evicted bytes, else uploaded for that call alone; a call never
+ * evicts what it has itself resolved, nor prewarmed ranges; on a device out-of-memory further ranges are evicted and
+ * the allocation retried.
+ * rnb_hip_residency_stats fills up to 12 counters, the fields of ExpertBundleCacheStats (sparse_expert_cache.rs:383-395)
+ * as they apply here: lookups, hits, sub-range hits, misses, admissions, evictions, admitted bytes, evicted bytes,
+ * resident h2d bytes, per-call (temporary) h2d bytes, out-of-memory retries, and the budget in bytes. */
+int rnb_hip_residency_stats(uint64_t *out, size_t n);
+int rnb_hip_set_resident_budget(uint64_t bytes);
+/* offload_non_pinned_resident_q4k, q4k_cache.rs:276-303: frees every range that is not prewarmed */
+int rnb_hip_offload_unpinned(uint64_t *freed_bytes);
 
 /* ---- activation quantisers (bit-exact contract) --------------------------------------------- */
 /* quantize_input_q8k, crates/rnb-cpu/src/gemm/activation_q8.rs:109-139: n floats (n % 256 == 0)

@@ -349,6 +349,14 @@ void rnbo_dequantize_q6_k(const uint8_t *blocks, size_t n_blocks, float *out) {
 /* Activation quantisers                                                             */
 /* ================================================================================ */
 
+/* Rust's `f32 as i32`: NaN -> 0, out-of-range values saturate (the C conversion is undefined for both) */
+static inline int32_t f32_as_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+
 /* crates/rnb-cpu/src/gemm/activation_q8.rs:149-173 (quantize_q8k_block_ggml) */
 static void quantize_q8k_block(const float *x, rnbo_q8k_block *blk) {
     float amax = 0.0f, max_val = 0.0f;
@@ -366,7 +374,7 @@ static void quantize_q8k_block(const float *x, rnbo_q8k_block *blk) {
     blk->d = d;
     for (int i = 0; i < 256; i++) {
         volatile float prod = iscale * x[i];
-        int v = (int)rintf(prod); /* round half to even (default rounding mode) */
+        int v = f32_as_i32(rintf(prod)); /* round half to even (default rounding mode), then `as i32` */
         if (v > 127) v = 127;     /* upper clamp only */
         int8_t q = (int8_t)v;
         blk->qs[i] = q;
@@ -388,7 +396,7 @@ void rnbo_quantize_q8(const float *x, size_t n, rnbo_q8_block *out) {
         float amax = 0.0f;
         for (int i = 0; i < 32; i++) {
             float ax = fabsf(c[i]);
-            /* f32::max ignores NaN on one side; inputs here are finite */
+            /* f32::max ignores a NaN operand, as this comparison does */
             if (ax > amax) amax = ax;
         }
         volatile float d = amax / 127.0f;
@@ -399,7 +407,7 @@ void rnbo_quantize_q8(const float *x, size_t n, rnbo_q8_block *out) {
             float r = roundf(prod); /* half away from zero */
             if (r < -128.0f) r = -128.0f;
             if (r > 127.0f) r = 127.0f;
-            out[b].qs[i] = (int8_t)r;
+            out[b].qs[i] = (int8_t)f32_as_i32(r); /* NaN.clamp(..) stays NaN, `as i8` makes it 0 */
         }
     }
 }

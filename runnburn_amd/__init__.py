@@ -89,6 +89,9 @@ from .binding import (  # noqa: F401
     qwen35_sparse_experts_selected_base_by_token,
     release,
     resident_bytes,
+    residency_stats,
+    set_resident_budget,
+    offload_unpinned,
     stream_handle,
     sync,
     transfer_counters,

@@ -31,6 +31,9 @@ SYMBOLS = [
     ("rnb_hip_prewarm", _i, [C.POINTER(_vp), C.POINTER(_sz), _sz]),
     ("rnb_hip_release", _i, [_vp, _sz]),
     ("rnb_hip_resident_bytes", _i, [_u64p, _u64p]),
+    ("rnb_hip_residency_stats", _i, [_u64p, _sz]),
+    ("rnb_hip_set_resident_budget", _i, [C.c_uint64]),
+    ("rnb_hip_offload_unpinned", _i, [_u64p]),
     ("rnb_hip_quantize_q8k", _i, [_vp, _sz, _vp, _sz]),
     ("rnb_hip_quantize_q8", _i, [_vp, _sz, _vp, _sz]),
     ("rnb_hip_q4k_gemv", _i, _MATMUL_ARGS),
@@ -174,6 +177,27 @@ def resident_bytes() -> tuple[int, int]:
     a, b = C.c_uint64(), C.c_uint64()
     _check(lib().rnb_hip_resident_bytes(C.byref(a), C.byref(b)))
     return a.value, b.value
+
+
+RESIDENCY_STAT_NAMES = ("lookups", "hits", "sub_range_hits", "misses", "admissions", "evictions", "admitted_bytes",
+                        "evicted_bytes", "h2d_bytes", "temp_h2d_bytes", "oom_retries", "budget_bytes")
+
+
+def residency_stats() -> dict:
+    """Counters of the resident-weight table (the fields of ExpertBundleCacheStats that apply) and its budget."""
+    out = (C.c_uint64 * 12)()
+    _check(lib().rnb_hip_residency_stats(out, 12))
+    return dict(zip(RESIDENCY_STAT_NAMES, (int(v) for v in out)))
+
+
+def set_resident_budget(nbytes: int) -> None:
+    _check(lib().rnb_hip_set_resident_budget(int(nbytes)))
+
+
+def offload_unpinned() -> int:
+    freed = C.c_uint64()
+    _check(lib().rnb_hip_offload_unpinned(C.byref(freed)))
+    return int(freed.value)
 
 
 def _bytes_view(w) -> np.ndarray:

@@ -31,11 +31,13 @@ __device__ __forceinline__ void q8k_quantize_vals(const float4 v, int lane, int8
     // the element that attains it first in index order: lowest lane with a match, lowest element inside that lane
     const bool hit[4] = {ax[0] == amax, ax[1] == amax, ax[2] == amax, ax[3] == amax};
     const unsigned long long lanes = __builtin_amdgcn_ballot_w64(hit[0] || hit[1] || hit[2] || hit[3]);
-    const int first_lane = __builtin_ctzll(lanes);  // amax is one of the |x|, so at least one lane matches
+    // amax is one of the |x| unless every comparison failed (a block of NaNs: the reference's `ax > amax` is never
+    // true either, it keeps amax = 0 and writes d = 0 with all-zero codes)
+    const int first_lane = lanes != 0 ? __builtin_ctzll(lanes) : 0;
     const float mine = hit[0] ? e[0] : hit[1] ? e[1] : hit[2] ? e[2] : e[3];
     const float max_val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), first_lane));
     float iscale = 0.0f, d = 0.0f;
-    if (amax != 0.0f) {
+    if (lanes != 0 && amax != 0.0f) {
         iscale = -127.0f / max_val;
         d = 1.0f / iscale;
     }
@@ -109,6 +111,7 @@ __device__ __forceinline__ void q8_quantize_vals(const float4 v, int lane, int l
     float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
 #pragma unroll
     for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+    amax = fmaxf(amax, 0.0f);  // a block of NaNs: the reference's fold starts from 0.0 and f32::max ignores NaN
     const float d = amax / 127.0f;
     const float id = (d != 0.0f) ? 1.0f / d : 0.0f;
     uint32_t packed = 0;
@@ -117,6 +120,7 @@ __device__ __forceinline__ void q8_quantize_vals(const float4 v, int lane, int l
         const float prod = e[i] * id;
         float r = roundf(prod);  // half away from zero
         r = fminf(fmaxf(r, -128.0f), 127.0f);
+        r = prod != prod ? 0.0f : r;  // NaN (a NaN input, or inf * 0): the reference's NaN.clamp(..) as i8 is 0
         packed |= (static_cast<uint32_t>(static_cast<int>(r)) & 0xffu) << (8 * i);
     }
     if (live) {

@@ -76,6 +76,29 @@ constexpr uint64_t kGemmBigTilesMin = 32;
 // Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
 constexpr size_t kTokensMinSeq = 4;
 
+// After enqueuing kernels: a launcher that could not configure its kernel (and therefore did not launch) left the
+// reason; otherwise whatever the runtime recorded.
+int check_launches() {
+    const std::string pending = take_launch_failure();
+    if (!pending.empty()) return fail(RNB_HIP_EXECUTION_FAILED, pending);
+    HIP_TRY(hipGetLastError());
+    return RNB_HIP_OK;
+}
+
+// Growing a scratch buffer: refused with a message while the library stream is capturing into a graph.
+int reserve_fail(hipError_t e) {
+    if (e == hipErrorStreamCaptureUnsupported)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    "scratch would have to grow while the library stream is capturing: run this shape once before the "
+                    "capture, or use rnb_hip_gemv_dev_noalloc");
+    return hip_fail("scratch allocation", e);
+}
+#define RESERVE_TRY(buf, bytes)                                \
+    do {                                                       \
+        hipError_t _e = (buf).reserve(bytes);                  \
+        if (_e != hipSuccess) return reserve_fail(_e);         \
+    } while (0)
+
 // A fixed span of device memory that a call carves its scratch from instead of the state's grow-only buffers: the
 // entry point that must not allocate passes one over its static array.
 struct Arena {
@@ -97,7 +120,7 @@ int take_scratch(DeviceBuf &slot, Arena *arena, size_t bytes, void **out) {
         arena->used = at + bytes;
         return RNB_HIP_OK;
     }
-    HIP_TRY(slot.reserve(bytes));
+    RESERVE_TRY(slot, bytes);
     *out = slot.ptr;
     return RNB_HIP_OK;
 }
@@ -133,7 +156,7 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
         launch_quantize_q8k(x_dev, n / 256, qs, d, bsums, digits, s.stream);
         *view = {qs, d, bsums, digits};
     }
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     if (!arena) {
         s.act_has_digits = has_digits;
         s.act_family = is_block32(quant) ? kQ8_0 : kQ4K;
@@ -160,13 +183,13 @@ int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, 
         gemv_kquant_f32_pays(quant, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 256))) {
         launch_gemv_kquant_f32(w_dev, quant, x_dev, out_dev, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 256),
                                1, s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
     if (seq == 1 && is_block32(quant) && gemv_block32_f32_supported(static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 32), x_dev)) {
         launch_gemv_block32_f32(w_dev, quant, x_dev, out_dev, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 32), 1,
                                 s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
     ActView act;
@@ -240,7 +263,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     } else {
         launch_gemv_block32(w_dev, quant, act, out_dev, r, static_cast<uint32_t>(cols / 32), q, s.stream);
     }
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     return RNB_HIP_OK;
 }
 
@@ -296,10 +319,10 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
     if (!g.state) return g.status;
     State &s = *g.state;
     const uint8_t *w_dev = nullptr;
-    HIP_TRY(s.resident_ptr(w, w_len, &w_dev));
+    if (int rs = s.resident_ptr(w, w_len, &w_dev); rs != RNB_HIP_OK) return rs;
     const size_t in_bytes = seq * cols * sizeof(float), out_bytes = seq * rows * sizeof(float);
-    HIP_TRY(s.bounce_in.reserve(in_bytes));
-    HIP_TRY(s.bounce_out.reserve(out_bytes));
+    RESERVE_TRY(s.bounce_in, in_bytes);
+    RESERVE_TRY(s.bounce_out, out_bytes);
     HIP_TRY(s.x_f32.reserve(in_bytes));
     HIP_TRY(s.out_f32.reserve(out_bytes));
     std::memcpy(s.bounce_in.ptr, x, in_bytes);
@@ -362,7 +385,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
                       uint32_t down_quant, size_t n_ff, size_t n_embd, size_t seq, const float *x_dev, float *out_dev,
                       bool gelu = false) {
     const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
-    HIP_TRY(s.ffn_mid.reserve(mid_bytes));
+    RESERVE_TRY(s.ffn_mid, mid_bytes);
     const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
     const bool small = seq < gemm_min_seq(kQ4K, n_ff, n_embd) && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
     ActView act;
@@ -372,7 +395,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         // repeated quantisation costs more than the launch it saves (measured)
         launch_gemv_q4k_gate_up_f32(gate_dev, up_dev, x_dev, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
                                     static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), gelu, s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return run_matmul_dev(s, down_quant, down_dev, n_embd, n_ff, s.ffn_mid.as<float>(), seq, out_dev);
     }
     st = quantize_activations(s, kQ4K, x_dev, seq, n_embd, &act);
@@ -381,8 +404,8 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         launch_gemv_q4k_gate_up(gate_dev, up_dev, act, s.ffn_mid.as<float>(), static_cast<uint32_t>(n_ff),
                                 static_cast<uint32_t>(nb_in), static_cast<uint32_t>(seq), gelu, s.stream);
     } else {
-        HIP_TRY(s.ffn_gate.reserve(mid_bytes));
-        HIP_TRY(s.ffn_up.reserve(mid_bytes));
+        RESERVE_TRY(s.ffn_gate, mid_bytes);
+        RESERVE_TRY(s.ffn_up, mid_bytes);
         st = run_matmul_quantized_dev(s, kQ4K, gate_dev, n_ff, n_embd, seq, s.ffn_gate.as<float>(), act);
         if (st != RNB_HIP_OK) return st;
         st = run_matmul_quantized_dev(s, kQ4K, up_dev, n_ff, n_embd, seq, s.ffn_up.as<float>(), act);
@@ -390,15 +413,15 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         if (!is_block32(down_quant)) {
             // K-quant down projection: act(gate) * up is quantised to Q8_K as it is made, no f32 intermediate in memory
             const size_t n = seq * n_ff;
-            HIP_TRY(s.act_qs.reserve(n));
-            HIP_TRY(s.act_d.reserve(n / 256 * sizeof(float)));
-            HIP_TRY(s.act_bsums.reserve(n / 256 * 16 * sizeof(int16_t)));
+            RESERVE_TRY(s.act_qs, n);
+            RESERVE_TRY(s.act_d, n / 256 * sizeof(float));
+            RESERVE_TRY(s.act_bsums, n / 256 * 16 * sizeof(int16_t));
             s.act_has_digits = seq >= kDigitsMinSeq;
-            if (s.act_has_digits) HIP_TRY(s.act_digits.reserve(n / 256 * 16));
+            if (s.act_has_digits) RESERVE_TRY(s.act_digits, n / 256 * 16);
             launch_quantize_q8k_gated(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), n / 256, gelu, s.act_qs.as<int8_t>(),
                                       s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
                                       s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr, s.stream);
-            HIP_TRY(hipGetLastError());
+            if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
             s.act_family = kQ4K;
             s.act_seq = seq;
             s.act_cols = n_ff;
@@ -407,7 +430,7 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
         }
         launch_act_mul(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), s.ffn_mid.as<float>(), seq * n_ff, gelu, s.stream);
     }
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     // the intermediate is re-quantised in the form the down projection's rows take, then the down matmul runs
     return run_matmul_dev(s, down_quant, down_dev, n_embd, n_ff, s.ffn_mid.as<float>(), seq, out_dev);
 }
@@ -491,11 +514,11 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
             table.expert[i] = i < n_slots ? expert_ids[i] : 0;
             table.route[i] = i < n_slots ? route[i] : 0.0f;
         }
-        HIP_TRY(s.moe_mid.reserve(n_slots * n_ff * sizeof(float)));
+        RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
         launch_moe_decode(gate_dev, up_dev, down_dev, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
                           static_cast<uint32_t>(n_ff), static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_in),
                           static_cast<uint32_t>(sh.nb_mid), s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
     // slots are grouped by expert, keeping slot order inside a group
@@ -525,6 +548,10 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     uint32_t *h = inl.words;
     TableSlot *ring_slot = nullptr;
     if (!inline_tables) {
+        if (s.capturing())
+            return fail(RNB_HIP_INVALID_REQUEST,
+                        "Qwen35 full-layer routing tables of this size are uploaded from host memory and cannot be captured "
+                        "into a graph (one token with at most 16 slots, or tables of at most 240 words, can)");
         // larger tables go through one of a ring of pinned buffers, so that a call never waits for the
         // previous call's upload to drain
         ring_slot = &s.table_ring[s.table_ring_next];
@@ -533,10 +560,10 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
             HIP_TRY(hipEventCreateWithFlags(&ring_slot->event, hipEventDisableTiming));
         else
             HIP_TRY(hipEventSynchronize(ring_slot->event));
-        HIP_TRY(ring_slot->host.reserve(table_words * 4));
+        RESERVE_TRY(ring_slot->host, table_words * 4);
         h = ring_slot->host.as<uint32_t>();
     }
-    HIP_TRY(s.moe_tables.reserve(table_words * 4));
+    RESERVE_TRY(s.moe_tables, table_words * 4);
     float *h_route = reinterpret_cast<float *>(h);
     uint32_t *h_off = h + n_slots, *h_list = h_off + token_count + 1;
     uint32_t *h_sslot = h_list + n_slots, *h_stok = h_sslot + n_slots;
@@ -569,12 +596,12 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     if (inline_tables) {
         // quantise x and drop the tables into device memory with the same launch
         const size_t nq = token_count * n_embd;
-        HIP_TRY(s.act_qs.reserve(nq));
-        HIP_TRY(s.act_d.reserve(nq / 256 * sizeof(float)));
-        HIP_TRY(s.act_bsums.reserve(nq / 256 * 16 * sizeof(int16_t)));
+        RESERVE_TRY(s.act_qs, nq);
+        RESERVE_TRY(s.act_d, nq / 256 * sizeof(float));
+        RESERVE_TRY(s.act_bsums, nq / 256 * 16 * sizeof(int16_t));
         launch_quantize_q8k_with_tables(x_dev, nq / 256, s.act_qs.as<int8_t>(), s.act_d.as<float>(),
                                         s.act_bsums.as<int16_t>(), inl, static_cast<uint32_t>(table_words), d, s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         act = {s.act_qs.as<int8_t>(), s.act_d.as<float>(), s.act_bsums.as<int16_t>()};
         s.act_family = kQ4K;
         s.act_has_digits = false;
@@ -587,19 +614,19 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     if (n_slots == 0) {  // nothing routed: the reduce kernel alone writes the zero rows
         launch_moe_reduce(nullptr, d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
-    HIP_TRY(s.moe_mid.reserve(n_slots * n_ff * sizeof(float)));
-    HIP_TRY(s.moe_mid_qs.reserve(n_slots * n_ff));
-    HIP_TRY(s.moe_mid_d.reserve(n_slots * sh.nb_mid * sizeof(float)));
-    HIP_TRY(s.moe_mid_bsums.reserve(n_slots * sh.nb_mid * 16 * sizeof(int16_t)));
-    HIP_TRY(s.moe_slot_out.reserve(n_slots * n_embd * sizeof(float)));
+    RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
+    RESERVE_TRY(s.moe_mid_qs, n_slots * n_ff);
+    RESERVE_TRY(s.moe_mid_d, n_slots * sh.nb_mid * sizeof(float));
+    RESERVE_TRY(s.moe_mid_bsums, n_slots * sh.nb_mid * 16 * sizeof(int16_t));
+    RESERVE_TRY(s.moe_slot_out, n_slots * n_embd * sizeof(float));
     if (mfma && act.digits != nullptr) {
         // prefill: grouped GEMMs, 32-token tiles per expert
         uint8_t *mid_digits = nullptr;
         if (down_quant != kQ6K) {  // Q4_K / Q5_K mins need the 32-element sums' digits
-            HIP_TRY(s.moe_mid_digits.reserve(n_slots * sh.nb_mid * 16));
+            RESERVE_TRY(s.moe_mid_digits, n_slots * sh.nb_mid * 16);
             mid_digits = s.moe_mid_digits.as<uint8_t>();
         }
         launch_moe_gate_up_mfma(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
@@ -611,7 +638,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                              static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
-        HIP_TRY(hipGetLastError());
+        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
     launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
@@ -631,7 +658,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
     }
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     return RNB_HIP_OK;
 }
 
@@ -679,7 +706,8 @@ int rnb_hip_sync(void) {
 int rnb_hip_transfer_counters(uint64_t *h2d_bytes, uint64_t *d2h_bytes) {
     Guard g;
     if (!g.state) return g.status;
-    if (h2d_bytes) *h2d_bytes = g.state->h2d_bytes;
+    const ResidencyStats &rs = g.state->table->stats();
+    if (h2d_bytes) *h2d_bytes = g.state->h2d_bytes + rs.h2d_bytes + rs.temp_h2d_bytes;
     if (d2h_bytes) *d2h_bytes = g.state->d2h_bytes;
     return RNB_HIP_OK;
 }
@@ -695,7 +723,7 @@ int rnb_hip_prewarm(const uint8_t *const *ptrs, const size_t *lens, size_t n) {
     for (size_t i = 0; i < n; i++) {
         if (!ptrs[i] || lens[i] == 0) continue;
         const uint8_t *dev = nullptr;
-        HIP_TRY(g.state->resident_ptr(ptrs[i], lens[i], &dev, /*pin=*/true));
+        if (int rs = g.state->resident_ptr(ptrs[i], lens[i], &dev, /*pin=*/true); rs != RNB_HIP_OK) return rs;
     }
     return RNB_HIP_OK;
 }
@@ -710,8 +738,36 @@ int rnb_hip_release(const uint8_t *ptr, size_t len) {
 int rnb_hip_resident_bytes(uint64_t *bytes, uint64_t *entries) {
     Guard g;
     if (!g.state) return g.status;
-    if (bytes) *bytes = g.state->resident_bytes;
-    if (entries) *entries = g.state->residents.size();
+    if (bytes) *bytes = g.state->table->resident_bytes();
+    if (entries) *entries = g.state->table->entries();
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_residency_stats(uint64_t *out, size_t n) {
+    Guard g;
+    if (!g.state) return g.status;
+    const ResidencyStats &rs = g.state->table->stats();
+    const uint64_t v[12] = {rs.lookups, rs.hits, rs.sub_range_hits, rs.misses, rs.admissions, rs.evictions,
+                            rs.admitted_bytes, rs.evicted_bytes, rs.h2d_bytes, rs.temp_h2d_bytes, rs.oom_retries,
+                            g.state->table->budget()};
+    for (size_t i = 0; i < n && i < 12; i++) out[i] = v[i];
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_set_resident_budget(uint64_t bytes) {
+    Guard g;
+    if (!g.state) return g.status;
+    g.state->table->set_budget(bytes);
+    return RNB_HIP_OK;
+}
+
+int rnb_hip_offload_unpinned(uint64_t *freed_bytes) {
+    Guard g;
+    if (!g.state) return g.status;
+    std::string err;
+    const uint64_t freed = g.state->table->offload_unpinned(&err);
+    if (freed_bytes) *freed_bytes = freed;
+    if (!err.empty()) return fail(RNB_HIP_EXECUTION_FAILED, err);
     return RNB_HIP_OK;
 }
 
@@ -726,7 +782,7 @@ int rnb_hip_quantize_q8k(const float *x, size_t n, void *out_blocks, size_t out_
     Guard g;
     if (!g.state) return g.status;
     State &s = *g.state;
-    HIP_TRY(s.bounce_in.reserve(n * 4));
+    RESERVE_TRY(s.bounce_in, n * 4);
     HIP_TRY(s.x_f32.reserve(n * 4));
     std::memcpy(s.bounce_in.ptr, x, n * 4);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, n * 4, hipMemcpyHostToDevice, s.stream));
@@ -734,7 +790,7 @@ int rnb_hip_quantize_q8k(const float *x, size_t n, void *out_blocks, size_t out_
     int st = quantize_activations(s, kQ4K, s.x_f32.as<float>(), 1, n, &act);
     if (st != RNB_HIP_OK) return st;
     const size_t qs_b = n, d_b = nb * 4, bs_b = nb * 32;
-    HIP_TRY(s.bounce_out.reserve(qs_b + d_b + bs_b));
+    RESERVE_TRY(s.bounce_out, qs_b + d_b + bs_b);
     uint8_t *h = s.bounce_out.as<uint8_t>();
     HIP_TRY(hipMemcpyAsync(h, act.qs, qs_b, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipMemcpyAsync(h + qs_b, act.d, d_b, hipMemcpyDeviceToHost, s.stream));
@@ -763,14 +819,14 @@ int rnb_hip_quantize_q8(const float *x, size_t n, void *out_blocks, size_t out_b
     Guard g;
     if (!g.state) return g.status;
     State &s = *g.state;
-    HIP_TRY(s.bounce_in.reserve(n * 4));
+    RESERVE_TRY(s.bounce_in, n * 4);
     HIP_TRY(s.x_f32.reserve(n * 4 + 1024));
     std::memcpy(s.bounce_in.ptr, x, n * 4);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, n * 4, hipMemcpyHostToDevice, s.stream));
     ActView act;
     int st = quantize_activations(s, kQ8_0, s.x_f32.as<float>(), 1, n, &act);
     if (st != RNB_HIP_OK) return st;
-    HIP_TRY(s.bounce_out.reserve(n + nb * 4));
+    RESERVE_TRY(s.bounce_out, n + nb * 4);
     uint8_t *h = s.bounce_out.as<uint8_t>();
     HIP_TRY(hipMemcpyAsync(h, act.qs, n, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipMemcpyAsync(h + n, act.d, nb * 4, hipMemcpyDeviceToHost, s.stream));
@@ -865,12 +921,12 @@ int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len
     if (!g.state) return g.status;
     State &s = *g.state;
     const uint8_t *gate_dev = nullptr, *up_dev = nullptr, *down_dev = nullptr;
-    HIP_TRY(s.resident_ptr(gate_all, gate_len, &gate_dev));
-    HIP_TRY(s.resident_ptr(up_all, up_len, &up_dev));
-    HIP_TRY(s.resident_ptr(down_all, down_len, &down_dev));
+    if (int rs = s.resident_ptr(gate_all, gate_len, &gate_dev); rs != RNB_HIP_OK) return rs;
+    if (int rs = s.resident_ptr(up_all, up_len, &up_dev); rs != RNB_HIP_OK) return rs;
+    if (int rs = s.resident_ptr(down_all, down_len, &down_dev); rs != RNB_HIP_OK) return rs;
     const size_t io_bytes = token_count * n_embd * sizeof(float);
-    HIP_TRY(s.bounce_in.reserve(io_bytes));
-    HIP_TRY(s.bounce_out.reserve(io_bytes));
+    RESERVE_TRY(s.bounce_in, io_bytes);
+    RESERVE_TRY(s.bounce_out, io_bytes);
     HIP_TRY(s.x_f32.reserve(io_bytes));
     HIP_TRY(s.out_f32.reserve(io_bytes));
     std::memcpy(s.bounce_in.ptr, x, io_bytes);
@@ -946,13 +1002,13 @@ int gemv_argmax_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows
     if (!g.state) return g.status;
     State &s = *g.state;
     const uint8_t *w_dev = nullptr;
-    HIP_TRY(s.resident_ptr(w, w_len, &w_dev));
+    if (int rs = s.resident_ptr(w, w_len, &w_dev); rs != RNB_HIP_OK) return rs;
     const size_t in_bytes = cols * sizeof(float);
-    HIP_TRY(s.bounce_in.reserve(in_bytes));
-    HIP_TRY(s.bounce_out.reserve(16));
+    RESERVE_TRY(s.bounce_in, in_bytes);
+    RESERVE_TRY(s.bounce_out, 16);
     HIP_TRY(s.x_f32.reserve(in_bytes));
     HIP_TRY(s.out_f32.reserve(rows * sizeof(float)));
-    HIP_TRY(s.argmax_scratch.reserve(257 * 8));
+    RESERVE_TRY(s.argmax_scratch, 257 * 8);
     std::memcpy(s.bounce_in.ptr, x, in_bytes);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += in_bytes;
@@ -961,7 +1017,7 @@ int gemv_argmax_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows
     float *vals = s.argmax_scratch.as<float>();
     uint32_t *idxs = reinterpret_cast<uint32_t *>(vals + 257);
     launch_argmax(s.out_f32.as<float>(), static_cast<uint32_t>(rows), vals, idxs, vals + 256, idxs + 256, s.stream);
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     // only the winner crosses the bus: 8 bytes instead of rows * 4
     HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, vals + 256, 4, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipMemcpyAsync(static_cast<uint8_t *>(s.bounce_out.ptr) + 4, idxs + 256, 4, hipMemcpyDeviceToHost, s.stream));
@@ -1019,12 +1075,12 @@ int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint
     if (!g.state) return g.status;
     State &s = *g.state;
     const uint8_t *w_dev[3] = {nullptr, nullptr, nullptr};
-    if (q_len) HIP_TRY(s.resident_ptr(q_w, q_len, &w_dev[0]));
-    if (k_len) HIP_TRY(s.resident_ptr(k_w, k_len, &w_dev[1]));
-    if (v_len) HIP_TRY(s.resident_ptr(v_w, v_len, &w_dev[2]));
+    if (q_len) if (int rs = s.resident_ptr(q_w, q_len, &w_dev[0]); rs != RNB_HIP_OK) return rs;
+    if (k_len) if (int rs = s.resident_ptr(k_w, k_len, &w_dev[1]); rs != RNB_HIP_OK) return rs;
+    if (v_len) if (int rs = s.resident_ptr(v_w, v_len, &w_dev[2]); rs != RNB_HIP_OK) return rs;
     const size_t in_bytes = n_embd * sizeof(float), out_bytes = total * sizeof(float);
-    HIP_TRY(s.bounce_in.reserve(in_bytes));
-    HIP_TRY(s.bounce_out.reserve(out_bytes));
+    RESERVE_TRY(s.bounce_in, in_bytes);
+    RESERVE_TRY(s.bounce_out, out_bytes);
     HIP_TRY(s.x_f32.reserve(in_bytes));
     HIP_TRY(s.out_f32.reserve(out_bytes));
     std::memcpy(s.bounce_in.ptr, x, in_bytes);
@@ -1040,7 +1096,7 @@ int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint
         if (st != RNB_HIP_OK) return st;
         launch_gemv_q4k_multi(w_dev, rows, act, s.out_f32.as<float>(), static_cast<uint32_t>(n_embd / 256), s.stream);
     }
-    HIP_TRY(hipGetLastError());
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
     HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
     HIP_TRY(hipStreamSynchronize(s.stream));
     s.d2h_bytes += out_bytes;
@@ -1068,12 +1124,12 @@ int dense_ffn_host(const uint8_t *gate, size_t gate_len, const uint8_t *up, size
     if (!g.state) return g.status;
     State &s = *g.state;
     const uint8_t *gate_dev = nullptr, *up_dev = nullptr, *down_dev = nullptr;
-    HIP_TRY(s.resident_ptr(gate, gate_len, &gate_dev));
-    HIP_TRY(s.resident_ptr(up, up_len, &up_dev));
-    HIP_TRY(s.resident_ptr(down, down_len, &down_dev));
+    if (int rs = s.resident_ptr(gate, gate_len, &gate_dev); rs != RNB_HIP_OK) return rs;
+    if (int rs = s.resident_ptr(up, up_len, &up_dev); rs != RNB_HIP_OK) return rs;
+    if (int rs = s.resident_ptr(down, down_len, &down_dev); rs != RNB_HIP_OK) return rs;
     const size_t io_bytes = seq_len * n_embd * sizeof(float);
-    HIP_TRY(s.bounce_in.reserve(io_bytes));
-    HIP_TRY(s.bounce_out.reserve(io_bytes));
+    RESERVE_TRY(s.bounce_in, io_bytes);
+    RESERVE_TRY(s.bounce_out, io_bytes);
     HIP_TRY(s.x_f32.reserve(io_bytes));
     HIP_TRY(s.out_f32.reserve(io_bytes));
     std::memcpy(s.bounce_in.ptr, x, io_bytes);
@@ -1195,25 +1251,13 @@ int rnb_hip_gemv_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols
 
 namespace {
 
-// Scratch of rnb_hip_gemv_dev_noalloc: part of the code object, so every GPU that loads the library holds its own copy
-// until the process ends.  Host code never uses the array's name as an address; it asks the runtime for the device
-// address once per device and passes that to the kernels.
-constexpr size_t kStaticScratchBytes = size_t(8) << 20;
-static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
-constexpr int kStaticScratchMaxDevices = 64;
-uint8_t *g_static_scratch[kStaticScratchMaxDevices] = {};
-
-// device address of `scratch` on the state's device (the Guard has made it current)
+// device address of the no-allocation entry point's scratch array on the state's device (the Guard has made it current)
 int static_scratch_ptr(State &s, uint8_t **out) {
-    if (s.device < 0 || s.device >= kStaticScratchMaxDevices)
-        return fail(RNB_HIP_EXECUTION_FAILED, "static scratch: device ordinal " + std::to_string(s.device) + " out of range");
-    if (g_static_scratch[s.device] == nullptr) {
-        void *p = nullptr;
-        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-        if (p == nullptr) return fail(RNB_HIP_EXECUTION_FAILED, "static scratch: hipGetSymbolAddress returned null");
-        g_static_scratch[s.device] = static_cast<uint8_t *>(p);
-    }
-    *out = g_static_scratch[s.device];
+    void *p = nullptr;
+    const hipError_t e = static_scratch_address(s.device, &p);
+    if (e != hipSuccess) return hip_fail("static scratch: hipGetSymbolAddress", e);
+    if (p == nullptr) return fail(RNB_HIP_EXECUTION_FAILED, "static scratch: no address for device " + std::to_string(s.device));
+    *out = static_cast<uint8_t *>(p);
     return RNB_HIP_OK;
 }
 

@@ -1040,12 +1040,10 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
 #define RNB_LAUNCH_Q8R(TT, FMT, R)                                                                                     \
     {                                                                                                                  \
         constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
-        static bool configured = false;                                                                                \
-        if (!configured) { /* above the default 64 KB of dynamic LDS in the routed 64-token form */                    \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, FMT, R>),                 \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));              \
-            configured = true;                                                                                         \
-        }                                                                                                              \
+        static bool configured = false; /* above the default 64 KB of dynamic LDS in the routed 64-token form */       \
+        if (!allow_dynamic_lds(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, FMT, R>), lds, &configured,      \
+                               "gemm_q8_mfma_kernel"))                                                                 \
+            return;                                                                                                    \
         hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, FMT, R>), grid, block, lds, stream, w, act.qs, act.d, dst, rows,   \
                            nb32, seq, steps_slice);                                                                    \
     }

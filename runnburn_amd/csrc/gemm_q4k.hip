@@ -311,12 +311,9 @@ size_t gemm_q4k_slice_floats(uint32_t rows, uint32_t nb, uint32_t seq) {
 void launch_gemm_q4k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
-    static bool configured = false;
-    if (!configured) {  // 111 KB exceed the default 64 KB dynamic LDS limit
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kPpLdsBytes);
-        configured = true;
-    }
+    static bool configured = false;  // 111 KB exceed the default 64 KB dynamic LDS limit
+    if (!allow_dynamic_lds(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), kPpLdsBytes, &configured, "gemm_q4k_mfma_kernel"))
+        return;
     const uint32_t slices = slice_out ? pp_slices(rows, nb, seq) : 1;
     const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
     const dim3 grid((rows + kPpRowsPerWg - 1) / kPpRowsPerWg, (seq + kPpToks - 1) / kPpToks, nz);

@@ -6,6 +6,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <string>
+
 namespace rnb {
 
 constexpr uint32_t kQ4_0 = 2, kQ4_1 = 3, kQ5_0 = 6, kQ5_1 = 7, kQ8_0 = 8, kQ8_1 = 9, kQ2K = 10, kQ3K = 11, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
@@ -171,5 +173,18 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
 // tok_offsets [token_count+1], tok_slots [n_slots] (CSR built by the host)
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,
                        float *out, uint32_t token_count, uint32_t n_embd, hipStream_t stream);
+
+// ---- launch configuration failures ------------------------------------------------------------------
+// Raises `kernel`'s dynamic LDS limit to `bytes` (above the default 64 KB) once: `*done` is set only when the runtime
+// accepted it, so a failure is tried again by the next launch.  On failure the launcher must not launch; the reason is
+// kept for the API layer, which reports it instead of an unrelated launch error (take_launch_failure).
+bool allow_dynamic_lds(const void *kernel, size_t bytes, bool *done, const char *kernel_name);
+// the pending failure text of this thread, cleared by the call; empty when there is none
+std::string take_launch_failure();
+
+// ---- scratch that is part of the code object (static_scratch.hip) ---------------------------------
+// Device address of the library's fixed scratch array on `device` (which must be current): looked up once per device.
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;
+hipError_t static_scratch_address(int device, void **out);
 
 }  // namespace rnb

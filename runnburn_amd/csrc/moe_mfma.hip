@@ -407,12 +407,9 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 // raises a kernel's dynamic LDS limit above the default 64 KB, once per kernel (K is a distinct type per kernel only
 // through the tag)
 template <int kTag, typename K>
-void allow_lds(K kernel, size_t bytes) {
+bool allow_lds(K kernel, size_t bytes) {
     static bool done = false;
-    if (done) return;
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(bytes));
-    done = true;
+    return allow_dynamic_lds(reinterpret_cast<const void *>(kernel), bytes, &done, "MoE matrix-core kernel");
 }
 
 }  // namespace
@@ -431,7 +428,7 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
                              uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0 || n_ff == 0) return;
     const size_t lds = TileImage<kGbStride128, true>::bytes(nb_in);
-    allow_lds<0>(moe_gate_up_mfma_kernel, kMmLdsLimit);
+    if (!allow_lds<0>(moe_gate_up_mfma_kernel, kMmLdsLimit)) return;
     const dim3 grid((n_ff + kGbRows - 1) / kGbRows, groups.n_groups, 1);
     hipLaunchKernelGGL(moe_gate_up_mfma_kernel, grid, dim3(kGbThreads), lds, stream, gate_all, up_all, act.qs, act.d, act.digits,
                        groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in);
@@ -449,7 +446,7 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView 
         tiles_per_wg *= 2;
     const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1), block(kGbThreads);
 #define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
-    allow_lds<static_cast<int>(Q)>(moe_down_mfma_kernel<Q>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit);                                           \
+    if (!allow_lds<static_cast<int>(Q)>(moe_down_mfma_kernel<Q>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return;                            \
     hipLaunchKernelGGL((moe_down_mfma_kernel<Q>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
                        groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg)
     if (down_quant == kQ6K) {

@@ -5,6 +5,7 @@
 #include <cstring>
 
 #include "../../include/rnb_hip.h"
+#include "kernels.h"
 
 namespace rnb {
 
@@ -39,16 +40,49 @@ uint64_t fingerprint(const uint8_t *p, size_t len) {
 }
 }  // namespace
 
+namespace {
+thread_local std::string t_launch_failure;
+}
+
+bool allow_dynamic_lds(const void *kernel, size_t bytes, bool *done, const char *kernel_name) {
+    if (*done) return true;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        t_launch_failure = std::string(kernel_name) + ": hipFuncSetAttribute(max dynamic LDS = " + std::to_string(bytes) +
+                           "): " + hipGetErrorString(e);
+        return false;
+    }
+    *done = true;
+    return true;
+}
+
+std::string take_launch_failure() {
+    std::string out;
+    out.swap(t_launch_failure);
+    return out;
+}
+
 void set_last_error(const std::string &msg) { t_last_error = msg; }
 const char *last_error_cstr() { return t_last_error.c_str(); }
 
 hipError_t DeviceBuf::reserve(size_t bytes) {
     if (bytes <= cap) return hipSuccess;
+    State *s = g_state;
+    if (s != nullptr && s->capturing()) return hipErrorStreamCaptureUnsupported;
     if (ptr) {
-        hipError_t e = hipFree(ptr);
+        if (s != nullptr && s->capture_seen) {
+            s->retired.push_back(ptr);  // a graph instantiated earlier may replay with this address
+        } else {
+            hipError_t e = hipFree(ptr);
+            if (e != hipSuccess) {
+                ptr = nullptr;
+                cap = 0;
+                return e;
+            }
+        }
         ptr = nullptr;
         cap = 0;
-        if (e != hipSuccess) return e;
     }
     const size_t want = round_up(bytes + bytes / 4, 4096);
     hipError_t e = hipMalloc(&ptr, want);
@@ -58,6 +92,16 @@ hipError_t DeviceBuf::reserve(size_t bytes) {
     }
     cap = want;
     return hipSuccess;
+}
+
+bool State::capturing() {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (st != hipStreamCaptureStatusNone) capture_seen = true;
+    return st != hipStreamCaptureStatusNone;
 }
 
 hipError_t PinnedBuf::reserve(size_t bytes) {
@@ -78,95 +122,62 @@ hipError_t PinnedBuf::reserve(size_t bytes) {
     return hipSuccess;
 }
 
-void State::evict_unpinned_until(uint64_t need) {
-    // least-recently-used first (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:789-823)
-    while (resident_bytes + need > resident_budget) {
-        auto victim = residents.end();
-        for (auto it = residents.begin(); it != residents.end(); ++it)
-            if (!it->second.pinned && (victim == residents.end() || it->second.epoch < victim->second.epoch)) victim = it;
-        if (victim == residents.end()) return;
-        (void)hipStreamSynchronize(stream);
-        (void)hipFree(victim->second.dev);
-        resident_bytes -= victim->second.len;
-        residents.erase(victim);
-    }
-}
-
-hipError_t State::resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out, bool pin) {
-    const uintptr_t key = reinterpret_cast<uintptr_t>(ptr);
-    ++epoch;
-    auto it = residents.find(key);
-    if (it != residents.end() && it->second.len == len) {
-        if (it->second.fingerprint == fingerprint(ptr, len)) {
-            it->second.epoch = epoch;
-            it->second.pinned = it->second.pinned || pin;
-            *dev_out = static_cast<const uint8_t *>(it->second.dev);
-            return hipSuccess;
-        }
-        // same address and length, different bytes: the host range was reused
-        resident_bytes -= it->second.len;
-        (void)hipStreamSynchronize(stream);
-        (void)hipFree(it->second.dev);
-        residents.erase(it);
-    } else if (!pin) {
-        // sub-range of a pinned parent slab (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:722-741).
-        // Unpinned entries never serve sub-ranges: their host memory may have been freed and reused.
-        auto up = residents.upper_bound(key);
-        while (up != residents.begin()) {
-            --up;
-            const uintptr_t base = up->first;
-            if (up->second.pinned && key >= base && key + len <= base + up->second.len) {
-                up->second.epoch = epoch;
-                *dev_out = static_cast<const uint8_t *>(up->second.dev) + (key - base);
-                return hipSuccess;
-            }
-        }
-    }
-    // an entry that starts at this address with another length is stale
-    it = residents.find(key);
-    if (it != residents.end()) {
-        resident_bytes -= it->second.len;
-        (void)hipStreamSynchronize(stream);
-        (void)hipFree(it->second.dev);
-        residents.erase(it);
-    }
-    evict_unpinned_until(len);
-    void *dev = nullptr;
-    hipError_t e = hipMalloc(&dev, round_up(len, 256) + 256);
-    if (e != hipSuccess) {
+namespace {
+// hipMalloc / hipFree / blocking upload on the state's stream, for the resident table
+class HipAllocator final : public DeviceAllocator {
+  public:
+    explicit HipAllocator(State *s) : s_(s) {}
+    int alloc(size_t bytes, void **out, std::string *err) override {
+        hipError_t e = hipMalloc(out, round_up(bytes, 256) + 256);
+        if (e == hipSuccess) return 0;
         (void)hipGetLastError();
-        resident_budget = resident_bytes;  // out of memory: shrink the budget to what fits and retry once
-        evict_unpinned_until(len);
-        e = hipMalloc(&dev, round_up(len, 256) + 256);
-        if (e != hipSuccess) return e;
+        *err = std::string("hipMalloc of ") + std::to_string(bytes) + " bytes: " + hipGetErrorString(e);
+        return e == hipErrorOutOfMemory ? 1 : 2;
     }
-    e = hipMemcpyAsync(dev, ptr, len, hipMemcpyHostToDevice, stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) {
-        (void)hipFree(dev);
-        return e;
+    int free(void *ptr, std::string *err) override {
+        // kernels of earlier calls may still read the range
+        hipError_t e = hipStreamSynchronize(s_->stream);
+        if (e == hipSuccess) e = hipFree(ptr);
+        if (e == hipSuccess) return 0;
+        *err = std::string("hipFree: ") + hipGetErrorString(e);
+        return 2;
     }
-    h2d_bytes += len;
-    Resident r;
-    r.len = len;
-    r.dev = dev;
-    r.fingerprint = fingerprint(ptr, len);
-    r.epoch = epoch;
-    r.pinned = pin;
-    residents[key] = r;
-    resident_bytes += len;
-    *dev_out = static_cast<const uint8_t *>(dev);
-    return hipSuccess;
+    int upload(void *dst, const void *src, size_t bytes, std::string *err) override {
+        hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s_->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(s_->stream);
+        if (e == hipSuccess) return 0;
+        *err = std::string("weight upload: ") + hipGetErrorString(e);
+        return 2;
+    }
+
+  private:
+    State *s_;
+};
+}  // namespace
+
+int State::resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out, bool pin) {
+    if (capturing()) {
+        set_last_error("host-pointer weights cannot be resolved while the library stream is capturing");
+        return RNB_HIP_INVALID_REQUEST;
+    }
+    std::string err;
+    const int rc = table->resolve(ptr, len, fingerprint(ptr, len), pin, dev_out, &err);
+    if (rc == 0) return RNB_HIP_OK;
+    set_last_error(err);
+    return RNB_HIP_EXECUTION_FAILED;
 }
 
 bool State::release(const uint8_t *ptr, size_t len) {
-    auto it = residents.find(reinterpret_cast<uintptr_t>(ptr));
-    if (it == residents.end() || it->second.len != len) return false;
-    (void)hipStreamSynchronize(stream);
-    (void)hipFree(it->second.dev);
-    resident_bytes -= it->second.len;
-    residents.erase(it);
-    return true;
+    std::string err;
+    return table->release(ptr, len, &err);
+}
+
+Guard::~Guard() {
+    if (state != nullptr && state->table->has_call_temps()) {
+        (void)hipStreamSynchronize(state->stream);
+        std::string err;
+        (void)state->table->end_call(&err);
+    }
 }
 
 Guard::Guard() : lock(g_mutex) {
@@ -177,7 +188,9 @@ Guard::Guard() : lock(g_mutex) {
             set_last_error(std::string("hipSetDevice: ") + hipGetErrorString(e));
             status = RNB_HIP_EXECUTION_FAILED;
             state = nullptr;
+            return;
         }
+        state->table->begin_call();
         return;
     }
     if (g_open_status > 0) {  // an earlier open failed; report the same thing without retrying
@@ -230,13 +243,16 @@ Guard::Guard() : lock(g_mutex) {
         fail(RNB_HIP_EXECUTION_FAILED, std::string("hipStreamCreate: ") + hipGetErrorString(e));
         return;
     }
+    s->allocator.reset(new HipAllocator(s));
+    s->table.reset(new ResidentTable(s->allocator.get()));
     // resident weights may take 85% of what is free now unless RNB_HIP_RESIDENT_BUDGET_MB says otherwise
     size_t free_b = 0, total_b = 0;
-    if (hipMemGetInfo(&free_b, &total_b) == hipSuccess) s->resident_budget = free_b / 100 * 85;
-    if (const char *env = std::getenv("RNB_HIP_RESIDENT_BUDGET_MB")) s->resident_budget = std::strtoull(env, nullptr, 10) << 20;
+    if (hipMemGetInfo(&free_b, &total_b) == hipSuccess) s->table->set_budget(free_b / 100 * 85);
+    if (const char *env = std::getenv("RNB_HIP_RESIDENT_BUDGET_MB")) s->table->set_budget(std::strtoull(env, nullptr, 10) << 20);
     g_state = s;
     g_open_status = 0;
     state = s;
+    s->table->begin_call();
 }
 
 }  // namespace rnb

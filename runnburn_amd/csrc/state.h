@@ -8,18 +8,26 @@
 #include <stdint.h>
 
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
+#include <vector>
+
+#include "residency.h"
 
 namespace rnb {
 
 void set_last_error(const std::string &msg);
 const char *last_error_cstr();
 
-// Grow-only device allocation (reference: compute_*_ptr slots, state/buffers.rs:68-310).
+// Grow-only device allocation (reference: compute_*_ptr slots, state/buffers.rs:68-310).  Growing replaces the
+// allocation; the old one is freed at once unless a stream capture has ever been seen on the library stream, in
+// which case an instantiated graph may still hold its address and it is kept until the process ends (`retired`).
+// While the stream is capturing, growth is refused: an allocation has no place inside a graph.
 struct DeviceBuf {
     void *ptr = nullptr;
     size_t cap = 0;
+    // hipErrorStreamCaptureUnsupported when the stream is capturing and the buffer would have to grow
     hipError_t reserve(size_t bytes);
     template <typename T>
     T *as() const { return static_cast<T *>(ptr); }
@@ -31,14 +39,6 @@ struct PinnedBuf {
     hipError_t reserve(size_t bytes);
     template <typename T>
     T *as() const { return static_cast<T *>(ptr); }
-};
-
-struct Resident {
-    size_t len = 0;
-    void *dev = nullptr;
-    uint64_t fingerprint = 0;
-    uint64_t epoch = 0;   // last use, for least-recently-used eviction
-    bool pinned = false;  // prewarmed: never evicted, and the only kind a sub-range may resolve to
 };
 
 struct TableSlot {
@@ -68,22 +68,23 @@ struct State {
     TableSlot table_ring[kTableRing];  // MoE routing tables too large for a kernel argument
     int table_ring_next = 0;
 
-    std::map<uintptr_t, Resident> residents;  // keyed by host base address
+    std::unique_ptr<DeviceAllocator> allocator;
+    std::unique_ptr<ResidentTable> table;  // resident weights: (host range) -> device copy, budget, eviction, admission
     // what the activation scratch currently holds (set by quantize_activations)
     uint32_t act_family = 0;  // 8 = 32-wide Q8, 12 = Q8_K
     size_t act_seq = 0, act_cols = 0;
 
-    uint64_t resident_bytes = 0;
-    uint64_t resident_budget = 0;  // bytes of unpinned + pinned residents before unpinned ones are evicted
-    uint64_t epoch = 0;
-    uint64_t h2d_bytes = 0, d2h_bytes = 0;
+    uint64_t h2d_bytes = 0, d2h_bytes = 0;  // activations, outputs, tables (weights are counted by the table)
+    bool capture_seen = false;              // a stream capture was observed: scratch that is replaced is retired, not freed
+    std::vector<void *> retired;
 
-    // Returns the device address of [ptr, ptr+len): an exact resident match (same address, length
-    // and fingerprint), a sub-range of a pinned (prewarmed) parent, or a fresh untouched upload
-    // that becomes resident.  `pin` marks the entry as prewarmed.
-    hipError_t resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out, bool pin = false);
-    void evict_unpinned_until(uint64_t need);
+    // Device address of [ptr, ptr+len) through the resident table (residency.h): an exact resident match, a sub-range
+    // of a pinned (prewarmed) parent, a fresh untouched upload that becomes resident, or an upload for this call only.
+    // Returns an rnb_hip_status with the message set.
+    int resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out, bool pin = false);
     bool release(const uint8_t *ptr, size_t len);
+    // true while the library stream is capturing into a graph (also remembers that a capture happened)
+    bool capturing();
 };
 
 // Locks the global mutex and opens the device on first use.  On failure returns a status
@@ -93,6 +94,7 @@ struct Guard {
     State *state = nullptr;
     int status = 0;
     Guard();
+    ~Guard();  // frees the weight uploads that were made for this call only (after the stream has drained)
 };
 
 }  // namespace rnb

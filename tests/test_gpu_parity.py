@@ -61,6 +61,13 @@ def _q8k_inputs(oracle):
     cases["tiny_and_huge"] = np.concatenate([rng.standard_normal(256).astype(np.float32) * np.float32(1e-30),
                                              rng.standard_normal(256).astype(np.float32) * np.float32(1e30)])
     cases["half_integers"] = (rng.integers(-254, 255, 2048).astype(np.float32) * np.float32(0.5))
+    nf = np.zeros(4 * 256, np.float32)                        # NaN and infinity: see test_quantisers_on_non_finite_inputs
+    nf[0:256] = np.nan
+    nf[256:512] = np.linspace(-1.0, 1.0, 256, dtype=np.float32)
+    nf[256 + 17] = np.nan
+    nf[512 + 3], nf[512 + 4] = np.inf, 5.0
+    nf[768 + 9], nf[768 + 200] = -np.inf, np.nan
+    cases["non_finite"] = nf
     return cases
 
 
@@ -82,6 +89,12 @@ def test_q8_activation_quantiser_bit_exact(rnb, oracle):
     xs = [oracle.fill_normal(4096, 2, 1.0), np.zeros(64, np.float32),
           rng.integers(-254, 255, 32 * 9).astype(np.float32) * np.float32(0.5),   # 9 blocks: ragged last wave
           rng.standard_normal(32 * 64 * 5 + 32).astype(np.float32) * np.float32(1e-20)]
+    nf = np.zeros(3 * 32, np.float32)  # a NaN among finite values, an infinite block, a block of NaNs
+    nf[0:32] = np.arange(32, dtype=np.float32) - 16.0
+    nf[5] = np.nan
+    nf[32 + 1], nf[32 + 2] = np.inf, 7.0
+    nf[64:96] = np.nan
+    xs.append(nf)
     for x in xs:
         got, want = rnb.quantize_input_q8(x), oracle.quantize_q8(x)
         assert np.array_equal(got["d"].view(np.uint32), want["d"].view(np.uint32))
@@ -946,4 +959,59 @@ def test_graph_replay_matches_eager(rnb, quant, rows, cols, seq):
         hip.rt.hipGraphExecDestroy(gexec)
         hip.rt.hipGraphDestroy(graph)
         for b in (w, x_dev, out_dev):
+            b.free()
+
+
+def test_graph_survives_scratch_growth_and_capture_refuses_growth(rnb):
+    """A graph captured on a small shape keeps the scratch addresses of that moment.  A later, larger eager call grows
+    the scratch: the replaced allocation is retired, not freed, once a capture has been seen, so the graph's replay
+    still reads and writes live memory and gives the eager bits.  A capture whose call would itself have to grow the
+    scratch is refused with a message, as is a host-pointer call (it would upload weights and synchronise); the
+    no-allocation entry point captures without a warm-up."""
+    import ctypes as C
+    import bench
+    hip = bench.Hip()
+    lib = rnb.lib()
+    stream = C.c_void_p(rnb.stream_handle())
+    rng = np.random.default_rng(77)
+    rows, cols, seq = 384, 1024, 6
+    w = rnb.DeviceBuffer.from_host(bench.synth_weights(Q4_K, rows, cols, 78))
+    x = rng.standard_normal(seq * cols).astype(np.float32)
+    x_dev, out_dev = rnb.DeviceBuffer.from_host(x), rnb.DeviceBuffer(seq * rows * 4)
+    rnb.gemv_dev(Q4_K, w, rows, cols, x_dev, seq, out_dev)  # eager: sizes the scratch for this shape
+    want = out_dev.to_host(np.float32)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.check(hip.rt.hipStreamBeginCapture(stream, 2), "hipStreamBeginCapture")
+    try:
+        rnb.gemv_dev(Q4_K, w, rows, cols, x_dev, seq, out_dev)
+        # while capturing: a shape that needs more scratch than there is, and a host-pointer call, are refused
+        big_seq = 4096
+        xb, ob = rnb.DeviceBuffer(big_seq * cols * 4), rnb.DeviceBuffer(big_seq * rows * 4)
+        with pytest.raises(rnb.BackendError) as err:
+            rnb.gemv_dev(Q4_K, w, rows, cols, xb, big_seq, ob)
+        assert err.value.kind == "InvalidRequest" and "capturing" in str(err.value)
+        # the no-allocation form of the same call is captured
+        out2 = rnb.DeviceBuffer(seq * rows * 4)
+        rnb.gemv_dev_noalloc(Q4_K, w, rows, cols, x_dev, seq, out2)
+    finally:
+        rc = hip.rt.hipStreamEndCapture(stream, C.byref(graph))
+    hip.check(rc, "hipStreamEndCapture")
+    hip.check(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0), "hipGraphInstantiate")
+    try:
+        # a larger eager call grows every scratch buffer the graph's nodes point into
+        rnb.gemv_dev(Q4_K, w, rows, cols, xb, big_seq, ob)
+        rnb.sync()
+        for _ in range(3):
+            assert lib.rnb_hip_dev_upload(out_dev.ptr, np.zeros(seq * rows, np.float32).ctypes.data_as(C.c_void_p),
+                                          seq * rows * 4) == 0
+            hip.check(hip.rt.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            rnb.sync()
+            assert np.array_equal(out_dev.to_host(np.float32), want)
+            assert np.array_equal(out2.to_host(np.float32), want)
+            rnb.gemv_dev(Q4_K, w, rows, cols, xb, big_seq, ob)  # eager work between the replays
+            rnb.sync()
+    finally:
+        hip.rt.hipGraphExecDestroy(gexec)
+        hip.rt.hipGraphDestroy(graph)
+        for b in (w, x_dev, out_dev, xb, ob, out2):
             b.free()

@@ -406,6 +406,43 @@ def test_q8_activation_quantiser(oracle):
     assert np.array_equal(got["qs"], qs)
 
 
+def test_quantisers_on_non_finite_inputs(oracle):
+    """What the Rust does with NaN and infinity, stated by hand from the source.  Q8_K
+    (crates/rnb-cpu/src/gemm/activation_q8.rs:149-173): `ax > amax` is false for NaN, so a NaN never becomes the
+    maximum and a block of NaNs returns the zero block; `(iscale * NaN).round_ties_even() as i32` is 0.  An infinite
+    maximum gives iscale = -127/inf = -0.0 and d = 1/-0.0 = -inf; every product is +-0 or NaN, every code 0.  Q8
+    (:14-32): f32::max ignores a NaN operand, `NaN.clamp(-128, 127) as i8` is 0; an infinite maximum gives d = inf,
+    id = 0 and inf * 0 = NaN."""
+    nan, inf = np.float32(np.nan), np.float32(np.inf)
+    x = np.zeros(4 * 256, np.float32)
+    x[0:256] = nan                                    # block 0: all NaN
+    x[256:512] = np.linspace(-1.0, 1.0, 256, dtype=np.float32)
+    clean = oracle.quantize_q8k(x[256:512].copy())[0]
+    x[256 + 17] = nan                                 # block 1: one NaN among finite values
+    x[512 + 3], x[512 + 4] = inf, 5.0                 # block 2: +inf
+    x[768 + 9], x[768 + 200] = -inf, nan              # block 3: -inf and a NaN
+    b = oracle.quantize_q8k(x)
+    assert b["d"][0] == 0.0 and not b["qs"][0].any() and not b["bsums"][0].any()
+    want = clean["qs"].copy()
+    want[17] = 0
+    assert b["d"][1].view(np.uint32) == clean["d"].view(np.uint32) and np.array_equal(b["qs"][1], want)
+    assert np.array_equal(b["bsums"][1], want.astype(np.int16).reshape(16, 16).sum(axis=1))
+    assert b["d"][2] == -inf and not b["qs"][2].any()
+    assert b["d"][3] == inf and not b["qs"][3].any()   # max_val = -inf: iscale = +0.0, d = +inf
+    y = np.zeros(3 * 32, np.float32)
+    y[0:32] = np.arange(32, dtype=np.float32) - 16.0
+    ref = oracle.quantize_q8(y[0:32].copy())[0]
+    y[5] = nan
+    y[32 + 1], y[32 + 2] = inf, 7.0
+    y[64:96] = nan
+    q = oracle.quantize_q8(y)
+    want = ref["qs"].copy()
+    want[5] = 0
+    assert q["d"][0].view(np.uint32) == ref["d"].view(np.uint32) and np.array_equal(q["qs"][0], want)
+    assert q["d"][1] == inf and not q["qs"][1].any()
+    assert q["d"][2] == 0.0 and not q["qs"][2].any()
+
+
 # ---- Q4_K x Q8_K dot ------------------------------------------------------------------
 
 def _act_from_parts(d, qs, bsums=None):
