@@ -12,11 +12,15 @@ weights of every step come from HBM.
 
 Prints ONE JSON line on stdout (progress goes to stderr):
   value      whole-job GB/s = algorithmic bytes per step * K / wall time of K steps
-  roofline   that kernel: algorithmic bytes per launch / mean kernel duration measured with HIP events on the
-             library's stream, against the 8 TB/s HBM peak (the GEMV over an already quantised token beside it)
+  roofline   that kernel: algorithmic bytes per launch / mean kernel duration, against the 8 TB/s HBM peak.  Kernel
+             times come from HIP events on the library's stream over 200 launches after 20 warm-ups, whatever --steps
+             says: mean over all of them, median / p10 / p90 over batches of 10.  `read_ceiling` is what a kernel that
+             only reads the same bytes reaches in the same run (context; the peak stays 8 TB/s).
+  roofline_gemm  the metric's second half: the Q4_K prefill GEMM (512 tokens) against the 5 POP/s int8 peak, with what a
+             kernel of int8 matrix instructions alone reaches in the same run beside it
   cpu_baseline  the CPU restatement of rnb-cpu's x86 path (oracle/, AVX2+FMA, row-chunk threads) timed on
-             the host cores on the same workload
-  secondary  the other BASELINE configs (kernel-level, same protocol), Q4_K prefill GEMM in TOP/s
+             the host cores on the same workload; cpu_baseline_gemm and cpu_baseline_moe for the GEMM and MoE configs
+  secondary  the other BASELINE configs (same protocol; `step` = everything one call enqueues)
 """
 from __future__ import annotations
 
@@ -184,10 +188,35 @@ class Hip:
         return float(ms.value)
 
 
+KERNEL_LAUNCHES, KERNEL_WARMUPS, KERNEL_BATCH = 200, 20, 10
+
+
+def kernel_stats(hip, stream, launch, launches=KERNEL_LAUNCHES, warmups=KERNEL_WARMUPS, batch=KERNEL_BATCH):
+    """Duration of `launch(i)` in ms from HIP events recorded on the stream the kernels run on: `warmups` untimed
+    launches, then `launches` back-to-back ones with an event after every `batch` of them (same-stream launches
+    serialise, so a batch's elapsed time / batch is the kernel duration plus the inter-launch gap).  mean = first to
+    last event over all launches; median, p10 and p90 are taken over the batches."""
+    for i in range(warmups):
+        launch(i)
+    n_batches = max(1, launches // batch)
+    events = [hip.event() for _ in range(n_batches + 1)]
+    hip.record(events[0], stream)
+    k = 0
+    for b in range(n_batches):
+        for _ in range(batch):
+            launch(k)
+            k += 1
+        hip.record(events[b + 1], stream)
+    total = hip.elapsed_ms(events[0], events[-1])
+    per = np.array([hip.elapsed_ms(events[b], events[b + 1]) / batch for b in range(n_batches)])
+    for ev in events:
+        hip.rt.hipEventDestroy(ev)
+    return {"mean": total / (n_batches * batch), "median": float(np.median(per)), "p10": float(np.percentile(per, 10)),
+            "p90": float(np.percentile(per, 90)), "launches": n_batches * batch, "warmups": warmups, "batch": batch}
+
+
 def kernel_time_ms(hip, stream, launch, n):
-    """Mean duration of `launch(i)` over n back-to-back launches: one HIP event before the first and one
-    after the last, both recorded on the stream the kernel runs on (same-stream launches serialise, so
-    elapsed / n is the kernel duration plus the inter-launch gap)."""
+    """Mean duration of `launch(i)` over n back-to-back launches (one event before, one after)."""
     e0, e1 = hip.event(), hip.event()
     hip.record(e0, stream)
     for i in range(n):
@@ -197,6 +226,35 @@ def kernel_time_ms(hip, stream, launch, n):
     hip.rt.hipEventDestroy(e0)
     hip.rt.hipEventDestroy(e1)
     return ms / n
+
+
+def read_ceiling(hip, rnb, stream, nbytes):
+    """What a read-only kernel reaches on `nbytes` in this run (plain and non-temporal 16-byte loads), rotating over
+    enough buffers to miss the 256 MiB Infinity Cache: context for the HBM-bound rows, not a peak."""
+    n = copies_for(nbytes)
+    bufs = [rnb.DeviceBuffer(nbytes) for _ in range(n)]
+    out = {"bytes": nbytes, "copies": n}
+    for label, nt in (("plain", False), ("non_temporal", True)):
+        st = kernel_stats(hip, stream, lambda i: rnb.calib_read(bufs[i % n], nbytes, nt))
+        out[label] = {"ms_median": st["median"], "ms_p10": st["p10"], "ms_p90": st["p90"], "GB/s": nbytes / st["median"] / 1e6}
+    for b in bufs:
+        b.free()
+    out["GB/s"] = max(out["plain"]["GB/s"], out["non_temporal"]["GB/s"])
+    out["frac_of_peak"] = out["GB/s"] / HBM_PEAK_GBPS
+    return out
+
+
+def mfma_ceiling(hip, rnb, stream):
+    """What a kernel of int8 matrix instructions alone (registers only, 2 waves per SIMD on every compute unit) reaches in
+    this run: the part's clock under matrix load decides it.  Context for the GEMM row, not a peak."""
+    ops = [0]
+
+    def launch(_i):
+        ops[0] = rnb.calib_mfma_i8(2000, 256)
+
+    st = kernel_stats(hip, stream, launch, launches=40, warmups=5, batch=5)
+    return {"ops_per_launch": ops[0], "ms_median": st["median"], "TOP/s": ops[0] / st["median"] / 1e9,
+            "frac_of_peak": ops[0] / st["median"] / 1e9 / INT8_PEAK_TOPS}
 
 
 def calibration_copy(hip, rnb, stream, nbytes=64 << 20, reps=5):
@@ -287,8 +345,18 @@ def copies_for(nbytes):
     return max(2, -(-2 * MALL_BYTES // nbytes))
 
 
+def one_launch_step(quant, rows, cols, seq):
+    """True when the library runs the whole step (token quantisation + GEMV) as one kernel."""
+    if seq != 1:
+        return False
+    if quant in (10, 11, Q4_K, Q5_K, Q6_K):
+        nb = cols // 256
+        return nb <= 16 and (nb <= 8 or rows * nb * BLOCK_BYTES.get(quant, 144) < (190 << 20))
+    return cols // 32 <= 128 and rows * (cols // 32) >= 1 << 18
+
+
 def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, name, want_graph=True,
-                 cache_resident=False):
+                 cache_resident=False, want_wall=True):
     w_host = synth_weights(quant, rows, cols, seed)
     n_copies = copies_for(w_host.nbytes)
     log(f"[{name}] weights {w_host.nbytes / 1e6:.1f} MB x {n_copies} device copies")
@@ -300,10 +368,12 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
     def step(i):
         rnb.gemv_dev(quant, w_dev[i % n_copies], rows, cols, x_dev, seq, out_dev)
 
-    for i in range(warmup):
-        step(i)
-    wall_ms = wall_steps(rnb, step, steps)
-    res = {"wall_ms_per_step": wall_ms / steps, "launch": "stream"}
+    res = {"launch": "stream"}
+    if want_wall:
+        for i in range(warmup):
+            step(i)
+        wall_ms = wall_steps(rnb, step, steps)
+        res["wall_ms_per_step"] = wall_ms / steps
     if want_graph:
         try:
             per = n_copies if steps >= n_copies else steps
@@ -312,28 +382,21 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
             res["graph_ms_per_step"] = g_ms / (per * reps)
         except Exception as exc:  # keep the stream number if capture is unavailable
             log(f"[{name}] graph replay unavailable: {exc}")
+    # the step as the library enqueues it (one launch, or activation quantiser + GEMV / GEMM [+ slice sum])
+    res["step"] = kernel_stats(hip, stream, step)
+    res["one_launch_step"] = one_launch_step(quant, rows, cols, seq)
+    # the GEMV / GEMM alone over an already quantised activation
     rnb.quantize_dev(quant, x_dev, seq, cols)
-    n_k = min(steps, 1000)
-    launch = lambda i: rnb.gemv_quantized_dev(quant, w_dev[i % n_copies], rows, cols, seq, out_dev)  # noqa: E731
-    for i in range(min(20, n_k)):
-        launch(i)
-    reps = [kernel_time_ms(hip, stream, launch, n_k) for _ in range(3)]
-    # One token against K-quant rows of at most 16 super-blocks is ONE launch in the library (the GEMV's workgroups
-    # quantise the token themselves): that kernel is the step, so it is the one the roofline is quoted on; the GEMV
-    # over an already quantised token is kept beside it.
-    res["one_launch_step"] = seq == 1 and ((quant in (10, 11, Q4_K, Q5_K, Q6_K) and cols // 256 <= 16) or
-                                           (quant in (2, 3, 6, 7, Q8_0) and cols // 32 <= 128 and rows * (cols // 32) >= 1 << 18))
-    if res["one_launch_step"]:
-        res["prequantised_kernel_ms_mean"] = float(np.mean(reps))
-        reps = [kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]
-    res["kernel_ms_mean"] = float(np.mean(reps))
-    res["kernel_ms_runs"] = [float(v) for v in reps]
+    res["prequantised"] = kernel_stats(
+        hip, stream, lambda i: rnb.gemv_quantized_dev(quant, w_dev[i % n_copies], rows, cols, seq, out_dev))
     if cache_resident:
         # one copy only: the weights may stay in the 256 MiB Infinity Cache; labelled, never `value`
-        one = lambda i: rnb.gemv_quantized_dev(quant, w_dev[0], rows, cols, seq, out_dev)  # noqa: E731
-        res["kernel_ms_mean_cache_resident"] = kernel_time_ms(hip, stream, one, min(steps, 300))
+        res["cache_resident"] = kernel_stats(hip, stream,
+                                             lambda i: rnb.gemv_quantized_dev(quant, w_dev[0], rows, cols, seq, out_dev))
     res["bytes"] = gemv_bytes(quant, rows, cols, seq)
     res["copies"] = n_copies
+    step(0)
+    rnb.sync()
     out = out_dev.to_host(np.float32)
     for b in w_dev:
         b.free()
@@ -342,31 +405,41 @@ def bench_matmul(rnb, hip, stream, quant, rows, cols, seq, steps, warmup, seed, 
     return res, w_host, x, out
 
 
+def _cpu_threads():
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    return min(threads, os.cpu_count() or threads)
+
+
+def _matches(gpu, ref):
+    e = np.asarray(ref, np.float64).ravel()
+    g = np.asarray(gpu, np.float64).ravel()
+    tol = np.maximum(1e-3 * np.sqrt(np.mean(e * e)), 1e-3 * np.abs(e))
+    return bool(np.all(np.isfinite(g)) and np.all(np.abs(g - e) <= tol))
+
+
 def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=10.0):
     """The CPU leg: rnb-cpu's x86 path restated in oracle/ (AVX2+FMA dots, contiguous row chunks per
     thread), timed on this host; also checks the GPU result against it (abs-or-rel 1e-3)."""
     from oracle import oracle as ora
 
     ora.lib()
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
-    threads = min(threads, os.cpu_count() or threads)
-    fn = (lambda: ora.gemv(quant, w_host, rows, cols, x, avx2=True, n_threads=threads)) if ora.have_avx2() else \
-        (lambda: ora.gemv(quant, w_host, rows, cols, x, n_threads=threads))
-    ref = fn()
-    for _ in range(2):
-        fn()
-    # cache-resident figure first (one copy of the weights, a few hundred passes) ...
-    hot, t_start = [], time.perf_counter()
-    while len(hot) < 200 and time.perf_counter() - t_start < 2.0:
-        t0 = time.perf_counter()
-        fn()
-        hot.append(time.perf_counter() - t0)
-    # ... then the figure that is reported: the weights rotate over copies totalling more than the host's last-level
-    # caches, as the GPU leg rotates over more than the Infinity Cache, for about `budget_s` seconds of CPU work
+    threads = _cpu_threads()
+    avx2 = ora.have_avx2()
+    run = lambda w: ora.gemv(quant, w, rows, cols, x, avx2=avx2, n_threads=threads)  # noqa: E731
+    ref = run(w_host)
+    # the scalar restatement on one thread, a few passes: sanity figure beside the threaded one
+    t0 = time.perf_counter()
+    n_scalar = 0
+    while time.perf_counter() - t0 < 1.5:
+        ora.gemv(quant, w_host, rows, cols, x, n_threads=1)
+        n_scalar += 1
+    scalar_ms = (time.perf_counter() - t0) / n_scalar * 1e3
+    # the figure that is reported: the weights rotate over copies totalling more than the host's last-level caches,
+    # as the GPU leg rotates over more than the Infinity Cache, for about `budget_s` seconds of CPU work
     n_copies = max(2, -(-(1 << 30) // max(1, w_host.nbytes)))
     copies = [w_host] + [w_host.copy() for _ in range(n_copies - 1)]
-    run = (lambda w: ora.gemv(quant, w, rows, cols, x, avx2=True, n_threads=threads)) if ora.have_avx2() else \
-        (lambda w: ora.gemv(quant, w, rows, cols, x, n_threads=threads))
+    for i in range(n_copies):  # thread pool and clocks warm before anything is timed
+        run(copies[i])
     times, t_start, i = [], time.perf_counter(), 0
     while time.perf_counter() - t_start < budget_s:
         t0 = time.perf_counter()
@@ -374,18 +447,50 @@ def cpu_baseline_gemv(quant, w_host, rows, cols, x, gpu_out, budget_s=10.0):
         times.append(time.perf_counter() - t0)
         i += 1
     med = float(np.median(times))
-    e = np.asarray(ref, np.float64).ravel()
-    g = np.asarray(gpu_out, np.float64).ravel()
-    tol = np.maximum(1e-3 * np.sqrt(np.mean(e * e)), 1e-3 * np.abs(e))
-    ok = bool(np.all(np.abs(g - e) <= tol))
-    return {"value": gemv_bytes(quant, rows, cols, x.size // cols) / med / 1e9, "unit": "GB/s", "cores": threads,
-            "kind": "port",
+    # one copy only, after the rotating loop (same warm threads): whatever the host caches keep of 33 MB
+    single = []
+    t_start = time.perf_counter()
+    while len(single) < 200 and time.perf_counter() - t_start < 2.0:
+        t0 = time.perf_counter()
+        run(w_host)
+        single.append(time.perf_counter() - t0)
+    nbytes = gemv_bytes(quant, rows, cols, x.size // cols)
+    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{len(times)} full passes of the same {rows}x{cols} GEMV over {n_copies} rotating weight copies "
                       f"({n_copies * w_host.nbytes / 1e6:.0f} MB, ~{budget_s:.0f} s of wall time), median per pass",
-            "ms": med * 1e3, "cache_resident_GB/s": gemv_bytes(quant, rows, cols, x.size // cols) / float(np.median(hot)) / 1e9, "isa": "avx2+fma" if ora.have_avx2() else "scalar", "gpu_matches_cpu": ok}
+            "ms": med * 1e3, "single_copy_GB/s": nbytes / float(np.median(single)) / 1e9,
+            "scalar_1_thread_ms": scalar_ms, "scalar_1_thread_GB/s": nbytes / scalar_ms / 1e6,
+            "isa": "avx2+fma" if avx2 else "scalar", "gpu_matches_cpu": _matches(gpu_out, ref),
+            "note": "restatement of rnb-cpu's x86 path (Rust toolchain unavailable); a baseline, not a target"}
 
 
-def bench_moe(rnb, hip, stream, tokens, steps, seed):
+def cpu_baseline_gemm(w_host, rows, cols, x, gpu_out, sample_tokens=64, budget_s=12.0):
+    """cfg4 on the CPU: the batch driver of crates/rnb-cpu/src/gemm/quant_gemv.rs:1127-1196 restated (rows chunked over
+    threads, every row against every token), on the first `sample_tokens` of the 512 tokens; checks those tokens of the
+    GPU result."""
+    from oracle import oracle as ora
+
+    ora.lib()
+    threads = _cpu_threads()
+    avx2 = ora.have_avx2()
+    xs = np.ascontiguousarray(x[:sample_tokens * cols])
+    run = lambda: ora.gemv(Q4_K, w_host, rows, cols, xs, avx2=avx2, n_threads=threads)  # noqa: E731
+    ref = run()
+    times, t_start = [], time.perf_counter()
+    while time.perf_counter() - t_start < budget_s and len(times) < 50:
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    ops = 2 * sample_tokens * rows * cols
+    got = np.asarray(gpu_out, np.float32).reshape(-1, rows)[:sample_tokens]
+    return {"value": ops / med / 1e12, "unit": "TOP/s", "cores": threads, "kind": "port",
+            "sample": f"{len(times)} passes over the first {sample_tokens} of the 512 tokens against all {rows} rows "
+                      f"(an eighth of the workload per pass), median per pass", "ms": med * 1e3,
+            "isa": "avx2+fma" if avx2 else "scalar", "gpu_matches_cpu": _matches(got, ref)}
+
+
+def bench_moe(rnb, hip, stream, tokens, steps, seed, cpu=True):
     n_expert, n_ff, n_embd, k = 128, 768, 2048, 8
     gen = 16  # distinct experts generated; tiled to 128 (addresses differ)
     per_gate = n_ff * (n_embd // 256) * 144
@@ -395,7 +500,8 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed):
     d = np.tile(synth_weights(Q6_K, gen * n_embd, n_ff, seed + 2), n_expert // gen)
     gd, ud, dd = (rnb.DeviceBuffer.from_host(a) for a in (g, u, d))
     rng = np.random.default_rng(seed + 3)
-    x_dev = rnb.DeviceBuffer.from_host(rng.standard_normal(tokens * n_embd).astype(np.float32))
+    x_host = rng.standard_normal(tokens * n_embd).astype(np.float32)
+    x_dev = rnb.DeviceBuffer.from_host(x_host)
     out_dev = rnb.DeviceBuffer(tokens * n_embd * 4)
     routes = []
     for it in range(8):  # the route changes per iteration, so 392 MB of experts are cycled through
@@ -416,19 +522,46 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed):
         e, r, t = routes[i % len(routes)]
         rnb.moe_sparse_experts_by_token_dev(gd, ud, dd, n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, x_dev, out_dev)
 
-    for i in range(10):
-        step(i)
-    n_k = min(steps, 200)
-    ms = float(np.mean([kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]))
+    st = kernel_stats(hip, stream, step)
+    ms = st["mean"]
     distinct = float(np.mean([len(np.unique(rt[0])) for rt in routes]))
     weight_bytes = distinct * (2 * per_gate + per_down)
     nbytes = weight_bytes + tokens * k * 292 + tokens * n_embd * 4
+    res = {"workload": f"cfg5 sparse MoE 128 experts top-8, hidden 2048, ffn 768, tokens={tokens}", "ms": ms,
+           "ms_median": st["median"], "ms_p10": st["p10"], "ms_p90": st["p90"], "launches": st["launches"],
+           "distinct_experts_mean": distinct, "bytes": nbytes, "GB/s": nbytes / ms / 1e6,
+           "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "ops": 2 * tokens * k * 3 * n_ff * n_embd,
+           "note": "events around the whole call (table upload + quantise + gate/up + re-quantise + down + reduce)"}
+    if cpu:
+        try:
+            from oracle import oracle as ora
+
+            ora.lib()
+            threads = _cpu_threads()
+            e, r, t = routes[0]
+            step(0)
+            rnb.sync()
+            gpu_out = out_dev.to_host(np.float32)
+            run = lambda rt: ora.moe_sparse_experts_by_token(g, u, d, n_expert, rt[0], rt[1], rt[2], tokens, Q6_K, n_ff,  # noqa: E731
+                                                             n_embd, x_host, n_threads=threads)
+            ref = run(routes[0])
+            times, t_start, i = [], time.perf_counter(), 0
+            while time.perf_counter() - t_start < 6.0 and len(times) < 200:
+                t0 = time.perf_counter()
+                run(routes[i % len(routes)])
+                times.append(time.perf_counter() - t0)
+                i += 1
+            med = float(np.median(times))
+            res["cpu_baseline"] = {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                                   "sample": f"{len(times)} full passes of the same routed call (routes rotate as on the GPU), "
+                                             f"median per pass", "ms": med * 1e3, "gpu_matches_cpu": _matches(gpu_out, ref),
+                                   "note": "the per-token loop of prefill_cpu.rs:167-194 over the scalar block dots, "
+                                           "experts of a token on threads"}
+        except Exception as exc:
+            res["cpu_baseline"] = {"error": str(exc)}
     for b in (gd, ud, dd, x_dev, out_dev):
         b.free()
-    return {"workload": f"cfg5 sparse MoE 128 experts top-8, hidden 2048, ffn 768, tokens={tokens}", "ms": ms,
-            "distinct_experts_mean": distinct, "bytes": nbytes, "GB/s": nbytes / ms / 1e6,
-            "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS, "ops": 2 * tokens * k * 3 * n_ff * n_embd,
-            "note": "events around the whole call (table upload + quantise + gate/up + re-quantise + down + reduce)"}
+    return res
 
 
 def bench_ffn(rnb, hip, stream, tokens, steps, seed):
@@ -448,10 +581,8 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
         gd, ud, dd = sets[i % n_copies]
         rnb.dense_q4k_silu_ffn_dev(gd, ud, dd, Q6_K, n_ff, n_embd, tokens, x_dev, out_dev)
 
-    for i in range(10):
-        step(i)
-    n_k = min(steps, 300)
-    ms = float(np.mean([kernel_time_ms(hip, stream, step, n_k) for _ in range(3)]))
+    st = kernel_stats(hip, stream, step, launches=200 if tokens < 16 else 40, warmups=10, batch=10)
+    ms = st["mean"]
     nbytes = wbytes + tokens * (n_embd // 256 * 292 + n_ff // 256 * 292 + n_embd * 4)
     for trio in sets:
         for b in trio:
@@ -459,7 +590,7 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
     x_dev.free()
     out_dev.free()
     res = {"workload": f"dense SwiGLU FFN 4096 -> 14336 -> 4096 (Q4_K gate/up, Q6_K down), tokens={tokens}", "ms": ms,
-           "copies": n_copies}
+           "ms_median": st["median"], "ms_p10": st["p10"], "ms_p90": st["p90"], "launches": st["launches"], "copies": n_copies}
     if tokens < 16:  # decode: weight streaming
         res.update({"bytes": nbytes, "GB/s": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS,
                     "note": "events around the whole call (token quantisation + gate/up/SiLU in one launch, re-quantise, down)"})
@@ -504,7 +635,8 @@ def main() -> int:
     nbytes = main_res["bytes"]
     step_ms = min(main_res["wall_ms_per_step"], main_res.get("graph_ms_per_step", float("inf")))
     launch = "graph" if main_res.get("graph_ms_per_step", float("inf")) <= main_res["wall_ms_per_step"] else "stream"
-    achieved = nbytes / main_res["kernel_ms_mean"] / 1e6
+    kst = main_res["step"]
+    achieved = nbytes / kst["mean"] / 1e6
     result = {
         "metric": "Q4_K decode GEMV HBM GB/s (% of 8 TB/s); prefill GEMM TOPS (% MFMA)",
         "value": nbytes / step_ms / 1e6,
@@ -517,7 +649,9 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "u4 x i8 -> i32, f32 scales",
-        "data": "synthetic: fp32 N(0,0.02) weights fitted to GGUF Q4_K blocks, fp32 N(0,1) activation, seeded",
+        "data": "synthetic, seeded: fp32 N(0,0.02) weights fitted to valid GGUF blocks by a vectorised numpy min/max fit "
+                "inside bench.py (not the restated ggml quantiser: kernel speed does not depend on the values), fp32 N(0,1) "
+                "activations",
         "config": {"workload": "configs[1]: Q4_K decode GEMV, weights 14336x4096 (Llama-3-8B FFN up/gate), 1 token, "
                                "step = device Q8_K quantisation + GEMV (one launch)", "rows": rows, "cols": cols, "tokens": 1,
                    "weight_copies_rotated": main_res["copies"], "step_launch": launch,
@@ -526,17 +660,24 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("gemv_kquant_f32_kernel<12,1>"),
                      "kernel": "gemv_kquant_f32_kernel<12,1> (Q8_K quantisation of the token + GEMV in one launch)",
-                     "bytes_per_launch": nbytes, "kernel_ms_mean": main_res["kernel_ms_mean"],
-                     "prequantised_gemv_kernel_ms_mean": main_res.get("prequantised_kernel_ms_mean"),
-                     "kernel_ms_runs": main_res["kernel_ms_runs"],
-                     "timing": "HIP events around back-to-back launches on the library stream, 3 runs"},
+                     "bytes_per_launch": nbytes, "kernel_ms_mean": kst["mean"], "kernel_ms_median": kst["median"],
+                     "kernel_ms_p10": kst["p10"], "kernel_ms_p90": kst["p90"], "launches": kst["launches"],
+                     "warmup_launches": kst["warmups"],
+                     "prequantised_gemv_kernel_ms_median": main_res["prequantised"]["median"],
+                     "timing": "HIP events on the library stream: 200 back-to-back launches after 20 warm-ups, an event every "
+                               "10 launches; mean over all, median / p10 / p90 over the batches"},
     }
-    try:  # what a plain device copy of the same number of bytes reaches on this box, for context
+    try:  # what a kernel that only reads reaches in this run: on the headline's bytes and on cfg3b's
+        result["roofline"]["read_ceiling"] = read_ceiling(hip, rnb, stream, 33030144)
+        result["roofline"]["read_ceiling_431MB"] = read_ceiling(hip, rnb, stream, 430940160)
+    except Exception as exc:
+        log(f"read ceiling skipped: {exc}")
+    try:  # what the runtime's own device copy reaches on the same number of bytes, for context
         result["roofline"]["device_copy_same_size"] = copy_context(hip, rnb, stream, 33030144)
     except Exception as exc:
         log(f"copy context skipped: {exc}")
-    if "kernel_ms_mean_cache_resident" in main_res:
-        result["roofline"]["cache_resident_GBps"] = nbytes / main_res["kernel_ms_mean_cache_resident"] / 1e6
+    if "cache_resident" in main_res:
+        result["roofline"]["cache_resident_GBps"] = nbytes / main_res["cache_resident"]["median"] / 1e6
     if not args.no_cpu_baseline:
         try:
             result["cpu_baseline"] = cpu_baseline_gemv(Q4_K, w_host, rows, cols, x, gpu_out)
@@ -544,6 +685,34 @@ def main() -> int:
             log(f"cpu baseline failed: {exc}")
             result["cpu_baseline"] = None
     del w_host
+
+    # ---- the metric's second half: cfg4, Q4_K prefill GEMM, 512 tokens x 4096 -> 14336 -----------------------------
+    try:
+        res4, w4, x4, out4 = bench_matmul(rnb, hip, stream, Q4_K, 14336, 4096, 512, 40, 5, 99, "cfg4 q4k gemm",
+                                          want_graph=False, want_wall=False)
+        ops = 2 * 512 * 14336 * 4096
+        pq = res4["prequantised"]
+        tops = ops / pq["mean"] / 1e9
+        result["roofline_gemm"] = {
+            "bound": "mfma", "achieved": tops, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": tops / INT8_PEAK_TOPS,
+            "traffic": None, "workload": "configs[3]: Q4_K prefill GEMM, 512 tokens x 4096 -> 14336",
+            "kernel": "gemm_q4k_mfma_kernel (Q4_K x Q8_K on v_mfma_i32_32x32x32_i8)", "ops_per_launch": ops,
+            "kernel_ms_mean": pq["mean"], "kernel_ms_median": pq["median"], "kernel_ms_p10": pq["p10"],
+            "kernel_ms_p90": pq["p90"], "launches": pq["launches"],
+            "step_ms_median": res4["step"]["median"], "step": "activation quantiser (512 x 4096 f32 -> Q8_K) + GEMM"}
+        try:
+            result["roofline_gemm"]["mfma_ceiling"] = mfma_ceiling(hip, rnb, stream)
+        except Exception as exc:
+            log(f"mfma ceiling skipped: {exc}")
+        if not args.no_cpu_baseline:
+            try:
+                result["cpu_baseline_gemm"] = cpu_baseline_gemm(w4, 14336, 4096, x4, out4)
+            except Exception as exc:
+                log(f"cpu baseline (gemm) failed: {exc}")
+                result["cpu_baseline_gemm"] = None
+        del w4, x4, out4
+    except Exception as exc:
+        result["roofline_gemm"] = {"error": str(exc)}
 
     if not args.quick:
         sec = {}
@@ -553,41 +722,38 @@ def main() -> int:
                                       ("cfg3b_q6k_gemv_128256x4096", Q6_K, 128256, 4096, 1),
                                       ("q5k_gemv_14336x4096", Q5_K, 14336, 4096, 1)):
             try:
-                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, seq, s2 if r < 100000 else 60, 10, 7 + r, key,
-                                            want_graph=False, cache_resident=args.cache_resident)
-                gbps = res["bytes"] / res["kernel_ms_mean"] / 1e6
-                sec[key] = {"kernel_ms_mean": res["kernel_ms_mean"], "bytes": res["bytes"], "GB/s": gbps,
-                            "hbm_frac": gbps / HBM_PEAK_GBPS, "copies": res["copies"]}
-                if res.get("one_launch_step"):  # kernel_ms_mean is the whole step (token quantisation + GEMV, one launch)
-                    sec[key]["kernel"] = "one launch: token quantisation + GEMV"
-                    sec[key]["prequantised_gemv_kernel_ms_mean"] = res["prequantised_kernel_ms_mean"]
-                    sec[key]["prequantised_gemv_GB/s"] = res["bytes"] / res["prequantised_kernel_ms_mean"] / 1e6
-                if "kernel_ms_mean_cache_resident" in res:
-                    sec[key]["cache_resident_GB/s"] = res["bytes"] / res["kernel_ms_mean_cache_resident"] / 1e6
+                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, seq, s2, 10, 7 + r, key, want_graph=False,
+                                            cache_resident=args.cache_resident, want_wall=False)
+                st, pq = res["step"], res["prequantised"]
+                gbps = res["bytes"] / st["mean"] / 1e6
+                sec[key] = {"step_ms_mean": st["mean"], "step_ms_median": st["median"], "step_ms_p10": st["p10"],
+                            "step_ms_p90": st["p90"], "launches": st["launches"], "bytes": res["bytes"], "GB/s": gbps,
+                            "hbm_frac": gbps / HBM_PEAK_GBPS, "copies": res["copies"],
+                            "step": "one launch: token quantisation + GEMV" if res["one_launch_step"]
+                            else "two launches: activation quantiser, then the GEMV",
+                            "prequantised_gemv_ms_median": pq["median"],
+                            "prequantised_gemv_GB/s": res["bytes"] / pq["median"] / 1e6}
+                if "cache_resident" in res:
+                    sec[key]["cache_resident_GB/s"] = res["bytes"] / res["cache_resident"]["median"] / 1e6
             except Exception as exc:
                 sec[key] = {"error": str(exc)}
-        try:
-            res, _, _, _ = bench_matmul(rnb, hip, stream, Q4_K, 14336, 4096, 512, 40, 5, 99, "cfg4 q4k gemm",
-                                        want_graph=False)
-            ops = 2 * 512 * 14336 * 4096
-            tops = ops / res["kernel_ms_mean"] / 1e9
-            sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"kernel_ms_mean": res["kernel_ms_mean"], "ops": ops, "TOP/s": tops,
-                                                      "mfma_frac": tops / INT8_PEAK_TOPS}
-        except Exception as exc:
-            sec["cfg4_q4k_gemm_512x4096_to_14336"] = {"error": str(exc)}
         # prefill on the formats whose scales cannot ride on an int8 operand (scale groups applied on the vector units)
         for key, quant, r, c in (("q6k_gemm_512x14336_to_4096", Q6_K, 4096, 14336), ("q5k_gemm_512x4096_to_14336", Q5_K, 14336, 4096),
                                  ("q8_0_gemm_512x4096_to_4096", Q8_0, 4096, 4096)):
             try:
-                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, 512, 20, 3, 101, key, want_graph=False)
+                res, _, _, _ = bench_matmul(rnb, hip, stream, quant, r, c, 512, 20, 3, 101, key, want_graph=False,
+                                            want_wall=False)
                 ops = 2 * 512 * r * c
-                tops = ops / res["kernel_ms_mean"] / 1e9
-                sec[key] = {"kernel_ms_mean": res["kernel_ms_mean"], "ops": ops, "TOP/s": tops, "mfma_frac": tops / INT8_PEAK_TOPS}
+                pq = res["prequantised"]
+                tops = ops / pq["mean"] / 1e9
+                sec[key] = {"kernel_ms_mean": pq["mean"], "kernel_ms_median": pq["median"], "kernel_ms_p10": pq["p10"],
+                            "kernel_ms_p90": pq["p90"], "ops": ops, "TOP/s": tops, "mfma_frac": tops / INT8_PEAK_TOPS}
             except Exception as exc:
                 sec[key] = {"error": str(exc)}
         for tokens in (1, 64):
             try:
-                sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens)
+                sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens,
+                                                            cpu=not args.no_cpu_baseline)
             except Exception as exc:
                 sec[f"cfg5_moe_tokens{tokens}"] = {"error": str(exc)}
         for tokens, n in ((1, s2), (512, 20)):

@@ -78,6 +78,13 @@ int rnb_hip_transfer_counters(uint64_t *h2d_bytes, uint64_t *d2h_bytes);
 /* the library's only stream, as a hipStream_t */
 void *rnb_hip_stream(void);
 
+/* ---- calibration for the benchmark's roofline lines (no counterpart in the reference) ------------
+ * rnb_hip_calib_read enqueues a kernel that only reads `bytes` of device memory (16-byte loads, optionally
+ * non-temporal); rnb_hip_calib_mfma_i8 one that only issues v_mfma_i32_32x32x32_i8 (`workgroups` x 8 waves x 4 chains x
+ * `iters`) and reports the integer operations it performs.  Both run on the library stream and do not synchronise. */
+int rnb_hip_calib_read(const void *dev, size_t bytes, int non_temporal);
+int rnb_hip_calib_mfma_i8(uint32_t iters, uint32_t workgroups, uint64_t *ops);
+
 /* ---- weight residency: crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:399-405,757-851 */
 /* prewarm_q4k_weights (api/quant_api.rs:952): upload host ranges untouched and keep them
  * resident, keyed by (pointer, length, sampled fingerprint).  Sub-ranges of a resident range

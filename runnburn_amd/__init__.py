@@ -44,6 +44,8 @@ from .binding import (  # noqa: F401
     dense_q4k_silu_ffn_dev,
     device_available,
     device_name,
+    calib_mfma_i8,
+    calib_read,
     gemv_dev,
     gemv_dev_noalloc,
     gemv_dev_noalloc_scratch_bytes,

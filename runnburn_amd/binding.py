@@ -31,6 +31,8 @@ SYMBOLS = [
     ("rnb_hip_prewarm", _i, [C.POINTER(_vp), C.POINTER(_sz), _sz]),
     ("rnb_hip_release", _i, [_vp, _sz]),
     ("rnb_hip_resident_bytes", _i, [_u64p, _u64p]),
+    ("rnb_hip_calib_read", _i, [_vp, _sz, _i]),
+    ("rnb_hip_calib_mfma_i8", _i, [_u32, _u32, _u64p]),
     ("rnb_hip_residency_stats", _i, [_u64p, _sz]),
     ("rnb_hip_set_resident_budget", _i, [C.c_uint64]),
     ("rnb_hip_offload_unpinned", _i, [_u64p]),
@@ -428,6 +430,18 @@ class DeviceBuffer:
             self.free()
         except Exception:
             pass
+
+
+def calib_read(buf: DeviceBuffer, nbytes: int, non_temporal: bool = False) -> None:
+    """Enqueue the read-only calibration kernel over the first nbytes of buf."""
+    _check(lib().rnb_hip_calib_read(buf.ptr, nbytes, 1 if non_temporal else 0))
+
+
+def calib_mfma_i8(iters: int, workgroups: int) -> int:
+    """Enqueue the matrix-instruction-only calibration kernel; returns the integer operations it performs."""
+    ops = C.c_uint64()
+    _check(lib().rnb_hip_calib_mfma_i8(iters, workgroups, C.byref(ops)))
+    return int(ops.value)
 
 
 def gemv_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, x: DeviceBuffer, seq_len: int,

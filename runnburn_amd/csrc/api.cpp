@@ -743,6 +743,24 @@ int rnb_hip_resident_bytes(uint64_t *bytes, uint64_t *entries) {
     return RNB_HIP_OK;
 }
 
+int rnb_hip_calib_read(const void *dev, size_t bytes, int non_temporal) {
+    if (!dev || (reinterpret_cast<uintptr_t>(dev) & 15u)) return fail(RNB_HIP_INVALID_REQUEST, "calibration read needs a 16-byte aligned device pointer");
+    Guard g;
+    if (!g.state) return g.status;
+    RESERVE_TRY(g.state->argmax_scratch, 257 * 8);
+    launch_calib_read(dev, bytes, non_temporal != 0, g.state->argmax_scratch.as<uint32_t>(), g.state->stream);
+    return check_launches();
+}
+
+int rnb_hip_calib_mfma_i8(uint32_t iters, uint32_t workgroups, uint64_t *ops) {
+    Guard g;
+    if (!g.state) return g.status;
+    RESERVE_TRY(g.state->argmax_scratch, 257 * 8);
+    const uint64_t n = launch_calib_mfma_i8(iters, workgroups, g.state->argmax_scratch.as<int>(), g.state->stream);
+    if (ops) *ops = n;
+    return check_launches();
+}
+
 int rnb_hip_residency_stats(uint64_t *out, size_t n) {
     Guard g;
     if (!g.state) return g.status;

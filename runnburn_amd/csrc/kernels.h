@@ -174,6 +174,11 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,
                        float *out, uint32_t token_count, uint32_t n_embd, hipStream_t stream);
 
+// ---- calibration (calib.hip): a read-only stream over `bytes` of device memory, and int8 matrix instructions only ----
+void launch_calib_read(const void *dev, size_t bytes, bool non_temporal, uint32_t *sink, hipStream_t stream);
+// returns the integer operations the launch performs (2 per multiply-add)
+uint64_t launch_calib_mfma_i8(uint32_t iters, uint32_t workgroups, int *sink, hipStream_t stream);
+
 // ---- launch configuration failures ------------------------------------------------------------------
 // Raises `kernel`'s dynamic LDS limit to `bytes` (above the default 64 KB) once: `*done` is set only when the runtime
 // accepted it, so a failure is tried again by the next launch.  On failure the launcher must not launch; the reason is
