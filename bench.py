@@ -601,12 +601,35 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
     return res
 
 
+# configs that --only can run alone: quant, rows, cols, tokens
+ONLY = {"cfg1": (Q8_0, 4096, 4096, 1), "cfg2": (Q4_K, 14336, 4096, 1), "cfg3a": (Q6_K, 4096, 14336, 1),
+        "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512)}
+
+
+def run_only(rnb, hip, stream, name, calibration):
+    """One config, 60 steps after 10 warm-ups (plus the calibration copies when asked): what a counter run profiles."""
+    quant, rows, cols, seq = ONLY[name]
+    if calibration:
+        calibration_copy(hip, rnb, stream)
+    w_host = synth_weights(quant, rows, cols, 20240607)
+    n_copies = copies_for(w_host.nbytes)
+    w_dev = [rnb.DeviceBuffer.from_host(w_host) for _ in range(n_copies)]
+    x_dev = rnb.DeviceBuffer.from_host(np.random.default_rng(1).standard_normal(seq * cols).astype(np.float32))
+    out_dev = rnb.DeviceBuffer(seq * rows * 4)
+    st = kernel_stats(hip, stream, lambda i: rnb.gemv_dev(quant, w_dev[i % n_copies], rows, cols, x_dev, seq, out_dev),
+                      launches=60, warmups=10, batch=10)
+    print(json.dumps({"only": name, "step_ms_median": st["median"], "launches": st["launches"], "copies": n_copies}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--quick", action="store_true", help="headline config only (skip the secondary configs)")
+    ap.add_argument("--only", choices=sorted(ONLY), help="one config's step, a few dozen launches, for counter runs under "
+                                                         "rocprofv3 --pmc (prints a short JSON line of its own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a 64 MiB device-to-device copy (reference for FETCH_SIZE / WRITE_SIZE under --pmc)")
@@ -627,6 +650,8 @@ def main() -> int:
     stream = C.c_void_p(rnb.stream_handle())
     log(f"device: {rnb.device_name()}")
 
+    if args.only:
+        return run_only(rnb, hip, stream, args.only, args.calibration_copy)
     if args.calibration_copy:
         calibration_copy(hip, rnb, stream)
     rows, cols = 14336, 4096
