@@ -228,6 +228,30 @@ int rnb_hip_gemv_dev_noalloc(uint32_t quant, const void *w_dev, size_t rows, siz
 int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols);
 int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, size_t cols,
                                size_t seq_len, float *out_dev);
+/* RMS norm in front of the GEMVs, device-resident.  Arithmetic of crates/rnb-cpu/src/kernels/norm.rs:140-225: mean square
+ * in f64 and out = (x / rms) * weight (rms_norm_into, the default path); with unit_offset != 0 the mean square in f32 and
+ * out = (x / rms) * (1 + weight) (rms_norm_unit_offset_into).  x_dev [seq_len][hidden], hidden % 256 == 0.
+ * rnb_hip_rms_norm_dev replaces rnb_rms_norm_f32 (crates/rnb-backend/cuda/cuda/kernels/quant_batch_and_ops.cuh:4031).
+ * rnb_hip_rms_norm_quantize_dev also leaves Q8_K(out) in the library's activation scratch, exactly what
+ * rnb_hip_quantize_dev would make of `out`, so that rnb_hip_gemv_quantized_dev (K-quant weights, cols == hidden) follows
+ * without a quantiser launch; out_dev may be null when only the quantised form is wanted. */
+int rnb_hip_rms_norm_dev(const float *x_dev, const float *weight_dev, float eps, int unit_offset, size_t seq_len,
+                         size_t hidden, float *out_dev);
+int rnb_hip_rms_norm_quantize_dev(const float *x_dev, const float *weight_dev, float eps, int unit_offset, size_t seq_len,
+                                  size_t hidden, float *out_dev);
+/* rnb_rms_norm_add_then_rms_norm_q8_1_f32 (quant_batch_and_ops.cuh:4275) with rnb-cpu's arithmetic and Q8_K output:
+ * residual += norm(input, post_weight, post_eps); out = norm(residual, pre_weight, pre_eps); Q8_K(out) -> activation
+ * scratch.  residual_dev is updated in place; out_dev may be null. */
+int rnb_hip_rms_norm_add_rms_norm_quantize_dev(const float *input_dev, const float *post_weight_dev, float post_eps,
+                                               int post_unit_offset, float *residual_dev, const float *pre_weight_dev,
+                                               float pre_eps, int pre_unit_offset, size_t seq_len, size_t hidden,
+                                               float *out_dev);
+/* rnb_moe_route_topk_f32 (quant_batch_and_ops.cuh) with the selection rule of
+ * crates/rnb-llm/src/engine/models/shared_expert_moe/routing.rs:18-64: per token the k largest logits (ties to the lower
+ * expert id, NaN never selected), softmax over the selected logits, rank order.  logits_dev [token_count][n_expert];
+ * idx_dev / weights_dev [token_count][min(k, n_expert)]; n_expert <= 512, k <= 32. */
+int rnb_hip_moe_route_topk_dev(const float *logits_dev, size_t token_count, size_t n_expert, size_t k, uint32_t *idx_dev,
+                               float *weights_dev);
 /* device-resident form of rnb_hip_moe_sparse_experts_by_token: weights, x and out on the device;
  * the slot arrays stay on the host (the caller routes on the host, as the reference does). */
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev,

@@ -254,6 +254,28 @@ def dense_silu_ffn(gate, up, down, down_quant: int, n_ff: int, n_embd: int, x) -
     return gemv(down_quant, down, n_embd, n_ff, mid)
 
 
+def rms_norm(x, weight, eps: float, unit_offset: bool = False) -> np.ndarray:
+    """crates/rnb-cpu/src/kernels/norm.rs:180-196 (rms_norm_into_f64, the default of rms_norm_into: mean square summed in
+    f64 in element order, rms = f32(sqrt(mean + eps)), out = (x / rms) * weight) and :211-224
+    (rms_norm_unit_offset_into_scalar: f32 sum in element order, out = (x / rms) * (1 + weight)).  x is [rows][hidden]."""
+    w = _f32(weight)
+    rows = _f32(x).reshape(-1, w.size)
+    out = np.empty_like(rows)
+    e32 = np.float32(eps)
+    for r in range(rows.shape[0]):
+        row = rows[r]
+        if unit_offset:
+            total = np.cumsum(row * row, dtype=np.float32)[-1]  # cumsum accumulates strictly in order
+            rms = np.sqrt(np.float32(total / np.float32(w.size)) + e32, dtype=np.float32)
+            out[r] = (row / rms) * (np.float32(1.0) + w)
+        else:
+            r64 = row.astype(np.float64)
+            total = np.cumsum(r64 * r64)[-1]
+            rms = np.float32(np.sqrt(total / float(w.size) + float(e32)))
+            out[r] = (row / rms) * w
+    return out
+
+
 def route_topk(logits, k: int) -> tuple[np.ndarray, np.ndarray]:
     lg = _f32(logits)
     idx = np.zeros(min(k, lg.size), dtype=np.uint32)

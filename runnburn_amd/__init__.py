@@ -51,6 +51,9 @@ from .binding import (  # noqa: F401
     gemv_dev_noalloc_scratch_bytes,
     gemv_quantized_dev,
     quantize_dev,
+    rms_norm_dev,
+    rms_norm_add_rms_norm_quantize_dev,
+    moe_route_topk_dev,
     last_error,
     lib,
     lib_path,

@@ -70,6 +70,10 @@ SYMBOLS = [
     ("rnb_hip_gemv_dev_noalloc", _i, [_u32, _vp, _sz, _sz, _vp, _sz, _vp]),
     ("rnb_hip_gemv_dev_noalloc_scratch_bytes", _sz, []),
     ("rnb_hip_quantize_dev", _i, [_u32, _vp, _sz, _sz]),
+    ("rnb_hip_rms_norm_dev", _i, [_vp, _vp, C.c_float, _i, _sz, _sz, _vp]),
+    ("rnb_hip_rms_norm_quantize_dev", _i, [_vp, _vp, C.c_float, _i, _sz, _sz, _vp]),
+    ("rnb_hip_rms_norm_add_rms_norm_quantize_dev", _i, [_vp, _vp, C.c_float, _i, _vp, _vp, C.c_float, _i, _sz, _sz, _vp]),
+    ("rnb_hip_moe_route_topk_dev", _i, [_vp, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
      [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
@@ -458,6 +462,30 @@ def gemv_dev_noalloc(quant: int, w: DeviceBuffer, rows: int, cols: int, x: Devic
 
 def gemv_dev_noalloc_scratch_bytes() -> int:
     return int(lib().rnb_hip_gemv_dev_noalloc_scratch_bytes())
+
+
+def rms_norm_dev(x: DeviceBuffer, weight: DeviceBuffer, eps: float, seq_len: int, hidden: int, out: DeviceBuffer,
+                 unit_offset: bool = False, quantize: bool = False) -> None:
+    """RMS norm of [seq_len][hidden] rows; with quantize=True Q8_K(out) is also left in the activation scratch
+    (out may then be None)."""
+    fn = lib().rnb_hip_rms_norm_quantize_dev if quantize else lib().rnb_hip_rms_norm_dev
+    _check(fn(x.ptr, weight.ptr, eps, 1 if unit_offset else 0, seq_len, hidden, out.ptr if out is not None else None))
+
+
+def rms_norm_add_rms_norm_quantize_dev(inp: DeviceBuffer, post_weight: DeviceBuffer, post_eps: float, residual: DeviceBuffer,
+                                       pre_weight: DeviceBuffer, pre_eps: float, seq_len: int, hidden: int,
+                                       out: Optional[DeviceBuffer], post_unit_offset: bool = False,
+                                       pre_unit_offset: bool = False) -> None:
+    """residual += norm(inp, post_weight); out = norm(residual, pre_weight); Q8_K(out) -> activation scratch."""
+    _check(lib().rnb_hip_rms_norm_add_rms_norm_quantize_dev(
+        inp.ptr, post_weight.ptr, post_eps, 1 if post_unit_offset else 0, residual.ptr, pre_weight.ptr, pre_eps,
+        1 if pre_unit_offset else 0, seq_len, hidden, out.ptr if out is not None else None))
+
+
+def moe_route_topk_dev(logits: DeviceBuffer, token_count: int, n_expert: int, k: int, idx: DeviceBuffer,
+                       weights: DeviceBuffer) -> None:
+    """Per token: top-k expert ids (ties to the lower id) and the softmax over their logits, in rank order."""
+    _check(lib().rnb_hip_moe_route_topk_dev(logits.ptr, token_count, n_expert, k, idx.ptr, weights.ptr))
 
 
 def quantize_dev(quant: int, x: DeviceBuffer, seq_len: int, cols: int) -> None:

@@ -1316,6 +1316,91 @@ int rnb_hip_gemv_dev_noalloc(uint32_t quant, const void *w_dev, size_t rows, siz
     return run_matmul_dev(*g.state, quant, static_cast<const uint8_t *>(w_dev), rows, cols, x_dev, seq_len, out_dev, &arena);
 }
 
+}  // extern "C"
+
+namespace {
+
+// shared by the three norm entry points: checks, activation scratch for the Q8_K output, launch
+int rms_norm_dev(const char *what, const float *input, const float *post_weight, float post_eps, int post_unit,
+                 float *residual, const float *weight, float eps, int unit, size_t seq_len, size_t hidden, float *out_f32,
+                 bool quantize) {
+    const std::string name = what;
+    if (hidden == 0 || hidden % 256 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, name + " hidden size must be divisible by 256, got " + std::to_string(hidden));
+    if (!input || !weight || (residual && !post_weight) || (!quantize && !out_f32))
+        return fail(RNB_HIP_INVALID_REQUEST, name + " null device pointer");
+    if ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(residual) |
+         reinterpret_cast<uintptr_t>(post_weight) | reinterpret_cast<uintptr_t>(out_f32)) & 15u)
+        return fail(RNB_HIP_INVALID_REQUEST, name + " device pointers must be 16-byte aligned");
+    if (hidden > 0x00ffffffu || seq_len > 65535u) return fail(RNB_HIP_INVALID_REQUEST, name + " shape out of range");
+    if (seq_len == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    int8_t *qs = nullptr;
+    float *d = nullptr;
+    int16_t *bsums = nullptr;
+    uint8_t *digits = nullptr;
+    if (quantize) {
+        const size_t n = seq_len * hidden;
+        RESERVE_TRY(s.act_qs, n);
+        RESERVE_TRY(s.act_d, n / 256 * sizeof(float));
+        RESERVE_TRY(s.act_bsums, n / 256 * 16 * sizeof(int16_t));
+        s.act_has_digits = seq_len >= kDigitsMinSeq;
+        if (s.act_has_digits) RESERVE_TRY(s.act_digits, n / 256 * 16);
+        qs = s.act_qs.as<int8_t>();
+        d = s.act_d.as<float>();
+        bsums = s.act_bsums.as<int16_t>();
+        digits = s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr;
+        s.act_family = kQ4K;
+        s.act_seq = seq_len;
+        s.act_cols = hidden;
+    }
+    launch_rms_norm(input, post_weight, post_eps, post_unit != 0, residual, weight, eps, unit != 0,
+                    static_cast<uint32_t>(seq_len), static_cast<uint32_t>(hidden / 256), out_f32, qs, d, bsums, digits, s.stream);
+    return check_launches();
+}
+
+}  // namespace
+
+extern "C" {
+
+int rnb_hip_rms_norm_dev(const float *x_dev, const float *weight_dev, float eps, int unit_offset, size_t seq_len,
+                         size_t hidden, float *out_dev) {
+    return rms_norm_dev("RMS norm", x_dev, nullptr, 0.0f, 0, nullptr, weight_dev, eps, unit_offset, seq_len, hidden, out_dev,
+                        false);
+}
+
+int rnb_hip_rms_norm_quantize_dev(const float *x_dev, const float *weight_dev, float eps, int unit_offset, size_t seq_len,
+                                  size_t hidden, float *out_dev) {
+    return rms_norm_dev("RMS norm + Q8_K", x_dev, nullptr, 0.0f, 0, nullptr, weight_dev, eps, unit_offset, seq_len, hidden,
+                        out_dev, true);
+}
+
+int rnb_hip_rms_norm_add_rms_norm_quantize_dev(const float *input_dev, const float *post_weight_dev, float post_eps,
+                                               int post_unit_offset, float *residual_dev, const float *pre_weight_dev,
+                                               float pre_eps, int pre_unit_offset, size_t seq_len, size_t hidden,
+                                               float *out_dev) {
+    if (!residual_dev) return fail(RNB_HIP_INVALID_REQUEST, "RMS norm + add + RMS norm + Q8_K null device pointer");
+    return rms_norm_dev("RMS norm + add + RMS norm + Q8_K", input_dev, post_weight_dev, post_eps, post_unit_offset,
+                        residual_dev, pre_weight_dev, pre_eps, pre_unit_offset, seq_len, hidden, out_dev, true);
+}
+
+int rnb_hip_moe_route_topk_dev(const float *logits_dev, size_t token_count, size_t n_expert, size_t k, uint32_t *idx_dev,
+                               float *weights_dev) {
+    if (!logits_dev || !idx_dev || !weights_dev) return fail(RNB_HIP_INVALID_REQUEST, "router null device pointer");
+    if (n_expert > 0xffffu || k > 0xffffu || token_count > 0x00ffffffu ||
+        !route_topk_supported(static_cast<uint32_t>(n_expert), static_cast<uint32_t>(k)))
+        return fail(RNB_HIP_INVALID_REQUEST, "router supports 1..512 experts and top-1..32, got n_expert=" +
+                                                 std::to_string(n_expert) + " k=" + std::to_string(k));
+    if (token_count == 0) return RNB_HIP_OK;
+    Guard g;
+    if (!g.state) return g.status;
+    launch_route_topk(logits_dev, static_cast<uint32_t>(token_count), static_cast<uint32_t>(n_expert), static_cast<uint32_t>(k),
+                      idx_dev, weights_dev, g.state->stream);
+    return check_launches();
+}
+
 int rnb_hip_quantize_dev(uint32_t quant, const float *x_dev, size_t seq_len, size_t cols) {
     QuantInfo qi;
     if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));

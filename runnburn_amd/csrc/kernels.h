@@ -174,6 +174,18 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots,
                        float *out, uint32_t token_count, uint32_t n_embd, hipStream_t stream);
 
+// ---- RMS norm (+ residual add) with optional Q8_K output, router (norm_route.hip) ------------------------------------
+// Rows of nb * 256 floats, one workgroup each.  residual != null: residual += norm(input, post_weight, post_eps) first and
+// the normalised row is the new residual; else it is input.  out_f32 and (qs, d, bsums[, digits]) are optional outputs.
+void launch_rms_norm(const float *input, const float *post_weight, float post_eps, bool post_unit, float *residual,
+                     const float *weight, float eps, bool unit, uint32_t seq, uint32_t nb, float *out_f32, int8_t *qs,
+                     float *d, int16_t *bsums, uint8_t *digits, hipStream_t stream);
+// top-k of each token's logits (ties to the lower id), softmax over the selected ones, rank order: idx_out / w_out
+// [tokens][min(k, n_expert)]
+bool route_topk_supported(uint32_t n_expert, uint32_t k);
+void launch_route_topk(const float *logits, uint32_t tokens, uint32_t n_expert, uint32_t k, uint32_t *idx_out, float *w_out,
+                       hipStream_t stream);
+
 // ---- calibration (calib.hip): a read-only stream over `bytes` of device memory, and int8 matrix instructions only ----
 void launch_calib_read(const void *dev, size_t bytes, bool non_temporal, uint32_t *sink, hipStream_t stream);
 // returns the integer operations the launch performs (2 per multiply-add)

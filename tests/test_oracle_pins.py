@@ -892,3 +892,36 @@ def test_generator_is_counter_based_and_normal(oracle):
     assert np.array_equal(w1, w2)
     row3 = oracle.quantize_row(Q4_K, oracle.fill_normal(8 * 512, 77, 0.02)[3 * 512:4 * 512])
     assert np.array_equal(w1[3 * 288:4 * 288], row3)
+
+
+# ---- RMS norm ------------------------------------------------------------------------------------------
+
+def test_rms_norm_reference_vectors_and_closed_forms(oracle):
+    """crates/rnb-cpu/src/kernels/norm.rs:339-385: [1, 2, 3, 4] with unit weights gives x / sqrt(7.5 + 1e-5); the weighted
+    and unit-offset forms multiply by w and 1 + w.  Against Python's own f64 arithmetic, then properties the
+    mathematics fixes: a power-of-two scaling of x with eps = 0 leaves the output bits alone, a constant row of c
+    gives sign(c) * w / sqrt(1 + eps / c^2), rows are independent."""
+    import math
+
+    x = np.array([1.0, 2.0, 3.0, 4.0], np.float32)
+    one = oracle.rms_norm(x, np.ones(4, np.float32), 1e-5)[0]
+    rms = math.sqrt(7.5 + float(np.float32(1e-5)))
+    assert abs(one[0] - 1.0 / rms) < 1e-7 and abs(one[1] - 2.0 / rms) < 1e-7 and abs(one[3] - 4.0 / rms) < 2e-7
+    w = np.array([1.0, 0.5, 2.0, 0.25], np.float32)
+    got = oracle.rms_norm(x, w, 1e-5)[0]
+    assert np.allclose(got, x.astype(np.float64) / rms * w, rtol=2e-7, atol=0)
+    wu = np.array([0.0, -0.5, 1.0, -0.75], np.float32)
+    gu = oracle.rms_norm(x, wu, 1e-5, unit_offset=True)[0]
+    assert np.allclose(gu, x.astype(np.float64) / rms * (1.0 + wu), rtol=3e-7, atol=0)
+    rng = np.random.default_rng(5)
+    xr = rng.standard_normal(3 * 1536).astype(np.float32)
+    wr = rng.standard_normal(1536).astype(np.float32)
+    base = oracle.rms_norm(xr, wr, 0.0)
+    assert np.array_equal(oracle.rms_norm(4.0 * xr, wr, 0.0).view(np.uint32), base.view(np.uint32))
+    assert np.array_equal(oracle.rms_norm(xr[1536:3072], wr, 0.0)[0].view(np.uint32), base[1].view(np.uint32))
+    f64 = xr.reshape(3, 1536).astype(np.float64)
+    want = f64 / np.sqrt((f64 * f64).mean(axis=1, keepdims=True) + float(np.float32(1e-6))) * wr
+    assert np.allclose(oracle.rms_norm(xr, wr, 1e-6), want, rtol=3e-7, atol=1e-9)
+    assert np.allclose(oracle.rms_norm(xr, wr, 1e-6, unit_offset=True), want / wr * (1.0 + wr.astype(np.float64)), rtol=2e-6, atol=1e-8)
+    c = np.full(256, -3.0, np.float32)
+    assert np.allclose(oracle.rms_norm(c, np.ones(256, np.float32), 1e-5)[0], -1.0 / math.sqrt(1.0 + 1e-5 / 9.0), rtol=2e-7)
