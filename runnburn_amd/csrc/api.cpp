@@ -541,7 +541,9 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     // Batches with at least four slots per routed expert on average: the expert GEMMs run on the matrix cores (a
     // 32-token tile costs the same whatever its number of live tokens, the integer-dot kernels cost per token; measured
     // crossover on 128 experts x top-8: 64 tokens) and need the quantiser's digits
-    const bool mfma = token_count >= kMoeMfmaMinTokens && n_slots >= 4 * n_groups &&
+    // (its gate/up rows arrive as 16-byte LDS-direct loads: other alignments take the vector kernels)
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) & 15u) == 0;
+    const bool mfma = token_count >= kMoeMfmaMinTokens && n_slots >= 4 * n_groups && aligned16 &&
                       moe_mfma_supported(static_cast<uint32_t>(sh.nb_in), static_cast<uint32_t>(sh.nb_mid), down_quant);
     const bool inline_tables = !mfma && table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
     MoeInlineTables inl;
@@ -589,8 +591,10 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     }
     const float *d_route = reinterpret_cast<const float *>(d);
     const uint32_t *d_off = d + n_slots, *d_list = d_off + token_count + 1;
+    uint32_t max_group = 0;
+    for (size_t g = 0; g < n_groups; g++) max_group = std::max(max_group, grp_start[g + 1] - grp_start[g]);
     const MoeGroups groups{d_list + 3 * n_slots, d_list + 3 * n_slots + n_groups, d_list + n_slots, d_list + 2 * n_slots,
-                           static_cast<uint32_t>(n_groups)};
+                           static_cast<uint32_t>(n_groups), max_group};
 
     ActView act;
     if (inline_tables) {

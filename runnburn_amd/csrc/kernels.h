@@ -127,6 +127,7 @@ struct MoeGroups {
     const uint32_t *sorted_slot;   // [n_slots]
     const uint32_t *sorted_token;  // [n_slots]
     uint32_t n_groups;
+    uint32_t max_group = 32;       // slots of the largest group (host-side knowledge: sizes the matrix-core kernels' LDS)
 };
 // Q8_K of act(gate[i]) * up[i] (SiLU, or the tanh form of GELU): the gated FFN's intermediate quantised as it is made
 void launch_quantize_q8k_gated(const float *gate, const float *up, size_t n_blocks, bool gelu, int8_t *qs, float *d,

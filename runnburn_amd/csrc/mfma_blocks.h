@@ -137,6 +137,16 @@ __device__ __forceinline__ void route_store(const RowRoute<kPieces> &rt, uint8_t
     }
 }
 
+// 128-bit stores, for strips whose row stride is a multiple of 16
+template <int kPieces>
+__device__ __forceinline__ void route_store16(const RowRoute<kPieces> &rt, uint8_t *strip, int lane) {
+#pragma unroll
+    for (int i = 0; i < RowRoute<kPieces>::kN; i++) {
+        if ((i + 1) * kWave <= 32 * kPieces || lane + i * kWave < 32 * kPieces)
+            *reinterpret_cast<uint4 *>(strip + rt.loff[i]) = rt.v[i];
+    }
+}
+
 constexpr int kQ6Pieces = 13;        // ql, qh and scales: 208 bytes; d is read by the row's lanes themselves
 constexpr int kQ6StripStride = 216;  // 54 dwords: the 32 rows' 64-bit reads fall on 32 different bank pairs
 
@@ -217,6 +227,18 @@ __device__ __forceinline__ Q5Row q45_load_row(const uint8_t *__restrict__ blk, i
 #pragma unroll
     for (int g = 0; g < 4; g++) r.qs[g] = ld_u4_a2(blk + (kFifth ? 48 : 16) + 32 * g + 16 * khalf);
     return r;
+}
+
+// Q4_K rows through the wave's strip: a block is nine 16-byte pieces; rows 144 bytes (36 dwords) apart, which keeps the
+// 32 rows' 128-bit reads on different banks
+constexpr int kQ4Pieces = 9;
+constexpr int kQ4StripStride = 144;
+constexpr int kQ4StripBytes = 32 * kQ4StripStride;
+__device__ __forceinline__ void q4_row_from_strip(Q5Row &r, const uint8_t *row, int khalf) {
+    r.hdr = *reinterpret_cast<const uint4 *>(row);
+    r.qh = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.qs[g] = *reinterpret_cast<const uint4 *>(row + 16 + 32 * g + 16 * khalf);
 }
 
 template <int kSb, bool kFifth>

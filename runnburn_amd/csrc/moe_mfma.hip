@@ -3,8 +3,11 @@
 // of 32 tokens: the tokens' quantised activations are gathered into LDS by the sorted lists, the expert's weight rows go
 // from global memory to the registers of the lane that owns the row, one int8 matrix instruction per scale group, the
 // group's scale on the vector units (see gemm_blocks.hip).  With a handful of tokens per expert most of a 32-token tile
-// is padding, which costs nothing extra: the work per tile is the same whatever the number of live tokens, where the
-// integer-dot kernels of moe.hip cost per token (measured crossover on 128 experts x top-8: 64 tokens).
+// is padding, which costs no arithmetic: the work per tile is the same whatever the number of live tokens, where the
+// integer-dot kernels of moe.hip cost per token (measured crossover on 128 experts x top-8: 64 tokens).  Padding costs
+// no LDS either: only the live tokens are staged, the matrix instruction's padding lanes read the last live token's
+// row, and the launch sizes the image for the largest group of the call, so that several workgroups share a compute
+// unit when the groups are small.
 //   gate/up   mid[slot][n_ff] = silu(Wg[e] . a_tok) * (Wu[e] . a_tok), both Q4_K: the two matrices share the activation
 //             operand of every instruction                        fanout.rs:260-327, activation.rs:73-89
 //   down      slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])), Q4_K, Q5_K or Q6_K
@@ -12,12 +15,16 @@
 #include "device_utils.h"
 #include "kernels.h"
 #include "mfma_blocks.h"
+#include <algorithm>
 
 namespace rnb {
 
 namespace {
 
 constexpr int kMmToks = 32;  // tokens per tile
+constexpr int kQ4FillInstr = (32 * kQ4Pieces + kWave - 1) / kWave;  // 5 wave-wide 16-byte loads per 32 rows of a Q4_K block
+constexpr int kQ4FillBytes = kQ4FillInstr * 1024;                   // what they write: 32 x 144 bytes of rows + the tail
+constexpr int kMmGateUpStripBytes = kGbWaves * 2 * kQ4FillBytes;    // gate and up strips of the four waves
 
 // the tile's list entries: activation row, output row (0xffffffff past the end of the group) and output scale
 struct TileMap {
@@ -27,10 +34,10 @@ struct TileMap {
 };
 
 __device__ __forceinline__ void tile_map_fill(TileMap &m, const uint32_t *__restrict__ act_idx, const uint32_t *__restrict__ out_idx,
-                                              const float *__restrict__ out_scale, uint32_t first, uint32_t left, int tid) {
+                                              const float *__restrict__ out_scale, uint32_t first, uint32_t n_live, int tid) {
     if (tid < kMmToks) {
-        const bool live = static_cast<uint32_t>(tid) < left;
-        const uint32_t p = first + (live ? static_cast<uint32_t>(tid) : left - 1);  // padding repeats the last entry
+        const bool live = static_cast<uint32_t>(tid) < n_live;
+        const uint32_t p = first + (live ? static_cast<uint32_t>(tid) : n_live - 1);  // padding repeats the last entry
         m.act_row[tid] = act_idx[p];
         const uint32_t o = out_idx[p];
         m.out_row[tid] = live ? o : 0xffffffffu;
@@ -48,11 +55,13 @@ struct TileStage {
 template <bool kDigits>
 __device__ __forceinline__ void tile_stage_load(TileStage &st, const TileMap &m, const int8_t *__restrict__ aq,
                                                 const float *__restrict__ ad, const uint8_t *__restrict__ adig, size_t nb,
-                                                size_t b, int tid) {
+                                                size_t b, int tid, uint32_t live) {
 #pragma unroll
     for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
         const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
-        st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(m.act_row[c >> 5]) * nb + b) * 256 + (c & 31) * 8);
+        st.v[i] = make_uint2(0, 0);
+        if ((c >> 5) < live)
+            st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(m.act_row[c >> 5]) * nb + b) * 256 + (c & 31) * 8);
     }
     st.dx = 0.0f;
     st.dig = make_uint4(0, 0, 0, 0);
@@ -64,11 +73,12 @@ __device__ __forceinline__ void tile_stage_load(TileStage &st, const TileMap &m,
 }
 
 template <int kStride, bool kDigits>
-__device__ __forceinline__ void tile_stage_store(const TileStage &st, uint8_t *abuf, float *dxbuf, uint4 *digbuf, int tid) {
+__device__ __forceinline__ void tile_stage_store(const TileStage &st, uint8_t *abuf, float *dxbuf, uint4 *digbuf, int tid,
+                                                 uint32_t live) {
 #pragma unroll
     for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
         const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
-        *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kStride + (c & 31) * 8) = st.v[i];
+        if ((c >> 5) < live) *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kStride + (c & 31) * 8) = st.v[i];
     }
     if (tid < kMmToks) {
         dxbuf[tid] = st.dx;
@@ -78,28 +88,31 @@ __device__ __forceinline__ void tile_stage_store(const TileStage &st, uint8_t *a
 
 // One super-block of one 32-token tile against one Q4_K / Q5_K row share: I = sum_sb sc * (codes . a) and the mins sum
 // S = sum_sb mn * bsum32 (through the digits); returns d * I - dmin * S per result in `val`.
+// kJ = 1, 2 or 4: only the results of the tile's first 8 kJ tokens are finished on the vector units (result r of a lane
+// is token 8 * (r / 4) + 4 * khalf + r % 4, so they are the lane's first 4 kJ results); the matrix instructions always
+// compute all 32 tokens, which costs nothing extra.
 #define RNB_Q45_SUB_BLOCK(SB, ROW, TOT)                                                                  \
     {                                                                                                    \
         const v4i bop = q45_operand<SB, kFifth>(ROW);                                                    \
         const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                \
         const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * (SB));                               \
         const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);               \
-        _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                 \
+        _Pragma("unroll") for (int i = 0; i < 4 * kJ; i++) {                                             \
             TOT[i] += mul24(acc[i], sc);                                                                 \
             asm volatile("" : "+v"(TOT[i])); /* keep the eight additions a chain, not a tree */          \
         }                                                                                                \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 
-template <bool kFifth>
+template <bool kFifth, int kJ>
 __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *abase, const uint4 dig, int khalf,
-                                               float (&val)[16]) {
+                                               float (&val)[4 * kJ]) {
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const Q4KScales sc8 = unpack_q4k_scales(row.hdr.y, row.hdr.z, row.hdr.w);
-    int tot[16];
+    int tot[4 * kJ];
     if constexpr (kFifth) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) tot[i] = 0;
+        for (int i = 0; i < 4 * kJ; i++) tot[i] = 0;
         RNB_Q45_SUB_BLOCK(0, row, tot)
         RNB_Q45_SUB_BLOCK(1, row, tot)
         RNB_Q45_SUB_BLOCK(2, row, tot)
@@ -135,7 +148,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
         RNB_Q4_FOLD_SUB_BLOCK(7)
 #undef RNB_Q4_FOLD_SUB_BLOCK
 #pragma unroll
-        for (int i = 0; i < 16; i++) tot[i] = acc_lo[i] + 8 * acc_hi[i];
+        for (int i = 0; i < 4 * kJ; i++) tot[i] = acc_lo[i] + 8 * acc_hi[i];
     }
     const float d = f16_bits_to_f32(row.hdr.x), dmin = f16_bits_to_f32(row.hdr.x >> 16);
     // K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
@@ -145,7 +158,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
     const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op0, mnop, zero16, 0, 0, 0);
     const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op1, mnop, zero16, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 16; i++) val[i] = d * static_cast<float>(tot[i]) - dmin * static_cast<float>(c0[i] + 64 * c1[i]);
+    for (int i = 0; i < 4 * kJ; i++) val[i] = d * static_cast<float>(tot[i]) - dmin * static_cast<float>(c0[i] + 64 * c1[i]);
 }
 #undef RNB_Q45_SUB_BLOCK
 
@@ -156,17 +169,18 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
         const int sc = q6_scale<SB>(row);                                                                \
         const long aop = *reinterpret_cast<const long *>(abase + 16 * (SB));                             \
         const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);               \
-        _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                 \
+        _Pragma("unroll") for (int i = 0; i < 4 * kJ; i++) {                                             \
             tot[i] += mul24(acc[i], sc);                                                                 \
             asm volatile("" : "+v"(tot[i]));                                                             \
         }                                                                                                \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
-__device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *abase, float (&val)[16]) {
+template <int kJ>
+__device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *abase, float (&val)[4 * kJ]) {
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    int tot[16];
+    int tot[4 * kJ];
 #pragma unroll
-    for (int i = 0; i < 16; i++) tot[i] = 0;
+    for (int i = 0; i < 4 * kJ; i++) tot[i] = 0;
     RNB_Q6_TILE_SUB_BLOCK(0)
     RNB_Q6_TILE_SUB_BLOCK(1)
     RNB_Q6_TILE_SUB_BLOCK(2)
@@ -184,14 +198,15 @@ __device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *a
     RNB_Q6_TILE_SUB_BLOCK(14)
     RNB_Q6_TILE_SUB_BLOCK(15)
 #pragma unroll
-    for (int i = 0; i < 16; i++) val[i] = row.d * static_cast<float>(tot[i]);
+    for (int i = 0; i < 4 * kJ; i++) val[i] = row.d * static_cast<float>(tot[i]);
 }
 #undef RNB_Q6_TILE_SUB_BLOCK
 
 // accf[r] += d_x[token of result r] * val[r]; result r of a tile is token 8 * (r / 4) + 4 * khalf + r % 4
-__device__ __forceinline__ void tile_scale_add(const float *dxbuf, int khalf, const float (&val)[16], float (&accf)[16]) {
+template <int kJ>
+__device__ __forceinline__ void tile_scale_add(const float *dxbuf, int khalf, const float (&val)[4 * kJ], float (&accf)[4 * kJ]) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < kJ; j++) {
         const float4 dx4 = reinterpret_cast<const float4 *>(dxbuf)[2 * j + khalf];
         const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
@@ -199,90 +214,126 @@ __device__ __forceinline__ void tile_scale_add(const float *dxbuf, int khalf, co
     }
 }
 
-// LDS image of one tile: every 256-element block of the tile's tokens, staged once and then only read
-//   act[nb][32 tokens][kStride] | d_x[nb][32] | digits[nb][32] (16 bytes each; absent for Q6_K weights)
+// LDS image of one tile: every 256-element block of the tile's live tokens, staged once and then only read
+//   act[nb][toks][kStride] | d_x[nb][32] | digits[nb][32] (16 bytes each; absent for Q6_K weights)
+// toks <= 32 is the number of token rows the launch made room for (the largest group of the call, capped at a tile)
 template <int kStride, bool kDigits>
 struct TileImage {
-    static __host__ __device__ size_t act_bytes(uint32_t nb) { return static_cast<size_t>(nb) * kMmToks * kStride; }
-    static __host__ __device__ size_t bytes(uint32_t nb) {
-        return act_bytes(nb) + static_cast<size_t>(nb) * kMmToks * (4 + (kDigits ? 16 : 0));
+    static __host__ __device__ size_t act_bytes(uint32_t nb, uint32_t toks) { return static_cast<size_t>(nb) * toks * kStride; }
+    static __host__ __device__ size_t bytes(uint32_t nb, uint32_t toks = kMmToks) {
+        return act_bytes(nb, toks) + static_cast<size_t>(nb) * kMmToks * (4 + (kDigits ? 16 : 0));
     }
     uint8_t *base;
-    uint32_t nb;
-    __device__ uint8_t *act(uint32_t b) const { return base + static_cast<size_t>(b) * kMmToks * kStride; }
-    __device__ float *dx(uint32_t b) const { return reinterpret_cast<float *>(base + act_bytes(nb)) + b * kMmToks; }
+    uint32_t nb, toks;
+    __device__ uint8_t *act(uint32_t b) const { return base + static_cast<size_t>(b) * toks * kStride; }
+    __device__ float *dx(uint32_t b) const { return reinterpret_cast<float *>(base + act_bytes(nb, toks)) + b * kMmToks; }
     __device__ uint4 *dig(uint32_t b) const {
-        return reinterpret_cast<uint4 *>(base + act_bytes(nb) + static_cast<size_t>(nb) * kMmToks * 4) + b * kMmToks;
+        return reinterpret_cast<uint4 *>(base + act_bytes(nb, toks) + static_cast<size_t>(nb) * kMmToks * 4) + b * kMmToks;
     }
 };
 
 template <int kStride, bool kDigits>
 __device__ __forceinline__ void tile_image_fill(const TileImage<kStride, kDigits> &img, const TileMap &m,
                                                 const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                                                const uint8_t *__restrict__ adig, int tid) {
+                                                const uint8_t *__restrict__ adig, int tid, uint32_t live) {
     const uint32_t nb = img.nb;
     for (uint32_t b = 0; b < nb; b += 2) {  // two blocks' loads in flight before their stores
         TileStage st0, st1;
         const uint32_t b1 = b + 1 < nb ? b + 1 : b;
-        tile_stage_load<kDigits>(st0, m, aq, ad, adig, nb, b, tid);
-        tile_stage_load<kDigits>(st1, m, aq, ad, adig, nb, b1, tid);
-        tile_stage_store<kStride, kDigits>(st0, img.act(b), img.dx(b), img.dig(b), tid);
-        tile_stage_store<kStride, kDigits>(st1, img.act(b1), img.dx(b1), img.dig(b1), tid);
+        tile_stage_load<kDigits>(st0, m, aq, ad, adig, nb, b, tid, live);
+        tile_stage_load<kDigits>(st1, m, aq, ad, adig, nb, b1, tid, live);
+        tile_stage_store<kStride, kDigits>(st0, img.act(b), img.dx(b), img.dig(b), tid, live);
+        tile_stage_store<kStride, kDigits>(st1, img.act(b1), img.dx(b1), img.dig(b1), tid, live);
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // gate + up + SiLU * up.  Grid (row tiles of 128, expert groups).  The tile's activations are staged once, all blocks;
-// after that the waves run without barriers, each streaming its 32 rows of both matrices one block ahead.
+// after that the waves run without barriers, each streaming its 32 rows of both matrices one block ahead.  The rows
+// come in by whole cache lines as LDS-direct loads into the wave's two strips (consecutive lanes take consecutive
+// 16-byte pieces of a row, see RowRoute for why; no vector registers hold the data in flight), and each lane reads its
+// row's share back from there.  Dynamic LDS: the four waves' strips, then the tile image.
 // ---------------------------------------------------------------------------------------------
+template <int kJ>
 __global__ void __launch_bounds__(kGbThreads, 2)
     moe_gate_up_mfma_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const uint8_t *__restrict__ adig,
                             const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
                             const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
-                            float *__restrict__ mid, uint32_t n_ff, uint32_t nb) {
+                            float *__restrict__ mid, uint32_t n_ff, uint32_t nb, uint32_t img_toks) {
     constexpr bool kFifth = false;
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     __shared__ TileMap s_map;
-    const TileImage<kGbStride128, true> img{s_dyn, nb};
+    const TileImage<kGbStride128, true> img{s_dyn + kMmGateUpStripBytes, nb, img_toks};
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS-direct loads take their target from a scalar register
     const int lrow = lane & 31, khalf = lane >> 5;
+    uint8_t *strip_g = s_dyn + wave * 2 * kQ4FillBytes, *strip_u = strip_g + kQ4FillBytes;
+    const uint32_t lds_g = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)strip_g)), lds_u = lds_g + kQ4FillBytes;
     const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
-    const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
-    const size_t woff = (static_cast<size_t>(expert) * n_ff + min(row, n_ff - 1)) * row_bytes;
-    const uint8_t *grow = gate_all + woff, *urow = up_all + woff;
-
-    for (uint32_t tile0 = 0; tile0 < count; tile0 += kMmToks) {
-        // the first weight blocks do not depend on the token lists: requested before them
-        Q5Row cg = q45_load_row<kFifth>(grow, khalf), cu = q45_load_row<kFifth>(urow, khalf);
-        if (tile0) __syncthreads();  // the previous tile's readers of the map and the image are done
-        tile_map_fill(s_map, sorted_token, sorted_slot, nullptr, start + tile0, count - tile0, tid);
-        __syncthreads();
-        tile_image_fill(img, s_map, aq, ad, adig, tid);
-        __syncthreads();
-        float accg[16], accu[16];
+    const uint32_t row_bytes = nb * static_cast<uint32_t>(kQ4KBytes);
+    // the wave's first row (a wave wholly past the end streams the last row and stores nothing)
+    const uint32_t first = min(blockIdx.x * kGbRows + wave * 32, n_ff - 1);
+    const size_t woff = (static_cast<size_t>(expert) * n_ff + first) * row_bytes;
+    const uint8_t *gbase = gate_all + woff, *ubase = up_all + woff;
+    // piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at byte 16 c of
+    // the strip, which puts the rows 144 bytes apart (rows past the end of the matrix repeat the last row; the pieces past
+    // 288 of the fifth instruction repeat the last piece and land behind the rows)
+    uint32_t goff[kQ4FillInstr];
 #pragma unroll
-        for (int i = 0; i < 16; i++) accg[i] = accu[i] = 0.0f;
+    for (int i = 0; i < kQ4FillInstr; i++) {
+        const uint32_t c = min(static_cast<uint32_t>(lane) + i * kWave, 32u * kQ4Pieces - 1);
+        const uint32_t r = c / kQ4Pieces, j = c - r * kQ4Pieces;
+        goff[i] = min(r, n_ff - first - 1) * row_bytes + 16 * j;
+    }
+    auto request = [&](uint32_t b) {
+        // the strips' previous contents have been read out (the reads are ahead of these fills in program order; make
+        // sure they have executed)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const uint8_t *gsrc = gbase + b * static_cast<uint32_t>(kQ4KBytes), *usrc = ubase + b * static_cast<uint32_t>(kQ4KBytes);
+#pragma unroll
+        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(gsrc, goff[i], lds_g + i * 1024);
+#pragma unroll
+        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(usrc, goff[i], lds_u + i * 1024);
+    };
+    auto take = [&](Q5Row &g, Q5Row &u) {
+        wait_fills();
+        q4_row_from_strip(g, strip_g + lrow * kQ4StripStride, khalf);
+        q4_row_from_strip(u, strip_u + lrow * kQ4StripStride, khalf);
+    };
+
+    for (uint32_t tile0 = 0; tile0 < count; tile0 += img_toks) {
+        // the first weight blocks do not depend on the token lists: requested before them
+        request(0);
+        const uint32_t live = min(count - tile0, img_toks);
+        const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);  // padding lanes read the last live row
+        if (tile0) __syncthreads();  // the previous tile's readers of the map and the image are done
+        tile_map_fill(s_map, sorted_token, sorted_slot, nullptr, start + tile0, live, tid);
+        __syncthreads();
+        tile_image_fill(img, s_map, aq, ad, adig, tid, live);
+        Q5Row cg, cu;
+        take(cg, cu);
+        __syncthreads();
+        float accg[4 * kJ], accu[4 * kJ];
+#pragma unroll
+        for (int i = 0; i < 4 * kJ; i++) accg[i] = accu[i] = 0.0f;
         for (uint32_t b = 0; b < nb; b++) {
-            const uint32_t bn = b + 1 < nb ? b + 1 : b;  // the last step reloads its own block, unused
-            const Q5Row ng = q45_load_row<kFifth>(grow + static_cast<size_t>(bn) * kQ4KBytes, khalf);
-            const Q5Row nu = q45_load_row<kFifth>(urow + static_cast<size_t>(bn) * kQ4KBytes, khalf);
-            const uint8_t *abase = img.act(b) + lrow * kGbStride128 + 16 * khalf;
+            request(b + 1 < nb ? b + 1 : b);  // the last step reloads its own block, unused
+            const uint8_t *abase = img.act(b) + arow * kGbStride128 + 16 * khalf;
             const uint4 dig = img.dig(b)[lrow];
-            float val[16];
-            q45_block_tile<kFifth>(cg, abase, dig, khalf, val);
-            tile_scale_add(img.dx(b), khalf, val, accg);
-            q45_block_tile<kFifth>(cu, abase, dig, khalf, val);
-            tile_scale_add(img.dx(b), khalf, val, accu);
-            cg = ng;
-            cu = nu;
+            float val[4 * kJ];
+            q45_block_tile<kFifth, kJ>(cg, abase, dig, khalf, val);
+            tile_scale_add<kJ>(img.dx(b), khalf, val, accg);
+            q45_block_tile<kFifth, kJ>(cu, abase, dig, khalf, val);
+            tile_scale_add<kJ>(img.dx(b), khalf, val, accu);
+            take(cg, cu);
         }
         if (row < n_ff) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
+            for (int r = 0; r < 4 * kJ; r++) {
                 const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
                 if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
             }
@@ -293,20 +344,20 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 // ---------------------------------------------------------------------------------------------
 // down projection of the re-quantised intermediate, scaled by the route weight.  Grid (row tiles of 128, expert groups).
 // ---------------------------------------------------------------------------------------------
-template <uint32_t kQuant>
+template <uint32_t kQuant, int kJ>
 __global__ void __launch_bounds__(kGbThreads, 2)
     moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
                          const uint8_t *__restrict__ mdig, const uint32_t *__restrict__ grp_expert,
                          const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
                          const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
-                         uint32_t tiles_per_wg) {
+                         uint32_t tiles_per_wg, uint32_t img_toks) {
     constexpr bool kSix = kQuant == kQ6K;
     constexpr bool kFifth = kQuant == kQ5K;
     constexpr int kStride = kSix ? kGbStride64 : kGbStride128;
     constexpr size_t kBlockBytes = kSix ? kQ6KBytes : (kFifth ? kQ5KBytes : kQ4KBytes);
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     __shared__ TileMap s_map;
-    const TileImage<kStride, !kSix> img{s_dyn, nb};
+    const TileImage<kStride, !kSix> img{s_dyn, nb, img_toks};
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid >> 6;
     const int lrow = lane & 31, khalf = lane >> 5;
@@ -343,7 +394,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         r.d = d_next;
     };
 
-    for (uint32_t tile0 = 0; tile0 < count; tile0 += kMmToks) {
+    for (uint32_t tile0 = 0; tile0 < count; tile0 += img_toks) {
         Q6Row c6{};
         Q5Row c5{};
         // the first weight block does not depend on the token lists: requested before them
@@ -352,14 +403,16 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         else
             c5 = q45_load_row<kFifth>(block_ptr(0, 0), khalf);
         if (tile0) __syncthreads();
-        tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, count - tile0, tid);
+        const uint32_t live = min(count - tile0, img_toks);
+        const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);
+        tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, live, tid);
         __syncthreads();
-        tile_image_fill(img, s_map, mq, md, mdig, tid);
+        tile_image_fill(img, s_map, mq, md, mdig, tid, live);
         if constexpr (kSix) q6_take(c6);
         __syncthreads();
-        float accf[16];
+        float accf[4 * kJ];
 #pragma unroll
-        for (int i = 0; i < 16; i++) accf[i] = 0.0f;
+        for (int i = 0; i < 4 * kJ; i++) accf[i] = 0.0f;
         uint32_t rt = 0, b = 0;
         for (uint32_t s = 0; s < steps; s++) {
             uint32_t rtn = rt, bn = b + 1;  // the step after this one; the last step reloads its own block, unused
@@ -372,22 +425,22 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                 bn = b;
             }
             Q5Row n5{};
-            float val[16];
+            float val[4 * kJ];
             if constexpr (kSix) {
                 q6_request(rtn, bn);
-                q6_block_tile(c6, img.act(b) + lrow * kStride + 8 * khalf, val);
+                q6_block_tile<kJ>(c6, img.act(b) + arow * kStride + 8 * khalf, val);
             } else {
                 n5 = q45_load_row<kFifth>(block_ptr(rtn, bn), khalf);
-                q45_block_tile<kFifth>(c5, img.act(b) + lrow * kStride + 16 * khalf, img.dig(b)[lrow], khalf, val);
+                q45_block_tile<kFifth, kJ>(c5, img.act(b) + arow * kStride + 16 * khalf, img.dig(b)[lrow], khalf, val);
             }
-            tile_scale_add(img.dx(b), khalf, val, accf);
+            tile_scale_add<kJ>(img.dx(b), khalf, val, accf);
             if constexpr (kSix) q6_take(c6);
             c5 = n5;
             if (b + 1 == nb) {  // the row tile is complete
                 const uint32_t row = row_of(rt);
                 if (row < n_embd) {
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
+                    for (int r = 0; r < 4 * kJ; r++) {
                         const int t = 8 * (r >> 2) + 4 * khalf + (r & 3);
                         const uint32_t slot = s_map.out_row[t];
                         // fanout.rs:306-308: the expert's output times the slot's route weight
@@ -396,7 +449,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 16; i++) accf[i] = 0.0f;
+                for (int i = 0; i < 4 * kJ; i++) accf[i] = 0.0f;
             }
             rt = rtn;
             b = bn;
@@ -414,24 +467,49 @@ bool allow_lds(K kernel, size_t bytes) {
 
 }  // namespace
 
-// the tile image (all blocks of 32 tokens) must fit the LDS of a compute unit beside the small static arrays
+// the tile image (all blocks of the tile's tokens) must fit the LDS of a compute unit beside the waves' strips and the
+// small static arrays; a tile holds as many tokens as fit, at most 32
 constexpr size_t kMmLdsLimit = 150 * 1024;
-constexpr size_t kMmQ6DownLdsLimit = kMmLdsLimit - kGbWaves * 32 * kQ6StripStride;  // beside the four waves' strips
+constexpr size_t kMmGateUpImageLimit = kMmLdsLimit - kMmGateUpStripBytes;
+constexpr size_t kMmQ6DownLdsLimit = kMmLdsLimit - kGbWaves * 32 * kQ6StripStride;
+constexpr uint32_t kMmMinToks = 16;  // below this the matrix-core path re-reads the weights too often to pay
+
+template <int kStride, bool kDigits>
+static uint32_t tile_tokens_that_fit(size_t limit, uint32_t nb) {
+    uint32_t toks = kMmToks;
+    while (toks > 0 && TileImage<kStride, kDigits>::bytes(nb, toks) > limit) toks--;
+    return toks;
+}
+static uint32_t gate_up_tile_tokens(uint32_t nb_in) { return tile_tokens_that_fit<kGbStride128, true>(kMmGateUpImageLimit, nb_in); }
+static uint32_t down_tile_tokens(uint32_t nb_mid, uint32_t down_quant) {
+    return down_quant == kQ6K ? tile_tokens_that_fit<kGbStride64, false>(kMmQ6DownLdsLimit, nb_mid)
+                              : tile_tokens_that_fit<kGbStride128, true>(kMmLdsLimit, nb_mid);
+}
 
 bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
-    const size_t gu = TileImage<kGbStride128, true>::bytes(nb_in);
-    const size_t dn = down_quant == kQ6K ? TileImage<kGbStride64, false>::bytes(nb_mid) : TileImage<kGbStride128, true>::bytes(nb_mid);
-    return nb_in >= 1 && nb_mid >= 1 && gu <= kMmLdsLimit && dn <= (down_quant == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit);
+    return nb_in >= 1 && nb_mid >= 1 && gate_up_tile_tokens(nb_in) >= kMmMinToks && down_tile_tokens(nb_mid, down_quant) >= kMmMinToks;
 }
 
 void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                              uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0 || n_ff == 0) return;
-    const size_t lds = TileImage<kGbStride128, true>::bytes(nb_in);
-    if (!allow_lds<0>(moe_gate_up_mfma_kernel, kMmLdsLimit)) return;
+    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
+    if (toks == 0) return;  // moe_mfma_supported said no
+    const size_t lds = kMmGateUpStripBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
     const dim3 grid((n_ff + kGbRows - 1) / kGbRows, groups.n_groups, 1);
-    hipLaunchKernelGGL(moe_gate_up_mfma_kernel, grid, dim3(kGbThreads), lds, stream, gate_all, up_all, act.qs, act.d, act.digits,
-                       groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in);
+    // tiles of at most 8 / 16 / 32 tokens: the kernel finishes only that many results per lane
+#define RNB_LAUNCH_GU(J)                                                                                              \
+    if (!allow_lds<J>(moe_gate_up_mfma_kernel<J>, kMmLdsLimit)) return;                                               \
+    hipLaunchKernelGGL(moe_gate_up_mfma_kernel<J>, grid, dim3(kGbThreads), lds, stream, gate_all, up_all, act.qs, act.d, \
+                       act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
+    if (toks <= 8) {
+        RNB_LAUNCH_GU(1);
+    } else if (toks <= 16) {
+        RNB_LAUNCH_GU(2);
+    } else {
+        RNB_LAUNCH_GU(4);
+    }
+#undef RNB_LAUNCH_GU
 }
 
 void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
@@ -445,18 +523,29 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView 
     while (tiles_per_wg < 4 && static_cast<uint64_t>((row_tiles + tiles_per_wg - 1) / tiles_per_wg) * groups.n_groups > 768)
         tiles_per_wg *= 2;
     const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1), block(kGbThreads);
+    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), down_tile_tokens(nb_mid, down_quant));
+    if (toks == 0) return;
+#define RNB_LAUNCH_DMJ(Q, J, LDS)                                                                                     \
+    if (!allow_lds<static_cast<int>(Q) * 8 + J>(moe_down_mfma_kernel<Q, J>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return; \
+    hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
+                       groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg, toks)
 #define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
-    if (!allow_lds<static_cast<int>(Q)>(moe_down_mfma_kernel<Q>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return;                            \
-    hipLaunchKernelGGL((moe_down_mfma_kernel<Q>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
-                       groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg)
+    if (toks <= 8) {                                                                                                  \
+        RNB_LAUNCH_DMJ(Q, 1, LDS);                                                                                    \
+    } else if (toks <= 16) {                                                                                          \
+        RNB_LAUNCH_DMJ(Q, 2, LDS);                                                                                    \
+    } else {                                                                                                          \
+        RNB_LAUNCH_DMJ(Q, 4, LDS);                                                                                    \
+    }
     if (down_quant == kQ6K) {
-        RNB_LAUNCH_DM(kQ6K, (TileImage<kGbStride64, false>::bytes(nb_mid)));
+        RNB_LAUNCH_DM(kQ6K, (TileImage<kGbStride64, false>::bytes(nb_mid, toks)));
     } else if (down_quant == kQ5K) {
-        RNB_LAUNCH_DM(kQ5K, (TileImage<kGbStride128, true>::bytes(nb_mid)));
+        RNB_LAUNCH_DM(kQ5K, (TileImage<kGbStride128, true>::bytes(nb_mid, toks)));
     } else {
-        RNB_LAUNCH_DM(kQ4K, (TileImage<kGbStride128, true>::bytes(nb_mid)));
+        RNB_LAUNCH_DM(kQ4K, (TileImage<kGbStride128, true>::bytes(nb_mid, toks)));
     }
 #undef RNB_LAUNCH_DM
+#undef RNB_LAUNCH_DMJ
 }
 
 }  // namespace rnb
