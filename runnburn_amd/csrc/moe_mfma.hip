@@ -16,6 +16,7 @@
 #include "kernels.h"
 #include "mfma_blocks.h"
 #include <algorithm>
+#include <cstdlib>
 
 namespace rnb {
 
@@ -46,19 +47,21 @@ __device__ __forceinline__ void tile_map_fill(TileMap &m, const uint32_t *__rest
 }
 
 // the tile's quantised activations of block b (256 int8 per token, 8-byte chunks), scale and digits
+template <int kThreads>
 struct TileStage {
-    uint2 v[kMmToks * 32 / kGbThreads];  // 4 chunks per thread
+    static constexpr int kN = (kMmToks * 32 + kThreads - 1) / kThreads;  // chunks per thread
+    uint2 v[kN];
     float dx;
     uint4 dig;
 };
 
-template <bool kDigits>
-__device__ __forceinline__ void tile_stage_load(TileStage &st, const TileMap &m, const int8_t *__restrict__ aq,
+template <bool kDigits, int kThreads>
+__device__ __forceinline__ void tile_stage_load(TileStage<kThreads> &st, const TileMap &m, const int8_t *__restrict__ aq,
                                                 const float *__restrict__ ad, const uint8_t *__restrict__ adig, size_t nb,
                                                 size_t b, int tid, uint32_t live) {
 #pragma unroll
-    for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
-        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+    for (int i = 0; i < TileStage<kThreads>::kN; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kThreads;
         st.v[i] = make_uint2(0, 0);
         if ((c >> 5) < live)
             st.v[i] = *reinterpret_cast<const uint2 *>(aq + (static_cast<size_t>(m.act_row[c >> 5]) * nb + b) * 256 + (c & 31) * 8);
@@ -72,12 +75,12 @@ __device__ __forceinline__ void tile_stage_load(TileStage &st, const TileMap &m,
     }
 }
 
-template <int kStride, bool kDigits>
-__device__ __forceinline__ void tile_stage_store(const TileStage &st, uint8_t *abuf, float *dxbuf, uint4 *digbuf, int tid,
+template <int kStride, bool kDigits, int kThreads>
+__device__ __forceinline__ void tile_stage_store(const TileStage<kThreads> &st, uint8_t *abuf, float *dxbuf, uint4 *digbuf, int tid,
                                                  uint32_t live) {
 #pragma unroll
-    for (int i = 0; i < kMmToks * 32 / kGbThreads; i++) {
-        const uint32_t c = static_cast<uint32_t>(tid) + i * kGbThreads;
+    for (int i = 0; i < TileStage<kThreads>::kN; i++) {
+        const uint32_t c = static_cast<uint32_t>(tid) + i * kThreads;
         if ((c >> 5) < live) *reinterpret_cast<uint2 *>(abuf + (c >> 5) * kStride + (c & 31) * 8) = st.v[i];
     }
     if (tid < kMmToks) {
@@ -232,18 +235,18 @@ struct TileImage {
     }
 };
 
-template <int kStride, bool kDigits>
+template <int kThreads, int kStride, bool kDigits>
 __device__ __forceinline__ void tile_image_fill(const TileImage<kStride, kDigits> &img, const TileMap &m,
                                                 const int8_t *__restrict__ aq, const float *__restrict__ ad,
                                                 const uint8_t *__restrict__ adig, int tid, uint32_t live) {
     const uint32_t nb = img.nb;
     for (uint32_t b = 0; b < nb; b += 2) {  // two blocks' loads in flight before their stores
-        TileStage st0, st1;
+        TileStage<kThreads> st0, st1;
         const uint32_t b1 = b + 1 < nb ? b + 1 : b;
-        tile_stage_load<kDigits>(st0, m, aq, ad, adig, nb, b, tid, live);
-        tile_stage_load<kDigits>(st1, m, aq, ad, adig, nb, b1, tid, live);
-        tile_stage_store<kStride, kDigits>(st0, img.act(b), img.dx(b), img.dig(b), tid, live);
-        tile_stage_store<kStride, kDigits>(st1, img.act(b1), img.dx(b1), img.dig(b1), tid, live);
+        tile_stage_load<kDigits, kThreads>(st0, m, aq, ad, adig, nb, b, tid, live);
+        tile_stage_load<kDigits, kThreads>(st1, m, aq, ad, adig, nb, b1, tid, live);
+        tile_stage_store<kStride, kDigits, kThreads>(st0, img.act(b), img.dx(b), img.dig(b), tid, live);
+        tile_stage_store<kStride, kDigits, kThreads>(st1, img.act(b1), img.dx(b1), img.dig(b1), tid, live);
     }
 }
 
@@ -254,8 +257,8 @@ __device__ __forceinline__ void tile_image_fill(const TileImage<kStride, kDigits
 // 16-byte pieces of a row, see RowRoute for why; no vector registers hold the data in flight), and each lane reads its
 // row's share back from there.  Dynamic LDS: the four waves' strips, then the tile image.
 // ---------------------------------------------------------------------------------------------
-template <int kJ>
-__global__ void __launch_bounds__(kGbThreads, 2)
+template <int kJ, int kW>
+__global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * kW), amdgpu_waves_per_eu(2)))
     moe_gate_up_mfma_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const uint8_t *__restrict__ adig,
                             const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
@@ -264,19 +267,19 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     constexpr bool kFifth = false;
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     __shared__ TileMap s_map;
-    const TileImage<kGbStride128, true> img{s_dyn + kMmGateUpStripBytes, nb, img_toks};
+    const TileImage<kGbStride128, true> img{s_dyn + kW * 2 * kQ4FillBytes, nb, img_toks};
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS-direct loads take their target from a scalar register
     const int lrow = lane & 31, khalf = lane >> 5;
     uint8_t *strip_g = s_dyn + wave * 2 * kQ4FillBytes, *strip_u = strip_g + kQ4FillBytes;
     const uint32_t lds_g = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)strip_g)), lds_u = lds_g + kQ4FillBytes;
-    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t row = blockIdx.x * (32 * kW) + wave * 32 + lrow;
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const uint32_t row_bytes = nb * static_cast<uint32_t>(kQ4KBytes);
     // the wave's first row (a wave wholly past the end streams the last row and stores nothing)
-    const uint32_t first = min(blockIdx.x * kGbRows + wave * 32, n_ff - 1);
+    const uint32_t first = min(blockIdx.x * (32 * kW) + wave * 32, n_ff - 1);
     const size_t woff = (static_cast<size_t>(expert) * n_ff + first) * row_bytes;
     const uint8_t *gbase = gate_all + woff, *ubase = up_all + woff;
     // piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at byte 16 c of
@@ -313,7 +316,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         if (tile0) __syncthreads();  // the previous tile's readers of the map and the image are done
         tile_map_fill(s_map, sorted_token, sorted_slot, nullptr, start + tile0, live, tid);
         __syncthreads();
-        tile_image_fill(img, s_map, aq, ad, adig, tid, live);
+        tile_image_fill<kWave * kW>(img, s_map, aq, ad, adig, tid, live);
         Q5Row cg, cu;
         take(cg, cu);
         __syncthreads();
@@ -407,7 +410,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);
         tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, live, tid);
         __syncthreads();
-        tile_image_fill(img, s_map, mq, md, mdig, tid, live);
+        tile_image_fill<kGbThreads>(img, s_map, mq, md, mdig, tid, live);
         if constexpr (kSix) q6_take(c6);
         __syncthreads();
         float accf[4 * kJ];
@@ -493,15 +496,28 @@ bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
 void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                              uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0 || n_ff == 0) return;
-    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
+    uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
     if (toks == 0) return;  // moe_mfma_supported said no
-    const size_t lds = kMmGateUpStripBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
-    const dim3 grid((n_ff + kGbRows - 1) / kGbRows, groups.n_groups, 1);
+    int waves = kGbWaves;
+    if (const char *e = getenv("RNB_PROBE_GU_WAVES")) waves = atoi(e);
+    const size_t lds = static_cast<size_t>(waves) * 2 * kQ4FillBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
+    const uint32_t rows_per_wg = 32 * waves;
+    const dim3 grid((n_ff + rows_per_wg - 1) / rows_per_wg, groups.n_groups, 1);
     // tiles of at most 8 / 16 / 32 tokens: the kernel finishes only that many results per lane
-#define RNB_LAUNCH_GU(J)                                                                                              \
-    if (!allow_lds<J>(moe_gate_up_mfma_kernel<J>, kMmLdsLimit)) return;                                               \
-    hipLaunchKernelGGL(moe_gate_up_mfma_kernel<J>, grid, dim3(kGbThreads), lds, stream, gate_all, up_all, act.qs, act.d, \
+#define RNB_LAUNCH_GUW(J, W)                                                                                          \
+    if (!allow_lds<J * 16 + W>(moe_gate_up_mfma_kernel<J, W>, kMmLdsLimit)) return;                                   \
+    hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, act.qs, act.d, \
                        act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
+#define RNB_LAUNCH_GU(J)                                                                                              \
+    if (waves == 2) {                                                                                                 \
+        RNB_LAUNCH_GUW(J, 2);                                                                                         \
+    } else if (waves == 3) {                                                                                          \
+        RNB_LAUNCH_GUW(J, 3);                                                                                         \
+    } else if (waves == 6) {                                                                                          \
+        RNB_LAUNCH_GUW(J, 6);                                                                                         \
+    } else {                                                                                                          \
+        RNB_LAUNCH_GUW(J, 4);                                                                                         \
+    }
     if (toks <= 8) {
         RNB_LAUNCH_GU(1);
     } else if (toks <= 16) {
@@ -510,6 +526,7 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
         RNB_LAUNCH_GU(4);
     }
 #undef RNB_LAUNCH_GU
+#undef RNB_LAUNCH_GUW
 }
 
 void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
@@ -523,8 +540,9 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView 
     while (tiles_per_wg < 4 && static_cast<uint64_t>((row_tiles + tiles_per_wg - 1) / tiles_per_wg) * groups.n_groups > 768)
         tiles_per_wg *= 2;
     const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1), block(kGbThreads);
-    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), down_tile_tokens(nb_mid, down_quant));
+    uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), down_tile_tokens(nb_mid, down_quant));
     if (toks == 0) return;
+    if (const char *e = getenv("RNB_PROBE_CAP_DN")) toks = std::min<uint32_t>(toks, atoi(e));
 #define RNB_LAUNCH_DMJ(Q, J, LDS)                                                                                     \
     if (!allow_lds<static_cast<int>(Q) * 8 + J>(moe_down_mfma_kernel<Q, J>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return; \
     hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \

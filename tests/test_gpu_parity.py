@@ -331,14 +331,16 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
                                              (Q4_K, 5, 256), (Q4_K, 20001, 256), (Q6_K, 9001, 1024), (Q5_K, 4099, 4096),
                                              (Q3_K, 8200, 2304), (Q8_0, 4100, 2048), (Q8_0, 5000, 2080), (2, 2100, 4096), (3, 8200, 1056),
                                              (6, 4100, 4096), (7, 90000, 96), (9, 4100, 2048), (9, 50, 96), (Q4_K, 4096, 14336), (Q6_K, 4099, 11008),
-                                             (Q4_K, 37, 4352), (Q5_K, 300, 8192), (Q6_K, 9, 16384), (Q2_K, 100, 16640)])
+                                             (Q4_K, 37, 4352), (Q5_K, 300, 8192), (Q6_K, 9, 16384), (Q2_K, 100, 16640),
+                                             (Q4_K, 33, 32768), (Q6_K, 21, 33024), (Q3_K, 4101, 5120), (Q6_K, 1030, 28672)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
     feed several matrices from one activation) run the same arithmetic: identical bits.  For K-quant rows of at most
-    16 super-blocks, and 32-element formats with rows of at most 128 blocks, gemv_dev is the one-launch kernel whose
-    workgroups quantise the token themselves (longer rows keep the separate quantiser: a one-launch split-K form,
-    every wave quantising its own 16 super-blocks, measured 19.8 against 15.5 us on 4096 x 14336 Q6_K); the shapes cover
-    1, 2 and 4 rows per wave, row counts that are no multiple of those, and more row groups than waves."""
+    128 super-blocks, and 32-element formats with rows of at most 128 blocks, gemv_dev is a one-launch kernel whose
+    workgroups quantise the token themselves (rows of more than 16 super-blocks: sixteen-wave workgroups that quantise
+    the token once and split K across their waves; 129 super-blocks and more keep the separate quantiser); the shapes
+    cover 1, 2 and 4 rows per wave, row counts that are no multiple of those, more row groups than waves, and 2 to 8
+    K slices with full and partly idle last slices."""
     w = oracle.make_weights(quant, rows, cols, 900 + rows)
     x = oracle.fill_normal(cols, 901 + cols, 1.0)
     wd, xd = rnb.DeviceBuffer.from_host(w), rnb.DeviceBuffer.from_host(x)
