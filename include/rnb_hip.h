@@ -47,6 +47,10 @@ typedef enum {
 #define RNB_GGML_Q4_K 12u
 #define RNB_GGML_Q5_K 13u
 #define RNB_GGML_Q6_K 14u
+#define RNB_GGML_IQ2_XXS 16u
+#define RNB_GGML_IQ3_XXS 18u
+#define RNB_GGML_IQ2_S 22u
+#define RNB_GGML_IQ4_XS 23u
 
 /* BackendOp, crates/rnb-backend/api/src/lib.rs:12-18 */
 #define RNB_OP_MATMUL 0
@@ -61,7 +65,7 @@ typedef enum {
 int rnb_hip_backend_kind(void);
 /* capabilities(): 1 when `op` (RNB_OP_*) executes on this backend, else 0. */
 int rnb_hip_backend_supports(int op);
-/* 1 when (op, ggml quant id) is supported: MatMul x {Q4_0,Q4_1,Q5_0,Q5_1,Q8_0,Q8_1,Q2_K..Q6_K}; MoE x gate/up Q4_K with
+/* 1 when (op, ggml quant id) is supported: MatMul x {Q4_0,Q4_1,Q5_0,Q5_1,Q8_0,Q8_1,Q2_K..Q6_K,IQ2_XXS,IQ2_S,IQ3_XXS,IQ4_XS}; MoE x gate/up Q4_K with
  * down Q4_K|Q5_K|Q6_K (pass the down quant). */
 int rnb_hip_backend_supports_quant(int op, uint32_t quant);
 
@@ -161,6 +165,26 @@ int rnb_hip_q3k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, c
                      size_t x_len, float *out, size_t out_len);
 int rnb_hip_q3k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                            const float *x, size_t x_len, float *out, size_t out_len);
+/* iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv and their batch forms, quant_api.rs:543-722 (same checks and
+ * texts): importance-quant rows (66 / 82 / 98 / 136-byte blocks of 256 elements) x Q8_K(x), the block dots of
+ * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Every
+ * batch size runs one GEMV pass per token. */
+int rnb_hip_iq2_xxs_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                         size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq2_xxs_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                               const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq2_s_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                       size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq2_s_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                             const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq3_xxs_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                         size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq3_xxs_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                               const float *x, size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq4_xs_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
+                        size_t x_len, float *out, size_t out_len);
+int rnb_hip_iq4_xs_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                              const float *x, size_t x_len, float *out, size_t out_len);
 /* q5k_gemv / q5k_gemv_into, quant_api.rs:2207-2281: Q5_K rows (176-byte blocks) x Q8_K(x), the block dot of
  * crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800 */
 int rnb_hip_q5k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,

@@ -17,8 +17,12 @@ _LIB_PATH = os.path.join(_HERE, "librnb_oracle.so")
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_1 = 2, 3, 6, 7, 9
 LEGACY = (Q4_0, Q4_1, Q5_0, Q5_1, Q8_1)  # 32-element blocks other than Q8_0, dotted against 32-wide Q8 activations
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14  # ggml type ids (crates/rnb-loader/src/gguf/types.rs:5-41)
-BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210}
-BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q2_K: 256, Q3_K: 256, Q4_K: 256, Q5_K: 256, Q6_K: 256}
+IQ2_XXS, IQ3_XXS, IQ2_S, IQ4_XS = 16, 18, 22, 23  # importance quants (crates/rnb-cpu/src/quantize/iq.rs), against Q8_K activations
+IQ = (IQ2_XXS, IQ3_XXS, IQ2_S, IQ4_XS)
+BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210,
+               IQ2_XXS: 66, IQ3_XXS: 98, IQ2_S: 82, IQ4_XS: 136}
+BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q2_K: 256, Q3_K: 256, Q4_K: 256, Q5_K: 256, Q6_K: 256,
+               IQ2_XXS: 256, IQ3_XXS: 256, IQ2_S: 256, IQ4_XS: 256}
 
 Q8K_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (256,)), ("bsums", "<i2", (16,))])
 Q8_DTYPE = np.dtype([("d", "<f4"), ("qs", "i1", (32,))])
@@ -50,7 +54,8 @@ def lib() -> C.CDLL:
         L.rnbo_get_scale_min_k4.restype = None
         L.rnbo_get_scale_min_k4.argtypes = [i32, vp, vp, vp]
         for name in ("rnbo_dequantize_q8_0", "rnbo_dequantize_q2_k", "rnbo_dequantize_q3_k", "rnbo_dequantize_q4_k",
-                     "rnbo_dequantize_q5_k", "rnbo_dequantize_q6_k"):
+                     "rnbo_dequantize_q5_k", "rnbo_dequantize_q6_k", "rnbo_dequantize_iq2_xxs", "rnbo_dequantize_iq2_s",
+                     "rnbo_dequantize_iq3_xxs", "rnbo_dequantize_iq4_xs"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, sz, vp]
         for name in ("rnbo_quantize_q8k", "rnbo_quantize_q8"):
@@ -95,6 +100,12 @@ def lib() -> C.CDLL:
         L.rnbo_make_weights.argtypes = [u32, sz, sz, u64, f32, vp, i32]
         L.rnbo_have_avx2.restype = i32
         L.rnbo_have_avx2.argtypes = []
+        L.rnbo_dot_iq_q8k.restype = f32
+        L.rnbo_dot_iq_q8k.argtypes = [u32, vp, vp, sz]
+        L.rnbo_dot_iq_q8k_f64.restype = C.c_double
+        L.rnbo_dot_iq_q8k_f64.argtypes = [u32, vp, vp, sz]
+        L.rnbo_iq_grid.restype = sz
+        L.rnbo_iq_grid.argtypes = [i32, vp]
         _lib = L
     return _lib
 
@@ -146,9 +157,18 @@ def dequantize(quant: int, blocks) -> np.ndarray:
         assert lib().rnbo_dequantize_legacy(quant, _p(b), n, _p(out)) == 0
         return out
     fn = {Q8_0: "rnbo_dequantize_q8_0", Q2_K: "rnbo_dequantize_q2_k", Q3_K: "rnbo_dequantize_q3_k",
-          Q4_K: "rnbo_dequantize_q4_k", Q5_K: "rnbo_dequantize_q5_k", Q6_K: "rnbo_dequantize_q6_k"}[quant]
+          Q4_K: "rnbo_dequantize_q4_k", Q5_K: "rnbo_dequantize_q5_k", Q6_K: "rnbo_dequantize_q6_k",
+          IQ2_XXS: "rnbo_dequantize_iq2_xxs", IQ2_S: "rnbo_dequantize_iq2_s", IQ3_XXS: "rnbo_dequantize_iq3_xxs",
+          IQ4_XS: "rnbo_dequantize_iq4_xs"}[quant]
     getattr(lib(), fn)(_p(b), n, _p(out))
     return out
+
+
+def iq_grid(which: int) -> np.ndarray:
+    """The expanded codebook: 0 IQ2_XXS (256 entries of 8 bytes), 1 IQ2_S (1024 of 8), 2 IQ3_XXS (256 of 4, widened)."""
+    out = np.zeros(1024, dtype=np.uint64)
+    n = lib().rnbo_iq_grid(which, _p(out))
+    return out[:n]
 
 
 # ---- activation quantisers ----------------------------------------------------------
@@ -179,6 +199,11 @@ def dot(quant: int, row, act: np.ndarray, gold: bool = False, avx2: bool = False
         assert not avx2
         act = np.ascontiguousarray(act)
         fn = lib().rnbo_dot_legacy_q8_f64 if gold else lib().rnbo_dot_legacy_q8
+        return float(fn(quant, _p(r), _p(act), nb))
+    if quant in IQ:
+        assert not avx2
+        act = np.ascontiguousarray(act)
+        fn = lib().rnbo_dot_iq_q8k_f64 if gold else lib().rnbo_dot_iq_q8k
         return float(fn(quant, _p(r), _p(act), nb))
     base = {Q8_0: "rnbo_dot_q8_0_q8", Q2_K: "rnbo_dot_q2k_q8k", Q3_K: "rnbo_dot_q3k_q8k", Q4_K: "rnbo_dot_q4k_q8k",
             Q5_K: "rnbo_dot_q5k_q8k", Q6_K: "rnbo_dot_q6k_q8k"}[quant]

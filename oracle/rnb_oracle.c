@@ -777,6 +777,10 @@ static size_t block_bytes_of(uint32_t quant, size_t *elems) {
     case 12: *elems = 256; return RNBO_Q4_K_BLOCK_BYTES;
     case 13: *elems = 256; return RNBO_Q5_K_BLOCK_BYTES;
     case 14: *elems = 256; return RNBO_Q6_K_BLOCK_BYTES;
+    case 16: *elems = 256; return RNBO_IQ2_XXS_BLOCK_BYTES;
+    case 18: *elems = 256; return RNBO_IQ3_XXS_BLOCK_BYTES;
+    case 22: *elems = 256; return RNBO_IQ2_S_BLOCK_BYTES;
+    case 23: *elems = 256; return RNBO_IQ4_XS_BLOCK_BYTES;
     default: *elems = 0; return 0;
     }
 }
@@ -787,6 +791,7 @@ static float kquant_dot(uint32_t quant, const uint8_t *row, const rnbo_q8k_block
     case 11: return rnbo_dot_q3k_q8k(row, act, nb);
     case 12: return rnbo_dot_q4k_q8k(row, act, nb);
     case 13: return rnbo_dot_q5k_q8k(row, act, nb);
+    case 16: case 18: case 22: case 23: return rnbo_dot_iq_q8k(quant, row, act, nb);
     default: return rnbo_dot_q6k_q8k(row, act, nb);
     }
 }
@@ -797,6 +802,7 @@ static double kquant_dot_f64(uint32_t quant, const uint8_t *row, const rnbo_q8k_
     case 11: return rnbo_dot_q3k_q8k_f64(row, act, nb);
     case 12: return rnbo_dot_q4k_q8k_f64(row, act, nb);
     case 13: return rnbo_dot_q5k_q8k_f64(row, act, nb);
+    case 16: case 18: case 22: case 23: return rnbo_dot_iq_q8k_f64(quant, row, act, nb);
     default: return rnbo_dot_q6k_q8k_f64(row, act, nb);
     }
 }
@@ -1528,7 +1534,9 @@ int rnbo_make_weights(uint32_t quant, size_t rows, size_t cols, uint64_t seed, f
         for (long r = 0; r < (long)rows; r++) {
             for (size_t c = 0; c < cols; c++) row[c] = normal_at(seed, (uint64_t)r * cols + c, sigma);
             uint8_t *dst = out + (size_t)r * row_bytes;
-            if (quant == 2 || quant == 3 || quant == 6 || quant == 7 || quant == 9)
+            if (quant == 16 || quant == 18 || quant == 22 || quant == 23)
+                rnbo_make_iq_row(quant, cols / 256, seed * 1000003ull + (uint64_t)r, sigma, dst);
+            else if (quant == 2 || quant == 3 || quant == 6 || quant == 7 || quant == 9)
                 rnbo_quantize_row_legacy(quant, row, cols, dst);
             else if (quant == 10)
                 rnbo_quantize_row_q2_k(row, cols, dst);

@@ -35,6 +35,11 @@ extern "C" {
 #define RNBO_Q4_K_BLOCK_BYTES 144
 #define RNBO_Q5_K_BLOCK_BYTES 176
 #define RNBO_Q6_K_BLOCK_BYTES 210
+/* importance quants (ggml type ids 16, 22, 18, 23), crates/rnb-cpu/src/quantize/iq.rs:23-116 */
+#define RNBO_IQ2_XXS_BLOCK_BYTES 66
+#define RNBO_IQ2_S_BLOCK_BYTES 82
+#define RNBO_IQ3_XXS_BLOCK_BYTES 98
+#define RNBO_IQ4_XS_BLOCK_BYTES 136
 
 /* Q8_K activation block, crates/rnb-cpu/src/gemm/activation_q8.rs:66-72 (repr(C), 292 B). */
 typedef struct {
@@ -86,6 +91,20 @@ double rnbo_dot_q4k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_
 double rnbo_dot_q5k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 double rnbo_dot_q6k_q8k_f64(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 double rnbo_dot_q8_0_q8_f64(const uint8_t *row, const rnbo_q8_block *act, size_t n_blocks);
+
+/* ---- importance quants (rnb_oracle_iq.c) ------------------------------------------ */
+void rnbo_dequantize_iq2_xxs(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_iq2_s(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_iq3_xxs(const uint8_t *blocks, size_t n_blocks, float *out);
+void rnbo_dequantize_iq4_xs(const uint8_t *blocks, size_t n_blocks, float *out);
+float rnbo_dot_iq2_xxs_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_iq2_s_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_iq3_xxs_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_iq4_xs_q8k(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+float rnbo_dot_iq_q8k(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+double rnbo_dot_iq_q8k_f64(uint32_t quant, const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
+size_t rnbo_iq_grid(int which, uint64_t *out);
+void rnbo_make_iq_row(uint32_t quant, size_t n_blocks, uint64_t seed, float sigma, uint8_t *out);
 
 /* ---- GEMV / GEMM drivers: out[s*rows + row], x is [seq_len][cols] --------------- */
 /* quant: 2 = Q4_0, 3 = Q4_1, 6 = Q5_0, 7 = Q5_1, 8 = Q8_0 (all against 32-wide Q8 activations), 10 = Q2_K, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K (ggml type ids).  */

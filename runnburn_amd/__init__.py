@@ -8,6 +8,7 @@ functions keep the reference's names, argument meaning and error behaviour:
   q4_0 / q4_1 / q5_0 / q5_1 _gemv (+ _batch)  quant_api.rs:374-496
   q8_1_gemv (+ _batch)                         quant_api.rs:507-541
   q2k_gemv / q3k_gemv (+ _batch)              quant_api.rs:73-181
+  iq2_xxs / iq2_s / iq3_xxs / iq4_xs _gemv (+ _batch)  quant_api.rs:543-722
   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
@@ -72,6 +73,18 @@ from .binding import (  # noqa: F401
     q5_1_gemv_batch,
     q8_1_gemv,
     q8_1_gemv_batch,
+    iq2_xxs_gemv,
+    iq2_xxs_gemv_batch,
+    iq2_s_gemv,
+    iq2_s_gemv_batch,
+    iq3_xxs_gemv,
+    iq3_xxs_gemv_batch,
+    iq4_xs_gemv,
+    iq4_xs_gemv_batch,
+    GGML_IQ2_XXS,
+    GGML_IQ3_XXS,
+    GGML_IQ2_S,
+    GGML_IQ4_XS,
     q2k_gemv,
     q2k_gemv_batch,
     q3k_gemv,

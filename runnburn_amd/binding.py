@@ -12,6 +12,7 @@ _LIB_PATH = os.path.join(_PKG, "librnb_hip.so")
 
 GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1, GGML_Q8_1 = 2, 3, 6, 7, 9
 GGML_Q8_0, GGML_Q2_K, GGML_Q3_K, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 10, 11, 12, 13, 14
+GGML_IQ2_XXS, GGML_IQ3_XXS, GGML_IQ2_S, GGML_IQ4_XS = 16, 18, 22, 23
 OP_MATMUL, OP_ATTENTION, OP_GDN, OP_MOE, OP_SAMPLER = 0, 1, 2, 3, 4
 STATUS_NAMES = {0: "Ok", 1: "InvalidRequest", 2: "UnsupportedOp", 3: "ExecutionFailed", 4: "NoDevice"}
 
@@ -54,6 +55,14 @@ SYMBOLS = [
     ("rnb_hip_q2k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q3k_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q3k_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq2_xxs_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq2_xxs_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq2_s_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq2_s_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq3_xxs_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq3_xxs_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq4_xs_gemv", _i, _MATMUL_ARGS),
+    ("rnb_hip_iq4_xs_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q5k_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q5k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q6k_gemv", _i, _MATMUL_ARGS),
@@ -330,6 +339,38 @@ def q8_1_gemv(weights, rows, cols, input):  # noqa: A002
 
 def q8_1_gemv_batch(weights, rows, cols, input):  # noqa: A002
     return _gemv_batch("rnb_hip_q8_1_gemv_batch", weights, rows, cols, input)
+
+
+def iq2_xxs_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_iq2_xxs_gemv", weights, rows, cols, input)
+
+
+def iq2_xxs_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_iq2_xxs_gemv_batch", weights, rows, cols, input)
+
+
+def iq2_s_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_iq2_s_gemv", weights, rows, cols, input)
+
+
+def iq2_s_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_iq2_s_gemv_batch", weights, rows, cols, input)
+
+
+def iq3_xxs_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_iq3_xxs_gemv", weights, rows, cols, input)
+
+
+def iq3_xxs_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_iq3_xxs_gemv_batch", weights, rows, cols, input)
+
+
+def iq4_xs_gemv(weights, rows, cols, input):  # noqa: A002
+    return _gemv("rnb_hip_iq4_xs_gemv", weights, rows, cols, input)
+
+
+def iq4_xs_gemv_batch(weights, rows, cols, input):  # noqa: A002
+    return _gemv_batch("rnb_hip_iq4_xs_gemv_batch", weights, rows, cols, input)
 
 
 def q2k_gemv(weights, rows, cols, input):  # noqa: A002

@@ -33,6 +33,10 @@ bool quant_info(uint32_t quant, QuantInfo *qi) {
     case kQ4K: *qi = {"Q4_K", 256, kQ4KBytes}; return true;
     case kQ5K: *qi = {"Q5_K", 256, kQ5KBytes}; return true;
     case kQ6K: *qi = {"Q6_K", 256, kQ6KBytes}; return true;
+    case kIQ2XXS: *qi = {"IQ2_XXS", 256, kIQ2XXSBytes}; return true;
+    case kIQ2S: *qi = {"IQ2_S", 256, kIQ2SBytes}; return true;
+    case kIQ3XXS: *qi = {"IQ3_XXS", 256, kIQ3XXSBytes}; return true;
+    case kIQ4XS: *qi = {"IQ4_XS", 256, kIQ4XSBytes}; return true;
     default: return false;
     }
 }
@@ -215,7 +219,10 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         return slice_floats(gemm_blocks_slice_floats(quant, r, k_steps, q), ws);
     };
     float *ws = nullptr;
-    if (quant == kQ4K) {
+    if (is_iq_quant(quant)) {
+        // importance quants: one GEMV pass per token (grid row per token) at every batch size
+        launch_gemv_iq(w_dev, quant, act, out_dev, r, nb, q, s.stream);
+    } else if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
         // gemm_q4k.hip's 256-row x 64-token workgroups (K cut into slices up to 128 tiles) win from 32 tiles on when the
         // token tile is more than half full; below that the 128 x 32 kernel of gemm_blocks.hip, sliced as well, does
@@ -677,7 +684,7 @@ int rnb_hip_backend_kind(void) { return 6; }
 int rnb_hip_backend_supports(int op) { return (op == RNB_OP_MATMUL || op == RNB_OP_MOE) ? 1 : 0; }
 
 int rnb_hip_backend_supports_quant(int op, uint32_t quant) {
-    if (op == RNB_OP_MATMUL) return (is_block32(quant) || (quant >= kQ2K && quant <= kQ6K)) ? 1 : 0;
+    if (op == RNB_OP_MATMUL) return (is_block32(quant) || (quant >= kQ2K && quant <= kQ6K) || is_iq_quant(quant)) ? 1 : 0;
     if (op == RNB_OP_MOE) return (quant == kQ4K || quant == kQ5K || quant == kQ6K) ? 1 : 0;
     return 0;
 }
@@ -903,6 +910,21 @@ int rnb_hip_q3k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t c
                            float *out, size_t out_len) {
     return matmul_host(kQ3K, w, w_len, rows, cols, x, x_len, out, out_len, true);
 }
+#define RNB_IQ_ENTRY(name, quant)                                                                                   \
+    int rnb_hip_##name##_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,  \
+                              float *out, size_t out_len) {                                                          \
+        return matmul_host(quant, w, w_len, rows, cols, x, x_len, out, out_len, false);                              \
+    }                                                                                                                \
+    int rnb_hip_##name##_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,          \
+                                    size_t x_len, float *out, size_t out_len) {                                      \
+        return matmul_host(quant, w, w_len, rows, cols, x, x_len, out, out_len, true);                               \
+    }
+RNB_IQ_ENTRY(iq2_xxs, kIQ2XXS)
+RNB_IQ_ENTRY(iq2_s, kIQ2S)
+RNB_IQ_ENTRY(iq3_xxs, kIQ3XXS)
+RNB_IQ_ENTRY(iq4_xs, kIQ4XS)
+#undef RNB_IQ_ENTRY
+
 int rnb_hip_q5k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                      float *out, size_t out_len) {
     return matmul_host(kQ5K, w, w_len, rows, cols, x, x_len, out, out_len, false);

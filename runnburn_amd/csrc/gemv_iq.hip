@@ -1,0 +1,255 @@
+// GEMV of the importance-quant formats against Q8_K activations: IQ2_XXS (66-byte blocks), IQ2_S (82), IQ3_XXS (98) and
+// IQ4_XS (136), 256 elements a block, every block 2-byte aligned.  The arithmetic is the reference's Q8_K form
+// (crates/rnb-cpu/src/gemm/neon_quant.rs:273-411; element layouts crates/rnb-cpu/src/quantize/iq.rs:23-116): exact
+// int8 dot products per 32-element group, the group scale, then d * d_x per block in f32.
+//   IQ2_XXS  group = 4 grid indices + u32 {4 x 7 sign bits | scale << 28}; value = +-grid byte; d d_x / 4 * sum (0.5 + s) dot
+//   IQ2_S    group = 4 low index bytes (+ 2 high bits each in qh), 4 sign bytes, scale nibbles per 16;  d d_x / 8 * sum (1 + 2 s) dot
+//   IQ3_XXS  group = 8 grid indices (4 bytes each) + u32 as IQ2_XXS;                                    d d_x / 2 * sum (0.5 + s) dot
+//   IQ4_XS   group = 16 bytes of nibbles through the 16-entry table, 6-bit scale - 32;                  d d_x * sum s dot
+// Lane mapping as for the K-quants: four lanes per block, lane g owning groups 2g and 2g + 1 (64 consecutive elements),
+// sixteen blocks per wave and pass; one wave per row, the lanes' partial sums added on the DPP path.
+// The grids are ggml's codebooks, kept packed (a 16-bit word per entry: every byte of an IQ2 entry is one of 8, 25, 43,
+// every byte of an IQ3_XXS entry is 4 + 8 c, 62 for c = 7) and expanded at compile time into device tables; a sign
+// index of seven bits stands for those bits and their parity.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace rnb {
+
+namespace {
+
+#include "iq_grids_packed.inc"
+
+struct Grid64x256 { uint64_t v[256]; };
+struct Grid64x1024 { uint64_t v[1024]; };
+struct Grid32x256 { uint32_t v[256]; };
+
+constexpr uint64_t expand2(uint16_t w) {
+    uint64_t v = 0;
+    for (int j = 0; j < 8; j++) {
+        const uint32_t c = (w >> (2 * j)) & 3;
+        v |= static_cast<uint64_t>(c == 0 ? 8 : (c == 1 ? 25 : 43)) << (8 * j);
+    }
+    return v;
+}
+constexpr uint32_t expand3(uint16_t w) {
+    uint32_t v = 0;
+    for (int j = 0; j < 4; j++) {
+        const uint32_t c = (w >> (3 * j)) & 7;
+        v |= (c == 7 ? 62u : 4u + 8u * c) << (8 * j);
+    }
+    return v;
+}
+constexpr Grid64x256 make_iq2xxs() {
+    Grid64x256 t{};
+    for (int i = 0; i < 256; i++) t.v[i] = expand2(kIq2xxsPacked[i]);
+    return t;
+}
+constexpr Grid64x1024 make_iq2s() {
+    Grid64x1024 t{};
+    for (int i = 0; i < 1024; i++) t.v[i] = expand2(kIq2sPacked[i]);
+    return t;
+}
+constexpr Grid32x256 make_iq3xxs() {
+    Grid32x256 t{};
+    for (int i = 0; i < 256; i++) t.v[i] = expand3(kIq3xxsPacked[i]);
+    return t;
+}
+__device__ const Grid64x256 g_iq2xxs = make_iq2xxs();
+__device__ const Grid64x1024 g_iq2s = make_iq2s();
+__device__ const Grid32x256 g_iq3xxs = make_iq3xxs();
+
+// four bytes of a grid entry with the signs of four bits applied: byte j negated when bit j of `bits` is set (the bytes
+// are positive and below 128, so v ^ 0xff plus one never carries into the next byte)
+__device__ __forceinline__ uint32_t apply_signs4(uint32_t v, uint32_t bits) {
+    const uint32_t m01 = ((bits & 15u) * 0x00204081u) & 0x01010101u;  // bit j -> byte j
+    const uint32_t mask = (m01 << 8) - m01;
+    return (v ^ mask) + m01;
+}
+// seven sign bits and their parity
+__device__ __forceinline__ uint32_t sign_byte(uint32_t seven) {
+    seven &= 127u;
+    return seven | ((__builtin_popcount(seven) & 1u) << 7);
+}
+
+// the lane's 64 activations: groups 2g and 2g + 1
+struct IqAct {
+    uint4 a[4];
+    float dx;
+};
+__device__ __forceinline__ IqAct iq_load_act(const int8_t *aq_blk, float dx, int g) {
+    IqAct r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.a[i] = *reinterpret_cast<const uint4 *>(aq_blk + 64 * g + 16 * i);
+    r.dx = dx;
+    return r;
+}
+__device__ __forceinline__ int dot8(uint32_t lo, uint32_t hi, const uint4 &a, int half, int acc) {
+    return half == 0 ? dot4(hi, a.y, dot4(lo, a.x, acc)) : dot4(hi, a.w, dot4(lo, a.z, acc));
+}
+
+template <uint32_t kQuant>
+struct Iq;
+
+template <>
+struct Iq<kIQ2XXS> {
+    static constexpr size_t kBytes = kIQ2XXSBytes;
+    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g) {
+        const uint4 raw = ld_u4_a2(blk + 2 + 16 * g);  // two groups: {indices, scales and signs} each
+        const uint32_t idx[2] = {raw.x, raw.z}, ss[2] = {raw.y, raw.w};
+        float fsum = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int isum = 0;
+#pragma unroll
+            for (int l = 0; l < 4; l++) {
+                const uint64_t grid = g_iq2xxs.v[(idx[h] >> (8 * l)) & 0xffu];
+                const uint32_t s = sign_byte(ss[h] >> (7 * l));
+                const uint32_t lo = apply_signs4(static_cast<uint32_t>(grid), s);
+                const uint32_t hi = apply_signs4(static_cast<uint32_t>(grid >> 32), s >> 4);
+                isum = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, isum);
+            }
+            fsum += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum);
+        }
+        return ld_f16(blk) * act.dx * 0.25f * fsum;
+    }
+};
+
+template <>
+struct Iq<kIQ2S> {
+    static constexpr size_t kBytes = kIQ2SBytes;
+    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g) {
+        const uint2 lowb = ld_u2_a2(blk + 2 + 8 * g), signb = ld_u2_a2(blk + 34 + 8 * g);
+        const uint32_t qh2 = *reinterpret_cast<const unsigned short *>(blk + 66 + 2 * g);
+        const uint32_t sc2 = *reinterpret_cast<const unsigned short *>(blk + 74 + 2 * g);
+        const uint32_t low[2] = {lowb.x, lowb.y}, sg[2] = {signb.x, signb.y};
+        int isum = 0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t qh = (qh2 >> (8 * h)) & 0xffu, sc = (sc2 >> (8 * h)) & 0xffu;
+            int half_sum[2] = {0, 0};
+#pragma unroll
+            for (int l = 0; l < 4; l++) {
+                const uint32_t index = ((low[h] >> (8 * l)) & 0xffu) | ((qh << (8 - 2 * l)) & 0x300u);
+                const uint64_t grid = g_iq2s.v[index];
+                const uint32_t s = (sg[h] >> (8 * l)) & 0xffu;
+                const uint32_t lo = apply_signs4(static_cast<uint32_t>(grid), s);
+                const uint32_t hi = apply_signs4(static_cast<uint32_t>(grid >> 32), s >> 4);
+                half_sum[l >> 1] = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, half_sum[l >> 1]);
+            }
+            isum += half_sum[0] * static_cast<int>(1 + 2 * (sc & 15u)) + half_sum[1] * static_cast<int>(1 + 2 * (sc >> 4));
+        }
+        return ld_f16(blk) * act.dx * 0.125f * static_cast<float>(isum);
+    }
+};
+
+template <>
+struct Iq<kIQ3XXS> {
+    static constexpr size_t kBytes = kIQ3XXSBytes;
+    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g) {
+        const uint4 idx = ld_u4_a2(blk + 2 + 16 * g);  // eight indices per group, two groups
+        const uint2 ssb = ld_u2_a2(blk + 66 + 8 * g);
+        const uint32_t iw[4] = {idx.x, idx.y, idx.z, idx.w}, ss[2] = {ssb.x, ssb.y};
+        float fsum = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int isum = 0;
+#pragma unroll
+            for (int l = 0; l < 4; l++) {
+                const uint32_t pair = iw[2 * h + (l >> 1)] >> (16 * (l & 1));  // indices 2l and 2l + 1 of the group
+                const uint32_t s = sign_byte(ss[h] >> (7 * l));
+                const uint32_t lo = apply_signs4(g_iq3xxs.v[pair & 0xffu], s);
+                const uint32_t hi = apply_signs4(g_iq3xxs.v[(pair >> 8) & 0xffu], s >> 4);
+                isum = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, isum);
+            }
+            fsum += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum);
+        }
+        return ld_f16(blk) * act.dx * 0.5f * fsum;
+    }
+};
+
+// four table values for four indices 0..15, one per byte
+__device__ __forceinline__ uint32_t iq4nl_lookup(uint32_t idx4) {
+    // -127 -104 -83 -65 | -49 -35 -22 -10 | 1 13 25 38 | 53 69 89 113 as bytes, little-endian words
+    constexpr uint32_t t0 = 0xbfad9881u, t1 = 0xf6eaddcfu, t2 = 0x26190d01u, t3 = 0x71594535u;
+    const uint32_t low3 = idx4 & 0x07070707u;
+    const uint32_t below = __builtin_amdgcn_perm(t1, t0, low3), above = __builtin_amdgcn_perm(t3, t2, low3);
+    const uint32_t m01 = (idx4 >> 3) & 0x01010101u, mask = (m01 << 8) - m01;
+    return (below & ~mask) | (above & mask);
+}
+
+template <>
+struct Iq<kIQ4XS> {
+    static constexpr size_t kBytes = kIQ4XSBytes;
+    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g) {
+        const uint2 hdr = ld_u2_a2(blk);  // f16 d | scales_h << 16, then scales_l
+        const uint4 q0 = ld_u4_a2(blk + 8 + 32 * g), q1 = ld_u4_a2(blk + 24 + 32 * g);
+        const uint32_t scales_h = hdr.x >> 16;
+        const uint32_t both = (hdr.y >> (8 * g)) & 0xffu;  // scales_l[g]: groups 2g (low nibble) and 2g + 1
+        const int s0 = static_cast<int>((both & 15u) | (((scales_h >> (4 * g)) & 3u) << 4)) - 32;
+        const int s1 = static_cast<int>((both >> 4) | (((scales_h >> (4 * g + 2)) & 3u) << 4)) - 32;
+        const uint32_t w0[4] = {q0.x, q0.y, q0.z, q0.w}, w1[4] = {q1.x, q1.y, q1.z, q1.w};
+        const uint32_t a0[4] = {act.a[0].x, act.a[0].y, act.a[0].z, act.a[0].w};
+        const uint32_t a1[4] = {act.a[1].x, act.a[1].y, act.a[1].z, act.a[1].w};
+        const uint32_t a2[4] = {act.a[2].x, act.a[2].y, act.a[2].z, act.a[2].w};
+        const uint32_t a3[4] = {act.a[3].x, act.a[3].y, act.a[3].z, act.a[3].w};
+        int d0 = 0, d1 = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            // byte j of the group: element j (low nibble) and element 16 + j (high nibble)
+            d0 = dot4(iq4nl_lookup(w0[i] & 0x0f0f0f0fu), a0[i], d0);
+            d0 = dot4(iq4nl_lookup((w0[i] >> 4) & 0x0f0f0f0fu), a1[i], d0);
+            d1 = dot4(iq4nl_lookup(w1[i] & 0x0f0f0f0fu), a2[i], d1);
+            d1 = dot4(iq4nl_lookup((w1[i] >> 4) & 0x0f0f0f0fu), a3[i], d1);
+        }
+        return f16_bits_to_f32(hdr.x) * act.dx * static_cast<float>(d0 * s0 + d1 * s1);
+    }
+};
+
+constexpr int kIqWaves = 4;
+
+template <uint32_t kQuant>
+__global__ void __launch_bounds__(kWave *kIqWaves)
+    gemv_iq_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                   float *__restrict__ out, uint32_t rows, uint32_t nb) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const int g = lane & 3;
+    const uint32_t tok = blockIdx.y;
+    const size_t row_bytes = static_cast<size_t>(nb) * Iq<kQuant>::kBytes;
+    const uint32_t n_waves = gridDim.x * kIqWaves;
+    for (uint32_t row = blockIdx.x * kIqWaves + wave; row < rows; row += n_waves) {
+        float acc = 0.0f;
+        for (uint32_t b = lane >> 2; b < nb; b += 16) {
+            const size_t ab = static_cast<size_t>(tok) * nb + b;
+            const IqAct act = iq_load_act(aq + ab * 256, ad[ab], g);
+            acc += Iq<kQuant>::partial(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * Iq<kQuant>::kBytes, act, g);
+        }
+        acc = seg_sum<kWave>(acc);
+        if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
+    }
+}
+
+template <uint32_t kQuant>
+void launch_iq(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq, hipStream_t stream) {
+    const uint32_t want = (rows + kIqWaves - 1) / kIqWaves;
+    const dim3 grid(want < 4096 ? want : 4096, seq, 1);
+    hipLaunchKernelGGL((gemv_iq_kernel<kQuant>), grid, dim3(kWave * kIqWaves), 0, stream, w, act.qs, act.d, out, rows, nb);
+}
+
+}  // namespace
+
+bool is_iq_quant(uint32_t quant) { return quant == kIQ2XXS || quant == kIQ2S || quant == kIQ3XXS || quant == kIQ4XS; }
+
+void launch_gemv_iq(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
+                    hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb == 0) return;
+    switch (quant) {
+    case kIQ2XXS: launch_iq<kIQ2XXS>(w, act, out, rows, nb, seq, stream); break;
+    case kIQ2S: launch_iq<kIQ2S>(w, act, out, rows, nb, seq, stream); break;
+    case kIQ3XXS: launch_iq<kIQ3XXS>(w, act, out, rows, nb, seq, stream); break;
+    default: launch_iq<kIQ4XS>(w, act, out, rows, nb, seq, stream); break;
+    }
+}
+
+}  // namespace rnb

@@ -16,7 +16,6 @@
 #include "kernels.h"
 #include "mfma_blocks.h"
 #include <algorithm>
-#include <cstdlib>
 
 namespace rnb {
 
@@ -496,10 +495,9 @@ bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
 void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                              uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0 || n_ff == 0) return;
-    uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
+    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
     if (toks == 0) return;  // moe_mfma_supported said no
-    int waves = kGbWaves;
-    if (const char *e = getenv("RNB_PROBE_GU_WAVES")) waves = atoi(e);
+    const int waves = kGbWaves;  // 2, 3 and 6 waves per workgroup measured within 3 % of 4 on 128 experts x top-8, 64 tokens
     const size_t lds = static_cast<size_t>(waves) * 2 * kQ4FillBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
     const uint32_t rows_per_wg = 32 * waves;
     const dim3 grid((n_ff + rows_per_wg - 1) / rows_per_wg, groups.n_groups, 1);
@@ -508,16 +506,7 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
     if (!allow_lds<J * 16 + W>(moe_gate_up_mfma_kernel<J, W>, kMmLdsLimit)) return;                                   \
     hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, act.qs, act.d, \
                        act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
-#define RNB_LAUNCH_GU(J)                                                                                              \
-    if (waves == 2) {                                                                                                 \
-        RNB_LAUNCH_GUW(J, 2);                                                                                         \
-    } else if (waves == 3) {                                                                                          \
-        RNB_LAUNCH_GUW(J, 3);                                                                                         \
-    } else if (waves == 6) {                                                                                          \
-        RNB_LAUNCH_GUW(J, 6);                                                                                         \
-    } else {                                                                                                          \
-        RNB_LAUNCH_GUW(J, 4);                                                                                         \
-    }
+#define RNB_LAUNCH_GU(J) RNB_LAUNCH_GUW(J, kGbWaves)
     if (toks <= 8) {
         RNB_LAUNCH_GU(1);
     } else if (toks <= 16) {
@@ -540,9 +529,8 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView 
     while (tiles_per_wg < 4 && static_cast<uint64_t>((row_tiles + tiles_per_wg - 1) / tiles_per_wg) * groups.n_groups > 768)
         tiles_per_wg *= 2;
     const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1), block(kGbThreads);
-    uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), down_tile_tokens(nb_mid, down_quant));
+    const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), down_tile_tokens(nb_mid, down_quant));
     if (toks == 0) return;
-    if (const char *e = getenv("RNB_PROBE_CAP_DN")) toks = std::min<uint32_t>(toks, atoi(e));
 #define RNB_LAUNCH_DMJ(Q, J, LDS)                                                                                     \
     if (!allow_lds<static_cast<int>(Q) * 8 + J>(moe_down_mfma_kernel<Q, J>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return; \
     hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \

@@ -39,7 +39,9 @@ def test_trait_facade():
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q2_K) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q3_K)
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q4_0) and b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q5_1)
     assert b.supports_quant(rnb.OP_MATMUL, rnb.GGML_Q8_1)
-    assert not b.supports_quant(rnb.OP_MATMUL, 16) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # IQ2_XXS; Q8_0 down
+    for iq in (rnb.GGML_IQ2_XXS, rnb.GGML_IQ2_S, rnb.GGML_IQ3_XXS, rnb.GGML_IQ4_XS):
+        assert b.supports_quant(rnb.OP_MATMUL, iq) and not b.supports_quant(rnb.OP_MOE, iq)
+    assert not b.supports_quant(rnb.OP_MATMUL, 17) and not b.supports_quant(rnb.OP_MOE, rnb.GGML_Q8_0)  # IQ2_XS; Q8_0 down
     with pytest.raises(rnb.BackendError) as ei:
         b.execute(object())
     assert ei.value.kind == "UnsupportedOp"

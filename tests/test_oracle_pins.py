@@ -925,3 +925,99 @@ def test_rms_norm_reference_vectors_and_closed_forms(oracle):
     assert np.allclose(oracle.rms_norm(xr, wr, 1e-6, unit_offset=True), want / wr * (1.0 + wr.astype(np.float64)), rtol=2e-6, atol=1e-8)
     c = np.full(256, -3.0, np.float32)
     assert np.allclose(oracle.rms_norm(c, np.ones(256, np.float32), 1e-5)[0], -1.0 / math.sqrt(1.0 + 1e-5 / 9.0), rtol=2e-7)
+
+
+# ---- importance quants -------------------------------------------------------------------------------------------------
+
+def _fnv1a_of_f32(values):
+    h = 0xcbf29ce484222325
+    for b in np.asarray(values, np.float32).tobytes():
+        h = ((h ^ b) * 0x100000001b3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+_ONE_F16 = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+_IQ_HASHES = {16: 0x0ead89a48d8fee11, 22: 0x69e6a32989d193d1, 18: 0xbcf1592321ede577, 23: 0x0c822de33756fd50}
+
+
+@pytest.mark.parametrize("quant", [16, 22, 18, 23])
+def test_iq_dequantisers_reproduce_the_references_known_answers(oracle, quant):
+    """crates/rnb-cpu/src/quantize/iq.rs:258-334: the FNV-1a hash over the f32 bits of the decoded block whose byte i is
+    73 i + 19 (mod 256) behind a leading f16 1.0 -- one known answer per format, which also fixes every codebook entry,
+    sign and scale the block touches; and iq.rs:281-299: zero codes decode to +1.0 everywhere (IQ4_XS: scale -32 times
+    the first table value, -127)."""
+    n = oracle.BLOCK_BYTES[quant]
+    blk = np.array([(i * 73 + 19) & 0xFF for i in range(n)], np.uint8)
+    blk[:2] = _ONE_F16
+    assert _fnv1a_of_f32(oracle.dequantize(quant, blk)) == _IQ_HASHES[quant]
+    zero = np.zeros(n, np.uint8)
+    zero[:2] = _ONE_F16
+    want = 4064.0 if quant == 23 else 1.0
+    assert np.array_equal(oracle.dequantize(quant, zero), np.full(256, want, np.float32))
+
+
+def test_iq4_xs_reference_vector(oracle):
+    """crates/rnb-cpu/src/gemm/dequant.rs:542-556: scales_h 0xaaaa, scales_l 0x11 -> every 6-bit scale is 33, i.e. +1;
+    bytes 0xf0 -> low nibble 0 (-127) for the first 16 elements of a sub-block, high nibble 15 (113) for the other 16."""
+    b = np.zeros(136, np.uint8)
+    b[:2] = _ONE_F16
+    b[2:4] = (0xAA, 0xAA)
+    b[4:8] = 0x11
+    b[8:] = 0xF0
+    out = oracle.dequantize(23, b)
+    assert out[0] == -127.0 and out[16] == 113.0 and out[32] == -127.0
+    assert np.array_equal(out.reshape(8, 2, 16), np.broadcast_to(np.array([-127.0, 113.0], np.float32)[None, :, None], (8, 2, 16)))
+
+
+def test_iq_codebooks_have_the_published_shape(oracle):
+    """The packed codebooks expand to ggml's tables: the byte alphabets ({8, 25, 43}; 4 + 8 c with 62 for c = 7), the
+    first and last entries, all entries distinct.  (The hashes above check the entries a block touches by value.)"""
+    g2, g2s, g3 = oracle.iq_grid(0), oracle.iq_grid(1), oracle.iq_grid(2)
+    assert g2.size == 256 and g2s.size == 1024 and g3.size == 256
+    for g, nbytes in ((g2, 8), (g2s, 8)):
+        by = g.view(np.uint8).reshape(-1, 8)[:, :nbytes]
+        assert set(np.unique(by)) == {8, 25, 43}
+        assert np.unique(g).size == g.size
+    by3 = g3.astype(np.uint32).view(np.uint8).reshape(-1, 4)
+    assert set(np.unique(by3)) == {4, 12, 20, 28, 36, 44, 52, 62}
+    assert np.unique(g3).size == 256
+    assert g2[0] == 0x0808080808080808 and g2[1] == 0x080808080808082B and g2s[0] == 0x0808080808080808 and g3[0] == 0x04040404
+
+
+@pytest.mark.parametrize("quant", [16, 22, 18, 23])
+def test_iq_dots_equal_the_dequantised_statement(oracle, quant):
+    """dot(W, Q8_K(x)) restated independently: f64 sum of dequantise(W) * (d_x * q_x).  The integer forms of
+    crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 must give the same number to f32 rounding, the f64 gold form to 1e-12;
+    a wrong sign bit, scale nibble or element order shows as an O(1) relative error."""
+    nb = 6
+    w = oracle.make_weights(quant, 5, nb * 256, 4242 + quant)
+    x = oracle.fill_normal(nb * 256, 99 + quant, 1.0)
+    act = oracle.quantize_q8k(x)
+    xq = (act["d"][:, None].astype(np.float64) * act["qs"].astype(np.float64)).ravel()
+    rb = nb * oracle.BLOCK_BYTES[quant]
+    for r in range(5):
+        row = w[r * rb:(r + 1) * rb]
+        want = float(np.dot(oracle.dequantize(quant, row).astype(np.float64), xq))
+        scale = float(np.sqrt(np.sum(oracle.dequantize(quant, row).astype(np.float64) ** 2) * np.sum(xq ** 2)))
+        assert abs(oracle.dot(quant, row, act, gold=True) - want) <= 1e-9 * scale
+        assert abs(oracle.dot(quant, row, act) - want) <= 2e-6 * scale
+
+
+def test_iq_dot_hand_built_blocks(oracle):
+    """One block, activations 1 (Q8_K codes 127 at d = 1/127): IQ4_XS with every nibble 8 (value +1) and scale code 33
+    (+1) gives 256 * 127 * (1/127) = 256 = the reference's d * d_x * block_sum; raising the scale code of sub-block 3
+    alone to 47 (+15) adds 14 * 32.  IQ2_XXS zero codes (every element decodes to 1.0): 256 as well."""
+    x = np.ones(256, np.float32)
+    act = oracle.quantize_q8k(x)
+    b = np.zeros(136, np.uint8)
+    b[:2] = _ONE_F16
+    b[2:4] = (0xAA, 0xAA)
+    b[4:8] = 0x11
+    b[8:] = 0x88
+    assert oracle.dot(23, b, act) == pytest.approx(256.0, rel=1e-6)
+    b2 = b.copy()
+    b2[5] = 0xF1  # scales_l[1]: sub-block 2 keeps low nibble 1, sub-block 3 gets 15 -> code 2 << 4 | 15 = 47 -> +15
+    assert oracle.dot(23, b2, act) == pytest.approx(256.0 + 14 * 32, rel=1e-6)
+    z = np.zeros(66, np.uint8)
+    z[:2] = _ONE_F16
+    assert oracle.dot(16, z, act) == pytest.approx(256.0, rel=1e-6)
