@@ -965,8 +965,10 @@ bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
 }
 
 bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
-    // From about 190 MB on, the separate quantiser launch (2.5 us) costs less than what the chunked kernel gains over
-    // the one-launch kernel, whose workgroups loop (264 MB of Q4_K: 41.5 + 2.5 against 48.0 us).
+    // From about 300 MB on, the separate quantiser launch costs less than what the chunked kernel gains over the
+    // one-launch kernel, whose workgroups loop (steps measured back to back: 264 MB of Q4_K 49.5 us in one launch against
+    // 51.1 in two, 431 MB of Q6_K 83.1 against 79.0).  The chunked kernel with the quantiser in front (one chunk per wave,
+    // one barrier per workgroup of 4, 8 or 16 waves) was tried: 431 MB of Q6_K 81 / 86 / 94 us, 264 MB of Q4_K 71 / 56 us.
     size_t bytes = 0;
     switch (quant) {
     case kQ2K: bytes = kQ2KBytes; break;
@@ -975,7 +977,7 @@ bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
     case kQ5K: bytes = kQ5KBytes; break;
     default: bytes = kQ6KBytes; break;
     }
-    return nb <= 8 || static_cast<uint64_t>(rows) * nb * bytes < (uint64_t(190) << 20);
+    return nb <= 8 || static_cast<uint64_t>(rows) * nb * bytes < (uint64_t(300) << 20);
 }
 
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
