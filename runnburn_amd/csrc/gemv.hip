@@ -215,15 +215,9 @@ void launch_kquant_f32(const uint8_t *w, const float *x, float *out, uint32_t ro
 }
 
 template <uint32_t kQuant>
-void launch_kquant_splitk_f32(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                              hipStream_t stream);
-
-template <uint32_t kQuant>
 void launch_kquant_f32_any(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                            hipStream_t stream) {
-    if (nb > 16)
-        launch_kquant_splitk_f32<kQuant>(w, x, out, rows, nb, seq, stream);
-    else if (nb <= 4)
+    if (nb <= 4)
         launch_kquant_f32<kQuant, 4>(w, x, out, rows, nb, seq, stream);
     else if (nb <= 8)
         launch_kquant_f32<kQuant, 2>(w, x, out, rows, nb, seq, stream);
@@ -485,9 +479,10 @@ __global__ void __launch_bounds__(256) act_mul_kernel(const float *__restrict__ 
 // Long rows (more than 16 super-blocks): the K dimension is split across the waves of a workgroup, wave j
 // owning super-blocks [16j, 16j+16) of every row, so each lane's activation slice is loaded once and stays
 // in registers; the per-wave partial sums of kSplitRows consecutive rows meet in LDS and are added in
-// wave order.
+// wave order.  A step's blocks are requested at its start and reduced at once: requesting the next step's blocks
+// ahead (before or after the barrier) measured 9 - 13 % slower, as did more rows per step.
 // ---------------------------------------------------------------------------------------------
-constexpr int kSplitRows = 4;
+constexpr int kSplitRows = 1;  // rows per workgroup and step: 1 / 2 / 4 / 8 measured 11.6 / 12.8 / 13.5 / 33 us on 4096 x 14336 Q6_K
 constexpr uint32_t kSplitMaxWaves = 16;  // rows of up to 256 super-blocks
 
 template <uint32_t kQuant>
@@ -544,106 +539,6 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
     const dim3 grid(row_chunks < want ? row_chunks : want, seq, 1);
     hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
                        act.bsums, out, rows, nb, row_chunks);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Long rows against an f32 token in one launch.  A workgroup is kSplitMaxWaves waves: wave (q, j) owns super-blocks
-// [16j, 16j+16) of the rows of row group q (16 / slices groups per workgroup).  The token is quantised once per
-// workgroup (wave v takes blocks v, v + 16, ...: the stand-alone quantiser's arithmetic, so the same bits) into LDS,
-// the first rows' weights already in flight; after that every wave keeps its activation slice in registers and the
-// row groups run the split-K loop side by side, their partial sums meeting in LDS and added in slice order.
-// Dynamic LDS: qs[nb][256] | bsums[nb][16] | d[nb].
-// ---------------------------------------------------------------------------------------------
-constexpr uint32_t kSplitFusedMaxNb = 128;  // 32768 columns: 36.5 KB of LDS
-constexpr int kSplitFusedRows = 2;          // rows per wave and round (this round's and the next one's blocks fit 128 registers)
-template <uint32_t kQuant>
-__global__ void __launch_bounds__(kWave *kSplitMaxWaves)
-    gemv_kquant_splitk_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
-                                  uint32_t rows, uint32_t nb, uint32_t row_chunks, uint32_t n_slices, uint32_t n_groups) {
-    using Q = KQuant<kQuant>;
-    using Regs = typename Q::Regs;
-    constexpr size_t kBlockBytes = Q::kBytes;
-    extern __shared__ __attribute__((aligned(16))) uint8_t s_token[];
-    __shared__ float s_part[2][kSplitMaxWaves][kSplitFusedRows];
-    int8_t *s_qs = reinterpret_cast<int8_t *>(s_token);
-    int16_t *s_bsums = reinterpret_cast<int16_t *>(s_token + static_cast<size_t>(nb) * 256);  // 16-byte aligned
-    float *s_d = reinterpret_cast<float *>(s_token + static_cast<size_t>(nb) * 288);
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
-    const uint32_t q = wave / n_slices, j = wave - q * n_slices;  // row group, K slice
-    const int g = lane & 3;
-    const uint32_t b = j * 16 + (lane >> 2);
-    const bool has_block = b < nb;
-    const uint32_t tok = blockIdx.y;
-    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    const float *x_tok = x + static_cast<size_t>(tok) * nb * 256;
-    const uint32_t chunk_step = gridDim.x * n_groups;
-    uint32_t chunk = blockIdx.x * n_groups + q;
-    auto fetch = [&](uint32_t c, Regs (&r)[kSplitFusedRows]) {
-        const uint32_t row0 = c * kSplitFusedRows;
-#pragma unroll
-        for (int i = 0; i < kSplitFusedRows; i++) {
-            r[i] = Regs{};  // idle lanes and rows past the end keep zeros
-            if (has_block && c < row_chunks && row0 + i < rows)
-                r[i] = Q::load_block(w + static_cast<size_t>(row0 + i) * row_bytes + static_cast<size_t>(b) * kBlockBytes, g);
-        }
-    };
-    // the token first (loads return in order and the quantiser must not wait for weights), then the first rows
-    constexpr int kTokBatch = 8;  // blocks of the token a wave holds at a time (128 waves x blocks cover nb <= 128)
-    float4 xv[kTokBatch];
-#pragma unroll
-    for (int i = 0; i < kTokBatch; i++) {
-        const uint32_t blk = wave + i * n_waves;
-        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x_tok + static_cast<size_t>(blk) * 256)[lane];
-    }
-    Regs r[kSplitFusedRows];
-    fetch(chunk, r);
-#pragma unroll
-    for (int i = 0; i < kTokBatch; i++) {
-        const uint32_t blk = wave + i * n_waves;
-        if (blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
-    }
-    __syncthreads();
-    const uint32_t ab = has_block ? b : 0;
-    const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
-
-    // every wave runs the same number of rounds (the barrier is the workgroup's); waves without a chunk add zeros
-    const uint32_t rounds = (row_chunks + chunk_step - 1) / chunk_step;
-    uint32_t parity = 0;
-    for (uint32_t it = 0; it < rounds; it++, chunk += chunk_step, parity ^= 1) {
-        Regs nxt[kSplitFusedRows];
-        fetch(chunk + chunk_step, nxt);
-#pragma unroll
-        for (int i = 0; i < kSplitFusedRows; i++) {
-            float acc = kquant_partial<kQuant>(r[i], a, g);
-            acc = seg_sum<kWave>(has_block ? acc : 0.0f);
-            if (lane == kWave - 1) s_part[parity][wave][i] = acc;
-        }
-        __syncthreads();  // the other parity's buffer is reused only after the next barrier
-        if (j == 0 && lane < kSplitFusedRows && q < n_groups && chunk < row_chunks && chunk * kSplitFusedRows + lane < rows) {
-            float sum = 0.0f;
-            for (uint32_t k = 0; k < n_slices; k++) sum += s_part[parity][q * n_slices + k][lane];
-            out[static_cast<size_t>(tok) * rows + chunk * kSplitFusedRows + lane] = sum;
-        }
-#pragma unroll
-        for (int i = 0; i < kSplitFusedRows; i++) r[i] = nxt[i];
-    }
-}
-
-template <uint32_t kQuant>
-void launch_kquant_splitk_f32(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
-                              hipStream_t stream) {
-    const uint32_t n_slices = (nb + 15) / 16;
-    const uint32_t n_groups = kSplitMaxWaves / n_slices;
-    const uint32_t row_chunks = (rows + kSplitFusedRows - 1) / kSplitFusedRows;
-    // one workgroup per compute unit quantises the token once for 16 waves; more workgroups than that only when the
-    // matrix has rows for them
-    const uint32_t want = (row_chunks + n_groups - 1) / n_groups;
-    const dim3 grid(want < 256 ? want : 256, seq, 1);
-    const size_t lds = static_cast<size_t>(nb) * (256 + 4 + 32);
-    hipLaunchKernelGGL((gemv_kquant_splitk_f32_kernel<kQuant>), grid, dim3(kWave * n_slices * n_groups), lds, stream, w, x, out,
-                       rows, nb, row_chunks, n_slices, n_groups);
 }
 
 template <uint32_t kQuant, int kRowsPerWave>
@@ -961,7 +856,7 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 
 bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
     const bool kq = quant == kQ2K || quant == kQ3K || quant == kQ4K || quant == kQ5K || quant == kQ6K;
-    return kq && nb >= 1 && nb <= kSplitFusedMaxNb && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    return kq && nb >= 1 && nb <= 16 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
 bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
