@@ -165,6 +165,14 @@ int rnb_hip_q3k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, c
                      size_t x_len, float *out, size_t out_len);
 int rnb_hip_q3k_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                            const float *x, size_t x_len, float *out, size_t out_len);
+/* q4k_gemv_with_device_input / q6k_gemv_with_device_input, quant_api.rs:242-330: one token that already lives on the
+ * device (x_dev: cols floats, 16-byte aligned, e.g. the output of rnb_hip_rms_norm_dev) against host-resident weights,
+ * result to the host.  Checks and texts in the reference's order: cols, weight bytes, "<fmt> output too small: got {},
+ * expected >= {rows}". */
+int rnb_hip_q4k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                       const float *x_dev, float *out, size_t out_len);
+int rnb_hip_q6k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                       const float *x_dev, float *out, size_t out_len);
 /* iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv and their batch forms, quant_api.rs:543-722 (same checks and
  * texts): importance-quant rows (66 / 82 / 98 / 136-byte blocks of 256 elements) x Q8_K(x), the block dots of
  * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Every

@@ -73,6 +73,8 @@ from .binding import (  # noqa: F401
     q5_1_gemv_batch,
     q8_1_gemv,
     q8_1_gemv_batch,
+    q4k_gemv_with_device_input,
+    q6k_gemv_with_device_input,
     iq2_xxs_gemv,
     iq2_xxs_gemv_batch,
     iq2_s_gemv,

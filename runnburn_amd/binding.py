@@ -55,6 +55,8 @@ SYMBOLS = [
     ("rnb_hip_q2k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q3k_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q3k_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_q4k_gemv_with_device_input", _i, [_vp, _sz, _sz, _sz, _vp, _vp, _sz]),
+    ("rnb_hip_q6k_gemv_with_device_input", _i, [_vp, _sz, _sz, _sz, _vp, _vp, _sz]),
     ("rnb_hip_iq2_xxs_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_iq2_xxs_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_iq2_s_gemv", _i, _MATMUL_ARGS),
@@ -339,6 +341,24 @@ def q8_1_gemv(weights, rows, cols, input):  # noqa: A002
 
 def q8_1_gemv_batch(weights, rows, cols, input):  # noqa: A002
     return _gemv_batch("rnb_hip_q8_1_gemv_batch", weights, rows, cols, input)
+
+
+def _gemv_with_device_input(fn_name: str, weights, rows: int, cols: int, input_dev, output: np.ndarray) -> None:
+    w = _bytes_view(weights)
+    if output.dtype != np.float32 or not output.flags.c_contiguous:
+        raise TypeError("output must be a C-contiguous float32 array")
+    _check(getattr(lib(), fn_name)(_ptr(w), w.size, rows, cols, input_dev.ptr, _ptr(output), output.size))
+
+
+def q4k_gemv_with_device_input(weights, rows, cols, input_dev, output):
+    """quant_api.rs:288-330: host-resident Q4_K weights, one token on the device (a DeviceBuffer of cols floats), result
+    into the caller's host array."""
+    _gemv_with_device_input("rnb_hip_q4k_gemv_with_device_input", weights, rows, cols, input_dev, output)
+
+
+def q6k_gemv_with_device_input(weights, rows, cols, input_dev, output):
+    """quant_api.rs:242-284, the Q6_K form."""
+    _gemv_with_device_input("rnb_hip_q6k_gemv_with_device_input", weights, rows, cols, input_dev, output)
 
 
 def iq2_xxs_gemv(weights, rows, cols, input):  # noqa: A002

@@ -344,6 +344,46 @@ int matmul_host(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, siz
     return RNB_HIP_OK;
 }
 
+// One token that already lives on the device (a norm's output, say) against host-resident weights, result to the host:
+// q4k_gemv_with_device_input / q6k_gemv_with_device_input, crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:242-330
+// (checks and texts: cols, weight bytes, output size, in that order).
+int matmul_device_input(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x_dev,
+                        float *out, size_t out_len) {
+    QuantInfo qi;
+    if (!quant_info(quant, &qi)) return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    const std::string label = qi.label;
+    if (cols % qi.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    label + " cols must be divisible by " + std::to_string(qi.elems) + ", got " + std::to_string(cols));
+    const size_t row_bytes = cols / qi.elems * qi.bytes;
+    if (w_len != rows * row_bytes)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " weight byte mismatch: got " + std::to_string(w_len) + ", expected " +
+                                                 std::to_string(rows * row_bytes));
+    if (out_len < rows)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    label + " output too small: got " + std::to_string(out_len) + ", expected >= " + std::to_string(rows));
+    if ((w_len && !w) || (out_len && !out)) return fail(RNB_HIP_INVALID_REQUEST, label + " null pointer argument");
+    if (rows == 0) return RNB_HIP_OK;
+    if (cols == 0 || !x_dev || (reinterpret_cast<uintptr_t>(x_dev) & 15u))
+        return fail(RNB_HIP_INVALID_REQUEST, label + " device input must be a 16-byte aligned device pointer to cols floats");
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu)
+        return fail(RNB_HIP_INVALID_REQUEST, label + " shape out of range: rows=" + std::to_string(rows) + " cols=" + std::to_string(cols));
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *w_dev = nullptr;
+    if (int rs = s.resident_ptr(w, w_len, &w_dev); rs != RNB_HIP_OK) return rs;
+    const size_t out_bytes = rows * sizeof(float);
+    RESERVE_TRY(s.bounce_out, out_bytes);
+    HIP_TRY(s.out_f32.reserve(out_bytes));
+    if (int st = run_matmul_dev(s, quant, w_dev, rows, cols, x_dev, 1, s.out_f32.as<float>()); st != RNB_HIP_OK) return st;
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += out_bytes;
+    std::memcpy(out, s.bounce_out.ptr, out_bytes);
+    return RNB_HIP_OK;
+}
+
 // ---- dense gated FFN --------------------------------------------------------------------------
 // out[s] = W_down . Q(act(W_gate . Q8_K(x_s)) * (W_up . Q8_K(x_s))), act = SiLU or GELU: the composition the reference
 // runs per token on the CPU (gate/up GEMV, fused_silu_mul / fused_gelu_mul, down GEMV).  Gate and up are Q4_K; down is Q4_K, Q5_K, Q6_K, Q8_0 or Q5_1.
@@ -924,6 +964,15 @@ RNB_IQ_ENTRY(iq2_s, kIQ2S)
 RNB_IQ_ENTRY(iq3_xxs, kIQ3XXS)
 RNB_IQ_ENTRY(iq4_xs, kIQ4XS)
 #undef RNB_IQ_ENTRY
+
+int rnb_hip_q4k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x_dev,
+                                       float *out, size_t out_len) {
+    return matmul_device_input(kQ4K, w, w_len, rows, cols, x_dev, out, out_len);
+}
+int rnb_hip_q6k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x_dev,
+                                       float *out, size_t out_len) {
+    return matmul_device_input(kQ6K, w, w_len, rows, cols, x_dev, out, out_len);
+}
 
 int rnb_hip_q5k_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                      float *out, size_t out_len) {

@@ -133,3 +133,36 @@ def test_router_topk_softmax(rnb, oracle, tokens, n_expert, k):
         buf.free()
     with pytest.raises(rnb.BackendError):
         rnb.moe_route_topk_dev(ld, 1, 600, 8, idx_d, w_d)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q6_K, 129, 2048), (Q6_K, 40, 14336)])
+def test_gemv_with_device_input(rnb, oracle, quant, rows, cols):
+    """crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:242-330: host-resident weights, a token that is already on
+    the device (here: the output of the device RMS norm), result to the host; the same bits as the all-host call on the
+    norm's output, and the reference's texts for its three checks."""
+    fn = rnb.q4k_gemv_with_device_input if quant == Q4_K else rnb.q6k_gemv_with_device_input
+    host = rnb.q4k_gemv if quant == Q4_K else rnb.q6k_gemv
+    label = "Q4_K" if quant == Q4_K else "Q6_K"
+    w = oracle.make_weights(quant, rows, cols, 5150 + rows)
+    x = oracle.fill_normal(cols, 5151, 2.0)
+    nw = np.ones(cols, np.float32)
+    xd, wd = rnb.DeviceBuffer.from_host(x), rnb.DeviceBuffer.from_host(nw)
+    normed = rnb.DeviceBuffer(cols * 4)
+    rnb.rms_norm_dev(xd, wd, 1e-5, 1, cols, normed)
+    out = np.zeros(rows + 3, np.float32)
+    fn(w, rows, cols, normed, out)
+    n_host = normed.to_host(np.float32)
+    assert np.array_equal(out[:rows], host(w, rows, cols, n_host)) and np.all(out[rows:] == 0)
+    want = oracle.gemv(quant, w, rows, cols, n_host)[0]
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert float(np.abs(out[:rows].astype(np.float64) - want).max()) <= 1e-3 * rms
+    with pytest.raises(rnb.BackendError, match=f"{label} cols must be divisible by 256, got {cols + 1}"):
+        fn(w, rows, cols + 1, normed, out)
+    with pytest.raises(rnb.BackendError, match=f"{label} weight byte mismatch: got {w.size}, expected"):
+        fn(w, rows + 1, cols, normed, out)
+    with pytest.raises(rnb.BackendError, match=f"{label} output too small: got {rows - 1}, expected >= {rows}"):
+        fn(w, rows, cols, normed, out[:rows - 1])
+    rnb.release(w)
+    for b in (xd, wd, normed):
+        b.free()
