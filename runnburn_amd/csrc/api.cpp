@@ -669,29 +669,21 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
         return RNB_HIP_OK;
     }
     RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
-    RESERVE_TRY(s.moe_mid_qs, n_slots * n_ff);
-    RESERVE_TRY(s.moe_mid_d, n_slots * sh.nb_mid * sizeof(float));
-    RESERVE_TRY(s.moe_mid_bsums, n_slots * sh.nb_mid * 16 * sizeof(int16_t));
     RESERVE_TRY(s.moe_slot_out, n_slots * n_embd * sizeof(float));
     if (mfma && act.digits != nullptr) {
-        // prefill: grouped GEMMs, 32-token tiles per expert
-        uint8_t *mid_digits = nullptr;
-        if (down_quant != kQ6K) {  // Q4_K / Q5_K mins need the 32-element sums' digits
-            RESERVE_TRY(s.moe_mid_digits, n_slots * sh.nb_mid * 16);
-            mid_digits = s.moe_mid_digits.as<uint8_t>();
-        }
+        // prefill: grouped GEMMs on the matrix cores; the down kernel quantises the intermediate as it stages it
         launch_moe_gate_up_mfma(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                                 static_cast<uint32_t>(sh.nb_in), s.stream);
-        launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
-                            s.moe_mid_bsums.as<int16_t>(), mid_digits, s.stream);
-        const ActView mid_act{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>(), mid_digits};
-        launch_moe_down_mfma(down_dev, down_quant, mid_act, groups, d_route, s.moe_slot_out.as<float>(),
+        launch_moe_down_mfma(down_dev, down_quant, s.moe_mid.as<float>(), groups, d_route, s.moe_slot_out.as<float>(),
                              static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
         if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
         return RNB_HIP_OK;
     }
+    RESERVE_TRY(s.moe_mid_qs, n_slots * n_ff);
+    RESERVE_TRY(s.moe_mid_d, n_slots * sh.nb_mid * sizeof(float));
+    RESERVE_TRY(s.moe_mid_bsums, n_slots * sh.nb_mid * 16 * sizeof(int16_t));
     launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
     launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),

@@ -158,7 +158,7 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
 bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant);  // the tiles' LDS images fit
 void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                              uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
-void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const float *mid, MoeGroups groups,
                           const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // down + route weight + ordered per-token sum in one launch (rows of at most 16 super-blocks); slot_expert [n_slots]
 void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,

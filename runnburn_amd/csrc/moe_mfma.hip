@@ -10,8 +10,10 @@
 // unit when the groups are small.
 //   gate/up   mid[slot][n_ff] = silu(Wg[e] . a_tok) * (Wu[e] . a_tok), both Q4_K: the two matrices share the activation
 //             operand of every instruction                        fanout.rs:260-327, activation.rs:73-89
-//   down      slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])), Q4_K, Q5_K or Q6_K
+//   down      slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])), Q4_K, Q5_K or Q6_K; mid is quantised as the
+//             kernel stages it (no quantiser launch between the two kernels)
 // (crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs, crates/rnb-cpu/src/kernels/activation.rs)
+#include "act_quant.h"
 #include "device_utils.h"
 #include "kernels.h"
 #include "mfma_blocks.h"
@@ -348,8 +350,8 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant, int kJ>
 __global__ void __launch_bounds__(kGbThreads, 2)
-    moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
-                         const uint8_t *__restrict__ mdig, const uint32_t *__restrict__ grp_expert,
+    moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const float *__restrict__ mid,
+                         const uint32_t *__restrict__ grp_expert,
                          const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
                          const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
                          uint32_t tiles_per_wg, uint32_t img_toks) {
@@ -377,6 +379,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     };
     // Q6_K rows come in by whole cache lines through the wave's strip of LDS (RowRoute: the lane-owns-row loads of
     // q6_load_row touch 64 lines per instruction); the other formats' 16-byte loads go straight to the lane
+    __shared__ int16_t s_bsums[kGbWaves][16];  // the quantiser's 16-element sums: not used by these kernels
     __shared__ __attribute__((aligned(16))) uint8_t s_w[kSix ? kGbWaves : 1][kSix ? 32 * kQ6StripStride : 16];
     uint8_t *strip = s_w[kSix ? wave : 0];
     RowRoute<kQ6Pieces> route;
@@ -409,7 +412,33 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);
         tile_map_fill(s_map, sorted_slot, sorted_slot, slot_route, start + tile0, live, tid);
         __syncthreads();
-        tile_image_fill<kGbThreads>(img, s_map, mq, md, mdig, tid, live);
+        // the tile's slots' intermediates (f32, [slot][nb * 256]) are quantised to Q8_K as they are staged, with the
+        // stand-alone quantiser's wave-level routine (the same bits): wave w takes (token, block) pairs w, w + 4, ...,
+        // four loads in flight.  The workgroups of a group's other row tiles repeat this; it is a few blocks each.
+        {
+            const uint32_t pairs = live * nb;
+            for (uint32_t p0 = wave; p0 < pairs; p0 += 4 * kGbWaves) {
+                float4 v[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t p = p0 + k * kGbWaves;
+                    v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (p < pairs) {
+                        const uint32_t t = p / nb, b = p - t * nb;
+                        v[k] = reinterpret_cast<const float4 *>(mid + (static_cast<size_t>(s_map.act_row[t]) * nb + b) * 256)[lane];
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t p = p0 + k * kGbWaves;
+                    if (p < pairs) {  // wave-uniform
+                        const uint32_t t = p / nb, b = p - t * nb;
+                        q8k_quantize_vals(v[k], lane, reinterpret_cast<int8_t *>(img.act(b) + t * kStride), &img.dx(b)[t], s_bsums[wave],
+                                          kSix ? nullptr : reinterpret_cast<uint8_t *>(&img.dig(b)[t]));
+                    }
+                }
+            }
+        }
         if constexpr (kSix) q6_take(c6);
         __syncthreads();
         float accf[4 * kJ];
@@ -518,7 +547,7 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
 #undef RNB_LAUNCH_GUW
 }
 
-void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const float *mid, MoeGroups groups,
                           const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (groups.n_groups == 0 || n_embd == 0) return;
     // A workgroup's setup (group, map, image: a chain of dependent loads) costs more than a row tile's few blocks, and
@@ -533,7 +562,7 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, ActView 
     if (toks == 0) return;
 #define RNB_LAUNCH_DMJ(Q, J, LDS)                                                                                     \
     if (!allow_lds<static_cast<int>(Q) * 8 + J>(moe_down_mfma_kernel<Q, J>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return; \
-    hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid_act.qs, mid_act.d, mid_act.digits, \
+    hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid,                         \
                        groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg, toks)
 #define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
     if (toks <= 8) {                                                                                                  \

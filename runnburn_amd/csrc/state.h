@@ -63,7 +63,7 @@ struct State {
     bool act_has_digits = false;
     DeviceBuf out_f32;    // staged outputs
     DeviceBuf gemm_slices;  // per-slice outputs of a GEMM whose K range was cut to fill the chip
-    DeviceBuf moe_mid, moe_mid_qs, moe_mid_d, moe_mid_bsums, moe_mid_digits, moe_slot_out, moe_tables;
+    DeviceBuf moe_mid, moe_mid_qs, moe_mid_d, moe_mid_bsums, moe_slot_out, moe_tables;
     PinnedBuf bounce_in, bounce_out;
     TableSlot table_ring[kTableRing];  // MoE routing tables too large for a kernel argument
     int table_ring_next = 0;
