@@ -5,6 +5,7 @@
 //   q4k_gemv / q4k_gemv_into / q4k_gemv_batch   crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:183-238, 2283-2319
 //   q4_0 / q4_1 / q5_0 / q5_1 _gemv (+ _batch)  quant_api.rs:374-496
 //   q8_1_gemv (+ _batch)                         quant_api.rs:507-541
+//   iq2_xxs / iq2_s / iq3_xxs / iq4_xs _gemv (+ _batch)  quant_api.rs:543-722
 //   q2k_gemv / q3k_gemv (+ _batch)              quant_api.rs:73-181
 //   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
 //   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
@@ -124,6 +125,11 @@ RNB_HIP_BLOCK32_MIRROR(q4_1)
 RNB_HIP_BLOCK32_MIRROR(q5_0)
 RNB_HIP_BLOCK32_MIRROR(q5_1)
 RNB_HIP_BLOCK32_MIRROR(q8_1)
+// iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv (+ _batch), quant_api.rs:543-722: the same shape of function
+RNB_HIP_BLOCK32_MIRROR(iq2_xxs)
+RNB_HIP_BLOCK32_MIRROR(iq2_s)
+RNB_HIP_BLOCK32_MIRROR(iq3_xxs)
+RNB_HIP_BLOCK32_MIRROR(iq4_xs)
 #undef RNB_HIP_BLOCK32_MIRROR
 inline Result<std::vector<float>> q2k_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {
     return gemv_impl(rnb_hip_q2k_gemv, weights, rows, cols, input, rows);

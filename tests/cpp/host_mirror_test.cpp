@@ -146,6 +146,10 @@ int main(int argc, char **argv) {
         run_case(dir, "q6k_gemm", 33, 512, 20, q6k_gemv_batch);
         run_case(dir, "q5k_gemm", 40, 256, 17, q5k_gemv_batch);
         run_case(dir, "q8_0_gemm", 35, 96, 18, q8_0_gemv_batch);
+        run_case(dir, "iq4_xs_gemv", 17, 768, 1, iq4_xs_gemv);
+        run_case(dir, "iq2_xxs_batch", 12, 512, 3, iq2_xxs_gemv_batch);
+        run_case(dir, "iq3_xxs_gemv", 14, 512, 1, iq3_xxs_gemv);
+        run_case(dir, "iq2_s_batch", 9, 256, 2, iq2_s_gemv_batch);
         std::printf("run: %d failure(s)\n", failures);
         return failures ? 1 : 0;
     }

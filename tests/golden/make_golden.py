@@ -20,6 +20,7 @@ from oracle import oracle as ora  # noqa: E402
 
 Q4_0, Q5_1, Q8_1 = 2, 7, 9
 Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K = 8, 10, 11, 12, 13, 14
+IQ2_XXS, IQ3_XXS, IQ2_S, IQ4_XS = 16, 18, 22, 23
 
 
 def main():
@@ -44,7 +45,10 @@ def main():
                                          ("q4_0_gemv", Q4_0, 21, 608, 1), ("q5_1_batch", Q5_1, 10, 160, 3),
                                          # 16+ tokens: the matrix-core GEMMs of the formats other than Q4_K
                                          ("q8_1_gemv", Q8_1, 19, 160, 1), ("q6k_gemm", Q6_K, 33, 512, 20),
-                                         ("q5k_gemm", Q5_K, 40, 256, 17), ("q8_0_gemm", Q8_0, 35, 96, 18)):
+                                         ("q5k_gemm", Q5_K, 40, 256, 17), ("q8_0_gemm", Q8_0, 35, 96, 18),
+                                         # importance quants
+                                         ("iq4_xs_gemv", IQ4_XS, 17, 768, 1), ("iq2_xxs_batch", IQ2_XXS, 12, 512, 3),
+                                         ("iq3_xxs_gemv", IQ3_XXS, 14, 512, 1), ("iq2_s_batch", IQ2_S, 9, 256, 2)):
         w = ora.make_weights(quant, rows, cols, ora.tensor_seed(name, "w"))
         xin = ora.fill_normal(seq * cols, ora.tensor_seed(name, "x"), 1.0)
         ref = ora.gemv(quant, w, rows, cols, xin)

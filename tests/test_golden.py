@@ -13,7 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 GOLD = os.path.join(HERE, "golden")
 CPP_BIN = os.path.join(HERE, "cpp", "host_mirror_test")
 MATMUL_CASES = ["q4k_gemv", "q6k_gemv", "q8_0_gemv", "q4k_batch", "q6k_batch", "q8_0_batch", "q5k_gemv", "q5k_batch", "q2k_gemv",
-                "q3k_batch", "q4_0_gemv", "q5_1_batch", "q8_1_gemv", "q6k_gemm", "q5k_gemm", "q8_0_gemm"]
+                "q3k_batch", "q4_0_gemv", "q5_1_batch", "q8_1_gemv", "q6k_gemm", "q5k_gemm", "q8_0_gemm",
+                "iq4_xs_gemv", "iq2_xxs_batch", "iq3_xxs_gemv", "iq2_s_batch"]
 
 
 @pytest.fixture(scope="module")
@@ -63,7 +64,8 @@ def test_hip_reproduces_golden(rnb, gold):
            "q5k_gemv": rnb.q5k_gemv, "q5k_batch": rnb.q5k_gemv_batch, "q2k_gemv": rnb.q2k_gemv,
            "q3k_batch": rnb.q3k_gemv_batch, "q4_0_gemv": rnb.q4_0_gemv, "q5_1_batch": rnb.q5_1_gemv_batch,
            "q8_1_gemv": rnb.q8_1_gemv, "q6k_gemm": rnb.q6k_gemv_batch, "q5k_gemm": rnb.q5k_gemv_batch,
-           "q8_0_gemm": rnb.q8_0_gemv_batch}
+           "q8_0_gemm": rnb.q8_0_gemv_batch, "iq4_xs_gemv": rnb.iq4_xs_gemv, "iq2_xxs_batch": rnb.iq2_xxs_gemv_batch,
+           "iq3_xxs_gemv": rnb.iq3_xxs_gemv, "iq2_s_batch": rnb.iq2_s_gemv_batch}
     for name in MATMUL_CASES:
         _, rows, cols, _ = (int(v) for v in gold[f"{name}_shape"])
         w = np.ascontiguousarray(gold[f"{name}_w"])
