@@ -863,7 +863,9 @@ bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
     // From about 300 MB on, the separate quantiser launch costs less than what the chunked kernel gains over the
     // one-launch kernel, whose workgroups loop (steps measured back to back: 264 MB of Q4_K 49.5 us in one launch against
     // 51.1 in two, 431 MB of Q6_K 83.1 against 79.0).  The chunked kernel with the quantiser in front (one chunk per wave,
-    // one barrier per workgroup of 4, 8 or 16 waves) was tried: 431 MB of Q6_K 81 / 86 / 94 us, 264 MB of Q4_K 71 / 56 us.
+    // one barrier per workgroup of 4, 8 or 16 waves) was tried: 431 MB of Q6_K 81 / 86 / 94 us, 264 MB of Q4_K 71 / 56 us;
+    // so was the one-launch kernel looping over chunks of consecutive rows (1, 2 or 4 rows, with and without the next
+    // chunk requested ahead): 79.5 - 82.4 us and 47.2 - 50.0 us, inside the spread between boxes of what is here.
     size_t bytes = 0;
     switch (quant) {
     case kQ2K: bytes = kQ2KBytes; break;
