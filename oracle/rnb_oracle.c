@@ -51,6 +51,9 @@
  *   quantize_row_q4_0 .. _q5_1, _q8_1  not in the reference (ggml reference semantics).  Input generation only.
  *   quantize_row_q6_k/_q8_0     not in the reference at all (ggml reference semantics); round
  *                               trip through the pinned dequantisers.  Input generation only.
+ *   IQ2_XXS / IQ2_S / IQ3_XXS / IQ4_XS  dequantisers and Q8_K dots live in rnb_oracle_iq.c (pins listed there: the
+ *                               reference's FNV-1a known answers, iq.rs:258-334); rms_norm is numpy, in oracle.py
+ *                               (pinned on the reference's vectors, norm.rs tests)
  */
 #include "rnb_oracle.h"
 
