@@ -166,3 +166,66 @@ def test_gemv_with_device_input(rnb, oracle, quant, rows, cols):
     rnb.release(w)
     for b in (xd, wd, normed):
         b.free()
+
+
+@pytest.mark.gpu
+def test_decode_layer_fragment_in_a_graph(rnb, oracle):
+    """residual += post-norm(branch); pre-norm -> Q8_K in the activation scratch; two projections from that scratch and the
+    router on one of their outputs, captured into one graph after an eager run of the same shapes (which sizes the
+    scratch): three replays with new inputs uploaded between them, each compared bit for bit with the eager sequence on the
+    same inputs.  No quantiser launch and no allocation happens inside the capture."""
+    import ctypes as C
+    import bench
+    hip = bench.Hip()
+    lib = rnb.lib()
+    stream = C.c_void_p(rnb.stream_handle())
+    hidden, rows_a, n_expert, k = 2048, 640, 64, 8
+    rng = np.random.default_rng(2024)
+    wa = rnb.DeviceBuffer.from_host(oracle.make_weights(Q4_K, rows_a, hidden, 31))
+    wr = rnb.DeviceBuffer.from_host(oracle.make_weights(Q6_K, n_expert, hidden, 32))
+    pw = rnb.DeviceBuffer.from_host((rng.standard_normal(hidden) * 0.2 + 1.0).astype(np.float32))
+    qw = rnb.DeviceBuffer.from_host((rng.standard_normal(hidden) * 0.2 + 1.0).astype(np.float32))
+    branch, resid = rnb.DeviceBuffer(hidden * 4), rnb.DeviceBuffer(hidden * 4)
+    proj, logits = rnb.DeviceBuffer(rows_a * 4), rnb.DeviceBuffer(n_expert * 4)
+    ids, wts = rnb.DeviceBuffer(k * 4), rnb.DeviceBuffer(k * 4)
+    inputs = [(rng.standard_normal(hidden).astype(np.float32), rng.standard_normal(hidden).astype(np.float32)) for _ in range(3)]
+
+    def upload(b, r):
+        assert lib.rnb_hip_dev_upload(branch.ptr, b.ctypes.data_as(C.c_void_p), b.nbytes) == 0
+        assert lib.rnb_hip_dev_upload(resid.ptr, r.ctypes.data_as(C.c_void_p), r.nbytes) == 0
+
+    def enqueue():
+        rnb.rms_norm_add_rms_norm_quantize_dev(branch, pw, 1e-6, resid, qw, 1e-5, 1, hidden, None)
+        rnb.gemv_quantized_dev(Q4_K, wa, rows_a, hidden, 1, proj)
+        rnb.gemv_quantized_dev(Q6_K, wr, n_expert, hidden, 1, logits)
+        rnb.moe_route_topk_dev(logits, 1, n_expert, k, ids, wts)
+
+    def results():
+        rnb.sync()
+        return (resid.to_host(np.float32), proj.to_host(np.float32), ids.to_host(np.uint32), wts.to_host(np.float32))
+
+    eager = []
+    for b, r in inputs:
+        upload(b, r)
+        enqueue()
+        eager.append(results())
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.check(hip.rt.hipStreamBeginCapture(stream, 2), "hipStreamBeginCapture")
+    try:
+        enqueue()
+    finally:
+        rc = hip.rt.hipStreamEndCapture(stream, C.byref(graph))
+    hip.check(rc, "hipStreamEndCapture")
+    hip.check(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0), "hipGraphInstantiate")
+    try:
+        for (b, r), want in zip(inputs, eager):
+            upload(b, r)
+            hip.check(hip.rt.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            got = results()
+            for g, w_ in zip(got, want):
+                assert np.array_equal(g.view(np.uint32), w_.view(np.uint32))
+    finally:
+        hip.rt.hipGraphExecDestroy(gexec)
+        hip.rt.hipGraphDestroy(graph)
+        for buf in (wa, wr, pw, qw, branch, resid, proj, logits, ids, wts):
+            buf.free()
