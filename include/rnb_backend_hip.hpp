@@ -131,6 +131,16 @@ RNB_HIP_BLOCK32_MIRROR(iq2_s)
 RNB_HIP_BLOCK32_MIRROR(iq3_xxs)
 RNB_HIP_BLOCK32_MIRROR(iq4_xs)
 #undef RNB_HIP_BLOCK32_MIRROR
+// quant_embedding_gather(quant, weights, rows, cols, token_ids), quant_api.rs:1827-1975; `quant` is the ggml type id
+// (RNB_GGML_*), the reference's QuantFormat value
+inline Result<std::vector<float>> quant_embedding_gather(uint32_t quant, Bytes weights, size_t rows, size_t cols,
+                                                         const std::vector<uint32_t> &token_ids) {
+    std::vector<float> out(token_ids.size() * cols);
+    const int st = rnb_hip_quant_embedding_gather(quant, weights.ptr, weights.len, rows, cols, token_ids.data(),
+                                                  token_ids.size(), out.data(), out.size());
+    if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
+    return make_ok(std::move(out));
+}
 inline Result<std::vector<float>> q2k_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {
     return gemv_impl(rnb_hip_q2k_gemv, weights, rows, cols, input, rows);
 }

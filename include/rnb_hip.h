@@ -51,6 +51,10 @@ typedef enum {
 #define RNB_GGML_IQ3_XXS 18u
 #define RNB_GGML_IQ2_S 22u
 #define RNB_GGML_IQ4_XS 23u
+/* float formats: embedding tables only (rnb_hip_quant_embedding_gather) */
+#define RNB_GGML_F32 0u
+#define RNB_GGML_F16 1u
+#define RNB_GGML_BF16 30u
 
 /* BackendOp, crates/rnb-backend/api/src/lib.rs:12-18 */
 #define RNB_OP_MATMUL 0
@@ -173,6 +177,21 @@ int rnb_hip_q4k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t ro
                                        const float *x_dev, float *out, size_t out_len);
 int rnb_hip_q6k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                                        const float *x_dev, float *out, size_t out_len);
+/* quant_embedding_gather, quant_api.rs:1827-1975: out[t][cols] = row token_ids[t] of a rows x cols matrix in any of the
+ * block formats above or f32 / f16 / bf16 (quant = ggml type id), dequantised to f32 with the float operations of the
+ * reference's dequantisers in their order (crates/rnb-cpu/src/quantize/dequant.rs, iq.rs), so the values are theirs bit
+ * for bit.  Checks and texts in the reference's order, with its names for the formats (Q4K, Q80, IQ2XXS, ...):
+ * "<fmt> embedding cols must be non-zero and divisible by {32|256}, got {}", an empty id list returns at once,
+ * "<fmt> embedding token id {} is out of range for {} rows", "<fmt> embedding weight byte mismatch: got {}, expected {}".
+ * A matrix that is resident already (rnb_hip_prewarm or an earlier matmul) is read in place; otherwise only the rows
+ * named by the ids are uploaded, for this call.  out_len >= n_tokens * cols. */
+int rnb_hip_quant_embedding_gather(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                   const uint32_t *token_ids, size_t n_tokens, float *out, size_t out_len);
+/* the same with the result left on the device (out_dev: n_tokens * cols floats, 16-byte aligned), where
+ * rnb_hip_rms_norm_dev picks it up: launch_quant_embedding_gather_with_weights_dev,
+ * crates/rnb-backend/cuda/src/runtime/state/launchers.rs:4062 */
+int rnb_hip_quant_embedding_gather_dev(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                       const uint32_t *token_ids, size_t n_tokens, float *out_dev);
 /* iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv and their batch forms, quant_api.rs:543-722 (same checks and
  * texts): importance-quant rows (66 / 82 / 98 / 136-byte blocks of 256 elements) x Q8_K(x), the block dots of
  * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Every

@@ -9,6 +9,7 @@ functions keep the reference's names, argument meaning and error behaviour:
   q8_1_gemv (+ _batch)                         quant_api.rs:507-541
   q2k_gemv / q3k_gemv (+ _batch)              quant_api.rs:73-181
   iq2_xxs / iq2_s / iq3_xxs / iq4_xs _gemv (+ _batch)  quant_api.rs:543-722
+  quant_embedding_gather                       quant_api.rs:1827-1975
   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
@@ -87,6 +88,11 @@ from .binding import (  # noqa: F401
     GGML_IQ3_XXS,
     GGML_IQ2_S,
     GGML_IQ4_XS,
+    GGML_F32,
+    GGML_F16,
+    GGML_BF16,
+    quant_embedding_gather,
+    quant_embedding_gather_dev,
     q2k_gemv,
     q2k_gemv_batch,
     q3k_gemv,

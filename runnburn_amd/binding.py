@@ -13,6 +13,7 @@ _LIB_PATH = os.path.join(_PKG, "librnb_hip.so")
 GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1, GGML_Q8_1 = 2, 3, 6, 7, 9
 GGML_Q8_0, GGML_Q2_K, GGML_Q3_K, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 10, 11, 12, 13, 14
 GGML_IQ2_XXS, GGML_IQ3_XXS, GGML_IQ2_S, GGML_IQ4_XS = 16, 18, 22, 23
+GGML_F32, GGML_F16, GGML_BF16 = 0, 1, 30  # embedding tables only
 OP_MATMUL, OP_ATTENTION, OP_GDN, OP_MOE, OP_SAMPLER = 0, 1, 2, 3, 4
 STATUS_NAMES = {0: "Ok", 1: "InvalidRequest", 2: "UnsupportedOp", 3: "ExecutionFailed", 4: "NoDevice"}
 
@@ -57,6 +58,8 @@ SYMBOLS = [
     ("rnb_hip_q3k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q4k_gemv_with_device_input", _i, [_vp, _sz, _sz, _sz, _vp, _vp, _sz]),
     ("rnb_hip_q6k_gemv_with_device_input", _i, [_vp, _sz, _sz, _sz, _vp, _vp, _sz]),
+    ("rnb_hip_quant_embedding_gather", _i, [_u32, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
+    ("rnb_hip_quant_embedding_gather_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp, _sz, _vp]),
     ("rnb_hip_iq2_xxs_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_iq2_xxs_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_iq2_s_gemv", _i, _MATMUL_ARGS),
@@ -359,6 +362,25 @@ def q4k_gemv_with_device_input(weights, rows, cols, input_dev, output):
 def q6k_gemv_with_device_input(weights, rows, cols, input_dev, output):
     """quant_api.rs:242-284, the Q6_K form."""
     _gemv_with_device_input("rnb_hip_q6k_gemv_with_device_input", weights, rows, cols, input_dev, output)
+
+
+def quant_embedding_gather(quant: int, weights, rows: int, cols: int, token_ids) -> np.ndarray:
+    """quant_api.rs:1827-1975: the rows `token_ids` name, dequantised to f32 [len(token_ids)][cols]; `quant` is the ggml
+    type id of any block format or of f32 / f16 / bf16."""
+    w = _bytes_view(weights)
+    ids = np.ascontiguousarray(token_ids, dtype=np.uint32)
+    out = np.empty(ids.size * cols, dtype=np.float32)
+    _check(lib().rnb_hip_quant_embedding_gather(quant, _ptr(w), w.size, rows, cols, _ptr(ids), ids.size, _ptr(out), out.size))
+    return out
+
+
+def quant_embedding_gather_dev(quant: int, weights, rows: int, cols: int, token_ids, out: "DeviceBuffer") -> None:
+    """The same with the rows left on the device (launchers.rs:4062), e.g. as the input of rms_norm_dev."""
+    w = _bytes_view(weights)
+    ids = np.ascontiguousarray(token_ids, dtype=np.uint32)
+    if out.nbytes < ids.size * cols * 4:
+        raise ValueError("output buffer too small")
+    _check(lib().rnb_hip_quant_embedding_gather_dev(quant, _ptr(w), w.size, rows, cols, _ptr(ids), ids.size, out.ptr))
 
 
 def iq2_xxs_gemv(weights, rows, cols, input):  # noqa: A002

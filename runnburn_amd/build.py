@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(PKG, "librnb_hip.so")
 
-SOURCES = ["state.cpp", "residency.cpp", "api.cpp", "gguf.cpp", "quantize_act.hip", "gemv.hip", "gemm_q4k.hip", "gemm_blocks.hip", "moe.hip", "moe_mfma.hip", "static_scratch.hip", "calib.hip", "norm_route.hip", "gemv_iq.hip"]
+SOURCES = ["state.cpp", "residency.cpp", "api.cpp", "gguf.cpp", "quantize_act.hip", "gemv.hip", "gemm_q4k.hip", "gemm_blocks.hip", "moe.hip", "moe_mfma.hip", "static_scratch.hip", "calib.hip", "norm_route.hip", "gemv_iq.hip", "dequant.hip"]
 
 # -ffp-contract=off: the activation quantisers must perform single IEEE multiplies (no FMA fusion).
 # packed-fp32 ops are disabled for every kernel in this library.

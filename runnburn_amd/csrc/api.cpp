@@ -1540,3 +1540,136 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
 }
 
 }  // extern "C"
+
+namespace {
+
+// The formats of the embedding gather with the names the reference prints (`{quant:?}` of its QuantFormat) and its
+// table of elements and bytes per block: crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:1834-1853.
+struct EmbedFormat {
+    const char *name;
+    size_t elems, bytes;
+};
+bool embed_format(uint32_t quant, EmbedFormat *f) {
+    switch (quant) {
+    case kF32: *f = {"F32", 32, 128}; return true;
+    case kF16: *f = {"F16", 32, 64}; return true;
+    case kBF16: *f = {"BF16", 32, 64}; return true;
+    case kQ4_0: *f = {"Q40", 32, kQ4_0Bytes}; return true;
+    case kQ4_1: *f = {"Q41", 32, kQ4_1Bytes}; return true;
+    case kQ5_0: *f = {"Q50", 32, kQ5_0Bytes}; return true;
+    case kQ5_1: *f = {"Q51", 32, kQ5_1Bytes}; return true;
+    case kQ8_0: *f = {"Q80", 32, kQ8_0Bytes}; return true;
+    case kQ8_1: *f = {"Q81", 32, kQ8_1Bytes}; return true;
+    case kQ2K: *f = {"Q2K", 256, kQ2KBytes}; return true;
+    case kQ3K: *f = {"Q3K", 256, kQ3KBytes}; return true;
+    case kQ4K: *f = {"Q4K", 256, kQ4KBytes}; return true;
+    case kQ5K: *f = {"Q5K", 256, kQ5KBytes}; return true;
+    case kQ6K: *f = {"Q6K", 256, kQ6KBytes}; return true;
+    case kIQ2XXS: *f = {"IQ2XXS", 256, kIQ2XXSBytes}; return true;
+    case kIQ2S: *f = {"IQ2S", 256, kIQ2SBytes}; return true;
+    case kIQ3XXS: *f = {"IQ3XXS", 256, kIQ3XXSBytes}; return true;
+    case kIQ4XS: *f = {"IQ4XS", 256, kIQ4XSBytes}; return true;
+    default: return false;
+    }
+}
+
+// quant_embedding_gather (quant_api.rs:1827-1975): checks and texts in the reference's order (cols, empty id list, id
+// range, weight bytes).  A matrix that is resident already (prewarmed, or uploaded by an earlier call) is read where
+// it is; otherwise only the rows the ids name travel, one per id, and the kernel reads them in order (the
+// reference's compact_embedding_rows).  Output to the host (out_host) or to device memory (out_dev), never both.
+int embedding_gather(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols, const uint32_t *token_ids,
+                     size_t n_tokens, float *out_host, size_t out_len, float *out_dev) {
+    EmbedFormat f;
+    if (!embed_format(quant, &f) || !embed_gather_supported(quant))
+        return fail(RNB_HIP_UNSUPPORTED_OP, "unsupported quant id " + std::to_string(quant));
+    const std::string name = f.name;
+    if (cols == 0 || cols % f.elems != 0)
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding cols must be non-zero and divisible by " +
+                                                 std::to_string(f.elems) + ", got " + std::to_string(cols));
+    if (n_tokens == 0) return RNB_HIP_OK;
+    if (!token_ids) return fail(RNB_HIP_INVALID_REQUEST, name + " embedding null pointer argument");
+    for (size_t i = 0; i < n_tokens; i++)
+        if (token_ids[i] >= rows)
+            return fail(RNB_HIP_INVALID_REQUEST, name + " embedding token id " + std::to_string(token_ids[i]) +
+                                                     " is out of range for " + std::to_string(rows) + " rows");
+    const size_t blocks_per_row = cols / f.elems;
+    size_t row_bytes = 0, expected = 0, out_need = 0;
+    if (__builtin_mul_overflow(blocks_per_row, f.bytes, &row_bytes) || __builtin_mul_overflow(rows, row_bytes, &expected))
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding weight byte size overflow");
+    if (w_len != expected)
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding weight byte mismatch: got " + std::to_string(w_len) +
+                                                 ", expected " + std::to_string(expected));
+    if (__builtin_mul_overflow(n_tokens, cols, &out_need) || out_need > (~size_t(0)) / sizeof(float))
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding output length overflow");
+    if (out_host != nullptr && out_len < out_need)
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding output too small: got " + std::to_string(out_len) +
+                                                 ", expected >= " + std::to_string(out_need));
+    if (!w || (out_host == nullptr && out_dev == nullptr))
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding null pointer argument");
+    if (out_dev != nullptr && (reinterpret_cast<uintptr_t>(out_dev) & 15u))
+        return fail(RNB_HIP_INVALID_REQUEST, name + " embedding output must be a 16-byte aligned device pointer");
+    if (cols > 0x7fffffffu) return fail(RNB_HIP_INVALID_REQUEST, name + " embedding shape out of range");
+
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    if (s.capturing())
+        return fail(RNB_HIP_INVALID_REQUEST, "host-pointer weights cannot be resolved while the library stream is capturing");
+    const size_t ids_bytes = n_tokens * sizeof(uint32_t), out_bytes = out_need * sizeof(float);
+    const uint8_t *w_dev = nullptr;
+    const uint32_t *ids_dev = nullptr;
+    if (s.resident_peek(w, w_len, &w_dev)) {
+        RESERVE_TRY(s.bounce_in, ids_bytes);
+        HIP_TRY(s.gather_ids.reserve(ids_bytes));
+        std::memcpy(s.bounce_in.ptr, token_ids, ids_bytes);
+        HIP_TRY(hipMemcpyAsync(s.gather_ids.ptr, s.bounce_in.ptr, ids_bytes, hipMemcpyHostToDevice, s.stream));
+        s.h2d_bytes += ids_bytes;
+        ids_dev = s.gather_ids.as<uint32_t>();
+    } else {
+        size_t compact_bytes = 0;
+        if (__builtin_mul_overflow(n_tokens, row_bytes, &compact_bytes))
+            return fail(RNB_HIP_INVALID_REQUEST, name + " embedding row byte size overflow");
+        RESERVE_TRY(s.bounce_in, compact_bytes);
+        HIP_TRY(s.gather_rows.reserve(compact_bytes));
+        uint8_t *stage = static_cast<uint8_t *>(s.bounce_in.ptr);
+        for (size_t i = 0; i < n_tokens; i++) std::memcpy(stage + i * row_bytes, w + token_ids[i] * row_bytes, row_bytes);
+        HIP_TRY(hipMemcpyAsync(s.gather_rows.ptr, stage, compact_bytes, hipMemcpyHostToDevice, s.stream));
+        s.h2d_bytes += compact_bytes;
+        w_dev = s.gather_rows.as<uint8_t>();
+    }
+    float *dst = out_dev;
+    if (dst == nullptr) {
+        HIP_TRY(s.out_f32.reserve(out_bytes));
+        dst = s.out_f32.as<float>();
+    }
+    for (size_t t0 = 0; t0 < n_tokens; t0 += 65535) {  // grid.y carries the token
+        const uint32_t n = static_cast<uint32_t>(std::min<size_t>(65535, n_tokens - t0));
+        launch_embed_gather(quant, ids_dev ? w_dev : w_dev + t0 * row_bytes, row_bytes, ids_dev ? ids_dev + t0 : nullptr, n,
+                            static_cast<uint32_t>(cols), dst + t0 * cols, s.stream);
+    }
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
+    if (out_host != nullptr) {
+        RESERVE_TRY(s.bounce_out, out_bytes);
+        HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, dst, out_bytes, hipMemcpyDeviceToHost, s.stream));
+        HIP_TRY(hipStreamSynchronize(s.stream));
+        s.d2h_bytes += out_bytes;
+        std::memcpy(out_host, s.bounce_out.ptr, out_bytes);
+    }
+    return RNB_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rnb_hip_quant_embedding_gather(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                   const uint32_t *token_ids, size_t n_tokens, float *out, size_t out_len) {
+    return embedding_gather(quant, w, w_len, rows, cols, token_ids, n_tokens, out, out_len, nullptr);
+}
+
+int rnb_hip_quant_embedding_gather_dev(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
+                                       const uint32_t *token_ids, size_t n_tokens, float *out_dev) {
+    return embedding_gather(quant, w, w_len, rows, cols, token_ids, n_tokens, nullptr, 0, out_dev);
+}
+
+}  // extern "C"

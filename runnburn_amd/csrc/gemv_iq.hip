@@ -12,7 +12,7 @@
 // every byte of an IQ3_XXS entry is 4 + 8 c, 62 for c = 7) and expanded at compile time into device tables, which every
 // workgroup copies into LDS once (the look-ups are gathers: 14336 x 4096 IQ2_XXS 13.7 -> 9.6 us, IQ3_XXS 19.6 -> 11.2 us
 // against tables read through the vector cache); a sign index of seven bits stands for those bits and their parity.
-#include "device_utils.h"
+#include "embed_gather.h"
 #include "kernels.h"
 
 namespace rnb {
@@ -218,6 +218,69 @@ struct Iq<kIQ4XS> {
     }
 };
 
+// ---- dequantisers of the embedding gather (crates/rnb-cpu/src/quantize/iq.rs:23-116): the group scale first,
+// d * (0.5 + s) * 0.25 (IQ3_XXS: * 0.5) or d * (s - 32), then times the signed code -------------------------------
+__device__ __forceinline__ uint32_t ld_u32_le(const uint8_t *p) {
+    return static_cast<uint32_t>(p[0]) | (static_cast<uint32_t>(p[1]) << 8) | (static_cast<uint32_t>(p[2]) << 16) |
+           (static_cast<uint32_t>(p[3]) << 24);
+}
+// eight bytes of a grid entry, byte j negated when bit j of `signs` is set
+__device__ __forceinline__ void signed_codes8(uint64_t grid, uint32_t signs, float db, float (&y)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int v = static_cast<int>((grid >> (8 * j)) & 0xffu);
+        y[j] = db * static_cast<float>((signs >> j) & 1u ? -v : v);
+    }
+}
+struct DqIQ2XXS {  // {f16 d, 8 x {u8 index[4], u32 signs and scale}}
+    static constexpr uint32_t kElems = 256, kBytes = kIQ2XXSBytes;
+    static __device__ __forceinline__ void octet(const uint8_t *blk, int o, float (&y)[8]) {
+        const int ib = o >> 2, l = o & 3;
+        const uint8_t *packed = blk + 2 + 8 * ib;
+        const uint32_t ss = ld_u32_le(packed + 4);
+        const float t = ld_f16(blk) * (0.5f + static_cast<float>(ss >> 28));
+        signed_codes8(g_iq2xxs.v[packed[l]], sign_byte(ss >> (7 * l)), t * 0.25f, y);
+    }
+};
+struct DqIQ2S {  // {f16 d, u8 index_low[32], u8 signs[32], u8 qh[8], u8 scales[8]}
+    static constexpr uint32_t kElems = 256, kBytes = kIQ2SBytes;
+    static __device__ __forceinline__ void octet(const uint8_t *blk, int o, float (&y)[8]) {
+        const int ib = o >> 2, l = o & 3;
+        const uint32_t high = (static_cast<uint32_t>(blk[66 + ib]) << (8 - 2 * l)) & 0x300u;
+        const uint32_t sc = l < 2 ? (blk[74 + ib] & 0x0fu) : (blk[74 + ib] >> 4);
+        const float t = ld_f16(blk) * (0.5f + static_cast<float>(sc));
+        signed_codes8(g_iq2s.v[blk[2 + 4 * ib + l] | high], blk[34 + 4 * ib + l], t * 0.25f, y);
+    }
+};
+struct DqIQ3XXS {  // {f16 d, u8 index[64], 8 x u32 signs and scale}
+    static constexpr uint32_t kElems = 256, kBytes = kIQ3XXSBytes;
+    static __device__ __forceinline__ void octet(const uint8_t *blk, int o, float (&y)[8]) {
+        const int ib = o >> 2, l = o & 3;
+        const uint32_t packed = ld_u32_le(blk + 66 + 4 * ib);
+        const float t = ld_f16(blk) * (0.5f + static_cast<float>(packed >> 28));
+        const uint64_t grid = static_cast<uint64_t>(g_iq3xxs.v[blk[2 + 8 * ib + 2 * l]]) |
+                              (static_cast<uint64_t>(g_iq3xxs.v[blk[2 + 8 * ib + 2 * l + 1]]) << 32);
+        signed_codes8(grid, sign_byte(packed >> (7 * l)), t * 0.5f, y);
+    }
+};
+struct DqIQ4XS {  // {f16 d, u16 scales_h, u8 scales_l[4], u8 qs[128]}: byte j of a group = elements j and 16 + j
+    static constexpr uint32_t kElems = 256, kBytes = kIQ4XSBytes;
+    static __device__ __forceinline__ void octet(const uint8_t *blk, int o, float (&y)[8]) {
+        const int ib = o >> 2, m = o & 3;
+        const uint32_t scales_h = blk[2] | (static_cast<uint32_t>(blk[3]) << 8);
+        const uint32_t low = (blk[4 + ib / 2] >> (4 * (ib % 2))) & 0x0fu, high = ((scales_h >> (2 * ib)) & 3u) << 4;
+        const float dl = ld_f16(blk) * (static_cast<float>(low | high) - 32.0f);
+        const uint8_t *qs = blk + 8 + 16 * ib + 8 * (m & 1);
+        const uint32_t w0 = ld_u32_le(qs) >> (4 * (m >> 1)), w1 = ld_u32_le(qs + 4) >> (4 * (m >> 1));
+        const uint32_t c0 = iq4nl_lookup(w0 & 0x0f0f0f0fu), c1 = iq4nl_lookup(w1 & 0x0f0f0f0fu);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            y[j] = dl * static_cast<float>(static_cast<int8_t>((c0 >> (8 * j)) & 0xffu));
+            y[4 + j] = dl * static_cast<float>(static_cast<int8_t>((c1 >> (8 * j)) & 0xffu));
+        }
+    }
+};
+
 constexpr int kIqWaves = 4;
 
 template <uint32_t kQuant>
@@ -268,6 +331,16 @@ void launch_gemv_iq(const uint8_t *w, uint32_t quant, ActView act, float *out, u
     case kIQ2S: launch_iq<kIQ2S>(w, act, out, rows, nb, seq, stream); break;
     case kIQ3XXS: launch_iq<kIQ3XXS>(w, act, out, rows, nb, seq, stream); break;
     default: launch_iq<kIQ4XS>(w, act, out, rows, nb, seq, stream); break;
+    }
+}
+
+void launch_embed_gather_iq(uint32_t quant, const uint8_t *w, size_t row_bytes, const uint32_t *ids, uint32_t n_tokens,
+                            uint32_t cols, float *out, hipStream_t stream) {
+    switch (quant) {
+    case kIQ2XXS: launch_embed_gather_format<DqIQ2XXS>(w, row_bytes, ids, n_tokens, cols, out, stream); break;
+    case kIQ2S: launch_embed_gather_format<DqIQ2S>(w, row_bytes, ids, n_tokens, cols, out, stream); break;
+    case kIQ3XXS: launch_embed_gather_format<DqIQ3XXS>(w, row_bytes, ids, n_tokens, cols, out, stream); break;
+    default: launch_embed_gather_format<DqIQ4XS>(w, row_bytes, ids, n_tokens, cols, out, stream); break;
     }
 }
 

@@ -11,6 +11,7 @@
 namespace rnb {
 
 constexpr uint32_t kQ4_0 = 2, kQ4_1 = 3, kQ5_0 = 6, kQ5_1 = 7, kQ8_0 = 8, kQ8_1 = 9, kQ2K = 10, kQ3K = 11, kQ4K = 12, kQ5K = 13, kQ6K = 14;  // ggml type ids
+constexpr uint32_t kF32 = 0, kF16 = 1, kBF16 = 30;  // float formats (embedding tables only)
 constexpr uint32_t kIQ2XXS = 16, kIQ3XXS = 18, kIQ2S = 22, kIQ4XS = 23;  // importance quants (256-element blocks, Q8_K activations)
 constexpr size_t kIQ2XXSBytes = 66, kIQ3XXSBytes = 98, kIQ2SBytes = 82, kIQ4XSBytes = 136;
 constexpr size_t kQ4_0Bytes = 18, kQ4_1Bytes = 20, kQ5_0Bytes = 22, kQ5_1Bytes = 24, kQ8_0Bytes = 34, kQ8_1Bytes = 36, kQ2KBytes = 84, kQ3KBytes = 110, kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210;
@@ -46,6 +47,13 @@ void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 bool is_iq_quant(uint32_t quant);
 void launch_gemv_iq(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                     hipStream_t stream);
+// Embedding gather: out[t][cols] = dequantised row ids[t] (row t when ids is null) of a matrix in any of the block formats
+// or f32 / f16 / bf16; values bit-identical to the reference's dequantisers.  n_tokens <= 65535, cols % 32 (256) == 0.
+bool embed_gather_supported(uint32_t quant);
+void launch_embed_gather(uint32_t quant, const uint8_t *w, size_t row_bytes, const uint32_t *ids, uint32_t n_tokens,
+                         uint32_t cols, float *out, hipStream_t stream);
+void launch_embed_gather_iq(uint32_t quant, const uint8_t *w, size_t row_bytes, const uint32_t *ids, uint32_t n_tokens,
+                            uint32_t cols, float *out, hipStream_t stream);
 // Q2_K / Q3_K rows (84 / 110-byte blocks at 4- / 2-byte alignment); quant is kQ2K or kQ3K
 void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                          uint32_t seq, hipStream_t stream);

@@ -137,6 +137,32 @@ int ResidentTable::alloc_with_retry(size_t bytes, void **dev, std::string *err) 
     }
 }
 
+bool ResidentTable::peek(const uint8_t *ptr, size_t len, uint64_t fingerprint, const uint8_t **dev_out) {
+    const Key key = reinterpret_cast<Key>(ptr);
+    auto it = table_.find(key);
+    if (it != table_.end() && it->second.len == len) {
+        if (it->second.fingerprint != fingerprint) return false;
+        ++stats_.lookups;
+        ++stats_.hits;
+        touch(key, it->second);
+        *dev_out = static_cast<const uint8_t *>(it->second.dev);
+        return true;
+    }
+    auto up = table_.upper_bound(key);
+    while (up != table_.begin()) {
+        --up;
+        const Key base = up->first;
+        if (up->second.pinned && key >= base && key + len <= base + up->second.len) {
+            ++stats_.lookups;
+            ++stats_.sub_range_hits;
+            touch(base, up->second);
+            *dev_out = static_cast<const uint8_t *>(up->second.dev) + (key - base);
+            return true;
+        }
+    }
+    return false;
+}
+
 int ResidentTable::resolve(const uint8_t *ptr, size_t len, uint64_t fingerprint, bool pin, const uint8_t **dev_out,
                            std::string *err) {
     const Key key = reinterpret_cast<Key>(ptr);

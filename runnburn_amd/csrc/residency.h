@@ -100,6 +100,9 @@ class ResidentTable {
     // of a pinned parent, a fresh upload that becomes resident, or an upload for this call only.  `fingerprint` is the
     // caller's cheap content hash of the range.  Returns 0, or an error code of the allocator with *err set.
     int resolve(const uint8_t *ptr, size_t len, uint64_t fingerprint, bool pin, const uint8_t **dev_out, std::string *err);
+    // Device address of [ptr, ptr + len) when it is resident already (exact match or sub-range of a pinned parent);
+    // false otherwise: nothing is uploaded and nothing evicted (the embedding gather then moves only the rows it needs).
+    bool peek(const uint8_t *ptr, size_t len, uint64_t fingerprint, const uint8_t **dev_out);
     // Drops the entry that starts at ptr with this length; false when there is none.
     bool release(const uint8_t *ptr, size_t len, std::string *err);
     // Frees every unpinned entry (offload_non_pinned_resident_q4k, q4k_cache.rs:276-303); returns the bytes freed.

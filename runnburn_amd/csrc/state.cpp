@@ -167,6 +167,10 @@ int State::resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out,
     return RNB_HIP_EXECUTION_FAILED;
 }
 
+bool State::resident_peek(const uint8_t *ptr, size_t len, const uint8_t **dev_out) {
+    return table->peek(ptr, len, fingerprint(ptr, len), dev_out);
+}
+
 bool State::release(const uint8_t *ptr, size_t len) {
     std::string err;
     return table->release(ptr, len, &err);

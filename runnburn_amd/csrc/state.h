@@ -64,6 +64,7 @@ struct State {
     DeviceBuf out_f32;    // staged outputs
     DeviceBuf gemm_slices;  // per-slice outputs of a GEMM whose K range was cut to fill the chip
     DeviceBuf moe_mid, moe_mid_qs, moe_mid_d, moe_mid_bsums, moe_slot_out, moe_tables;
+    DeviceBuf gather_ids, gather_rows;  // embedding gather: token ids; the rows of a matrix that is not resident
     PinnedBuf bounce_in, bounce_out;
     TableSlot table_ring[kTableRing];  // MoE routing tables too large for a kernel argument
     int table_ring_next = 0;
@@ -82,6 +83,8 @@ struct State {
     // of a pinned (prewarmed) parent, a fresh untouched upload that becomes resident, or an upload for this call only.
     // Returns an rnb_hip_status with the message set.
     int resident_ptr(const uint8_t *ptr, size_t len, const uint8_t **dev_out, bool pin = false);
+    // the device copy of [ptr, ptr+len) if there is one already (no upload); false otherwise
+    bool resident_peek(const uint8_t *ptr, size_t len, const uint8_t **dev_out);
     bool release(const uint8_t *ptr, size_t len);
     // true while the library stream is capturing into a graph (also remembers that a capture happened)
     bool capturing();

@@ -53,6 +53,11 @@ static int validate() {
     float out1 = 0;
     auto u = q4k_gemv_into({w.data(), 144}, 1, 256, {x.data(), 256}, &out1, 0);
     EXPECT(!u && u.error == "Q4_K shape mismatch: input=256 output=0 expected input=256 output>=1", "into message");
+    auto eg = quant_embedding_gather(RNB_GGML_Q4_K, {w.data(), 144}, 1, 256, {0, 1});
+    EXPECT(!eg && eg.status == RNB_HIP_INVALID_REQUEST && eg.error == "Q4K embedding token id 1 is out of range for 1 rows",
+           "embedding id message");
+    eg = quant_embedding_gather(RNB_GGML_Q6_K, {w.data(), 144}, 1, 256, {0});
+    EXPECT(!eg && eg.error == "Q6K embedding weight byte mismatch: got 144, expected 210", "embedding weight bytes message");
     auto m = qwen35_sparse_experts_selected_base_by_token({w.data(), 144}, {w.data(), 144}, {w.data(), 144}, {0, 1}, {1.0f}, {0}, 1, 14, 256, 256, {x.data(), 256});
     EXPECT(!m && m.error.find("length mismatch") != std::string::npos, "moe slot arrays message");
     {
@@ -118,6 +123,25 @@ static void run_case(const std::string &dir, const char *name, size_t rows, size
     std::printf("%s: %zu outputs, max |diff| %.3g (rms %.3g)\n", name, want.size(), worst, rms);
 }
 
+// rows [last, 0, 2, 2] of a golden weight file, dequantised on the device: bit-identical to the fixture
+static void embed_case(const std::string &dir, const char *name, uint32_t quant, size_t rows, size_t cols) {
+    const auto w = read_file<uint8_t>(dir + "/" + name + "_w.bin");
+    const auto want = read_file<float>(dir + "/embed_" + name + "_out.bin");
+    if (w.empty() || want.empty()) return;
+    auto r = quant_embedding_gather(quant, {w.data(), w.size()}, rows, cols, {static_cast<uint32_t>(rows - 1), 0, 2, 2});
+    if (!r) {
+        std::printf("FAIL: embed %s: %s\n", name, r.error.c_str());
+        failures++;
+        return;
+    }
+    EXPECT(r.value.size() == want.size() && want.size() == 4 * cols, "embedding output size");
+    size_t differing = 0;
+    for (size_t i = 0; i < want.size() && i < r.value.size(); i++)
+        differing += std::memcmp(&r.value[i], &want[i], sizeof(float)) != 0;
+    if (differing) failures++;
+    std::printf("embed %s: %zu values, %zu differ\n", name, want.size(), differing);
+}
+
 int main(int argc, char **argv) {
     if (argc >= 2 && std::strcmp(argv[1], "validate") == 0) {
         const int f = validate();
@@ -150,6 +174,10 @@ int main(int argc, char **argv) {
         run_case(dir, "iq2_xxs_batch", 12, 512, 3, iq2_xxs_gemv_batch);
         run_case(dir, "iq3_xxs_gemv", 14, 512, 1, iq3_xxs_gemv);
         run_case(dir, "iq2_s_batch", 9, 256, 2, iq2_s_gemv_batch);
+        embed_case(dir, "q4k_gemv", RNB_GGML_Q4_K, 24, 1024);
+        embed_case(dir, "q6k_gemv", RNB_GGML_Q6_K, 20, 768);
+        embed_case(dir, "q8_0_gemv", RNB_GGML_Q8_0, 16, 544);
+        embed_case(dir, "iq2_s_batch", RNB_GGML_IQ2_S, 9, 256);
         std::printf("run: %d failure(s)\n", failures);
         return failures ? 1 : 0;
     }

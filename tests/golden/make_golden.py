@@ -5,6 +5,7 @@
 golden_small.npz   inputs + expected outputs for small cases of every operator on the path, so that a
                    GPU box can check the HIP library with nothing but numpy.
 <name>_{w,x,out}.bin  the same matmul cases as raw little-endian files (u8 weights, f32 input, f32 output)
+embed_<name>_out.bin  rows [last, 0, 2, 2] of <name>_w.bin dequantised (f32), the embedding-gather cases
                    for the C++ host-mirror test (tests/cpp/host_mirror_test.cpp).
 The vectors come from OUR oracle, which tests/test_oracle_pins.py pins against the reference's
 known-answer tests; the reference itself (Rust) cannot run here.
@@ -57,6 +58,14 @@ def main():
         w.tofile(os.path.join(HERE, f"{name}_w.bin"))
         xin.astype("<f4").tofile(os.path.join(HERE, f"{name}_x.bin"))
         ref.astype("<f4").tofile(os.path.join(HERE, f"{name}_out.bin"))
+    # embedding gather: rows [last, 0, 2, 2] of four of the matrices above, dequantised
+    for name in ("q4k_gemv", "q6k_gemv", "q8_0_gemv", "iq2_s_batch"):
+        quant, rows, cols, _ = (int(v) for v in out[f"{name}_shape"])
+        ids = np.array([rows - 1, 0, 2, 2], np.uint32)
+        table = out[f"{name}_w"].reshape(rows, -1)
+        emb = np.concatenate([ora.dequantize(quant, table[i]) for i in ids])
+        out[f"embed_{name}_ids"], out[f"embed_{name}_out"] = ids, emb
+        emb.astype("<f4").tofile(os.path.join(HERE, f"embed_{name}_out.bin"))
     # MoE: 4 experts, 2 tokens, top-2
     n_expert, n_ff, n_embd = 4, 256, 512
     gate = ora.make_weights(Q4_K, n_expert * n_ff, n_embd, ora.tensor_seed("moe", "gate"))

@@ -258,3 +258,23 @@ def test_dense_ffn_validation_messages():
     assert str(e) == "dense SiLU FFN batch down byte mismatch: got 45055, expected 45056"
     e = _err(f, g, g, z(256 * 8 * 24 + 1, np.uint8), 7, 256, 256, 2, z(512, np.float32))  # Q5_1 down: 24-byte blocks
     assert str(e) == "dense SiLU FFN batch down byte mismatch: got 49153, expected 49152"
+
+
+def test_embedding_gather_validation_messages_match_reference():
+    """crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:1854-1885: the format's Debug name, checks in this order."""
+    z = np.zeros
+    ids = np.array([0, 5], dtype=np.uint32)
+    e = _err(rnb.quant_embedding_gather, rnb.GGML_Q4_K, z(144, np.uint8), 1, 255, ids)
+    assert (e.kind, str(e)) == ("InvalidRequest", "Q4K embedding cols must be non-zero and divisible by 256, got 255")
+    e = _err(rnb.quant_embedding_gather, rnb.GGML_Q8_0, z(34, np.uint8), 1, 0, ids)
+    assert str(e) == "Q80 embedding cols must be non-zero and divisible by 32, got 0"
+    # an empty id list returns before the other checks
+    assert rnb.quant_embedding_gather(rnb.GGML_Q6_K, z(1, np.uint8), 4, 256, np.zeros(0, np.uint32)).size == 0
+    e = _err(rnb.quant_embedding_gather, rnb.GGML_IQ2_XXS, z(66 * 5, np.uint8), 5, 256, ids)
+    assert str(e) == "IQ2XXS embedding token id 5 is out of range for 5 rows"
+    e = _err(rnb.quant_embedding_gather, rnb.GGML_Q6_K, z(210 * 6 - 1, np.uint8), 6, 256, ids)
+    assert str(e) == "Q6K embedding weight byte mismatch: got 1259, expected 1260"
+    e = _err(rnb.quant_embedding_gather, rnb.GGML_BF16, z(64 * 6 * 2 + 2, np.uint8), 6, 64, ids)
+    assert str(e) == "BF16 embedding weight byte mismatch: got 770, expected 768"
+    e = _err(rnb.quant_embedding_gather, 17, z(74 * 6, np.uint8), 6, 256, ids)
+    assert e.kind == "UnsupportedOp"

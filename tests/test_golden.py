@@ -15,6 +15,7 @@ CPP_BIN = os.path.join(HERE, "cpp", "host_mirror_test")
 MATMUL_CASES = ["q4k_gemv", "q6k_gemv", "q8_0_gemv", "q4k_batch", "q6k_batch", "q8_0_batch", "q5k_gemv", "q5k_batch", "q2k_gemv",
                 "q3k_batch", "q4_0_gemv", "q5_1_batch", "q8_1_gemv", "q6k_gemm", "q5k_gemm", "q8_0_gemm",
                 "iq4_xs_gemv", "iq2_xxs_batch", "iq3_xxs_gemv", "iq2_s_batch"]
+EMBED_CASES = ["q4k_gemv", "q6k_gemv", "q8_0_gemv", "iq2_s_batch"]
 
 
 @pytest.fixture(scope="module")
@@ -34,6 +35,13 @@ def test_oracle_reproduces_golden(oracle, gold):
         assert np.array_equal(out, gold[f"{name}_out"]), name
         raw = np.fromfile(os.path.join(GOLD, f"{name}_out.bin"), dtype="<f4")
         assert np.array_equal(raw, gold[f"{name}_out"].ravel())
+    for name in EMBED_CASES:
+        quant, rows, cols, _ = (int(v) for v in gold[f"{name}_shape"])
+        table = gold[f"{name}_w"].reshape(rows, -1)
+        emb = np.concatenate([oracle.dequantize(quant, table[i]) for i in gold[f"embed_{name}_ids"]])
+        assert np.array_equal(emb.view(np.uint32), gold[f"embed_{name}_out"].view(np.uint32)), name
+        raw = np.fromfile(os.path.join(GOLD, f"embed_{name}_out.bin"), dtype="<f4")
+        assert np.array_equal(raw.view(np.uint32), emb.view(np.uint32))
     n_expert, n_ff, n_embd, tokens = (int(v) for v in gold["moe_shape"])
     out = oracle.moe_sparse_experts_by_token(gold["moe_gate"], gold["moe_up"], gold["moe_down"], n_expert,
                                              gold["moe_expert"], gold["moe_route"], gold["moe_token"], tokens, 14, n_ff,
@@ -73,6 +81,10 @@ def test_hip_reproduces_golden(rnb, gold):
         bad, diff, _ = npref.close_rows(got, gold[f"{name}_out"], rel=1e-3)
         assert np.all(np.isfinite(got)) and bad.size == 0, (name, diff.max())
         rnb.release(w)
+    for name in EMBED_CASES:  # embedding gather: the dequantiser's bits
+        quant, rows, cols, _ = (int(v) for v in gold[f"{name}_shape"])
+        got = rnb.quant_embedding_gather(quant, np.ascontiguousarray(gold[f"{name}_w"]), rows, cols, gold[f"embed_{name}_ids"])
+        assert np.array_equal(got.view(np.uint32), gold[f"embed_{name}_out"].view(np.uint32)), name
     n_expert, n_ff, n_embd, tokens = (int(v) for v in gold["moe_shape"])
     g, u, d = (np.ascontiguousarray(gold[k]) for k in ("moe_gate", "moe_up", "moe_down"))
     got = rnb.qwen35_sparse_experts_selected_base_by_token(g, u, d, gold["moe_expert"], gold["moe_route"],
