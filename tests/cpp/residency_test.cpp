@@ -206,6 +206,34 @@ static void test_pinned_and_sub_ranges() {
     CHECK(d.is_live(slab) && d.is_live(slab2) && t.entries() == 2);
 }
 
+static void test_peek_never_uploads() {
+    // the embedding gather asks whether a table is resident already and moves single rows when it is not
+    FakeDevice d;
+    ResidentTable t(&d);
+    t.set_budget(64);
+    const uint8_t *dev = nullptr;
+    CHECK(!t.peek(H(0), 16, 1, &dev) && d.uploads == 0 && t.entries() == 0 && t.stats().lookups == 0);
+    t.begin_call();
+    const uint8_t *table = resolve_ok(t, 0, 16);
+    t.begin_call();
+    CHECK(t.peek(H(0), 16, 1, &dev) && dev == table && d.uploads == 1 && t.stats().hits == 1);
+    CHECK(!t.peek(H(0), 16, /*fingerprint=*/2, &dev));  // the host range now holds other bytes: not the resident copy
+    CHECK(!t.peek(H(0), 8, 1, &dev) && !t.peek(H(4), 8, 1, &dev));  // unpinned entries serve no sub-ranges
+    t.begin_call();
+    const uint8_t *slab = resolve_ok(t, 100, 32, /*pin=*/true);
+    CHECK(t.peek(H(108), 8, 7, &dev) && dev == slab + 8 && t.stats().sub_range_hits == 1);
+    CHECK(!t.peek(H(124), 16, 7, &dev));  // runs past the end of the parent
+    CHECK(d.uploads == 2 && t.entries() == 2 && t.stats().misses == 2);
+    // a peek counts as a use: the peeked entry is not the next victim
+    t.begin_call();
+    const uint8_t *other = resolve_ok(t, 200, 8);
+    t.begin_call();
+    CHECK(t.peek(H(0), 16, 1, &dev));
+    t.begin_call();
+    t.set_budget(t.resident_bytes() - 1);  // one unpinned entry has to go: the one at 200, the older use
+    CHECK(d.is_live(table) && !d.is_live(other) && t.stats().evictions == 1 && t.entries() == 2);
+}
+
 static void test_oom_ladder() {
     FakeDevice d;
     d.capacity = 12;  // the device holds less than the budget allows
@@ -267,6 +295,7 @@ int main() {
     test_admission_and_lru_order();
     test_current_call_is_protected();
     test_pinned_and_sub_ranges();
+    test_peek_never_uploads();
     test_oom_ladder();
     test_reuse_history();
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
