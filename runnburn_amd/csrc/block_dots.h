@@ -188,6 +188,11 @@ struct Q6KRegs {
     uint32_t d_bits;
 };
 
+// Every other 210-byte block starts 2 bytes off a 4-byte boundary.  Fetching the pieces from the boundary below them
+// with one dword more and funnel-shifting them into place (nine dword-aligned loads instead of five) was measured
+// slower in every kernel (4096 x 14336: 11.3 -> 15.5 us, 14336 x 4096: 11.2 -> 12.0 us, 128256 x 4096: 78 -> 83 us): the
+// number of load instructions counts for more than their alignment here, unlike the 32-element formats, whose pairs
+// need fewer loads when aligned (gemv.hip::block32_load_pair).
 __device__ __forceinline__ Q6KRegs q6k_load_block(const uint8_t *__restrict__ blk, int q) {
     Q6KRegs r;
     const int n = q >> 1, th = q & 1;

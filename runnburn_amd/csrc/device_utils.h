@@ -17,6 +17,10 @@ typedef uint4 __attribute__((aligned(2))) uint4_a2;
 typedef uint2 __attribute__((aligned(2))) uint2_a2;
 typedef uint32_t __attribute__((aligned(2))) uint32_a2;
 
+// loads known to sit on a 4-byte boundary
+typedef uint4 __attribute__((aligned(4))) uint4_a4;
+typedef uint2 __attribute__((aligned(4))) uint2_a4;
+
 __device__ __forceinline__ uint4 ld_u4_a2(const uint8_t *p) { return *reinterpret_cast<const uint4_a2 *>(p); }
 __device__ __forceinline__ uint2 ld_u2_a2(const uint8_t *p) { return *reinterpret_cast<const uint2_a2 *>(p); }
 __device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) { return *reinterpret_cast<const uint32_a2 *>(p); }

@@ -677,8 +677,6 @@ template <uint32_t kQuant>
 constexpr bool block32_pairs() {
     return kQuant == kQ8_0 || kQuant == kQ4_0 || kQuant == kQ5_0;
 }
-typedef uint4 __attribute__((aligned(4))) uint4_a4;
-typedef uint2 __attribute__((aligned(4))) uint2_a4;
 __device__ __forceinline__ uint32_t mid32(uint32_t hi, uint32_t lo) { return __builtin_amdgcn_alignbit(hi, lo, 16); }
 template <uint32_t kQuant>
 __device__ __forceinline__ void block32_load_pair(const uint8_t *__restrict__ pair, Block32Regs &a, Block32Regs &b) {
