@@ -139,8 +139,15 @@ int take_scratch(DeviceBuf &slot, Arena *arena, size_t bytes, void **out) {
 
 // Quantise seq*cols f32 values on the device into activation scratch (the state's, which then remembers what it holds,
 // or the arena's).
+// words that the quantiser's launch copies into device memory on the side (the MoE routing tables of a batch)
+struct WordCopy {
+    const uint32_t *src = nullptr;  // device memory or pinned host memory
+    uint32_t *dst = nullptr;
+    uint32_t n_words = 0;
+};
+
 int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t seq, size_t cols, ActView *view,
-                         Arena *arena = nullptr) {
+                         Arena *arena = nullptr, const WordCopy *copy = nullptr) {
     const size_t n = seq * cols;
     SCRATCH_TRY(s.act_qs, n, int8_t, qs);
     bool has_digits = false;
@@ -157,7 +164,10 @@ int quantize_activations(State &s, uint32_t quant, const float *x_dev, size_t se
             SCRATCH_TRY(s.act_digits, n / 256 * 16, uint8_t, dg);
             digits = dg;
         }
-        launch_quantize_q8k(x_dev, n / 256, qs, d, bsums, digits, s.stream);
+        if (copy != nullptr && copy->n_words != 0)
+            launch_quantize_q8k_copy(x_dev, n / 256, qs, d, bsums, digits, copy->src, copy->n_words, copy->dst, s.stream);
+        else
+            launch_quantize_q8k(x_dev, n / 256, qs, d, bsums, digits, s.stream);
         *view = {qs, d, bsums, digits};
     }
     if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
@@ -631,11 +641,6 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     if (n_groups) std::memcpy(h_gexp, grp_expert.data(), n_groups * 4);
     std::memcpy(h_gstart, grp_start.data(), (n_groups + 1) * 4);
     uint32_t *d = s.moe_tables.as<uint32_t>();
-    if (ring_slot) {
-        HIP_TRY(hipMemcpyAsync(d, h, table_words * 4, hipMemcpyHostToDevice, s.stream));
-        HIP_TRY(hipEventRecord(ring_slot->event, s.stream));
-        s.h2d_bytes += table_words * 4;
-    }
     const float *d_route = reinterpret_cast<const float *>(d);
     const uint32_t *d_off = d + n_slots, *d_list = d_off + token_count + 1;
     uint32_t max_group = 0;
@@ -659,8 +664,12 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
         s.act_seq = token_count;
         s.act_cols = n_embd;
     } else {
-        int st = quantize_activations(s, kQ4K, x_dev, token_count, n_embd, &act);
+        // the quantiser's launch reads the tables from the pinned buffer and leaves them in device memory (no copy command)
+        const WordCopy tables{h, d, static_cast<uint32_t>(table_words)};
+        int st = quantize_activations(s, kQ4K, x_dev, token_count, n_embd, &act, nullptr, &tables);
         if (st != RNB_HIP_OK) return st;
+        HIP_TRY(hipEventRecord(ring_slot->event, s.stream));  // the pinned buffer is free again once that launch is done
+        s.h2d_bytes += table_words * 4;
     }
     if (n_slots == 0) {  // nothing routed: the reduce kernel alone writes the zero rows
         launch_moe_reduce(nullptr, d_off, d_list, out_dev, static_cast<uint32_t>(token_count),

@@ -35,6 +35,9 @@ struct ActView {
 // digits may be null
 void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
                          hipStream_t stream);
+// the same launch also copies n_words 32-bit words from words_src (device memory or pinned host memory) to words_dst
+void launch_quantize_q8k_copy(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
+                              const uint32_t *words_src, uint32_t n_words, uint32_t *words_dst, hipStream_t stream);
 // x: f32, 16-byte aligned, n_blocks*32 values; n_blocks % 8 == 0 not required
 void launch_quantize_q8(const float *x, size_t n_blocks, int8_t *qs, float *d, hipStream_t stream);
 

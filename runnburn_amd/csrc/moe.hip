@@ -438,16 +438,35 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     if (lane == 0 && row < n_embd) out[row] = acc;
 }
 
+// out[token] = sum of its slots' rows in list (= rank) order.  A thread owns four consecutive columns (n_embd is a
+// multiple of 256) and requests the rows of up to eight slots before the first addition: the additions keep the list
+// order, the loads no longer wait for one another.
 __global__ void __launch_bounds__(256)
     moe_reduce_kernel(const float *__restrict__ slot_out, const uint32_t *__restrict__ tok_offsets,
                       const uint32_t *__restrict__ tok_slots, float *__restrict__ out, uint32_t n_embd) {
     const uint32_t tok = blockIdx.y;
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= n_embd) return;
     const uint32_t begin = tok_offsets[tok], end = tok_offsets[tok + 1];
-    float acc = 0.0f;
-    for (uint32_t k = begin; k < end; k++) acc += slot_out[static_cast<size_t>(tok_slots[k]) * n_embd + i];
-    out[static_cast<size_t>(tok) * n_embd + i] = acc;
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (uint32_t k0 = begin; k0 < end; k0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t k = min(k0 + j, end - 1);
+            v[j] = *reinterpret_cast<const float4 *>(slot_out + static_cast<size_t>(tok_slots[k]) * n_embd + i);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if (k0 + j < end) {
+                acc.x += v[j].x;
+                acc.y += v[j].y;
+                acc.z += v[j].z;
+                acc.w += v[j].w;
+            }
+        }
+    }
+    *reinterpret_cast<float4 *>(out + static_cast<size_t>(tok) * n_embd + i) = acc;
 }
 
 struct TilePlan {
@@ -594,7 +613,7 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots, float *out,
                        uint32_t token_count, uint32_t n_embd, hipStream_t stream) {
     if (token_count == 0) return;
-    dim3 grid((n_embd + 255) / 256, token_count, 1);
+    dim3 grid((n_embd / 4 + 255) / 256, token_count, 1);
     hipLaunchKernelGGL(moe_reduce_kernel, grid, dim3(256), 0, stream, slot_out, tok_offsets, tok_slots, out, n_embd);
 }
 

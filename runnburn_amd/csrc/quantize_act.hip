@@ -38,6 +38,25 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     q8k_quantize_vals(v, lane, qs + blk * 256, d_out + blk, bsums + blk * 16, digits != nullptr ? digits + blk * 16 : nullptr);
 }
 
+// Same as quantize_q8k_kernel with a copy job riding along: the workgroups past the quantiser's copy `n_words` words from
+// `src`, which may be pinned host memory (the MoE routing tables of a batch: read over the bus by the kernel that runs
+// anyway instead of a copy command with a launch and a gap of its own), to `dst` in device memory.
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    quantize_q8k_copy_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ qs, float *__restrict__ d_out,
+                             int16_t *__restrict__ bsums, uint8_t *__restrict__ digits, const uint32_t *__restrict__ src,
+                             uint32_t n_words, uint32_t *__restrict__ dst, uint32_t quant_wgs) {
+    if (blockIdx.x >= quant_wgs) {  // workgroup-uniform
+        const uint32_t i = (blockIdx.x - quant_wgs) * (kWave * kWavesPerWg) + threadIdx.x;
+        if (i < n_words) dst[i] = src[i];
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t blk = static_cast<size_t>(blockIdx.x) * kWavesPerWg + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;  // wave-uniform
+    q8k_quantize_span(x + blk * 256, lane, qs + blk * 256, d_out + blk, bsums + blk * 16,
+                      digits != nullptr ? digits + blk * 16 : nullptr);
+}
+
 // Same as quantize_q8k_kernel; workgroup 0 additionally copies `n_words` routing-table words from the
 // kernel argument to device memory (n_words <= 256 = one word per thread).
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
@@ -111,6 +130,15 @@ void launch_quantize_q8k(const float *x, size_t n_blocks, int8_t *qs, float *d, 
     const unsigned grid = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
     hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(kWave * kWavesPerWg), 0, stream, x, n_blocks, qs,
                        d, bsums, digits);
+}
+
+void launch_quantize_q8k_copy(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums, uint8_t *digits,
+                              const uint32_t *words_src, uint32_t n_words, uint32_t *words_dst, hipStream_t stream) {
+    const unsigned quant_wgs = static_cast<unsigned>((n_blocks + kWavesPerWg - 1) / kWavesPerWg);
+    const unsigned copy_wgs = (n_words + kWave * kWavesPerWg - 1) / (kWave * kWavesPerWg);
+    if (quant_wgs + copy_wgs == 0) return;
+    hipLaunchKernelGGL(quantize_q8k_copy_kernel, dim3(quant_wgs + copy_wgs), dim3(kWave * kWavesPerWg), 0, stream, x, n_blocks,
+                       qs, d, bsums, digits, words_src, n_words, words_dst, quant_wgs);
 }
 
 void launch_quantize_q8k_gated(const float *gate, const float *up, size_t n_blocks, bool gelu, int8_t *qs, float *d,
