@@ -150,6 +150,58 @@ __device__ __forceinline__ void route_store16(const RowRoute<kPieces> &rt, uint8
 constexpr int kQ6Pieces = 13;        // ql, qh and scales: 208 bytes; d is read by the row's lanes themselves
 constexpr int kQ6StripStride = 216;  // 54 dwords: the 32 rows' 64-bit reads fall on 32 different bank pairs
 
+// The same route for Q6_K rows whose blocks do not all start on a 4-byte boundary (rows of an odd number of blocks: every
+// other row and every other block starts 2 bytes off), where the 16-byte loads of RowRoute take the address path about
+// a fifth longer (128 experts x top-8 at 64 tokens, loads forced onto 4-byte boundaries: down kernel 51 -> 45 us).
+// A piece is fetched from the boundary below it, and the two bytes it lacks come from the lane that holds the next
+// piece (one DPP move inside a row of sixteen lanes); a fourteenth slot per row fetches the block's last 16 bytes for
+// piece twelve.  Sixteen slots a row, four rows an instruction, eight instructions a block.  The instructions of a
+// request are four rows apart and 4 * row_bytes is a multiple of 4, so one shift serves them all.  Needs rows and base
+// at even addresses and whole 32-row tiles (no clamping of rows past the end).
+struct Q6RouteDw {
+    static constexpr int kN = 8;
+    uint32_t goff[kN];  // byte offset of this lane's piece from the wave's first row, were the row's block aligned
+    uint32_t loff;      // where the piece of instruction 0 goes in the strip; instruction i is four rows further
+    uint32_t sh;        // funnel shift of the request in flight: 0 or 16 bits
+    uint4 v[kN];
+};
+__device__ __forceinline__ void q6dw_setup(Q6RouteDw &rt, uint32_t row_bytes, int lane) {
+    const uint32_t rr = static_cast<uint32_t>(lane) >> 4, j = lane & 15;
+#pragma unroll
+    for (int i = 0; i < Q6RouteDw::kN; i++) rt.goff[i] = (4 * i + rr) * row_bytes + (j < 13 ? 16 * j : 192);
+    rt.loff = rr * kQ6StripStride + 16 * (j < 13 ? j : 12);
+    rt.sh = 0;
+}
+// base: block b of the wave's first row
+__device__ __forceinline__ void q6dw_load(Q6RouteDw &rt, const uint8_t *__restrict__ base, int lane) {
+    const uint32_t j = lane & 15;
+    const uint32_t m = (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(base)) + rt.goff[0]) & 2u;  // the row's block start mod 4
+    // pieces start m bytes early; slot 13 takes bytes 192 + m .. 208 + m of the block.  Signed: the first piece of the
+    // wave's first row sits at offset -m
+    const int32_t adj = j < 13 ? -static_cast<int32_t>(m) : static_cast<int32_t>(m);
+    rt.sh = 8 * m;
+#pragma unroll
+    for (int i = 0; i < Q6RouteDw::kN; i++)
+        rt.v[i] = *reinterpret_cast<const uint4_a4 *>(base + static_cast<ptrdiff_t>(static_cast<int32_t>(rt.goff[i]) + adj));
+}
+__device__ __forceinline__ void q6dw_store(const Q6RouteDw &rt, uint8_t *strip, int lane) {
+    const uint32_t j = lane & 15;
+#pragma unroll
+    for (int i = 0; i < Q6RouteDw::kN; i++) {
+        const uint4 v = rt.v[i];
+        // the dword after this piece: the next slot's first one, or for piece twelve the block's last four bytes
+        const uint32_t give = j == 13 ? v.w : v.x;
+        const uint32_t nx = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(give), 0x101, 0xf, 0xf, false));  // row_shl:1
+        const uint32_t o0 = __builtin_amdgcn_alignbit(v.y, v.x, rt.sh), o1 = __builtin_amdgcn_alignbit(v.z, v.y, rt.sh);
+        const uint32_t o2 = __builtin_amdgcn_alignbit(v.w, v.z, rt.sh), o3 = __builtin_amdgcn_alignbit(nx, v.w, rt.sh);
+        if (j < 13) {
+            uint8_t *dst = strip + rt.loff + i * 4 * kQ6StripStride;
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(o0, o1);
+            *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(o2, o3);
+        }
+    }
+}
+
 // a lane's share of a Q6_K block from the wave's strip (same pieces as q6_load_row, without d)
 __device__ __forceinline__ void q6_row_from_strip(Q6Row &r, const uint8_t *row, int khalf) {
 #pragma unroll

@@ -382,19 +382,17 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     __shared__ int16_t s_bsums[kGbWaves][16];  // the quantiser's 16-element sums: not used by these kernels
     __shared__ __attribute__((aligned(16))) uint8_t s_w[kSix ? kGbWaves : 1][kSix ? 32 * kQ6StripStride : 16];
     uint8_t *strip = s_w[kSix ? wave : 0];
-    RowRoute<kQ6Pieces> route;
+    // (n_embd is a multiple of 128 and down_all is 16-byte aligned: whole tiles, even addresses, as Q6RouteDw needs)
+    Q6RouteDw route;
+    if constexpr (kSix) q6dw_setup(route, static_cast<uint32_t>(row_bytes), lane);
     float d_next = 0.0f;
     auto q6_request = [&](uint32_t rt, uint32_t b) {  // block b of row tile rt: pieces into route.v, d into d_next
-        const uint32_t first = min((rt0 + rt) * kGbRows + wave * 32, n_embd - 1);  // the wave's first row
-        // offsets of rows past the end were clamped to the last row at set-up for the first row tile's distance to the
-        // end; row tiles further down are never short of rows unless they are the last one, which set-up cannot know,
-        // so the clamp is redone per request
-        route_setup<kQ6Pieces, kQ6StripStride>(route, n_embd - first, row_bytes, lane);
-        route_load(route, down_all + (static_cast<size_t>(expert) * n_embd + first) * row_bytes + b * kBlockBytes);
+        const uint32_t first = (rt0 + rt) * kGbRows + wave * 32;  // the wave's first row
+        q6dw_load(route, down_all + (static_cast<size_t>(expert) * n_embd + first) * row_bytes + b * kBlockBytes, lane);
         d_next = ld_f16(block_ptr(rt, b) + 208);
     };
     auto q6_take = [&](Q6Row &r) {
-        route_store(route, strip, lane);
+        q6dw_store(route, strip, lane);
         q6_row_from_strip(r, strip + lrow * kQ6StripStride, khalf);
         r.d = d_next;
     };
