@@ -187,15 +187,16 @@ int rnb_hip_q6k_gemv_with_device_input(const uint8_t *w, size_t w_len, size_t ro
  * named by the ids are uploaded, for this call.  out_len >= n_tokens * cols. */
 int rnb_hip_quant_embedding_gather(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                                    const uint32_t *token_ids, size_t n_tokens, float *out, size_t out_len);
-/* the same with the result left on the device (out_dev: n_tokens * cols floats, 16-byte aligned), where
+/* the same with the result left on the device (out_dev: n_tokens * cols floats, 16-byte aligned; the call returns when
+ * the rows are there), where
  * rnb_hip_rms_norm_dev picks it up: launch_quant_embedding_gather_with_weights_dev,
  * crates/rnb-backend/cuda/src/runtime/state/launchers.rs:4062 */
 int rnb_hip_quant_embedding_gather_dev(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                                        const uint32_t *token_ids, size_t n_tokens, float *out_dev);
 /* iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv and their batch forms, quant_api.rs:543-722 (same checks and
  * texts): importance-quant rows (66 / 82 / 98 / 136-byte blocks of 256 elements) x Q8_K(x), the block dots of
- * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Every
- * batch size runs one GEMV pass per token. */
+ * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Batches
+ * of four tokens and more run on the matrix cores (the same integer group sums, one f32 update per block). */
 int rnb_hip_iq2_xxs_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
                          size_t x_len, float *out, size_t out_len);
 int rnb_hip_iq2_xxs_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,

@@ -73,6 +73,8 @@ size_t gemm_min_seq(uint32_t quant, size_t rows, size_t cols) {
 }
 // The Q8_K quantiser adds the per-32 sums as two digits (the Q4_K / Q5_K GEMMs' mins term) from this many tokens on.
 constexpr size_t kDigitsMinSeq = kGemmMinSeqLarge < kGemmMinSeqSmall ? kGemmMinSeqLarge : kGemmMinSeqSmall;
+// Minimum tokens for which the importance-quant formats take their matrix-core GEMM instead of one GEMV pass per token.
+constexpr size_t kIqGemmMinSeq = 4;
 // Minimum tokens for which the grouped MoE GEMMs on the matrix cores are considered.
 constexpr size_t kMoeMfmaMinTokens = 16;
 // Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
@@ -230,8 +232,13 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     };
     float *ws = nullptr;
     if (is_iq_quant(quant)) {
-        // importance quants: one GEMV pass per token (grid row per token) at every batch size
-        launch_gemv_iq(w_dev, quant, act, out_dev, r, nb, q, s.stream);
+        // importance quants: the matrix-core GEMM for batches, else one GEMV pass per token (grid row per token)
+        if (seq >= kIqGemmMinSeq) {
+            if (int st = slice_floats(gemm_iq_slice_floats(r, nb, q), &ws); st != RNB_HIP_OK) return st;
+            launch_gemm_iq_mfma(w_dev, quant, act, out_dev, ws, r, nb, q, s.stream);
+        } else {
+            launch_gemv_iq(w_dev, quant, act, out_dev, r, nb, q, s.stream);
+        }
     } else if (quant == kQ4K) {
         // the GEMM fills LDS with 16-byte loads: weights at other alignments take the vector kernels
         // gemm_q4k.hip's 256-row x 64-token workgroups (K cut into slices up to 128 tiles) win from 32 tiles on when the
@@ -1665,6 +1672,9 @@ int embedding_gather(uint32_t quant, const uint8_t *w, size_t w_len, size_t rows
         HIP_TRY(hipStreamSynchronize(s.stream));
         s.d2h_bytes += out_bytes;
         std::memcpy(out_host, s.bounce_out.ptr, out_bytes);
+    } else {
+        // the ids (or rows) went through the shared pinned buffer: the next call may refill it, so the copy must be done
+        HIP_TRY(hipStreamSynchronize(s.stream));
     }
     return RNB_HIP_OK;
 }

@@ -12,8 +12,11 @@
 // every byte of an IQ3_XXS entry is 4 + 8 c, 62 for c = 7) and expanded at compile time into device tables, which every
 // workgroup copies into LDS once (the look-ups are gathers: 14336 x 4096 IQ2_XXS 13.7 -> 9.6 us, IQ3_XXS 19.6 -> 11.2 us
 // against tables read through the vector cache); a sign index of seven bits stands for those bits and their parity.
+#include <algorithm>
+
 #include "embed_gather.h"
 #include "kernels.h"
+#include "mfma_blocks.h"
 
 namespace rnb {
 
@@ -319,6 +322,267 @@ void launch_iq(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_
     hipLaunchKernelGGL((gemv_iq_kernel<kQuant>), grid, dim3(kWave * kIqWaves), 0, stream, w, act.qs, act.d, out, rows, nb);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Batches on the matrix cores: the scheme of gemm_blocks.hip's Q2_K / Q3_K kernel.  M = token, N = weight row, lane =
+// (row lane % 32, K-half lane / 32); one K=16 instruction (v_mfma_i32_32x32x16_i8) per 16 elements, i.e. two per
+// 32-element group, the lane supplying the eight signed codes of elements 16 sb + 8 khalf .. + 8: one grid entry
+// (IQ2_XXS, IQ2_S), two four-code entries (IQ3_XXS) or eight nibbles through the 16-entry table (IQ4_XS).  The group's
+// integer scale goes onto the sixteen results (tot += sc * I, 24-bit multiplies), one f32 update per block:
+//   IQ2_XXS, IQ2_S  out += (d / 8) d_x sum (2 s + 1) I      IQ3_XXS  out += (d / 4) d_x sum (2 s + 1) I
+//   IQ4_XS          out += d d_x sum (s - 32) I
+// which are the reference's sums (crates/rnb-cpu/src/gemm/neon_quant.rs:273-411) with the halves made integers.  The
+// tokens' int8 activations are staged in LDS, double-buffered, one barrier per block; the grids sit in LDS as in the
+// GEMV.  Small grids cut K into slices (blockIdx.z), summed in slice order by sum_slices_kernel.
+// ---------------------------------------------------------------------------------------------
+template <uint32_t kQuant>
+struct IqRow;
+
+template <>
+struct IqRow<kIQ2XXS> {  // 8 x {u8 index[4], u32 signs | scale << 28}
+    uint32_t w[16];
+    float d;
+    __device__ __forceinline__ void load(const uint8_t *blk, int) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint4 v = ld_u4_a2(blk + 2 + 16 * i);
+            w[4 * i] = v.x, w[4 * i + 1] = v.y, w[4 * i + 2] = v.z, w[4 * i + 3] = v.w;
+        }
+        d = ld_f16(blk) * 0.125f;
+    }
+    template <int kSb>
+    __device__ __forceinline__ long operand(int khalf, const void *tab, int *scale) const {
+        constexpr int ib = kSb >> 1;
+        const int l = 2 * (kSb & 1) + khalf;
+        const uint32_t ss = w[2 * ib + 1];
+        const uint64_t grid = static_cast<const uint64_t *>(tab)[(w[2 * ib] >> (8 * l)) & 0xffu];
+        const uint32_t sg = sign_byte(ss >> (7 * l));
+        *scale = static_cast<int>(2 * (ss >> 28) + 1);
+        return static_cast<long>(static_cast<uint64_t>(apply_signs4(static_cast<uint32_t>(grid), sg)) |
+                                 (static_cast<uint64_t>(apply_signs4(static_cast<uint32_t>(grid >> 32), sg >> 4)) << 32));
+    }
+};
+
+template <>
+struct IqRow<kIQ2S> {  // u8 index_low[32], u8 signs[32], u8 qh[8], u8 scales[8]
+    uint32_t w[20];
+    float d;
+    __device__ __forceinline__ void load(const uint8_t *blk, int) {
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            const uint4 v = ld_u4_a2(blk + 2 + 16 * i);
+            w[4 * i] = v.x, w[4 * i + 1] = v.y, w[4 * i + 2] = v.z, w[4 * i + 3] = v.w;
+        }
+        d = ld_f16(blk) * 0.125f;
+    }
+    template <int kSb>
+    __device__ __forceinline__ long operand(int khalf, const void *tab, int *scale) const {
+        constexpr int ib = kSb >> 1;
+        const int l = 2 * (kSb & 1) + khalf;
+        const uint32_t qh = (w[16 + (ib >> 2)] >> (8 * (ib & 3))) & 0xffu, sc = (w[18 + (ib >> 2)] >> (8 * (ib & 3))) & 0xffu;
+        const uint32_t index = ((w[ib] >> (8 * l)) & 0xffu) | ((qh << (8 - 2 * l)) & 0x300u);
+        const uint64_t grid = static_cast<const uint64_t *>(tab)[index];
+        const uint32_t sg = (w[8 + ib] >> (8 * l)) & 0xffu;
+        *scale = static_cast<int>(2 * ((kSb & 1) ? (sc >> 4) : (sc & 15u)) + 1);
+        return static_cast<long>(static_cast<uint64_t>(apply_signs4(static_cast<uint32_t>(grid), sg)) |
+                                 (static_cast<uint64_t>(apply_signs4(static_cast<uint32_t>(grid >> 32), sg >> 4)) << 32));
+    }
+};
+
+template <>
+struct IqRow<kIQ3XXS> {  // u8 index[64], 8 x u32 signs | scale << 28
+    uint32_t w[24];
+    float d;
+    __device__ __forceinline__ void load(const uint8_t *blk, int) {
+#pragma unroll
+        for (int i = 0; i < 6; i++) {
+            const uint4 v = ld_u4_a2(blk + 2 + 16 * i);
+            w[4 * i] = v.x, w[4 * i + 1] = v.y, w[4 * i + 2] = v.z, w[4 * i + 3] = v.w;
+        }
+        d = ld_f16(blk) * 0.25f;
+    }
+    template <int kSb>
+    __device__ __forceinline__ long operand(int khalf, const void *tab, int *scale) const {
+        constexpr int ib = kSb >> 1;
+        const int l = 2 * (kSb & 1) + khalf;
+        const uint32_t packed = w[16 + ib];
+        const uint32_t pair = (khalf ? (w[2 * ib + (kSb & 1)] >> 16) : w[2 * ib + (kSb & 1)]) & 0xffffu;  // indices 2 l, 2 l + 1
+        const uint32_t *grid = static_cast<const uint32_t *>(tab);
+        const uint32_t sg = sign_byte(packed >> (7 * l));
+        *scale = static_cast<int>(2 * (packed >> 28) + 1);
+        return static_cast<long>(static_cast<uint64_t>(apply_signs4(grid[pair & 0xffu], sg)) |
+                                 (static_cast<uint64_t>(apply_signs4(grid[pair >> 8], sg >> 4)) << 32));
+    }
+};
+
+template <>
+struct IqRow<kIQ4XS> {  // u16 scales_h, u8 scales_l[4], u8 qs[128]: byte j of a group = elements j and 16 + j
+    uint32_t w[16];  // the lane's eight bytes of every group: bytes 8 khalf .. + 8
+    uint32_t scales_h, scales_l;
+    float d;
+    __device__ __forceinline__ void load(const uint8_t *blk, int khalf) {
+        const uint2 hdr = ld_u2_a2(blk);
+#pragma unroll
+        for (int ib = 0; ib < 8; ib++) {
+            const uint2 v = ld_u2_a2(blk + 8 + 16 * ib + 8 * khalf);
+            w[2 * ib] = v.x, w[2 * ib + 1] = v.y;
+        }
+        scales_h = hdr.x >> 16;
+        scales_l = hdr.y;
+        d = f16_bits_to_f32(hdr.x);
+    }
+    template <int kSb>
+    __device__ __forceinline__ long operand(int, const void *, int *scale) const {
+        constexpr int ib = kSb >> 1, h = kSb & 1;
+        *scale = static_cast<int>(((scales_l >> (4 * ib)) & 15u) | (((scales_h >> (2 * ib)) & 3u) << 4)) - 32;
+        return static_cast<long>(static_cast<uint64_t>(iq4nl_lookup((w[2 * ib] >> (4 * h)) & 0x0f0f0f0fu)) |
+                                 (static_cast<uint64_t>(iq4nl_lookup((w[2 * ib + 1] >> (4 * h)) & 0x0f0f0f0fu)) << 32));
+    }
+};
+
+template <uint32_t kQuant, int kTT>
+__global__ void __launch_bounds__(kGbThreads, 2)
+    gemm_iq_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                        float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq, uint32_t nb_slice) {
+    constexpr int kToks = 32 * kTT;
+    constexpr size_t kBlockBytes = Iq<kQuant>::kBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kToks * kGbStride64];
+    __shared__ __attribute__((aligned(16))) float s_dx[2][kToks];
+    __shared__ __attribute__((aligned(16))) uint8_t s_table[Iq<kQuant>::kTableBytes > 0 ? Iq<kQuant>::kTableBytes : 16];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lrow = lane & 31, khalf = lane >> 5;
+    const uint32_t row = blockIdx.x * kGbRows + wave * 32 + lrow;
+    const uint32_t tok0 = blockIdx.y * kToks, last_tok = seq - 1;
+    const uint8_t *wrow = w + static_cast<size_t>(min(row, rows - 1)) * nb * kBlockBytes;
+    if constexpr (Iq<kQuant>::kTableBytes > 0) {
+        const uint4 *src = static_cast<const uint4 *>(Iq<kQuant>::table());
+        for (int i = tid; i < Iq<kQuant>::kTableBytes / 16; i += kGbThreads) reinterpret_cast<uint4 *>(s_table)[i] = src[i];
+    }
+
+    float accf[kTT][16];
+    int tot[kTT][16];
+#pragma unroll
+    for (int t = 0; t < kTT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            accf[t][i] = 0.0f;
+            tot[t][i] = 0;
+        }
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    // K slice of this workgroup (blockIdx.z): blocks b0 .. b1, its sums go to the slice's own copy of the output
+    const uint32_t b0 = blockIdx.z * nb_slice, b1 = min(nb, b0 + nb_slice);
+    out += static_cast<size_t>(blockIdx.z) * seq * rows;
+    Stage<kToks> st;
+    stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, b0, tid);
+    IqRow<kQuant> cur;
+    cur.load(wrow + static_cast<size_t>(b0) * kBlockBytes, khalf);
+    stage_store<kToks>(st, s_a[0], s_dx[0], tid);
+    __syncthreads();  // also: the table is in place
+
+    for (uint32_t b = b0; b < b1; b++) {
+        const int buf = (b - b0) & 1;
+        const uint32_t bn = b + 1 < b1 ? b + 1 : b;  // the last step reloads its own block, unused
+        stage_load<kToks>(st, aq, ad, tok0, last_tok, nb, bn, tid);
+        IqRow<kQuant> nxt;
+        nxt.load(wrow + static_cast<size_t>(bn) * kBlockBytes, khalf);
+        const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
+
+        // the empty asm and the scheduling barrier keep the sixteen sub-blocks a chain (a tree keeps 256 products alive)
+#define RNB_IQ_SUB_BLOCK(SB)                                                                                           \
+    {                                                                                                                  \
+        int sc;                                                                                                        \
+        const long bop = cur.template operand<SB>(khalf, s_table, &sc);                                                \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
+            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
+            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+                tot[t][i] += mul24(acc[i], sc); /* |I| <= 16 * 127 * 127 */                                            \
+                asm volatile("" : "+v"(tot[t][i]));                                                                    \
+            }                                                                                                          \
+        }                                                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                                             \
+    }
+        RNB_IQ_SUB_BLOCK(0)
+        RNB_IQ_SUB_BLOCK(1)
+        RNB_IQ_SUB_BLOCK(2)
+        RNB_IQ_SUB_BLOCK(3)
+        RNB_IQ_SUB_BLOCK(4)
+        RNB_IQ_SUB_BLOCK(5)
+        RNB_IQ_SUB_BLOCK(6)
+        RNB_IQ_SUB_BLOCK(7)
+        RNB_IQ_SUB_BLOCK(8)
+        RNB_IQ_SUB_BLOCK(9)
+        RNB_IQ_SUB_BLOCK(10)
+        RNB_IQ_SUB_BLOCK(11)
+        RNB_IQ_SUB_BLOCK(12)
+        RNB_IQ_SUB_BLOCK(13)
+        RNB_IQ_SUB_BLOCK(14)
+        RNB_IQ_SUB_BLOCK(15)
+#undef RNB_IQ_SUB_BLOCK
+
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
+                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = 4 * j + i;
+                    accf[t][r] += (cur.d * dx[i]) * static_cast<float>(tot[t][r]);
+                    tot[t][r] = 0;
+                }
+            }
+        stage_store<kToks>(st, s_a[buf ^ 1], s_dx[buf ^ 1], tid);
+        cur = nxt;
+        __syncthreads();
+    }
+
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < kTT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
+                if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
+            }
+    }
+}
+
+// the tiling and slicing choices, shared by the launcher and the workspace size
+struct IqGemmPlan {
+    bool wide;  // 64-token workgroups
+    uint32_t slices;
+};
+IqGemmPlan iq_gemm_plan(uint32_t rows, uint32_t nb, uint32_t seq) {
+    const uint64_t row_tiles = (rows + kGbRows - 1) / kGbRows;
+    IqGemmPlan p;
+    p.wide = seq > 32 && row_tiles * ((seq + 63) / 64) >= 512;  // the wider tile while it leaves two workgroups per compute unit
+    const uint64_t wgs = row_tiles * (p.wide ? (seq + 63) / 64 : (seq + 31) / 32);
+    p.slices = 1;
+    if (wgs <= 256) {  // K slices until the grid has about 512 workgroups; a slice keeps four blocks, two on the smallest grids
+        const uint64_t want = (512 + wgs - 1) / wgs, min_steps = wgs <= 32 ? 2 : 4;
+        p.slices = static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>({want, nb / min_steps, 16})));
+    }
+    return p;
+}
+
+template <uint32_t kQuant>
+void launch_iq_gemm(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb, uint32_t seq,
+                    hipStream_t stream) {
+    const IqGemmPlan p = iq_gemm_plan(rows, nb, seq);
+    const uint32_t slices = slice_out ? p.slices : 1;
+    const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
+    float *dst = nz > 1 ? slice_out : out;
+    const dim3 grid((rows + kGbRows - 1) / kGbRows, p.wide ? (seq + 63) / 64 : (seq + 31) / 32, nz), block(kGbThreads);
+    if (p.wide)
+        hipLaunchKernelGGL((gemm_iq_mfma_kernel<kQuant, 2>), grid, block, 0, stream, w, act.qs, act.d, dst, rows, nb, seq, nb_slice);
+    else
+        hipLaunchKernelGGL((gemm_iq_mfma_kernel<kQuant, 1>), grid, block, 0, stream, w, act.qs, act.d, dst, rows, nb, seq, nb_slice);
+    if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
+}
+
 }  // namespace
 
 bool is_iq_quant(uint32_t quant) { return quant == kIQ2XXS || quant == kIQ2S || quant == kIQ3XXS || quant == kIQ4XS; }
@@ -331,6 +595,23 @@ void launch_gemv_iq(const uint8_t *w, uint32_t quant, ActView act, float *out, u
     case kIQ2S: launch_iq<kIQ2S>(w, act, out, rows, nb, seq, stream); break;
     case kIQ3XXS: launch_iq<kIQ3XXS>(w, act, out, rows, nb, seq, stream); break;
     default: launch_iq<kIQ4XS>(w, act, out, rows, nb, seq, stream); break;
+    }
+}
+
+size_t gemm_iq_slice_floats(uint32_t rows, uint32_t nb, uint32_t seq) {
+    if (rows == 0 || nb == 0 || seq == 0) return 0;
+    const IqGemmPlan p = iq_gemm_plan(rows, nb, seq);
+    return p.slices > 1 ? static_cast<size_t>(p.slices) * seq * rows : 0;
+}
+
+void launch_gemm_iq_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                         uint32_t seq, hipStream_t stream) {
+    if (rows == 0 || seq == 0 || nb == 0) return;
+    switch (quant) {
+    case kIQ2XXS: launch_iq_gemm<kIQ2XXS>(w, act, out, slice_out, rows, nb, seq, stream); break;
+    case kIQ2S: launch_iq_gemm<kIQ2S>(w, act, out, slice_out, rows, nb, seq, stream); break;
+    case kIQ3XXS: launch_iq_gemm<kIQ3XXS>(w, act, out, slice_out, rows, nb, seq, stream); break;
+    default: launch_iq_gemm<kIQ4XS>(w, act, out, slice_out, rows, nb, seq, stream); break;
     }
 }
 

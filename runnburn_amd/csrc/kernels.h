@@ -57,6 +57,11 @@ void launch_embed_gather(uint32_t quant, const uint8_t *w, size_t row_bytes, con
                          uint32_t cols, float *out, hipStream_t stream);
 void launch_embed_gather_iq(uint32_t quant, const uint8_t *w, size_t row_bytes, const uint32_t *ids, uint32_t n_tokens,
                             uint32_t cols, float *out, hipStream_t stream);
+// the same formats for batches, on the matrix cores; slice_out: workspace of gemm_iq_slice_floats(rows, nb, seq) floats (or
+// null: no K slices)
+size_t gemm_iq_slice_floats(uint32_t rows, uint32_t nb, uint32_t seq);
+void launch_gemm_iq_mfma(const uint8_t *w, uint32_t quant, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
+                         uint32_t seq, hipStream_t stream);
 // Q2_K / Q3_K rows (84 / 110-byte blocks at 4- / 2-byte alignment); quant is kQ2K or kQ3K
 void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
                          uint32_t seq, hipStream_t stream);

@@ -39,8 +39,9 @@ def test_iq_gemv_against_oracle(rnb, oracle, quant, rows, cols):
 @pytest.mark.parametrize("quant", [IQ2_XXS, IQ2_S, IQ3_XXS, IQ4_XS])
 @pytest.mark.parametrize("seq", [2, 5, 33])
 def test_iq_gemv_batch_layout(rnb, oracle, quant, seq):
-    """Batch form: out[s * rows + r] (crates/rnb-cpu/src/gemm/quant_gemv.rs:1185-1196), and every token's row equals the
-    one-token call bit for bit (same kernel, one grid row per token)."""
+    """Batch form: out[s * rows + r] (crates/rnb-cpu/src/gemm/quant_gemv.rs:1185-1196).  Below four tokens every token's
+    row equals the one-token call bit for bit (same kernel, one grid row per token); from four on the batch runs on the
+    matrix cores (integer group sums, one f32 update per block) and agrees to rounding."""
     rows, cols = 203, 1024
     w = oracle.make_weights(quant, rows, cols, 800 + quant)
     x = oracle.fill_normal(seq * cols, 900 + seq, 1.0)
@@ -48,8 +49,43 @@ def test_iq_gemv_batch_layout(rnb, oracle, quant, seq):
     got = batch(w, rows, cols, x).reshape(seq, rows)
     _check(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True), f"{LABEL[quant]} batch {seq}")
     for s in (0, seq - 1):
-        assert np.array_equal(got[s], one(w, rows, cols, x[s * cols:(s + 1) * cols]))
+        alone = one(w, rows, cols, x[s * cols:(s + 1) * cols])
+        if seq < 4:
+            assert np.array_equal(got[s], alone)
+        else:
+            assert np.abs(got[s] - alone).max() <= 1e-5 * np.abs(alone).max()
     rnb.release(w)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quant", [IQ2_XXS, IQ2_S, IQ3_XXS, IQ4_XS])
+@pytest.mark.parametrize("rows,cols,seq", [(203, 1024, 4), (130, 256, 33), (129, 4096, 65), (4096, 2048, 96), (37, 14336, 17),
+                                           (300, 768, 512), (8192, 512, 500)])
+def test_iq_gemm_matrix_cores(rnb, oracle, quant, rows, cols, seq):
+    """Batches of four tokens and more: ragged row and token tiles, 32- and 64-token workgroups (8192 rows x 500 tokens),
+    K cut into slices on small grids (37 rows x 56 blocks: sixteen slices)."""
+    w = oracle.make_weights(quant, rows, cols, 1200 + quant + rows)
+    x = oracle.fill_normal(seq * cols, 1300 + seq, 1.0)
+    got = _fns(rnb, quant)[1](w, rows, cols, x).reshape(seq, rows)
+    _check(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+           f"{LABEL[quant]} gemm {rows}x{cols}x{seq}")
+    rnb.release(w)
+
+
+@pytest.mark.gpu
+def test_iq_gemm_every_code_and_scale(rnb, oracle):
+    """Blocks of random bytes (every grid index, sign pattern and scale value) with a finite d, eight tokens."""
+    rng = np.random.default_rng(99)
+    bb = {IQ2_XXS: 66, IQ2_S: 82, IQ3_XXS: 98, IQ4_XS: 136}
+    for quant in (IQ2_XXS, IQ2_S, IQ3_XXS, IQ4_XS):
+        rows, cols, seq = 160, 1024, 8
+        w = rng.integers(0, 256, size=(rows * cols // 256, bb[quant]), dtype=np.uint8)
+        w[:, 0:2] = (rng.standard_normal((w.shape[0], 1)) * 0.05).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        w = w.reshape(-1)
+        x = oracle.fill_normal(seq * cols, 77 + quant, 1.0)
+        got = _fns(rnb, quant)[1](w, rows, cols, x).reshape(seq, rows)
+        _check(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True), f"{LABEL[quant]} random codes")
+        rnb.release(w)
 
 
 @pytest.mark.gpu
