@@ -182,26 +182,48 @@ __device__ __forceinline__ Q6KAct q6k_load_act(const int8_t *__restrict__ aq_blk
     return a;
 }
 
+// A lane's share of a block as loaded.  Every other 210-byte block starts 2 bytes off a 4-byte boundary, and 16-byte
+// loads from such addresses are slow (forcing them onto 4-byte boundaries, wrong data: 4096 x 14336 11.3 -> 10.6 us,
+// 14336 x 4096 11.2 -> 10.3, 128256 x 4096 71.6 -> 67.8).  So every piece is fetched from the boundary below it (m = 0 or
+// 2 bytes early) and lacks its last m bytes, which are the first bytes of the piece that follows it in the block; that
+// piece is in a register of a lane of the same quad (the four lanes of a block hold its twelve 16-byte pieces and the
+// scales, in memory order A00 A01 B00 B01 A10 A11 B10 B11 H00 H01 H10 H11 S0 S1), and q6k_prepare puts the pieces right
+// with six quad-permute moves, five selects and fourteen funnel shifts: no load more than before, and none waited for
+// before the block is used.  The dword at byte 206 carries the scales' last two bytes and d.  (Fetching one dword more per
+// piece instead, nine loads for five, was slower than the misaligned loads everywhere.)
 struct Q6KRegs {
-    uint4 A, B, H;
+    uint4 A, B, H;  // as fetched: m bytes early
     uint2 S;
-    uint32_t d_bits;
+    uint32_t t;     // bytes 206..209 of the block
+    uint32_t sh;    // 8 m: the funnel shift that puts the pieces right
 };
 
-// Every other 210-byte block starts 2 bytes off a 4-byte boundary.  Fetching the pieces from the boundary below them
-// with one dword more and funnel-shifting them into place (nine dword-aligned loads instead of five) was measured
-// slower in every kernel (4096 x 14336: 11.3 -> 15.5 us, 14336 x 4096: 11.2 -> 12.0 us, 128256 x 4096: 78 -> 83 us): the
-// number of load instructions counts for more than their alignment here, unlike the 32-element formats, whose pairs
-// need fewer loads when aligned (gemv.hip::block32_load_pair).
 __device__ __forceinline__ Q6KRegs q6k_load_block(const uint8_t *__restrict__ blk, int q) {
     Q6KRegs r;
     const int n = q >> 1, th = q & 1;
-    r.A = ld_u4_a2(blk + 64 * n + 16 * th);
-    r.B = ld_u4_a2(blk + 64 * n + 32 + 16 * th);
-    r.H = ld_u4_a2(blk + 128 + 32 * n + 16 * th);
-    r.S = ld_u2_a2(blk + 192 + 8 * n);
-    r.d_bits = *reinterpret_cast<const unsigned short *>(blk + 208);
+    uint32_t m = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(blk)) & 3u;
+    if (m & 1u) {  // a matrix at an odd address (the same for every lane): the pieces themselves, whatever it costs
+        r.A = ld_u4_a2(blk + 64 * n + 16 * th);
+        r.B = ld_u4_a2(blk + 64 * n + 32 + 16 * th);
+        r.H = ld_u4_a2(blk + 128 + 32 * n + 16 * th);
+        r.S = ld_u2_a2(blk + 192 + 8 * n);
+        m = 0;
+    } else {
+        const uint8_t *base = blk - m;
+        r.A = *reinterpret_cast<const uint4_a4 *>(base + 64 * n + 16 * th);
+        r.B = *reinterpret_cast<const uint4_a4 *>(base + 64 * n + 32 + 16 * th);
+        r.H = *reinterpret_cast<const uint4_a4 *>(base + 128 + 32 * n + 16 * th);
+        r.S = *reinterpret_cast<const uint2_a4 *>(base + 192 + 8 * n);
+    }
+    r.t = ld_u32_a2(blk + 206);
+    r.sh = 8 * m;
     return r;
+}
+
+template <int kL0, int kL1, int kL2, int kL3>
+__device__ __forceinline__ uint32_t quad_take(uint32_t v) {  // lane i of a quad reads lane kLi's v
+    return static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(v), kL0 | (kL1 << 2) | (kL2 << 4) | (kL3 << 6), 0xf, 0xf, false));
 }
 
 __device__ __forceinline__ int sext8(uint32_t v, int shift) {
@@ -214,14 +236,36 @@ struct Q6KPrep {
     float d;
 };
 
-__device__ __forceinline__ Q6KPrep q6k_prepare(const Q6KRegs &r, int q) {
+// All four lanes of a quad must be active (they exchange the pieces' first dwords).
+__device__ __forceinline__ Q6KPrep q6k_prepare(const Q6KRegs &raw, int q) {
     Q6KPrep p;
+    // the first dword of the piece after each of this lane's pieces, then the pieces moved into place
+    const int n = q >> 1, th = q & 1;
+    const uint32_t a1 = quad_take<1, 0, 3, 2>(raw.A.x), b1 = quad_take<1, 0, 3, 2>(raw.B.x);
+    const uint32_t ar = quad_take<1, 2, 3, 0>(raw.A.x), hr = quad_take<1, 2, 3, 0>(raw.H.x), sr = quad_take<1, 2, 3, 0>(raw.S.x);
+    const uint32_t s2 = quad_take<2, 3, 0, 1>(raw.S.x);
+    const uint32_t after_a = th ? b1 : a1;
+    const uint32_t after_b = th ? (n ? hr : ar) : b1;
+    const uint32_t after_h = q == 3 ? sr : hr;
+    const uint32_t after_s = n ? raw.t : s2;
+    const uint32_t sh = raw.sh;
+    struct {
+        uint4 A, B, H;
+        uint2 S;
+    } r;
+    r.A = make_uint4(__builtin_amdgcn_alignbit(raw.A.y, raw.A.x, sh), __builtin_amdgcn_alignbit(raw.A.z, raw.A.y, sh),
+                     __builtin_amdgcn_alignbit(raw.A.w, raw.A.z, sh), __builtin_amdgcn_alignbit(after_a, raw.A.w, sh));
+    r.B = make_uint4(__builtin_amdgcn_alignbit(raw.B.y, raw.B.x, sh), __builtin_amdgcn_alignbit(raw.B.z, raw.B.y, sh),
+                     __builtin_amdgcn_alignbit(raw.B.w, raw.B.z, sh), __builtin_amdgcn_alignbit(after_b, raw.B.w, sh));
+    r.H = make_uint4(__builtin_amdgcn_alignbit(raw.H.y, raw.H.x, sh), __builtin_amdgcn_alignbit(raw.H.z, raw.H.y, sh),
+                     __builtin_amdgcn_alignbit(raw.H.w, raw.H.z, sh), __builtin_amdgcn_alignbit(after_h, raw.H.w, sh));
+    r.S = make_uint2(__builtin_amdgcn_alignbit(raw.S.y, raw.S.x, sh), __builtin_amdgcn_alignbit(after_s, raw.S.y, sh));
     const int is = (q & 1) * 8;  // l / 16 selects scale byte 0 or 1 of each pair
     p.s0 = sext8(r.S.x, is);
     p.s1 = sext8(r.S.x, is + 16);
     p.s2 = sext8(r.S.y, is);
     p.s3 = sext8(r.S.y, is + 16);
-    p.d = f16_bits_to_f32(r.d_bits);
+    p.d = f16_bits_to_f32(raw.t >> 16);
 #define RNB_Q6_UNPACK(k)                                                          \
     p.u0.k = (r.A.k & 0x0f0f0f0fu) | ((r.H.k & 0x03030303u) << 4);                \
     p.u1.k = (r.B.k & 0x0f0f0f0fu) | ((r.H.k & 0x0c0c0c0cu) << 2);                \
