@@ -485,7 +485,14 @@ __global__ void __launch_bounds__(256) act_mul_kernel(const float *__restrict__ 
 constexpr int kSplitRows = 1;  // rows per workgroup and step: 1 / 2 / 4 / 8 measured 11.6 / 12.8 / 13.5 / 33 us on 4096 x 14336 Q6_K
 constexpr uint32_t kSplitMaxWaves = 16;  // rows of up to 256 super-blocks
 
-template <uint32_t kQuant>
+// kDefer: the waves do not meet after every row; the partial sums of up to kSplitBatch of the workgroup's rows wait in
+// LDS for one barrier (same additions in the same order, so the same bits).  It pays for two and four waves per workgroup
+// (4096 x 14336 Q6_K 11.4 -> 10.7 us, 5120 x 13824 13.4 -> 12.4, 16384 x 6144 18.2 -> 17.0, Q4_K 4096 x 14336 8.4 -> 8.1)
+// and costs for three, five and seven (4096 x 11008 9.8 -> 10.1, 4096 x 20480 16.2 -> 17.2, 8192 x 28672 39.4 -> 41.9):
+// the launcher chooses.  One row requested ahead on top of it is slower again (10.7 -> 12.7 us).
+constexpr int kSplitBatch = 8;
+
+template <uint32_t kQuant, bool kDefer>
 __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     gemv_kquant_splitk_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                               const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
@@ -493,7 +500,7 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     using Q = KQuant<kQuant>;
     using Regs = typename Q::Regs;
     constexpr size_t kBlockBytes = Q::kBytes;
-    __shared__ float s_part[2][kSplitRows][kSplitMaxWaves];
+    __shared__ float s_part[kDefer ? kSplitBatch : 2][kSplitRows][kSplitMaxWaves];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = threadIdx.x >> 6, n_slices = blockDim.x >> 6;
     const int g = lane & 3;
@@ -503,6 +510,27 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? b : 0);
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
     const typename Q::Act a = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    if constexpr (kDefer) {
+        static_assert(kSplitRows == 1, "one row per step");
+        for (uint32_t chunk0 = blockIdx.x; chunk0 < row_chunks; chunk0 += kSplitBatch * gridDim.x) {
+            uint32_t n = 0;
+            for (uint32_t chunk = chunk0; chunk < row_chunks && n < kSplitBatch; chunk += gridDim.x, n++) {
+                Regs r = Regs{};  // idle lanes keep zeros
+                if (has_block) r = Q::load_block(w + static_cast<size_t>(chunk) * row_bytes + static_cast<size_t>(b) * kBlockBytes, g);
+                float acc = kquant_partial<kQuant>(r, a, g);
+                acc = seg_sum<kWave>(has_block ? acc : 0.0f);
+                if (lane == kWave - 1) s_part[n][0][wave] = acc;
+            }
+            __syncthreads();
+            if (threadIdx.x < n) {
+                float sum = 0.0f;
+                for (uint32_t j = 0; j < n_slices; j++) sum += s_part[threadIdx.x][0][j];
+                out[static_cast<size_t>(tok) * rows + chunk0 + threadIdx.x * gridDim.x] = sum;
+            }
+            __syncthreads();  // the sums are read before the next batch overwrites them
+        }
+        return;
+    }
     uint32_t parity = 0;
     for (uint32_t chunk = blockIdx.x; chunk < row_chunks; chunk += gridDim.x, parity ^= 1) {
         const uint32_t row0 = chunk * kSplitRows;
@@ -537,8 +565,12 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
     const uint32_t row_chunks = (rows + kSplitRows - 1) / kSplitRows;
     const uint32_t want = kTargetWaves / n_slices;  // workgroups for about kTargetWaves waves
     const dim3 grid(row_chunks < want ? row_chunks : want, seq, 1);
-    hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
-                       act.bsums, out, rows, nb, row_chunks);
+    if (n_slices == 2 || n_slices == 4)
+        hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant, true>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
+                           act.bsums, out, rows, nb, row_chunks);
+    else
+        hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant, false>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
+                           act.bsums, out, rows, nb, row_chunks);
 }
 
 template <uint32_t kQuant, int kRowsPerWave>
