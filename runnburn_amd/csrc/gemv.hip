@@ -573,6 +573,110 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
                            act.bsums, out, rows, nb, row_chunks);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Split-K GEMV of ONE f32 token in one launch, rows of 17 to 32 super-blocks: a workgroup of 16 waves quantises the whole
+// token to Q8_K in its LDS (two blocks per wave, the wave-level quantiser of the stand-alone kernel, so the same bits),
+// then works as `teams` split-K teams of n_slices waves, each team on rows of its own; the partial sums of up to
+// kSplitBatch rows per team wait for one barrier and are added in slice order, as in gemv_kquant_splitk_kernel (the same
+// bits).  The teams of a launch are as many as the split-K kernel has workgroups, so the weight stream looks the same;
+// the token is read once per 16 waves, and the quantiser's launch and the gap behind it go: 8192 x 8192 Q4_K 10.9 ->
+// 9.9 us per step, 13824 x 5120 12.3 -> 11.2, 28672 x 8192 25.7 -> 24.8, 2048 x 8192 7.1 -> 5.5.  The kernel is written for
+// any number of slices up to 16 waves' worth, but with three and four slices (rows of up to 64 super-blocks, four blocks
+// to quantise per wave) it loses to the two launches (4096 x 14336 Q6_K 13.2 vs 12.9 us, 4096 x 11008 16.0 vs 12.0),
+// and with four rows per team requested before the quantisation instead of one it loses more (17.7 us).
+// ---------------------------------------------------------------------------------------------
+constexpr int kWideWaves = 16;
+constexpr uint32_t kWideMaxBlocks = 32;
+constexpr int kWidePre = 1;  // rows per team requested before the token is quantised (at most kSplitBatch)
+template <uint32_t kQuant>
+__global__ void __launch_bounds__(kWave *kWideWaves)
+    gemv_kquant_wide_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
+                                uint32_t rows, uint32_t nb, uint32_t n_slices, uint32_t teams) {
+    using Q = KQuant<kQuant>;
+    using Regs = typename Q::Regs;
+    constexpr size_t kBlockBytes = Q::kBytes;
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[kWideMaxBlocks * 256];
+    __shared__ float s_d[kWideMaxBlocks];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[kWideMaxBlocks * 16];
+    __shared__ float s_part[kSplitBatch][kWideWaves];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t team = wave / n_slices, slice = wave - team * n_slices;
+    const int g = lane & 3;
+    const uint32_t b = slice * 16 + (lane >> 2);
+    const bool has_block = team < teams && b < nb;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t stride = gridDim.x * teams;          // rows per pass of the whole launch
+    const uint32_t first = blockIdx.x * teams;          // this workgroup's first row of pass 0
+    const uint32_t n_pass = (rows + stride - 1) / stride;
+    // the token is requested first: loads return in order, and the quantiser must not wait for weights
+    float4 xv[kWideMaxBlocks / kWideWaves];
+#pragma unroll
+    for (int i = 0; i < static_cast<int>(kWideMaxBlocks) / kWideWaves; i++) {
+        const uint32_t blk = wave + i * kWideWaves;
+        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 256)[lane];
+    }
+    auto fetch = [&](uint32_t pass) {
+        const uint32_t row = pass * stride + first + team;
+        Regs r = Regs{};  // idle lanes and rows past the end keep zeros
+        if (has_block && row < rows) r = Q::load_block(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes, g);
+        return r;
+    };
+    Regs pre[kWidePre];  // the first passes' rows: in flight while the token is quantised
+#pragma unroll
+    for (int i = 0; i < kWidePre; i++) pre[i] = fetch(i);
+#pragma unroll
+    for (int i = 0; i < static_cast<int>(kWideMaxBlocks) / kWideWaves; i++) {
+        const uint32_t blk = wave + i * kWideWaves;
+        if (blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+    }
+    __syncthreads();
+    const uint32_t ab = has_block ? b : 0;
+    const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
+    for (uint32_t p0 = 0; p0 < n_pass; p0 += kSplitBatch) {
+        const uint32_t n = n_pass - p0 < static_cast<uint32_t>(kSplitBatch) ? n_pass - p0 : kSplitBatch;
+        if (p0 == 0) {
+#pragma unroll
+            for (int k = 0; k < kWidePre; k++) {
+                if (static_cast<uint32_t>(k) < n) {
+                    float acc = kquant_partial<kQuant>(pre[k], a, g);
+                    acc = seg_sum<kWave>(has_block ? acc : 0.0f);
+                    if (lane == kWave - 1) s_part[k][wave] = acc;
+                }
+            }
+        }
+        for (uint32_t k = p0 == 0 ? kWidePre : 0; k < n; k++) {
+            const Regs r = fetch(p0 + k);
+            float acc = kquant_partial<kQuant>(r, a, g);
+            acc = seg_sum<kWave>(has_block ? acc : 0.0f);
+            if (lane == kWave - 1) s_part[k][wave] = acc;
+        }
+        __syncthreads();
+        if (threadIdx.x < n * teams) {
+            const uint32_t k = threadIdx.x / teams, tm = threadIdx.x - k * teams;
+            const uint32_t row = (p0 + k) * stride + first + tm;
+            if (row < rows) {
+                float sum = 0.0f;
+                for (uint32_t j = 0; j < n_slices; j++) sum += s_part[k][tm * n_slices + j];
+                out[row] = sum;
+            }
+        }
+        __syncthreads();  // the sums are read before the next batch overwrites them
+    }
+}
+
+template <uint32_t kQuant>
+void launch_kquant_wide_f32(const uint8_t *w, const float *x, float *out, uint32_t rows, uint32_t nb, hipStream_t stream) {
+    const uint32_t n_slices = (nb + 15) / 16;
+    const uint32_t teams = kWideWaves / n_slices;
+    // one workgroup of sixteen waves per compute unit's share of kTargetWaves
+    const uint32_t want = kTargetWaves / kWideWaves;
+    const uint32_t all = (rows + teams - 1) / teams;
+    hipLaunchKernelGGL((gemv_kquant_wide_f32_kernel<kQuant>), dim3(all < want ? all : want), dim3(kWave * kWideWaves), 0, stream,
+                       w, x, out, rows, nb, n_slices, teams);
+}
+
 template <uint32_t kQuant, int kRowsPerWave>
 void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                    hipStream_t stream) {
@@ -990,7 +1094,7 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
 
 bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
     const bool kq = quant == kQ2K || quant == kQ3K || quant == kQ4K || quant == kQ5K || quant == kQ6K;
-    return kq && nb >= 1 && nb <= 16 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    return kq && nb >= 1 && nb <= kWideMaxBlocks && reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
 bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
@@ -1014,6 +1118,20 @@ bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
                             uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
+    if (nb > 16) {  // rows of 17 to 32 super-blocks: one token per launch
+        for (uint32_t t = 0; t < seq; t++) {
+            const float *xt = x + static_cast<size_t>(t) * nb * 256;
+            float *ot = out + static_cast<size_t>(t) * rows;
+            switch (quant) {
+            case kQ2K: launch_kquant_wide_f32<kQ2K>(w, xt, ot, rows, nb, stream); break;
+            case kQ3K: launch_kquant_wide_f32<kQ3K>(w, xt, ot, rows, nb, stream); break;
+            case kQ4K: launch_kquant_wide_f32<kQ4K>(w, xt, ot, rows, nb, stream); break;
+            case kQ5K: launch_kquant_wide_f32<kQ5K>(w, xt, ot, rows, nb, stream); break;
+            default: launch_kquant_wide_f32<kQ6K>(w, xt, ot, rows, nb, stream); break;
+            }
+        }
+        return;
+    }
     switch (quant) {
     case kQ2K: launch_kquant_f32_any<kQ2K>(w, x, out, rows, nb, seq, stream); break;
     case kQ3K: launch_kquant_f32_any<kQ3K>(w, x, out, rows, nb, seq, stream); break;

@@ -70,14 +70,15 @@ void launch_gemv_q2k_q3k(const uint8_t *w, uint32_t quant, ActView act, float *o
 bool gemv_block32_f32_supported(uint32_t rows, uint32_t nb32, const void *x);  // false below the size where it pays
 void launch_gemv_block32_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb32,
                              uint32_t seq, hipStream_t stream);
-// the f32-token forms of launch_gemv_q4k_gate_up and launch_gemv_q4k_multi (same limits as gemv_kquant_f32_supported:
-// rows of at most 16 super-blocks, x 16-byte aligned; weights 16-byte aligned as for the quantised forms)
+// the f32-token forms of launch_gemv_q4k_gate_up and launch_gemv_q4k_multi (rows of at most 16 super-blocks, x 16-byte
+// aligned; weights 16-byte aligned as for the quantised forms)
 void launch_gemv_q4k_gate_up_f32(const uint8_t *wg, const uint8_t *wu, const float *x, float *mid, uint32_t rows,
                                  uint32_t nb, uint32_t seq, bool gelu, hipStream_t stream);
 void launch_gemv_q4k_multi_f32(const uint8_t *const w[3], const uint32_t rows[3], const float *x, float *out, uint32_t nb,
                                hipStream_t stream);
-// K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 16
-// super-blocks, x 16-byte aligned; same output contract as launch_gemv_q4k
+// K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 32
+// super-blocks (beyond 16 a workgroup of sixteen waves works as eight split-K teams of two waves), x 16-byte aligned; same output
+// contract and the same bits as launch_gemv_q4k on the stand-alone quantiser's output
 bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x);
 // false for matrices so large that quantising with a launch of its own and running the chunked GEMV is faster
 bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb);
