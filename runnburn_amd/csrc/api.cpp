@@ -570,20 +570,32 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                 size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
                 const float *x_dev, float *out_dev) {
     if (token_count == 0) return RNB_HIP_OK;
-    if (token_count == 1 && moe_decode_supported(n_slots, sh.nb_in, sh.nb_mid, x_dev)) {
-        // decode: no host-side tables, two launches
-        MoeDecodeTable table;
+    if (token_count <= kMoeDecodeMaxTokens && n_slots <= kMoeDecodeMaxSlots) {
+        // decode and small batches: no host-side sort by expert and no table image, two launches
+        MoeDecodeTable table = {};
         table.n_slots = static_cast<uint32_t>(n_slots);
-        for (size_t i = 0; i < kMoeDecodeMaxSlots; i++) {
-            table.expert[i] = i < n_slots ? expert_ids[i] : 0;
-            table.route[i] = i < n_slots ? route[i] : 0.0f;
+        table.n_tokens = static_cast<uint32_t>(token_count);
+        size_t max_per_token = 0;
+        for (size_t i = 0; i < n_slots; i++) table.tok_off[token_ids[i] + 1]++;  // token ids are validated
+        for (size_t t = 0; t < token_count; t++) {
+            max_per_token = std::max<size_t>(max_per_token, table.tok_off[t + 1]);
+            table.tok_off[t + 1] += table.tok_off[t];
         }
-        RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
-        launch_moe_decode(gate_dev, up_dev, down_dev, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
-                          static_cast<uint32_t>(n_ff), static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_in),
-                          static_cast<uint32_t>(sh.nb_mid), s.stream);
-        if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
-        return RNB_HIP_OK;
+        if (moe_decode_supported(token_count, n_slots, max_per_token, sh.nb_in, sh.nb_mid, x_dev)) {
+            uint32_t fill[kMoeDecodeMaxTokens] = {};
+            for (size_t i = 0; i < n_slots; i++) {  // token by token, list order kept inside a token
+                const uint32_t t = token_ids[i], at = table.tok_off[t] + fill[t]++;
+                table.expert[at] = expert_ids[i];
+                table.route[at] = route[i];
+                table.token[at] = t;
+            }
+            RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
+            launch_moe_decode(gate_dev, up_dev, down_dev, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
+                              static_cast<uint32_t>(n_ff), static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_in),
+                              static_cast<uint32_t>(sh.nb_mid), s.stream);
+            if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
+            return RNB_HIP_OK;
+        }
     }
     // slots are grouped by expert, keeping slot order inside a group
     std::vector<uint32_t> order(n_slots);

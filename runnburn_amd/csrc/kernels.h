@@ -181,15 +181,20 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const fl
 void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
                            const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
                            uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
-// One token, at most 16 slots: the whole expert step in two launches, the routing table as a kernel argument (x f32
-// [n_embd] 16-byte aligned, mid scratch [n_slots][n_ff], out [n_embd]); the same bits as the general sequence
-constexpr uint32_t kMoeDecodeMaxSlots = 16;
+// A few tokens (decode and small batches: at most 8 tokens and 64 slots, at most 16 slots per token): the whole expert
+// step in two launches, the routing table as a kernel argument.  Slots are listed token by token, in list order inside a
+// token (tok_off[t] .. tok_off[t + 1]); x f32 [n_tokens][n_embd] 16-byte aligned, mid scratch [n_slots][n_ff], out
+// [n_tokens][n_embd]; the same bits as the general sequence
+constexpr uint32_t kMoeDecodeMaxSlots = 64, kMoeDecodeMaxTokens = 8, kMoeDecodeMaxPerToken = 16;
 struct MoeDecodeTable {
-    uint32_t n_slots;
+    uint32_t n_slots, n_tokens;
     uint32_t expert[kMoeDecodeMaxSlots];
     float route[kMoeDecodeMaxSlots];
+    uint32_t token[kMoeDecodeMaxSlots];
+    uint32_t tok_off[kMoeDecodeMaxTokens + 1];
 };
-bool moe_decode_supported(size_t n_slots, size_t nb_in, size_t nb_mid, const void *x);
+// max_per_token: the largest number of slots any one token has
+bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x);
 void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
                        const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
                        uint32_t nb_in, uint32_t nb_mid, hipStream_t stream);

@@ -323,12 +323,15 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
-// One token (decode): two launches for the whole expert step, the routing table riding in the kernel arguments.
-//   moe_decode_gate_up_kernel   grid (row groups / 8, slots): the workgroup quantises the token to Q8_K in LDS (as
+// A few tokens (decode, small batches): two launches for the whole expert step, the routing table riding in the kernel
+// arguments, slots listed token by token.
+//   moe_decode_gate_up_kernel   grid (row groups / 8, slots): the workgroup quantises its slot's token to Q8_K in LDS (as
 //                               gemv_kquant_f32_kernel does), every wave makes one group of rows of its slot's expert
-//   moe_decode_down_kernel      the workgroup quantises the slots' intermediates (n_slots * nb_mid <= 64 blocks) in
-//                               LDS, then moe_down_token_kernel's row scheme: down, route weight, ordered sum
-// Same quantiser, dots and order of additions as the general path, so the same bits.
+//   moe_decode_down_kernel      grid (rows / 8, tokens): the workgroup quantises its token's slots' intermediates
+//                               (slots * nb_mid <= 64 blocks) in LDS, then moe_down_token_kernel's row scheme: down,
+//                               route weight, ordered sum
+// Same quantiser, dots and order of additions as the general path, so the same bits.  An expert that several tokens
+// chose is read once per slot here (the second time mostly from the L2), which is what bounds the batch this pays for.
 // ---------------------------------------------------------------------------------------------
 constexpr int kDecodeWaves = 8;
 
@@ -352,7 +355,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     const bool live = bslot < nb && row < n_ff;
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
     TokenSpans<kDecodeWaves> xv;
-    token_load<kDecodeWaves>(x, nb, wave, lane, xv);
+    token_load<kDecodeWaves>(x + static_cast<size_t>(table.token[slot]) * nb * 256, nb, wave, lane, xv);
     // dead lanes read the expert's first block
     const size_t off = static_cast<size_t>(table.expert[slot]) * n_ff * row_bytes +
                        (live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0);
@@ -390,7 +393,9 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     const uint32_t grp = lane / kLanes;
     const int g = sub & 3;
     const uint32_t b = sub >> 2;
-    const uint32_t n_slots = table.n_slots, n_blocks = n_slots * nb;
+    const uint32_t tok = blockIdx.y;
+    const uint32_t first = table.tok_off[tok], n_slots = table.tok_off[tok + 1] - first, n_blocks = n_slots * nb;
+    mid += static_cast<size_t>(first) * nb * 256;  // this token's slots: k below counts from `first`
     const bool lane_ok = b < nb && row < n_embd;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
     // the intermediates first, then the weights of the first kGroups slots, then the quantisation
@@ -403,7 +408,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     }
     auto fetch = [&](uint32_t k, bool *ok) {
         *ok = lane_ok && k < n_slots;
-        const size_t off = *ok ? (static_cast<size_t>(table.expert[k]) * n_embd + row) * row_bytes + static_cast<size_t>(b) * kBlockBytes
+        const size_t off = *ok ? (static_cast<size_t>(table.expert[first + k]) * n_embd + row) * row_bytes + static_cast<size_t>(b) * kBlockBytes
                                : 0;  // dead lanes read the first block of the tensor
         return Q::load_block(down_all + off, g);
     };
@@ -426,7 +431,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
             o = kquant_partial<kQuant>(cur, Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g), g);
         }
         o = seg_sum<kLanes>(o);
-        if (k < n_slots) o *= table.route[k];  // fanout.rs:306-308; only the group's last lane is read below
+        if (k < n_slots) o *= table.route[first + k];  // fanout.rs:306-308; only the group's last lane is read below
 #pragma unroll
         for (int j = 0; j < kGroups; j++) {
             const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
@@ -435,7 +440,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
         cur = nxt;
         cur_ok = nxt_ok;
     }
-    if (lane == 0 && row < n_embd) out[row] = acc;
+    if (lane == 0 && row < n_embd) out[static_cast<size_t>(tok) * n_embd + row] = acc;
 }
 
 // out[token] = sum of its slots' rows in list (= rank) order.  A thread owns four consecutive columns (n_embd is a
@@ -585,9 +590,10 @@ void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView
 #undef RNB_LAUNCH_DT
 }
 
-bool moe_decode_supported(size_t n_slots, size_t nb_in, size_t nb_mid, const void *x) {
-    return n_slots >= 1 && n_slots <= kMoeDecodeMaxSlots && nb_in >= 1 && nb_in <= 16 && nb_mid >= 1 && nb_mid <= 16 &&
-           n_slots * nb_mid <= 64 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x) {
+    return n_tokens >= 1 && n_tokens <= kMoeDecodeMaxTokens && n_slots >= 1 && n_slots <= kMoeDecodeMaxSlots &&
+           max_per_token <= kMoeDecodeMaxPerToken && nb_in >= 1 && nb_in <= 16 && nb_mid >= 1 && nb_mid <= 16 &&
+           max_per_token * nb_mid <= 64 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
 void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
@@ -603,7 +609,7 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
         RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU);
 #undef RNB_LAUNCH_DGU
     }
-    const dim3 grid((n_embd + kDecodeWaves - 1) / kDecodeWaves, 1, 1);
+    const dim3 grid((n_embd + kDecodeWaves - 1) / kDecodeWaves, table.n_tokens, 1);
 #define RNB_LAUNCH_DD(Q, G) \
     hipLaunchKernelGGL((moe_decode_down_kernel<Q, G>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
     RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD);

@@ -714,9 +714,9 @@ def test_moe_small(rnb, oracle, tokens, down_quant):
                                                      (512, 256, 5, Q5_K)])
 def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant):
     """One token takes the two-launch decode path (token and intermediates quantised inside the kernels, routing table
-    in the kernel arguments) when it has at most 16 slots and 64 intermediate blocks; otherwise, and for batches, the
-    general sequence.  Same arithmetic: the token alone equals its row in a two-token batch bit for bit, with an
-    expert repeated in the slot list, and both agree with the oracle."""
+    in the kernel arguments) when it has at most 16 slots and 64 intermediate blocks; otherwise, and for batches of more
+    than eight tokens, the general sequence.  Same arithmetic: the token alone equals its row in a nine-token batch bit
+    for bit, with an expert repeated in the slot list, and both agree with the oracle."""
     n_expert = 20
     gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, 1, k, 77 + k, down_quant)
     if k >= 3:
@@ -724,12 +724,45 @@ def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant
     got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, 1, down_quant, n_ff, n_embd, x)
     ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, 1, down_quant, n_ff, n_embd, x)
     check_close(got, ref, None, f"moe decode n_ff {n_ff} n_embd {n_embd} k {k}")
-    x2 = np.concatenate([oracle.fill_normal(n_embd, 5, 1.0), x])
+    x9 = np.concatenate([oracle.fill_normal(8 * n_embd, 5, 1.0), x])
     m = min(2, e.size)
-    e2, r2 = np.concatenate([e[:m], e]), np.concatenate([r[:m], r])
-    t2 = np.concatenate([np.zeros(m, np.uint32), np.ones(e.size, np.uint32)])
-    both = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e2, r2, t2, 2, down_quant, n_ff, n_embd, x2)
-    assert np.array_equal(both[1], got[0])
+    e9, r9 = np.concatenate([np.tile(e[:m], 8), e]), np.concatenate([np.tile(r[:m], 8), r])
+    t9 = np.concatenate([np.repeat(np.arange(8, dtype=np.uint32), m), np.full(e.size, 8, np.uint32)])
+    batch = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e9, r9, t9, 9, down_quant, n_ff, n_embd, x9)
+    assert np.array_equal(batch[8], got[0])
+    for w in (gate, up, down):
+        rnb.release(w)
+
+
+@pytest.mark.parametrize("tokens,n_ff,n_embd,k,down_quant", [(2, 768, 2048, 8, Q6_K), (3, 256, 512, 1, Q4_K), (4, 512, 1280, 16, Q5_K),
+                                                            (8, 768, 2048, 8, Q6_K), (5, 1024, 768, 3, Q6_K), (8, 2304, 512, 7, Q4_K),
+                                                            (7, 256, 4096, 9, Q5_K)])
+def test_moe_small_batch_equals_general_sequence(rnb, oracle, tokens, n_ff, n_embd, k, down_quant):
+    """Two to eight tokens with at most 64 slots take the decode kernels too (a workgroup of the first kernel quantises
+    its slot's token, one of the second its token's intermediates).  The slot list comes interleaved (rank-major, not
+    token by token), one token has no slot at all, and an expert is shared by several tokens.  Against the oracle, and
+    bit for bit against the same tokens inside a batch of twelve, which takes the general sequence."""
+    n_expert = 20
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 170 + tokens, down_quant)
+    e[(t == 1).nonzero()[0][:1]] = e[0]  # tokens 0 and 1 share an expert
+    order = np.lexsort((t, np.concatenate([np.arange(k)] * tokens)))  # rank-major: token ids interleave
+    e, r, t = e[order], r[order], t[order]
+    if tokens >= 3:
+        keep = t != 2  # token 2 is routed nowhere: its row must be exactly zero
+        e, r, t = e[keep], r[keep], t[keep]
+    assert e.size <= 64
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    ref = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"moe small batch tokens {tokens} k {k}")
+    if tokens >= 3:
+        assert np.all(got[2] == 0.0)
+    pad = 12 - tokens
+    x12 = np.concatenate([x, oracle.fill_normal(pad * n_embd, 6, 1.0)])
+    e12 = np.concatenate([e, np.arange(pad, dtype=np.uint32) % n_expert])
+    r12 = np.concatenate([r, np.full(pad, 0.5, np.float32)])
+    t12 = np.concatenate([t, np.arange(tokens, 12, dtype=np.uint32)])
+    big = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e12, r12, t12, 12, down_quant, n_ff, n_embd, x12)
+    assert np.array_equal(big[:tokens], got)
     for w in (gate, up, down):
         rnb.release(w)
 
