@@ -61,26 +61,43 @@ int hip_fail(const char *what, hipError_t e) {
         if (_e != hipSuccess) return hip_fail(#expr, _e);  \
     } while (0)
 
-// Minimum tokens for which the MFMA GEMMs replace the vector-unit kernels, whose time grows with every token while a
-// GEMM's 32-token tile costs the same from 1 to 32.  Measured crossovers: Q6_K 4096 x 14336 (48 MB) 4 tokens (26.9 us
-// either way; 8 tokens 47 vs 27), Q4_K 14336 x 4096 (33 MB) 4 (21 vs 16 us), Q8_0 4096 x 14336 (62 MB) 3, Q8_0
-// 4096 x 4096 (18 MB) 5, Q4_K and Q5_K 4096 x 4096 (9 and 12 MB) 8 (10.4 vs 9.8 us).
-constexpr size_t kGemmMinSeqLarge = 4, kGemmMinSeqSmall = 8, kGemmLargeBytes = size_t(16) << 20;
+// Minimum tokens for which the MFMA GEMMs replace the vector-unit kernels.  Below it a batch runs the GEMV kernels that
+// keep two to four tokens in registers per pass over the matrix (a pass per group of four tokens: time grows with every
+// token), while a GEMM's 32-token tile costs the same from 1 to 32.  Measured crossovers (us, GEMV groups vs GEMM):
+// Q4_K 14336 x 4096 (33 MB) 4 tokens 14.7 vs 17.7, 5 tokens 18.2 vs 17.5; Q5_K likewise 16.1 vs 20.3, 20.8 vs 20.0; Q6_K
+// 14336 x 4096 6 tokens 23.2 vs 25.6, 7 tokens 25.9 vs 25.5 (4096 x 14336: 27.7 vs 28.6, 31.0 vs 28.7); Q2_K / Q3_K 6 tokens
+// 18.1 / 21.9 vs 21.0 / 23.1, 7 tokens 22.8 / 24.9 vs 21.0 / 23.0; Q8_0 4096 x 4096 6 tokens 13.8 vs 17.1, 7 tokens 17.0
+// vs 17.3 (14336 x 4096: 28.7 vs 33.2, 32.9 vs 33.1); Q4_0 14336 x 4096 8 tokens 22.5 vs 25.8, 12 tokens 29.7 vs 26.0.
+// Matrices that take the chunked GEMV (rows of 9 - 16 super-blocks, 48 MB and more): Q6_K 128256 x 4096 4 tokens 107 vs
+// 122, 5 tokens 163 vs 121; Q4_K / Q5_K 65536 x 4096 3 tokens 43.6 / 49.6, 4 tokens 54.5 / 60.1 vs 42.0 / 46.2.  Small
+// ones: Q4_K 4096 x 4096 (9 MB) 6 tokens 11.6 vs 13.0 (the staged multi-token kernel; GEMM 11.9 from 8), 7 tokens 13.7;
+// Q6_K 4096 x 4096 (14 MB) 8 tokens 14.9 vs 16.2, 12 tokens 19.7 vs 16.3; Q4_K 2048 x 2048 (2.4 MB) 16 tokens 9.0 vs 10.0.
+constexpr size_t kGemmTinyBytes = size_t(4) << 20, kGemmSmallBytes = size_t(16) << 20, kGemmChunkBytes = size_t(48) << 20;
 size_t gemm_min_seq(uint32_t quant, size_t rows, size_t cols) {
     QuantInfo qi;
-    if (!quant_info(quant, &qi)) return kGemmMinSeqSmall;
-    return rows * (cols / qi.elems) * qi.bytes >= kGemmLargeBytes ? kGemmMinSeqLarge : kGemmMinSeqSmall;
+    if (!quant_info(quant, &qi)) return 8;
+    const size_t per_row = cols / qi.elems, bytes = rows * per_row * qi.bytes;
+    if (bytes < kGemmTinyBytes) return 17;
+    const bool chunked = bytes >= kGemmChunkBytes && qi.elems == 256 && per_row > 8 && per_row <= 16;
+    switch (quant) {
+    case kQ4K:
+    case kQ5K: return chunked ? 4 : (bytes < kGemmSmallBytes ? 7 : 5);
+    case kQ6K: return chunked ? 5 : (bytes < kGemmSmallBytes ? 9 : 7);
+    case kQ2K:
+    case kQ3K: return chunked ? 4 : 7;
+    case kQ8_0:
+    case kQ8_1: return 7;
+    default: return 9;  // Q4_0, Q4_1, Q5_0, Q5_1
+    }
 }
 // The Q8_K quantiser adds the per-32 sums as two digits (the Q4_K / Q5_K GEMMs' mins term) from this many tokens on.
-constexpr size_t kDigitsMinSeq = kGemmMinSeqLarge < kGemmMinSeqSmall ? kGemmMinSeqLarge : kGemmMinSeqSmall;
+constexpr size_t kDigitsMinSeq = 4;  // the smallest value gemm_min_seq returns
 // Minimum tokens for which the importance-quant formats take their matrix-core GEMM instead of one GEMV pass per token.
 constexpr size_t kIqGemmMinSeq = 4;
 // Minimum tokens for which the grouped MoE GEMMs on the matrix cores are considered.
 constexpr size_t kMoeMfmaMinTokens = 16;
 // Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
 constexpr uint64_t kGemmBigTilesMin = 32;
-// Minimum tokens for which the staged multi-token kernel replaces one GEMV pass per token.
-constexpr size_t kTokensMinSeq = 4;
 
 // After enqueuing kernels: a launcher that could not configure its kernel (and therefore did not launch) left the
 // reason; otherwise whatever the runtime recorded.
@@ -252,34 +269,30 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
         } else if (seq >= min_gemm_seq && act.digits != nullptr && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0) {
             if (int st = slice_floats(gemm_q4k_slice_floats(r, nb, q), &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q4k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kTokensMinSeq && reinterpret_cast<uintptr_t>(w_dev) % 16 == 0)
-            launch_matmul_tokens(w_dev, kQ4K, act, out_dev, r, nb, q, s.stream);
-        else
+        } else {
             launch_gemv_q4k(w_dev, act, out_dev, r, nb, q, s.stream);
+        }
     } else if (quant == kQ2K || quant == kQ3K) {
         if (seq >= min_gemm_seq) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q23k_mfma(w_dev, quant, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kTokensMinSeq)
-            launch_matmul_tokens(w_dev, quant, act, out_dev, r, nb, q, s.stream);
-        else
+        } else {
             launch_gemv_q2k_q3k(w_dev, quant, act, out_dev, r, nb, q, s.stream);
+        }
     } else if (quant == kQ5K) {
         if (seq >= min_gemm_seq && act.digits != nullptr) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q5k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kTokensMinSeq)
-            launch_matmul_tokens(w_dev, kQ5K, act, out_dev, r, nb, q, s.stream);
-        else
+        } else {
             launch_gemv_q5k(w_dev, act, out_dev, r, nb, q, s.stream);
+        }
     } else if (quant == kQ6K) {
         if (seq >= min_gemm_seq) {
             if (int st = slice_ws(nb, &ws); st != RNB_HIP_OK) return st;
             launch_gemm_q6k_mfma(w_dev, act, out_dev, ws, r, nb, q, s.stream);
-        } else if (seq >= kTokensMinSeq)
-            launch_matmul_tokens(w_dev, kQ6K, act, out_dev, r, nb, q, s.stream);
-        else
+        } else {
             launch_gemv_q6k(w_dev, act, out_dev, r, nb, q, s.stream);
+        }
     } else if (seq >= min_gemm_seq && gemm_q8_mfma_supported(quant, static_cast<uint32_t>(cols / 32))) {
         const uint32_t nb32 = static_cast<uint32_t>(cols / 32);
         if (int st = slice_ws((nb32 + 7) / 8, &ws); st != RNB_HIP_OK) return st;
@@ -451,7 +464,9 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
     const size_t nb_in = n_embd / 256, mid_bytes = seq * n_ff * sizeof(float);
     RESERVE_TRY(s.ffn_mid, mid_bytes);
     const bool aligned = (reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev)) % 16 == 0;
-    const bool small = seq < gemm_min_seq(kQ4K, n_ff, n_embd) && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
+    // the paired gate/up GEMV runs one pass per token: it gives way to the GEMMs earlier than the plain GEMV does
+    const size_t pair_max = n_ff * nb_in * kQ4KBytes >= kGemmSmallBytes ? 4 : 8;
+    const bool small = seq < pair_max && aligned && gemv_q4k_gate_up_supported(static_cast<uint32_t>(nb_in));
     ActView act;
     int st = RNB_HIP_OK;
     if (small && seq == 1 && reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) {

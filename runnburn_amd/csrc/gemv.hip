@@ -89,6 +89,51 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
+// Two to four tokens per pass over the matrix (small decode batches, rows of at most 16 super-blocks): the lane keeps
+// the activation slices of kTokens tokens in registers, every weight block is fetched and unpacked once and dotted
+// against each of them.  Per token the arithmetic and the cross-lane sum are those of gemv_kquant_kernel: same bits.
+// grid.y = token groups; the last group may hold fewer tokens (its spare slots repeat the last token and are not stored).
+// ---------------------------------------------------------------------------------------------
+template <uint32_t kQuant, int kRowsPerWave, int kTokens>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_kquant_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                              const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                              uint32_t row_groups, uint32_t seq) {
+    using Q = KQuant<kQuant>;
+    constexpr int kLanesPerRow = kWave / kRowsPerWave;
+    constexpr size_t kBlockBytes = Q::kBytes;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
+    const int g = sub & 3;
+    const uint32_t bslot = sub >> 2;
+    const uint32_t tok0 = blockIdx.y * kTokens;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const bool has_block = bslot < nb;
+    typename Q::Act a[kTokens];
+#pragma unroll
+    for (int t = 0; t < kTokens; t++) {
+        const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
+        const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+        a[t] = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    }
+    for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
+        const uint32_t row = grp * kRowsPerWave + rsel;
+        const bool live = has_block && row < rows;
+        const uint8_t *blk = w + (live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kBlockBytes : 0);
+        const typename Q::Prep p = Q::prepare(Q::load_block(blk, g), g);  // rows >= 1 and nb >= 1: offset 0 is readable
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) {
+            float acc = live ? Q::dot(p, a[t]) : 0.0f;
+            acc = seg_sum<kLanesPerRow>(acc);
+            if (sub == kLanesPerRow - 1 && row < rows && tok0 + t < seq) out[static_cast<size_t>(tok0 + t) * rows + row] = acc;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // The same GEMV for matrices far larger than what the chip holds in flight (rows of 9 to 16 super-blocks): every wave
 // takes kRows CONSECUTIVE rows, requests all of them at once and retires; with one wave per chunk the hardware
 // dispatcher keeps the CUs supplied with fresh waves, so the window of outstanding requests sweeps the matrix in
@@ -132,6 +177,51 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         }
         const uint32_t row = c * kRows + (kWave - 1 - lane);
         if (lane >= kWave - kRows && row < rows) out[static_cast<size_t>(tok) * rows + row] = v;
+    }
+}
+
+// The chunked GEMV for two to four tokens per pass over the matrix (per token the arithmetic of
+// gemv_kquant_chunks_kernel: same bits); grid.y = token groups.
+template <uint32_t kQuant, int kRows, int kTokens>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_kquant_chunks_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                     const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                                     uint32_t n_chunks, uint32_t seq) {
+    using Q = KQuant<kQuant>;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int g = lane & 3;
+    const uint32_t bslot = lane >> 2;
+    const bool has_block = bslot < nb;
+    const uint32_t tok0 = blockIdx.y * kTokens;
+    const size_t row_bytes = static_cast<size_t>(nb) * Q::kBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    typename Q::Act a[kTokens];
+#pragma unroll
+    for (int t = 0; t < kTokens; t++) {
+        const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
+        const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+        a[t] = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    }
+    for (uint32_t c = wave_global; c < n_chunks; c += n_waves) {
+        typename Q::Regs r[kRows];
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t row = c * kRows + k;
+            const bool ok = has_block && row < rows;  // rows >= 1 and nb >= 1: offset 0 is readable
+            r[k] = Q::load_block(w + (ok ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * Q::kBytes : 0), g);
+        }
+#pragma unroll
+        for (int k = 0; k < kRows; k++) {
+            const uint32_t row = c * kRows + k;
+            const typename Q::Prep p = Q::prepare(r[k], g);
+#pragma unroll
+            for (int t = 0; t < kTokens; t++) {
+                float acc = (has_block && row < rows) ? Q::dot(p, a[t]) : 0.0f;
+                acc = seg_sum<kWave>(acc);
+                if (lane == kWave - 1 && row < rows && tok0 + t < seq) out[static_cast<size_t>(tok0 + t) * rows + row] = acc;
+            }
+        }
     }
 }
 
@@ -558,12 +648,73 @@ __global__ void __launch_bounds__(kWave *kSplitMaxWaves)
     }
 }
 
+// The split-K GEMV for two to four tokens per pass over the matrix: each wave keeps its K slice of kTokens tokens in
+// registers and dots every fetched block against all of them; one barrier per row, partial sums added in wave order
+// (per token the same sums in the same order as gemv_kquant_splitk_kernel: same bits).  grid.y = token groups.
+template <uint32_t kQuant, int kTokens>
+__global__ void __launch_bounds__(kWave *kSplitMaxWaves)
+    gemv_kquant_splitk_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                     const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
+                                     uint32_t seq) {
+    using Q = KQuant<kQuant>;
+    using Regs = typename Q::Regs;
+    constexpr size_t kBlockBytes = Q::kBytes;
+    __shared__ float s_part[2][kTokens][kSplitMaxWaves];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6, n_slices = blockDim.x >> 6;
+    const int g = lane & 3;
+    const uint32_t b = wave * 16 + (lane >> 2);
+    const bool has_block = b < nb;
+    const uint32_t tok0 = blockIdx.y * kTokens;
+    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    typename Q::Act a[kTokens];
+#pragma unroll
+    for (int t = 0; t < kTokens; t++) {
+        const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
+        const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? b : 0);
+        a[t] = Q::load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    }
+    uint32_t parity = 0;
+    for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1) {
+        Regs r = Regs{};  // idle lanes keep zeros
+        if (has_block) r = Q::load_block(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes, g);
+        const typename Q::Prep p = Q::prepare(r, g);
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) {
+            float acc = Q::dot(p, a[t]);
+            acc = seg_sum<kWave>(has_block ? acc : 0.0f);
+            if (lane == kWave - 1) s_part[parity][t][wave] = acc;
+        }
+        __syncthreads();  // the other parity's buffer is reused only after the next barrier
+        if (threadIdx.x < kTokens && tok0 + threadIdx.x < seq) {
+            float sum = 0.0f;
+            for (uint32_t j = 0; j < n_slices; j++) sum += s_part[parity][threadIdx.x][j];
+            out[static_cast<size_t>(tok0 + threadIdx.x) * rows + row] = sum;
+        }
+    }
+}
+
 template <uint32_t kQuant>
 void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                           hipStream_t stream) {
     const uint32_t n_slices = (nb + 15) / 16;
     const uint32_t row_chunks = (rows + kSplitRows - 1) / kSplitRows;
     const uint32_t want = kTargetWaves / n_slices;  // workgroups for about kTargetWaves waves
+    if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
+        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const dim3 tgrid(rows < want ? rows : want, groups, 1);
+#define RNB_LAUNCH_TOKENS(T)                                                                                                  \
+    hipLaunchKernelGGL((gemv_kquant_splitk_tokens_kernel<kQuant, T>), tgrid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d, \
+                       act.bsums, out, rows, nb, seq)
+        if (per == 2)
+            RNB_LAUNCH_TOKENS(2);
+        else if (per == 3)
+            RNB_LAUNCH_TOKENS(3);
+        else
+            RNB_LAUNCH_TOKENS(4);
+#undef RNB_LAUNCH_TOKENS
+        return;
+    }
     const dim3 grid(row_chunks < want ? row_chunks : want, seq, 1);
     if (n_slices == 2 || n_slices == 4)
         hipLaunchKernelGGL((gemv_kquant_splitk_kernel<kQuant, true>), grid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d,
@@ -682,6 +833,21 @@ void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uin
                    hipStream_t stream) {
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
+    if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
+        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
+#define RNB_LAUNCH_TOKENS(T)                                                                                                 \
+    hipLaunchKernelGGL((gemv_kquant_tokens_kernel<kQuant, kRowsPerWave, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, \
+                       act.qs, act.d, act.bsums, out, rows, nb, row_groups, seq)
+        if (per == 2)
+            RNB_LAUNCH_TOKENS(2);
+        else if (per == 3)
+            RNB_LAUNCH_TOKENS(3);
+        else
+            RNB_LAUNCH_TOKENS(4);
+#undef RNB_LAUNCH_TOKENS
+        return;
+    }
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
     hipLaunchKernelGGL((gemv_kquant_kernel<kQuant, kRowsPerWave>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
                        act.d, act.bsums, out, rows, nb, row_groups);
@@ -694,6 +860,21 @@ void launch_kquant_chunks(const uint8_t *w, ActView act, float *out, uint32_t ro
                           hipStream_t stream) {
     const uint32_t n_chunks = (rows + kRows - 1) / kRows;
     const uint32_t waves = n_chunks < kChunkMaxWaves ? n_chunks : kChunkMaxWaves;
+    if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
+        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const dim3 tgrid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
+#define RNB_LAUNCH_TOKENS(T)                                                                                                  \
+    hipLaunchKernelGGL((gemv_kquant_chunks_tokens_kernel<kQuant, kRows, T>), tgrid, dim3(kWave * kWavesPerWg), 0, stream, w,  \
+                       act.qs, act.d, act.bsums, out, rows, nb, n_chunks, seq)
+        if (per == 2)
+            RNB_LAUNCH_TOKENS(2);
+        else if (per == 3)
+            RNB_LAUNCH_TOKENS(3);
+        else
+            RNB_LAUNCH_TOKENS(4);
+#undef RNB_LAUNCH_TOKENS
+        return;
+    }
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
     hipLaunchKernelGGL((gemv_kquant_chunks_kernel<kQuant, kRows>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs,
                        act.d, act.bsums, out, rows, nb, n_chunks);
@@ -971,10 +1152,86 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     }
 }
 
+// Two to four tokens per pass over the matrix, rows of at most 128 blocks (the register-resident branches of
+// gemv_block32_kernel): a lane keeps its two activation blocks of kTokens tokens and dots each fetched weight block
+// against all of them; per token the same expression as the one-token kernel (same bits).  grid.y = token groups.
+template <uint32_t kQuant, bool kPaired, int kTokens>
+__global__ void __launch_bounds__(kWave *kWavesPerWg)
+    gemv_block32_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                               float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq) {
+    constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
+    constexpr bool kSum = kQuant != kQ8_0 && kQuant != kQ8_1;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t tok0 = blockIdx.y * kTokens;
+    const size_t row_bytes = static_cast<size_t>(nb32) * kBlockBytes;
+    const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const uint32_t b0 = kPaired ? 2 * lane : lane, b1 = kPaired ? 2 * lane + 1 : lane + kWave;
+    const bool has0 = b0 < nb32, has1 = b1 < nb32;  // kPaired: nb32 is even, a pair is there or not as a whole
+    Q8Act a0[kTokens], a1[kTokens];
+#pragma unroll
+    for (int t = 0; t < kTokens; t++) {
+        const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
+        const size_t abase = static_cast<size_t>(tok) * nb32;
+        a0[t] = q8_load_act<kSum>(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
+        a1[t] = q8_load_act<kSum>(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
+    }
+    for (uint32_t row = wave_global; row < rows; row += n_waves) {
+        const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+        Block32Regs c0 = Block32Regs{}, c1 = Block32Regs{};
+        if constexpr (kPaired) {
+            if (has0) block32_load_pair<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes, c0, c1);
+        } else {
+            if (has0) c0 = block32_load<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes);
+            if (has1) c1 = block32_load<kQuant>(rowp + static_cast<size_t>(b1) * kBlockBytes);
+        }
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) {
+            float acc = 0.0f;
+            if constexpr (kPaired) {
+                if (has0) acc = block32_dot<kQuant>(c0, a0[t]) + block32_dot<kQuant>(c1, a1[t]);
+            } else {
+                if (has0) acc = block32_dot<kQuant>(c0, a0[t]);
+                if (has1) acc += block32_dot<kQuant>(c1, a1[t]);
+            }
+            acc = seg_sum<kWave>(acc);
+            if (lane == kWave - 1 && tok0 + t < seq) out[static_cast<size_t>(tok0 + t) * rows + row] = acc;
+        }
+    }
+}
+
 template <uint32_t kQuant>
 void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32, uint32_t seq,
                     hipStream_t stream) {
     const uint32_t waves = rows < kTargetWaves ? rows : kTargetWaves;
+    if (seq >= 2 && nb32 <= 2 * kWave) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
+        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const dim3 tgrid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
+        bool paired = false;
+        if constexpr (block32_pairs<kQuant>()) paired = nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0;
+#define RNB_LAUNCH_TOKENS(P, T)                                                                                              \
+    hipLaunchKernelGGL((gemv_block32_tokens_kernel<kQuant, P, T>), tgrid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, \
+                       act.d, out, rows, nb32, seq)
+#define RNB_LAUNCH_TOKENS_P(P)    \
+    do {                          \
+        if (per == 2)             \
+            RNB_LAUNCH_TOKENS(P, 2); \
+        else if (per == 3)        \
+            RNB_LAUNCH_TOKENS(P, 3); \
+        else                      \
+            RNB_LAUNCH_TOKENS(P, 4); \
+    } while (0)
+        if constexpr (block32_pairs<kQuant>()) {
+            if (paired) {
+                RNB_LAUNCH_TOKENS_P(true);
+                return;
+            }
+        }
+        RNB_LAUNCH_TOKENS_P(false);
+#undef RNB_LAUNCH_TOKENS_P
+#undef RNB_LAUNCH_TOKENS
+        return;
+    }
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
     if constexpr (block32_pairs<kQuant>()) {
         if (nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0) {  // every pair of every row starts on a 4-byte boundary

@@ -107,11 +107,6 @@ void launch_argmax(const float *values, uint32_t len, float *scratch_values, uin
 // out[i] = act(gate[i]) * up[i]
 void launch_act_mul(const float *gate, const float *up, float *out, size_t n, bool gelu, hipStream_t stream);
 
-// Multi-token matmul on the vector ALUs for Q2_K ... Q6_K (weights decoded once per eight staged tokens);
-// same output contract as launch_gemv_q4k
-void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
-                          uint32_t seq, hipStream_t stream);
-
 // Q6_K / Q5_K x Q8_K and 32-element formats (Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1) x Q8 GEMMs on int8 MFMA (scale groups applied on the vector units); same contracts as
 // launch_gemv_q6k / launch_gemv_block32, intended for seq >= 16.  Small grids are cut into K slices that are summed by
 // a second kernel: slice_out is the workspace for that, gemm_blocks_slice_floats(quant, rows, k_steps, seq) floats

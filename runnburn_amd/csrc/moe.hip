@@ -213,66 +213,6 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Dense multi-token matmul on the vector ALUs (Q5_K and Q6_K at any batch size, Q4_K below the MFMA GEMM's minimum): the same
-// "stage up to eight tokens in LDS, decode a weight block once, dot it per token" walk as the expert kernels, over
-// one weight matrix and consecutive tokens.  out[token * rows + row].
-// ---------------------------------------------------------------------------------------------
-template <uint32_t kQuant, int kRowsPerWave>
-__global__ void __launch_bounds__(kWave *kWavesPerWg)
-    matmul_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                         const int16_t *__restrict__ abs, float *__restrict__ out, uint32_t rows, uint32_t nb,
-                         uint32_t seq, uint32_t iters, uint32_t tmax, uint32_t chunks_per_wg) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int kLanesPerRow = kWave / kRowsPerWave;
-    constexpr uint32_t kBlocksPerPass = kLanesPerRow / 4;
-    using Q = KQuant<kQuant>;
-    constexpr size_t kBlockBytes = Q::kBytes;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-    const int sub = lane & (kLanesPerRow - 1);
-    const uint32_t rsel = lane / kLanesPerRow;
-    const int g = sub & 3;
-    const uint32_t bslot = sub >> 2;
-    const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
-    const Staged st = stage_layout(lds, tmax, nb);
-    const uint32_t tok_begin = blockIdx.y * chunks_per_wg * tmax;
-    const uint32_t tok_end = min(seq, tok_begin + chunks_per_wg * tmax);
-
-    for (uint32_t c0 = tok_begin; c0 < tok_end; c0 += tmax) {
-        const uint32_t nt = min(tmax, tok_end - c0);
-        if (c0 != tok_begin) __syncthreads();
-        for (uint32_t t = 0; t < nt; t++) stage_row(lds, tmax, nb, t, c0 + t, aq, ad, abs);
-        __syncthreads();
-        for (uint32_t it = 0; it < iters; it++) {
-            const uint32_t row = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave + rsel;
-            const bool row_ok = row < rows;
-            float acc[kMaxChunkTokens];
-#pragma unroll
-            for (int t = 0; t < kMaxChunkTokens; t++) acc[t] = 0.0f;
-            for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
-                if (!row_ok) break;
-                const uint8_t *blk = w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-                const typename Q::Prep p = Q::prepare(Q::load_block(blk, g), g);
-#pragma unroll
-                for (int t = 0; t < kMaxChunkTokens; t++) {
-                    if (static_cast<uint32_t>(t) < nt) {
-                        const size_t ab = static_cast<size_t>(t) * nb + b;
-                        acc[t] += Q::dot(p, Q::load_act(st.qs + ab * kStageBlk, st.d[ab], st.bsums + ab * 16, g));
-                    }
-                }
-            }
-#pragma unroll
-            for (int t = 0; t < kMaxChunkTokens; t++) {
-                if (static_cast<uint32_t>(t) < nt) {
-                    const float s = seg_sum<kLanesPerRow>(acc[t]);
-                    if (sub == kLanesPerRow - 1 && row_ok) out[static_cast<size_t>(c0 + t) * rows + row] = s;
-                }
-            }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
 // Decode-sized calls: down projection, route weight and the per-token ordered sum in one launch, no slot_out round
 // trip.  A wave owns ONE output row of one token; its lanes are split into 64/L groups of L = 4 * (blocks a group can
 // hold) lanes, each group dotting that row of a different slot's expert against that slot's quantised intermediate.
@@ -553,29 +493,6 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
                        nb_mid, p.iters, p.tmax)
     RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN);
 #undef RNB_LAUNCH_DOWN
-}
-
-void launch_matmul_tokens(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb,
-                          uint32_t seq, hipStream_t stream) {
-    if (rows == 0 || seq == 0) return;
-    const int rpw = rows_per_wave_for(nb);
-    TilePlan p = plan_tiles(rows, nb, 1, rpw);  // more than 48 KiB of staging costs more in occupancy than it saves
-    const uint32_t chunks = (seq + p.tmax - 1) / p.tmax;
-    // enough workgroups to fill the chip: split the token chunks over grid.y while row tiles alone are too few
-    uint32_t ysplit = 1;
-    while (p.tiles * ysplit < 1024 && ysplit < chunks) ysplit *= 2;
-    const uint32_t chunks_per_wg = (chunks + ysplit - 1) / ysplit;
-    const dim3 grid(p.tiles, (chunks + chunks_per_wg - 1) / chunks_per_wg, 1), block(kWave * kWavesPerWg);
-#define RNB_LAUNCH_MT(Q, R)                                                                                           \
-    hipLaunchKernelGGL((matmul_tokens_kernel<Q, R>), grid, block, p.lds_bytes, stream, w, act.qs, act.d, act.bsums,   \
-                       out, rows, nb, seq, p.iters, p.tmax, chunks_per_wg)
-    if (quant == kQ2K)
-        RNB_DISPATCH_KQUANT_R(kQ2K, rpw, RNB_LAUNCH_MT);
-    else if (quant == kQ3K)
-        RNB_DISPATCH_KQUANT_R(kQ3K, rpw, RNB_LAUNCH_MT);
-    else
-        RNB_DISPATCH_KQUANT(quant, rpw, RNB_LAUNCH_MT);
-#undef RNB_LAUNCH_MT
 }
 
 void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,

@@ -372,10 +372,32 @@ def test_gemv_batch_small(rnb, oracle, quant, seq):
                 f"batch quant {quant} seq {seq}")
 
 
+@pytest.mark.parametrize("quant,rows,cols", [(Q4_K, 300, 4096), (Q6_K, 131, 2048), (Q5_K, 70, 1024), (Q2_K, 257, 3072),
+                                             (Q3_K, 90, 512), (Q6_K, 45, 14336), (Q4_K, 33, 8192), (Q3_K, 21, 5120),
+                                             (Q8_0, 200, 4096), (Q8_0, 77, 1056), (Q4_0, 130, 4096), (Q5_1, 64, 2080),
+                                             (Q4_1, 99, 96), (Q8_1, 50, 4096), (Q5_0, 41, 4096)])
+def test_small_batches_equal_one_token_calls_bit_for_bit(rnb, oracle, quant, rows, cols):
+    """Two to eight tokens run the GEMV kernels that fetch and unpack every weight block once and dot it against the
+    activation slices of up to four tokens held in registers (row loop, K split for rows of more than 16 super-blocks,
+    the 32-element formats with and without paired blocks): per token the same sums in the same order as the one-token
+    kernel, so every row of the batch equals the one-token call."""
+    w = oracle.make_weights(quant, rows, cols, 2300 + rows)
+    one = gemv_fn(rnb, quant, batch=False)
+    many = gemv_fn(rnb, quant, batch=True)
+    x = oracle.fill_normal(8 * cols, 2301 + cols, 1.0)
+    alone = np.stack([one(w, rows, cols, x[t * cols:(t + 1) * cols]) for t in range(8)])
+    for seq in (2, 3, 4, 5, 7, 8):
+        got = many(w, rows, cols, x[:seq * cols]).reshape(seq, rows)
+        assert np.array_equal(got.view(np.uint32), alone[:seq].view(np.uint32)), (quant, rows, cols, seq)
+    check_close(alone, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True),
+                f"small batches quant {quant} {rows}x{cols}")
+    rnb.release(w)
+
+
 @pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_gemv_batch_long_rows(rnb, oracle, quant):
-    """Rows longer than 16 super-blocks: the K-split kernel with tokens on grid.y up to 3 tokens, the staged
-    multi-token kernel from 4 tokens on."""
+    """Rows longer than 16 super-blocks in small batches: the K-split kernel with groups of up to four tokens per pass
+    (3, then 4 + 4 + 3, then 3 + 3)."""
     for rows, cols, seq in ((21, 20 * 256, 3), (19, 20 * 256, 11), (5, 56 * 256, 6)):
         w = oracle.make_weights(quant, rows, cols, 150 + quant)
         x = oracle.fill_normal(seq * cols, 160, 1.0)
@@ -384,11 +406,11 @@ def test_gemv_batch_long_rows(rnb, oracle, quant):
                     f"long-row batch quant {quant} rows {rows} seq {seq}")
 
 
-@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
-                                           (1, 1, 16), (257, 5, 40), (4097, 1, 513), (8200, 2, 260), (2050, 9, 260),
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 17), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 18),
+                                           (1, 1, 17), (257, 5, 40), (4097, 1, 513), (8200, 2, 260), (2050, 9, 260),
                                            (8192, 8, 65)])
 def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
-    """Q4_K with 16+ tokens: shapes with fewer than 32 tiles of 256 rows x 64 tokens take the 128 x 32 / 64 kernel of
+    """Q4_K batches on the matrix cores: shapes with fewer than 32 tiles of 256 rows x 64 tokens take the 128 x 32 / 64 kernel of
     gemm_blocks.hip, the last four the ping-pong kernel of gemm_q4k.hip: 153 and 165 tiles, both dimensions off the
     tile, then 45 and 64 tiles, where K is cut into two slices (5 + 4 blocks, 4 + 4) that a second kernel adds."""
     cols = nblk * 256
@@ -399,10 +421,10 @@ def test_q4k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
                 f"gemm rows {rows} nblk {nblk} seq {seq}")
 
 
-@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
-                                           (1, 1, 16), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 17), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 18),
+                                           (1, 1, 17), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
 def test_q6k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
-    """16 or more tokens on Q6_K take the matrix-core GEMM (one K=16 instruction per sub-block, sub-block scales on
+    """Batches on Q6_K take the matrix-core GEMM (one K=16 instruction per sub-block, sub-block scales on
     the vector units): row and token counts off the 128 x 32 / 64 tile, one token tile and two."""
     cols = nblk * 256
     w = oracle.make_weights(Q6_K, rows, cols, 170 + rows)
@@ -434,10 +456,10 @@ def test_q6k_gemm_extreme_blocks(rnb, oracle):
                 "q6k gemm extremes")
 
 
-@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 16),
-                                           (1, 1, 16), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 17), (33, 3, 17), (64, 4, 129), (100, 2, 33), (40, 20, 18),
+                                           (1, 1, 17), (257, 5, 40), (129, 1, 65), (4096, 2, 64)])
 def test_q5k_gemm_mfma_ragged_tiles(rnb, oracle, rows, nblk, seq):
-    """16 or more tokens on Q5_K: one K=32 matrix instruction per sub-block, 6-bit scales on the vector units, the mins
+    """Batches on Q5_K: one K=32 matrix instruction per sub-block, 6-bit scales on the vector units, the mins
     term through the quantiser's digits."""
     cols = nblk * 256
     w = oracle.make_weights(Q5_K, rows, cols, 470 + rows)
@@ -472,12 +494,16 @@ def test_q5k_gemm_extreme_blocks(rnb, oracle):
                 "q5k gemm extremes")
 
 
-@pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 8192, 4096, 4), (Q4_K, 8192, 4096, 7), (Q5_K, 6144, 4096, 6),
-                                                 (Q6_K, 4096, 5120, 5), (Q8_0, 4096, 4096, 4), (Q8_1, 4096, 4096, 15),
-                                                 (Q4_K, 4096, 4096, 8), (Q6_K, 2048, 4096, 11)])
+@pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 8192, 4096, 4), (Q4_K, 8192, 4096, 5), (Q5_K, 6144, 4096, 6),
+                                                 (Q6_K, 4096, 5120, 6), (Q6_K, 4096, 5120, 7), (Q8_0, 4096, 4096, 6),
+                                                 (Q8_0, 4096, 4096, 7), (Q8_1, 4096, 4096, 15), (Q4_K, 4096, 4096, 6),
+                                                 (Q4_K, 4096, 4096, 8), (Q6_K, 2048, 4096, 8), (Q6_K, 2048, 4096, 11),
+                                                 (Q4_0, 4096, 4096, 8), (Q4_0, 4096, 4096, 9), (Q2_K, 8192, 4096, 7)])
 def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
-    """Matrices of 16 MB and more go to the matrix-core GEMMs from 4 tokens on, smaller ones from 8 (a 32-token tile
-    mostly empty: loads of the missing tokens repeat the last one, their results are not stored)."""
+    """Either side of the token count at which a format's matrix-core GEMM takes over from the GEMV kernels that keep two
+    to four tokens in registers (5 for Q4_K / Q5_K, 7 for Q6_K, Q2_K, Q3_K, Q8_0, Q8_1, 9 for the nibble formats; two more
+    under 16 MB): on the GEMV side groups of 4, 3 + 3, 4 + 4 tokens, on the GEMM side a 32-token tile mostly empty (loads
+    of the missing tokens repeat the last one, their results are not stored)."""
     w = oracle.make_weights(quant, rows, cols, 1200 + seq)
     x = oracle.fill_normal(seq * cols, 1210 + seq, 1.0)
     got = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x)
@@ -488,7 +514,7 @@ def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
 
 
 @pytest.mark.parametrize("quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K])
-@pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 16), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
+@pytest.mark.parametrize("rows,nblk,seq", [(128, 37, 17), (200, 11, 48), (4096, 16, 64), (1024, 8, 96)])
 def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
     """Grids too small for the chip are cut along K (blockIdx.z) and the slices' outputs added by a second kernel in
     slice order: 13 slices of 3 blocks and one of 1 (the cap of 16 slices asked for), slices of unequal length, and the
@@ -504,7 +530,7 @@ def test_gemm_k_slices(rnb, oracle, quant, rows, nblk, seq):
 
 
 @pytest.mark.parametrize("quant", [Q2_K, Q3_K])
-@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 16), (33, 3, 17), (64, 4, 129), (100, 2, 33), (1, 1, 8),
+@pytest.mark.parametrize("rows,nblk,seq", [(32, 1, 32), (31, 2, 17), (33, 3, 17), (64, 4, 129), (100, 2, 33), (1, 1, 17),
                                            (257, 5, 40), (129, 1, 65), (640, 3, 600)])
 def test_q2k_q3k_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, nblk, seq):
     """Batches on Q2_K / Q3_K take the matrix-core GEMM (one K=16 instruction per 16-element sub-block, its scale on the
@@ -521,8 +547,8 @@ def test_q2k_q3k_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, nblk, seq):
 
 
 @pytest.mark.parametrize("quant", [Q8_0, Q8_1, Q4_0, Q4_1, Q5_0, Q5_1])
-@pytest.mark.parametrize("rows,cols,seq", [(32, 32, 16), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
-                                           (1, 4096, 16), (300, 288, 100)])
+@pytest.mark.parametrize("rows,cols,seq", [(32, 32, 17), (31, 96, 17), (33, 1056, 33), (130, 2080, 64), (257, 256, 65),
+                                           (1, 4096, 17), (300, 288, 100)])
 def test_q8_gemm_mfma_ragged_tiles(rnb, oracle, quant, rows, cols, seq):
     """Batches on the 32-element formats take the matrix-core GEMM (one K=32 instruction per block, the two f32 scales
     on the vector units; the nibble formats' codes are split, given their fifth bit and offset in packed bytes, the
@@ -591,12 +617,14 @@ def test_config3b_q6k_gemv_lm_head_128256x4096(rnb, oracle):
 
 
 @pytest.mark.parametrize("quant,rows,cols,seq", [(Q4_K, 21001, 4096, 1), (Q6_K, 15003, 4096, 1), (Q5_K, 17921, 4096, 3),
-                                                 (Q4_K, 38839, 2304, 2), (Q2_K, 40001, 4096, 1), (Q3_K, 30001, 4096, 1)])
+                                                 (Q4_K, 38839, 2304, 2), (Q2_K, 40001, 4096, 1), (Q3_K, 30001, 4096, 1),
+                                                 (Q6_K, 15003, 4096, 4)])
 def test_gemv_chunked_rows_kernel_large_matrices(rnb, oracle, quant, rows, cols, seq):
     """Matrices of 48 MB and more with rows of 9 to 16 super-blocks take the kernel whose waves each reduce a chunk of
     consecutive rows (two, four for Q6_K): row counts that are no multiple of the chunk, 9 super-blocks per row (idle
-    lanes), and two or three tokens (one grid row per token).  The arithmetic per row is the grid-stride kernel's, so
-    the first 4096 rows alone, a matrix small enough for that kernel, give the same bits."""
+    lanes), and two to four tokens (their activation slices kept in registers, one pass over the matrix).  The arithmetic
+    per row is the grid-stride kernel's, so the first 4096 rows alone, a matrix small enough for that kernel, give the
+    same bits."""
     w = oracle.make_weights(quant, rows, cols, 7000 + rows)
     x = oracle.fill_normal(seq * cols, 7001 + rows, 1.0)
     fn = gemv_fn(rnb, quant, batch=seq > 1)

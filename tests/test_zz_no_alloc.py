@@ -26,7 +26,7 @@ def _both(rnb, oracle, quant, rows, cols, seq, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("quant,big,small", [
-    (Q4_K, (1024, 4096, 48), (300, 1024, 5)),      # MFMA GEMM with digits, then the staged multi-token kernel
+    (Q4_K, (1024, 4096, 48), (300, 1024, 5)),      # MFMA GEMM with digits, then the GEMV that keeps several tokens in registers
     (Q6_K, (512, 14336, 24), (257, 5120, 1)),      # K cut into slices (workspace in the array), then split-K GEMV
     (Q8_0, (768, 4096, 40), (64, 96, 3)),          # 32-wide Q8 activations
     (Q4_K, (2048, 4096, 1), (40, 512, 2)),         # one-launch decode GEMV (no scratch), then a tiny batch
