@@ -351,7 +351,7 @@ def one_launch_step(quant, rows, cols, seq):
         return False
     if quant in (10, 11, Q4_K, Q5_K, Q6_K):
         nb = cols // 256
-        return nb <= 16 and (nb <= 8 or rows * nb * BLOCK_BYTES.get(quant, 144) < (300 << 20))
+        return nb <= 32 and (nb <= 8 or rows * nb * BLOCK_BYTES.get(quant, 144) < (300 << 20))
     return cols // 32 <= 128 and rows * (cols // 32) >= 1 << 18
 
 
@@ -775,7 +775,18 @@ def main() -> int:
                             "kernel_ms_p90": pq["p90"], "ops": ops, "TOP/s": tops, "mfma_frac": tops / INT8_PEAK_TOPS}
             except Exception as exc:
                 sec[key] = {"error": str(exc)}
-        for tokens in (1, 64):
+        # small batches (several sequences decoding together): the GEMV that keeps four tokens in registers per pass
+        try:
+            res, _, _, _ = bench_matmul(rnb, hip, stream, Q4_K, 14336, 4096, 4, s2, 10, 7 + 4, "q4k 14336x4096 x 4 tokens",
+                                        want_graph=False, want_wall=False)
+            st = res["step"]
+            sec["q4k_14336x4096_tokens4"] = {"step_ms_mean": st["mean"], "step_ms_median": st["median"], "step_ms_p10": st["p10"],
+                                             "step_ms_p90": st["p90"], "launches": st["launches"],
+                                             "step": "two launches: activation quantiser, then one pass over the matrix for "
+                                                     "the four tokens"}
+        except Exception as exc:
+            sec["q4k_14336x4096_tokens4"] = {"error": str(exc)}
+        for tokens in (1, 4, 64):
             try:
                 sec[f"cfg5_moe_tokens{tokens}"] = bench_moe(rnb, hip, stream, tokens, s2, 1234 + tokens,
                                                             cpu=not args.no_cpu_baseline)
