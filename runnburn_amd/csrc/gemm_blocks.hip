@@ -37,7 +37,7 @@ namespace rnb {
 
 namespace {
 
-template <int kTT>
+template <int kTT, int kLive>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q6k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                          float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq, uint32_t nb_slice) {
@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
             const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
                 tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 32 * 127 */                                          \
                 asm volatile("" : "+v"(tot[t][i])); /* no re-association of the sixteen sums into a tree */            \
             }                                                                                                          \
@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
         for (int t = 0; t < kTT; t++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < kLive / 4; j++) {
                 const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
                 const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
@@ -153,7 +153,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
         for (int t = 0; t < kTT; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
+            for (int r = 0; r < kLive; r++) {
                 const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
                 if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
             }
@@ -228,7 +228,7 @@ __device__ __forceinline__ int q23_scale(const Q23Row &r) {
     }
 }
 
-template <int kTT, bool kThree>
+template <int kTT, bool kThree, int kLive>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q23k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                           const int16_t *__restrict__ abs16, float *__restrict__ out, uint32_t rows, uint32_t nb,
@@ -310,7 +310,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
             const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
                 tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 4 * 127 */                                           \
                 asm volatile("" : "+v"(tot[t][i]));                                                                    \
             }                                                                                                          \
@@ -347,10 +347,10 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                 const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(lo, mnop, zero16, 0, 0, 0);
                 const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(hi, mnop, zero16, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 16; i++) mins[i] = c0[i] + 64 * c1[i];
+                for (int i = 0; i < kLive; i++) mins[i] = c0[i] + 64 * c1[i];
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < kLive / 4; j++) {
                 const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
                 const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
@@ -371,7 +371,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
         for (int t = 0; t < kTT; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
+            for (int r = 0; r < kLive; r++) {
                 const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
                 if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
             }
@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 // quantiser's digits (bsum32 = b0 + 64 * b1): two K=16 instructions with eight live K slots per token tile.
 // Per super-block out += d_x * (d * float(tot) - dmin * float(S)): crates/rnb-cpu/src/gemm/neon_dot.rs:1742-1800.
 // ---------------------------------------------------------------------------------------------
-template <int kTT, bool kFifth>
+template <int kTT, bool kFifth, int kLive>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q45k_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                          const uint8_t *__restrict__ adig, float *__restrict__ out, uint32_t rows, uint32_t nb,
@@ -455,7 +455,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * (SB));                 \
             const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < 16; i++) {                                                           \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
                 tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 32 * 31 * 127 */                                          \
                 asm volatile("" : "+v"(tot[t][i])); /* no re-association of the eight sums into a tree */              \
             }                                                                                                          \
@@ -504,7 +504,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
             for (int t = 0; t < kTT; t++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) tot[t][i] = acc_lo[t][i] + 8 * acc_hi[t][i];
+                for (int i = 0; i < kLive; i++) tot[t][i] = acc_lo[t][i] + 8 * acc_hi[t][i];
         }
 
         // mins: K slots 0..7 of the lower K-half carry the eight mins (weights) and the eight digits (tokens)
@@ -520,7 +520,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
             const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op0, mnop, zero16, 0, 0, 0);
             const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(op1, mnop, zero16, 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < kLive / 4; j++) {
                 const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf])[8 * t + 2 * j + khalf];
                 const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
@@ -541,7 +541,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
         for (int t = 0; t < kTT; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
+            for (int r = 0; r < kLive; r++) {
                 const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
                 if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
             }
@@ -724,7 +724,7 @@ constexpr size_t q8_lds_bytes(bool routed) {
     return 2 * (32 * kTT) * kGbStride128 + 2 * 8 * (32 * kTT) * sizeof(float) + (routed ? kGbWaves * kQ8StripBytes : 0);
 }
 
-template <int kTT, uint32_t kFmt, bool kRouted>
+template <int kTT, uint32_t kFmt, bool kRouted, int kLive>
 __global__ void __launch_bounds__(kGbThreads, 2)
     gemm_q8_mfma_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                         float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq, uint32_t steps_slice) {
@@ -836,7 +836,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                         sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, ones, zero16, 0, 0, 0);
                     }
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
+                    for (int j = 0; j < kLive / 4; j++) {
                         const float4 dx4 = reinterpret_cast<const float4 *>(s_dx[buf][k])[8 * t + 2 * j + khalf];
                         const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
@@ -868,7 +868,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
 #pragma unroll
         for (int t = 0; t < kTT; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
+            for (int r = 0; r < kLive; r++) {
                 const uint32_t tok = tok0 + 32 * t + 8 * (r >> 2) + 4 * khalf + (r & 3);
                 if (tok < seq) out[static_cast<size_t>(tok) * rows + row] = accf[t][r];
             }
@@ -945,6 +945,19 @@ size_t gemm_blocks_slice_floats(uint32_t quant, uint32_t rows, uint32_t k_steps,
     return slices > 1 ? static_cast<size_t>(slices) * seq * rows : 0;
 }
 
+// A batch of at most 8 / 16 tokens fills only the first 4 / 8 of the sixteen results a lane holds per 32-token tile
+// (result r is token 8 (r / 4) + 4 khalf + r % 4): the kernels are instantiated for 4, 8 and 16 live results and apply
+// scales, float updates and stores to those only.
+#define RNB_BY_LIVE_TOKENS(SEQ, LAUNCH) \
+    do {                                \
+        if ((SEQ) <= 8)                 \
+            LAUNCH(4);                  \
+        else if ((SEQ) <= 16)           \
+            LAUNCH(8);                  \
+        else                            \
+            LAUNCH(16);                 \
+    } while (0)
+
 void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slice_out, uint32_t rows, uint32_t nb,
                           uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0 || nb == 0) return;
@@ -955,12 +968,15 @@ void launch_gemm_q6k_mfma(const uint8_t *w, ActView act, float *out, float *slic
     float *dst = nz > 1 ? slice_out : out;
     if (wide) {
         const dim3 grid(row_tiles, (seq + 63) / 64, nz);
-        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<2>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
-                           nb_slice);
+        hipLaunchKernelGGL((gemm_q6k_mfma_kernel<2, 16>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb,
+                           seq, nb_slice);
     } else {
         const dim3 grid(row_tiles, (seq + 31) / 32, nz);
-        hipLaunchKernelGGL(gemm_q6k_mfma_kernel<1>, grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, seq,
-                           nb_slice);
+#define RNB_LAUNCH_Q6(LIVE)                                                                                            \
+    hipLaunchKernelGGL((gemm_q6k_mfma_kernel<1, LIVE>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, dst, rows, nb, \
+                       seq, nb_slice)
+        RNB_BY_LIVE_TOKENS(seq, RNB_LAUNCH_Q6);
+#undef RNB_LAUNCH_Q6
     }
     if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
@@ -974,20 +990,24 @@ void launch_gemm_q23k_mfma(const uint8_t *w, uint32_t quant, ActView act, float 
     const uint32_t nb_slice = (nb + slices - 1) / slices, nz = (nb + nb_slice - 1) / nb_slice;
     float *dst = nz > 1 ? slice_out : out;
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : (seq + 31) / 32, nz), block(kGbThreads);
-#define RNB_LAUNCH_Q23(TT, THREE)                                                                                      \
-    hipLaunchKernelGGL((gemm_q23k_mfma_kernel<TT, THREE>), grid, block, 0, stream, w, act.qs, act.d, act.bsums, dst, rows, nb, \
-                       seq, nb_slice)
+#define RNB_LAUNCH_Q23(TT, THREE, LIVE)                                                                                \
+    hipLaunchKernelGGL((gemm_q23k_mfma_kernel<TT, THREE, LIVE>), grid, block, 0, stream, w, act.qs, act.d, act.bsums, dst, \
+                       rows, nb, seq, nb_slice)
+#define RNB_LAUNCH_Q3_LIVE(LIVE) RNB_LAUNCH_Q23(1, true, LIVE)
+#define RNB_LAUNCH_Q2_LIVE(LIVE) RNB_LAUNCH_Q23(1, false, LIVE)
     if (quant == kQ3K) {
         if (wide)
-            RNB_LAUNCH_Q23(2, true);
+            RNB_LAUNCH_Q23(2, true, 16);
         else
-            RNB_LAUNCH_Q23(1, true);
+            RNB_BY_LIVE_TOKENS(seq, RNB_LAUNCH_Q3_LIVE);
     } else {
         if (wide)
-            RNB_LAUNCH_Q23(2, false);
+            RNB_LAUNCH_Q23(2, false, 16);
         else
-            RNB_LAUNCH_Q23(1, false);
+            RNB_BY_LIVE_TOKENS(seq, RNB_LAUNCH_Q2_LIVE);
     }
+#undef RNB_LAUNCH_Q2_LIVE
+#undef RNB_LAUNCH_Q3_LIVE
 #undef RNB_LAUNCH_Q23
     if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
@@ -1003,12 +1023,15 @@ static void launch_gemm_q45k(const uint8_t *w, ActView act, float *out, float *s
     float *dst = nz > 1 ? slice_out : out;
     if (wide) {
         const dim3 grid(row_tiles, (seq + 63) / 64, nz);
-        hipLaunchKernelGGL((gemm_q45k_mfma_kernel<2, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
-                           dst, rows, nb, seq, nb_slice);
+        hipLaunchKernelGGL((gemm_q45k_mfma_kernel<2, kFifth, 16>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d,
+                           act.digits, dst, rows, nb, seq, nb_slice);
     } else {
         const dim3 grid(row_tiles, (seq + 31) / 32, nz);
-        hipLaunchKernelGGL((gemm_q45k_mfma_kernel<1, kFifth>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d, act.digits,
-                           dst, rows, nb, seq, nb_slice);
+#define RNB_LAUNCH_Q45(LIVE)                                                                                           \
+    hipLaunchKernelGGL((gemm_q45k_mfma_kernel<1, kFifth, LIVE>), grid, dim3(kGbThreads), 0, stream, w, act.qs, act.d,  \
+                       act.digits, dst, rows, nb, seq, nb_slice)
+        RNB_BY_LIVE_TOKENS(seq, RNB_LAUNCH_Q45);
+#undef RNB_LAUNCH_Q45
     }
     if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
 }
@@ -1037,25 +1060,31 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     const dim3 grid(row_tiles, wide ? (seq + 63) / 64 : 1, nz), block(kGbThreads);
     // the strip routes: whole steps only (a partial step's pieces would leave the last row)
     const bool routed = nb32 % 8 == 0;
-#define RNB_LAUNCH_Q8R(TT, FMT, R)                                                                                     \
+#define RNB_LAUNCH_Q8R(TT, FMT, R, LIVE)                                                                               \
     {                                                                                                                  \
         constexpr size_t lds = q8_lds_bytes<TT>(R);                                                                    \
         static bool configured = false; /* above the default 64 KB of dynamic LDS in the routed 64-token form */       \
-        if (!allow_dynamic_lds(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, FMT, R>), lds, &configured,      \
+        if (!allow_dynamic_lds(reinterpret_cast<const void *>(gemm_q8_mfma_kernel<TT, FMT, R, LIVE>), lds, &configured, \
                                "gemm_q8_mfma_kernel"))                                                                 \
             return;                                                                                                    \
-        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, FMT, R>), grid, block, lds, stream, w, act.qs, act.d, dst, rows,   \
-                           nb32, seq, steps_slice);                                                                    \
+        hipLaunchKernelGGL((gemm_q8_mfma_kernel<TT, FMT, R, LIVE>), grid, block, lds, stream, w, act.qs, act.d, dst,   \
+                           rows, nb32, seq, steps_slice);                                                              \
+    }
+#define RNB_LAUNCH_Q8N(FMT, R) /* one 32-token tile: by the number of live results */                                  \
+    {                                                                                                                  \
+        if (seq <= 8) RNB_LAUNCH_Q8R(1, FMT, R, 4)                                                                     \
+        else if (seq <= 16) RNB_LAUNCH_Q8R(1, FMT, R, 8)                                                               \
+        else RNB_LAUNCH_Q8R(1, FMT, R, 16)                                                                             \
     }
 #define RNB_LAUNCH_Q8(FMT, ROUTABLE)                                                                                   \
     if constexpr (ROUTABLE) {                                                                                          \
-        if (routed && wide) RNB_LAUNCH_Q8R(2, FMT, true)                                                               \
-        else if (routed) RNB_LAUNCH_Q8R(1, FMT, true)                                                                  \
-        else if (wide) RNB_LAUNCH_Q8R(2, FMT, false)                                                                   \
-        else RNB_LAUNCH_Q8R(1, FMT, false)                                                                             \
+        if (routed && wide) RNB_LAUNCH_Q8R(2, FMT, true, 16)                                                           \
+        else if (routed) RNB_LAUNCH_Q8N(FMT, true)                                                                     \
+        else if (wide) RNB_LAUNCH_Q8R(2, FMT, false, 16)                                                               \
+        else RNB_LAUNCH_Q8N(FMT, false)                                                                                \
     } else {                                                                                                           \
-        if (wide) RNB_LAUNCH_Q8R(2, FMT, false)                                                                        \
-        else RNB_LAUNCH_Q8R(1, FMT, false)                                                                             \
+        if (wide) RNB_LAUNCH_Q8R(2, FMT, false, 16)                                                                    \
+        else RNB_LAUNCH_Q8N(FMT, false)                                                                                \
     }
     switch (quant) {
     case kQ8_0: RNB_LAUNCH_Q8(kQ8_0, true) break;
@@ -1065,6 +1094,7 @@ void launch_gemm_q8_mfma(const uint8_t *w, uint32_t quant, ActView act, float *o
     case kQ5_0: RNB_LAUNCH_Q8(kQ5_0, true) break;
     default: RNB_LAUNCH_Q8(kQ5_1, true) break;
     }
+#undef RNB_LAUNCH_Q8N
 #undef RNB_LAUNCH_Q8R
 #undef RNB_LAUNCH_Q8
     if (nz > 1) launch_sum_slices(slice_out, out, static_cast<size_t>(seq) * rows, nz, stream);
