@@ -320,11 +320,11 @@ void launch_kquant_f32_any(const uint8_t *w, const float *x, float *out, uint32_
 // mapping as gemv_kquant_kernel (rows of at most 16 super-blocks); a wave fetches row r of BOTH matrices against the
 // one activation slice it holds, so the activation is loaded once and gate/up never travel through memory.
 // ---------------------------------------------------------------------------------------------
-template <int kRowsPerWave, bool kGelu>
+template <int kRowsPerWave, bool kGelu, int kTokens>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_q4k_gate_up_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ abs,
-                            float *__restrict__ mid, uint32_t rows, uint32_t nb, uint32_t row_groups) {
+                            float *__restrict__ mid, uint32_t rows, uint32_t nb, uint32_t row_groups, uint32_t seq) {
     constexpr int kLanesPerRow = kWave / kRowsPerWave;
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane & (kLanesPerRow - 1);
@@ -332,24 +332,30 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     const int g = sub & 3;
     const uint32_t bslot = sub >> 2;
     const bool has_block = bslot < nb;
-    const uint32_t tok = blockIdx.y;
-    const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+    const uint32_t tok0 = blockIdx.y * kTokens;  // a group of kTokens tokens per pass over the two matrices
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
     const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     const uint32_t n_waves = gridDim.x * kWavesPerWg;
-    const Q4KAct a4 = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    Q4KAct a4[kTokens];
+#pragma unroll
+    for (int t = 0; t < kTokens; t++) {
+        const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;  // the last group's spare slots repeat the last token
+        const size_t ab = static_cast<size_t>(tok) * nb + (has_block ? bslot : 0);
+        a4[t] = q4k_load_act(aq + ab * 256, ad[ab], abs + ab * 16, g);
+    }
     for (uint32_t grp = wave_global; grp < row_groups; grp += n_waves) {
         const uint32_t row = grp * kRowsPerWave + rsel;
-        float gs = 0.0f, us = 0.0f;
-        if (has_block && row < rows) {
-            const size_t off = static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes;
-            const Q4KRegs rg = q4k_load_block(wg + off, g), ru = q4k_load_block(wu + off, g);
-            gs = q4k_partial(rg, a4, g);
-            us = q4k_partial(ru, a4, g);
+        const bool live = has_block && row < rows;
+        const size_t off = live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0;
+        const Q4KPrep pg = q4k_prepare(q4k_load_block(wg + off, g), g), pu = q4k_prepare(q4k_load_block(wu + off, g), g);
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) {
+            float gs = live ? q4k_dot(pg, a4[t]) : 0.0f, us = live ? q4k_dot(pu, a4[t]) : 0.0f;
+            gs = seg_sum<kLanesPerRow>(gs);
+            us = seg_sum<kLanesPerRow>(us);
+            if (sub == kLanesPerRow - 1 && row < rows && tok0 + t < seq)
+                mid[static_cast<size_t>(tok0 + t) * rows + row] = act_mul<kGelu>(gs, us);
         }
-        gs = seg_sum<kLanesPerRow>(gs);
-        us = seg_sum<kLanesPerRow>(us);
-        if (sub == kLanesPerRow - 1 && row < rows) mid[static_cast<size_t>(tok) * rows + row] = act_mul<kGelu>(gs, us);
     }
 }
 
@@ -358,13 +364,29 @@ void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mi
                     uint32_t seq, bool gelu, hipStream_t stream) {
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
-    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, seq, 1);
+    // groups of equal size, at most four tokens each
+    const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
+#define RNB_LAUNCH_GU(GELU, T)                                                                                              \
+    hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, GELU, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu, \
+                       act.qs, act.d, act.bsums, mid, rows, nb, row_groups, seq)
+#define RNB_LAUNCH_GU_T(GELU)      \
+    do {                           \
+        if (per == 1)              \
+            RNB_LAUNCH_GU(GELU, 1); \
+        else if (per == 2)         \
+            RNB_LAUNCH_GU(GELU, 2); \
+        else if (per == 3)         \
+            RNB_LAUNCH_GU(GELU, 3); \
+        else                       \
+            RNB_LAUNCH_GU(GELU, 4); \
+    } while (0)
     if (gelu)
-        hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, true>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu,
-                           act.qs, act.d, act.bsums, mid, rows, nb, row_groups);
+        RNB_LAUNCH_GU_T(true);
     else
-        hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, false>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu,
-                           act.qs, act.d, act.bsums, mid, rows, nb, row_groups);
+        RNB_LAUNCH_GU_T(false);
+#undef RNB_LAUNCH_GU_T
+#undef RNB_LAUNCH_GU
 }
 
 // The same front half straight from f32 tokens: the workgroup quantises token blockIdx.y to Q8_K in LDS as

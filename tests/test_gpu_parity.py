@@ -898,20 +898,53 @@ def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
 
 # ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
 
+def check_ffn(oracle, got, gate, up, down, down_quant, n_ff, n_embd, x, gelu, label):
+    """The oracle's composition within the usual row check, plus what quantising the intermediate allows: act(gate) * up
+    goes through expf / tanhf, whose last bit differs between the device and the host, and the two GEMV sums before it are
+    added in different orders.  An element of the intermediate that lies within 1e-4 (relative) of a rounding boundary of
+    its Q8_K / Q8 block may therefore be quantised one code apart; one code of element k is worth |W_down[r][k]| * d_block
+    in output row r.  Rows are held to the usual tolerance plus that sum over the token's near-boundary elements (a few
+    per token); every other difference fails."""
+    seq = x.size // n_embd
+    ref = (oracle.dense_gelu_ffn if gelu else oracle.dense_silu_ffn)(gate, up, down, down_quant, n_ff, n_embd, x)
+    g = oracle.gemv(Q4_K, gate, n_ff, n_embd, x).ravel()
+    u = oracle.gemv(Q4_K, up, n_ff, n_embd, x).ravel()
+    mid = (oracle.gelu_mul if gelu else oracle.silu_mul)(g, u).reshape(seq, n_ff).astype(np.float64)
+    blk = oracle.BLOCK_ELEMS[down_quant]
+    m = mid.reshape(seq, n_ff // blk, blk)
+    amax = np.abs(m).max(axis=2, keepdims=True)
+    d = amax / 127.0                                    # one code step of the block, both quantisers
+    v = np.divide(m, d, out=np.zeros_like(m), where=d > 0)
+    near = np.abs(np.abs(v - np.floor(v)) - 0.5) < 1e-4 * np.maximum(1.0, np.abs(v))
+    w = np.abs(oracle.dequantize(down_quant, down).reshape(n_embd, n_ff).astype(np.float64))
+    step = np.broadcast_to(d, m.shape).reshape(seq, n_ff)
+    near = near.reshape(seq, n_ff)
+    slack = np.stack([w[:, near[t]] @ step[t, near[t]] for t in range(seq)])
+    got = np.asarray(got, np.float64).reshape(seq, n_embd)
+    r64 = ref.astype(np.float64).reshape(seq, n_embd)
+    assert np.all(np.isfinite(got)), f"{label}: non-finite output"
+    rms = float(np.sqrt(np.mean(r64 * r64))) or 1.0
+    tol = np.maximum(REL * rms, REL * np.abs(r64)) + slack
+    bad = np.abs(got - r64) > tol
+    assert not bad.any(), (f"{label}: {int(bad.sum())} elements outside 1e-3 plus the quantiser's near-boundary slack "
+                           f"(near-boundary elements per token: {near.sum(axis=1).tolist()}); worst excess "
+                           f"{float((np.abs(got - r64) - tol).max())}")
+
+
 @pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K, Q8_0, Q5_1])
 @pytest.mark.parametrize("seq,n_ff,n_embd", [(2, 256, 256), (3, 768, 512), (5, 512, 4608), (17, 512, 768), (40, 1024, 256)])
 def test_dense_silu_ffn_batch(rnb, oracle, down_quant, seq, n_ff, n_embd):
-    """Decode-sized batches take the fused gate/up GEMV, 8+ tokens (these matrices are small) the MFMA GEMMs and the gated
-    quantiser, rows longer than 16 super-blocks the unfused pair; all must equal the per-token composition of the
+    """Decode-sized batches take the fused gate/up GEMV (groups of up to four tokens per pass over the two matrices), 9+
+    tokens (these matrices are small) the MFMA GEMMs and the gated quantiser, rows longer than 16 super-blocks the unfused pair; all must equal the per-token composition of the
     oracle's pinned pieces."""
     gate = oracle.make_weights(Q4_K, n_ff, n_embd, 300 + seq)
     up = oracle.make_weights(Q4_K, n_ff, n_embd, 301 + seq)
     down = oracle.make_weights(down_quant, n_embd, n_ff, 302 + seq)
     x = oracle.fill_normal(seq * n_embd, 303 + seq, 1.0)
     got = rnb.dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
-    ref = oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x)
-    assert got.shape == ref.shape == (seq, n_embd)
-    check_close(got, ref, None, f"dense ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
+    assert got.shape == (seq, n_embd)
+    check_ffn(oracle, got, gate, up, down, down_quant, n_ff, n_embd, x, False,
+              f"dense ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
 
 
 @pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K])
@@ -928,23 +961,25 @@ def test_dense_gelu_ffn(rnb, oracle, down_quant, seq, n_ff, n_embd):
         got = rnb.dense_q4k_gelu_ffn(gate, up, down, down_quant, n_ff, n_embd, x).reshape(1, n_embd)
     else:
         got = rnb.dense_q4k_gelu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
-    check_close(got, ref, None, f"gelu ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
+    check_ffn(oracle, got, gate, up, down, down_quant, n_ff, n_embd, x, True,
+              f"gelu ffn seq {seq} n_ff {n_ff} n_embd {n_embd} down {down_quant}")
     # and it is not the SiLU result
     assert not np.allclose(got, oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x), rtol=1e-3, atol=0)
 
 
-@pytest.mark.parametrize("seq,down_quant", [(5, Q6_K), (9, Q4_K)])
+@pytest.mark.parametrize("seq,down_quant", [(5, Q6_K), (6, Q4_K), (7, Q6_K), (9, Q4_K)])
 def test_dense_silu_ffn_few_tokens_large_matrices(rnb, oracle, seq, down_quant):
-    """Gate / up matrices of 16 MB and more (8192 x 4096 Q4_K) leave the fused gate/up GEMV for the GEMMs from 4 tokens
-    on: gate and up GEMMs, SiLU * up quantised as it is made, down GEMM (K slices on these small grids)."""
+    """Gate / up matrices of 16 MB and more (8192 x 4096 Q4_K) keep the fused gate/up GEMV up to six tokens (groups of
+    3 + 2 and 3 + 3) and leave it for the GEMMs from seven on: gate and up GEMMs, SiLU * up quantised as it is made, down
+    GEMM (K slices on these small grids)."""
     n_ff, n_embd = 8192, 4096
     gate = oracle.make_weights(Q4_K, n_ff, n_embd, 340 + seq)
     up = oracle.make_weights(Q4_K, n_ff, n_embd, 341 + seq)
     down = oracle.make_weights(down_quant, n_embd, n_ff, 342 + seq)
     x = oracle.fill_normal(seq * n_embd, 343 + seq, 1.0)
     got = rnb.dense_q4k_silu_ffn_batch(gate, up, down, down_quant, n_ff, n_embd, seq, x)
-    ref = oracle.dense_silu_ffn(gate, up, down, down_quant, n_ff, n_embd, x)
-    check_close(got, ref, None, f"dense ffn, large matrices, seq {seq} down {down_quant}")
+    check_ffn(oracle, got, gate, up, down, down_quant, n_ff, n_embd, x, False,
+              f"dense ffn, large matrices, seq {seq} down {down_quant}")
 
 
 def test_dense_silu_ffn_dev_single_token_and_residency(rnb, oracle):
