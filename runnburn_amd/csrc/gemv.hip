@@ -855,7 +855,9 @@ void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uin
                    hipStream_t stream) {
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
-    if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
+    // several tokens per pass over the matrix, in groups of equal size (at most four); rows longer than one wave pass
+    // (only reached beyond the K-split kernel's 256 super-blocks) keep one pass per token
+    if (seq >= 2 && nb <= static_cast<uint32_t>(kWave / kRowsPerWave / 4)) {
         const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
         const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
 #define RNB_LAUNCH_TOKENS(T)                                                                                                 \

@@ -397,8 +397,9 @@ def test_small_batches_equal_one_token_calls_bit_for_bit(rnb, oracle, quant, row
 @pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K])
 def test_gemv_batch_long_rows(rnb, oracle, quant):
     """Rows longer than 16 super-blocks in small batches: the K-split kernel with groups of up to four tokens per pass
-    (3, then 4 + 4 + 3, then 3 + 3)."""
-    for rows, cols, seq in ((21, 20 * 256, 3), (19, 20 * 256, 11), (5, 56 * 256, 6)):
+    (3, then 4 + 4 + 3, then 3 + 3); rows beyond the K-split kernel's 256 super-blocks keep one pass per token (the row
+    loop walks them in passes of 16 super-blocks)."""
+    for rows, cols, seq in ((21, 20 * 256, 3), (19, 20 * 256, 11), (5, 56 * 256, 6), (3, 257 * 256, 2)):
         w = oracle.make_weights(quant, rows, cols, 150 + quant)
         x = oracle.fill_normal(seq * cols, 160, 1.0)
         got = gemv_fn(rnb, quant, True)(w, rows, cols, x)
