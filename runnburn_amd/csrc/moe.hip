@@ -275,7 +275,9 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // ---------------------------------------------------------------------------------------------
 constexpr int kDecodeWaves = 8;
 
-template <int kRowsPerWave>
+// kOne: a call of one token (token index 0 for every slot, the whole list is the token's): no table look-ups in front of
+// the first loads
+template <int kRowsPerWave, bool kOne>
 __global__ void __launch_bounds__(kWave *kDecodeWaves)
     moe_decode_gate_up_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
                               const float *__restrict__ x, const MoeDecodeTable table, float *__restrict__ mid,
@@ -295,7 +297,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     const bool live = bslot < nb && row < n_ff;
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
     TokenSpans<kDecodeWaves> xv;
-    token_load<kDecodeWaves>(x + static_cast<size_t>(table.token[slot]) * nb * 256, nb, wave, lane, xv);
+    token_load<kDecodeWaves>(x + (kOne ? 0 : static_cast<size_t>(table.token[slot]) * nb * 256), nb, wave, lane, xv);
     // dead lanes read the expert's first block
     const size_t off = static_cast<size_t>(table.expert[slot]) * n_ff * row_bytes +
                        (live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0);
@@ -315,7 +317,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     if (sub == kLanesPerRow - 1 && row < n_ff) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(gs, us);
 }
 
-template <uint32_t kQuant, int kGroups>
+template <uint32_t kQuant, int kGroups, bool kOne>
 __global__ void __launch_bounds__(kWave *kDecodeWaves)
     moe_decode_down_kernel(const uint8_t *__restrict__ down_all, const float *__restrict__ mid, const MoeDecodeTable table,
                            float *__restrict__ out, uint32_t n_embd, uint32_t nb) {
@@ -334,7 +336,8 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     const int g = sub & 3;
     const uint32_t b = sub >> 2;
     const uint32_t tok = blockIdx.y;
-    const uint32_t first = table.tok_off[tok], n_slots = table.tok_off[tok + 1] - first, n_blocks = n_slots * nb;
+    const uint32_t first = kOne ? 0 : table.tok_off[tok];
+    const uint32_t n_slots = kOne ? table.n_slots : table.tok_off[tok + 1] - first, n_blocks = n_slots * nb;
     mid += static_cast<size_t>(first) * nb * 256;  // this token's slots: k below counts from `first`
     const bool lane_ok = b < nb && row < n_embd;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
@@ -521,16 +524,28 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
         const int rpw = rows_per_wave_for(nb_in);
         const uint32_t row_groups = (n_ff + rpw - 1) / rpw;
         const dim3 grid((row_groups + kDecodeWaves - 1) / kDecodeWaves, table.n_slots, 1);
+#define RNB_LAUNCH_DGU1(Q, R) \
+    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, true>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
 #define RNB_LAUNCH_DGU(Q, R) \
-    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
-        RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU);
+    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, false>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
+        if (table.n_tokens == 1)
+            RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU1);
+        else
+            RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU);
 #undef RNB_LAUNCH_DGU
+#undef RNB_LAUNCH_DGU1
     }
     const dim3 grid((n_embd + kDecodeWaves - 1) / kDecodeWaves, table.n_tokens, 1);
+#define RNB_LAUNCH_DD1(Q, G) \
+    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, true>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
 #define RNB_LAUNCH_DD(Q, G) \
-    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
-    RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD);
+    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, false>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
+    if (table.n_tokens == 1)
+        RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD1);
+    else
+        RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD);
 #undef RNB_LAUNCH_DD
+#undef RNB_LAUNCH_DD1
 }
 
 void launch_moe_reduce(const float *slot_out, const uint32_t *tok_offsets, const uint32_t *tok_slots, float *out,
