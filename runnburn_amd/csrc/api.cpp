@@ -733,17 +733,22 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     RESERVE_TRY(s.moe_mid_bsums, n_slots * sh.nb_mid * 16 * sizeof(int16_t));
     launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
-    launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
-                        s.moe_mid_bsums.as<int16_t>(), nullptr, s.stream);
+    const bool token_major = n_slots <= kMoeTokenMajorSlots && sh.nb_mid <= 16;
+    // expert-major with short intermediates: the down kernel quantises the rows it stages, one launch fewer
+    const bool down_quantises = !token_major && moe_down_quantises(static_cast<uint32_t>(sh.nb_mid));
+    if (!down_quantises)
+        launch_quantize_q8k(s.moe_mid.as<float>(), n_slots * sh.nb_mid, s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(),
+                            s.moe_mid_bsums.as<int16_t>(), nullptr, s.stream);
     ActView mid{s.moe_mid_qs.as<int8_t>(), s.moe_mid_d.as<float>(), s.moe_mid_bsums.as<int16_t>()};
-    if (n_slots <= kMoeTokenMajorSlots && sh.nb_mid <= 16) {
+    if (token_major) {
         // decode: few slots, every expert is read by one token anyway; one launch does down, route and the ordered sum
         const uint32_t *d_sexp = d_list + 3 * n_slots + n_groups + (n_groups + 1);
         launch_moe_down_token(down_dev, down_quant, mid, d_off, d_list, d_sexp, d_route, out_dev,
                               static_cast<uint32_t>(token_count), static_cast<uint32_t>(n_embd),
                               static_cast<uint32_t>(sh.nb_mid), s.stream);
     } else {
-        launch_moe_down(down_dev, down_quant, mid, groups, d_route, s.moe_slot_out.as<float>(),
+        launch_moe_down(down_dev, down_quant, mid, down_quantises ? s.moe_mid.as<float>() : nullptr, groups, d_route,
+                        s.moe_slot_out.as<float>(),
                         static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);

@@ -162,8 +162,10 @@ void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs
 // mid[slot][n_ff] = silu(Wg[e] . h_tok) * (Wu[e] . h_tok); act = Q8_K(x) per token
 void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
                         uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
-// slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])); mid_act is indexed by slot
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+// slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])); mid_act is indexed by slot; with mid_f32
+// ([slot][nb_mid * 256], non-null) the workgroups quantise the rows they stage themselves and mid_act is not read
+bool moe_down_quantises(uint32_t nb_mid);  // whether that pays (short intermediates)
+void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const float *mid_f32, MoeGroups groups,
                      const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // the same two steps on the matrix cores for batches (act / mid_act carry digits, except a Q6_K down's mid_act):
 // 32-token tiles per expert group, see moe_mfma.hip

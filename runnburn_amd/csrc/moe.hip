@@ -67,6 +67,18 @@ __device__ __forceinline__ void stage_row(uint8_t *lds, uint32_t tmax, uint32_t 
     for (uint32_t i = threadIdx.x; i < nb * 2; i += blockDim.x) db[i] = sb[i];
 }
 
+// quantises f32 row `src` (nb blocks of 256) into staging slot t: the stand-alone quantiser's wave routine, a wave per
+// block (the same bits); must be called by the whole workgroup
+__device__ __forceinline__ void stage_row_f32(uint8_t *lds, uint32_t tmax, uint32_t nb, uint32_t t, const float *__restrict__ src) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    int8_t *dq = reinterpret_cast<int8_t *>(lds) + static_cast<size_t>(t) * nb * kStageBlk;
+    float *dd = reinterpret_cast<float *>(lds + stage_d_offset(tmax, nb)) + static_cast<size_t>(t) * nb;
+    int16_t *db = reinterpret_cast<int16_t *>(lds + stage_bsums_offset(tmax, nb)) + static_cast<size_t>(t) * nb * 16;
+    for (uint32_t b = wave; b < nb; b += n_waves)
+        q8k_quantize_span(src + static_cast<size_t>(b) * 256, lane, dq + static_cast<size_t>(b) * kStageBlk, dd + b, db + b * 16);
+}
+
 // ---------------------------------------------------------------------------------------------
 // gate + up + SiLU*up.  Grid (row tiles, expert groups).  kRowsPerWave rows side by side per wave.
 // ---------------------------------------------------------------------------------------------
@@ -151,10 +163,12 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // ---------------------------------------------------------------------------------------------
 // down projection of the re-quantised intermediate, scaled by the route weight.
 // ---------------------------------------------------------------------------------------------
-template <uint32_t kQuant, int kRowsPerWave>
+// kFromF32: the intermediates come as f32 rows (mid_f32[slot][nb * 256]) and are quantised while they are staged
+template <uint32_t kQuant, int kRowsPerWave, bool kFromF32>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_down_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
-                    const int16_t *__restrict__ mbs, const uint32_t *__restrict__ grp_expert,
+                    const int16_t *__restrict__ mbs, const float *__restrict__ mid_f32,
+                    const uint32_t *__restrict__ grp_expert,
                     const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
                     const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
                     uint32_t iters, uint32_t tmax) {
@@ -178,7 +192,13 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     for (uint32_t c0 = 0; c0 < count; c0 += tmax) {
         const uint32_t nt = min(tmax, count - c0);
         if (c0) __syncthreads();
-        for (uint32_t t = 0; t < nt; t++) stage_row(lds, tmax, nb, t, sorted_slot[start + c0 + t], mq, md, mbs);
+        for (uint32_t t = 0; t < nt; t++) {
+            const uint32_t slot = sorted_slot[start + c0 + t];
+            if constexpr (kFromF32)
+                stage_row_f32(lds, tmax, nb, t, mid_f32 + static_cast<size_t>(slot) * nb * 256);
+            else
+                stage_row(lds, tmax, nb, t, slot, mq, md, mbs);
+        }
         __syncthreads();
         for (uint32_t it = 0; it < iters; it++) {
             const uint32_t row = blockIdx.x * rows_per_wg + (it * kWavesPerWg + wave) * kRowsPerWave + rsel;
@@ -484,17 +504,28 @@ void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView 
 #undef RNB_LAUNCH_GU
 }
 
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, MoeGroups groups,
+// every workgroup of an expert group repeats the quantisation of the group's rows: worth it for short intermediates
+bool moe_down_quantises(uint32_t nb_mid) { return nb_mid <= 8; }
+
+void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const float *mid_f32, MoeGroups groups,
                      const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (groups.n_groups == 0) return;
     const int rpw = rows_per_wave_for(nb_mid);
     const TilePlan p = plan_tiles(n_embd, nb_mid, groups.n_groups, rpw);
     const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
-#define RNB_LAUNCH_DOWN(Q, R)                                                                                        \
-    hipLaunchKernelGGL((moe_down_kernel<Q, R>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d,    \
-                       mid_act.bsums, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, \
+#define RNB_LAUNCH_DOWN(Q, R)                                                                                             \
+    hipLaunchKernelGGL((moe_down_kernel<Q, R, false>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d, \
+                       mid_act.bsums, nullptr, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out,     \
+                       n_embd, nb_mid, p.iters, p.tmax)
+#define RNB_LAUNCH_DOWN_F32(Q, R)                                                                                         \
+    hipLaunchKernelGGL((moe_down_kernel<Q, R, true>), grid, block, p.lds_bytes, stream, down_all, nullptr, nullptr,       \
+                       nullptr, mid_f32, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd,   \
                        nb_mid, p.iters, p.tmax)
-    RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN);
+    if (mid_f32 != nullptr)
+        RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN_F32);
+    else
+        RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN);
+#undef RNB_LAUNCH_DOWN_F32
 #undef RNB_LAUNCH_DOWN
 }
 
