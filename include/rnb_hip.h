@@ -196,7 +196,8 @@ int rnb_hip_quant_embedding_gather_dev(uint32_t quant, const uint8_t *w, size_t 
 /* iq2_xxs_gemv / iq2_s_gemv / iq3_xxs_gemv / iq4_xs_gemv and their batch forms, quant_api.rs:543-722 (same checks and
  * texts): importance-quant rows (66 / 82 / 98 / 136-byte blocks of 256 elements) x Q8_K(x), the block dots of
  * crates/rnb-cpu/src/gemm/neon_quant.rs:273-411 over the layouts of crates/rnb-cpu/src/quantize/iq.rs:23-116.  Batches
- * of four tokens and more run on the matrix cores (the same integer group sums, one f32 update per block). */
+ * of five tokens and more run on the matrix cores (the same integer group sums, one f32 update per block); smaller
+ * ones on the GEMV, a decoded block dotted against up to four tokens per pass. */
 int rnb_hip_iq2_xxs_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x,
                          size_t x_len, float *out, size_t out_len);
 int rnb_hip_iq2_xxs_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,

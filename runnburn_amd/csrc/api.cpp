@@ -92,8 +92,10 @@ size_t gemm_min_seq(uint32_t quant, size_t rows, size_t cols) {
 }
 // The Q8_K quantiser adds the per-32 sums as two digits (the Q4_K / Q5_K GEMMs' mins term) from this many tokens on.
 constexpr size_t kDigitsMinSeq = 4;  // the smallest value gemm_min_seq returns
-// Minimum tokens for which the importance-quant formats take their matrix-core GEMM instead of one GEMV pass per token.
-constexpr size_t kIqGemmMinSeq = 4;
+// Minimum tokens for which the importance-quant formats take their matrix-core GEMM instead of the GEMV that dots a
+// decoded block against up to four tokens (14336 x 4096, 4 tokens: 20.8 - 22.9 us against 21.8 - 25.8; 5 tokens: 29 - 35
+// against 21.5 - 25.7).
+constexpr size_t kIqGemmMinSeq = 5;
 // Minimum tokens for which the grouped MoE GEMMs on the matrix cores are considered.
 constexpr size_t kMoeMfmaMinTokens = 16;
 // Minimum number of 256 x 64 tiles for which the Q4_K ping-pong GEMM replaces the smaller-tile kernel.
@@ -249,7 +251,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
     };
     float *ws = nullptr;
     if (is_iq_quant(quant)) {
-        // importance quants: the matrix-core GEMM for batches, else one GEMV pass per token (grid row per token)
+        // importance quants: the matrix-core GEMM for batches, else the GEMV (a pass per group of up to four tokens)
         if (seq >= kIqGemmMinSeq) {
             if (int st = slice_floats(gemm_iq_slice_floats(r, nb, q), &ws); st != RNB_HIP_OK) return st;
             launch_gemm_iq_mfma(w_dev, quant, act, out_dev, ws, r, nb, q, s.stream);

@@ -100,25 +100,36 @@ struct Iq<kIQ2XXS> {
     static constexpr size_t kBytes = kIQ2XXSBytes;
     static constexpr int kTableBytes = 2048;
     static __device__ __forceinline__ const void *table() { return g_iq2xxs.v; }
-    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g, const void *tab) {
+    // kT tokens against one decoded block: res[t] = this lane's part of token t's dot (per token the one-token arithmetic)
+    template <int kT>
+    static __device__ __forceinline__ void partial(const uint8_t *blk, const IqAct (&act)[kT], int g, const void *tab,
+                                                   float (&res)[kT]) {
         const uint64_t *grid_tab = static_cast<const uint64_t *>(tab);
         const uint4 raw = ld_u4_a2(blk + 2 + 16 * g);  // two groups: {indices, scales and signs} each
         const uint32_t idx[2] = {raw.x, raw.z}, ss[2] = {raw.y, raw.w};
-        float fsum = 0.0f;
+        float fsum[kT];
+#pragma unroll
+        for (int t = 0; t < kT; t++) fsum[t] = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            int isum = 0;
+            int isum[kT];
+#pragma unroll
+            for (int t = 0; t < kT; t++) isum[t] = 0;
 #pragma unroll
             for (int l = 0; l < 4; l++) {
                 const uint64_t grid = grid_tab[(idx[h] >> (8 * l)) & 0xffu];
                 const uint32_t s = sign_byte(ss[h] >> (7 * l));
                 const uint32_t lo = apply_signs4(static_cast<uint32_t>(grid), s);
                 const uint32_t hi = apply_signs4(static_cast<uint32_t>(grid >> 32), s >> 4);
-                isum = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, isum);
+#pragma unroll
+                for (int t = 0; t < kT; t++) isum[t] = dot8(lo, hi, act[t].a[2 * h + (l >> 1)], l & 1, isum[t]);
             }
-            fsum += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum);
+#pragma unroll
+            for (int t = 0; t < kT; t++) fsum[t] += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum[t]);
         }
-        return ld_f16(blk) * act.dx * 0.25f * fsum;
+        const float d = ld_f16(blk);
+#pragma unroll
+        for (int t = 0; t < kT; t++) res[t] = d * act[t].dx * 0.25f * fsum[t];
     }
 };
 
@@ -127,17 +138,23 @@ struct Iq<kIQ2S> {
     static constexpr size_t kBytes = kIQ2SBytes;
     static constexpr int kTableBytes = 8192;
     static __device__ __forceinline__ const void *table() { return g_iq2s.v; }
-    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g, const void *tab) {
+    template <int kT>
+    static __device__ __forceinline__ void partial(const uint8_t *blk, const IqAct (&act)[kT], int g, const void *tab,
+                                                   float (&res)[kT]) {
         const uint64_t *grid_tab = static_cast<const uint64_t *>(tab);
         const uint2 lowb = ld_u2_a2(blk + 2 + 8 * g), signb = ld_u2_a2(blk + 34 + 8 * g);
         const uint32_t qh2 = *reinterpret_cast<const unsigned short *>(blk + 66 + 2 * g);
         const uint32_t sc2 = *reinterpret_cast<const unsigned short *>(blk + 74 + 2 * g);
         const uint32_t low[2] = {lowb.x, lowb.y}, sg[2] = {signb.x, signb.y};
-        int isum = 0;
+        int isum[kT];
+#pragma unroll
+        for (int t = 0; t < kT; t++) isum[t] = 0;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const uint32_t qh = (qh2 >> (8 * h)) & 0xffu, sc = (sc2 >> (8 * h)) & 0xffu;
-            int half_sum[2] = {0, 0};
+            int half_sum[kT][2];
+#pragma unroll
+            for (int t = 0; t < kT; t++) half_sum[t][0] = half_sum[t][1] = 0;
 #pragma unroll
             for (int l = 0; l < 4; l++) {
                 const uint32_t index = ((low[h] >> (8 * l)) & 0xffu) | ((qh << (8 - 2 * l)) & 0x300u);
@@ -145,11 +162,17 @@ struct Iq<kIQ2S> {
                 const uint32_t s = (sg[h] >> (8 * l)) & 0xffu;
                 const uint32_t lo = apply_signs4(static_cast<uint32_t>(grid), s);
                 const uint32_t hi = apply_signs4(static_cast<uint32_t>(grid >> 32), s >> 4);
-                half_sum[l >> 1] = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, half_sum[l >> 1]);
+#pragma unroll
+                for (int t = 0; t < kT; t++)
+                    half_sum[t][l >> 1] = dot8(lo, hi, act[t].a[2 * h + (l >> 1)], l & 1, half_sum[t][l >> 1]);
             }
-            isum += half_sum[0] * static_cast<int>(1 + 2 * (sc & 15u)) + half_sum[1] * static_cast<int>(1 + 2 * (sc >> 4));
+#pragma unroll
+            for (int t = 0; t < kT; t++)
+                isum[t] += half_sum[t][0] * static_cast<int>(1 + 2 * (sc & 15u)) + half_sum[t][1] * static_cast<int>(1 + 2 * (sc >> 4));
         }
-        return ld_f16(blk) * act.dx * 0.125f * static_cast<float>(isum);
+        const float d = ld_f16(blk);
+#pragma unroll
+        for (int t = 0; t < kT; t++) res[t] = d * act[t].dx * 0.125f * static_cast<float>(isum[t]);
     }
 };
 
@@ -158,26 +181,36 @@ struct Iq<kIQ3XXS> {
     static constexpr size_t kBytes = kIQ3XXSBytes;
     static constexpr int kTableBytes = 1024;
     static __device__ __forceinline__ const void *table() { return g_iq3xxs.v; }
-    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g, const void *tab) {
+    template <int kT>
+    static __device__ __forceinline__ void partial(const uint8_t *blk, const IqAct (&act)[kT], int g, const void *tab,
+                                                   float (&res)[kT]) {
         const uint32_t *grid_tab = static_cast<const uint32_t *>(tab);
         const uint4 idx = ld_u4_a2(blk + 2 + 16 * g);  // eight indices per group, two groups
         const uint2 ssb = ld_u2_a2(blk + 66 + 8 * g);
         const uint32_t iw[4] = {idx.x, idx.y, idx.z, idx.w}, ss[2] = {ssb.x, ssb.y};
-        float fsum = 0.0f;
+        float fsum[kT];
+#pragma unroll
+        for (int t = 0; t < kT; t++) fsum[t] = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            int isum = 0;
+            int isum[kT];
+#pragma unroll
+            for (int t = 0; t < kT; t++) isum[t] = 0;
 #pragma unroll
             for (int l = 0; l < 4; l++) {
                 const uint32_t pair = iw[2 * h + (l >> 1)] >> (16 * (l & 1));  // indices 2l and 2l + 1 of the group
                 const uint32_t s = sign_byte(ss[h] >> (7 * l));
                 const uint32_t lo = apply_signs4(grid_tab[pair & 0xffu], s);
                 const uint32_t hi = apply_signs4(grid_tab[(pair >> 8) & 0xffu], s >> 4);
-                isum = dot8(lo, hi, act.a[2 * h + (l >> 1)], l & 1, isum);
+#pragma unroll
+                for (int t = 0; t < kT; t++) isum[t] = dot8(lo, hi, act[t].a[2 * h + (l >> 1)], l & 1, isum[t]);
             }
-            fsum += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum);
+#pragma unroll
+            for (int t = 0; t < kT; t++) fsum[t] += (0.5f + static_cast<float>(ss[h] >> 28)) * static_cast<float>(isum[t]);
         }
-        return ld_f16(blk) * act.dx * 0.5f * fsum;
+        const float d = ld_f16(blk);
+#pragma unroll
+        for (int t = 0; t < kT; t++) res[t] = d * act[t].dx * 0.5f * fsum[t];
     }
 };
 
@@ -196,7 +229,9 @@ struct Iq<kIQ4XS> {
     static constexpr size_t kBytes = kIQ4XSBytes;
     static constexpr int kTableBytes = 0;
     static __device__ __forceinline__ const void *table() { return nullptr; }
-    static __device__ __forceinline__ float partial(const uint8_t *blk, const IqAct &act, int g, const void *) {
+    template <int kT>
+    static __device__ __forceinline__ void partial(const uint8_t *blk, const IqAct (&act)[kT], int g, const void *,
+                                                   float (&res)[kT]) {
         const uint2 hdr = ld_u2_a2(blk);  // f16 d | scales_h << 16, then scales_l
         const uint4 q0 = ld_u4_a2(blk + 8 + 32 * g), q1 = ld_u4_a2(blk + 24 + 32 * g);
         const uint32_t scales_h = hdr.x >> 16;
@@ -204,20 +239,29 @@ struct Iq<kIQ4XS> {
         const int s0 = static_cast<int>((both & 15u) | (((scales_h >> (4 * g)) & 3u) << 4)) - 32;
         const int s1 = static_cast<int>((both >> 4) | (((scales_h >> (4 * g + 2)) & 3u) << 4)) - 32;
         const uint32_t w0[4] = {q0.x, q0.y, q0.z, q0.w}, w1[4] = {q1.x, q1.y, q1.z, q1.w};
-        const uint32_t a0[4] = {act.a[0].x, act.a[0].y, act.a[0].z, act.a[0].w};
-        const uint32_t a1[4] = {act.a[1].x, act.a[1].y, act.a[1].z, act.a[1].w};
-        const uint32_t a2[4] = {act.a[2].x, act.a[2].y, act.a[2].z, act.a[2].w};
-        const uint32_t a3[4] = {act.a[3].x, act.a[3].y, act.a[3].z, act.a[3].w};
-        int d0 = 0, d1 = 0;
+        int d0[kT], d1[kT];
+#pragma unroll
+        for (int t = 0; t < kT; t++) d0[t] = d1[t] = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             // byte j of the group: element j (low nibble) and element 16 + j (high nibble)
-            d0 = dot4(iq4nl_lookup(w0[i] & 0x0f0f0f0fu), a0[i], d0);
-            d0 = dot4(iq4nl_lookup((w0[i] >> 4) & 0x0f0f0f0fu), a1[i], d0);
-            d1 = dot4(iq4nl_lookup(w1[i] & 0x0f0f0f0fu), a2[i], d1);
-            d1 = dot4(iq4nl_lookup((w1[i] >> 4) & 0x0f0f0f0fu), a3[i], d1);
+            const uint32_t c00 = iq4nl_lookup(w0[i] & 0x0f0f0f0fu), c01 = iq4nl_lookup((w0[i] >> 4) & 0x0f0f0f0fu);
+            const uint32_t c10 = iq4nl_lookup(w1[i] & 0x0f0f0f0fu), c11 = iq4nl_lookup((w1[i] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int t = 0; t < kT; t++) {
+                const uint32_t a0[4] = {act[t].a[0].x, act[t].a[0].y, act[t].a[0].z, act[t].a[0].w};
+                const uint32_t a1[4] = {act[t].a[1].x, act[t].a[1].y, act[t].a[1].z, act[t].a[1].w};
+                const uint32_t a2[4] = {act[t].a[2].x, act[t].a[2].y, act[t].a[2].z, act[t].a[2].w};
+                const uint32_t a3[4] = {act[t].a[3].x, act[t].a[3].y, act[t].a[3].z, act[t].a[3].w};
+                d0[t] = dot4(c00, a0[i], d0[t]);
+                d0[t] = dot4(c01, a1[i], d0[t]);
+                d1[t] = dot4(c10, a2[i], d1[t]);
+                d1[t] = dot4(c11, a3[i], d1[t]);
+            }
         }
-        return f16_bits_to_f32(hdr.x) * act.dx * static_cast<float>(d0 * s0 + d1 * s1);
+        const float d = f16_bits_to_f32(hdr.x);
+#pragma unroll
+        for (int t = 0; t < kT; t++) res[t] = d * act[t].dx * static_cast<float>(d0[t] * s0 + d1[t] * s1);
     }
 };
 
@@ -286,10 +330,13 @@ struct DqIQ4XS {  // {f16 d, u16 scales_h, u8 scales_l[4], u8 qs[128]}: byte j o
 
 constexpr int kIqWaves = 4;
 
-template <uint32_t kQuant>
+// kTokens tokens per pass over the matrix (grid.y = token groups; the last group's spare slots repeat the last token and
+// are not stored): a block's codes are looked up and signed once and dotted against every token of the group, which is
+// most of the work of these formats; per token the one-token arithmetic, so the same bits.
+template <uint32_t kQuant, int kTokens>
 __global__ void __launch_bounds__(kWave *kIqWaves)
     gemv_iq_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                   float *__restrict__ out, uint32_t rows, uint32_t nb) {
+                   float *__restrict__ out, uint32_t rows, uint32_t nb, uint32_t seq) {
     // the format's grid goes to LDS once per workgroup: the look-ups are gathers, which LDS serves faster than the vector cache
     __shared__ __attribute__((aligned(16))) uint8_t s_table[Iq<kQuant>::kTableBytes > 0 ? Iq<kQuant>::kTableBytes : 16];
     if constexpr (Iq<kQuant>::kTableBytes > 0) {
@@ -300,26 +347,52 @@ __global__ void __launch_bounds__(kWave *kIqWaves)
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = threadIdx.x >> 6;
     const int g = lane & 3;
-    const uint32_t tok = blockIdx.y;
+    const uint32_t tok0 = blockIdx.y * kTokens;
     const size_t row_bytes = static_cast<size_t>(nb) * Iq<kQuant>::kBytes;
     const uint32_t n_waves = gridDim.x * kIqWaves;
     for (uint32_t row = blockIdx.x * kIqWaves + wave; row < rows; row += n_waves) {
-        float acc = 0.0f;
+        float acc[kTokens];
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) acc[t] = 0.0f;
         for (uint32_t b = lane >> 2; b < nb; b += 16) {
-            const size_t ab = static_cast<size_t>(tok) * nb + b;
-            const IqAct act = iq_load_act(aq + ab * 256, ad[ab], g);
-            acc += Iq<kQuant>::partial(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * Iq<kQuant>::kBytes, act, g, s_table);
+            IqAct act[kTokens];
+#pragma unroll
+            for (int t = 0; t < kTokens; t++) {
+                const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
+                const size_t ab = static_cast<size_t>(tok) * nb + b;
+                act[t] = iq_load_act(aq + ab * 256, ad[ab], g);
+            }
+            float part[kTokens];
+            Iq<kQuant>::template partial<kTokens>(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * Iq<kQuant>::kBytes,
+                                                  act, g, s_table, part);
+#pragma unroll
+            for (int t = 0; t < kTokens; t++) acc[t] += part[t];
         }
-        acc = seg_sum<kWave>(acc);
-        if (lane == kWave - 1) out[static_cast<size_t>(tok) * rows + row] = acc;
+#pragma unroll
+        for (int t = 0; t < kTokens; t++) {
+            const float sum = seg_sum<kWave>(acc[t]);
+            if (lane == kWave - 1 && tok0 + t < seq) out[static_cast<size_t>(tok0 + t) * rows + row] = sum;
+        }
     }
 }
 
 template <uint32_t kQuant>
 void launch_iq(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq, hipStream_t stream) {
     const uint32_t want = (rows + kIqWaves - 1) / kIqWaves;
-    const dim3 grid(want < 1024 ? want : 1024, seq, 1);  // 4096 waves; every workgroup stages the grid once
-    hipLaunchKernelGGL((gemv_iq_kernel<kQuant>), grid, dim3(kWave * kIqWaves), 0, stream, w, act.qs, act.d, out, rows, nb);
+    // groups of equal size, at most four tokens each
+    const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+    const dim3 grid(want < 1024 ? want : 1024, groups, 1);  // 4096 waves; every workgroup stages the grid once
+#define RNB_LAUNCH_IQ(T) \
+    hipLaunchKernelGGL((gemv_iq_kernel<kQuant, T>), grid, dim3(kWave * kIqWaves), 0, stream, w, act.qs, act.d, out, rows, nb, seq)
+    if (per == 1)
+        RNB_LAUNCH_IQ(1);
+    else if (per == 2)
+        RNB_LAUNCH_IQ(2);
+    else if (per == 3)
+        RNB_LAUNCH_IQ(3);
+    else
+        RNB_LAUNCH_IQ(4);
+#undef RNB_LAUNCH_IQ
 }
 
 // ---------------------------------------------------------------------------------------------

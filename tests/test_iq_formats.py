@@ -37,11 +37,12 @@ def test_iq_gemv_against_oracle(rnb, oracle, quant, rows, cols):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("quant", [IQ2_XXS, IQ2_S, IQ3_XXS, IQ4_XS])
-@pytest.mark.parametrize("seq", [2, 5, 33])
+@pytest.mark.parametrize("seq", [2, 3, 4, 5, 33])
 def test_iq_gemv_batch_layout(rnb, oracle, quant, seq):
-    """Batch form: out[s * rows + r] (crates/rnb-cpu/src/gemm/quant_gemv.rs:1185-1196).  Below four tokens every token's
-    row equals the one-token call bit for bit (same kernel, one grid row per token); from four on the batch runs on the
-    matrix cores (integer group sums, one f32 update per block) and agrees to rounding."""
+    """Batch form: out[s * rows + r] (crates/rnb-cpu/src/gemm/quant_gemv.rs:1185-1196).  Up to four tokens every token's
+    row equals the one-token call bit for bit (the GEMV decodes a block once and dots it against each token of the group
+    with the one-token arithmetic); from five on the batch runs on the matrix cores (integer group sums, one f32 update
+    per block) and agrees to rounding."""
     rows, cols = 203, 1024
     w = oracle.make_weights(quant, rows, cols, 800 + quant)
     x = oracle.fill_normal(seq * cols, 900 + seq, 1.0)
@@ -50,7 +51,7 @@ def test_iq_gemv_batch_layout(rnb, oracle, quant, seq):
     _check(got, oracle.gemv(quant, w, rows, cols, x), oracle.gemv(quant, w, rows, cols, x, gold=True), f"{LABEL[quant]} batch {seq}")
     for s in (0, seq - 1):
         alone = one(w, rows, cols, x[s * cols:(s + 1) * cols])
-        if seq < 4:
+        if seq < 5:
             assert np.array_equal(got[s], alone)
         else:
             assert np.abs(got[s] - alone).max() <= 1e-5 * np.abs(alone).max()
@@ -59,10 +60,10 @@ def test_iq_gemv_batch_layout(rnb, oracle, quant, seq):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("quant", [IQ2_XXS, IQ2_S, IQ3_XXS, IQ4_XS])
-@pytest.mark.parametrize("rows,cols,seq", [(203, 1024, 4), (130, 256, 33), (129, 4096, 65), (4096, 2048, 96), (37, 14336, 17),
+@pytest.mark.parametrize("rows,cols,seq", [(203, 1024, 5), (130, 256, 33), (129, 4096, 65), (4096, 2048, 96), (37, 14336, 17),
                                            (300, 768, 512), (8192, 512, 500)])
 def test_iq_gemm_matrix_cores(rnb, oracle, quant, rows, cols, seq):
-    """Batches of four tokens and more: ragged row and token tiles, 32- and 64-token workgroups (8192 rows x 500 tokens),
+    """Batches of five tokens and more: ragged row and token tiles, 32- and 64-token workgroups (8192 rows x 500 tokens),
     K cut into slices on small grids (37 rows x 56 blocks: sixteen slices)."""
     w = oracle.make_weights(quant, rows, cols, 1200 + quant + rows)
     x = oracle.fill_normal(seq * cols, 1300 + seq, 1.0)
