@@ -499,12 +499,15 @@ def test_q5k_gemm_extreme_blocks(rnb, oracle):
                                                  (Q6_K, 4096, 5120, 6), (Q6_K, 4096, 5120, 7), (Q8_0, 4096, 4096, 6),
                                                  (Q8_0, 4096, 4096, 7), (Q8_1, 4096, 4096, 15), (Q4_K, 4096, 4096, 6),
                                                  (Q4_K, 4096, 4096, 8), (Q6_K, 2048, 4096, 8), (Q6_K, 2048, 4096, 11),
-                                                 (Q4_0, 4096, 4096, 8), (Q4_0, 4096, 4096, 9), (Q2_K, 8192, 4096, 7)])
+                                                 (Q4_0, 4096, 4096, 8), (Q4_0, 4096, 4096, 9), (Q2_K, 8192, 4096, 7),
+                                                 (Q3_K, 8192, 4096, 9), (Q5_K, 6144, 4096, 12), (Q4_K, 8192, 4096, 12),
+                                                 (Q5_1, 4096, 4096, 13)])
 def test_gemm_few_tokens(rnb, oracle, quant, rows, cols, seq):
     """Either side of the token count at which a format's matrix-core GEMM takes over from the GEMV kernels that keep two
     to four tokens in registers (5 for Q4_K / Q5_K, 7 for Q6_K, Q2_K, Q3_K, Q8_0, Q8_1, 9 for the nibble formats; two more
     under 16 MB): on the GEMV side groups of 4, 3 + 3, 4 + 4 tokens, on the GEMM side a 32-token tile mostly empty (loads
-    of the missing tokens repeat the last one, their results are not stored)."""
+    of the missing tokens repeat the last one, their results are not stored; up to 8 / 16 tokens the kernels that finish
+    only the first 4 / 8 results of a lane)."""
     w = oracle.make_weights(quant, rows, cols, 1200 + seq)
     x = oracle.fill_normal(seq * cols, 1210 + seq, 1.0)
     got = gemv_fn(rnb, quant, batch=True)(w, rows, cols, x)
