@@ -17,8 +17,8 @@
 //   Q2_K Q3_K   Q6_K's scheme; Q2_K's mins term through two K=16 instructions over the sub-block sums' digits:
 //          crates/rnb-cpu/src/gemm/avx2_dot.rs:169-242 (Q2_K), :247-375 (Q3_K).
 // That is 16 (Q6_K) or 48 (Q8) vector instructions per matrix instruction, so these kernels are bound by the vector
-// port, not the matrix pipe; they replace one GEMV pass per token (Q8) or the integer-dot multi-token kernel (Q5_K,
-// Q6_K), which measured 9 to 17 times slower at 512 tokens.
+// port, not the matrix pipe; at 512 tokens they measured 9 to 17 times faster than GEMV passes over the tokens on the
+// vector units' integer dots.
 //
 // Tiling: workgroup = 4 waves = 128 weight rows x kTT*32 tokens; a wave owns 32 rows and all the workgroup's tokens.
 // MFMA "M" = token, "N" = weight row: a lane's 16 results belong to ONE row (lane % 32), so that row's scales are

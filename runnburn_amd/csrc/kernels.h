@@ -46,7 +46,8 @@ void launch_gemv_q4k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q5k(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb,
                      uint32_t seq, hipStream_t stream);
-// IQ2_XXS / IQ2_S / IQ3_XXS / IQ4_XS rows (2-byte aligned blocks) against Q8_K activations, one grid row per token
+// IQ2_XXS / IQ2_S / IQ3_XXS / IQ4_XS rows (2-byte aligned blocks) against Q8_K activations, a grid row per group of up
+// to four tokens
 bool is_iq_quant(uint32_t quant);
 void launch_gemv_iq(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq,
                     hipStream_t stream);
