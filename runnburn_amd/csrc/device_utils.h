@@ -25,6 +25,16 @@ __device__ __forceinline__ uint4 ld_u4_a2(const uint8_t *p) { return *reinterpre
 __device__ __forceinline__ uint2 ld_u2_a2(const uint8_t *p) { return *reinterpret_cast<const uint2_a2 *>(p); }
 __device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) { return *reinterpret_cast<const uint32_a2 *>(p); }
 
+// A batch of `seq` tokens cut into groups of equal size, at most four tokens each (the multi-token GEMV kernels keep a
+// group's activation slices in registers and make one pass over the matrix per group): 5 -> 3 + 2, 7 -> 4 + 3, 8 -> 4 + 4.
+struct TokenGroups {
+    uint32_t groups, per;
+};
+inline TokenGroups token_groups(uint32_t seq) {
+    const uint32_t groups = (seq + 3) / 4;
+    return {groups, groups ? (seq + groups - 1) / groups : 0};
+}
+
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(bits & 0xffffu)));
 }

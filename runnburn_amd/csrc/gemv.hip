@@ -375,7 +375,7 @@ void launch_gate_up(const uint8_t *wg, const uint8_t *wu, ActView act, float *mi
     const uint32_t row_groups = (rows + kRowsPerWave - 1) / kRowsPerWave;
     const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
     // groups of equal size, at most four tokens each
-    const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+    const auto [groups, per] = token_groups(seq);
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
 #define RNB_LAUNCH_GU(GELU, T)                                                                                              \
     hipLaunchKernelGGL((gemv_q4k_gate_up_kernel<kRowsPerWave, GELU, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, wg, wu, \
@@ -733,7 +733,7 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
     const uint32_t row_chunks = (rows + kSplitRows - 1) / kSplitRows;
     const uint32_t want = kTargetWaves / n_slices;  // workgroups for about kTargetWaves waves
     if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
-        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const auto [groups, per] = token_groups(seq);
         const dim3 tgrid(rows < want ? rows : want, groups, 1);
 #define RNB_LAUNCH_TOKENS(T)                                                                                                  \
     hipLaunchKernelGGL((gemv_kquant_splitk_tokens_kernel<kQuant, T>), tgrid, dim3(kWave * n_slices), 0, stream, w, act.qs, act.d, \
@@ -868,7 +868,7 @@ void launch_kquant(const uint8_t *w, ActView act, float *out, uint32_t rows, uin
     // several tokens per pass over the matrix, in groups of equal size (at most four); rows longer than one wave pass
     // (only reached beyond the K-split kernel's 256 super-blocks) keep one pass per token
     if (seq >= 2 && nb <= static_cast<uint32_t>(kWave / kRowsPerWave / 4)) {
-        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const auto [groups, per] = token_groups(seq);
         const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
 #define RNB_LAUNCH_TOKENS(T)                                                                                                 \
     hipLaunchKernelGGL((gemv_kquant_tokens_kernel<kQuant, kRowsPerWave, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, \
@@ -895,7 +895,7 @@ void launch_kquant_chunks(const uint8_t *w, ActView act, float *out, uint32_t ro
     const uint32_t n_chunks = (rows + kRows - 1) / kRows;
     const uint32_t waves = n_chunks < kChunkMaxWaves ? n_chunks : kChunkMaxWaves;
     if (seq >= 2) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
-        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const auto [groups, per] = token_groups(seq);
         const dim3 tgrid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
 #define RNB_LAUNCH_TOKENS(T)                                                                                                  \
     hipLaunchKernelGGL((gemv_kquant_chunks_tokens_kernel<kQuant, kRows, T>), tgrid, dim3(kWave * kWavesPerWg), 0, stream, w,  \
@@ -1239,7 +1239,7 @@ void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, ui
                     hipStream_t stream) {
     const uint32_t waves = rows < kTargetWaves ? rows : kTargetWaves;
     if (seq >= 2 && nb32 <= 2 * kWave) {  // several tokens per pass over the matrix, in groups of equal size (at most four)
-        const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+        const auto [groups, per] = token_groups(seq);
         const dim3 tgrid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, 1);
         bool paired = false;
         if constexpr (block32_pairs<kQuant>()) paired = nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0;

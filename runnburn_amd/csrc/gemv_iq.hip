@@ -380,7 +380,7 @@ template <uint32_t kQuant>
 void launch_iq(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb, uint32_t seq, hipStream_t stream) {
     const uint32_t want = (rows + kIqWaves - 1) / kIqWaves;
     // groups of equal size, at most four tokens each
-    const uint32_t groups = (seq + 3) / 4, per = (seq + groups - 1) / groups;
+    const auto [groups, per] = token_groups(seq);
     const dim3 grid(want < 1024 ? want : 1024, groups, 1);  // 4096 waves; every workgroup stages the grid once
 #define RNB_LAUNCH_IQ(T) \
     hipLaunchKernelGGL((gemv_iq_kernel<kQuant, T>), grid, dim3(kWave * kIqWaves), 0, stream, w, act.qs, act.d, out, rows, nb, seq)
