@@ -10,6 +10,7 @@
 //   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
 //   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
 //   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
+//   q8_0_head_gemv_batch                        quant_api.rs:824-882
 //   q6k_gemv_argmax / q8_0_gemv_argmax          quant_api.rs:2170-2204, 733-768
 //   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
 //   dense_q4k_silu_ffn_batch                    api/dense_api.rs:297-337
@@ -176,6 +177,15 @@ inline Result<std::vector<float>> q8_0_gemv(Bytes weights, size_t rows, size_t c
 }
 inline Result<std::vector<float>> q8_0_gemv_batch(Bytes weights, size_t rows, size_t cols, Floats input) {
     return gemv_impl(rnb_hip_q8_0_gemv_batch, weights, rows, cols, input, batch_seq(input, cols) * rows);
+}
+// q8_0_head_gemv_batch(weights, head_count, rows_per_head, cols, token_count, input), quant_api.rs:824-882
+inline Result<std::vector<float>> q8_0_head_gemv_batch(Bytes weights, size_t head_count, size_t rows_per_head, size_t cols,
+                                                       size_t token_count, Floats input) {
+    std::vector<float> out(token_count * head_count * rows_per_head);
+    const int st = rnb_hip_q8_0_head_gemv_batch(weights.ptr, weights.len, head_count, rows_per_head, cols, token_count,
+                                                input.ptr, input.len, out.data(), out.size());
+    if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);
+    return make_ok(std::move(out));
 }
 
 // prewarm_q4k_weights(&[&[u8]]), quant_api.rs:952

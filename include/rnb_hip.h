@@ -234,6 +234,13 @@ int rnb_hip_q8_0_gemv(const uint8_t *w, size_t w_len, size_t rows, size_t cols, 
 /* q8_0_gemv_batch, quant_api.rs:807-822 */
 int rnb_hip_q8_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t cols,
                             const float *x, size_t x_len, float *out, size_t out_len);
+/* q8_0_head_gemv_batch(weights, head_count, rows_per_head, cols, token_count, input) -> Vec<f32>, quant_api.rs:824-882
+ * (the per-head projections of the GLM MLA path, crates/rnb-llm/src/engine/models/glm_dsa.rs:95-122): weights
+ * [head_count][rows_per_head][cols / 32 blocks of 34 bytes], x [token_count][head_count][cols], out
+ * [token_count][head_count * rows_per_head].  Every (token, head) group is the Q8_0 GEMV of that head's rows on that
+ * vector (Q8 x Q8_0 integer dots, the bits of rnb_hip_q8_0_gemv on the head's sub-matrix); cols <= 4096. */
+int rnb_hip_q8_0_head_gemv_batch(const uint8_t *w, size_t w_len, size_t head_count, size_t rows_per_head, size_t cols,
+                                 size_t token_count, const float *x, size_t x_len, float *out, size_t out_len);
 
 /* qwen35_sparse_experts_selected_base_by_token, crates/rnb-backend/cuda/src/runtime/api/
  * qwen_moe_api.rs:2529-2541 (validation: runtime/helpers.rs:1496-1600, 2747-2800): whole-layer

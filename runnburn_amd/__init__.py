@@ -13,6 +13,7 @@ functions keep the reference's names, argument meaning and error behaviour:
   q5k_gemv / q5k_gemv_into / q5k_gemv_batch   quant_api.rs:2207-2281, 3957-3993
   q6k_gemv / q6k_gemv_into / q6k_gemv_batch   quant_api.rs:2071-2168, 3919-3955
   q8_0_gemv / q8_0_gemv_batch                 quant_api.rs:498-505, 807-822
+  q8_0_head_gemv_batch                        quant_api.rs:824-882
   qwen35_sparse_experts_selected_base_by_token  api/qwen_moe_api.rs:2529-2541
   HipBackend                                  crates/rnb-backend/api/src/lib.rs:1281-1285 (trait Backend)
 
@@ -110,6 +111,7 @@ from .binding import (  # noqa: F401
     q8_0_gemv_argmax,
     q8_0_gemv,
     q8_0_gemv_batch,
+    q8_0_head_gemv_batch,
     quantize_input_q8,
     quantize_input_q8k,
     qwen35_sparse_experts_selected_base_by_token,

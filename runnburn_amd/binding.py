@@ -74,6 +74,7 @@ SYMBOLS = [
     ("rnb_hip_q6k_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q8_0_gemv", _i, _MATMUL_ARGS),
     ("rnb_hip_q8_0_gemv_batch", _i, _MATMUL_ARGS),
+    ("rnb_hip_q8_0_head_gemv_batch", _i, [_vp, _sz, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_moe_sparse_experts_by_token", _i,
      [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dev_alloc", _vp, [_sz]),
@@ -461,6 +462,16 @@ def q8_0_gemv(weights, rows, cols, input):  # noqa: A002
 
 def q8_0_gemv_batch(weights, rows, cols, input):  # noqa: A002
     return _gemv_batch("rnb_hip_q8_0_gemv_batch", weights, rows, cols, input)
+
+
+def q8_0_head_gemv_batch(weights, head_count: int, rows_per_head: int, cols: int, token_count: int, input) -> np.ndarray:  # noqa: A002
+    """quant_api.rs:824-882: weights [head][rows_per_head][cols], input [token][head][cols]; returns
+    out[token][head_count * rows_per_head]."""
+    w, x = _bytes_view(weights), _f32(input).ravel()
+    out = np.empty((token_count, head_count * rows_per_head), dtype=np.float32)
+    _check(lib().rnb_hip_q8_0_head_gemv_batch(_ptr(w), w.size, head_count, rows_per_head, cols, token_count, _ptr(x), x.size,
+                                              _ptr(out), out.size))
+    return out
 
 
 def qwen35_sparse_experts_selected_base_by_token(gate_all, up_all, down_all, expert_ids, route_weights, token_ids,

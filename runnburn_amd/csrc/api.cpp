@@ -1045,6 +1045,69 @@ int rnb_hip_q8_0_gemv_batch(const uint8_t *w, size_t w_len, size_t rows, size_t 
     return matmul_host(kQ8_0, w, w_len, rows, cols, x, x_len, out, out_len, true);
 }
 
+// q8_0_head_gemv_batch, crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:824-882 (checks and texts in its order):
+// head h has its own rows_per_head rows, token t's input for it is x[(t * head_count + h) * cols ..], out is
+// [token][head_count * rows_per_head].  Every (token, head) group is the Q8_0 GEMV on that head's rows.
+int rnb_hip_q8_0_head_gemv_batch(const uint8_t *w, size_t w_len, size_t head_count, size_t rows_per_head, size_t cols,
+                                 size_t token_count, const float *x, size_t x_len, float *out, size_t out_len) {
+    if (head_count == 0 || rows_per_head == 0 || token_count == 0)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch dimensions must be non-zero: heads=" + std::to_string(head_count) +
+                                                 " rows_per_head=" + std::to_string(rows_per_head) +
+                                                 " tokens=" + std::to_string(token_count));
+    if (cols == 0 || cols % 32 != 0)
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    "Q8_0 head batch cols must be non-zero and divisible by 32, got " + std::to_string(cols));
+    const size_t nb32 = cols / 32;
+    size_t rows = 0, blocks = 0, expected_w = 0;
+    if (__builtin_mul_overflow(head_count, rows_per_head, &rows) || __builtin_mul_overflow(rows, nb32, &blocks) ||
+        __builtin_mul_overflow(blocks, size_t(34), &expected_w))
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch weight byte size overflow");
+    if (w_len != expected_w)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch weight byte mismatch: got " + std::to_string(w_len) +
+                                                 ", expected " + std::to_string(expected_w));
+    size_t vecs = 0, expected_x = 0;
+    if (__builtin_mul_overflow(token_count, head_count, &vecs) || __builtin_mul_overflow(vecs, cols, &expected_x))
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch input length overflow");
+    if (x_len != expected_x)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch input length mismatch: got " + std::to_string(x_len) +
+                                                 ", expected " + std::to_string(expected_x));
+    size_t n_out = 0;
+    if (__builtin_mul_overflow(token_count, rows, &n_out) || out_len < n_out)
+        return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch output too small: got " + std::to_string(out_len) +
+                                                 ", expected >= " + std::to_string(token_count) + " x " + std::to_string(rows));
+    if (!w || !x || !out) return fail(RNB_HIP_INVALID_REQUEST, "Q8_0 head batch null pointer argument");
+    if (!gemv_q8_0_heads_supported(static_cast<uint32_t>(nb32 > 0xffffffffu ? 0xffffffffu : nb32)) || head_count > 65535 ||
+        rows_per_head > 0x7fffffffu || token_count > 262140u)
+        return fail(RNB_HIP_UNSUPPORTED_OP, "Q8_0 head batch shape not supported: cols=" + std::to_string(cols) + " heads=" +
+                                                std::to_string(head_count) + " tokens=" + std::to_string(token_count) +
+                                                " (cols <= 4096, heads <= 65535, tokens <= 262140)");
+    Guard g;
+    if (!g.state) return g.status;
+    State &s = *g.state;
+    const uint8_t *w_dev = nullptr;
+    if (int rs = s.resident_ptr(w, w_len, &w_dev); rs != RNB_HIP_OK) return rs;
+    const size_t in_bytes = expected_x * sizeof(float), out_bytes = n_out * sizeof(float);
+    RESERVE_TRY(s.bounce_in, in_bytes);
+    RESERVE_TRY(s.bounce_out, out_bytes);
+    HIP_TRY(s.x_f32.reserve(in_bytes));
+    HIP_TRY(s.out_f32.reserve(out_bytes));
+    std::memcpy(s.bounce_in.ptr, x, in_bytes);
+    HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, in_bytes, hipMemcpyHostToDevice, s.stream));
+    s.h2d_bytes += in_bytes;
+    ActView act;
+    // every (token, head) vector is quantised as a row of its own: token_count * head_count rows of cols
+    if (int st = quantize_activations(s, kQ8_0, s.x_f32.as<float>(), vecs, cols, &act); st != RNB_HIP_OK) return st;
+    launch_gemv_q8_0_heads(w_dev, act, s.out_f32.as<float>(), static_cast<uint32_t>(head_count),
+                           static_cast<uint32_t>(rows_per_head), static_cast<uint32_t>(nb32), static_cast<uint32_t>(token_count),
+                           s.stream);
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
+    HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, out_bytes, hipMemcpyDeviceToHost, s.stream));
+    HIP_TRY(hipStreamSynchronize(s.stream));
+    s.d2h_bytes += out_bytes;
+    std::memcpy(out, s.bounce_out.ptr, out_bytes);
+    return RNB_HIP_OK;
+}
+
 int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len, const uint8_t *up_all,
                                         size_t up_len, const uint8_t *down_all, size_t down_len,
                                         const uint32_t *expert_ids, const float *route_weights,

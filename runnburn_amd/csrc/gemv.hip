@@ -1189,6 +1189,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // Two to four tokens per pass over the matrix, rows of at most 128 blocks (the register-resident branches of
 // gemv_block32_kernel): a lane keeps its two activation blocks of kTokens tokens and dots each fetched weight block
 // against all of them; per token the same expression as the one-token kernel (same bits).  grid.y = token groups.
+// grid.z = heads (1 for a plain matrix): head z has its own `rows` rows of weights, reads activation row tok * heads + z
+// and writes out[tok][z * rows + row], the per-head projections of q8_0_head_gemv_batch.
 template <uint32_t kQuant, bool kPaired, int kTokens>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_block32_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
@@ -1196,7 +1198,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
     constexpr bool kSum = kQuant != kQ8_0 && kQuant != kQ8_1;
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t tok0 = blockIdx.y * kTokens;
+    const uint32_t tok0 = blockIdx.y * kTokens, heads = gridDim.z, head = blockIdx.z;
     const size_t row_bytes = static_cast<size_t>(nb32) * kBlockBytes;
     const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     const uint32_t n_waves = gridDim.x * kWavesPerWg;
@@ -1206,12 +1208,12 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 #pragma unroll
     for (int t = 0; t < kTokens; t++) {
         const uint32_t tok = tok0 + t < seq ? tok0 + t : seq - 1;
-        const size_t abase = static_cast<size_t>(tok) * nb32;
+        const size_t abase = (static_cast<size_t>(tok) * heads + head) * nb32;
         a0[t] = q8_load_act<kSum>(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
         a1[t] = q8_load_act<kSum>(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
     }
     for (uint32_t row = wave_global; row < rows; row += n_waves) {
-        const uint8_t *rowp = w + static_cast<size_t>(row) * row_bytes;
+        const uint8_t *rowp = w + (static_cast<size_t>(head) * rows + row) * row_bytes;
         Block32Regs c0 = Block32Regs{}, c1 = Block32Regs{};
         if constexpr (kPaired) {
             if (has0) block32_load_pair<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes, c0, c1);
@@ -1229,7 +1231,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
                 if (has1) acc += block32_dot<kQuant>(c1, a1[t]);
             }
             acc = seg_sum<kWave>(acc);
-            if (lane == kWave - 1 && tok0 + t < seq) out[static_cast<size_t>(tok0 + t) * rows + row] = acc;
+            if (lane == kWave - 1 && tok0 + t < seq) out[(static_cast<size_t>(tok0 + t) * heads + head) * rows + row] = acc;
         }
     }
 }
@@ -1276,6 +1278,36 @@ void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, ui
     }
     hipLaunchKernelGGL((gemv_block32_kernel<kQuant, false>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, act.d, out,
                        rows, nb32);
+}
+
+// Per-head Q8_0 projections of a token batch: weights [heads][rows_per_head][nb32 blocks], activations (32-wide Q8)
+// [tokens][heads][nb32], out [tokens][heads * rows_per_head]; rows of at most 128 blocks.
+void launch_heads_q8_0(const uint8_t *w, ActView act, float *out, uint32_t heads, uint32_t rows_per_head, uint32_t nb32,
+                       uint32_t tokens, hipStream_t stream) {
+    const uint32_t waves = rows_per_head < kTargetWaves ? rows_per_head : kTargetWaves;
+    const auto [groups, per] = token_groups(tokens);
+    const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, heads);
+    const bool paired = nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0;
+#define RNB_LAUNCH_HEADS(P, T)                                                                                             \
+    hipLaunchKernelGGL((gemv_block32_tokens_kernel<kQ8_0, P, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, \
+                       act.d, out, rows_per_head, nb32, tokens)
+#define RNB_LAUNCH_HEADS_P(P)      \
+    do {                           \
+        if (per == 1)              \
+            RNB_LAUNCH_HEADS(P, 1); \
+        else if (per == 2)         \
+            RNB_LAUNCH_HEADS(P, 2); \
+        else if (per == 3)         \
+            RNB_LAUNCH_HEADS(P, 3); \
+        else                       \
+            RNB_LAUNCH_HEADS(P, 4); \
+    } while (0)
+    if (paired)
+        RNB_LAUNCH_HEADS_P(true);
+    else
+        RNB_LAUNCH_HEADS_P(false);
+#undef RNB_LAUNCH_HEADS_P
+#undef RNB_LAUNCH_HEADS
 }
 
 // One f32 token against rows of at most 128 blocks: the workgroup quantises the token to 32-wide Q8 in LDS itself
@@ -1430,6 +1462,14 @@ void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, fl
     case kQ5K: launch_kquant_f32_any<kQ5K>(w, x, out, rows, nb, seq, stream); break;
     default: launch_kquant_f32_any<kQ6K>(w, x, out, rows, nb, seq, stream); break;
     }
+}
+
+bool gemv_q8_0_heads_supported(uint32_t nb32) { return nb32 >= 1 && nb32 <= 2 * kWave; }
+
+void launch_gemv_q8_0_heads(const uint8_t *w, ActView act, float *out, uint32_t heads, uint32_t rows_per_head, uint32_t nb32,
+                            uint32_t tokens, hipStream_t stream) {
+    if (heads == 0 || rows_per_head == 0 || tokens == 0) return;
+    launch_heads_q8_0(w, act, out, heads, rows_per_head, nb32, tokens, stream);
 }
 
 bool gemv_q4k_gate_up_supported(uint32_t nb) { return nb >= 1 && nb <= 16; }

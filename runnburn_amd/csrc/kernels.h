@@ -89,6 +89,12 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
                      uint32_t seq, hipStream_t stream);
 void launch_gemv_q8_0(const uint8_t *w, ActView act, float *out, uint32_t rows, uint32_t nb32,
                       uint32_t seq, hipStream_t stream);
+// Per-head Q8_0 projections (q8_0_head_gemv_batch): weights [heads][rows_per_head][nb32 blocks of 34 bytes], 32-wide Q8
+// activations [tokens][heads][nb32 * 32], out [tokens][heads * rows_per_head]; rows of at most 128 blocks; grid.z = heads
+// (at most 65535), every (token, head) row group has the bits of launch_gemv_q8_0 on that head's rows
+bool gemv_q8_0_heads_supported(uint32_t nb32);
+void launch_gemv_q8_0_heads(const uint8_t *w, ActView act, float *out, uint32_t heads, uint32_t rows_per_head, uint32_t nb32,
+                            uint32_t tokens, hipStream_t stream);
 // any 32-element format (kQ4_0, kQ4_1, kQ5_0, kQ5_1, kQ8_0, kQ8_1) against 32-wide Q8 activations
 void launch_gemv_block32(const uint8_t *w, uint32_t quant, ActView act, float *out, uint32_t rows, uint32_t nb32,
                          uint32_t seq, hipStream_t stream);

@@ -50,6 +50,8 @@ static int validate() {
     EXPECT(!r && r.error == "Q5_K weight byte mismatch: got 144, expected 176", "q5k weight bytes message");
     r = q8_0_gemv_batch({w.data(), 34}, 1, 32, {x.data(), 33});
     EXPECT(!r && r.error == "Q8_0 batch input length 33 is not divisible by cols 32", "q8_0 batch message");
+    r = q8_0_head_gemv_batch({w.data(), 34}, 1, 1, 32, 2, {x.data(), 63});
+    EXPECT(!r && r.error == "Q8_0 head batch input length mismatch: got 63, expected 64", "q8_0 head batch message");
     float out1 = 0;
     auto u = q4k_gemv_into({w.data(), 144}, 1, 256, {x.data(), 256}, &out1, 0);
     EXPECT(!u && u.error == "Q4_K shape mismatch: input=256 output=0 expected input=256 output>=1", "into message");
@@ -123,6 +125,26 @@ static void run_case(const std::string &dir, const char *name, size_t rows, size
     std::printf("%s: %zu outputs, max |diff| %.3g (rms %.3g)\n", name, want.size(), worst, rms);
 }
 
+// the golden Q8_0 batch read as a head batch: its 7 rows as one head, and as 7 heads of one row fed the same vector
+static void head_case(const std::string &dir) {
+    const size_t rows = 7, cols = 96, seq = 4;
+    const auto w = read_file<uint8_t>(dir + "/q8_0_batch_w.bin");
+    const auto x = read_file<float>(dir + "/q8_0_batch_x.bin");
+    const auto want = read_file<float>(dir + "/q8_0_batch_out.bin");
+    if (w.empty() || x.empty() || want.size() != seq * rows) return;
+    auto plain = q8_0_gemv_batch({w.data(), w.size()}, rows, cols, {x.data(), x.size()});
+    auto one = q8_0_head_gemv_batch({w.data(), w.size()}, 1, rows, cols, seq, {x.data(), x.size()});
+    std::vector<float> xr(seq * rows * cols);
+    for (size_t t = 0; t < seq; t++)
+        for (size_t h = 0; h < rows; h++) std::memcpy(&xr[(t * rows + h) * cols], &x[t * cols], cols * sizeof(float));
+    auto many = q8_0_head_gemv_batch({w.data(), w.size()}, rows, 1, cols, seq, {xr.data(), xr.size()});
+    EXPECT(plain && one && many, "head batch calls");
+    if (!(plain && one && many)) return;
+    EXPECT(std::memcmp(one.value.data(), plain.value.data(), want.size() * sizeof(float)) == 0, "one head == plain batch");
+    EXPECT(std::memcmp(many.value.data(), plain.value.data(), want.size() * sizeof(float)) == 0, "seven heads == plain batch");
+    std::printf("q8_0_head_gemv_batch: %zu outputs, both layouts bit-identical to q8_0_gemv_batch\n", want.size());
+}
+
 // rows [last, 0, 2, 2] of a golden weight file, dequantised on the device: bit-identical to the fixture
 static void embed_case(const std::string &dir, const char *name, uint32_t quant, size_t rows, size_t cols) {
     const auto w = read_file<uint8_t>(dir + "/" + name + "_w.bin");
@@ -174,6 +196,7 @@ int main(int argc, char **argv) {
         run_case(dir, "iq2_xxs_batch", 12, 512, 3, iq2_xxs_gemv_batch);
         run_case(dir, "iq3_xxs_gemv", 14, 512, 1, iq3_xxs_gemv);
         run_case(dir, "iq2_s_batch", 9, 256, 2, iq2_s_gemv_batch);
+        head_case(dir);
         embed_case(dir, "q4k_gemv", RNB_GGML_Q4_K, 24, 1024);
         embed_case(dir, "q6k_gemv", RNB_GGML_Q6_K, 20, 768);
         embed_case(dir, "q8_0_gemv", RNB_GGML_Q8_0, 16, 544);

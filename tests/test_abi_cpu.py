@@ -278,3 +278,22 @@ def test_embedding_gather_validation_messages_match_reference():
     assert str(e) == "BF16 embedding weight byte mismatch: got 770, expected 768"
     e = _err(rnb.quant_embedding_gather, 17, z(74 * 6, np.uint8), 6, 256, ids)
     assert e.kind == "UnsupportedOp"
+
+
+def test_q8_0_head_batch_validation_messages_match_reference():
+    """crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:832-866: dimensions, cols, weight bytes, input length, in
+    this order."""
+    z = np.zeros
+    e = _err(rnb.q8_0_head_gemv_batch, z(34, np.uint8), 0, 4, 32, 2, z(64, np.float32))
+    assert (e.kind, str(e)) == ("InvalidRequest", "Q8_0 head batch dimensions must be non-zero: heads=0 rows_per_head=4 tokens=2")
+    e = _err(rnb.q8_0_head_gemv_batch, z(34, np.uint8), 3, 4, 32, 0, z(0, np.float32))
+    assert str(e) == "Q8_0 head batch dimensions must be non-zero: heads=3 rows_per_head=4 tokens=0"
+    e = _err(rnb.q8_0_head_gemv_batch, z(34, np.uint8), 3, 4, 48, 2, z(288, np.float32))
+    assert str(e) == "Q8_0 head batch cols must be non-zero and divisible by 32, got 48"
+    e = _err(rnb.q8_0_head_gemv_batch, z(34, np.uint8), 3, 4, 0, 2, z(0, np.float32))
+    assert str(e) == "Q8_0 head batch cols must be non-zero and divisible by 32, got 0"
+    e = _err(rnb.q8_0_head_gemv_batch, z(3 * 4 * 3 * 34 - 1, np.uint8), 3, 4, 96, 3, z(3 * 3 * 96, np.float32))
+    assert str(e) == "Q8_0 head batch weight byte mismatch: got 1223, expected 1224"
+    e = _err(rnb.q8_0_head_gemv_batch, z(3 * 4 * 3 * 34, np.uint8), 3, 4, 96, 3, z(3 * 3 * 96 - 1, np.float32))
+    assert str(e) == "Q8_0 head batch input length mismatch: got 863, expected 864"
+

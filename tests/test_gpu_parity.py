@@ -900,6 +900,51 @@ def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
     assert idx2 == min(17, idx) and val2 == val
 
 
+# ---- per-head Q8_0 projections (crates/rnb-backend/cuda/src/runtime/api/quant_api.rs:824-882) ---------------------
+
+@pytest.mark.parametrize("heads,rows_per_head,cols,tokens", [(3, 4, 96, 3), (16, 128, 512, 5), (64, 512, 128, 9), (5, 33, 1056, 2),
+                                                             (1, 7, 4096, 1), (128, 64, 192, 6), (2, 300, 32, 4)])
+def test_q8_0_head_gemv_batch(rnb, oracle, heads, rows_per_head, cols, tokens):
+    """Every (token, head) group of the output is the Q8_0 GEMV of that head's rows on that token's vector for the head:
+    bit for bit the one-token operator on the head's sub-matrix (what the reference's per-head path computes,
+    crates/rnb-llm/src/engine/models/glm_dsa.rs:124-175), and within tolerance of the oracle; odd and even block counts
+    (single and paired block fetches), token groups of 1 to 4, one head and many."""
+    rows = heads * rows_per_head
+    w = oracle.make_weights(Q8_0, rows, cols, 600 + heads)
+    x = oracle.fill_normal(tokens * heads * cols, 601 + tokens, 1.0)
+    got = rnb.q8_0_head_gemv_batch(w, heads, rows_per_head, cols, tokens, x)
+    assert got.shape == (tokens, rows)
+    hb = rows_per_head * (cols // 32) * 34
+    xs = x.reshape(tokens, heads, cols)
+    for h in sorted({0, heads // 2, heads - 1}):
+        wh = w[h * hb:(h + 1) * hb].copy()
+        ref = oracle.gemv(Q8_0, wh, rows_per_head, cols, xs[:, h].copy())
+        gold = oracle.gemv(Q8_0, wh, rows_per_head, cols, xs[:, h].copy(), gold=True)
+        mine = got[:, h * rows_per_head:(h + 1) * rows_per_head]
+        check_close(mine, ref, gold, f"head batch head {h} of {heads}")
+        for t in sorted({0, tokens - 1}):
+            alone = rnb.q8_0_gemv(wh, rows_per_head, cols, xs[t, h].copy())
+            assert np.array_equal(alone.view(np.uint32), mine[t].view(np.uint32)), (h, t)
+        rnb.release(wh)
+    rnb.release(w)
+
+
+def test_q8_0_head_gemv_batch_reference_case(rnb, oracle):
+    """The reference's own case (crates/rnb-backend/cuda/src/runtime/tests.rs:21118-21155): 3 heads x 4 rows x 96 columns,
+    3 tokens, input ((i % 31) - 15) / 64, against dequantised weights times the f32 input (its cpu_q8_0_rows) within
+    its tolerance of 0.01."""
+    heads, rph, cols, tokens = 3, 4, 96, 3
+    w = oracle.make_weights(Q8_0, heads * rph, cols, 181)
+    x = (((np.arange(tokens * heads * cols) % 31).astype(np.float32)) - 15.0) * np.float32(0.015625)
+    got = rnb.q8_0_head_gemv_batch(w, heads, rph, cols, tokens, x)
+    hb = rph * (cols // 32) * 34
+    xs = x.reshape(tokens, heads, cols)
+    want = np.concatenate([oracle.gemv_q8_0_f32act(w[h * hb:(h + 1) * hb].copy(), rph, cols, xs[:, h].copy()) for h in range(heads)],
+                          axis=1)
+    assert np.abs(got - want).max() <= 0.01
+    rnb.release(w)
+
+
 # ---- dense SwiGLU FFN (crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:297-337) ----------------------------
 
 def check_ffn(oracle, got, gate, up, down, down_quant, n_ff, n_embd, x, gelu, label):
