@@ -114,6 +114,13 @@ inline Result<std::pair<uint32_t, float>> q8_0_gemv_argmax(Bytes weights, size_t
     if (st != RNB_HIP_OK) return make_err<std::pair<uint32_t, float>>(st);
     return make_ok(best);
 }
+// q8_0_gemv_argmax_q8dot, quant_api.rs:770-805
+inline Result<std::pair<uint32_t, float>> q8_0_gemv_argmax_q8dot(Bytes weights, size_t rows, size_t cols, Floats input) {
+    std::pair<uint32_t, float> best{0, 0.0f};
+    const int st = rnb_hip_q8_0_gemv_argmax_q8dot(weights.ptr, weights.len, rows, cols, input.ptr, input.len, &best.first, &best.second);
+    if (st != RNB_HIP_OK) return make_err<std::pair<uint32_t, float>>(st);
+    return make_ok(best);
+}
 #define RNB_HIP_BLOCK32_MIRROR(name)                                                                               \
     inline Result<std::vector<float>> name##_gemv(Bytes weights, size_t rows, size_t cols, Floats input) {         \
         return gemv_impl(rnb_hip_##name##_gemv, weights, rows, cols, input, rows);                                 \

@@ -330,6 +330,9 @@ int rnb_hip_q6k_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t 
 /* q8_0_gemv_argmax, quant_api.rs:733-768: the same for a Q8_0 head (Q8 x Q8_0 integer dot) */
 int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
                              uint32_t *index_out, float *value_out);
+/* q8_0_gemv_argmax_q8dot, quant_api.rs:770-805 (Q8 x Q8_0 integer dots by name): the same computation as the entry above */
+int rnb_hip_q8_0_gemv_argmax_q8dot(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                                   uint32_t *index_out, float *value_out);
 
 /* dense_q4k_attention_qkv(q_weights, k_weights, v_weights, q_rows, kv_rows, n_embd, input, q, k, v),
  * crates/rnb-backend/cuda/src/runtime/api/dense_api.rs:916-985 (validation order and texts :928-968): the three Q4_K

@@ -109,6 +109,7 @@ from .binding import (  # noqa: F401
     dense_q4k_gelu_ffn,
     dense_q4k_gelu_ffn_batch,
     q8_0_gemv_argmax,
+    q8_0_gemv_argmax_q8dot,
     q8_0_gemv,
     q8_0_gemv_batch,
     q8_0_head_gemv_batch,

@@ -95,6 +95,7 @@ SYMBOLS = [
     ("rnb_hip_q6k_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_attention_qkv", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_q8_0_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
+    ("rnb_hip_q8_0_gemv_argmax_q8dot", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_silu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_gelu_ffn_batch", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dense_q4k_gelu_ffn", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
@@ -653,6 +654,14 @@ def q8_0_gemv_argmax(weights, rows: int, cols: int, input) -> tuple:  # noqa: A0
     w, x = _bytes_view(weights), _f32(input).ravel()
     idx, val = _u32(), C.c_float()
     _check(lib().rnb_hip_q8_0_gemv_argmax(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
+    return int(idx.value), float(val.value)
+
+
+def q8_0_gemv_argmax_q8dot(weights, rows: int, cols: int, input) -> tuple:  # noqa: A002
+    """quant_api.rs:770-805 -> (row index, value); the same integer dots as q8_0_gemv_argmax"""
+    w, x = _bytes_view(weights), _f32(input).ravel()
+    idx, val = _u32(), C.c_float()
+    _check(lib().rnb_hip_q8_0_gemv_argmax_q8dot(_ptr(w), w.size, rows, cols, _ptr(x), x.size, C.byref(idx), C.byref(val)))
     return int(idx.value), float(val.value)
 
 

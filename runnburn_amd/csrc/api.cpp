@@ -1244,6 +1244,13 @@ int rnb_hip_q8_0_gemv_argmax(const uint8_t *w, size_t w_len, size_t rows, size_t
     return gemv_argmax_host(kQ8_0, w, w_len, rows, cols, x, x_len, index_out, value_out);
 }
 
+// q8_0_gemv_argmax_q8dot, quant_api.rs:770-805: the variant whose name says that the input is quantised to Q8 and dotted in
+// integers, which is what the entry above does as well
+int rnb_hip_q8_0_gemv_argmax_q8dot(const uint8_t *w, size_t w_len, size_t rows, size_t cols, const float *x, size_t x_len,
+                                   uint32_t *index_out, float *value_out) {
+    return gemv_argmax_host(kQ8_0, w, w_len, rows, cols, x, x_len, index_out, value_out);
+}
+
 int rnb_hip_dense_q4k_attention_qkv(const uint8_t *q_w, size_t q_len, const uint8_t *k_w, size_t k_len, const uint8_t *v_w,
                                     size_t v_len, size_t q_rows, size_t kv_rows, size_t n_embd, const float *x, size_t x_len,
                                     float *q, size_t q_cap, float *k, size_t k_cap, float *v, size_t v_cap) {

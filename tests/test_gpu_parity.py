@@ -891,6 +891,7 @@ def test_q8_0_gemv_argmax_matches_gemv(rnb, oracle):
     full = rnb.q8_0_gemv(w, rows, cols, x)
     idx, val = rnb.q8_0_gemv_argmax(w, rows, cols, x)
     assert idx == int(np.argmax(full)) and val == full[idx]
+    assert rnb.q8_0_gemv_argmax_q8dot(w, rows, cols, x) == (idx, val)  # quant_api.rs:770-805: the same integer dots by name
     # two identical rows that win: the lower index is reported
     rb = cols // 32 * 34
     w2 = w.copy().reshape(rows, rb)
