@@ -78,7 +78,8 @@ __device__ __forceinline__ float act_mul(float g, float up) {
 }
 
 // Cross-lane sums on the DPP data path (no LDS traffic).  After seg_sum<W>(v) the LAST lane of every
-// aligned W-lane segment (W = 16, 32 or 64) holds the sum over that segment.
+// aligned W-lane segment (W = 4, 8, 16, 32 or 64) holds the sum over that segment.  The steps of a narrower width are
+// the first steps of a wider one, so a segment's sum has the bits of a wider sum whose other lanes hold zeros.
 template <int kCtrl, int kRowMask>
 __device__ __forceinline__ float dpp_add(float v) {
     const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, kRowMask, 0xf, false);
@@ -91,11 +92,11 @@ __device__ __forceinline__ float dpp_max(float v) {  // for non-negative v (lane
 }
 template <int kWidth>
 __device__ __forceinline__ float seg_sum(float v) {
-    static_assert(kWidth == 16 || kWidth == 32 || kWidth == 64, "segment width");
+    static_assert(kWidth == 4 || kWidth == 8 || kWidth == 16 || kWidth == 32 || kWidth == 64, "segment width");
     v = dpp_add<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
     v = dpp_add<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141, 0xf>(v);  // row_half_mirror
-    v = dpp_add<0x140, 0xf>(v);  // row_mirror: all 16 lanes of a row hold the row sum
+    if (kWidth >= 8) v = dpp_add<0x141, 0xf>(v);   // row_half_mirror
+    if (kWidth >= 16) v = dpp_add<0x140, 0xf>(v);  // row_mirror: all 16 lanes of a row hold the row sum
     if (kWidth >= 32) v = dpp_add<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
     if (kWidth >= 64) v = dpp_add<0x143, 0xc>(v);  // row_bcast31 into rows 2 and 3
     return v;

@@ -1191,18 +1191,23 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // against all of them; per token the same expression as the one-token kernel (same bits).  grid.y = token groups.
 // grid.z = heads (1 for a plain matrix): head z has its own `rows` rows of weights, reads activation row tok * heads + z
 // and writes out[tok][z * rows + row], the per-head projections of q8_0_head_gemv_batch.
-template <uint32_t kQuant, bool kPaired, int kTokens>
+// kRows rows side by side in a wave (1, 4 or 16; a row's blocks must fit its 64 / kRows lanes): short rows, as the per-head
+// projections have, would leave most of a wave idle otherwise; a row's sum keeps the bits of the one-row-per-wave form.
+template <uint32_t kQuant, bool kPaired, int kTokens, int kRows = 1>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     gemv_block32_tokens_kernel(const uint8_t *__restrict__ w, const int8_t *__restrict__ aq, const float *__restrict__ ad,
                                float *__restrict__ out, uint32_t rows, uint32_t nb32, uint32_t seq) {
     constexpr size_t kBlockBytes = block32_layout<kQuant>().bytes;
     constexpr bool kSum = kQuant != kQ8_0 && kQuant != kQ8_1;
     const int lane = threadIdx.x & (kWave - 1);
+    constexpr int kLanesPerRow = kWave / kRows;
+    const int sub = lane & (kLanesPerRow - 1);
+    const uint32_t rsel = lane / kLanesPerRow;
     const uint32_t tok0 = blockIdx.y * kTokens, heads = gridDim.z, head = blockIdx.z;
     const size_t row_bytes = static_cast<size_t>(nb32) * kBlockBytes;
     const uint32_t wave_global = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     const uint32_t n_waves = gridDim.x * kWavesPerWg;
-    const uint32_t b0 = kPaired ? 2 * lane : lane, b1 = kPaired ? 2 * lane + 1 : lane + kWave;
+    const uint32_t b0 = kPaired ? 2 * sub : sub, b1 = kPaired ? 2 * sub + 1 : sub + kLanesPerRow;
     const bool has0 = b0 < nb32, has1 = b1 < nb32;  // kPaired: nb32 is even, a pair is there or not as a whole
     Q8Act a0[kTokens], a1[kTokens];
 #pragma unroll
@@ -1212,26 +1217,29 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         a0[t] = q8_load_act<kSum>(aq + (abase + (has0 ? b0 : 0)) * 32, ad[abase + (has0 ? b0 : 0)]);
         a1[t] = q8_load_act<kSum>(aq + (abase + (has1 ? b1 : 0)) * 32, ad[abase + (has1 ? b1 : 0)]);
     }
-    for (uint32_t row = wave_global; row < rows; row += n_waves) {
-        const uint8_t *rowp = w + (static_cast<size_t>(head) * rows + row) * row_bytes;
+    for (uint32_t grp = wave_global; grp * kRows < rows; grp += n_waves) {
+        const uint32_t row = grp * kRows + rsel;
+        const bool live0 = has0 && row < rows, live1 = has1 && row < rows;
+        const uint8_t *rowp = w + (static_cast<size_t>(head) * rows + (row < rows ? row : 0)) * row_bytes;
         Block32Regs c0 = Block32Regs{}, c1 = Block32Regs{};
         if constexpr (kPaired) {
-            if (has0) block32_load_pair<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes, c0, c1);
+            if (live0) block32_load_pair<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes, c0, c1);
         } else {
-            if (has0) c0 = block32_load<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes);
-            if (has1) c1 = block32_load<kQuant>(rowp + static_cast<size_t>(b1) * kBlockBytes);
+            if (live0) c0 = block32_load<kQuant>(rowp + static_cast<size_t>(b0) * kBlockBytes);
+            if (live1) c1 = block32_load<kQuant>(rowp + static_cast<size_t>(b1) * kBlockBytes);
         }
 #pragma unroll
         for (int t = 0; t < kTokens; t++) {
             float acc = 0.0f;
             if constexpr (kPaired) {
-                if (has0) acc = block32_dot<kQuant>(c0, a0[t]) + block32_dot<kQuant>(c1, a1[t]);
+                if (live0) acc = block32_dot<kQuant>(c0, a0[t]) + block32_dot<kQuant>(c1, a1[t]);
             } else {
-                if (has0) acc = block32_dot<kQuant>(c0, a0[t]);
-                if (has1) acc += block32_dot<kQuant>(c1, a1[t]);
+                if (live0) acc = block32_dot<kQuant>(c0, a0[t]);
+                if (live1) acc += block32_dot<kQuant>(c1, a1[t]);
             }
-            acc = seg_sum<kWave>(acc);
-            if (lane == kWave - 1 && tok0 + t < seq) out[(static_cast<size_t>(tok0 + t) * heads + head) * rows + row] = acc;
+            acc = seg_sum<kLanesPerRow>(acc);
+            if (sub == kLanesPerRow - 1 && row < rows && tok0 + t < seq)
+                out[(static_cast<size_t>(tok0 + t) * heads + head) * rows + row] = acc;
         }
     }
 }
@@ -1284,29 +1292,43 @@ void launch_block32(const uint8_t *w, ActView act, float *out, uint32_t rows, ui
 // [tokens][heads][nb32], out [tokens][heads * rows_per_head]; rows of at most 128 blocks.
 void launch_heads_q8_0(const uint8_t *w, ActView act, float *out, uint32_t heads, uint32_t rows_per_head, uint32_t nb32,
                        uint32_t tokens, hipStream_t stream) {
-    const uint32_t waves = rows_per_head < kTargetWaves ? rows_per_head : kTargetWaves;
+    const bool paired = nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0;
+    // rows per wave: as many as the row's blocks (two per lane when paired) leave room for
+    const uint32_t lanes = paired ? nb32 / 2 : nb32;
+    const uint32_t rpw = lanes <= 4 ? 16 : (lanes <= 16 ? 4 : 1);
+    const uint32_t row_groups = (rows_per_head + rpw - 1) / rpw;
+    const uint32_t waves = row_groups < kTargetWaves ? row_groups : kTargetWaves;
     const auto [groups, per] = token_groups(tokens);
     const dim3 grid((waves + kWavesPerWg - 1) / kWavesPerWg, groups, heads);
-    const bool paired = nb32 % 2 == 0 && reinterpret_cast<uintptr_t>(w) % 4 == 0;
-#define RNB_LAUNCH_HEADS(P, T)                                                                                             \
-    hipLaunchKernelGGL((gemv_block32_tokens_kernel<kQ8_0, P, T>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, \
+#define RNB_LAUNCH_HEADS(P, T, R)                                                                                             \
+    hipLaunchKernelGGL((gemv_block32_tokens_kernel<kQ8_0, P, T, R>), grid, dim3(kWave * kWavesPerWg), 0, stream, w, act.qs, \
                        act.d, out, rows_per_head, nb32, tokens)
-#define RNB_LAUNCH_HEADS_P(P)      \
-    do {                           \
-        if (per == 1)              \
-            RNB_LAUNCH_HEADS(P, 1); \
-        else if (per == 2)         \
-            RNB_LAUNCH_HEADS(P, 2); \
-        else if (per == 3)         \
-            RNB_LAUNCH_HEADS(P, 3); \
-        else                       \
-            RNB_LAUNCH_HEADS(P, 4); \
+#define RNB_LAUNCH_HEADS_T(P, R)      \
+    do {                              \
+        if (per == 1)                 \
+            RNB_LAUNCH_HEADS(P, 1, R); \
+        else if (per == 2)            \
+            RNB_LAUNCH_HEADS(P, 2, R); \
+        else if (per == 3)            \
+            RNB_LAUNCH_HEADS(P, 3, R); \
+        else                          \
+            RNB_LAUNCH_HEADS(P, 4, R); \
+    } while (0)
+#define RNB_LAUNCH_HEADS_R(P)         \
+    do {                              \
+        if (rpw == 16)                \
+            RNB_LAUNCH_HEADS_T(P, 16); \
+        else if (rpw == 4)            \
+            RNB_LAUNCH_HEADS_T(P, 4);  \
+        else                          \
+            RNB_LAUNCH_HEADS_T(P, 1);  \
     } while (0)
     if (paired)
-        RNB_LAUNCH_HEADS_P(true);
+        RNB_LAUNCH_HEADS_R(true);
     else
-        RNB_LAUNCH_HEADS_P(false);
-#undef RNB_LAUNCH_HEADS_P
+        RNB_LAUNCH_HEADS_R(false);
+#undef RNB_LAUNCH_HEADS_R
+#undef RNB_LAUNCH_HEADS_T
 #undef RNB_LAUNCH_HEADS
 }
 
