@@ -499,12 +499,15 @@ int run_dense_ffn_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, 
             RESERVE_TRY(s.act_qs, n);
             RESERVE_TRY(s.act_d, n / 256 * sizeof(float));
             RESERVE_TRY(s.act_bsums, n / 256 * 16 * sizeof(int16_t));
-            s.act_has_digits = seq >= kDigitsMinSeq;
-            if (s.act_has_digits) RESERVE_TRY(s.act_digits, n / 256 * 16);
+            // the scratch is about to be overwritten: it describes nothing until the launch is known to have gone out
+            s.act_seq = 0;
+            const bool want_digits = seq >= kDigitsMinSeq;
+            if (want_digits) RESERVE_TRY(s.act_digits, n / 256 * 16);
             launch_quantize_q8k_gated(s.ffn_gate.as<float>(), s.ffn_up.as<float>(), n / 256, gelu, s.act_qs.as<int8_t>(),
                                       s.act_d.as<float>(), s.act_bsums.as<int16_t>(),
-                                      s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr, s.stream);
+                                      want_digits ? s.act_digits.as<uint8_t>() : nullptr, s.stream);
             if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
+            s.act_has_digits = want_digits;
             s.act_family = kQ4K;
             s.act_seq = seq;
             s.act_cols = n_ff;
@@ -828,6 +831,8 @@ int rnb_hip_prewarm(const uint8_t *const *ptrs, const size_t *lens, size_t n) {
 int rnb_hip_release(const uint8_t *ptr, size_t len) {
     Guard g;
     if (!g.state) return g.status;
+    if (g.state->capturing())
+        return fail(RNB_HIP_INVALID_REQUEST, "release frees device memory and cannot run while the library stream is capturing");
     if (!g.state->release(ptr, len)) return fail(RNB_HIP_INVALID_REQUEST, "release: range is not resident");
     return RNB_HIP_OK;
 }
@@ -872,6 +877,8 @@ int rnb_hip_residency_stats(uint64_t *out, size_t n) {
 int rnb_hip_set_resident_budget(uint64_t bytes) {
     Guard g;
     if (!g.state) return g.status;
+    if (g.state->capturing())
+        return fail(RNB_HIP_INVALID_REQUEST, "set_resident_budget frees device memory and cannot run while the library stream is capturing");
     g.state->table->set_budget(bytes);
     return RNB_HIP_OK;
 }
@@ -879,6 +886,8 @@ int rnb_hip_set_resident_budget(uint64_t bytes) {
 int rnb_hip_offload_unpinned(uint64_t *freed_bytes) {
     Guard g;
     if (!g.state) return g.status;
+    if (g.state->capturing())
+        return fail(RNB_HIP_INVALID_REQUEST, "offload_unpinned frees device memory and cannot run while the library stream is capturing");
     std::string err;
     const uint64_t freed = g.state->table->offload_unpinned(&err);
     if (freed_bytes) *freed_bytes = freed;
@@ -1534,22 +1543,28 @@ int rms_norm_dev(const char *what, const float *input, const float *post_weight,
     uint8_t *digits = nullptr;
     if (quantize) {
         const size_t n = seq_len * hidden;
+        s.act_seq = 0;  // the scratch describes nothing until the launch below is known to have gone out
         RESERVE_TRY(s.act_qs, n);
         RESERVE_TRY(s.act_d, n / 256 * sizeof(float));
         RESERVE_TRY(s.act_bsums, n / 256 * 16 * sizeof(int16_t));
-        s.act_has_digits = seq_len >= kDigitsMinSeq;
-        if (s.act_has_digits) RESERVE_TRY(s.act_digits, n / 256 * 16);
+        if (seq_len >= kDigitsMinSeq) {
+            RESERVE_TRY(s.act_digits, n / 256 * 16);
+            digits = s.act_digits.as<uint8_t>();
+        }
         qs = s.act_qs.as<int8_t>();
         d = s.act_d.as<float>();
         bsums = s.act_bsums.as<int16_t>();
-        digits = s.act_has_digits ? s.act_digits.as<uint8_t>() : nullptr;
+    }
+    launch_rms_norm(input, post_weight, post_eps, post_unit != 0, residual, weight, eps, unit != 0,
+                    static_cast<uint32_t>(seq_len), static_cast<uint32_t>(hidden / 256), out_f32, qs, d, bsums, digits, s.stream);
+    if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
+    if (quantize) {
+        s.act_has_digits = digits != nullptr;
         s.act_family = kQ4K;
         s.act_seq = seq_len;
         s.act_cols = hidden;
     }
-    launch_rms_norm(input, post_weight, post_eps, post_unit != 0, residual, weight, eps, unit != 0,
-                    static_cast<uint32_t>(seq_len), static_cast<uint32_t>(hidden / 256), out_f32, qs, d, bsums, digits, s.stream);
-    return check_launches();
+    return RNB_HIP_OK;
 }
 
 }  // namespace

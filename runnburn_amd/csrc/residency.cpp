@@ -198,7 +198,9 @@ int ResidentTable::resolve(const uint8_t *ptr, size_t len, uint64_t fingerprint,
         if (int rc = drop(key, err, false); rc != 0) return rc;
 
     ++stats_.misses;
-    const uint64_t reuses = history_.observe({key, len});
+    // the history knows a range by address, length AND content: host memory that was freed and holds other data now is
+    // a range that has not been seen before
+    const uint64_t reuses = history_.observe({key, len + static_cast<size_t>(0x9E3779B97F4A7C15ull * fingerprint)});
     std::vector<Key> victims;
     uint64_t victim_bytes = 0;
     const bool fits = plan(len, &victims, &victim_bytes);

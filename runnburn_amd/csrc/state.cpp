@@ -194,6 +194,9 @@ Guard::Guard() : lock(g_mutex) {
             state = nullptr;
             return;
         }
+        // every entry looks at the stream once: a capture whose calls all fit the existing scratch never reaches the
+        // check in DeviceBuf::reserve, and a graph instantiated from it still points into that scratch
+        (void)state->capturing();
         state->table->begin_call();
         return;
     }

@@ -3,6 +3,7 @@ seeded inputs.  Activation quantisation must be bit-exact; f32 outputs must sati
 abs-or-rel row check (crates/rnb-backend/cuda/src/runtime/tests.rs:28525-28541) with
 rel = 1e-3 and abs floor = 1e-3 * rms(ref), and are additionally held to 2e-5 * rms against the
 f64-accumulated form of the same integer arithmetic."""
+import os
 import numpy as np
 import pytest
 
@@ -1140,6 +1141,10 @@ def test_graph_survives_scratch_growth_and_capture_refuses_growth(rnb):
         with pytest.raises(rnb.BackendError) as err:
             rnb.gemv_dev(Q4_K, w, rows, cols, xb, big_seq, ob)
         assert err.value.kind == "InvalidRequest" and "capturing" in str(err.value)
+        # entry points that free device memory synchronise the stream first: refused as well
+        for call in (lambda: rnb.lib().rnb_hip_set_resident_budget(1 << 30), lambda: rnb.lib().rnb_hip_offload_unpinned(None),
+                     lambda: rnb.lib().rnb_hip_release(x.ctypes.data_as(C.c_void_p), x.nbytes)):
+            assert call() == 1 and "capturing" in rnb.last_error()  # RNB_HIP_INVALID_REQUEST
         # the no-allocation form of the same call is captured
         out2 = rnb.DeviceBuffer(seq * rows * 4)
         rnb.gemv_dev_noalloc(Q4_K, w, rows, cols, x_dev, seq, out2)
@@ -1165,3 +1170,50 @@ def test_graph_survives_scratch_growth_and_capture_refuses_growth(rnb):
         hip.rt.hipGraphDestroy(graph)
         for b in (w, x_dev, out_dev, xb, ob, out2):
             b.free()
+
+
+_FIRST_CAPTURE_SCRIPT = r"""
+import ctypes as C, sys
+import numpy as np
+import bench
+import runnburn_amd as rnb
+Q4_K = 12
+hip = bench.Hip()
+stream = C.c_void_p(rnb.stream_handle())
+rows, cols, seq = 384, 1024, 6
+w = rnb.DeviceBuffer.from_host(bench.synth_weights(Q4_K, rows, cols, 78))
+x = np.random.default_rng(77).standard_normal(seq * cols).astype(np.float32)
+x_dev, out_dev = rnb.DeviceBuffer.from_host(x), rnb.DeviceBuffer(seq * rows * 4)
+rnb.gemv_dev(Q4_K, w, rows, cols, x_dev, seq, out_dev)  # eager warm-up: the scratch now fits this shape
+want = out_dev.to_host(np.float32)
+graph, gexec = C.c_void_p(), C.c_void_p()
+hip.check(hip.rt.hipStreamBeginCapture(stream, 2), "begin")
+rnb.gemv_dev(Q4_K, w, rows, cols, x_dev, seq, out_dev)  # the only captured call: nothing has to grow
+hip.check(hip.rt.hipStreamEndCapture(stream, C.byref(graph)), "end")
+hip.check(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0), "instantiate")
+big = 4096
+xb, ob = rnb.DeviceBuffer(big * cols * 4), rnb.DeviceBuffer(big * rows * 4)
+rnb.gemv_dev(Q4_K, w, rows, cols, xb, big, ob)  # grows every scratch buffer the graph points into
+rnb.sync()
+junk = [rnb.DeviceBuffer.from_host(np.full(1 << 20, 0x7f, np.uint8)) for _ in range(16)]  # reuse whatever was freed
+for _ in range(3):
+    rnb.lib().rnb_hip_dev_upload(out_dev.ptr, np.zeros(seq * rows, np.float32).ctypes.data_as(C.c_void_p), seq * rows * 4)
+    hip.check(hip.rt.hipGraphLaunch(gexec, stream), "launch")
+    rnb.sync()
+    if not np.array_equal(out_dev.to_host(np.float32), want):
+        print("REPLAY DIFFERS"); sys.exit(1)
+    rnb.gemv_dev(Q4_K, w, rows, cols, xb, big, ob)
+    rnb.sync()
+print("REPLAY OK")
+"""
+
+
+def test_first_capture_of_a_process_with_fitting_calls_only_keeps_its_scratch(rnb):
+    """In a fresh process: one eager call, then a capture whose only call fits the scratch that call left (so no buffer
+    is asked to grow while capturing), then a larger eager call.  The library must have noticed the capture anyway and
+    retire the replaced scratch instead of freeing it; the graph's replays give the eager bits."""
+    import subprocess
+    import sys as _sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([_sys.executable, "-c", _FIRST_CAPTURE_SCRIPT], cwd=root, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0 and "REPLAY OK" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-2000:]
