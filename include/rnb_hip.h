@@ -389,7 +389,14 @@ typedef struct rnb_hip_gguf_tensor {
     const uint8_t *data;   /* mapping + file_offset, or NULL if the tensor does not lie inside the file */
 } rnb_hip_gguf_tensor;
 
-/* mmap + parse + map_tensors checks; the handle owns the mapping until rnb_hip_gguf_close */
+/* mmap + parse + map_tensors checks; the handle owns the mapping until rnb_hip_gguf_close.
+ * Split models (crates/rnb-loader/src/gguf/sharded.rs:22-105, load_mapped_gguf): when the file's
+ * metadata carries `split.count`, `path` may name any shard `<prefix>-<index>-of-<count>.gguf`; every
+ * shard is mapped and checked (split.no / split.count / split.tensors.count agree with the selected
+ * file and with the name, :107-158 and :181-236), the handle lists all tensors in shard order with
+ * `file_offset` and `data` relative to the tensor's own shard, a name in two shards and a total that
+ * differs from split.tensors.count are refused (:62-104), and the metadata is shard zero's.  Failures
+ * read `parse error at offset 0: invalid split GGUF: ...` with the reference's texts. */
 int rnb_hip_gguf_open(const char *path, rnb_hip_gguf **out);
 /* GGUFFile::parse over caller-owned bytes (borrowed for the handle's lifetime); payload bounds are
  * not checked here, exactly as in the reference: call rnb_hip_gguf_map_tensors for that */

@@ -6,14 +6,22 @@
 // crates/rnb-loader/src/gguf/types.rs:5-41 (GGMLType ids), crates/rnb-loader/src/convert.rs:23-83 (block sizes,
 // checked_tensor_size) and :99-178 (map_tensors: bounds of every tensor against the file length).
 // Error texts are the reference's `LoaderError` Display strings (crates/rnb-loader/src/error.rs:4-16).
+// A file opened by path whose metadata declares split.count > 1 is one shard of a split model: the other shards are
+// found beside it, mapped and checked as crates/rnb-loader/src/gguf/sharded.rs:22-235 does, and the handle shows the
+// union of their tensor tables with shard zero's metadata.
 #include <fcntl.h>
 #include <string.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <errno.h>
+#include <stdlib.h>
+
+#include <algorithm>
 #include <limits>
 #include <memory>
+#include <set>
 #include <string>
 #include <unordered_set>
 #include <vector>
@@ -68,6 +76,7 @@ struct Tensor {
     uint64_t shape[4] = {0, 0, 0, 0};  // row-major: outermost first
     uint32_t ggml_type = 0;
     uint64_t offset = 0, file_offset = 0, n_bytes = 0;
+    const rnb_hip_gguf *home = nullptr;  // the shard whose mapping holds the payload (null: the handle itself)
 };
 
 struct ParseFailure {
@@ -215,6 +224,9 @@ struct rnb_hip_gguf {
     uint64_t alignment = 32, data_start = 0;
     std::vector<std::pair<std::string, rnb::Value>> metadata;
     std::vector<rnb::Tensor> tensors;
+    // a split file opened by path: the other shards (each owns its mapping); `tensors` above is then the union of all
+    // shards' tables and `metadata` that of shard zero
+    std::vector<std::unique_ptr<rnb_hip_gguf>> shards;
     ~rnb_hip_gguf() {
         if (owns_mapping && data != nullptr) munmap(const_cast<uint8_t *>(data), len);
     }
@@ -358,8 +370,9 @@ void parse_into(rnb_hip_gguf &g) {
 }
 
 // crates/rnb-loader/src/convert.rs:124-158: every tensor's shape is block-aligned and its bytes lie inside the file
-void map_tensors(const rnb_hip_gguf &g) {
-    for (const Tensor &t : g.tensors) {
+void map_tensors(const rnb_hip_gguf &handle) {
+    for (const Tensor &t : handle.tensors) {
+        const rnb_hip_gguf &g = t.home != nullptr ? *t.home : handle;  // a split model: the tensor's own shard
         std::string why;
         uint64_t n_bytes = 0;
         if (!tensor_size(t.shape, t.n_dims, t.ggml_type, &n_bytes, &why))
@@ -377,6 +390,7 @@ void map_tensors(const rnb_hip_gguf &g) {
 }
 
 bool tensor_in_bounds(const rnb_hip_gguf *g, const Tensor &t) {
+    if (t.home != nullptr) g = t.home;
     std::string why;
     uint64_t n = 0;
     return tensor_size(t.shape, t.n_dims, t.ggml_type, &n, &why) && t.offset <= g->len && g->data_start <= g->len &&
@@ -404,7 +418,7 @@ void fill_tensor(const rnb_hip_gguf *g, const Tensor &t, rnb_hip_gguf_tensor *ou
     out->offset = t.offset;
     out->file_offset = t.file_offset;
     out->n_bytes = t.n_bytes;
-    out->data = tensor_in_bounds(g, t) ? g->data + t.file_offset : nullptr;
+    out->data = tensor_in_bounds(g, t) ? (t.home != nullptr ? t.home : g)->data + t.file_offset : nullptr;
 }
 
 const Value *find_value(const rnb_hip_gguf *g, const char *key) {
@@ -417,17 +431,8 @@ const Value *find_value(const rnb_hip_gguf *g, const char *key) {
 bool is_signed_type(uint32_t t) { return t == 1 || t == 3 || t == 5 || t == 11; }
 bool is_integer_type(uint32_t t) { return t <= 5 || t == 10 || t == 11; }
 
-}  // namespace
-
-}  // namespace rnb
-
-using namespace rnb;
-
-extern "C" {
-
-int rnb_hip_gguf_open(const char *path, rnb_hip_gguf **out) {
-    if (path == nullptr || out == nullptr) return fail_gguf(RNB_HIP_INVALID_REQUEST, "null argument");
-    *out = nullptr;
+// mmap + parse + map_tensors of one file
+int open_one(const char *path, std::unique_ptr<rnb_hip_gguf> *out) {
     const int fd = open(path, O_RDONLY);
     if (fd < 0) return fail_gguf(RNB_HIP_EXECUTION_FAILED, std::string("I/O error: ") + strerror(errno) + ": " + path);
     struct stat st;
@@ -449,7 +454,145 @@ int rnb_hip_gguf_open(const char *path, rnb_hip_gguf **out) {
         g->owns_mapping = true;
     }
     close(fd);
-    return finish_open(std::move(g), out, true);
+    rnb_hip_gguf *raw = nullptr;
+    if (int rc = finish_open(std::move(g), &raw, true); rc != RNB_HIP_OK) return rc;
+    out->reset(raw);
+    return RNB_HIP_OK;
+}
+
+// ---- split files: crates/rnb-loader/src/gguf/sharded.rs:22-235 (load_mapped_gguf), same checks, same texts ---------
+[[noreturn]] void split_error(const std::string &msg) { parse_error(0, "invalid split GGUF: " + msg); }
+
+// split_value, sharded.rs:153-178: absent -> false; any non-negative integer type
+bool split_value(const rnb_hip_gguf &g, const char *key, uint64_t *out) {
+    const Value *v = find_value(&g, key);
+    if (v == nullptr) return false;
+    const bool integer = v->type <= 5 || v->type == 10 || v->type == 11;  // u8 i8 u16 i16 u32 i32, u64 i64
+    if (!integer || (is_signed_type(v->type) && static_cast<int64_t>(v->u) < 0))
+        split_error(std::string("metadata key ") + key + " must be a non-negative integer");
+    *out = v->u;
+    return true;
+}
+uint64_t required_split_value(const rnb_hip_gguf &g, const char *key) {
+    uint64_t v = 0;
+    if (!split_value(g, key, &v)) split_error(std::string("missing metadata key ") + key);
+    return v;
+}
+
+bool all_digits(const std::string &s) {
+    return !s.empty() && std::all_of(s.begin(), s.end(), [](unsigned char c) { return c >= '0' && c <= '9'; });
+}
+
+// resolve_shard_paths, sharded.rs:180-235: `<prefix>-<index>-of-<count>.gguf` beside the selected file, same digit widths
+std::vector<std::string> resolve_shard_paths(const std::string &selected, uint64_t selected_no, uint64_t split_count) {
+    const size_t slash = selected.find_last_of('/');
+    const std::string parent = slash == std::string::npos ? "" : selected.substr(0, slash + 1);
+    const std::string file_name = slash == std::string::npos ? selected : selected.substr(slash + 1);
+    const std::string ext = ".gguf";
+    if (file_name.size() < ext.size() || file_name.compare(file_name.size() - ext.size(), ext.size(), ext) != 0)
+        split_error("split GGUF file name must end in .gguf");
+    const std::string stem = file_name.substr(0, file_name.size() - ext.size());
+    const size_t of = stem.rfind("-of-");
+    if (of == std::string::npos) split_error("split GGUF file name must end in -00001-of-00001.gguf");
+    const std::string indexed_stem = stem.substr(0, of), file_count = stem.substr(of + 4);
+    const size_t dash = indexed_stem.rfind('-');
+    if (dash == std::string::npos) split_error("split GGUF file name is missing its shard index");
+    const std::string prefix = indexed_stem.substr(0, dash), file_index = indexed_stem.substr(dash + 1);
+    if (prefix.empty() || !all_digits(file_index) || !all_digits(file_count))
+        split_error("split GGUF file name has an invalid shard suffix");
+    errno = 0;
+    const unsigned long long parsed_index = std::strtoull(file_index.c_str(), nullptr, 10);
+    if (errno == ERANGE) split_error("split GGUF shard index is too large");
+    const unsigned long long parsed_count = std::strtoull(file_count.c_str(), nullptr, 10);
+    if (errno == ERANGE) split_error("split GGUF shard count is too large");
+    if (parsed_index != selected_no + 1 || parsed_count != split_count)
+        split_error("file name declares shard " + std::to_string(parsed_index) + " of " + std::to_string(parsed_count) +
+                    ", metadata declares shard " + std::to_string(selected_no + 1) + " of " + std::to_string(split_count));
+    auto padded = [](uint64_t v, size_t width) {
+        std::string t = std::to_string(v);
+        return t.size() < width ? std::string(width - t.size(), '0') + t : t;
+    };
+    std::vector<std::string> paths;
+    for (uint64_t index = 1; index <= split_count; index++)
+        paths.push_back(parent + prefix + "-" + padded(index, file_index.size()) + "-of-" + padded(split_count, file_count.size()) + ext);
+    return paths;
+}
+
+// The file that was opened declares split.count > 1: every shard is mapped and checked, `g` becomes shard zero with the
+// union of the tensor tables (a tensor keeps pointing into its own shard's mapping).
+void assemble_split(const char *path, std::unique_ptr<rnb_hip_gguf> &g) {
+    uint64_t split_count = 1;
+    if (split_value(*g, "split.count", &split_count) && split_count == 0) split_error("split.count must be positive");
+    if (split_count == 1) return;
+    const uint64_t selected_no = required_split_value(*g, "split.no");
+    if (selected_no >= split_count)
+        split_error("split.no " + std::to_string(selected_no) + " is outside split.count " + std::to_string(split_count));
+    const uint64_t expected_tensors = required_split_value(*g, "split.tensors.count");
+    const std::vector<std::string> paths = resolve_shard_paths(path, selected_no, split_count);
+    std::vector<std::unique_ptr<rnb_hip_gguf>> shards(split_count);
+    for (uint64_t no = 0; no < split_count; no++) {
+        if (no == selected_no) {
+            shards[no] = std::move(g);
+        } else if (open_one(paths[no].c_str(), &shards[no]) != RNB_HIP_OK) {
+            split_error("failed to load shard '" + paths[no] + "': " + last_error_cstr());
+        }
+        // validate_shard, sharded.rs:113-138
+        const rnb_hip_gguf &sh = *shards[no];
+        const uint64_t shard_no = required_split_value(sh, "split.no"), shard_count = required_split_value(sh, "split.count"),
+                       shard_tensors = required_split_value(sh, "split.tensors.count");
+        if (shard_no != no)
+            split_error("expected shard " + std::to_string(no) + ", but its metadata declares split.no " + std::to_string(shard_no));
+        if (shard_count != split_count)
+            split_error("shard " + std::to_string(shard_no) + " declares split.count " + std::to_string(shard_count) +
+                        ", expected " + std::to_string(split_count));
+        if (shard_tensors != expected_tensors)
+            split_error("shard " + std::to_string(shard_no) + " declares split.tensors.count " + std::to_string(shard_tensors) +
+                        ", expected " + std::to_string(expected_tensors));
+    }
+    // shard zero carries the metadata and becomes the handle; the tensors of all shards, in shard order
+    std::unique_ptr<rnb_hip_gguf> head = std::move(shards[0]);
+    std::vector<Tensor> all;
+    std::set<std::string> names;
+    auto take = [&](rnb_hip_gguf *from, const rnb_hip_gguf *home) {
+        for (Tensor &t : from->tensors) {
+            if (!names.insert(t.name).second) split_error("tensor '" + t.name + "' appears in more than one shard");
+            t.home = home;
+            all.push_back(std::move(t));
+        }
+        from->tensors.clear();
+    };
+    take(head.get(), nullptr);
+    for (uint64_t no = 1; no < split_count; no++) take(shards[no].get(), shards[no].get());
+    if (all.size() != expected_tensors)
+        split_error("split.tensors.count declares " + std::to_string(expected_tensors) + " tensors but " +
+                    std::to_string(all.size()) + " were loaded");
+    head->tensors = std::move(all);
+    for (uint64_t no = 1; no < split_count; no++) head->shards.push_back(std::move(shards[no]));
+    g = std::move(head);
+}
+
+}  // namespace
+
+}  // namespace rnb
+
+using namespace rnb;
+
+extern "C" {
+
+int rnb_hip_gguf_open(const char *path, rnb_hip_gguf **out) {
+    if (path == nullptr || out == nullptr) return fail_gguf(RNB_HIP_INVALID_REQUEST, "null argument");
+    *out = nullptr;
+    std::unique_ptr<rnb_hip_gguf> g;
+    if (int st = open_one(path, &g); st != RNB_HIP_OK) return st;
+    try {
+        assemble_split(path, g);
+    } catch (const ParseFailure &f) {
+        return fail_gguf(RNB_HIP_INVALID_REQUEST, f.text);
+    } catch (const std::bad_alloc &) {
+        return fail_gguf(RNB_HIP_EXECUTION_FAILED, "out of host memory while parsing GGUF header");
+    }
+    *out = g.release();
+    return RNB_HIP_OK;
 }
 
 int rnb_hip_gguf_parse(const uint8_t *data, size_t len, rnb_hip_gguf **out) {
@@ -585,7 +728,7 @@ int rnb_hip_gguf_prewarm_tensor(const rnb_hip_gguf *g, size_t index) {
     const Tensor &t = g->tensors[index];
     if (!tensor_in_bounds(g, t))
         return fail_gguf(RNB_HIP_INVALID_REQUEST, "tensor '" + t.name + "' does not lie inside the file");
-    const uint8_t *ptr = g->data + t.file_offset;
+    const uint8_t *ptr = (t.home != nullptr ? t.home : g)->data + t.file_offset;  // a split model: the tensor's own shard
     const size_t len = static_cast<size_t>(t.n_bytes);
     return rnb_hip_prewarm(&ptr, &len, 1);
 }

@@ -70,6 +70,40 @@ def test_gather_extreme_codes(rnb, oracle):
 
 
 @pytest.mark.gpu
+def test_gather_touches_every_codebook_entry(rnb, oracle):
+    """The device tables are expanded at compile time from packed words by code of their own: blocks whose index bytes
+    run through ALL 256 / 1024 / 256 grid entries (signs and scales random) must dequantise to the oracle's bits, whose
+    tables are pinned entry for entry on the reference's (test_iq_codebooks_equal_the_references_tables_entry_for_entry)."""
+    rng = np.random.default_rng(99)
+    for quant, n_blocks in ((IQ2_XXS, 8), (IQ2_S, 32), (IQ3_XXS, 4)):
+        bb = oracle.BLOCK_BYTES[quant]
+        w = rng.integers(0, 256, size=(n_blocks, bb), dtype=np.uint8)
+        w[:, 0:2] = np.frombuffer(np.float16(0.03125).tobytes(), np.uint8)
+        seen = set()
+        for k in range(n_blocks):
+            if quant == IQ2_XXS:
+                for ib in range(8):
+                    for l in range(4):
+                        w[k, 2 + 8 * ib + l] = 32 * k + 4 * ib + l
+                        seen.add(32 * k + 4 * ib + l)
+            elif quant == IQ2_S:
+                for i in range(32):
+                    w[k, 2 + i] = 32 * (k % 8) + i
+                    seen.add((32 * (k % 8) + i) | (k // 8) << 8)
+                w[k, 66:74] = 0x55 * (k // 8)  # the two high bits of every index of the block
+            else:
+                for i in range(64):
+                    w[k, 2 + i] = 64 * k + i
+                    seen.add(64 * k + i)
+        assert len(seen) == (1024 if quant == IQ2_S else 256)
+        w = w.reshape(-1)
+        ids = np.arange(n_blocks, dtype=np.uint32)
+        got = rnb.quant_embedding_gather(quant, w, n_blocks, 256, ids)
+        want = _expected(oracle, quant, w, n_blocks, 256, ids)
+        assert np.array_equal(_bits(got), _bits(want)), f"quant {quant}"
+
+
+@pytest.mark.gpu
 def test_gather_float_tables(rnb):
     rng = np.random.default_rng(5)
     rows, cols = 11, 96

@@ -260,6 +260,122 @@ def test_file_with_quantised_tensors_maps_untouched_bytes(tmp_path):
         assert g.tensor("blk.0.ffn_gate.weight").shape == [rows, cols]
 
 
+# ---- split files: crates/rnb-loader/src/gguf/sharded.rs -------------------------------------------------------------------
+
+def _shard(shard_no, shard_count, total_tensors, tensor_name, value, no_type=gw.T_U16, extra=()):
+    """make_split_shard of sharded.rs:245-274: architecture, the three split keys, one F32 tensor of one element."""
+    md = [("general.architecture", gw.T_STR, "llama")]
+    if shard_no is not None:
+        md.append(("split.no", no_type, shard_no))
+    if shard_count is not None:
+        md.append(("split.count", gw.T_U16, shard_count))
+    if total_tensors is not None:
+        md.append(("split.tensors.count", gw.T_U64, total_tensors))
+    b = gw.Builder(3, 1 + len(extra), len(md))
+    for item in md:
+        b.kv(*item)
+    b.tensor_info(tensor_name, [1], 0, 0)
+    for i, name in enumerate(extra):
+        b.tensor_info(name, [1], 0, 32 * (i + 1))
+    b.pad(32)
+    b.raw(np.float32(value).tobytes())
+    for i, _ in enumerate(extra):
+        b.pad(32)
+        b.raw(np.float32(value + i + 1).tobytes())
+    return b.build()
+
+
+def test_single_file_keeps_the_direct_path(tmp_path):
+    """sharded.rs:277-288: no split keys, one tensor."""
+    path = tmp_path / "model.gguf"
+    path.write_bytes(with_tensor())
+    with rnb.GGUFFile(str(path)) as g:
+        assert len(g) == 1 and g.tensor_at(0).name == "token_embd.weight"
+
+
+@pytest.mark.parametrize("selected", [0, 1, 2])
+def test_split_file_maps_every_shard_from_any_of_its_paths(tmp_path, selected):
+    """sharded.rs:290-311 (from the first path) and the same from the other shards: the handle shows all tensors, each
+    with the bytes of its own shard, and the metadata of shard zero."""
+    names = ["first.weight", "second.weight", "third.weight"]
+    values = [1.25, -2.5, 7.0]
+    for i in range(3):
+        data = _shard(i, 3, 3, names[i], values[i])
+        (tmp_path / f"model-0000{i + 1}-of-00003.gguf").write_bytes(data)
+    with rnb.GGUFFile(str(tmp_path / f"model-0000{selected + 1}-of-00003.gguf")) as g:
+        assert len(g) == 3
+        assert [t.name for t in g.tensors()] == names  # shard order
+        for name, v in zip(names, values):
+            t = g.tensor(name)
+            assert t.n_bytes == 4 and bytes(t.data) == np.float32(v).tobytes()
+        assert g.metadata("split.no") == 0 and g.metadata("general.architecture") == "llama"
+        g.map_tensors()  # each tensor is checked against its own shard's length
+
+
+def test_split_file_rejections(tmp_path):
+    """Every check of load_mapped_gguf / validate_shard / resolve_shard_paths with its message text
+    (`parse error at offset 0: invalid split GGUF: ...`)."""
+    def write(name, data):
+        (tmp_path / name).write_bytes(data)
+        return str(tmp_path / name)
+
+    def rejected(path, fragment):
+        with pytest.raises(rnb.BackendError) as e:
+            rnb.GGUFFile(path)
+        assert e.value.kind == "InvalidRequest"
+        assert str(e.value).startswith("parse error at offset 0: invalid split GGUF: ") and fragment in str(e.value), str(e.value)
+
+    # a missing shard is named (sharded.rs:313-328)
+    first = write("model-00001-of-00002.gguf", _shard(0, 2, 2, "first.weight", 1.25))
+    rejected(first, "model-00002-of-00002.gguf")
+    rejected(write("a-00001-of-00002.gguf", _shard(0, 0, 2, "w", 1.0)), "split.count must be positive")
+    rejected(write("b-00001-of-00002.gguf", _shard(None, 2, 2, "w", 1.0)), "missing metadata key split.no")
+    rejected(write("c-00001-of-00002.gguf", _shard(0, 2, None, "w", 1.0)), "missing metadata key split.tensors.count")
+    rejected(write("d-00001-of-00002.gguf", _shard(2, 2, 2, "w", 1.0)), "split.no 2 is outside split.count 2")
+    rejected(write("e-00001-of-00002.gguf", _shard(-1, 2, 2, "w", 1.0, no_type=gw.T_I16)),
+             "metadata key split.no must be a non-negative integer")
+    rejected(write("f-00001-of-00002.gguf", _shard("0", 2, 2, "w", 1.0, no_type=gw.T_STR)),
+             "metadata key split.no must be a non-negative integer")
+    # file names
+    rejected(write("model-00001-of-00002.bin", _shard(0, 2, 2, "w", 1.0)), "split GGUF file name must end in .gguf")
+    rejected(write("model.gguf", _shard(0, 2, 2, "w", 1.0)), "split GGUF file name must end in -00001-of-00001.gguf")
+    rejected(write("00001-of-00002.gguf", _shard(0, 2, 2, "w", 1.0)), "split GGUF file name is missing its shard index")
+    rejected(write("model-0000x-of-00002.gguf", _shard(0, 2, 2, "w", 1.0)), "split GGUF file name has an invalid shard suffix")
+    rejected(write("-00001-of-00002.gguf", _shard(0, 2, 2, "w", 1.0)), "split GGUF file name has an invalid shard suffix")
+    rejected(write("g-00002-of-00002.gguf", _shard(0, 2, 2, "w", 1.0)),
+             "file name declares shard 2 of 2, metadata declares shard 1 of 2")
+    rejected(write("h-00001-of-00003.gguf", _shard(0, 2, 2, "w", 1.0)),
+             "file name declares shard 1 of 3, metadata declares shard 1 of 2")
+    # the other shard disagrees with the selected one
+    write("i-00001-of-00002.gguf", _shard(0, 2, 2, "w0", 1.0))
+    write("i-00002-of-00002.gguf", _shard(0, 2, 2, "w1", 1.0))
+    rejected(str(tmp_path / "i-00001-of-00002.gguf"), "expected shard 1, but its metadata declares split.no 0")
+    write("j-00001-of-00002.gguf", _shard(0, 2, 2, "w0", 1.0))
+    write("j-00002-of-00002.gguf", _shard(1, 3, 2, "w1", 1.0))
+    rejected(str(tmp_path / "j-00001-of-00002.gguf"), "shard 1 declares split.count 3, expected 2")
+    write("k-00001-of-00002.gguf", _shard(0, 2, 2, "w0", 1.0))
+    write("k-00002-of-00002.gguf", _shard(1, 2, 5, "w1", 1.0))
+    rejected(str(tmp_path / "k-00001-of-00002.gguf"), "shard 1 declares split.tensors.count 5, expected 2")
+    write("l-00001-of-00002.gguf", _shard(0, 2, 2, "same.weight", 1.0))
+    write("l-00002-of-00002.gguf", _shard(1, 2, 2, "same.weight", 2.0))
+    rejected(str(tmp_path / "l-00001-of-00002.gguf"), "tensor 'same.weight' appears in more than one shard")
+    write("m-00001-of-00002.gguf", _shard(0, 2, 3, "w0", 1.0))
+    write("m-00002-of-00002.gguf", _shard(1, 2, 3, "w1", 1.0))
+    rejected(str(tmp_path / "m-00001-of-00002.gguf"), "split.tensors.count declares 3 tensors but 2 were loaded")
+    # a shard that does not parse is named with its own error
+    write("n-00001-of-00002.gguf", _shard(0, 2, 2, "w0", 1.0))
+    write("n-00002-of-00002.gguf", b"GGUX" + bytes(60))
+    rejected(str(tmp_path / "n-00001-of-00002.gguf"), "n-00002-of-00002.gguf': invalid GGUF magic bytes")
+
+
+def test_split_file_index_widths_follow_the_selected_name(tmp_path):
+    """resolve_shard_paths keeps the digit widths of the selected file's name (sharded.rs:223-234)."""
+    (tmp_path / "m-1-of-2.gguf").write_bytes(_shard(0, 2, 2, "a", 1.0))
+    (tmp_path / "m-2-of-2.gguf").write_bytes(_shard(1, 2, 2, "b", 2.0))
+    with rnb.GGUFFile(str(tmp_path / "m-2-of-2.gguf")) as g:
+        assert [t.name for t in g.tensors()] == ["a", "b"]
+
+
 @pytest.mark.gpu
 def test_gguf_tensors_run_from_the_untouched_upload(rnb, oracle, tmp_path):
     """File -> reader -> prewarm (upload as stored) -> GEMV / MoE on the mapped bytes == oracle on the same bytes."""
@@ -322,3 +438,25 @@ def test_reader_survives_mutated_files_under_sanitizers():
     p = subprocess.run([exe, "60000"], capture_output=True, text=True, timeout=300, env=env)
     assert p.returncode == 0, p.stdout[-2000:] + p.stderr[-4000:]
     assert "0 failure(s)" in p.stdout
+
+
+@pytest.mark.gpu
+def test_split_model_tensors_upload_from_their_own_shard(rnb, oracle, tmp_path):
+    """Two shards with one quantised matrix each, of different file lengths: prewarm + GEMV on the tensor of either shard,
+    opened through the second shard's path, equals the oracle on that shard's bytes."""
+    o = oracle
+    mats = [(o.make_weights(o.Q4_K, 24, 512, 51), 24, 512, 12, o.Q4_K), (o.make_weights(o.Q6_K, 56, 1024, 52), 56, 1024, 14, o.Q6_K)]
+    for no, (w, rows, cols, ggml_type, _) in enumerate(mats):
+        md = [("general.architecture", gw.T_STR, "llama"), ("split.no", gw.T_U16, no), ("split.count", gw.T_U16, 2),
+              ("split.tensors.count", gw.T_I32, 2)]
+        gw.write_model(str(tmp_path / f"m-0000{no + 1}-of-00002.gguf"), md, [(f"blk.{no}.weight", [rows, cols], ggml_type, w)])
+    with rnb.GGUFFile(str(tmp_path / "m-00002-of-00002.gguf")) as g:
+        assert [t.name for t in g.tensors()] == ["blk.0.weight", "blk.1.weight"]
+        for no, (w, rows, cols, _, q) in enumerate(mats):
+            t = g.tensor(f"blk.{no}.weight")
+            assert bytes(t.data) == w.tobytes()
+            t.prewarm()
+            x = o.fill_normal(cols, 60 + no, 1.0)
+            got = (rnb.q4k_gemv if q == o.Q4_K else rnb.q6k_gemv)(t.data, rows, cols, x)
+            ref = o.gemv(q, w, rows, cols, x)[0]
+            assert np.allclose(got, ref, rtol=1e-3, atol=1e-3 * np.abs(ref).max())

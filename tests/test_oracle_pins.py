@@ -984,6 +984,75 @@ def test_iq_codebooks_have_the_published_shape(oracle):
     assert g2[0] == 0x0808080808080808 and g2[1] == 0x080808080808082B and g2s[0] == 0x0808080808080808 and g3[0] == 0x04040404
 
 
+def _packed_inc_tables(path):
+    """The three packed codebooks of an .inc file (16 bits per entry), by name."""
+    import re
+
+    text = open(path).read()
+    out = {}
+    for name, n in (("kIq2xxsPacked", 256), ("kIq2sPacked", 1024), ("kIq3xxsPacked", 256)):
+        m = re.search(name + r"\[" + str(n) + r"\]\s*=\s*\{(.*?)\};", text, re.S)
+        assert m, f"{name} not found in {path}"
+        vals = [int(tok, 16) for tok in re.findall(r"0x[0-9a-fA-F]+", m.group(1))]
+        assert len(vals) == n
+        out[name] = vals
+    return out
+
+
+def _expand2(w):  # two bits per byte: 0 -> 8, 1 -> 25, 2 -> 43
+    return sum((8, 25, 43)[(w >> (2 * j)) & 3] << (8 * j) for j in range(8))
+
+
+def _expand3(w):  # three bits per byte: c -> 4 + 8 c, 7 -> 62
+    return sum((62 if ((w >> (3 * j)) & 7) == 7 else 4 + 8 * ((w >> (3 * j)) & 7)) << (8 * j) for j in range(4))
+
+
+def _digest(vals, width, signed=False):
+    import hashlib
+
+    return hashlib.sha256(b"".join(int(v).to_bytes(width, "little", signed=signed) for v in vals)).hexdigest()
+
+
+def test_iq_codebooks_equal_the_references_tables_entry_for_entry(oracle):
+    """Every entry of the three grids, the sign table and the IQ4_NL values against the reference's own tables
+    (crates/rnb-core/src/quant_codebooks.rs:3, 13, 787, 1814; crates/rnb-cpu/src/quantize/iq.rs:9), through the digests and
+    spot entries that tests/golden/make_iq_codebook_digests.py computed from the reference's text.  Three routes to the
+    same numbers: the oracle's expanded tables; the product's packed file expanded here by the packing rule (the product
+    and the oracle keep the same packed words, so a typo would be common to both: this is the check that is not); the
+    sign rule `i | parity(i) << 7` and the IQ4_NL values as the oracle's dequantiser applies them."""
+    import json
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    want = json.load(open(os.path.join(root, "tests", "golden", "iq_codebook_digests.json")))
+    # the oracle's expansion
+    for which, name, width in ((0, "IQ2XXS_GRID", 8), (1, "IQ2S_GRID", 8), (2, "IQ3XXS_GRID", 4)):
+        g = oracle.iq_grid(which)
+        assert g.size == want[name]["entries"]
+        assert _digest(g.tolist(), width) == want[name]["sha256"], name
+        for i, v in want[name]["spot"].items():
+            assert int(g[int(i)]) == v
+    # the product's and the oracle's packed files, expanded by the rule
+    for rel in (("runnburn_amd", "csrc", "iq_grids_packed.inc"), ("oracle", "iq_grids.inc")):
+        t = _packed_inc_tables(os.path.join(root, *rel))
+        assert _digest([_expand2(w) for w in t["kIq2xxsPacked"]], 8) == want["IQ2XXS_GRID"]["sha256"], rel
+        assert _digest([_expand2(w) for w in t["kIq2sPacked"]], 8) == want["IQ2S_GRID"]["sha256"], rel
+        assert _digest([_expand3(w) for w in t["kIq3xxsPacked"]], 4) == want["IQ3XXS_GRID"]["sha256"], rel
+    # the sign table: seven bits and their parity
+    signs = [i | (bin(i).count("1") & 1) << 7 for i in range(128)]
+    assert _digest(signs, 1) == want["KSIGNS_IQ2XS"]["sha256"]
+    # the IQ4_NL values through the oracle's IQ4_XS dequantiser: d = 1, every group scale 33 (dl = 1), nibble k at element k
+    blk = np.zeros(136, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.uint16(0xAAAA).tobytes(), np.uint8)  # high scale bits 2 for all eight groups: 32 + low nibble
+    blk[4:8] = 0x11                                                   # low nibbles 1: ls = 33
+    qs = blk[8:]
+    for j in range(16):
+        qs[j] = (j & 0x0F) | (((j + 1) & 0x0F) << 4)  # element j: nibble j; element j + 16: nibble j + 1
+    vals = oracle.dequantize(23, blk)[:16].astype(np.int64).tolist()
+    assert _digest(vals, 1, signed=True) == want["KVALUES_IQ4NL"]["sha256"]
+
+
 @pytest.mark.parametrize("quant", [16, 22, 18, 23])
 def test_iq_dots_equal_the_dequantised_statement(oracle, quant):
     """dot(W, Q8_K(x)) restated independently: f64 sum of dequantise(W) * (d_x * q_x).  The integer forms of
