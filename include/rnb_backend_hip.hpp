@@ -211,7 +211,10 @@ inline Result<Unit> prewarm_weights(const std::vector<Bytes> &ranges) {
 inline Result<std::vector<float>> qwen35_sparse_experts_selected_base_by_token(
     Bytes gate_all, Bytes up_all, Bytes down_all, const std::vector<uint32_t> &expert_ids,
     const std::vector<float> &route_weights, const std::vector<uint32_t> &token_ids, size_t token_count,
-    uint32_t down_quant, size_t n_ff, size_t n_embd, Floats input) {
+    uint32_t down_quant, size_t n_ff, size_t n_embd, Floats input, Bytes shared_gate = Bytes{}, Bytes shared_up = Bytes{},
+    Bytes shared_down = Bytes{}) {
+    // shared_*: the shared expert (slot id n_expert with the shared gate's scalar as its weight, the extra slot of the
+    // decode call in crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:804-812); empty = none
     if (route_weights.size() != expert_ids.size() || token_ids.size() != expert_ids.size()) {
         Result<std::vector<float>> r;
         r.status = RNB_HIP_INVALID_REQUEST;
@@ -221,7 +224,8 @@ inline Result<std::vector<float>> qwen35_sparse_experts_selected_base_by_token(
     }
     std::vector<float> out(token_count * n_embd);
     const int st = rnb_hip_moe_sparse_experts_by_token(
-        gate_all.ptr, gate_all.len, up_all.ptr, up_all.len, down_all.ptr, down_all.len, expert_ids.data(),
+        gate_all.ptr, gate_all.len, up_all.ptr, up_all.len, down_all.ptr, down_all.len, shared_gate.ptr, shared_gate.len,
+        shared_up.ptr, shared_up.len, shared_down.ptr, shared_down.len, expert_ids.data(),
         route_weights.data(), token_ids.data(), expert_ids.size(), token_count, down_quant, n_ff, n_embd, input.ptr,
         input.len, out.data(), out.size());
     if (st != RNB_HIP_OK) return make_err<std::vector<float>>(st);

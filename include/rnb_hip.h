@@ -247,10 +247,20 @@ int rnb_hip_q8_0_head_gemv_batch(const uint8_t *w, size_t w_len, size_t head_cou
  * expert tensors + per-slot (expert id, route weight, token id).  Gate/up are Q4_K
  * [n_expert][n_ff][n_embd]; down is [n_expert][n_embd][n_ff] in `down_quant` (12 = Q4_K,
  * 13 = Q5_K, 14 = Q6_K).  out[token][n_embd] = sum over that token's slots, in slot order, of
- * route * W_down[e] . Q8_K(silu(W_gate[e] . Q8_K(x)) * (W_up[e] . Q8_K(x))). */
+ * route * W_down[e] . Q8_K(silu(W_gate[e] . Q8_K(x)) * (W_up[e] . Q8_K(x))).
+ * The shared expert: the reference's decode call appends it to the slot list as expert id n_expert
+ * with the shared gate's scalar as its route weight and its three tensors beside the routed ones
+ * (crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:804-812; the id form is
+ * qwen_moe_decode_sparse_experts_id_into, crates/rnb-llm/src/engine/backend_runtime/qwen_moe.rs:
+ * 2807-2825).  shared_gate / shared_up / shared_down are those tensors, one expert's bytes each in
+ * the routed experts' formats (the reference's condition, fanout.rs:790-803), or all three NULL;
+ * with them a slot may carry expert id n_expert, without them that id is out of range. */
 int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len,
                                         const uint8_t *up_all, size_t up_len,
                                         const uint8_t *down_all, size_t down_len,
+                                        const uint8_t *shared_gate, size_t shared_gate_len,
+                                        const uint8_t *shared_up, size_t shared_up_len,
+                                        const uint8_t *shared_down, size_t shared_down_len,
                                         const uint32_t *expert_ids, const float *route_weights,
                                         const uint32_t *token_ids, size_t n_slots,
                                         size_t token_count, uint32_t down_quant, size_t n_ff,
@@ -313,9 +323,12 @@ int rnb_hip_rms_norm_add_rms_norm_quantize_dev(const float *input_dev, const flo
 int rnb_hip_moe_route_topk_dev(const float *logits_dev, size_t token_count, size_t n_expert, size_t k, uint32_t *idx_dev,
                                float *weights_dev);
 /* device-resident form of rnb_hip_moe_sparse_experts_by_token: weights, x and out on the device;
- * the slot arrays stay on the host (the caller routes on the host, as the reference does). */
+ * the slot arrays stay on the host (the caller routes on the host, as the reference does).  The
+ * shared expert's tensors (one expert each, on the device) or three NULLs. */
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev,
                                             const void *down_dev, size_t n_expert,
+                                            const void *shared_gate_dev, const void *shared_up_dev,
+                                            const void *shared_down_dev,
                                             const uint32_t *expert_ids,
                                             const float *route_weights, const uint32_t *token_ids,
                                             size_t n_slots, size_t token_count,

@@ -76,7 +76,7 @@ SYMBOLS = [
     ("rnb_hip_q8_0_gemv_batch", _i, _MATMUL_ARGS),
     ("rnb_hip_q8_0_head_gemv_batch", _i, [_vp, _sz, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_moe_sparse_experts_by_token", _i,
-     [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
+     [_vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_dev_alloc", _vp, [_sz]),
     ("rnb_hip_dev_free", _i, [_vp]),
     ("rnb_hip_dev_upload", _i, [_vp, _vp, _sz]),
@@ -91,7 +91,7 @@ SYMBOLS = [
     ("rnb_hip_moe_route_topk_dev", _i, [_vp, _sz, _sz, _sz, _vp, _vp]),
     ("rnb_hip_gemv_quantized_dev", _i, [_u32, _vp, _sz, _sz, _sz, _vp]),
     ("rnb_hip_moe_sparse_experts_by_token_dev", _i,
-     [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
+     [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _u32, _sz, _sz, _vp, _vp]),
     ("rnb_hip_q6k_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
     ("rnb_hip_dense_q4k_attention_qkv", _i, [_vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz]),
     ("rnb_hip_q8_0_gemv_argmax", _i, [_vp, _sz, _sz, _sz, _vp, _sz, C.POINTER(_u32), C.POINTER(C.c_float)]),
@@ -477,9 +477,12 @@ def q8_0_head_gemv_batch(weights, head_count: int, rows_per_head: int, cols: int
 
 def qwen35_sparse_experts_selected_base_by_token(gate_all, up_all, down_all, expert_ids, route_weights, token_ids,
                                                  token_count: int, down_quant: int, n_ff: int, n_embd: int,
-                                                 input) -> np.ndarray:  # noqa: A002
-    """api/qwen_moe_api.rs:2529-2541; returns out[token_count][n_embd]."""
+                                                 input, shared=None) -> np.ndarray:  # noqa: A002
+    """api/qwen_moe_api.rs:2529-2541; returns out[token_count][n_embd].  `shared`: the shared expert's (gate, up, down)
+    bytes; slots with expert id n_expert then run on it (the decode call's extra slot, moe_view/fanout.rs:804-812)."""
     g, u, d = _bytes_view(gate_all), _bytes_view(up_all), _bytes_view(down_all)
+    sh = [_bytes_view(a) for a in shared] if shared is not None else []
+    sh_args = [v for a in sh for v in (_ptr(a), a.size)] if sh else [None, 0, None, 0, None, 0]
     e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
     r = _f32(route_weights).ravel()
     t = np.ascontiguousarray(token_ids, dtype=np.uint32)
@@ -488,7 +491,7 @@ def qwen35_sparse_experts_selected_base_by_token(gate_all, up_all, down_all, exp
                               f"token={t.size}")
     x = _f32(input).ravel()
     out = np.empty((token_count, n_embd), dtype=np.float32)
-    _check(lib().rnb_hip_moe_sparse_experts_by_token(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, _ptr(e),
+    _check(lib().rnb_hip_moe_sparse_experts_by_token(_ptr(g), g.size, _ptr(u), u.size, _ptr(d), d.size, *sh_args, _ptr(e),
                                                      _ptr(r), _ptr(t), e.size, token_count, down_quant, n_ff, n_embd,
                                                      _ptr(x), x.size, _ptr(out), out.size))
     return out
@@ -595,11 +598,13 @@ def gemv_quantized_dev(quant: int, w: DeviceBuffer, rows: int, cols: int, seq_le
 
 def moe_sparse_experts_by_token_dev(gate: DeviceBuffer, up: DeviceBuffer, down: DeviceBuffer, n_expert: int,
                                     expert_ids, route_weights, token_ids, token_count: int, down_quant: int,
-                                    n_ff: int, n_embd: int, x: DeviceBuffer, out: DeviceBuffer) -> None:
+                                    n_ff: int, n_embd: int, x: DeviceBuffer, out: DeviceBuffer, shared=None) -> None:
+    """`shared`: three DeviceBuffers, the shared expert's gate, up and down (expert id n_expert in the slot list)."""
+    sh = [b.ptr for b in shared] if shared is not None else [None, None, None]
     e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
     r = _f32(route_weights).ravel()
     t = np.ascontiguousarray(token_ids, dtype=np.uint32)
-    _check(lib().rnb_hip_moe_sparse_experts_by_token_dev(gate.ptr, up.ptr, down.ptr, n_expert, _ptr(e), _ptr(r),
+    _check(lib().rnb_hip_moe_sparse_experts_by_token_dev(gate.ptr, up.ptr, down.ptr, n_expert, *sh, _ptr(e), _ptr(r),
                                                          _ptr(t), e.size, token_count, down_quant, n_ff, n_embd,
                                                          x.ptr, out.ptr))
 

@@ -529,7 +529,14 @@ struct MoeShape {
 
 // Messages: crates/rnb-backend/cuda/src/runtime/helpers.rs:1570-1600 (selected-base shape) and
 // :2747-2800 (full-layer token batch).
-int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t *expert_ids,
+// The shared expert of a call (the extra slot of the reference's decode call, fanout.rs:804-812, id n_expert): present
+// when all three tensors are given, each with one expert's length.
+struct SharedLens {
+    bool any = false, all = false;
+    size_t gate = 0, up = 0, down = 0;
+};
+
+int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const SharedLens &shared, const uint32_t *expert_ids,
                  const uint32_t *token_ids, size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff,
                  size_t n_embd, size_t x_len, size_t out_len, MoeShape *shape) {
     if (x_len != token_count * n_embd)
@@ -565,8 +572,17 @@ int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t
         return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base down length mismatch: len=" +
                                                  std::to_string(down_len) + " expected=" +
                                                  std::to_string(sh.n_expert * sh.per_down));
+    if (shared.any && !shared.all)
+        return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 shared expert needs its gate, up and down tensors together");
+    if (shared.all && (shared.gate != sh.per_gate || shared.up != sh.per_gate || shared.down != sh.per_down))
+        return fail(RNB_HIP_INVALID_REQUEST,
+                    "Qwen35 shared expert length mismatch: gate=" + std::to_string(shared.gate) + " up=" +
+                        std::to_string(shared.up) + " down=" + std::to_string(shared.down) + " expected gate=up=" +
+                        std::to_string(sh.per_gate) + " down=" + std::to_string(sh.per_down));
+    // id n_expert names the shared expert when the call carries one
+    const size_t id_limit = sh.n_expert + (shared.all ? 1 : 0);
     for (size_t i = 0; i < n_slots; i++)
-        if (expert_ids[i] >= sh.n_expert)
+        if (expert_ids[i] >= id_limit)
             return fail(RNB_HIP_INVALID_REQUEST, "Qwen35 selected-base expert id out of range: id=" +
                                                      std::to_string(expert_ids[i]) + " n_expert=" +
                                                      std::to_string(sh.n_expert));
@@ -587,7 +603,7 @@ int validate_moe(size_t gate_len, size_t up_len, size_t down_len, const uint32_t
 constexpr size_t kMoeTokenMajorSlots = 32;
 
 // Device-side sequence for the gathered expert path.  x_dev [token_count][n_embd], out_dev likewise.
-int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev,
+int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const uint8_t *down_dev, const MoeShared &shared,
                 const MoeShape &sh, const uint32_t *expert_ids, const float *route, const uint32_t *token_ids,
                 size_t n_slots, size_t token_count, uint32_t down_quant, size_t n_ff, size_t n_embd,
                 const float *x_dev, float *out_dev) {
@@ -612,7 +628,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
                 table.token[at] = t;
             }
             RESERVE_TRY(s.moe_mid, n_slots * n_ff * sizeof(float));
-            launch_moe_decode(gate_dev, up_dev, down_dev, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
+            launch_moe_decode(gate_dev, up_dev, down_dev, shared, down_quant, table, x_dev, s.moe_mid.as<float>(), out_dev,
                               static_cast<uint32_t>(n_ff), static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_in),
                               static_cast<uint32_t>(sh.nb_mid), s.stream);
             if (int ls = check_launches(); ls != RNB_HIP_OK) return ls;
@@ -642,7 +658,8 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     // (its gate/up rows arrive as 16-byte LDS-direct loads: other alignments take the vector kernels)
     // (and the Q6_K down rows as dword-aligned pieces: an even base address and whole 128-row tiles)
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev) |
-                             reinterpret_cast<uintptr_t>(down_dev)) & 15u) == 0;
+                             reinterpret_cast<uintptr_t>(down_dev) | reinterpret_cast<uintptr_t>(shared.gate) |
+                             reinterpret_cast<uintptr_t>(shared.up) | reinterpret_cast<uintptr_t>(shared.down)) & 15u) == 0;
     const bool mfma = token_count >= kMoeMfmaMinTokens && n_slots >= 2 * n_groups && aligned16 && n_embd % 128 == 0 &&
                       moe_mfma_supported(static_cast<uint32_t>(sh.nb_in), static_cast<uint32_t>(sh.nb_mid), down_quant);
     const bool inline_tables = !mfma && table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
@@ -724,9 +741,9 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     RESERVE_TRY(s.moe_slot_out, n_slots * n_embd * sizeof(float));
     if (mfma && act.digits != nullptr) {
         // prefill: grouped GEMMs on the matrix cores; the down kernel quantises the intermediate as it stages it
-        launch_moe_gate_up_mfma(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
+        launch_moe_gate_up_mfma(gate_dev, up_dev, shared, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                                 static_cast<uint32_t>(sh.nb_in), s.stream);
-        launch_moe_down_mfma(down_dev, down_quant, s.moe_mid.as<float>(), groups, d_route, s.moe_slot_out.as<float>(),
+        launch_moe_down_mfma(down_dev, shared, down_quant, s.moe_mid.as<float>(), groups, d_route, s.moe_slot_out.as<float>(),
                              static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
                           static_cast<uint32_t>(n_embd), s.stream);
@@ -736,7 +753,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     RESERVE_TRY(s.moe_mid_qs, n_slots * n_ff);
     RESERVE_TRY(s.moe_mid_d, n_slots * sh.nb_mid * sizeof(float));
     RESERVE_TRY(s.moe_mid_bsums, n_slots * sh.nb_mid * 16 * sizeof(int16_t));
-    launch_moe_gate_up(gate_dev, up_dev, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
+    launch_moe_gate_up(gate_dev, up_dev, shared, act, groups, s.moe_mid.as<float>(), static_cast<uint32_t>(n_ff),
                        static_cast<uint32_t>(sh.nb_in), s.stream);
     const bool token_major = n_slots <= kMoeTokenMajorSlots && sh.nb_mid <= 16;
     // expert-major with short intermediates: the down kernel quantises the rows it stages, one launch fewer
@@ -748,11 +765,11 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     if (token_major) {
         // decode: few slots, every expert is read by one token anyway; one launch does down, route and the ordered sum
         const uint32_t *d_sexp = d_list + 3 * n_slots + n_groups + (n_groups + 1);
-        launch_moe_down_token(down_dev, down_quant, mid, d_off, d_list, d_sexp, d_route, out_dev,
+        launch_moe_down_token(down_dev, shared, down_quant, mid, d_off, d_list, d_sexp, d_route, out_dev,
                               static_cast<uint32_t>(token_count), static_cast<uint32_t>(n_embd),
                               static_cast<uint32_t>(sh.nb_mid), s.stream);
     } else {
-        launch_moe_down(down_dev, down_quant, mid, down_quantises ? s.moe_mid.as<float>() : nullptr, groups, d_route,
+        launch_moe_down(down_dev, shared, down_quant, mid, down_quantises ? s.moe_mid.as<float>() : nullptr, groups, d_route,
                         s.moe_slot_out.as<float>(),
                         static_cast<uint32_t>(n_embd), static_cast<uint32_t>(sh.nb_mid), s.stream);
         launch_moe_reduce(s.moe_slot_out.as<float>(), d_off, d_list, out_dev, static_cast<uint32_t>(token_count),
@@ -1119,12 +1136,18 @@ int rnb_hip_q8_0_head_gemv_batch(const uint8_t *w, size_t w_len, size_t head_cou
 
 int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len, const uint8_t *up_all,
                                         size_t up_len, const uint8_t *down_all, size_t down_len,
+                                        const uint8_t *shared_gate, size_t shared_gate_len, const uint8_t *shared_up,
+                                        size_t shared_up_len, const uint8_t *shared_down, size_t shared_down_len,
                                         const uint32_t *expert_ids, const float *route_weights,
                                         const uint32_t *token_ids, size_t n_slots, size_t token_count,
                                         uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x, size_t x_len,
                                         float *out, size_t out_len) {
     MoeShape sh;
-    int st = validate_moe(gate_len, up_len, down_len, expert_ids, token_ids, n_slots, token_count, down_quant, n_ff,
+    SharedLens sl;
+    sl.any = shared_gate != nullptr || shared_up != nullptr || shared_down != nullptr;
+    sl.all = shared_gate != nullptr && shared_up != nullptr && shared_down != nullptr;
+    sl.gate = shared_gate_len, sl.up = shared_up_len, sl.down = shared_down_len;
+    int st = validate_moe(gate_len, up_len, down_len, sl, expert_ids, token_ids, n_slots, token_count, down_quant, n_ff,
                           n_embd, x_len, out_len, &sh);
     if (st != RNB_HIP_OK) return st;
     if (token_count == 0) return RNB_HIP_OK;
@@ -1135,6 +1158,13 @@ int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len
     if (int rs = s.resident_ptr(gate_all, gate_len, &gate_dev); rs != RNB_HIP_OK) return rs;
     if (int rs = s.resident_ptr(up_all, up_len, &up_dev); rs != RNB_HIP_OK) return rs;
     if (int rs = s.resident_ptr(down_all, down_len, &down_dev); rs != RNB_HIP_OK) return rs;
+    MoeShared shared;
+    if (sl.all) {
+        if (int rs = s.resident_ptr(shared_gate, shared_gate_len, &shared.gate); rs != RNB_HIP_OK) return rs;
+        if (int rs = s.resident_ptr(shared_up, shared_up_len, &shared.up); rs != RNB_HIP_OK) return rs;
+        if (int rs = s.resident_ptr(shared_down, shared_down_len, &shared.down); rs != RNB_HIP_OK) return rs;
+        shared.n_routed = static_cast<uint32_t>(sh.n_expert);
+    }
     const size_t io_bytes = token_count * n_embd * sizeof(float);
     RESERVE_TRY(s.bounce_in, io_bytes);
     RESERVE_TRY(s.bounce_out, io_bytes);
@@ -1143,7 +1173,7 @@ int rnb_hip_moe_sparse_experts_by_token(const uint8_t *gate_all, size_t gate_len
     std::memcpy(s.bounce_in.ptr, x, io_bytes);
     HIP_TRY(hipMemcpyAsync(s.x_f32.ptr, s.bounce_in.ptr, io_bytes, hipMemcpyHostToDevice, s.stream));
     s.h2d_bytes += io_bytes;
-    st = run_moe_dev(s, gate_dev, up_dev, down_dev, sh, expert_ids, route_weights, token_ids, n_slots, token_count,
+    st = run_moe_dev(s, gate_dev, up_dev, down_dev, shared, sh, expert_ids, route_weights, token_ids, n_slots, token_count,
                      down_quant, n_ff, n_embd, s.x_f32.as<float>(), s.out_f32.as<float>());
     if (st != RNB_HIP_OK) return st;
     HIP_TRY(hipMemcpyAsync(s.bounce_out.ptr, s.out_f32.ptr, io_bytes, hipMemcpyDeviceToHost, s.stream));
@@ -1647,7 +1677,8 @@ int rnb_hip_gemv_quantized_dev(uint32_t quant, const void *w_dev, size_t rows, s
 }
 
 int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up_dev, const void *down_dev,
-                                            size_t n_expert, const uint32_t *expert_ids, const float *route_weights,
+                                            size_t n_expert, const void *shared_gate_dev, const void *shared_up_dev,
+                                            const void *shared_down_dev, const uint32_t *expert_ids, const float *route_weights,
                                             const uint32_t *token_ids, size_t n_slots, size_t token_count,
                                             uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x_dev,
                                             float *out_dev) {
@@ -1665,7 +1696,18 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
     sh.per_down = n_embd * sh.nb_mid * down_block;
     sh.n_expert = n_expert;
     MoeShape checked;
-    int st = validate_moe(n_expert * sh.per_gate, n_expert * sh.per_gate, n_expert * sh.per_down, expert_ids, token_ids,
+    SharedLens sl;
+    sl.any = shared_gate_dev != nullptr || shared_up_dev != nullptr || shared_down_dev != nullptr;
+    sl.all = shared_gate_dev != nullptr && shared_up_dev != nullptr && shared_down_dev != nullptr;
+    sl.gate = sl.up = sh.per_gate, sl.down = sh.per_down;  // device tensors carry no length: one expert each
+    MoeShared shared;
+    if (sl.all) {
+        shared.gate = static_cast<const uint8_t *>(shared_gate_dev);
+        shared.up = static_cast<const uint8_t *>(shared_up_dev);
+        shared.down = static_cast<const uint8_t *>(shared_down_dev);
+        shared.n_routed = static_cast<uint32_t>(n_expert);
+    }
+    int st = validate_moe(n_expert * sh.per_gate, n_expert * sh.per_gate, n_expert * sh.per_down, sl, expert_ids, token_ids,
                           n_slots, token_count, down_quant, n_ff, n_embd, token_count * n_embd, token_count * n_embd,
                           &checked);
     if (st != RNB_HIP_OK) return st;
@@ -1674,7 +1716,7 @@ int rnb_hip_moe_sparse_experts_by_token_dev(const void *gate_dev, const void *up
     Guard g;
     if (!g.state) return g.status;
     return run_moe_dev(*g.state, static_cast<const uint8_t *>(gate_dev), static_cast<const uint8_t *>(up_dev),
-                       static_cast<const uint8_t *>(down_dev), sh, expert_ids, route_weights, token_ids, n_slots,
+                       static_cast<const uint8_t *>(down_dev), shared, sh, expert_ids, route_weights, token_ids, n_slots,
                        token_count, down_quant, n_ff, n_embd, x_dev, out_dev);
 }
 

@@ -135,4 +135,12 @@ __device__ __forceinline__ int byte_of(uint32_t lo, uint32_t hi, int j) {
     return static_cast<int>((wsel >> ((j & 3) * 8)) & 0xffu);
 }
 
+// Expert `e` of one projection: routed experts lie back to back in `all` (base + e * bytes_per_expert, the slicing of
+// crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:4-22); ids from n_routed up name the shared
+// expert, a tensor of its own (fanout.rs:804-812).
+__device__ __forceinline__ const uint8_t *expert_base(const uint8_t *all, const uint8_t *shared, uint32_t n_routed, uint32_t e,
+                                                      size_t bytes_per_expert) {
+    return e < n_routed ? all + static_cast<size_t>(e) * bytes_per_expert : shared;
+}
+
 }  // namespace rnb

@@ -166,23 +166,31 @@ struct MoeInlineTables {
 void launch_quantize_q8k_with_tables(const float *x, size_t n_blocks, int8_t *qs, float *d, int16_t *bsums,
                                      const MoeInlineTables &tables, uint32_t n_words, uint32_t *tables_dev,
                                      hipStream_t stream);
+// The shared expert of a call: the reference's decode call appends it to the slot list as expert id n_expert with the
+// shared gate's scalar as its route weight (crates/rnb-llm/src/engine/models/shared_expert_moe/moe_view/fanout.rs:804-812);
+// its three matrices have the routed experts' shapes and formats but live in allocations of their own.  Slots whose
+// expert id is >= n_routed read these; without a shared expert the pointers are null and n_routed is UINT32_MAX.
+struct MoeShared {
+    const uint8_t *gate = nullptr, *up = nullptr, *down = nullptr;
+    uint32_t n_routed = 0xffffffffu;
+};
 // mid[slot][n_ff] = silu(Wg[e] . h_tok) * (Wu[e] . h_tok); act = Q8_K(x) per token
-void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
-                        uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
+void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, const MoeShared &shared, ActView act, MoeGroups groups,
+                        float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
 // slot_out[slot][n_embd] = route[slot] * (Wd[e] . Q8_K(mid[slot])); mid_act is indexed by slot; with mid_f32
 // ([slot][nb_mid * 256], non-null) the workgroups quantise the rows they stage themselves and mid_act is not read
 bool moe_down_quantises(uint32_t nb_mid);  // whether that pays (short intermediates)
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const float *mid_f32, MoeGroups groups,
-                     const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
+void launch_moe_down(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, ActView mid_act,
+                     const float *mid_f32, MoeGroups groups, const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // the same two steps on the matrix cores for batches (act / mid_act carry digits, except a Q6_K down's mid_act):
 // 32-token tiles per expert group, see moe_mfma.hip
 bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant);  // the tiles' LDS images fit
-void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
-                             uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
-void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const float *mid, MoeGroups groups,
+void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, const MoeShared &shared, ActView act,
+                             MoeGroups groups, float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream);
+void launch_moe_down_mfma(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, const float *mid, MoeGroups groups,
                           const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // down + route weight + ordered per-token sum in one launch (rows of at most 16 super-blocks); slot_expert [n_slots]
-void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
+void launch_moe_down_token(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
                            const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
                            uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream);
 // A few tokens (decode and small batches: at most 8 tokens and 64 slots, at most 16 slots per token): the whole expert
@@ -199,7 +207,8 @@ struct MoeDecodeTable {
 };
 // max_per_token: the largest number of slots any one token has
 bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x);
-void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
+void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, const MoeShared &shared,
+                       uint32_t down_quant,
                        const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
                        uint32_t nb_in, uint32_t nb_mid, hipStream_t stream);
 // out[token][n_embd] = sum of slot_out over the token's slots, in list order;

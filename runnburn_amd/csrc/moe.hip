@@ -85,6 +85,7 @@ __device__ __forceinline__ void stage_row_f32(uint8_t *lds, uint32_t tmax, uint3
 template <int kRowsPerWave>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
     moe_gate_up_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
+                       const uint8_t *__restrict__ gate_shared, const uint8_t *__restrict__ up_shared, uint32_t n_routed,
                        const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ abs,
                        const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
                        const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
@@ -100,7 +101,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const size_t row_bytes = static_cast<size_t>(nb) * kQ4KBytes;
-    const size_t ebase = static_cast<size_t>(expert) * n_ff * row_bytes;
+    const uint8_t *gate_e = expert_base(gate_all, gate_shared, n_routed, expert, n_ff * row_bytes);
+    const uint8_t *up_e = expert_base(up_all, up_shared, n_routed, expert, n_ff * row_bytes);
     const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
     const Staged st = stage_layout(lds, tmax, nb);
     float2 *xch = reinterpret_cast<float2 *>(lds + stage_bytes(tmax, nb)) + wave * (kMaxChunkTokens * kRowsPerWave);
@@ -119,9 +121,9 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (int t = 0; t < kMaxChunkTokens; t++) gacc[t] = uacc[t] = 0.0f;
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
-                const size_t off = ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kQ4KBytes;
-                const Q4KPrep gp = q4k_prepare(q4k_load_block(gate_all + off, g), g);
-                const Q4KPrep up = q4k_prepare(q4k_load_block(up_all + off, g), g);
+                const size_t off = static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kQ4KBytes;
+                const Q4KPrep gp = q4k_prepare(q4k_load_block(gate_e + off, g), g);
+                const Q4KPrep up = q4k_prepare(q4k_load_block(up_e + off, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
                     if (static_cast<uint32_t>(t) < nt) {
@@ -166,7 +168,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // kFromF32: the intermediates come as f32 rows (mid_f32[slot][nb * 256]) and are quantised while they are staged
 template <uint32_t kQuant, int kRowsPerWave, bool kFromF32>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
-    moe_down_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq, const float *__restrict__ md,
+    moe_down_kernel(const uint8_t *__restrict__ down_all, const uint8_t *__restrict__ down_shared, uint32_t n_routed,
+                    const int8_t *__restrict__ mq, const float *__restrict__ md,
                     const int16_t *__restrict__ mbs, const float *__restrict__ mid_f32,
                     const uint32_t *__restrict__ grp_expert,
                     const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
@@ -185,7 +188,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
-    const size_t ebase = static_cast<size_t>(expert) * n_embd * row_bytes;
+    const uint8_t *down_e = expert_base(down_all, down_shared, n_routed, expert, n_embd * row_bytes);
     const uint32_t rows_per_wg = kWavesPerWg * kRowsPerWave * iters;
     const Staged st = stage_layout(lds, tmax, nb);
 
@@ -208,7 +211,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
             for (int t = 0; t < kMaxChunkTokens; t++) acc[t] = 0.0f;
             for (uint32_t b = bslot; b < nb; b += kBlocksPerPass) {
                 if (!row_ok) break;
-                const uint8_t *blk = down_all + ebase + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
+                const uint8_t *blk = down_e + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
                 const typename Q::Prep p = Q::prepare(Q::load_block(blk, g), g);
 #pragma unroll
                 for (int t = 0; t < kMaxChunkTokens; t++) {
@@ -241,7 +244,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant, int kGroups>
 __global__ void __launch_bounds__(kWave *kWavesPerWg)
-    moe_down_token_kernel(const uint8_t *__restrict__ down_all, const int8_t *__restrict__ mq,
+    moe_down_token_kernel(const uint8_t *__restrict__ down_all, const uint8_t *__restrict__ down_shared, uint32_t n_routed,
+                          const int8_t *__restrict__ mq,
                           const float *__restrict__ md, const int16_t *__restrict__ mbs,
                           const uint32_t *__restrict__ tok_offsets, const uint32_t *__restrict__ tok_slots,
                           const uint32_t *__restrict__ slot_expert, const float *__restrict__ slot_route,
@@ -266,8 +270,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
         float o = 0.0f;
         if (k < end && has_block) {
             const uint32_t slot = tok_slots[k];
-            const uint8_t *blk = down_all + (static_cast<size_t>(slot_expert[slot]) * n_embd + row) * row_bytes +
-                                 static_cast<size_t>(b) * kBlockBytes;
+            const uint8_t *blk = expert_base(down_all, down_shared, n_routed, slot_expert[slot], n_embd * row_bytes) +
+                                 static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
             const size_t ab = static_cast<size_t>(slot) * nb + b;
             o = kquant_partial<kQuant>(Q::load_block(blk, g), Q::load_act(mq + ab * 256, md[ab], mbs + ab * 16, g), g);
         }
@@ -300,7 +304,8 @@ constexpr int kDecodeWaves = 8;
 template <int kRowsPerWave, bool kOne>
 __global__ void __launch_bounds__(kWave *kDecodeWaves)
     moe_decode_gate_up_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
-                              const float *__restrict__ x, const MoeDecodeTable table, float *__restrict__ mid,
+                              const uint8_t *__restrict__ gate_shared, const uint8_t *__restrict__ up_shared,
+                              uint32_t n_routed, const float *__restrict__ x, const MoeDecodeTable table, float *__restrict__ mid,
                               uint32_t n_ff, uint32_t nb) {
     constexpr int kLanesPerRow = kWave / kRowsPerWave;
     __shared__ __attribute__((aligned(16))) int8_t s_qs[16 * 256];
@@ -319,9 +324,10 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     TokenSpans<kDecodeWaves> xv;
     token_load<kDecodeWaves>(x + (kOne ? 0 : static_cast<size_t>(table.token[slot]) * nb * 256), nb, wave, lane, xv);
     // dead lanes read the expert's first block
-    const size_t off = static_cast<size_t>(table.expert[slot]) * n_ff * row_bytes +
-                       (live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0);
-    const Q4KRegs rg = q4k_load_block(gate_all + off, g), ru = q4k_load_block(up_all + off, g);
+    const size_t off = live ? static_cast<size_t>(row) * row_bytes + static_cast<size_t>(bslot) * kQ4KBytes : 0;
+    const uint32_t expert = table.expert[slot];
+    const Q4KRegs rg = q4k_load_block(expert_base(gate_all, gate_shared, n_routed, expert, n_ff * row_bytes) + off, g),
+                  ru = q4k_load_block(expert_base(up_all, up_shared, n_routed, expert, n_ff * row_bytes) + off, g);
     token_quantize<kDecodeWaves>(xv, nb, wave, lane, s_qs, s_d, s_bsums);
     __syncthreads();
     const uint32_t ab = bslot < nb ? bslot : 0;
@@ -339,7 +345,8 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
 
 template <uint32_t kQuant, int kGroups, bool kOne>
 __global__ void __launch_bounds__(kWave *kDecodeWaves)
-    moe_decode_down_kernel(const uint8_t *__restrict__ down_all, const float *__restrict__ mid, const MoeDecodeTable table,
+    moe_decode_down_kernel(const uint8_t *__restrict__ down_all, const uint8_t *__restrict__ down_shared, uint32_t n_routed,
+                           const float *__restrict__ mid, const MoeDecodeTable table,
                            float *__restrict__ out, uint32_t n_embd, uint32_t nb) {
     constexpr int kLanes = kWave / kGroups;  // lanes per (slot, row) pair
     constexpr int kSpans = 64 / kDecodeWaves;
@@ -371,9 +378,11 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     }
     auto fetch = [&](uint32_t k, bool *ok) {
         *ok = lane_ok && k < n_slots;
-        const size_t off = *ok ? (static_cast<size_t>(table.expert[first + k]) * n_embd + row) * row_bytes + static_cast<size_t>(b) * kBlockBytes
-                               : 0;  // dead lanes read the first block of the tensor
-        return Q::load_block(down_all + off, g);
+        const uint8_t *blk = down_all;  // dead lanes read the first block of the tensor
+        if (*ok)
+            blk = expert_base(down_all, down_shared, n_routed, table.expert[first + k], n_embd * row_bytes) +
+                  static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
+        return Q::load_block(blk, g);
     };
     bool cur_ok;
     typename Q::Regs cur = fetch(grp, &cur_ok);
@@ -483,8 +492,8 @@ int rows_per_wave_for(uint32_t nb) { return nb <= 4 ? 4 : (nb <= 8 ? 2 : 1); }
 
 }  // namespace
 
-void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
-                        uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
+void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, const MoeShared &shared, ActView act, MoeGroups groups,
+                        float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0) return;
     const int rpw = rows_per_wave_for(nb_in);
     const TilePlan p = plan_tiles(n_ff, nb_in, groups.n_groups, rpw);
@@ -492,8 +501,8 @@ void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView 
     // staged activations, then one (gate, up) exchange slot per wave, staged token and row
     const size_t lds_bytes = p.lds_bytes + kWavesPerWg * kMaxChunkTokens * 4 * sizeof(float2);
 #define RNB_LAUNCH_GU(R)                                                                                             \
-    hipLaunchKernelGGL(moe_gate_up_kernel<R>, grid, block, lds_bytes, stream, gate_all, up_all, act.qs, act.d,        \
-                       act.bsums, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff,   \
+    hipLaunchKernelGGL(moe_gate_up_kernel<R>, grid, block, lds_bytes, stream, gate_all, up_all, shared.gate, shared.up, \
+                       shared.n_routed, act.qs, act.d, act.bsums, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff,   \
                        nb_in, p.iters, p.tmax)
     if (rpw == 4)
         RNB_LAUNCH_GU(4);
@@ -507,19 +516,19 @@ void launch_moe_gate_up(const uint8_t *gate_all, const uint8_t *up_all, ActView 
 // every workgroup of an expert group repeats the quantisation of the group's rows: worth it for short intermediates
 bool moe_down_quantises(uint32_t nb_mid) { return nb_mid <= 8; }
 
-void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const float *mid_f32, MoeGroups groups,
-                     const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
+void launch_moe_down(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, ActView mid_act,
+                     const float *mid_f32, MoeGroups groups, const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (groups.n_groups == 0) return;
     const int rpw = rows_per_wave_for(nb_mid);
     const TilePlan p = plan_tiles(n_embd, nb_mid, groups.n_groups, rpw);
     const dim3 grid(p.tiles, groups.n_groups, 1), block(kWave * kWavesPerWg);
 #define RNB_LAUNCH_DOWN(Q, R)                                                                                             \
-    hipLaunchKernelGGL((moe_down_kernel<Q, R, false>), grid, block, p.lds_bytes, stream, down_all, mid_act.qs, mid_act.d, \
-                       mid_act.bsums, nullptr, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out,     \
+    hipLaunchKernelGGL((moe_down_kernel<Q, R, false>), grid, block, p.lds_bytes, stream, down_all, shared.down,           \
+                       shared.n_routed, mid_act.qs, mid_act.d, mid_act.bsums, nullptr, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out,     \
                        n_embd, nb_mid, p.iters, p.tmax)
 #define RNB_LAUNCH_DOWN_F32(Q, R)                                                                                         \
-    hipLaunchKernelGGL((moe_down_kernel<Q, R, true>), grid, block, p.lds_bytes, stream, down_all, nullptr, nullptr,       \
-                       nullptr, mid_f32, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd,   \
+    hipLaunchKernelGGL((moe_down_kernel<Q, R, true>), grid, block, p.lds_bytes, stream, down_all, shared.down,            \
+                       shared.n_routed, nullptr, nullptr, nullptr, mid_f32, groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd,   \
                        nb_mid, p.iters, p.tmax)
     if (mid_f32 != nullptr)
         RNB_DISPATCH_KQUANT(down_quant, rpw, RNB_LAUNCH_DOWN_F32);
@@ -529,14 +538,14 @@ void launch_moe_down(const uint8_t *down_all, uint32_t down_quant, ActView mid_a
 #undef RNB_LAUNCH_DOWN
 }
 
-void launch_moe_down_token(const uint8_t *down_all, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
+void launch_moe_down_token(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, ActView mid_act, const uint32_t *tok_offsets,
                            const uint32_t *tok_slots, const uint32_t *slot_expert, const float *slot_route, float *out,
                            uint32_t token_count, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (token_count == 0) return;
     const dim3 grid((n_embd + kWavesPerWg - 1) / kWavesPerWg, token_count, 1), block(kWave * kWavesPerWg);
 #define RNB_LAUNCH_DT(Q, G)                                                                                           \
-    hipLaunchKernelGGL((moe_down_token_kernel<Q, G>), grid, block, 0, stream, down_all, mid_act.qs, mid_act.d,        \
-                       mid_act.bsums, tok_offsets, tok_slots, slot_expert, slot_route, out, n_embd, nb_mid)
+    hipLaunchKernelGGL((moe_down_token_kernel<Q, G>), grid, block, 0, stream, down_all, shared.down, shared.n_routed, \
+                       mid_act.qs, mid_act.d, mid_act.bsums, tok_offsets, tok_slots, slot_expert, slot_route, out, n_embd, nb_mid)
     RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DT);
 #undef RNB_LAUNCH_DT
 }
@@ -547,18 +556,20 @@ bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token,
            max_per_token * nb_mid <= 64 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
-void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, uint32_t down_quant,
-                       const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
+void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, const MoeShared &shared,
+                       uint32_t down_quant, const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,
                        uint32_t nb_in, uint32_t nb_mid, hipStream_t stream) {
     const dim3 block(kWave * kDecodeWaves);
     {
         const int rpw = rows_per_wave_for(nb_in);
         const uint32_t row_groups = (n_ff + rpw - 1) / rpw;
         const dim3 grid((row_groups + kDecodeWaves - 1) / kDecodeWaves, table.n_slots, 1);
-#define RNB_LAUNCH_DGU1(Q, R) \
-    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, true>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
-#define RNB_LAUNCH_DGU(Q, R) \
-    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, false>), grid, block, 0, stream, gate_all, up_all, x, table, mid, n_ff, nb_in)
+#define RNB_LAUNCH_DGU1(Q, R)                                                                                      \
+    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, true>), grid, block, 0, stream, gate_all, up_all, shared.gate, \
+                       shared.up, shared.n_routed, x, table, mid, n_ff, nb_in)
+#define RNB_LAUNCH_DGU(Q, R)                                                                                        \
+    hipLaunchKernelGGL((moe_decode_gate_up_kernel<R, false>), grid, block, 0, stream, gate_all, up_all, shared.gate, \
+                       shared.up, shared.n_routed, x, table, mid, n_ff, nb_in)
         if (table.n_tokens == 1)
             RNB_DISPATCH_KQUANT_R(kQ4K, rpw, RNB_LAUNCH_DGU1);
         else
@@ -567,10 +578,12 @@ void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uin
 #undef RNB_LAUNCH_DGU1
     }
     const dim3 grid((n_embd + kDecodeWaves - 1) / kDecodeWaves, table.n_tokens, 1);
-#define RNB_LAUNCH_DD1(Q, G) \
-    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, true>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
-#define RNB_LAUNCH_DD(Q, G) \
-    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, false>), grid, block, 0, stream, down_all, mid, table, out, n_embd, nb_mid)
+#define RNB_LAUNCH_DD1(Q, G)                                                                                     \
+    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, true>), grid, block, 0, stream, down_all, shared.down,       \
+                       shared.n_routed, mid, table, out, n_embd, nb_mid)
+#define RNB_LAUNCH_DD(Q, G)                                                                                       \
+    hipLaunchKernelGGL((moe_decode_down_kernel<Q, G, false>), grid, block, 0, stream, down_all, shared.down,      \
+                       shared.n_routed, mid, table, out, n_embd, nb_mid)
     if (table.n_tokens == 1)
         RNB_DISPATCH_KQUANT(down_quant, rows_per_wave_for(nb_mid), RNB_LAUNCH_DD1);
     else

@@ -261,6 +261,7 @@ __device__ __forceinline__ void tile_image_fill(const TileImage<kStride, kDigits
 template <int kJ, int kW>
 __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * kW), amdgpu_waves_per_eu(2)))
     moe_gate_up_mfma_kernel(const uint8_t *__restrict__ gate_all, const uint8_t *__restrict__ up_all,
+                            const uint8_t *__restrict__ gate_shared, const uint8_t *__restrict__ up_shared, uint32_t n_routed,
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const uint8_t *__restrict__ adig,
                             const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
                             const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
@@ -281,8 +282,9 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
     const uint32_t row_bytes = nb * static_cast<uint32_t>(kQ4KBytes);
     // the wave's first row (a wave wholly past the end streams the last row and stores nothing)
     const uint32_t first = min(blockIdx.x * (32 * kW) + wave * 32, n_ff - 1);
-    const size_t woff = (static_cast<size_t>(expert) * n_ff + first) * row_bytes;
-    const uint8_t *gbase = gate_all + woff, *ubase = up_all + woff;
+    const size_t per_expert = static_cast<size_t>(n_ff) * row_bytes, woff = static_cast<size_t>(first) * row_bytes;
+    const uint8_t *gbase = expert_base(gate_all, gate_shared, n_routed, expert, per_expert) + woff,
+                  *ubase = expert_base(up_all, up_shared, n_routed, expert, per_expert) + woff;
     // piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at byte 16 c of
     // the strip, which puts the rows 144 bytes apart (rows past the end of the matrix repeat the last row; the pieces past
     // 288 of the fifth instruction repeat the last piece and land behind the rows)
@@ -350,7 +352,8 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
 // ---------------------------------------------------------------------------------------------
 template <uint32_t kQuant, int kJ>
 __global__ void __launch_bounds__(kGbThreads, 2)
-    moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const float *__restrict__ mid,
+    moe_down_mfma_kernel(const uint8_t *__restrict__ down_all, const uint8_t *__restrict__ down_shared, uint32_t n_routed,
+                         const float *__restrict__ mid,
                          const uint32_t *__restrict__ grp_expert,
                          const uint32_t *__restrict__ grp_start, const uint32_t *__restrict__ sorted_slot,
                          const float *__restrict__ slot_route, float *__restrict__ slot_out, uint32_t n_embd, uint32_t nb,
@@ -368,6 +371,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const size_t row_bytes = static_cast<size_t>(nb) * kBlockBytes;
+    const uint8_t *down_e = expert_base(down_all, down_shared, n_routed, expert, n_embd * row_bytes);
     // The workgroup walks tiles_per_wg row tiles of 128 against one staged token tile: map and image are made once,
     // and the weight blocks of the whole walk form one stream that is requested one block ahead across row tiles.
     const uint32_t row_tiles = (n_embd + kGbRows - 1) / kGbRows;
@@ -375,7 +379,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     const uint32_t steps = rt_n * nb;
     auto row_of = [&](uint32_t rt) { return (rt0 + rt) * kGbRows + wave * 32 + lrow; };
     auto block_ptr = [&](uint32_t rt, uint32_t b) {
-        return down_all + (static_cast<size_t>(expert) * n_embd + min(row_of(rt), n_embd - 1)) * row_bytes + b * kBlockBytes;
+        return down_e + static_cast<size_t>(min(row_of(rt), n_embd - 1)) * row_bytes + b * kBlockBytes;
     };
     // Q6_K rows come in by whole cache lines through the wave's strip of LDS (RowRoute: the lane-owns-row loads of
     // q6_load_row touch 64 lines per instruction); the other formats' 16-byte loads go straight to the lane
@@ -388,7 +392,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     float d_next = 0.0f;
     auto q6_request = [&](uint32_t rt, uint32_t b) {  // block b of row tile rt: pieces into route.v, d into d_next
         const uint32_t first = (rt0 + rt) * kGbRows + wave * 32;  // the wave's first row
-        q6dw_load(route, down_all + (static_cast<size_t>(expert) * n_embd + first) * row_bytes + b * kBlockBytes, lane);
+        q6dw_load(route, down_e + static_cast<size_t>(first) * row_bytes + b * kBlockBytes, lane);
         d_next = ld_f16(block_ptr(rt, b) + 208);
     };
     auto q6_take = [&](Q6Row &r) {
@@ -519,8 +523,8 @@ bool moe_mfma_supported(uint32_t nb_in, uint32_t nb_mid, uint32_t down_quant) {
     return nb_in >= 1 && nb_mid >= 1 && gate_up_tile_tokens(nb_in) >= kMmMinToks && down_tile_tokens(nb_mid, down_quant) >= kMmMinToks;
 }
 
-void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, ActView act, MoeGroups groups, float *mid,
-                             uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
+void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, const MoeShared &shared, ActView act,
+                             MoeGroups groups, float *mid, uint32_t n_ff, uint32_t nb_in, hipStream_t stream) {
     if (groups.n_groups == 0 || n_ff == 0) return;
     const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
     if (toks == 0) return;  // moe_mfma_supported said no
@@ -531,8 +535,8 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
     // tiles of at most 8 / 16 / 32 tokens: the kernel finishes only that many results per lane
 #define RNB_LAUNCH_GUW(J, W)                                                                                          \
     if (!allow_lds<J * 16 + W>(moe_gate_up_mfma_kernel<J, W>, kMmLdsLimit)) return;                                   \
-    hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, act.qs, act.d, \
-                       act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
+    hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, shared.gate, \
+                       shared.up, shared.n_routed, act.qs, act.d, act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
 #define RNB_LAUNCH_GU(J) RNB_LAUNCH_GUW(J, kGbWaves)
     if (toks <= 8) {
         RNB_LAUNCH_GU(1);
@@ -545,7 +549,7 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, Act
 #undef RNB_LAUNCH_GUW
 }
 
-void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const float *mid, MoeGroups groups,
+void launch_moe_down_mfma(const uint8_t *down_all, const MoeShared &shared, uint32_t down_quant, const float *mid, MoeGroups groups,
                           const float *slot_route, float *slot_out, uint32_t n_embd, uint32_t nb_mid, hipStream_t stream) {
     if (groups.n_groups == 0 || n_embd == 0) return;
     // A workgroup's setup (group, map, image: a chain of dependent loads) costs more than a row tile's few blocks, and
@@ -560,7 +564,7 @@ void launch_moe_down_mfma(const uint8_t *down_all, uint32_t down_quant, const fl
     if (toks == 0) return;
 #define RNB_LAUNCH_DMJ(Q, J, LDS)                                                                                     \
     if (!allow_lds<static_cast<int>(Q) * 8 + J>(moe_down_mfma_kernel<Q, J>, Q == kQ6K ? kMmQ6DownLdsLimit : kMmLdsLimit)) return; \
-    hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, mid,                         \
+    hipLaunchKernelGGL((moe_down_mfma_kernel<Q, J>), grid, block, LDS, stream, down_all, shared.down, shared.n_routed, mid, \
                        groups.expert, groups.start, groups.sorted_slot, slot_route, slot_out, n_embd, nb_mid, tiles_per_wg, toks)
 #define RNB_LAUNCH_DM(Q, LDS)                                                                                         \
     if (toks <= 8) {                                                                                                  \

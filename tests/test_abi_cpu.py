@@ -47,9 +47,9 @@ def test_trait_facade():
     assert ei.value.kind == "UnsupportedOp"
 
 
-def _err(fn, *args):
+def _err(fn, *args, **kwargs):
     with pytest.raises(rnb.BackendError) as ei:
-        fn(*args)
+        fn(*args, **kwargs)
     return ei.value
 
 
@@ -207,6 +207,22 @@ def test_moe_validation_messages():
     assert str(e).startswith("Qwen35 selected-base expert id out of range")
     e = _err(call, g, u, d, [0, 1], [1.0], [0], 1, 14, n_ff, n_embd, x)
     assert "length mismatch" in str(e)
+    # the shared expert (slot id n_expert, moe_view/fanout.rs:804-812): all three tensors, one expert's bytes each
+    sg, su, sd = z(per_gate, np.uint8), z(per_gate, np.uint8), z(per_down, np.uint8)
+    e = _err(call, g, u, d, [3], [1.0], [0], 1, 14, n_ff, n_embd, x, shared=(sg, su, sd))
+    assert str(e) == "Qwen35 selected-base expert id out of range: id=3 n_expert=2"
+    e = _err(call, g, u, d, [2], [1.0], [0], 1, 14, n_ff, n_embd, x, shared=(sg, su, sd[:-1]))
+    assert str(e) == ("Qwen35 shared expert length mismatch: gate=36864 up=36864 down=53759 expected gate=up=36864 "
+                      "down=53760")
+    e = _err(call, g, u, d, [2], [1.0], [0], 1, 14, n_ff, n_embd, x, shared=(sg, su[:10], sd))
+    assert str(e).startswith("Qwen35 shared expert length mismatch")
+    lib = rnb.binding.lib()
+    ptr = lambda a: a.ctypes.data  # noqa: E731
+    ids, rt, tk, out = np.array([2], np.uint32), np.ones(1, np.float32), z(1, np.uint32), z(n_embd, np.float32)
+    rc = lib.rnb_hip_moe_sparse_experts_by_token(ptr(g), g.size, ptr(u), u.size, ptr(d), d.size, ptr(sg), sg.size, None, 0,
+                                                 ptr(sd), sd.size, ptr(ids), ptr(rt), ptr(tk), 1, 1, 14, n_ff, n_embd,
+                                                 ptr(x), x.size, ptr(out), out.size)
+    assert rc == 1 and rnb.last_error() == "Qwen35 shared expert needs its gate, up and down tensors together"
 
 
 def test_quantizer_validation():

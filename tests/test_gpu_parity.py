@@ -1217,3 +1217,78 @@ def test_first_capture_of_a_process_with_fitting_calls_only_keeps_its_scratch(rn
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     proc = subprocess.run([_sys.executable, "-c", _FIRST_CAPTURE_SCRIPT], cwd=root, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0 and "REPLAY OK" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-2000:]
+
+
+# ---- the shared expert as a slot of the call: moe_view/fanout.rs:804-812 -------------------------------------------------
+
+def _with_shared(oracle, n_expert, n_ff, n_embd, tokens, k, seed, down_quant):
+    """A routed case plus a shared expert: its slot (id n_expert, weight = a gate scalar per token) is appended to every
+    token's list, as the reference's decode call does.  The oracle sees the shared expert as expert n_expert of tensors
+    one expert longer, which is what that id means."""
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, seed, down_quant)
+    sg = oracle.make_weights(Q4_K, n_ff, n_embd, seed + 100)
+    su = oracle.make_weights(Q4_K, n_ff, n_embd, seed + 101)
+    sd = oracle.make_weights(down_quant, n_embd, n_ff, seed + 102)
+    scal = 1.0 / (1.0 + np.exp(-oracle.fill_normal(tokens, seed + 103, 1.0)))  # sigmoid of the shared gate's logit
+    es, rs, ts = [], [], []
+    for tok in range(tokens):
+        m = t == tok
+        es += e[m].tolist() + [n_expert]
+        rs += r[m].tolist() + [float(scal[tok])]
+        ts += [tok] * (int(m.sum()) + 1)
+    e, r, t = np.array(es, np.uint32), np.array(rs, np.float32), np.array(ts, np.uint32)
+    longer = tuple(np.concatenate([a, b]) for a, b in ((gate, sg), (up, su), (down, sd)))
+    return gate, up, down, (sg, su, sd), longer, x, e, r, t
+
+
+@pytest.mark.parametrize("tokens,n_ff,n_embd,k,down_quant", [(1, 768, 2048, 8, Q6_K), (1, 512, 1280, 15, Q5_K), (1, 256, 512, 1, Q4_K),
+                                                            (1, 256, 768, 17, Q6_K), (4, 768, 2048, 7, Q6_K), (8, 512, 768, 3, Q4_K),
+                                                            (12, 768, 1024, 4, Q6_K), (40, 512, 768, 3, Q5_K)])
+def test_moe_shared_expert_slot(rnb, oracle, tokens, n_ff, n_embd, k, down_quant):
+    """Decode (two launches), small batches, the token-major and the expert-major general sequences, each with the
+    shared expert as the last slot of every token: equal to the oracle run on tensors that hold the shared expert as
+    expert n_expert, and bit-equal to the product run on those longer tensors without a shared expert."""
+    n_expert = 12
+    gate, up, down, shared, longer, x, e, r, t = _with_shared(oracle, n_expert, n_ff, n_embd, tokens, k, 300 + tokens + k, down_quant)
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x,
+                                                           shared=shared)
+    ref = oracle.moe_sparse_experts_by_token(*longer, n_expert + 1, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    check_close(got, ref, None, f"moe shared tokens {tokens} k {k}")
+    same = rnb.qwen35_sparse_experts_selected_base_by_token(*longer, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    assert np.array_equal(got, same)
+    # the shared expert alone (no routed slot)
+    only = e == n_expert
+    got1 = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e[only], r[only], t[only], tokens, down_quant,
+                                                            n_ff, n_embd, x, shared=shared)
+    ref1 = oracle.moe_sparse_experts_by_token(*longer, n_expert + 1, e[only], r[only], t[only], tokens, down_quant, n_ff,
+                                              n_embd, x)
+    check_close(got1, ref1, None, f"moe shared only tokens {tokens}")
+    # without the tensors the id is refused
+    with pytest.raises(rnb.BackendError) as err:
+        rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    assert "expert id out of range" in str(err.value)
+    for w in (gate, up, down, *shared, *longer):
+        rnb.release(w)
+
+
+def test_moe_shared_expert_slot_on_the_matrix_cores_dev(rnb, oracle):
+    """64 tokens x top-4 of 16 experts + the shared expert for every token (a group of 64 slots), device buffers: the
+    grouped matrix-core kernels read the shared tensors for that group."""
+    n_expert, n_ff, n_embd, tokens, k = 16, 512, 1024, 64, 4
+    gate, up, down, shared, longer, x, e, r, t = _with_shared(oracle, n_expert, n_ff, n_embd, tokens, k, 411, Q6_K)
+    order = np.lexsort((t, e))  # the callers' (expert, token) order
+    e, r, t = e[order], r[order], t[order]
+    bufs = [rnb.DeviceBuffer.from_host(a) for a in (gate, up, down, *shared, x)]
+    out_dev = rnb.DeviceBuffer(tokens * n_embd * 4)
+    try:
+        rnb.moe_sparse_experts_by_token_dev(bufs[0], bufs[1], bufs[2], n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, bufs[6],
+                                            out_dev, shared=bufs[3:6])
+        rnb.sync()
+        got = out_dev.to_host(np.float32).reshape(tokens, n_embd).copy()
+    finally:
+        for b in bufs + [out_dev]:
+            b.free()
+    ref = oracle.moe_sparse_experts_by_token(*longer, n_expert + 1, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
+    from oracle import flips
+    v = flips.moe_verdict(got, ref, *longer, n_expert + 1, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
+    assert v["ok"] or v["flip_aware_ok"], v
