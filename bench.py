@@ -631,14 +631,19 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
 
 # configs that --only can run alone: quant, rows, cols, tokens
 ONLY = {"cfg1": (Q8_0, 4096, 4096, 1), "cfg2": (Q4_K, 14336, 4096, 1), "cfg3a": (Q6_K, 4096, 14336, 1),
-        "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512)}
+        "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512), "q6gemm": (Q6_K, 4096, 14336, 512),
+        "moe1": 1, "moe4": 4, "moe64": 64}  # moeN: configs[4] at N tokens
 
 
 def run_only(rnb, hip, stream, name, calibration):
     """One config, 60 steps after 10 warm-ups (plus the calibration copies when asked): what a counter run profiles."""
-    quant, rows, cols, seq = ONLY[name]
     if calibration:
         calibration_copy(hip, rnb, stream)
+    if name.startswith("moe"):
+        res = bench_moe(rnb, hip, stream, ONLY[name], 0, 1234 + ONLY[name], cpu=False)
+        print(json.dumps({"only": name, "step_ms_median": res["ms_median"], "launches": res["launches"]}), flush=True)
+        return 0
+    quant, rows, cols, seq = ONLY[name]
     w_host = synth_weights(quant, rows, cols, 20240607)
     n_copies = copies_for(w_host.nbytes)
     w_dev = [rnb.DeviceBuffer.from_host(w_host) for _ in range(n_copies)]

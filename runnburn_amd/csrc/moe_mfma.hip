@@ -18,6 +18,7 @@
 #include "kernels.h"
 #include "mfma_blocks.h"
 #include <algorithm>
+#include <type_traits>
 
 namespace rnb {
 
@@ -114,7 +115,10 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const Q4KScales sc8 = unpack_q4k_scales(row.hdr.y, row.hdr.z, row.hdr.w);
     int tot[4 * kJ];
-    if constexpr (kFifth) {
+    // With at most 16 live tokens the scale costs 4 kJ <= 8 multiply-adds per sub-block on the results: fewer vector
+    // instructions than folding it into the operand (8 per sub-block and a second matrix instruction), which pays for
+    // whole tiles only.
+    if constexpr (kFifth || kJ < 4) {
 #pragma unroll
         for (int i = 0; i < 4 * kJ; i++) tot[i] = 0;
         RNB_Q45_SUB_BLOCK(0, row, tot)
@@ -265,7 +269,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
                             const int8_t *__restrict__ aq, const float *__restrict__ ad, const uint8_t *__restrict__ adig,
                             const uint32_t *__restrict__ grp_expert, const uint32_t *__restrict__ grp_start,
                             const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
-                            float *__restrict__ mid, uint32_t n_ff, uint32_t nb, uint32_t img_toks) {
+                            float *__restrict__ mid, uint32_t n_ff, uint32_t nb, uint32_t img_toks, uint32_t tiles_per_wg) {
     constexpr bool kFifth = false;
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     __shared__ TileMap s_map;
@@ -276,25 +280,34 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
     const int lrow = lane & 31, khalf = lane >> 5;
     uint8_t *strip_g = s_dyn + wave * 2 * kQ4FillBytes, *strip_u = strip_g + kQ4FillBytes;
     const uint32_t lds_g = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)strip_g)), lds_u = lds_g + kQ4FillBytes;
-    const uint32_t row = blockIdx.x * (32 * kW) + wave * 32 + lrow;
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const uint32_t row_bytes = nb * static_cast<uint32_t>(kQ4KBytes);
-    // the wave's first row (a wave wholly past the end streams the last row and stores nothing)
-    const uint32_t first = min(blockIdx.x * (32 * kW) + wave * 32, n_ff - 1);
-    const size_t per_expert = static_cast<size_t>(n_ff) * row_bytes, woff = static_cast<size_t>(first) * row_bytes;
-    const uint8_t *gbase = expert_base(gate_all, gate_shared, n_routed, expert, per_expert) + woff,
-                  *ubase = expert_base(up_all, up_shared, n_routed, expert, per_expert) + woff;
-    // piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at byte 16 c of
-    // the strip, which puts the rows 144 bytes apart (rows past the end of the matrix repeat the last row; the pieces past
-    // 288 of the fifth instruction repeat the last piece and land behind the rows)
+    const size_t per_expert = static_cast<size_t>(n_ff) * row_bytes;
+    const uint8_t *gate_e = expert_base(gate_all, gate_shared, n_routed, expert, per_expert),
+                  *up_e = expert_base(up_all, up_shared, n_routed, expert, per_expert);
+    // The workgroup walks tiles_per_wg row tiles against one staged token tile (map and image are made once: a chain of
+    // dependent loads); the weight blocks of the whole walk form one stream, requested one block ahead across row tiles.
+    const uint32_t row_tiles = (n_ff + 32 * kW - 1) / (32 * kW);
+    const uint32_t rt0 = blockIdx.x * tiles_per_wg, rt_n = min(tiles_per_wg, row_tiles - rt0);
+    // Row tile rt: the wave's first row (a wave wholly past the end streams the last row and stores nothing) and its
+    // pieces.  Piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at
+    // byte 16 c of the strip, which puts the rows 144 bytes apart (rows past the end of the matrix repeat the last row;
+    // the pieces past 288 of the fifth instruction repeat the last piece and land behind the rows)
+    const uint8_t *gbase, *ubase;
     uint32_t goff[kQ4FillInstr];
+    auto set_tile = [&](uint32_t rt) {
+        const uint32_t first = min((rt0 + rt) * (32 * kW) + wave * 32, n_ff - 1);
+        const size_t woff = static_cast<size_t>(first) * row_bytes;
+        gbase = gate_e + woff;
+        ubase = up_e + woff;
 #pragma unroll
-    for (int i = 0; i < kQ4FillInstr; i++) {
-        const uint32_t c = min(static_cast<uint32_t>(lane) + i * kWave, 32u * kQ4Pieces - 1);
-        const uint32_t r = c / kQ4Pieces, j = c - r * kQ4Pieces;
-        goff[i] = min(r, n_ff - first - 1) * row_bytes + 16 * j;
-    }
+        for (int i = 0; i < kQ4FillInstr; i++) {
+            const uint32_t c = min(static_cast<uint32_t>(lane) + i * kWave, 32u * kQ4Pieces - 1);
+            const uint32_t r = c / kQ4Pieces, j = c - r * kQ4Pieces;
+            goff[i] = min(r, n_ff - first - 1) * row_bytes + 16 * j;
+        }
+    };
     auto request = [&](uint32_t b) {
         // the strips' previous contents have been read out (the reads are ahead of these fills in program order; make
         // sure they have executed)
@@ -313,6 +326,7 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
 
     for (uint32_t tile0 = 0; tile0 < count; tile0 += img_toks) {
         // the first weight blocks do not depend on the token lists: requested before them
+        set_tile(0);
         request(0);
         const uint32_t live = min(count - tile0, img_toks);
         const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);  // padding lanes read the last live row
@@ -323,26 +337,48 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
         Q5Row cg, cu;
         take(cg, cu);
         __syncthreads();
-        float accg[4 * kJ], accu[4 * kJ];
+        // a tile of at most eight live tokens (most groups of a routed batch) finishes only a lane's first four results
+        auto walk = [&](auto jtag) {
+        constexpr int kJl = decltype(jtag)::value;
+        for (uint32_t rt = 0; rt < rt_n; rt++) {
+            const uint32_t row = (rt0 + rt) * (32 * kW) + wave * 32 + lrow;
+            float accg[4 * kJl], accu[4 * kJl];
 #pragma unroll
-        for (int i = 0; i < 4 * kJ; i++) accg[i] = accu[i] = 0.0f;
-        for (uint32_t b = 0; b < nb; b++) {
-            request(b + 1 < nb ? b + 1 : b);  // the last step reloads its own block, unused
-            const uint8_t *abase = img.act(b) + arow * kGbStride128 + 16 * khalf;
-            const uint4 dig = img.dig(b)[lrow];
-            float val[4 * kJ];
-            q45_block_tile<kFifth, kJ>(cg, abase, dig, khalf, val);
-            tile_scale_add<kJ>(img.dx(b), khalf, val, accg);
-            q45_block_tile<kFifth, kJ>(cu, abase, dig, khalf, val);
-            tile_scale_add<kJ>(img.dx(b), khalf, val, accu);
-            take(cg, cu);
-        }
-        if (row < n_ff) {
-#pragma unroll
-            for (int r = 0; r < 4 * kJ; r++) {
-                const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
-                if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
+            for (int i = 0; i < 4 * kJl; i++) accg[i] = accu[i] = 0.0f;
+            for (uint32_t b = 0; b < nb; b++) {
+                if (b + 1 < nb) {
+                    request(b + 1);
+                } else if (rt + 1 < rt_n) {  // the walk goes on: block 0 of the next row tile
+                    set_tile(rt + 1);
+                    request(0);
+                } else {
+                    request(b);  // the last step reloads its own block, unused
+                }
+                const uint8_t *abase = img.act(b) + arow * kGbStride128 + 16 * khalf;
+                const uint4 dig = img.dig(b)[lrow];
+                float val[4 * kJl];
+                q45_block_tile<kFifth, kJl>(cg, abase, dig, khalf, val);
+                tile_scale_add<kJl>(img.dx(b), khalf, val, accg);
+                q45_block_tile<kFifth, kJl>(cu, abase, dig, khalf, val);
+                tile_scale_add<kJl>(img.dx(b), khalf, val, accu);
+                take(cg, cu);
             }
+            if (row < n_ff) {
+#pragma unroll
+                for (int r = 0; r < 4 * kJl; r++) {
+                    const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
+                    if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
+                }
+            }
+        }
+        };
+        if constexpr (kJ == 2) {  // (the 32-token kernel keeps its one form: its groups are large)
+            if (live <= 8)  // workgroup-uniform
+                walk(std::integral_constant<int, 1>{});
+            else
+                walk(std::integral_constant<int, 2>{});
+        } else {
+            walk(std::integral_constant<int, kJ>{});
         }
     }
 }
@@ -530,13 +566,26 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, con
     if (toks == 0) return;  // moe_mfma_supported said no
     const int waves = kGbWaves;  // 2, 3 and 6 waves per workgroup measured within 3 % of 4 on 128 experts x top-8, 64 tokens
     const size_t lds = static_cast<size_t>(waves) * 2 * kQ4FillBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
-    const uint32_t rows_per_wg = 32 * waves;
-    const dim3 grid((n_ff + rows_per_wg - 1) / rows_per_wg, groups.n_groups, 1);
+    const uint32_t rows_per_wg = 32 * waves, row_tiles = (n_ff + rows_per_wg - 1) / rows_per_wg;
+    // A wave's time is its chain of steps (a step waits for its own fill), much the same with one workgroup on the compute
+    // unit or two; a grid of more workgroups than fit at once runs in rounds, and a last round that is partly empty costs
+    // as much as a full one.  Where merging up to three row tiles into a workgroup brings the grid down to one workgroup
+    // per compute unit, that is done: one round, map and image made once per walk (128 experts x top-8 at 64 tokens,
+    // 6 row tiles x 126 groups: 1 / 2 / 3 tiles per workgroup 55.4 / 58.4 / 53.7 us; 2 leaves half the units with two
+    // workgroups and half with one).
+    uint32_t tiles_per_wg = 1;
+    {
+        const uint64_t total = static_cast<uint64_t>(row_tiles) * groups.n_groups;
+        const uint32_t t = static_cast<uint32_t>((total + 255) / 256);
+        if (t >= 2 && t <= 3 && static_cast<uint64_t>((row_tiles + t - 1) / t) * groups.n_groups <= 256) tiles_per_wg = t;
+    }
+    const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1);
     // tiles of at most 8 / 16 / 32 tokens: the kernel finishes only that many results per lane
 #define RNB_LAUNCH_GUW(J, W)                                                                                          \
     if (!allow_lds<J * 16 + W>(moe_gate_up_mfma_kernel<J, W>, kMmLdsLimit)) return;                                   \
     hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, shared.gate, \
-                       shared.up, shared.n_routed, act.qs, act.d, act.digits, groups.expert, groups.start, groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks)
+                       shared.up, shared.n_routed, act.qs, act.d, act.digits, groups.expert, groups.start,            \
+                       groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks, tiles_per_wg)
 #define RNB_LAUNCH_GU(J) RNB_LAUNCH_GUW(J, kGbWaves)
     if (toks <= 8) {
         RNB_LAUNCH_GU(1);
