@@ -717,6 +717,9 @@ def main() -> int:
                    "graph_ms_per_step": main_res.get("graph_ms_per_step")},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic("gemv_kquant_f32_kernel<12,1>"),
+                     "traffic_source": "not measured in this run: the committed counter summary "
+                                       "profiles/gemv_q4k_cfg2_hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE "
+                                       "of this kernel on this workload, each scaled by the calibration copy's reading)",
                      "kernel": "gemv_kquant_f32_kernel<12,1> (Q8_K quantisation of the token + GEMV in one launch)",
                      "bytes_per_launch": nbytes, "kernel_ms_mean": kst["mean"], "kernel_ms_median": kst["median"],
                      "kernel_ms_p10": kst["p10"], "kernel_ms_p90": kst["p90"], "launches": kst["launches"],
