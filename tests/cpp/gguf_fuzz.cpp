@@ -127,6 +127,132 @@ void exercise(rnb_hip_gguf *g) {
     (void)sink;
 }
 
+// ---- split models: rnb_hip_gguf_open on shard files (crates/rnb-loader/src/gguf/sharded.rs) -------------------------
+// shard `no` of `count`: the three split keys as the given types/values, `n_tensors` F32 tensors of one element
+std::vector<uint8_t> shard_image(uint64_t no, uint64_t count, uint64_t total, uint32_t key_type, int n_tensors, int name_base,
+                                 bool with_no, bool with_total) {
+    Image im;
+    im.num<uint32_t>(0x46554747u);
+    im.num<uint32_t>(3);
+    im.num<uint64_t>(static_cast<uint64_t>(n_tensors));
+    im.num<uint64_t>(2 + (with_no ? 1 : 0) + (with_total ? 1 : 0));
+    im.str("general.architecture"); im.num<uint32_t>(8); im.str("llama");
+    auto integer = [&](const char *key, uint64_t v) {
+        im.str(key);
+        im.num<uint32_t>(key_type);
+        switch (key_type) {
+        case 0: case 1: im.num<uint8_t>(static_cast<uint8_t>(v)); break;
+        case 2: case 3: im.num<uint16_t>(static_cast<uint16_t>(v)); break;
+        case 4: case 5: im.num<uint32_t>(static_cast<uint32_t>(v)); break;
+        case 6: im.num<float>(static_cast<float>(v)); break;
+        case 8: im.str(std::to_string(v)); break;
+        default: im.num<uint64_t>(v); break;  // 10, 11
+        }
+    };
+    if (with_no) integer("split.no", no);
+    integer("split.count", count);
+    if (with_total) integer("split.tensors.count", total);
+    for (int t = 0; t < n_tensors; t++) {
+        im.str("t" + std::to_string(name_base + t) + ".weight");
+        im.num<uint32_t>(1); im.num<uint64_t>(1); im.num<uint32_t>(0); im.num<uint64_t>(32u * static_cast<uint64_t>(t));
+    }
+    while (im.b.size() % 32) im.b.push_back(0);
+    for (int t = 0; t < n_tensors; t++) {
+        const float v = static_cast<float>(name_base + t) + 0.25f;
+        const size_t at = im.b.size();
+        im.b.resize(at + 32, 0);
+        std::memcpy(im.b.data() + at, &v, 4);
+    }
+    return im.b;
+}
+
+bool write_file(const std::string &path, const std::vector<uint8_t> &b) {
+    FILE *f = std::fopen(path.c_str(), "wb");
+    if (!f) return false;
+    const bool ok = b.empty() || std::fwrite(b.data(), 1, b.size(), f) == b.size();
+    std::fclose(f);
+    return ok;
+}
+
+// Rounds of two to four shard files in `dir`, most of them consistent, some damaged in one place (a key's type or value,
+// a missing key, a duplicate tensor name, a wrong total, a truncated or missing shard, a file name off the pattern);
+// every shard path is opened.  A consistent set must open from every shard with all tensors, each carrying its own
+// value; a damaged one must be refused with a message (or, where the damage is invisible from the selected shard,
+// opened); the sanitizers watch the rest.
+int split_rounds(const char *dir, long rounds, Rng &rng) {
+    int bad = 0;
+    long opened = 0, refused = 0;
+    const uint32_t int_types[] = {0, 1, 2, 3, 4, 5, 10, 11};
+    for (long r = 0; r < rounds; r++) {
+        const uint64_t count = 2 + rng.below(3);
+        const int damage = static_cast<int>(rng.below(12));  // 0..4: none
+        const uint64_t victim = rng.below(count);
+        std::vector<std::string> paths;
+        uint64_t total = 0;
+        std::vector<int> per(count);
+        for (uint64_t i = 0; i < count; i++) total += static_cast<uint64_t>(per[i] = 1 + static_cast<int>(rng.below(3)));
+        int base = 0;
+        char name[96];
+        for (uint64_t i = 0; i < count; i++) {
+            uint32_t type = int_types[rng.below(8)];
+            uint64_t no = i, cnt = count, tot = total;
+            bool with_no = true, with_total = true;
+            int nb = base;
+            if (i == victim) {
+                switch (damage) {
+                case 5: type = 6; break;            // a float where an integer belongs
+                case 6: type = 8; break;            // a string
+                case 7: no = count + rng.below(3); break;
+                case 8: cnt = rng.below(2) ? 0 : count + 1; break;
+                case 9: tot = total + 1 + rng.below(2); break;
+                case 10: with_no = false; break;
+                case 11: nb = 0; break;             // names of shard zero again (no damage when the victim is shard zero)
+                default: break;
+                }
+            }
+            std::vector<uint8_t> img = shard_image(no, cnt, tot, type, per[i], nb, with_no, with_total);
+            if (i == victim && damage == 4 && rng.below(2)) img.resize(rng.below(img.size()));  // truncated shard
+            std::snprintf(name, sizeof name, "%s/f%ld-%05llu-of-%05llu.gguf", dir, r, static_cast<unsigned long long>(i + 1),
+                          static_cast<unsigned long long>(count));
+            paths.push_back(name);
+            if (!write_file(name, img)) {
+                std::printf("split rounds: cannot write %s\n", name);
+                return 1;
+            }
+            base += per[i];
+        }
+        const bool consistent = damage < 4;
+        for (uint64_t i = 0; i < count; i++) {
+            rnb_hip_gguf *h = nullptr;
+            const int rc = rnb_hip_gguf_open(paths[i].c_str(), &h);
+            if (rc == RNB_HIP_OK && h) {
+                opened++;
+                exercise(h);
+                if (consistent) {
+                    if (rnb_hip_gguf_tensor_count(h) != total) bad++;
+                    for (size_t t = 0; t < rnb_hip_gguf_tensor_count(h); t++) {
+                        rnb_hip_gguf_tensor ti;
+                        float v = 0.0f;
+                        if (rnb_hip_gguf_tensor_at(h, t, &ti) != RNB_HIP_OK || !ti.data || ti.n_bytes != 4) { bad++; continue; }
+                        std::memcpy(&v, ti.data, 4);
+                        if (v != static_cast<float>(t) + 0.25f || ti.name != "t" + std::to_string(t) + ".weight") bad++;
+                    }
+                }
+                rnb_hip_gguf_close(h);
+            } else {
+                refused++;
+                if (consistent || std::strlen(rnb_hip_last_error()) == 0) {
+                    bad++;
+                    if (bad < 5) std::printf("split round %ld shard %llu: %s\n", r, static_cast<unsigned long long>(i), rnb_hip_last_error());
+                }
+            }
+        }
+        for (const std::string &p : paths) std::remove(p.c_str());
+    }
+    std::printf("gguf_fuzz split files: %ld rounds, %ld opened, %ld refused, %d failure(s)\n", rounds, opened, refused, bad);
+    return bad;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -190,5 +316,6 @@ int main(int argc, char **argv) {
         std::free(buf);
     }
     std::printf("gguf_fuzz: %ld rounds, %ld accepted, %ld rejected, %d failure(s)\n", rounds, accepted, rejected, failures);
+    if (argc > 2) failures += split_rounds(argv[2], rounds / 40 + 20, rng);
     return failures ? 1 : 0;
 }

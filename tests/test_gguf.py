@@ -426,18 +426,20 @@ def test_gguf_tensors_run_from_the_untouched_upload(rnb, oracle, tmp_path):
             rnb.release(t.data)
 
 
-def test_reader_survives_mutated_files_under_sanitizers():
+def test_reader_survives_mutated_files_under_sanitizers(tmp_path):
     """tests/cpp/gguf_fuzz (built by __graft_entry__.build with the address and undefined-behaviour sanitizers on the
-    host side): damaged copies of a valid file, every accessor exercised on what the parser accepts."""
+    host side): damaged copies of a valid file, every accessor exercised on what the parser accepts; then sets of shard
+    files, consistent (must open from every shard with every tensor's own value) or damaged in one place (a split key's
+    type or value, a missing key, a tensor name in two shards, a wrong total, a truncated shard)."""
     import subprocess
 
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "gguf_fuzz")
     if not os.path.exists(exe):
         pytest.skip("tests/cpp/gguf_fuzz not built (run __graft_entry__.build())")
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="halt_on_error=1")
-    p = subprocess.run([exe, "60000"], capture_output=True, text=True, timeout=300, env=env)
+    p = subprocess.run([exe, "60000", str(tmp_path)], capture_output=True, text=True, timeout=300, env=env)
     assert p.returncode == 0, p.stdout[-2000:] + p.stderr[-4000:]
-    assert "0 failure(s)" in p.stdout
+    assert p.stdout.count("0 failure(s)") == 2, p.stdout[-2000:]
 
 
 @pytest.mark.gpu
