@@ -96,21 +96,53 @@ __device__ __forceinline__ void tile_stage_store(const TileStage<kThreads> &st, 
 // kJ = 1, 2 or 4: only the results of the tile's first 8 kJ tokens are finished on the vector units (result r of a lane
 // is token 8 * (r / 4) + 4 * khalf + r % 4, so they are the lane's first 4 kJ results); the matrix instructions always
 // compute all 32 tokens, which costs nothing extra.
-#define RNB_Q45_SUB_BLOCK(SB, ROW, TOT)                                                                  \
+// The matrix instruction of sub-block SB is issued before the results of sub-block SB - 1 are scaled: a wave that has
+// its SIMD to itself would otherwise sit out the instruction's latency (16 passes) eight times per block.
+#define RNB_Q45_ISSUE(SB, ROW, ACC, SC)                                                                  \
     {                                                                                                    \
         const v4i bop = q45_operand<SB, kFifth>(ROW);                                                    \
-        const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                \
-        const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * (SB));                               \
-        const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);               \
+        SC = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                          \
+        ACC = __builtin_amdgcn_mfma_i32_32x32x32_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+    }
+#define RNB_Q45_TAKE(ACC, SC, TOT)                                                                       \
+    {                                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4 * kJ; i++) {                                             \
-            TOT[i] += mul24(acc[i], sc);                                                                 \
+            TOT[i] += mul24(ACC[i], SC);                                                                 \
             asm volatile("" : "+v"(TOT[i])); /* keep the eight additions a chain, not a tree */          \
         }                                                                                                \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
+#define RNB_Q45_SUB_BLOCK(SB, ROW, TOT)                                                                  \
+    {                                                                                                    \
+        if constexpr (((SB) & 1) == 0) {                                                                 \
+            RNB_Q45_ISSUE(SB, ROW, acc_a, sc_a)                                                          \
+            if constexpr ((SB) > 0) RNB_Q45_TAKE(acc_b, sc_b, TOT)                                       \
+        } else {                                                                                         \
+            RNB_Q45_ISSUE(SB, ROW, acc_b, sc_b)                                                          \
+            RNB_Q45_TAKE(acc_a, sc_a, TOT)                                                               \
+        }                                                                                                \
+    }
+
+// The lane's activation operands of one block: token lrow's 16 bytes of each 32-element sub-block.  Read from the
+// image in one batch, before the first matrix instruction, and used for both matrices of a gate/up step: read one by
+// one in front of their instructions they cost an LDS round trip per sub-block, which a wave alone on its SIMD sits out.
+struct TileOps128 {
+    v4i v[8];
+};
+__device__ __forceinline__ void tile_ops_load(TileOps128 &o, const uint8_t *abase) {
+#pragma unroll
+    for (int sb = 0; sb < 8; sb++) o.v[sb] = *reinterpret_cast<const v4i *>(abase + 32 * sb);
+}
+struct TileOps64 {
+    long v[16];
+};
+__device__ __forceinline__ void tile_ops_load(TileOps64 &o, const uint8_t *abase) {
+#pragma unroll
+    for (int sb = 0; sb < 16; sb++) o.v[sb] = *reinterpret_cast<const long *>(abase + 16 * sb);
+}
 
 template <bool kFifth, int kJ>
-__device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *abase, const uint4 dig, int khalf,
+__device__ __forceinline__ void q45_block_tile(const Q5Row &row, const TileOps128 &aops, const uint4 dig, int khalf,
                                                float (&val)[4 * kJ]) {
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const Q4KScales sc8 = unpack_q4k_scales(row.hdr.y, row.hdr.z, row.hdr.w);
@@ -121,6 +153,8 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
     if constexpr (kFifth || kJ < 4) {
 #pragma unroll
         for (int i = 0; i < 4 * kJ; i++) tot[i] = 0;
+        v16i acc_a, acc_b;
+        int sc_a, sc_b;
         RNB_Q45_SUB_BLOCK(0, row, tot)
         RNB_Q45_SUB_BLOCK(1, row, tot)
         RNB_Q45_SUB_BLOCK(2, row, tot)
@@ -129,6 +163,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
         RNB_Q45_SUB_BLOCK(5, row, tot)
         RNB_Q45_SUB_BLOCK(6, row, tot)
         RNB_Q45_SUB_BLOCK(7, row, tot)
+        RNB_Q45_TAKE(acc_b, sc_b, tot)
     } else {
         // Q4_K: the scale folded into the operand (sc = lo + 8 * hi, two accumulator chains), as in gemm_blocks.hip
         const uint32_t dlo[2] = {sc8.sc_lo & 0x07070707u, sc8.sc_hi & 0x07070707u};
@@ -142,9 +177,8 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
         const uint32_t shi = __builtin_amdgcn_perm(0u, dhi[(SB) >> 2], sel);                             \
         const v4i wlo = {pk_scale(nib[0], slo), pk_scale(nib[1], slo), pk_scale(nib[2], slo), pk_scale(nib[3], slo)}; \
         const v4i whi = {pk_scale(nib[0], shi), pk_scale(nib[1], shi), pk_scale(nib[2], shi), pk_scale(nib[3], shi)}; \
-        const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * (SB));                               \
-        acc_lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, wlo, acc_lo, 0, 0, 0);                       \
-        acc_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, whi, acc_hi, 0, 0, 0);                       \
+        acc_lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(aops.v[SB], wlo, acc_lo, 0, 0, 0);                \
+        acc_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(aops.v[SB], whi, acc_hi, 0, 0, 0);                \
     }
         RNB_Q4_FOLD_SUB_BLOCK(0)
         RNB_Q4_FOLD_SUB_BLOCK(1)
@@ -169,26 +203,43 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const uint8_t *
     for (int i = 0; i < 4 * kJ; i++) val[i] = d * static_cast<float>(tot[i]) - dmin * static_cast<float>(c0[i] + 64 * c1[i]);
 }
 #undef RNB_Q45_SUB_BLOCK
+#undef RNB_Q45_TAKE
+#undef RNB_Q45_ISSUE
 
 // ... and against one Q6_K row share: returns d * sum_sb sc * ((q - 32) . a)
-#define RNB_Q6_TILE_SUB_BLOCK(SB)                                                                        \
+#define RNB_Q6_TILE_ISSUE(SB, ACC, SC)                                                                   \
     {                                                                                                    \
         const long bop = q6_operand<SB>(row);                                                            \
-        const int sc = q6_scale<SB>(row);                                                                \
-        const long aop = *reinterpret_cast<const long *>(abase + 16 * (SB));                             \
-        const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);               \
+        SC = q6_scale<SB>(row);                                                                          \
+        ACC = __builtin_amdgcn_mfma_i32_32x32x16_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+    }
+#define RNB_Q6_TILE_TAKE(ACC, SC)                                                                        \
+    {                                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4 * kJ; i++) {                                             \
-            tot[i] += mul24(acc[i], sc);                                                                 \
+            tot[i] += mul24(ACC[i], SC);                                                                 \
             asm volatile("" : "+v"(tot[i]));                                                             \
         }                                                                                                \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
+// issue sub-block SB, then scale the results of SB - 1 (see RNB_Q45_SUB_BLOCK)
+#define RNB_Q6_TILE_SUB_BLOCK(SB)                                                                        \
+    {                                                                                                    \
+        if constexpr (((SB) & 1) == 0) {                                                                 \
+            RNB_Q6_TILE_ISSUE(SB, acc_a, sc_a)                                                           \
+            if constexpr ((SB) > 0) RNB_Q6_TILE_TAKE(acc_b, sc_b)                                        \
+        } else {                                                                                         \
+            RNB_Q6_TILE_ISSUE(SB, acc_b, sc_b)                                                           \
+            RNB_Q6_TILE_TAKE(acc_a, sc_a)                                                                \
+        }                                                                                                \
+    }
 template <int kJ>
-__device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *abase, float (&val)[4 * kJ]) {
+__device__ __forceinline__ void q6_block_tile(const Q6Row &row, const TileOps64 &aops, float (&val)[4 * kJ]) {
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     int tot[4 * kJ];
 #pragma unroll
     for (int i = 0; i < 4 * kJ; i++) tot[i] = 0;
+    v16i acc_a, acc_b;
+    int sc_a, sc_b;
     RNB_Q6_TILE_SUB_BLOCK(0)
     RNB_Q6_TILE_SUB_BLOCK(1)
     RNB_Q6_TILE_SUB_BLOCK(2)
@@ -205,10 +256,13 @@ __device__ __forceinline__ void q6_block_tile(const Q6Row &row, const uint8_t *a
     RNB_Q6_TILE_SUB_BLOCK(13)
     RNB_Q6_TILE_SUB_BLOCK(14)
     RNB_Q6_TILE_SUB_BLOCK(15)
+    RNB_Q6_TILE_TAKE(acc_b, sc_b)
 #pragma unroll
     for (int i = 0; i < 4 * kJ; i++) val[i] = row.d * static_cast<float>(tot[i]);
 }
 #undef RNB_Q6_TILE_SUB_BLOCK
+#undef RNB_Q6_TILE_TAKE
+#undef RNB_Q6_TILE_ISSUE
 
 // accf[r] += d_x[token of result r] * val[r]; result r of a tile is token 8 * (r / 4) + 4 * khalf + r % 4
 template <int kJ>
@@ -271,15 +325,16 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
                             const uint32_t *__restrict__ sorted_slot, const uint32_t *__restrict__ sorted_token,
                             float *__restrict__ mid, uint32_t n_ff, uint32_t nb, uint32_t img_toks, uint32_t tiles_per_wg) {
     constexpr bool kFifth = false;
+    constexpr int kPair = 2 * kQ4FillBytes;  // a gate strip and an up strip
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     __shared__ TileMap s_map;
-    const TileImage<kGbStride128, true> img{s_dyn + kW * 2 * kQ4FillBytes, nb, img_toks};
+    const TileImage<kGbStride128, true> img{s_dyn + kW * kPair, nb, img_toks};
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS-direct loads take their target from a scalar register
     const int lrow = lane & 31, khalf = lane >> 5;
-    uint8_t *strip_g = s_dyn + wave * 2 * kQ4FillBytes, *strip_u = strip_g + kQ4FillBytes;
-    const uint32_t lds_g = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)strip_g)), lds_u = lds_g + kQ4FillBytes;
+    uint8_t *strips = s_dyn + wave * kPair;
+    const uint32_t lds_strips = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)strips));
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
     const uint32_t row_bytes = nb * static_cast<uint32_t>(kQ4KBytes);
@@ -287,15 +342,17 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
     const uint8_t *gate_e = expert_base(gate_all, gate_shared, n_routed, expert, per_expert),
                   *up_e = expert_base(up_all, up_shared, n_routed, expert, per_expert);
     // The workgroup walks tiles_per_wg row tiles against one staged token tile (map and image are made once: a chain of
-    // dependent loads); the weight blocks of the whole walk form one stream, requested one block ahead across row tiles.
+    // dependent loads); the weight blocks of the whole walk form one stream of rt_n * nb steps, requested one step
+    // ahead across row tiles.  (Two steps ahead into a second pair of strips measured no faster: 53.3 against 50.6 us.)
     const uint32_t row_tiles = (n_ff + 32 * kW - 1) / (32 * kW);
     const uint32_t rt0 = blockIdx.x * tiles_per_wg, rt_n = min(tiles_per_wg, row_tiles - rt0);
-    // Row tile rt: the wave's first row (a wave wholly past the end streams the last row and stores nothing) and its
-    // pieces.  Piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column c % 9; it lands at
-    // byte 16 c of the strip, which puts the rows 144 bytes apart (rows past the end of the matrix repeat the last row;
-    // the pieces past 288 of the fifth instruction repeat the last piece and land behind the rows)
+    // The request cursor.  Row tile rt: the wave's first row (a wave wholly past the end streams the last row and stores
+    // nothing) and its pieces.  Piece c = 64 i + lane of the wave's 32 x 9 pieces of a block: row c / 9, 16-byte column
+    // c % 9; it lands at byte 16 c of the strip, which puts the rows 144 bytes apart (rows past the end of the matrix
+    // repeat the last row; the pieces past 288 of the fifth instruction repeat the last piece and land behind the rows)
     const uint8_t *gbase, *ubase;
     uint32_t goff[kQ4FillInstr];
+    uint32_t req_b = 0, req_rt = 0;  // next block / row tile to request
     auto set_tile = [&](uint32_t rt) {
         const uint32_t first = min((rt0 + rt) * (32 * kW) + wave * 32, n_ff - 1);
         const size_t woff = static_cast<size_t>(first) * row_bytes;
@@ -308,26 +365,36 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
             goff[i] = min(r, n_ff - first - 1) * row_bytes + 16 * j;
         }
     };
-    auto request = [&](uint32_t b) {
+    // the next step of the walk into the strips (past the end: the last step again, unused)
+    auto request = [&]() {
         // the strips' previous contents have been read out (the reads are ahead of these fills in program order; make
         // sure they have executed)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const uint8_t *gsrc = gbase + b * static_cast<uint32_t>(kQ4KBytes), *usrc = ubase + b * static_cast<uint32_t>(kQ4KBytes);
+        const uint32_t dst = lds_strips;
+        const uint8_t *gsrc = gbase + req_b * static_cast<uint32_t>(kQ4KBytes), *usrc = ubase + req_b * static_cast<uint32_t>(kQ4KBytes);
 #pragma unroll
-        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(gsrc, goff[i], lds_g + i * 1024);
+        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(gsrc, goff[i], dst + i * 1024);
 #pragma unroll
-        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(usrc, goff[i], lds_u + i * 1024);
+        for (int i = 0; i < kQ4FillInstr; i++) lds_fill16(usrc, goff[i], dst + kQ4FillBytes + i * 1024);
+        if (req_b + 1 < nb) {
+            req_b++;
+        } else if (req_rt + 1 < rt_n) {
+            req_rt++;
+            req_b = 0;
+            set_tile(req_rt);
+        }
     };
     auto take = [&](Q5Row &g, Q5Row &u) {
         wait_fills();
-        q4_row_from_strip(g, strip_g + lrow * kQ4StripStride, khalf);
-        q4_row_from_strip(u, strip_u + lrow * kQ4StripStride, khalf);
+        q4_row_from_strip(g, strips + lrow * kQ4StripStride, khalf);
+        q4_row_from_strip(u, strips + kQ4FillBytes + lrow * kQ4StripStride, khalf);
     };
 
     for (uint32_t tile0 = 0; tile0 < count; tile0 += img_toks) {
         // the first weight blocks do not depend on the token lists: requested before them
+        req_b = req_rt = 0;
         set_tile(0);
-        request(0);
+        request();
         const uint32_t live = min(count - tile0, img_toks);
         const uint32_t arow = min(static_cast<uint32_t>(lrow), live - 1);  // padding lanes read the last live row
         if (tile0) __syncthreads();  // the previous tile's readers of the map and the image are done
@@ -339,38 +406,33 @@ __global__ void __attribute__((amdgpu_flat_work_group_size(kWave * kW, kWave * k
         __syncthreads();
         // a tile of at most eight live tokens (most groups of a routed batch) finishes only a lane's first four results
         auto walk = [&](auto jtag) {
-        constexpr int kJl = decltype(jtag)::value;
-        for (uint32_t rt = 0; rt < rt_n; rt++) {
-            const uint32_t row = (rt0 + rt) * (32 * kW) + wave * 32 + lrow;
-            float accg[4 * kJl], accu[4 * kJl];
+            constexpr int kJl = decltype(jtag)::value;
+            for (uint32_t rt = 0; rt < rt_n; rt++) {
+                const uint32_t row = (rt0 + rt) * (32 * kW) + wave * 32 + lrow;
+                float accg[4 * kJl], accu[4 * kJl];
 #pragma unroll
-            for (int i = 0; i < 4 * kJl; i++) accg[i] = accu[i] = 0.0f;
-            for (uint32_t b = 0; b < nb; b++) {
-                if (b + 1 < nb) {
-                    request(b + 1);
-                } else if (rt + 1 < rt_n) {  // the walk goes on: block 0 of the next row tile
-                    set_tile(rt + 1);
-                    request(0);
-                } else {
-                    request(b);  // the last step reloads its own block, unused
+                for (int i = 0; i < 4 * kJl; i++) accg[i] = accu[i] = 0.0f;
+                for (uint32_t b = 0; b < nb; b++) {
+                    request();  // the step after this one
+                    const uint8_t *abase = img.act(b) + arow * kGbStride128 + 16 * khalf;
+                    const uint4 dig = img.dig(b)[lrow];
+                    float val[4 * kJl];
+                    TileOps128 aops;
+                    tile_ops_load(aops, abase);
+                    q45_block_tile<kFifth, kJl>(cg, aops, dig, khalf, val);
+                    tile_scale_add<kJl>(img.dx(b), khalf, val, accg);
+                    q45_block_tile<kFifth, kJl>(cu, aops, dig, khalf, val);
+                    tile_scale_add<kJl>(img.dx(b), khalf, val, accu);
+                    take(cg, cu);  // (after the last step: a repeat of it, unused)
                 }
-                const uint8_t *abase = img.act(b) + arow * kGbStride128 + 16 * khalf;
-                const uint4 dig = img.dig(b)[lrow];
-                float val[4 * kJl];
-                q45_block_tile<kFifth, kJl>(cg, abase, dig, khalf, val);
-                tile_scale_add<kJl>(img.dx(b), khalf, val, accg);
-                q45_block_tile<kFifth, kJl>(cu, abase, dig, khalf, val);
-                tile_scale_add<kJl>(img.dx(b), khalf, val, accu);
-                take(cg, cu);
-            }
-            if (row < n_ff) {
+                if (row < n_ff) {
 #pragma unroll
-                for (int r = 0; r < 4 * kJl; r++) {
-                    const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
-                    if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
+                    for (int r = 0; r < 4 * kJl; r++) {
+                        const uint32_t slot = s_map.out_row[8 * (r >> 2) + 4 * khalf + (r & 3)];
+                        if (slot != 0xffffffffu) mid[static_cast<size_t>(slot) * n_ff + row] = act_mul<false>(accg[r], accu[r]);
+                    }
                 }
             }
-        }
         };
         if constexpr (kJ == 2) {  // (the 32-token kernel keeps its one form: its groups are large)
             if (live <= 8)  // workgroup-uniform
@@ -497,10 +559,14 @@ __global__ void __launch_bounds__(kGbThreads, 2)
             float val[4 * kJ];
             if constexpr (kSix) {
                 q6_request(rtn, bn);
-                q6_block_tile<kJ>(c6, img.act(b) + arow * kStride + 8 * khalf, val);
+                TileOps64 aops;
+                tile_ops_load(aops, img.act(b) + arow * kStride + 8 * khalf);
+                q6_block_tile<kJ>(c6, aops, val);
             } else {
                 n5 = q45_load_row<kFifth>(block_ptr(rtn, bn), khalf);
-                q45_block_tile<kFifth, kJ>(c5, img.act(b) + arow * kStride + 16 * khalf, img.dig(b)[lrow], khalf, val);
+                TileOps128 aops;
+                tile_ops_load(aops, img.act(b) + arow * kStride + 16 * khalf);
+                q45_block_tile<kFifth, kJ>(c5, aops, img.dig(b)[lrow], khalf, val);
             }
             tile_scale_add<kJ>(img.dx(b), khalf, val, accf);
             if constexpr (kSix) q6_take(c6);
@@ -564,21 +630,29 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, con
     if (groups.n_groups == 0 || n_ff == 0) return;
     const uint32_t toks = std::min<uint32_t>(std::max<uint32_t>(groups.max_group, 1), gate_up_tile_tokens(nb_in));
     if (toks == 0) return;  // moe_mfma_supported said no
-    const int waves = kGbWaves;  // 2, 3 and 6 waves per workgroup measured within 3 % of 4 on 128 experts x top-8, 64 tokens
-    const size_t lds = static_cast<size_t>(waves) * 2 * kQ4FillBytes + TileImage<kGbStride128, true>::bytes(nb_in, toks);
-    const uint32_t rows_per_wg = 32 * waves, row_tiles = (n_ff + rows_per_wg - 1) / rows_per_wg;
-    // A wave's time is its chain of steps (a step waits for its own fill), much the same with one workgroup on the compute
-    // unit or two; a grid of more workgroups than fit at once runs in rounds, and a last round that is partly empty costs
-    // as much as a full one.  Where merging up to three row tiles into a workgroup brings the grid down to one workgroup
-    // per compute unit, that is done: one round, map and image made once per walk (128 experts x top-8 at 64 tokens,
-    // 6 row tiles x 126 groups: 1 / 2 / 3 tiles per workgroup 55.4 / 58.4 / 53.7 us; 2 leaves half the units with two
-    // workgroups and half with one).
+    const size_t image = TileImage<kGbStride128, true>::bytes(nb_in, toks);
+    // A wave's time is its chain of steps, and the chain is mostly instruction and LDS latency that only another wave on
+    // the SIMD hides (without its fills the kernel still takes 40 of its 50 us); a grid of more workgroups than fit at once
+    // runs in rounds, and a last round that is partly empty costs as much as a full one.  So: the widest workgroup (six
+    // waves = 192 rows, else four = 128) for which merging up to three row tiles into one walk brings the grid down to
+    // one workgroup per compute unit, map and image made once per walk.  128 experts x top-8 at 64 tokens (126 groups):
+    // four waves 1 / 2 / 3 tiles per workgroup 55.4 / 58.4 / 50.6 us (2 leaves half the units with two workgroups and
+    // half with one), six waves x 2 tiles 48.8 us, eight waves x 1 (two rounds) 61.6, twelve waves 67-74.
+    int waves = kGbWaves;
     uint32_t tiles_per_wg = 1;
-    {
-        const uint64_t total = static_cast<uint64_t>(row_tiles) * groups.n_groups;
-        const uint32_t t = static_cast<uint32_t>((total + 255) / 256);
-        if (t >= 2 && t <= 3 && static_cast<uint64_t>((row_tiles + t - 1) / t) * groups.n_groups <= 256) tiles_per_wg = t;
+    for (const int w : {6, 4}) {
+        if (w != kGbWaves && (toks > 16 || static_cast<size_t>(w) * 2 * kQ4FillBytes + image > kMmLdsLimit)) continue;
+        const uint32_t tiles = (n_ff + 32 * w - 1) / (32 * w);
+        const uint32_t t = static_cast<uint32_t>((static_cast<uint64_t>(tiles) * groups.n_groups + 255) / 256);
+        if (t >= 1 && t <= 3 && t <= tiles && static_cast<uint64_t>((tiles + t - 1) / t) * groups.n_groups <= 256 &&
+            (t > 1 || w == 4)) {
+            waves = w;
+            tiles_per_wg = t;
+            break;
+        }
     }
+    const size_t lds = static_cast<size_t>(waves) * 2 * kQ4FillBytes + image;
+    const uint32_t rows_per_wg = 32 * waves, row_tiles = (n_ff + rows_per_wg - 1) / rows_per_wg;
     const dim3 grid((row_tiles + tiles_per_wg - 1) / tiles_per_wg, groups.n_groups, 1);
     // tiles of at most 8 / 16 / 32 tokens: the kernel finishes only that many results per lane
 #define RNB_LAUNCH_GUW(J, W)                                                                                          \
@@ -586,15 +660,19 @@ void launch_moe_gate_up_mfma(const uint8_t *gate_all, const uint8_t *up_all, con
     hipLaunchKernelGGL((moe_gate_up_mfma_kernel<J, W>), grid, dim3(kWave * W), lds, stream, gate_all, up_all, shared.gate, \
                        shared.up, shared.n_routed, act.qs, act.d, act.digits, groups.expert, groups.start,            \
                        groups.sorted_slot, groups.sorted_token, mid, n_ff, nb_in, toks, tiles_per_wg)
-#define RNB_LAUNCH_GU(J) RNB_LAUNCH_GUW(J, kGbWaves)
-    if (toks <= 8) {
-        RNB_LAUNCH_GU(1);
-    } else if (toks <= 16) {
-        RNB_LAUNCH_GU(2);
+    if (toks > 16) {
+        RNB_LAUNCH_GUW(4, kGbWaves);
+    } else if (waves == 6) {
+        if (toks <= 8) {
+            RNB_LAUNCH_GUW(1, 6);
+        } else {
+            RNB_LAUNCH_GUW(2, 6);
+        }
+    } else if (toks <= 8) {
+        RNB_LAUNCH_GUW(1, kGbWaves);
     } else {
-        RNB_LAUNCH_GU(4);
+        RNB_LAUNCH_GUW(2, kGbWaves);
     }
-#undef RNB_LAUNCH_GU
 #undef RNB_LAUNCH_GUW
 }
 
