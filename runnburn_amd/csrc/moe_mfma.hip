@@ -541,9 +541,12 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         }
         if constexpr (kSix) q6_take(c6);
         __syncthreads();
-        float accf[4 * kJ];
+        // a tile of at most eight live tokens (most groups of a routed batch) finishes only a lane's first four results
+        auto walk = [&](auto jtag) {
+        constexpr int kJl = decltype(jtag)::value;
+        float accf[4 * kJl];
 #pragma unroll
-        for (int i = 0; i < 4 * kJ; i++) accf[i] = 0.0f;
+        for (int i = 0; i < 4 * kJl; i++) accf[i] = 0.0f;
         uint32_t rt = 0, b = 0;
         for (uint32_t s = 0; s < steps; s++) {
             uint32_t rtn = rt, bn = b + 1;  // the step after this one; the last step reloads its own block, unused
@@ -556,26 +559,26 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                 bn = b;
             }
             Q5Row n5{};
-            float val[4 * kJ];
+            float val[4 * kJl];
             if constexpr (kSix) {
                 q6_request(rtn, bn);
                 TileOps64 aops;
                 tile_ops_load(aops, img.act(b) + arow * kStride + 8 * khalf);
-                q6_block_tile<kJ>(c6, aops, val);
+                q6_block_tile<kJl>(c6, aops, val);
             } else {
                 n5 = q45_load_row<kFifth>(block_ptr(rtn, bn), khalf);
                 TileOps128 aops;
                 tile_ops_load(aops, img.act(b) + arow * kStride + 16 * khalf);
-                q45_block_tile<kFifth, kJ>(c5, aops, img.dig(b)[lrow], khalf, val);
+                q45_block_tile<kFifth, kJl>(c5, aops, img.dig(b)[lrow], khalf, val);
             }
-            tile_scale_add<kJ>(img.dx(b), khalf, val, accf);
+            tile_scale_add<kJl>(img.dx(b), khalf, val, accf);
             if constexpr (kSix) q6_take(c6);
             c5 = n5;
             if (b + 1 == nb) {  // the row tile is complete
                 const uint32_t row = row_of(rt);
                 if (row < n_embd) {
 #pragma unroll
-                    for (int r = 0; r < 4 * kJ; r++) {
+                    for (int r = 0; r < 4 * kJl; r++) {
                         const int t = 8 * (r >> 2) + 4 * khalf + (r & 3);
                         const uint32_t slot = s_map.out_row[t];
                         // fanout.rs:306-308: the expert's output times the slot's route weight
@@ -584,10 +587,19 @@ __global__ void __launch_bounds__(kGbThreads, 2)
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 4 * kJ; i++) accf[i] = 0.0f;
+                for (int i = 0; i < 4 * kJl; i++) accf[i] = 0.0f;
             }
             rt = rtn;
             b = bn;
+        }
+        };
+        if constexpr (kJ == 2) {
+            if (live <= 8)  // workgroup-uniform
+                walk(std::integral_constant<int, 1>{});
+            else
+                walk(std::integral_constant<int, 2>{});
+        } else {
+            walk(std::integral_constant<int, kJ>{});
         }
     }
 }
