@@ -93,21 +93,30 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const float d_cur = cur.d;
         const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
 
-        // one 16-element sub-block: operand from the packed row, one matrix instruction per token tile, the sub-block's
-        // scale applied to the 16 results.  The empty asm and the scheduling barrier keep the sub-blocks in order: left
-        // alone the compiler turns each result's sixteen additions into a tree and keeps all 256 products alive.
+        // One 16-element sub-block: operand from the packed row, one matrix instruction per token tile, the sub-block's
+        // scale applied to the 16 results.  The token tiles' instructions are issued together and their results
+        // scaled afterwards, so the second tile's instruction runs while the first tile's results are scaled.  The
+        // empty asm and the scheduling barrier keep the sub-blocks in order: left alone the compiler turns each
+        // result's sixteen additions into a tree and keeps all 256 products alive.
+        long aop_cur[kTT], aop_nxt[kTT];  // the tokens' operands are read from LDS one sub-block ahead of their use
+#pragma unroll
+        for (int t = 0; t < kTT; t++) aop_cur[t] = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64);
 #define RNB_Q6_SUB_BLOCK(SB)                                                                                           \
     {                                                                                                                  \
         const long bop = q6_operand<SB>(cur);                                                                          \
         const int sc = q6_scale<SB>(cur);                                                                              \
+        v16i acc[kTT];                                                                                                 \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++)                                                                \
+            aop_nxt[t] = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * ((SB) < 15 ? (SB) + 1 : 15)); \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++)                                                                \
+            acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop_cur[t], bop, zero16, 0, 0, 0);                          \
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
-            const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
-            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
-                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 32 * 127 */                                          \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
+                tot[t][i] += mul24(acc[t][i], sc); /* |I_sb| <= 16 * 32 * 127 */                                       \
                 asm volatile("" : "+v"(tot[t][i])); /* no re-association of the sixteen sums into a tree */            \
             }                                                                                                          \
         }                                                                                                              \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) aop_cur[t] = aop_nxt[t];                                       \
         __builtin_amdgcn_sched_barrier(0);                                                                             \
     }
         RNB_Q6_SUB_BLOCK(0)
