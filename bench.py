@@ -631,7 +631,7 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
 
 # configs that --only can run alone: quant, rows, cols, tokens
 ONLY = {"cfg1": (Q8_0, 4096, 4096, 1), "cfg2": (Q4_K, 14336, 4096, 1), "cfg3a": (Q6_K, 4096, 14336, 1),
-        "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512), "q6gemm": (Q6_K, 4096, 14336, 512),
+        "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512), "q6gemm": (Q6_K, 4096, 14336, 512), "q5gemm": (Q5_K, 14336, 4096, 512),
         "moe1": 1, "moe4": 4, "moe64": 64}  # moeN: configs[4] at N tokens
 
 

@@ -316,11 +316,14 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     {                                                                                                                  \
         const long bop = q23_operand<SB, kThree>(cur);                                                                 \
         const int sc = q23_scale<SB, kThree>(cur);                                                                     \
+        v16i acc[kTT]; /* the tiles' instructions first, then their results: see the Q6_K kernel */                    \
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
-            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
-                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 16 * 4 * 127 */                                           \
+            acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                                 \
+        }                                                                                                              \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
+                tot[t][i] += mul24(acc[t][i], sc); /* |I_sb| <= 16 * 4 * 127 */                                        \
                 asm volatile("" : "+v"(tot[t][i]));                                                                    \
             }                                                                                                          \
         }                                                                                                              \
@@ -461,11 +464,14 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     {                                                                                                                  \
         const v4i bop = q45_operand<SB, kFifth>(cur);                                                                  \
         const int sc = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                              \
+        v16i acc[kTT]; /* the tiles' instructions first, then their results: see the Q6_K kernel */                    \
         _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
             const v4i aop = *reinterpret_cast<const v4i *>(abase + 32 * t * kGbStride128 + 32 * (SB));                 \
-            const v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);                         \
-            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                           \
-                tot[t][i] += mul24(acc[i], sc); /* |I_sb| <= 32 * 31 * 127 */                                          \
+            acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop, zero16, 0, 0, 0);                                 \
+        }                                                                                                              \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
+                tot[t][i] += mul24(acc[t][i], sc); /* |I_sb| <= 32 * 31 * 127 */                                       \
                 asm volatile("" : "+v"(tot[t][i])); /* no re-association of the eight sums into a tree */              \
             }                                                                                                          \
         }                                                                                                              \
