@@ -652,15 +652,16 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
     // one table image: route[n] | tok_offsets[T+1] | tok_slots[n] | sorted_slot[n] | sorted_token[n] | grp_expert[G] |
     // grp_start[G+1] | slot_expert[n]
     const size_t table_words = 5 * n_slots + (token_count + 1) + n_groups + (n_groups + 1);
-    // Batches with at least two slots per routed expert on average: the expert GEMMs run on the matrix cores (a
+    // Batches with at least 1.8 slots per routed expert on average: the expert GEMMs run on the matrix cores (a
     // 32-token tile costs the same whatever its number of live tokens, the integer-dot kernels cost per token; measured
-    // crossover on 128 experts x top-8: between 24 and 32 tokens) and need the quantiser's digits
+    // on 128 experts x top-8: 16 / 20 / 24 tokens 71.9 / 84.2 / 93.9 us on the integer-dot kernels, 79.0 / 85.7 / 88.2
+    // on the matrix cores; the ratio is 1.6 / 1.8 / 1.9 there) and need the quantiser's digits
     // (its gate/up rows arrive as 16-byte LDS-direct loads: other alignments take the vector kernels)
     // (and the Q6_K down rows as dword-aligned pieces: an even base address and whole 128-row tiles)
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(gate_dev) | reinterpret_cast<uintptr_t>(up_dev) |
                              reinterpret_cast<uintptr_t>(down_dev) | reinterpret_cast<uintptr_t>(shared.gate) |
                              reinterpret_cast<uintptr_t>(shared.up) | reinterpret_cast<uintptr_t>(shared.down)) & 15u) == 0;
-    const bool mfma = token_count >= kMoeMfmaMinTokens && n_slots >= 2 * n_groups && aligned16 && n_embd % 128 == 0 &&
+    const bool mfma = token_count >= kMoeMfmaMinTokens && 10 * n_slots >= 18 * n_groups && aligned16 && n_embd % 128 == 0 &&
                       moe_mfma_supported(static_cast<uint32_t>(sh.nb_in), static_cast<uint32_t>(sh.nb_mid), down_quant);
     const bool inline_tables = !mfma && table_words <= kMoeInlineWords;  // decode-sized: rides in a kernel argument
     MoeInlineTables inl;

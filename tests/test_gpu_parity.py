@@ -805,7 +805,7 @@ def test_moe_small_batch_equals_general_sequence(rnb, oracle, tokens, n_ff, n_em
                                                                      (40, 5, 3, 1024, 256, Q4_K), (20, 64, 3, 256, 512, Q6_K),
                                                                      (64, 128, 8, 256, 1792, Q6_K), (48, 96, 8, 256, 1792, Q4_K)])
 def test_moe_prefill_matrix_core_path(rnb, oracle, tokens, n_expert, k, n_ff, n_embd, down_quant):
-    """16 or more tokens and at least two slots per routed expert on average: the grouped expert GEMMs on the matrix
+    """16 or more tokens and at least 1.8 slots per routed expert on average: the grouped expert GEMMs on the matrix
     cores (32-token tiles per expert; experts with more than 32 tokens take several tiles, experts with few run mostly
     padding); the sixth case stays below that average and keeps the integer-dot kernels; in the last two the down
     kernel's workgroups walk four row tiles each (14 row tiles x ~100 expert groups: the last workgroup of a group gets two).
