@@ -1292,3 +1292,44 @@ def test_moe_shared_expert_slot_on_the_matrix_cores_dev(rnb, oracle):
     from oracle import flips
     v = flips.moe_verdict(got, ref, *longer, n_expert + 1, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
     assert v["ok"] or v["flip_aware_ok"], v
+
+
+@pytest.mark.parametrize("tokens,n_expert,k,n_ff,n_embd,down_quant,shared", [(64, 128, 8, 1024, 512, Q6_K, False),
+                                                                            (48, 60, 8, 1280, 768, Q5_K, False),
+                                                                            (100, 128, 2, 512, 256, Q4_K, False),
+                                                                            (16, 48, 8, 1024, 512, Q6_K, True)])
+def test_moe_many_experts_wide_workgroups_ragged_row_tiles_dev(rnb, oracle, tokens, n_expert, k, n_ff, n_embd, down_quant, shared):
+    """Many routed experts with few tokens each: the gate/up kernel runs six-wave workgroups (192 rows a tile) that
+    walk two or three row tiles, and n_ff is no multiple of 192, so a group's last tile has idle waves and its last
+    workgroup fewer tiles.  Device buffers, slots in the callers' (expert, token) order; the last case has the shared
+    expert as the one group of sixteen tokens among groups of a few.  Against the oracle, and the same bits with the
+    tokens in reverse order."""
+    if shared:
+        gate, up, down, sh, longer, x, e, r, t = _with_shared(oracle, n_expert, n_ff, n_embd, tokens, k, 700 + tokens, down_quant)
+        ne = n_expert + 1
+    else:
+        gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 700 + tokens, down_quant)
+        sh, longer, ne = (), (gate, up, down), n_expert
+    order = np.lexsort((t, e))
+    e, r, t = e[order], r[order], t[order]
+    xr = x.reshape(tokens, n_embd)[::-1].copy()
+    tr = (tokens - 1 - t).astype(np.uint32)
+    order_r = np.lexsort((tr, e))
+    bufs = [rnb.DeviceBuffer.from_host(a) for a in (gate, up, down, x, xr, *sh)]
+    out_dev = rnb.DeviceBuffer(tokens * n_embd * 4)
+    try:
+        outs = []
+        for xb, ee, rr, tt in ((bufs[3], e, r, t), (bufs[4], e[order_r], r[order_r], tr[order_r])):
+            rnb.moe_sparse_experts_by_token_dev(bufs[0], bufs[1], bufs[2], n_expert, ee, rr, tt, tokens, down_quant, n_ff, n_embd,
+                                                xb, out_dev, shared=bufs[5:8] if shared else None)
+            rnb.sync()
+            outs.append(out_dev.to_host(np.float32).reshape(tokens, n_embd).copy())
+    finally:
+        for b in bufs + [out_dev]:
+            b.free()
+    got, rev = outs
+    ref = oracle.moe_sparse_experts_by_token(*longer, ne, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    from oracle import flips
+    v = flips.moe_verdict(got, ref, *longer, ne, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    assert v["ok"] or v["flip_aware_ok"], {key: v[key] for key in v if key != "flips"}
+    assert np.array_equal(rev[::-1], got)
