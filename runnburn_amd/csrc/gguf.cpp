@@ -483,8 +483,23 @@ bool all_digits(const std::string &s) {
     return !s.empty() && std::all_of(s.begin(), s.end(), [](unsigned char c) { return c >= '0' && c <= '9'; });
 }
 
+// The shard files' names, made one at a time: a header may declare any 64-bit shard count, and a list of that many
+// names would be allocated before the first missing file refuses the set.
+struct ShardPaths {
+    std::string parent, prefix, ext;
+    size_t index_width, count_width;
+    uint64_t split_count;
+    std::string of(uint64_t no) const {  // shard `no`, counted from zero
+        auto padded = [](uint64_t v, size_t width) {
+            std::string t = std::to_string(v);
+            return t.size() < width ? std::string(width - t.size(), '0') + t : t;
+        };
+        return parent + prefix + "-" + padded(no + 1, index_width) + "-of-" + padded(split_count, count_width) + ext;
+    }
+};
+
 // resolve_shard_paths, sharded.rs:180-235: `<prefix>-<index>-of-<count>.gguf` beside the selected file, same digit widths
-std::vector<std::string> resolve_shard_paths(const std::string &selected, uint64_t selected_no, uint64_t split_count) {
+ShardPaths resolve_shard_paths(const std::string &selected, uint64_t selected_no, uint64_t split_count) {
     const size_t slash = selected.find_last_of('/');
     const std::string parent = slash == std::string::npos ? "" : selected.substr(0, slash + 1);
     const std::string file_name = slash == std::string::npos ? selected : selected.substr(slash + 1);
@@ -508,14 +523,7 @@ std::vector<std::string> resolve_shard_paths(const std::string &selected, uint64
     if (parsed_index != selected_no + 1 || parsed_count != split_count)
         split_error("file name declares shard " + std::to_string(parsed_index) + " of " + std::to_string(parsed_count) +
                     ", metadata declares shard " + std::to_string(selected_no + 1) + " of " + std::to_string(split_count));
-    auto padded = [](uint64_t v, size_t width) {
-        std::string t = std::to_string(v);
-        return t.size() < width ? std::string(width - t.size(), '0') + t : t;
-    };
-    std::vector<std::string> paths;
-    for (uint64_t index = 1; index <= split_count; index++)
-        paths.push_back(parent + prefix + "-" + padded(index, file_index.size()) + "-of-" + padded(split_count, file_count.size()) + ext);
-    return paths;
+    return ShardPaths{parent, prefix, ext, file_index.size(), file_count.size(), split_count};
 }
 
 // The file that was opened declares split.count > 1: every shard is mapped and checked, `g` becomes shard zero with the
@@ -528,13 +536,14 @@ void assemble_split(const char *path, std::unique_ptr<rnb_hip_gguf> &g) {
     if (selected_no >= split_count)
         split_error("split.no " + std::to_string(selected_no) + " is outside split.count " + std::to_string(split_count));
     const uint64_t expected_tensors = required_split_value(*g, "split.tensors.count");
-    const std::vector<std::string> paths = resolve_shard_paths(path, selected_no, split_count);
-    std::vector<std::unique_ptr<rnb_hip_gguf>> shards(split_count);
+    const ShardPaths paths = resolve_shard_paths(path, selected_no, split_count);
+    std::vector<std::unique_ptr<rnb_hip_gguf>> shards;  // grows with the shards that open: a wrong count ends at the first missing file
     for (uint64_t no = 0; no < split_count; no++) {
+        shards.emplace_back();
         if (no == selected_no) {
             shards[no] = std::move(g);
-        } else if (open_one(paths[no].c_str(), &shards[no]) != RNB_HIP_OK) {
-            split_error("failed to load shard '" + paths[no] + "': " + last_error_cstr());
+        } else if (const std::string shard_path = paths.of(no); open_one(shard_path.c_str(), &shards[no]) != RNB_HIP_OK) {
+            split_error("failed to load shard '" + shard_path + "': " + last_error_cstr());
         }
         // validate_shard, sharded.rs:113-138
         const rnb_hip_gguf &sh = *shards[no];

@@ -262,13 +262,13 @@ def test_file_with_quantised_tensors_maps_untouched_bytes(tmp_path):
 
 # ---- split files: crates/rnb-loader/src/gguf/sharded.rs -------------------------------------------------------------------
 
-def _shard(shard_no, shard_count, total_tensors, tensor_name, value, no_type=gw.T_U16, extra=()):
+def _shard(shard_no, shard_count, total_tensors, tensor_name, value, no_type=gw.T_U16, extra=(), count_type=gw.T_U16):
     """make_split_shard of sharded.rs:245-274: architecture, the three split keys, one F32 tensor of one element."""
     md = [("general.architecture", gw.T_STR, "llama")]
     if shard_no is not None:
         md.append(("split.no", no_type, shard_no))
     if shard_count is not None:
-        md.append(("split.count", gw.T_U16, shard_count))
+        md.append(("split.count", count_type, shard_count))
     if total_tensors is not None:
         md.append(("split.tensors.count", gw.T_U64, total_tensors))
     b = gw.Builder(3, 1 + len(extra), len(md))
@@ -362,6 +362,9 @@ def test_split_file_rejections(tmp_path):
     write("m-00001-of-00002.gguf", _shard(0, 2, 3, "w0", 1.0))
     write("m-00002-of-00002.gguf", _shard(1, 2, 3, "w1", 1.0))
     rejected(str(tmp_path / "m-00001-of-00002.gguf"), "split.tensors.count declares 3 tensors but 2 were loaded")
+    # a count no set of files can have: refused at the first missing file, without a list of that many names
+    huge = 2 ** 64 - 1
+    rejected(write(f"o-00001-of-{huge}.gguf", _shard(0, huge, 2, "w", 1.0, count_type=gw.T_U64)), f"o-00002-of-{huge}.gguf")
     # a shard that does not parse is named with its own error
     write("n-00001-of-00002.gguf", _shard(0, 2, 2, "w0", 1.0))
     write("n-00002-of-00002.gguf", b"GGUX" + bytes(60))
