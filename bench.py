@@ -562,9 +562,11 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed, cpu=True):
             step(0)
             rnb.sync()
             gpu_out = out_dev.to_host(np.float32)
-            run = lambda rt: ora.moe_sparse_experts_by_token(g, u, d, n_expert, rt[0], rt[1], rt[2], tokens, Q6_K, n_ff,  # noqa: E731
-                                                             n_embd, x_host, n_threads=threads)
-            ref = run(routes[0])
+            simd = ora.have_avx2()  # the timed form runs rnb-cpu's AVX2 block dots; the check uses the scalar form
+            run = lambda rt, avx2=simd: ora.moe_sparse_experts_by_token(g, u, d, n_expert, rt[0], rt[1], rt[2], tokens,  # noqa: E731
+                                                                        Q6_K, n_ff, n_embd, x_host, n_threads=threads,
+                                                                        avx2=avx2)
+            ref = run(routes[0], False)
 
             def flip_verdict():
                 from oracle import flips
@@ -583,8 +585,9 @@ def bench_moe(rnb, hip, stream, tokens, steps, seed, cpu=True):
             res["cpu_baseline"] = {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
                                    "sample": f"{len(times)} full passes of the same routed call (routes rotate as on the GPU), "
                                              f"median per pass", "ms": med * 1e3, "gpu_matches_cpu": verdict,
-                                   "note": "the per-token loop of prefill_cpu.rs:167-194 over the scalar block dots, "
-                                           "experts of a token on threads"}
+                                   "note": "the per-token loop of prefill_cpu.rs:167-194 over the "
+                                           + ("AVX2+FMA" if simd else "scalar") + " block dots, slots on threads; "
+                                           "gpu_matches_cpu is taken against the scalar dots"}
         except Exception as exc:
             res["cpu_baseline"] = {"error": str(exc)}
     for b in (gd, ud, dd, x_dev, out_dev):

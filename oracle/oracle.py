@@ -79,9 +79,9 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes = [vp, vp, sz]
         L.rnbo_route_topk.restype = sz
         L.rnbo_route_topk.argtypes = [vp, sz, sz, vp, vp]
-        L.rnbo_moe_sparse_experts_by_token.restype = i32
-        L.rnbo_moe_sparse_experts_by_token.argtypes = [vp, vp, vp, sz, vp, vp, vp, sz, sz, u32, sz, sz,
-                                                       vp, vp, i32]
+        for name in ("rnbo_moe_sparse_experts_by_token", "rnbo_moe_sparse_experts_by_token_avx2"):
+            getattr(L, name).restype = i32
+            getattr(L, name).argtypes = [vp, vp, vp, sz, vp, vp, vp, sz, sz, u32, sz, sz, vp, vp, i32]
         for name in ("rnbo_quantize_row_q2_k", "rnbo_quantize_row_q3_k", "rnbo_quantize_row_q4_k", "rnbo_quantize_row_q5_k",
                      "rnbo_quantize_row_q6_k", "rnbo_quantize_row_q8_0"):
             getattr(L, name).restype = None
@@ -311,7 +311,9 @@ def route_topk(logits, k: int) -> tuple[np.ndarray, np.ndarray]:
 
 def moe_sparse_experts_by_token(gate_all, up_all, down_all, n_expert: int, expert_ids, route, token_ids,
                                 token_count: int, down_quant: int, n_ff: int, n_embd: int, x,
-                                n_threads: int = 0) -> np.ndarray:
+                                n_threads: int = 0, avx2: bool = False) -> np.ndarray:
+    """`avx2`: the block dots of rnb-cpu's x86_64 path (same integer sums, another f32 order inside a row): the form
+    that is timed as the CPU baseline; the checks use the scalar form."""
     g, u, d = _u8(gate_all), _u8(up_all), _u8(down_all)
     e = np.ascontiguousarray(expert_ids, dtype=np.uint32)
     r = _f32(route)
@@ -319,11 +321,11 @@ def moe_sparse_experts_by_token(gate_all, up_all, down_all, n_expert: int, exper
     x = _f32(x)
     assert x.size == token_count * n_embd
     out = np.empty((token_count, n_embd), dtype=np.float32)
-    rc = lib().rnbo_moe_sparse_experts_by_token(_p(g), _p(u), _p(d), n_expert, _p(e), _p(r), _p(t), e.size,
-                                                token_count, down_quant, n_ff, n_embd, _p(x), _p(out),
-                                                n_threads)
+    fn = lib().rnbo_moe_sparse_experts_by_token_avx2 if avx2 else lib().rnbo_moe_sparse_experts_by_token
+    rc = fn(_p(g), _p(u), _p(d), n_expert, _p(e), _p(r), _p(t), e.size, token_count, down_quant, n_ff, n_embd, _p(x),
+            _p(out), n_threads)
     if rc != 0:
-        raise RuntimeError(f"rnbo_moe_sparse_experts_by_token failed with code {rc}")
+        raise RuntimeError(f"rnbo_moe_sparse_experts_by_token{'_avx2' if avx2 else ''} failed with code {rc}")
     return out
 
 

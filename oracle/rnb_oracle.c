@@ -972,22 +972,25 @@ size_t rnbo_route_topk(const float *logits, size_t n_expert, size_t k, uint32_t 
  * (compute_expert_host_from_slices): gate/up GEMV on Q8_K(h), SiLU*up, down GEMV on the
  * re-quantised intermediate, scale by the route weight.  Gate/up are Q4_K; down is
  * Q4_K (12), Q5_K (13) or Q6_K (14).  `h_q8k` is the token's already-quantised activation. */
+typedef float (*moe_dot_fn)(const uint8_t *row, const rnbo_q8k_block *act, size_t nb);
+
 static void moe_slot(const uint8_t *gate, const uint8_t *up, const uint8_t *down,
                      uint32_t down_quant, size_t n_ff, size_t n_embd, const rnbo_q8k_block *h_q8k,
                      float route_weight, float *gate_out, float *up_out, rnbo_q8k_block *mid_q8k,
-                     float *expert_out) {
+                     float *expert_out, moe_dot_fn gate_dot, moe_dot_fn down_dot) {
     size_t nb_in = n_embd / 256, nb_mid = n_ff / 256;
     size_t gate_row = nb_in * RNBO_Q4_K_BLOCK_BYTES;
     for (size_t r = 0; r < n_ff; r++) {
-        gate_out[r] = rnbo_dot_q4k_q8k(gate + r * gate_row, h_q8k, nb_in);
-        up_out[r] = rnbo_dot_q4k_q8k(up + r * gate_row, h_q8k, nb_in);
+        gate_out[r] = gate_dot(gate + r * gate_row, h_q8k, nb_in);
+        up_out[r] = gate_dot(up + r * gate_row, h_q8k, nb_in);
     }
     rnbo_silu_mul_inplace(gate_out, up_out, n_ff);
     rnbo_quantize_q8k(gate_out, n_ff, mid_q8k);
     size_t elems;
     size_t down_row = nb_mid * block_bytes_of(down_quant, &elems);
     for (size_t r = 0; r < n_embd; r++) {
-        float o = kquant_dot(down_quant, down + r * down_row, mid_q8k, nb_mid);
+        float o = down_dot ? down_dot(down + r * down_row, mid_q8k, nb_mid)
+                           : kquant_dot(down_quant, down + r * down_row, mid_q8k, nb_mid);
         volatile float scaled = o * route_weight; /* fanout.rs:306-308 */
         expert_out[r] = scaled;
     }
@@ -998,12 +1001,11 @@ static void moe_slot(const uint8_t *gate, const uint8_t *up, const uint8_t *down
  * expert outputs are added in slot order (decode: crates/rnb-llm/.../moe_view.rs:416-426;
  * batched: .../prefill_cpu.rs:167-194 adds in rank order, which is slot order when the caller
  * lists a token's slots by rank). */
-int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_all,
-                                     const uint8_t *down_all, size_t n_expert,
-                                     const uint32_t *expert_ids, const float *route,
-                                     const uint32_t *token_ids, size_t n_slots, size_t token_count,
-                                     uint32_t down_quant, size_t n_ff, size_t n_embd,
-                                     const float *x, float *out, int n_threads) {
+static int moe_by_token(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all,
+                        size_t n_expert, const uint32_t *expert_ids, const float *route,
+                        const uint32_t *token_ids, size_t n_slots, size_t token_count,
+                        uint32_t down_quant, size_t n_ff, size_t n_embd, const float *x, float *out,
+                        int n_threads, moe_dot_fn gate_dot, moe_dot_fn down_dot) {
     if (n_ff % 256 != 0 || n_embd % 256 != 0) return 1;
     if (down_quant != 12 && down_quant != 13 && down_quant != 14) return 1;
     for (size_t s = 0; s < n_slots; s++)
@@ -1034,7 +1036,7 @@ int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_
             size_t e = expert_ids[s];
             moe_slot(gate_all + e * per_gate, up_all + e * per_gate, down_all + e * per_down,
                      down_quant, n_ff, n_embd, h_q8k + (size_t)token_ids[s] * nb_in, route[s],
-                     gate_out, up_out, mid, slot_out + (size_t)s * n_embd);
+                     gate_out, up_out, mid, slot_out + (size_t)s * n_embd, gate_dot, down_dot);
         }
         free(gate_out);
         free(up_out);
@@ -1049,6 +1051,33 @@ int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_
     free(h_q8k);
     free(slot_out);
     return 0;
+}
+
+int rnbo_moe_sparse_experts_by_token(const uint8_t *gate_all, const uint8_t *up_all,
+                                     const uint8_t *down_all, size_t n_expert,
+                                     const uint32_t *expert_ids, const float *route,
+                                     const uint32_t *token_ids, size_t n_slots, size_t token_count,
+                                     uint32_t down_quant, size_t n_ff, size_t n_embd,
+                                     const float *x, float *out, int n_threads) {
+    return moe_by_token(gate_all, up_all, down_all, n_expert, expert_ids, route, token_ids, n_slots,
+                        token_count, down_quant, n_ff, n_embd, x, out, n_threads, rnbo_dot_q4k_q8k, NULL);
+}
+
+/* The same call over the AVX2+FMA block dots (Q4_K gate/up; Q6_K down, the other down formats keep
+ * the scalar dot): what rnb-cpu runs on x86_64, timed as the CPU baseline of the MoE configurations.
+ * Integer sums are the scalar form's; the f32 accumulation order inside a row differs, so an
+ * intermediate on a rounding tie can re-quantise to the neighbouring int8. */
+int rnbo_moe_sparse_experts_by_token_avx2(const uint8_t *gate_all, const uint8_t *up_all,
+                                          const uint8_t *down_all, size_t n_expert,
+                                          const uint32_t *expert_ids, const float *route,
+                                          const uint32_t *token_ids, size_t n_slots,
+                                          size_t token_count, uint32_t down_quant, size_t n_ff,
+                                          size_t n_embd, const float *x, float *out, int n_threads) {
+    if (!rnbo_have_avx2()) return 3;
+    return moe_by_token(gate_all, up_all, down_all, n_expert, expert_ids, route, token_ids, n_slots,
+                        token_count, down_quant, n_ff, n_embd, x, out, n_threads, rnbo_dot_q4k_q8k_avx2,
+                        down_quant == 12 ? rnbo_dot_q4k_q8k_avx2
+                                         : (down_quant == 14 ? rnbo_dot_q6k_q8k_avx2 : NULL));
 }
 
 /* ================================================================================ */

@@ -147,6 +147,14 @@ float rnbo_dot_q4k_q8k_avx2(const uint8_t *row, const rnbo_q8k_block *act, size_
 float rnbo_dot_q6k_q8k_avx2(const uint8_t *row, const rnbo_q8k_block *act, size_t n_blocks);
 int rnbo_gemv_avx2(uint32_t quant, const uint8_t *w, size_t rows, size_t cols, const float *x,
                    size_t seq_len, float *out, int n_threads);
+/* rnbo_moe_sparse_experts_by_token over the AVX2 dots (Q5_K down keeps the scalar dot);
+ * returns 3 on a machine without AVX2+FMA.                                            */
+int rnbo_moe_sparse_experts_by_token_avx2(const uint8_t *gate_all, const uint8_t *up_all,
+                                          const uint8_t *down_all, size_t n_expert,
+                                          const uint32_t *expert_ids, const float *route,
+                                          const uint32_t *token_ids, size_t n_slots,
+                                          size_t token_count, uint32_t down_quant, size_t n_ff,
+                                          size_t n_embd, const float *x, float *out, int n_threads);
 
 #ifdef __cplusplus
 }

@@ -48,6 +48,32 @@ def _verdict(oracle, got, ref, g, u, d, e, r, t, tokens, x):
     return flips.moe_verdict(got, ref, g, u, d, N_EXPERT, e, r, t, tokens, Q6_K, N_FF, N_EMBD, x)
 
 
+# ---- CPU: the timed form of the CPU baseline ------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("down_quant", [Q4_K, Q5_K, Q6_K])
+def test_moe_over_the_avx2_dots_is_the_scalar_result_up_to_flips(oracle, down_quant):
+    """The benchmark times the routed call over the AVX2+FMA block dots (the f32 order of rnb-cpu's x86_64 path) and
+    checks the GPU against the scalar form.  Both forms hold the same integer sums: their outputs agree to f32 rounding,
+    or differ by explained re-quantisation flips."""
+    if not oracle.have_avx2():
+        pytest.skip("no AVX2+FMA on this machine")
+    from oracle import flips
+
+    n_expert, n_ff, n_embd, tokens, k = 9, 768, 1024, 6, 4
+    gate = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, 21)
+    up = oracle.make_weights(Q4_K, n_expert * n_ff, n_embd, 22)
+    down = oracle.make_weights(down_quant, n_expert * n_embd, n_ff, 23)
+    x = oracle.fill_normal(tokens * n_embd, 24, 1.0)
+    rng = np.random.default_rng(25)
+    e = np.concatenate([rng.permutation(n_expert)[:k] for _ in range(tokens)]).astype(np.uint32)
+    t = np.repeat(np.arange(tokens, dtype=np.uint32), k)
+    r = rng.random(tokens * k).astype(np.float32)
+    scalar = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    simd = oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x, avx2=True)
+    v = flips.moe_verdict(simd, scalar, gate, up, down, n_expert, e, r, t, tokens, down_quant, n_ff, n_embd, x)
+    assert v["ok"] or v["flip_aware_ok"], {key: v[key] for key in v if key != "flips"}
+
+
 # ---- CPU: the explainer itself ------------------------------------------------------------------------------------------
 
 def test_flip_explainer_accepts_flips_and_rejects_other_errors(oracle):
