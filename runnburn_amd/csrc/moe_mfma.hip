@@ -103,6 +103,7 @@ __device__ __forceinline__ void tile_stage_store(const TileStage<kThreads> &st, 
         const v4i bop = q45_operand<SB, kFifth>(ROW);                                                    \
         SC = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                          \
         ACC = __builtin_amdgcn_mfma_i32_32x32x32_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 #define RNB_Q45_TAKE(ACC, SC, TOT)                                                                       \
     {                                                                                                    \
@@ -110,6 +111,7 @@ __device__ __forceinline__ void tile_stage_store(const TileStage<kThreads> &st, 
             TOT[i] += mul24(ACC[i], SC);                                                                 \
             asm volatile("" : "+v"(TOT[i])); /* keep the eight additions a chain, not a tree */          \
         }                                                                                                \
+        asm volatile("" ::"v"(ACC)); /* all sixteen result registers stay the instruction's until here */ \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 #define RNB_Q45_SUB_BLOCK(SB, ROW, TOT)                                                                  \
@@ -212,6 +214,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const TileOps12
         const long bop = q6_operand<SB>(row);                                                            \
         SC = q6_scale<SB>(row);                                                                          \
         ACC = __builtin_amdgcn_mfma_i32_32x32x16_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 #define RNB_Q6_TILE_TAKE(ACC, SC)                                                                        \
     {                                                                                                    \
@@ -219,6 +222,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const TileOps12
             tot[i] += mul24(ACC[i], SC);                                                                 \
             asm volatile("" : "+v"(tot[i]));                                                             \
         }                                                                                                \
+        asm volatile("" ::"v"(ACC)); /* all sixteen result registers stay the instruction's until here */ \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 // issue sub-block SB, then scale the results of SB - 1 (see RNB_Q45_SUB_BLOCK)
