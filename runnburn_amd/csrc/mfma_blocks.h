@@ -172,17 +172,19 @@ __device__ __forceinline__ void q6dw_setup(Q6RouteDw &rt, uint32_t row_bytes, in
     rt.loff = rr * kQ6StripStride + 16 * (j < 13 ? j : 12);
     rt.sh = 0;
 }
-// base: block b of the wave's first row
+// base: block b of the wave's first row, the same for every lane (a scalar base and a 32-bit lane offset leave the
+// address arithmetic to the load instruction; the offsets count from four bytes below the base so that they stay
+// unsigned: the first piece of the wave's first row sits at offset -m)
 __device__ __forceinline__ void q6dw_load(Q6RouteDw &rt, const uint8_t *__restrict__ base, int lane) {
     const uint32_t j = lane & 15;
     const uint32_t m = (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(base)) + rt.goff[0]) & 2u;  // the row's block start mod 4
-    // pieces start m bytes early; slot 13 takes bytes 192 + m .. 208 + m of the block.  Signed: the first piece of the
-    // wave's first row sits at offset -m
-    const int32_t adj = j < 13 ? -static_cast<int32_t>(m) : static_cast<int32_t>(m);
+    // pieces start m bytes early; slot 13 takes bytes 192 + m .. 208 + m of the block
+    const uint32_t adj = j < 13 ? 4u - m : 4u + m;
     rt.sh = 8 * m;
+    const uint8_t *below = base - 4;
 #pragma unroll
     for (int i = 0; i < Q6RouteDw::kN; i++)
-        rt.v[i] = *reinterpret_cast<const uint4_a4 *>(base + static_cast<ptrdiff_t>(static_cast<int32_t>(rt.goff[i]) + adj));
+        rt.v[i] = *reinterpret_cast<const uint4_a4 *>(below + static_cast<size_t>(rt.goff[i] + adj));
 }
 __device__ __forceinline__ void q6dw_store(const Q6RouteDw &rt, uint8_t *strip, int lane) {
     const uint32_t j = lane & 15;

@@ -468,7 +468,8 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     __shared__ TileMap s_map;
     const TileImage<kStride, !kSix> img{s_dyn, nb, img_toks};
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: the wave's row addresses are scalar bases plus lane offsets
     const int lrow = lane & 31, khalf = lane >> 5;
     const uint32_t grp = blockIdx.y;
     const uint32_t expert = grp_expert[grp], start = grp_start[grp], count = grp_start[grp + 1] - start;
@@ -492,10 +493,12 @@ __global__ void __launch_bounds__(kGbThreads, 2)
     Q6RouteDw route;
     if constexpr (kSix) q6dw_setup(route, static_cast<uint32_t>(row_bytes), lane);
     float d_next = 0.0f;
+    const uint32_t d_off = static_cast<uint32_t>(lrow) * static_cast<uint32_t>(row_bytes) + 208;  // the lane's row's d from the wave's first row
     auto q6_request = [&](uint32_t rt, uint32_t b) {  // block b of row tile rt: pieces into route.v, d into d_next
-        const uint32_t first = (rt0 + rt) * kGbRows + wave * 32;  // the wave's first row
-        q6dw_load(route, down_e + static_cast<size_t>(first) * row_bytes + b * kBlockBytes, lane);
-        d_next = ld_f16(block_ptr(rt, b) + 208);
+        const uint32_t first = (rt0 + rt) * kGbRows + wave * 32;  // the wave's first row (whole tiles: no row past the end)
+        const uint8_t *base = down_e + static_cast<size_t>(first) * row_bytes + b * kBlockBytes;
+        q6dw_load(route, base, lane);
+        d_next = ld_f16(base + static_cast<size_t>(d_off));
     };
     auto q6_take = [&](Q6Row &r) {
         q6dw_store(route, strip, lane);
