@@ -101,24 +101,56 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         long aop_cur[kTT], aop_nxt[kTT];  // the tokens' operands are read from LDS one sub-block ahead of their use
 #pragma unroll
         for (int t = 0; t < kTT; t++) aop_cur[t] = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64);
+#define RNB_Q6_SCALE(ACC, SC)                                                                                          \
+    {                                                                                                                  \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
+                tot[t][i] += mul24(ACC[t][i], SC); /* |I_sb| <= 16 * 32 * 127 */                                       \
+                asm volatile("" : "+v"(tot[t][i])); /* no re-association of the sixteen sums into a tree */            \
+            }                                                                                                          \
+        }                                                                                                              \
+    }
 #define RNB_Q6_SUB_BLOCK(SB)                                                                                           \
     {                                                                                                                  \
         const long bop = q6_operand<SB>(cur);                                                                          \
         const int sc = q6_scale<SB>(cur);                                                                              \
-        v16i acc[kTT];                                                                                                 \
         _Pragma("unroll") for (int t = 0; t < kTT; t++)                                                                \
             aop_nxt[t] = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * ((SB) < 15 ? (SB) + 1 : 15)); \
-        _Pragma("unroll") for (int t = 0; t < kTT; t++)                                                                \
-            acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop_cur[t], bop, zero16, 0, 0, 0);                          \
-        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
-            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
-                tot[t][i] += mul24(acc[t][i], sc); /* |I_sb| <= 16 * 32 * 127 */                                       \
-                asm volatile("" : "+v"(tot[t][i])); /* no re-association of the sixteen sums into a tree */            \
+        if constexpr (kTT == 1) {                                                                                      \
+            /* one token tile: the instruction of this sub-block is issued before the previous sub-block's results */  \
+            /* are scaled (two result sets in turn, all sixteen registers of a set the instruction's until then) */    \
+            if constexpr (((SB) & 1) == 0) {                                                                           \
+                acc_a[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop_cur[0], bop, zero16, 0, 0, 0);                    \
+                sc_a = sc;                                                                                             \
+                asm volatile("" : "+v"(acc_a[0])); /* pins the instruction in front of the fence */                   \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                if constexpr ((SB) > 0) {                                                                              \
+                    RNB_Q6_SCALE(acc_b, sc_b)                                                                          \
+                    asm volatile("" ::"v"(acc_b[0]));                                                                  \
+                }                                                                                                      \
+            } else {                                                                                                   \
+                acc_b[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop_cur[0], bop, zero16, 0, 0, 0);                    \
+                sc_b = sc;                                                                                             \
+                asm volatile("" : "+v"(acc_b[0]));                                                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                RNB_Q6_SCALE(acc_a, sc_a)                                                                              \
+                asm volatile("" ::"v"(acc_a[0]));                                                                      \
             }                                                                                                          \
+            if constexpr ((SB) == 15) {                                                                                \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                RNB_Q6_SCALE(acc_b, sc_b)                                                                              \
+            }                                                                                                          \
+        } else {                                                                                                       \
+            v16i acc[kTT];                                                                                             \
+            _Pragma("unroll") for (int t = 0; t < kTT; t++)                                                            \
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop_cur[t], bop, zero16, 0, 0, 0);                      \
+            RNB_Q6_SCALE(acc, sc)                                                                                      \
         }                                                                                                              \
         _Pragma("unroll") for (int t = 0; t < kTT; t++) aop_cur[t] = aop_nxt[t];                                       \
         __builtin_amdgcn_sched_barrier(0);                                                                             \
     }
+        [[maybe_unused]] v16i acc_a[1], acc_b[1];  // the one-tile form's two result sets
+        [[maybe_unused]] int sc_a = 0, sc_b = 0;
         RNB_Q6_SUB_BLOCK(0)
         RNB_Q6_SUB_BLOCK(1)
         RNB_Q6_SUB_BLOCK(2)
@@ -135,6 +167,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         RNB_Q6_SUB_BLOCK(13)
         RNB_Q6_SUB_BLOCK(14)
         RNB_Q6_SUB_BLOCK(15)
+#undef RNB_Q6_SCALE
 #undef RNB_Q6_SUB_BLOCK
 
         // out += (d * d_x) * float(sum): result i of a tile is token 8 * (i / 4) + 4 * khalf + i % 4

@@ -103,6 +103,7 @@ __device__ __forceinline__ void tile_stage_store(const TileStage<kThreads> &st, 
         const v4i bop = q45_operand<SB, kFifth>(ROW);                                                    \
         SC = byte_of(sc8.sc_lo, sc8.sc_hi, SB);                                                          \
         ACC = __builtin_amdgcn_mfma_i32_32x32x32_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+        asm volatile("" : "+v"(ACC)); /* pins the instruction in front of the fence */                  \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 #define RNB_Q45_TAKE(ACC, SC, TOT)                                                                       \
@@ -214,6 +215,7 @@ __device__ __forceinline__ void q45_block_tile(const Q5Row &row, const TileOps12
         const long bop = q6_operand<SB>(row);                                                            \
         SC = q6_scale<SB>(row);                                                                          \
         ACC = __builtin_amdgcn_mfma_i32_32x32x16_i8(aops.v[SB], bop, zero16, 0, 0, 0);                   \
+        asm volatile("" : "+v"(ACC));                                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                               \
     }
 #define RNB_Q6_TILE_TAKE(ACC, SC)                                                                        \
