@@ -635,7 +635,8 @@ def bench_ffn(rnb, hip, stream, tokens, steps, seed):
 # configs that --only can run alone: quant, rows, cols, tokens
 ONLY = {"cfg1": (Q8_0, 4096, 4096, 1), "cfg2": (Q4_K, 14336, 4096, 1), "cfg3a": (Q6_K, 4096, 14336, 1),
         "cfg3b": (Q6_K, 128256, 4096, 1), "cfg4": (Q4_K, 14336, 4096, 512), "q6gemm": (Q6_K, 4096, 14336, 512), "q5gemm": (Q5_K, 14336, 4096, 512),
-        "moe1": 1, "moe4": 4, "moe64": 64}  # moeN: configs[4] at N tokens
+        "moe1": 1, "moe4": 4, "moe64": 64,  # moeN: configs[4] at N tokens
+        "ffn1": 1, "ffn512": 512}  # ffnN: the dense Llama-3-8B FFN at N tokens
 
 
 def run_only(rnb, hip, stream, name, calibration):
@@ -644,6 +645,10 @@ def run_only(rnb, hip, stream, name, calibration):
         calibration_copy(hip, rnb, stream)
     if name.startswith("moe"):
         res = bench_moe(rnb, hip, stream, ONLY[name], 0, 1234 + ONLY[name], cpu=False)
+        print(json.dumps({"only": name, "step_ms_median": res["ms_median"], "launches": res["launches"]}), flush=True)
+        return 0
+    if name.startswith("ffn"):
+        res = bench_ffn(rnb, hip, stream, ONLY[name], 0, 4321)
         print(json.dumps({"only": name, "step_ms_median": res["ms_median"], "launches": res["launches"]}), flush=True)
         return 0
     quant, rows, cols, seq = ONLY[name]

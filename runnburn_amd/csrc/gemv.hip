@@ -20,6 +20,7 @@
 #include "block_dots.h"
 #include "device_utils.h"
 #include "kernels.h"
+#include <cstdlib>
 
 namespace rnb {
 
@@ -233,7 +234,7 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 // gap behind it disappear from a decode step.
 // ---------------------------------------------------------------------------------------------
 constexpr int kFusedWaves = 8;   // waves per workgroup: each quantises 16 / 8 = 2 blocks of the token
-constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (more measured slower)
+constexpr int kDepth = 1;        // rows requested ahead of the one being reduced (two, with three register sets: 8.16 against 7.99 us)
 constexpr uint32_t kFusedTargetWaves = 4096;  // 3584, 4784 and 7168 (whole rows per wave for 14336 rows) measured slower
 // Waves of a one-launch decode kernel for `groups` row groups: one per group up to kFusedTargetWaves, except where two
 // groups per wave make 1536 - 2048 waves, i.e. one workgroup per compute unit or a little less: then half as many
@@ -287,20 +288,44 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     const uint32_t ab = has_block ? bslot : 0;
     const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
 
-    for (; grp < row_groups; grp += n_waves) {
+    auto reduce = [&](const typename Q::Regs &r, bool ok) {
         row = grp * kRowsPerWave + rsel;
-        bool far_live;
-        const typename Q::Regs far = fetch(grp + kDepth * n_waves, &far_live);
-        float acc = live[0] ? kquant_partial<kQuant>(regs[0], a, g) : 0.0f;
+        float acc = ok ? kquant_partial<kQuant>(r, a, g) : 0.0f;
         acc = seg_sum<kLanesPerRow>(acc);
         if (sub == kLanesPerRow - 1 && row < rows) out[static_cast<size_t>(tok) * rows + row] = acc;
-#pragma unroll
-        for (int i = 0; i + 1 < kDepth; i++) {
-            regs[i] = regs[i + 1];
-            live[i] = live[i + 1];
+    };
+    // The register sets take turns: handing the look-ahead row's registers over to "the current row" at the end of an
+    // iteration would be a copy, and a copy waits for the loads it copies, so that no request would be in flight while
+    // a wave waits
+    if constexpr (kDepth == 1) {
+        typename Q::Regs other;
+        bool other_live;
+        while (grp < row_groups) {
+            other = fetch(grp + n_waves, &other_live);
+            reduce(regs[0], live[0]);
+            grp += n_waves;
+            if (grp >= row_groups) break;
+            regs[0] = fetch(grp + n_waves, &live[0]);
+            reduce(other, other_live);
+            grp += n_waves;
         }
-        regs[kDepth - 1] = far;
-        live[kDepth - 1] = far_live;
+    } else {
+        static_assert(kDepth <= 2, "register sets of the row loop");
+        typename Q::Regs third;
+        bool third_live;
+        while (grp < row_groups) {
+            third = fetch(grp + 2 * n_waves, &third_live);
+            reduce(regs[0], live[0]);
+            grp += n_waves;
+            if (grp >= row_groups) break;
+            regs[0] = fetch(grp + 2 * n_waves, &live[0]);
+            reduce(regs[kDepth - 1], live[kDepth - 1]);
+            grp += n_waves;
+            if (grp >= row_groups) break;
+            regs[kDepth - 1] = fetch(grp + 2 * n_waves, &live[kDepth - 1]);
+            reduce(third, third_live);
+            grp += n_waves;
+        }
     }
 }
 
@@ -438,22 +463,29 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     const uint32_t ab = has_block ? bslot : 0;
     const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
 
-    for (; grp < row_groups; grp += n_waves) {
+    // Three register sets take turns as current, next and far row group: handing a set's registers on by copy would
+    // wait for the loads it copies at the end of every iteration, with nothing in flight meanwhile.  One step requests
+    // the group two ahead into the free set and reduces the current one.
+    Q4KRegs fg, fu;
+    bool far_live;
+    auto step = [&](const Q4KRegs &cg, const Q4KRegs &cu, bool clive, Q4KRegs &tg, Q4KRegs &tu, bool &tlive) {
         const uint32_t row = grp * kRowsPerWave + rsel;
-        bool far_live;
-        off = offset_of(grp + 2 * n_waves, &far_live);
-        const Q4KRegs fg = q4k_load_block(wg + off, g), fu = q4k_load_block(wu + off, g);
-        float gs = live ? q4k_partial(rg, a4, g) : 0.0f;
-        float us = live ? q4k_partial(ru, a4, g) : 0.0f;
+        const size_t o = offset_of(grp + 2 * n_waves, &tlive);
+        tg = q4k_load_block(wg + o, g);
+        tu = q4k_load_block(wu + o, g);
+        float gs = clive ? q4k_partial(cg, a4, g) : 0.0f;
+        float us = clive ? q4k_partial(cu, a4, g) : 0.0f;
         gs = seg_sum<kLanesPerRow>(gs);
         us = seg_sum<kLanesPerRow>(us);
         if (sub == kLanesPerRow - 1 && row < rows) mid[static_cast<size_t>(tok) * rows + row] = act_mul<kGelu>(gs, us);
-        rg = ng;
-        ru = nu;
-        live = next_live;
-        ng = fg;
-        nu = fu;
-        next_live = far_live;
+        grp += n_waves;
+    };
+    while (grp < row_groups) {
+        step(rg, ru, live, fg, fu, far_live);
+        if (grp >= row_groups) break;
+        step(ng, nu, next_live, rg, ru, live);
+        if (grp >= row_groups) break;
+        step(fg, fu, far_live, ng, nu, next_live);
     }
 }
 
@@ -565,17 +597,23 @@ __global__ void __launch_bounds__(kWave *kFusedWaves)
     const uint32_t ab = has_block ? bslot : 0;
     const Q4KAct a4 = q4k_load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
 
-    for (; grp < row_groups; grp += n_waves) {
+    // three register sets in turn (see gemv_q4k_gate_up_f32_kernel): no copies, so no wait for the rows in flight
+    Q4KRegs far;
+    bool far_live;
+    auto step = [&](const Q4KRegs &c, bool clive, Q4KRegs &t, bool &tlive) {
         const uint32_t row = grp * kRowsPerWave + rsel;
-        bool far_live;
-        const Q4KRegs far = fetch(grp + 2 * n_waves, &far_live);
-        float acc = live ? q4k_partial(cur, a4, g) : 0.0f;
+        t = fetch(grp + 2 * n_waves, &tlive);
+        float acc = clive ? q4k_partial(c, a4, g) : 0.0f;
         acc = seg_sum<kLanesPerRow>(acc);
         if (sub == kLanesPerRow - 1 && row < rows) out[row] = acc;
-        cur = nxt;
-        live = next_live;
-        nxt = far;
-        next_live = far_live;
+        grp += n_waves;
+    };
+    while (grp < row_groups) {
+        step(cur, live, far, far_live);
+        if (grp >= row_groups) break;
+        step(nxt, next_live, cur, live);
+        if (grp >= row_groups) break;
+        step(far, far_live, nxt, next_live);
     }
 }
 
