@@ -378,17 +378,29 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
         mv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (blk < n_blocks) mv[i] = reinterpret_cast<const float4 *>(mid + static_cast<size_t>(blk) * 256)[lane];
     }
+    // The token's expert ids and route weights go to LDS once: the table is a kernel argument, and a look-up by a lane's
+    // slot is a vector load from it that the compiler waits for together with every other load of the wave (the next
+    // slots' weights were only requested once the current ones had arrived, and each route weight cost a round trip).
+    // (Wave-uniform scalar look-ups with a select per lane instead of this copy measured slower.)
+    __shared__ uint32_t s_expert[kMoeDecodeMaxPerToken];
+    __shared__ float s_route[kMoeDecodeMaxPerToken];
+    if (threadIdx.x < n_slots) {
+        s_expert[threadIdx.x] = table.expert[first + threadIdx.x];
+        s_route[threadIdx.x] = table.route[first + threadIdx.x];
+    }
     // slot k of row `row`; past the token's slots the walk goes on with the next row's first slots
-    auto fetch = [&](uint32_t row, uint32_t k, bool *ok) {
+    auto fetch_of = [&](uint32_t row, uint32_t k, uint32_t expert, bool *ok) {
         *ok = b < nb && row < n_embd && k < n_slots;
         const uint8_t *blk = down_all;  // dead lanes read the first block of the tensor
         if (*ok)
-            blk = expert_base(down_all, down_shared, n_routed, table.expert[first + k], n_embd * row_bytes) +
+            blk = expert_base(down_all, down_shared, n_routed, expert, n_embd * row_bytes) +
                   static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
         return Q::load_block(blk, g);
     };
+    auto fetch = [&](uint32_t row, uint32_t k, bool *ok) { return fetch_of(row, k, s_expert[k < n_slots ? k : 0], ok); };
     bool cur_ok;
-    typename Q::Regs cur = fetch(row0, grp, &cur_ok);
+    // (the first request goes out before the barrier that publishes the LDS copy: it reads the table itself)
+    typename Q::Regs cur = fetch_of(row0, grp, table.expert[first + (grp < n_slots ? grp : 0)], &cur_ok);
 #pragma unroll
     for (int i = 0; i < kSpans; i++) {
         const uint32_t blk = wave + i * kDecodeWaves;
@@ -411,7 +423,7 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
                 o = kquant_partial<kQuant>(cur, Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g), g);
             }
             o = seg_sum<kLanes>(o);
-            if (k < n_slots) o *= table.route[first + k];  // fanout.rs:306-308; only the group's last lane is read below
+            if (k < n_slots) o *= s_route[k];  // fanout.rs:306-308; only the group's last lane is read below
 #pragma unroll
             for (int j = 0; j < kGroups; j++) {
                 const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
