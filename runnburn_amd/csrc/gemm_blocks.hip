@@ -345,23 +345,56 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         const uint8_t *abase = s_a[buf] + lrow * kGbStride64 + 8 * khalf;
 
         // as in the Q6_K kernel: the empty asm and the scheduling barrier keep the sixteen sub-blocks a chain
+#define RNB_Q23_SCALE(ACC, SC)                                                                                         \
+    {                                                                                                                  \
+        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
+            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
+                tot[t][i] += mul24(ACC[t][i], SC); /* |I_sb| <= 16 * 4 * 127 */                                        \
+                asm volatile("" : "+v"(tot[t][i]));                                                                    \
+            }                                                                                                          \
+        }                                                                                                              \
+    }
 #define RNB_Q23_SUB_BLOCK(SB)                                                                                          \
     {                                                                                                                  \
         const long bop = q23_operand<SB, kThree>(cur);                                                                 \
         const int sc = q23_scale<SB, kThree>(cur);                                                                     \
-        v16i acc[kTT]; /* the tiles' instructions first, then their results: see the Q6_K kernel */                    \
-        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
-            const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);                  \
-            acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                                 \
-        }                                                                                                              \
-        _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                              \
-            _Pragma("unroll") for (int i = 0; i < kLive; i++) {                                                        \
-                tot[t][i] += mul24(acc[t][i], sc); /* |I_sb| <= 16 * 4 * 127 */                                        \
-                asm volatile("" : "+v"(tot[t][i]));                                                                    \
+        if constexpr (kTT == 1) {                                                                                      \
+            /* one token tile: this sub-block's instruction before the previous sub-block's scaling, see the Q6_K */   \
+            /* kernel */                                                                                               \
+            const long aop = *reinterpret_cast<const long *>(abase + 16 * SB);                                         \
+            if constexpr (((SB) & 1) == 0) {                                                                           \
+                acc_a[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                           \
+                sc_a = sc;                                                                                             \
+                asm volatile("" : "+v"(acc_a[0]));                                                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                if constexpr ((SB) > 0) {                                                                              \
+                    RNB_Q23_SCALE(acc_b, sc_b)                                                                         \
+                    asm volatile("" ::"v"(acc_b[0]));                                                                  \
+                }                                                                                                      \
+            } else {                                                                                                   \
+                acc_b[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                           \
+                sc_b = sc;                                                                                             \
+                asm volatile("" : "+v"(acc_b[0]));                                                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                RNB_Q23_SCALE(acc_a, sc_a)                                                                             \
+                asm volatile("" ::"v"(acc_a[0]));                                                                      \
             }                                                                                                          \
+            if constexpr ((SB) == 15) {                                                                                \
+                __builtin_amdgcn_sched_barrier(0);                                                                     \
+                RNB_Q23_SCALE(acc_b, sc_b)                                                                             \
+            }                                                                                                          \
+        } else {                                                                                                       \
+            v16i acc[kTT]; /* the tiles' instructions first, then their results: see the Q6_K kernel */                \
+            _Pragma("unroll") for (int t = 0; t < kTT; t++) {                                                          \
+                const long aop = *reinterpret_cast<const long *>(abase + 32 * t * kGbStride64 + 16 * SB);              \
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop, zero16, 0, 0, 0);                             \
+            }                                                                                                          \
+            RNB_Q23_SCALE(acc, sc)                                                                                     \
         }                                                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                                                             \
     }
+        [[maybe_unused]] v16i acc_a[1], acc_b[1];  // the one-tile form's two result sets
+        [[maybe_unused]] int sc_a = 0, sc_b = 0;
         RNB_Q23_SUB_BLOCK(0)
         RNB_Q23_SUB_BLOCK(1)
         RNB_Q23_SUB_BLOCK(2)
@@ -379,6 +412,7 @@ __global__ void __launch_bounds__(kGbThreads, 2)
         RNB_Q23_SUB_BLOCK(14)
         RNB_Q23_SUB_BLOCK(15)
 #undef RNB_Q23_SUB_BLOCK
+#undef RNB_Q23_SCALE
 
         // Q2_K mins: K slot i of the lane's K-half is sub-block 8 khalf + i on both sides
         const uint32_t mn0 = ((khalf ? cur.sc.z : cur.sc.x) >> 4) & 0x0f0f0f0fu, mn1 = ((khalf ? cur.sc.w : cur.sc.y) >> 4) & 0x0f0f0f0fu;
