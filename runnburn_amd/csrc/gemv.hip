@@ -795,19 +795,21 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
 }
 
 // ---------------------------------------------------------------------------------------------
-// Split-K GEMV of ONE f32 token in one launch, rows of 17 to 32 super-blocks: a workgroup of 16 waves quantises the whole
-// token to Q8_K in its LDS (two blocks per wave, the wave-level quantiser of the stand-alone kernel, so the same bits),
+// Split-K GEMV of ONE f32 token in one launch, rows of 17 to 48 super-blocks: a workgroup of 16 waves quantises the whole
+// token to Q8_K in its LDS (up to three blocks per wave, the wave-level quantiser of the stand-alone kernel, so the same bits),
 // then works as `teams` split-K teams of n_slices waves, each team on rows of its own; the partial sums of up to
 // kSplitBatch rows per team wait for one barrier and are added in slice order, as in gemv_kquant_splitk_kernel (the same
 // bits).  The teams of a launch are as many as the split-K kernel has workgroups, so the weight stream looks the same;
 // the token is read once per 16 waves, and the quantiser's launch and the gap behind it go: 8192 x 8192 Q4_K 10.9 ->
-// 9.9 us per step, 13824 x 5120 12.3 -> 11.2, 28672 x 8192 25.7 -> 24.8, 2048 x 8192 7.1 -> 5.5.  The kernel is written for
-// any number of slices up to 16 waves' worth, but with three and four slices (rows of up to 64 super-blocks, four blocks
-// to quantise per wave) it loses to the two launches (4096 x 14336 Q6_K 13.2 vs 12.9 us, 4096 x 11008 16.0 vs 12.0),
-// and with four rows per team requested before the quantisation instead of one it loses more (17.7 us).
+// 9.9 us per step, 13824 x 5120 12.3 -> 11.2, 28672 x 8192 25.7 -> 24.8, 2048 x 8192 7.1 -> 5.5.  Inside a batch the next
+// row is requested before the current one is reduced, in two register sets that take turns: 8192 x 8192 10.2 -> 9.95,
+// 13824 x 5120 11.6 -> 10.3, Q6_K 5120 x 5120 9.6 -> 8.5, and with three slices the kernel now beats the two launches
+// (4096 x 11008 Q4_K 9.15 vs 10.07 us; it was 16.0 vs 12.0 with every row waited for before the next request).  With four
+// slices (four blocks to quantise per wave) it still does not (4096 x 14336 Q6_K 13.5 vs 13.3, Q4_K 10.7 vs 10.8), and
+// with four rows per team requested before the quantisation instead of one it loses more (17.7 us).
 // ---------------------------------------------------------------------------------------------
 constexpr int kWideWaves = 16;
-constexpr uint32_t kWideMaxBlocks = 32;
+constexpr uint32_t kWideMaxBlocks = 48;  // three K slices; with four the two launches win (below)
 constexpr int kWidePre = 1;  // rows per team requested before the token is quantised (at most kSplitBatch)
 template <uint32_t kQuant>
 __global__ void __launch_bounds__(kWave *kWideWaves)
@@ -838,11 +840,12 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 256)[lane];
     }
+    // (idle lanes and rows past the end read a valid block; their sums are masked out below)
+    const size_t lane_off = static_cast<size_t>(has_block ? b : 0) * kBlockBytes;
+    auto row_of = [&](uint32_t pass) { return pass * stride + first + team; };
     auto fetch = [&](uint32_t pass) {
-        const uint32_t row = pass * stride + first + team;
-        Regs r = Regs{};  // idle lanes and rows past the end keep zeros
-        if (has_block && row < rows) r = Q::load_block(w + static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes, g);
-        return r;
+        const uint32_t row = row_of(pass);
+        return Q::load_block(w + static_cast<size_t>(row < rows ? row : 0) * row_bytes + lane_off, g);
     };
     Regs pre[kWidePre];  // the first passes' rows: in flight while the token is quantised
 #pragma unroll
@@ -857,21 +860,32 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
     const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
     for (uint32_t p0 = 0; p0 < n_pass; p0 += kSplitBatch) {
         const uint32_t n = n_pass - p0 < static_cast<uint32_t>(kSplitBatch) ? n_pass - p0 : kSplitBatch;
+        auto partial = [&](const Regs &r, uint32_t k) {
+            float acc = kquant_partial<kQuant>(r, a, g);
+            acc = seg_sum<kWave>(has_block && row_of(p0 + k) < rows ? acc : 0.0f);
+            if (lane == kWave - 1) s_part[k][wave] = acc;
+        };
+        uint32_t k = 0;
         if (p0 == 0) {
 #pragma unroll
-            for (int k = 0; k < kWidePre; k++) {
-                if (static_cast<uint32_t>(k) < n) {
-                    float acc = kquant_partial<kQuant>(pre[k], a, g);
-                    acc = seg_sum<kWave>(has_block ? acc : 0.0f);
-                    if (lane == kWave - 1) s_part[k][wave] = acc;
-                }
+            for (int i = 0; i < kWidePre; i++) {
+                if (static_cast<uint32_t>(i) < n) partial(pre[i], i);
             }
+            k = kWidePre;
         }
-        for (uint32_t k = p0 == 0 ? kWidePre : 0; k < n; k++) {
-            const Regs r = fetch(p0 + k);
-            float acc = kquant_partial<kQuant>(r, a, g);
-            acc = seg_sum<kWave>(has_block ? acc : 0.0f);
-            if (lane == kWave - 1) s_part[k][wave] = acc;
+        // the batch's remaining rows, the next one requested before the current one is reduced; two register sets in
+        // turn (a copy from "next" to "current" would wait for the loads it copies)
+        if (k < n) {
+            Regs ra = fetch(p0 + k), rb;
+            while (k < n) {
+                rb = fetch(p0 + k + 1);
+                partial(ra, k);
+                k++;
+                if (k >= n) break;
+                ra = fetch(p0 + k + 1);
+                partial(rb, k);
+                k++;
+            }
         }
         __syncthreads();
         if (threadIdx.x < n * teams) {
@@ -1501,7 +1515,7 @@ bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb) {
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
                             uint32_t seq, hipStream_t stream) {
     if (rows == 0 || seq == 0) return;
-    if (nb > 16) {  // rows of 17 to 32 super-blocks: one token per launch
+    if (nb > 16) {  // rows of 17 to 64 super-blocks: one token per launch
         for (uint32_t t = 0; t < seq; t++) {
             const float *xt = x + static_cast<size_t>(t) * nb * 256;
             float *ot = out + static_cast<size_t>(t) * rows;
