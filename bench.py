@@ -351,7 +351,7 @@ def one_launch_step(quant, rows, cols, seq):
         return False
     if quant in (10, 11, Q4_K, Q5_K, Q6_K):
         nb = cols // 256
-        return nb <= 32 and (nb <= 8 or rows * nb * BLOCK_BYTES.get(quant, 144) < (300 << 20))
+        return nb <= 64 and (nb <= 8 or rows * nb * BLOCK_BYTES.get(quant, 144) < (300 << 20))
     return cols // 32 <= 128 and rows * (cols // 32) >= 1 << 18
 
 

@@ -795,32 +795,37 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
 }
 
 // ---------------------------------------------------------------------------------------------
-// Split-K GEMV of ONE f32 token in one launch, rows of 17 to 48 super-blocks: a workgroup of 16 waves quantises the whole
-// token to Q8_K in its LDS (up to three blocks per wave, the wave-level quantiser of the stand-alone kernel, so the same bits),
-// then works as `teams` split-K teams of n_slices waves, each team on rows of its own; the partial sums of up to
+// Split-K GEMV of ONE f32 token in one launch, rows of 17 to 64 super-blocks: a workgroup of 16 waves quantises the whole
+// token to Q8_K in its LDS (kSlices blocks per wave, the wave-level quantiser of the stand-alone kernel, so the same bits),
+// then works as `teams` split-K teams of kSlices waves, each team on rows of its own; the partial sums of up to
 // kSplitBatch rows per team wait for one barrier and are added in slice order, as in gemv_kquant_splitk_kernel (the same
 // bits).  The teams of a launch are as many as the split-K kernel has workgroups, so the weight stream looks the same;
 // the token is read once per 16 waves, and the quantiser's launch and the gap behind it go: 8192 x 8192 Q4_K 10.9 ->
 // 9.9 us per step, 13824 x 5120 12.3 -> 11.2, 28672 x 8192 25.7 -> 24.8, 2048 x 8192 7.1 -> 5.5.  Inside a batch the next
 // row is requested before the current one is reduced, in two register sets that take turns: 8192 x 8192 10.2 -> 9.95,
-// 13824 x 5120 11.6 -> 10.3, Q6_K 5120 x 5120 9.6 -> 8.5, and with three slices the kernel now beats the two launches
+// 13824 x 5120 11.6 -> 10.3, Q6_K 5120 x 5120 9.6 -> 8.5, and with three slices the kernel then beats the two launches
 // (4096 x 11008 Q4_K 9.15 vs 10.07 us; it was 16.0 vs 12.0 with every row waited for before the next request).  With four
-// slices (four blocks to quantise per wave) it still does not (4096 x 14336 Q6_K 13.5 vs 13.3, Q4_K 10.7 vs 10.8), and
-// with four rows per team requested before the quantisation instead of one it loses more (17.7 us).
+// slices it needs two rows per team in flight while the four blocks per wave are quantised (kWidePre, chosen by the
+// launcher): 4096 x 14336 Q4_K 10.1 us against 10.8 in two launches (10.7 with one early row), Q6_K 13.0 against 13.3
+// (13.5); three early rows spill.  The slice count is a template parameter: with two slices the blocks past the end
+// of the token are quantised as zeros rather than branched around, which lets the compiler interleave the two chains
+// of max, division and rounding (Q6_K 5120 x 5120 8.84 -> 8.45 us); with three or four that loses 1.5 % and the
+// branches stay.
 // ---------------------------------------------------------------------------------------------
 constexpr int kWideWaves = 16;
-constexpr uint32_t kWideMaxBlocks = 48;  // three K slices; with four the two launches win (below)
-constexpr int kWidePre = 1;  // rows per team requested before the token is quantised (at most kSplitBatch)
-template <uint32_t kQuant>
+constexpr uint32_t kWideMaxBlocks = 64;
+template <uint32_t kQuant, uint32_t kSlices, int kWidePre>
 __global__ void __launch_bounds__(kWave *kWideWaves)
     gemv_kquant_wide_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
-                                uint32_t rows, uint32_t nb, uint32_t n_slices, uint32_t teams) {
+                                uint32_t rows, uint32_t nb) {
     using Q = KQuant<kQuant>;
     using Regs = typename Q::Regs;
     constexpr size_t kBlockBytes = Q::kBytes;
-    __shared__ __attribute__((aligned(16))) int8_t s_qs[kWideMaxBlocks * 256];
-    __shared__ float s_d[kWideMaxBlocks];
-    __shared__ __attribute__((aligned(16))) int16_t s_bsums[kWideMaxBlocks * 16];
+    constexpr uint32_t n_slices = kSlices, teams = kWideWaves / kSlices;
+    constexpr uint32_t kBlocks = kSlices * 16;  // LDS image of the token: blocks past nb are quantised zeros
+    __shared__ __attribute__((aligned(16))) int8_t s_qs[kBlocks * 256];
+    __shared__ float s_d[kBlocks];
+    __shared__ __attribute__((aligned(16))) int16_t s_bsums[kBlocks * 16];
     __shared__ float s_part[kSplitBatch][kWideWaves];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = threadIdx.x >> 6;
@@ -833,9 +838,9 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
     const uint32_t first = blockIdx.x * teams;          // this workgroup's first row of pass 0
     const uint32_t n_pass = (rows + stride - 1) / stride;
     // the token is requested first: loads return in order, and the quantiser must not wait for weights
-    float4 xv[kWideMaxBlocks / kWideWaves];
+    float4 xv[kSlices];
 #pragma unroll
-    for (int i = 0; i < static_cast<int>(kWideMaxBlocks) / kWideWaves; i++) {
+    for (uint32_t i = 0; i < kSlices; i++) {
         const uint32_t blk = wave + i * kWideWaves;
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (blk < nb) xv[i] = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 256)[lane];
@@ -850,10 +855,11 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
     Regs pre[kWidePre];  // the first passes' rows: in flight while the token is quantised
 #pragma unroll
     for (int i = 0; i < kWidePre; i++) pre[i] = fetch(i);
+    // with two slices every wave quantises both of its blocks, whether they exist or not (zeros past nb)
 #pragma unroll
-    for (int i = 0; i < static_cast<int>(kWideMaxBlocks) / kWideWaves; i++) {
+    for (uint32_t i = 0; i < kSlices; i++) {
         const uint32_t blk = wave + i * kWideWaves;
-        if (blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
+        if (kSlices == 2 || blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
     }
     __syncthreads();
     const uint32_t ab = has_block ? b : 0;
@@ -908,8 +914,23 @@ void launch_kquant_wide_f32(const uint8_t *w, const float *x, float *out, uint32
     // one workgroup of sixteen waves per compute unit's share of kTargetWaves
     const uint32_t want = kTargetWaves / kWideWaves;
     const uint32_t all = (rows + teams - 1) / teams;
-    hipLaunchKernelGGL((gemv_kquant_wide_f32_kernel<kQuant>), dim3(all < want ? all : want), dim3(kWave * kWideWaves), 0, stream,
-                       w, x, out, rows, nb, n_slices, teams);
+    const dim3 grid(all < want ? all : want), block(kWave * kWideWaves);
+    // kWidePre, the rows per team requested before the token is quantised: two where a wave has four blocks to quantise,
+    // and with two slices when the launch makes four passes or more (8192 x 8192 Q4_K 9.8 -> 9.4 us, Q6_K 13.4 -> 13.1;
+    // with two or three passes the second early row costs more than it hides: 5120 x 5120 Q4_K 6.6 -> 7.0, Q6_K 8.4 -> 9.4);
+    // three with four slices spills (Q6_K 19.3 us)
+    const uint32_t n_pass = (rows + grid.x * teams - 1) / (grid.x * teams);
+#define RNB_LAUNCH_WIDE(S, P) \
+    hipLaunchKernelGGL((gemv_kquant_wide_f32_kernel<kQuant, S, P>), grid, block, 0, stream, w, x, out, rows, nb)
+    if (n_slices == 2 && n_pass >= 4)
+        RNB_LAUNCH_WIDE(2, 2);
+    else if (n_slices == 2)
+        RNB_LAUNCH_WIDE(2, 1);
+    else if (n_slices == 3)
+        RNB_LAUNCH_WIDE(3, 1);
+    else
+        RNB_LAUNCH_WIDE(4, 2);
+#undef RNB_LAUNCH_WIDE
 }
 
 template <uint32_t kQuant, int kRowsPerWave>

@@ -335,15 +335,16 @@ def test_gemv_into_and_zero_sized(rnb, oracle):
                                              (Q4_K, 37, 4352), (Q5_K, 300, 8192), (Q6_K, 9, 16384), (Q2_K, 100, 16640),
                                              (Q4_K, 33, 32768), (Q6_K, 21, 33024), (Q3_K, 4101, 5120), (Q6_K, 1030, 28672),
                                              (Q4_K, 20011, 8192), (Q2_K, 2050, 4608), (Q5_K, 7, 6144), (Q6_K, 8193, 8192),
-                                             (Q4_K, 301, 12288), (Q2_K, 77, 8448), (Q6_K, 5, 12544)])
+                                             (Q4_K, 301, 12288), (Q2_K, 77, 8448), (Q6_K, 5, 12544),
+                                             (Q5_K, 6200, 4352), (Q2_K, 10000, 4608), (Q3_K, 4097, 16384), (Q4_K, 1027, 13824)])
 def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols):
     """rnb_hip_gemv_dev and its two halves (rnb_hip_quantize_dev + rnb_hip_gemv_quantized_dev, for callers that
     feed several matrices from one activation) run the same arithmetic: identical bits.  For K-quant rows of at most
-    48 super-blocks, and 32-element formats with rows of at most 128 blocks, gemv_dev is a one-launch kernel whose
-    workgroups quantise the token themselves (from 17 super-blocks on as split-K teams inside sixteen-wave workgroups;
-    rows longer than 48 keep the separate quantiser, which measured faster there); the shapes cover 1, 2 and 4 rows per
-    wave, row counts that are no multiple of those or of the eight teams, more row groups than waves, and 2 to 9 K slices
-    with full and partly idle last slices."""
+    64 super-blocks, and 32-element formats with rows of at most 128 blocks, gemv_dev is a one-launch kernel whose
+    workgroups quantise the token themselves (from 17 super-blocks on as split-K teams inside sixteen-wave workgroups,
+    with one or two rows per team requested before the token is quantised; longer rows keep the separate quantiser);
+    the shapes cover 1, 2 and 4 rows per wave, row counts that are no multiple of those or of the teams, more row groups
+    than waves, launches of one to ten passes, and 2 to 9 K slices with full and partly idle last slices."""
     w = oracle.make_weights(quant, rows, cols, 900 + rows)
     x = oracle.fill_normal(cols, 901 + cols, 1.0)
     wd, xd = rnb.DeviceBuffer.from_host(w), rnb.DeviceBuffer.from_host(x)
