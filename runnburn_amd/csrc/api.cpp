@@ -214,7 +214,7 @@ int run_matmul_quantized_dev(State &s, uint32_t quant, const uint8_t *w_dev, siz
 int run_matmul_dev(State &s, uint32_t quant, const uint8_t *w_dev, size_t rows, size_t cols, const float *x_dev,
                    size_t seq, float *out_dev, Arena *arena = nullptr) {
     // one token against rows of at most 64 super-blocks: the GEMV's workgroups quantise the token themselves
-    if (seq == 1 && !is_block32(quant) && gemv_kquant_f32_supported(quant, static_cast<uint32_t>(cols / 256), x_dev) &&
+    if (seq == 1 && !is_block32(quant) && gemv_kquant_f32_supported(quant, static_cast<uint32_t>(cols / 256), x_dev, w_dev) &&
         gemv_kquant_f32_pays(quant, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 256))) {
         launch_gemv_kquant_f32(w_dev, quant, x_dev, out_dev, static_cast<uint32_t>(rows), static_cast<uint32_t>(cols / 256),
                                1, s.stream);

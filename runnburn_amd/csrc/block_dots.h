@@ -198,11 +198,16 @@ struct Q6KRegs {
     uint32_t sh;    // 8 m: the funnel shift that puts the pieces right
 };
 
+// kEvenBase: the caller has checked that the matrix starts at an even address.  Without the odd-address path the four
+// loads stay whole in the compiled code; with it the compiler merges the two paths into single-dword loads that it
+// groups again later, not always as they were (a piece fetched as 1 + 3 dwords needs a register copy and a wait where
+// a kernel assigns the register set).
+template <bool kEvenBase = false>
 __device__ __forceinline__ Q6KRegs q6k_load_block(const uint8_t *__restrict__ blk, int q) {
     Q6KRegs r;
     const int n = q >> 1, th = q & 1;
     uint32_t m = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(blk)) & 3u;
-    if (m & 1u) {  // a matrix at an odd address (the same for every lane): the pieces themselves, whatever it costs
+    if (!kEvenBase && (m & 1u)) {  // a matrix at an odd address (the same for every lane): the pieces themselves, whatever it costs
         r.A = ld_u4_a2(blk + 64 * n + 16 * th);
         r.B = ld_u4_a2(blk + 64 * n + 32 + 16 * th);
         r.H = ld_u4_a2(blk + 128 + 32 * n + 16 * th);
@@ -435,6 +440,7 @@ struct KQuant<kQ2K> {
         return q6k_load_act(aq_blk, dx, bs_blk, q);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q2k_load_block(blk, q); }
+    static __device__ __forceinline__ Regs load_block_even(const uint8_t *blk, int q) { return q2k_load_block(blk, q); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q2k_prepare(r, q); }
     static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q2k_dot(p, a); }
 };
@@ -449,6 +455,7 @@ struct KQuant<kQ3K> {
         return q6k_load_act(aq_blk, dx, bs_blk, q);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q3k_load_block(blk, q); }
+    static __device__ __forceinline__ Regs load_block_even(const uint8_t *blk, int q) { return q3k_load_block(blk, q); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q3k_prepare(r, q); }
     static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q3k_dot(p, a); }
 };
@@ -463,6 +470,7 @@ struct KQuant<kQ4K> {
         return q4k_load_act(aq_blk, dx, bs_blk, g);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int g) { return q4k_load_block(blk, g); }
+    static __device__ __forceinline__ Regs load_block_even(const uint8_t *blk, int g) { return q4k_load_block(blk, g); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int g) { return q4k_prepare(r, g); }
     static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q4k_dot(p, a); }
 };
@@ -477,6 +485,7 @@ struct KQuant<kQ5K> {
         return q4k_load_act(aq_blk, dx, bs_blk, g);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int g) { return q5k_load_block(blk, g); }
+    static __device__ __forceinline__ Regs load_block_even(const uint8_t *blk, int g) { return q5k_load_block(blk, g); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int g) { return q5k_prepare(r, g); }
     static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q4k_dot(p, a); }
 };
@@ -491,6 +500,8 @@ struct KQuant<kQ6K> {
         return q6k_load_act(aq_blk, dx, bs_blk, q);
     }
     static __device__ __forceinline__ Regs load_block(const uint8_t *blk, int q) { return q6k_load_block(blk, q); }
+    // for a matrix at an even address (checked on the host)
+    static __device__ __forceinline__ Regs load_block_even(const uint8_t *blk, int q) { return q6k_load_block<true>(blk, q); }
     static __device__ __forceinline__ Prep prepare(const Regs &r, int q) { return q6k_prepare(r, q); }
     static __device__ __forceinline__ float dot(const Prep &p, const Act &a) { return q6k_dot(p, a); }
 };

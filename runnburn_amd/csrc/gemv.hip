@@ -800,21 +800,31 @@ void launch_kquant_splitk(const uint8_t *w, ActView act, float *out, uint32_t ro
 // then works as `teams` split-K teams of kSlices waves, each team on rows of its own; the partial sums of up to
 // kSplitBatch rows per team wait for one barrier and are added in slice order, as in gemv_kquant_splitk_kernel (the same
 // bits).  The teams of a launch are as many as the split-K kernel has workgroups, so the weight stream looks the same;
-// the token is read once per 16 waves, and the quantiser's launch and the gap behind it go: 8192 x 8192 Q4_K 10.9 ->
-// 9.9 us per step, 13824 x 5120 12.3 -> 11.2, 28672 x 8192 25.7 -> 24.8, 2048 x 8192 7.1 -> 5.5.  Inside a batch the next
-// row is requested before the current one is reduced, in two register sets that take turns: 8192 x 8192 10.2 -> 9.95,
-// 13824 x 5120 11.6 -> 10.3, Q6_K 5120 x 5120 9.6 -> 8.5, and with three slices the kernel then beats the two launches
-// (4096 x 11008 Q4_K 9.15 vs 10.07 us; it was 16.0 vs 12.0 with every row waited for before the next request).  With four
-// slices it needs two rows per team in flight while the four blocks per wave are quantised (kWidePre, chosen by the
-// launcher): 4096 x 14336 Q4_K 10.1 us against 10.8 in two launches (10.7 with one early row), Q6_K 13.0 against 13.3
-// (13.5); three early rows spill.  The slice count is a template parameter: with two slices the blocks past the end
-// of the token are quantised as zeros rather than branched around, which lets the compiler interleave the two chains
-// of max, division and rounding (Q6_K 5120 x 5120 8.84 -> 8.45 us); with three or four that loses 1.5 % and the
-// branches stay.
+// the token is read once per 16 waves, and the quantiser's launch and the gap behind it go.
+//
+// Two register sets take turns over ALL of a wave's rows: the first is requested before the token is quantised, the
+// second right behind the quantisation (in front of the barrier), and each again as soon as its row is reduced, also
+// across the batches' barriers.  Steps measured against quantiser + split-K GEMV in two launches (us): 4096 x 14336 Q6_K
+// 11.2 vs 13.3, Q4_K 9.3 vs 10.8, 4096 x 11008 Q4_K 8.2 vs 10.1, 8192 x 8192 Q4_K 8.45 vs 10.9, Q6_K 11.9 vs 14.1,
+// 13824 x 5120 Q4_K 9.8 vs 12.3, 28672 x 8192 Q4_K 23.8 vs 25.7.  What it took, in the order found:
+//  * a loop that waited for every row before requesting the next lost to the two launches from three slices on
+//    (4096 x 11008 16.0 vs 12.0 us); with the next row of a batch requested ahead: 9.15;
+//  * that loop started its two sets anew after the early rows and after every batch, with nothing in flight in between,
+//    and needed TWO early rows with four slices to win (13.0 us on 4096 x 14336 Q6_K; three spill); as one pipeline over
+//    all rows ONE early row is best everywhere (11.2 us; two: 12.5; none: 12.9);
+//  * requests that only some paths make (the last rows, a second set when there is a second pass) cost every path a full
+//    wait, because the compiler's wait counts follow the issue order of the worst path: the steady-state loop requests
+//    unconditionally, and the last one to three rows are code of their own;
+//  * the Q6_K loader without its odd-address path (load_block_even; the launcher sends such matrices to the two
+//    launches): with it the compiler merged both paths into single-dword loads and grouped them again as 1 + 3 dwords
+//    for one piece, copied into place (and waited for) where the set is assigned, i.e. in front of the barrier.
+// The slice count is a template parameter: with two slices the blocks past the end of the token are quantised as
+// zeros rather than branched around, which lets the compiler interleave the two chains of max, division and rounding
+// (Q6_K 5120 x 5120 8.84 -> 8.45 us); with three or four that loses 1.5 % and the branches stay.
 // ---------------------------------------------------------------------------------------------
 constexpr int kWideWaves = 16;
 constexpr uint32_t kWideMaxBlocks = 64;
-template <uint32_t kQuant, uint32_t kSlices, int kWidePre>
+template <uint32_t kQuant, uint32_t kSlices>
 __global__ void __launch_bounds__(kWave *kWideWaves)
     gemv_kquant_wide_f32_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
                                 uint32_t rows, uint32_t nb) {
@@ -850,50 +860,31 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
     auto row_of = [&](uint32_t pass) { return pass * stride + first + team; };
     auto fetch = [&](uint32_t pass) {
         const uint32_t row = row_of(pass);
-        return Q::load_block(w + static_cast<size_t>(row < rows ? row : 0) * row_bytes + lane_off, g);
+        return Q::load_block_even(w + static_cast<size_t>(row < rows ? row : 0) * row_bytes + lane_off, g);
     };
-    Regs pre[kWidePre];  // the first passes' rows: in flight while the token is quantised
-#pragma unroll
-    for (int i = 0; i < kWidePre; i++) pre[i] = fetch(i);
+    // two register sets in turn (a copy from a "next" set to a "current" one would wait for the loads it copies)
+    Regs s0 = fetch(0), s1;
     // with two slices every wave quantises both of its blocks, whether they exist or not (zeros past nb)
 #pragma unroll
     for (uint32_t i = 0; i < kSlices; i++) {
         const uint32_t blk = wave + i * kWideWaves;
         if (kSlices == 2 || blk < nb) q8k_quantize_vals(xv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
     }
+    // (with a single pass the second set fetches the first row again: a request that only some launches make would
+    // cost all of them a full wait in front of the first row, see below)
+    s1 = fetch(1 < n_pass ? 1 : 0);
     __syncthreads();
     const uint32_t ab = has_block ? b : 0;
     const typename Q::Act a = Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g);
-    for (uint32_t p0 = 0; p0 < n_pass; p0 += kSplitBatch) {
-        const uint32_t n = n_pass - p0 < static_cast<uint32_t>(kSplitBatch) ? n_pass - p0 : kSplitBatch;
-        auto partial = [&](const Regs &r, uint32_t k) {
-            float acc = kquant_partial<kQuant>(r, a, g);
-            acc = seg_sum<kWave>(has_block && row_of(p0 + k) < rows ? acc : 0.0f);
-            if (lane == kWave - 1) s_part[k][wave] = acc;
-        };
-        uint32_t k = 0;
-        if (p0 == 0) {
-#pragma unroll
-            for (int i = 0; i < kWidePre; i++) {
-                if (static_cast<uint32_t>(i) < n) partial(pre[i], i);
-            }
-            k = kWidePre;
-        }
-        // the batch's remaining rows, the next one requested before the current one is reduced; two register sets in
-        // turn (a copy from "next" to "current" would wait for the loads it copies)
-        if (k < n) {
-            Regs ra = fetch(p0 + k), rb;
-            while (k < n) {
-                rb = fetch(p0 + k + 1);
-                partial(ra, k);
-                k++;
-                if (k >= n) break;
-                ra = fetch(p0 + k + 1);
-                partial(rb, k);
-                k++;
-            }
-        }
+    auto partial = [&](const Regs &r, uint32_t pass) {
+        float acc = kquant_partial<kQuant>(r, a, g);
+        acc = seg_sum<kWave>(has_block && row_of(pass) < rows ? acc : 0.0f);
+        if (lane == kWave - 1) s_part[pass % kSplitBatch][wave] = acc;
+    };
+    // the batch that ends with pass `last`: slice sums added in slice order, one thread per row
+    auto flush = [&](uint32_t last) {
         __syncthreads();
+        const uint32_t p0 = last - last % kSplitBatch, n = last - p0 + 1;
         if (threadIdx.x < n * teams) {
             const uint32_t k = threadIdx.x / teams, tm = threadIdx.x - k * teams;
             const uint32_t row = (p0 + k) * stride + first + tm;
@@ -904,7 +895,30 @@ __global__ void __launch_bounds__(kWave *kWideWaves)
             }
         }
         __syncthreads();  // the sums are read before the next batch overwrites them
+    };
+    static_assert(kSplitBatch % 2 == 0, "a batch ends behind the second register set");
+    // While both sets have a row left to request, the requests are unconditional: the waits the compiler places count
+    // requests in issue order, and a request that only one path makes costs every path a full wait.
+    uint32_t pass = 0;
+    for (; pass + 3 < n_pass; pass += 2) {
+        partial(s0, pass);
+        s0 = fetch(pass + 2);
+        partial(s1, pass + 1);
+        s1 = fetch(pass + 3);
+        if ((pass + 1) % kSplitBatch == kSplitBatch - 1) flush(pass + 1);
     }
+    // one to three passes are left: s0 holds the first of them, s1 the second
+    if (n_pass - pass == 3) {
+        partial(s0, pass);
+        s0 = fetch(pass + 2);
+        partial(s1, pass + 1);
+        if ((pass + 1) % kSplitBatch == kSplitBatch - 1) flush(pass + 1);
+        partial(s0, pass + 2);
+    } else {
+        partial(s0, pass);
+        if (n_pass - pass == 2) partial(s1, pass + 1);
+    }
+    flush(n_pass - 1);
 }
 
 template <uint32_t kQuant>
@@ -915,21 +929,14 @@ void launch_kquant_wide_f32(const uint8_t *w, const float *x, float *out, uint32
     const uint32_t want = kTargetWaves / kWideWaves;
     const uint32_t all = (rows + teams - 1) / teams;
     const dim3 grid(all < want ? all : want), block(kWave * kWideWaves);
-    // kWidePre, the rows per team requested before the token is quantised: two where a wave has four blocks to quantise,
-    // and with two slices when the launch makes four passes or more (8192 x 8192 Q4_K 9.8 -> 9.4 us, Q6_K 13.4 -> 13.1;
-    // with two or three passes the second early row costs more than it hides: 5120 x 5120 Q4_K 6.6 -> 7.0, Q6_K 8.4 -> 9.4);
-    // three with four slices spills (Q6_K 19.3 us)
-    const uint32_t n_pass = (rows + grid.x * teams - 1) / (grid.x * teams);
-#define RNB_LAUNCH_WIDE(S, P) \
-    hipLaunchKernelGGL((gemv_kquant_wide_f32_kernel<kQuant, S, P>), grid, block, 0, stream, w, x, out, rows, nb)
-    if (n_slices == 2 && n_pass >= 4)
-        RNB_LAUNCH_WIDE(2, 2);
-    else if (n_slices == 2)
-        RNB_LAUNCH_WIDE(2, 1);
+#define RNB_LAUNCH_WIDE(S) \
+    hipLaunchKernelGGL((gemv_kquant_wide_f32_kernel<kQuant, S>), grid, block, 0, stream, w, x, out, rows, nb)
+    if (n_slices == 2)
+        RNB_LAUNCH_WIDE(2);
     else if (n_slices == 3)
-        RNB_LAUNCH_WIDE(3, 1);
+        RNB_LAUNCH_WIDE(3);
     else
-        RNB_LAUNCH_WIDE(4, 2);
+        RNB_LAUNCH_WIDE(4);
 #undef RNB_LAUNCH_WIDE
 }
 
@@ -1510,8 +1517,10 @@ void launch_gemv_q6k(const uint8_t *w, ActView act, float *out, uint32_t rows, u
     launch_kquant_any<kQ6K>(w, act, out, rows, nb, seq, stream);
 }
 
-bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x) {
+bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x, const void *w) {
     const bool kq = quant == kQ2K || quant == kQ3K || quant == kQ4K || quant == kQ5K || quant == kQ6K;
+    // the sixteen-wave kernel fetches Q6_K blocks without the odd-address path
+    if (quant == kQ6K && nb > 16 && reinterpret_cast<uintptr_t>(w) % 2 != 0) return false;
     return kq && nb >= 1 && nb <= kWideMaxBlocks && reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 

@@ -77,10 +77,11 @@ void launch_gemv_q4k_gate_up_f32(const uint8_t *wg, const uint8_t *wu, const flo
                                  uint32_t nb, uint32_t seq, bool gelu, hipStream_t stream);
 void launch_gemv_q4k_multi_f32(const uint8_t *const w[3], const uint32_t rows[3], const float *x, float *out, uint32_t nb,
                                hipStream_t stream);
-// K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 32
-// super-blocks (beyond 16 a workgroup of sixteen waves works as eight split-K teams of two waves), x 16-byte aligned; same output
-// contract and the same bits as launch_gemv_q4k on the stand-alone quantiser's output
-bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x);
+// K-quant GEMV straight from f32 tokens (the workgroup quantises its token to Q8_K in LDS): rows of at most 64
+// super-blocks (beyond 16 a workgroup of sixteen waves works as split-K teams of two to four waves; its Q6_K form wants
+// the matrix at an even address), x 16-byte aligned; same output contract and the same bits as launch_gemv_q4k on the
+// stand-alone quantiser's output
+bool gemv_kquant_f32_supported(uint32_t quant, uint32_t nb, const void *x, const void *w);
 // false for matrices so large that quantising with a launch of its own and running the chunked GEMV is faster
 bool gemv_kquant_f32_pays(uint32_t quant, uint32_t rows, uint32_t nb);
 void launch_gemv_kquant_f32(const uint8_t *w, uint32_t quant, const float *x, float *out, uint32_t rows, uint32_t nb,
