@@ -361,6 +361,30 @@ def test_gemv_dev_equals_split_quantise_then_gemv(rnb, oracle, quant, rows, cols
         buf.free()
 
 
+@pytest.mark.parametrize("quant,rows,cols", [(Q6_K, 100, 5120), (Q6_K, 33, 14336), (Q4_K, 100, 5120), (Q5_K, 33, 11008),
+                                             (Q6_K, 50, 2048)])
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_gemv_sub_range_at_unaligned_device_address(rnb, oracle, quant, rows, cols, shift):
+    """A matrix that is a sub-range of a resident parent, 1, 2 or 3 bytes in, is read at parent + offset on the device
+    (crates/rnb-backend/cuda/src/runtime/state/q4k_cache.rs:722-741) and gives the bits of the aligned one (the reference
+    reads rows at any byte offset, crates/rnb-cpu/src/gemm/quant_gemv.rs:1257-1296).  Rows of 17 to 64 super-blocks: the
+    one-launch kernel fetches Q6_K blocks without the odd-address path, so a Q6_K matrix at an odd address must take the
+    quantiser + GEMV route."""
+    w = oracle.make_weights(quant, rows, cols, 77 + rows)
+    x = oracle.fill_normal(cols, 78, 1.0)
+    base = gemv_fn(rnb, quant)(w, rows, cols, x)
+    rnb.release(w)
+    parent = np.zeros(w.size + 8, np.uint8)
+    parent[shift:shift + w.size] = w
+    rnb.prewarm([parent])
+    before = rnb.transfer_counters()[0]
+    got = gemv_fn(rnb, quant)(parent[shift:shift + w.size], rows, cols, x)
+    assert rnb.transfer_counters()[0] - before == cols * 4, "the sub-range must not be uploaded again"
+    assert np.array_equal(got, base)
+    check_close(got, oracle.gemv(quant, w, rows, cols, x)[0], None, f"quant {quant} {rows}x{cols}")
+    rnb.release(parent)
+
+
 # ---- batches: seq-major layout, ragged token counts ----------------------------------------------
 
 @pytest.mark.parametrize("quant", [Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0])
