@@ -619,7 +619,7 @@ int run_moe_dev(State &s, const uint8_t *gate_dev, const uint8_t *up_dev, const 
             max_per_token = std::max<size_t>(max_per_token, table.tok_off[t + 1]);
             table.tok_off[t + 1] += table.tok_off[t];
         }
-        if (moe_decode_supported(token_count, n_slots, max_per_token, sh.nb_in, sh.nb_mid, x_dev)) {
+        if (moe_decode_supported(token_count, n_slots, max_per_token, sh.nb_in, sh.nb_mid, x_dev, down_quant, down_dev, shared.down)) {
             uint32_t fill[kMoeDecodeMaxTokens] = {};
             for (size_t i = 0; i < n_slots; i++) {  // token by token, list order kept inside a token
                 const uint32_t t = token_ids[i], at = table.tok_off[t] + fill[t]++;

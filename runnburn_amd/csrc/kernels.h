@@ -207,7 +207,8 @@ struct MoeDecodeTable {
     uint32_t tok_off[kMoeDecodeMaxTokens + 1];
 };
 // max_per_token: the largest number of slots any one token has
-bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x);
+bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x,
+                          uint32_t down_quant, const void *down, const void *down_shared);
 void launch_moe_decode(const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all, const MoeShared &shared,
                        uint32_t down_quant,
                        const MoeDecodeTable &table, const float *x, float *mid, float *out, uint32_t n_ff, uint32_t n_embd,

@@ -293,7 +293,8 @@ __global__ void __launch_bounds__(kWave *kWavesPerWg)
 //                               gemv_kquant_f32_kernel does), every wave makes one group of rows of its slot's expert
 //   moe_decode_down_kernel      grid (rows / 8, tokens): the workgroup quantises its token's slots' intermediates
 //                               (slots * nb_mid <= 64 blocks) in LDS, then moe_down_token_kernel's row scheme: down,
-//                               route weight, ordered sum
+//                               route weight, ordered sum; two register sets in turn over the wave's (row, slot group)
+//                               steps (four tokens of 8 slots on 128 experts 24.0 -> 23.0 us per call)
 // Same quantiser, dots and order of additions as the general path, so the same bits.  An expert that several tokens
 // chose is read once per slot here (the second time mostly from the L2), which is what bounds the batch this pays for.
 // ---------------------------------------------------------------------------------------------
@@ -384,10 +385,11 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     // (Wave-uniform scalar look-ups with a select per lane instead of this copy measured slower.)
     __shared__ uint32_t s_expert[kMoeDecodeMaxPerToken];
     __shared__ float s_route[kMoeDecodeMaxPerToken];
-    if (threadIdx.x < n_slots) {
-        s_expert[threadIdx.x] = table.expert[first + threadIdx.x];
-        s_route[threadIdx.x] = table.route[first + threadIdx.x];
-    }
+    // (every thread reads an entry, together with the first two steps' expert ids below and in front of the first weight
+    // request: one wait for all table reads; the copy itself is written behind that request)
+    const uint32_t stage = first + (threadIdx.x < n_slots ? threadIdx.x : 0);
+    const uint32_t stage_expert = table.expert[stage];
+    const float stage_route = table.route[stage];
     // slot k of row `row`; past the token's slots the walk goes on with the next row's first slots
     auto fetch_of = [&](uint32_t row, uint32_t k, uint32_t expert, bool *ok) {
         *ok = b < nb && row < n_embd && k < n_slots;
@@ -395,44 +397,92 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
         if (*ok)
             blk = expert_base(down_all, down_shared, n_routed, expert, n_embd * row_bytes) +
                   static_cast<size_t>(row) * row_bytes + static_cast<size_t>(b) * kBlockBytes;
-        return Q::load_block(blk, g);
+        return Q::load_block_even(blk, g);  // the launcher has checked the tensors' addresses
     };
-    auto fetch = [&](uint32_t row, uint32_t k, bool *ok) { return fetch_of(row, k, s_expert[k < n_slots ? k : 0], ok); };
-    bool cur_ok;
-    // (the first request goes out before the barrier that publishes the LDS copy: it reads the table itself)
-    typename Q::Regs cur = fetch_of(row0, grp, table.expert[first + (grp < n_slots ? grp : 0)], &cur_ok);
+    if (n_slots == 0) {  // workgroup-uniform: a token without slots gets zero rows
+        if (lane == 0) {
+            for (int r = 0; r < kRows; r++)
+                if (row0 + r < n_embd) out[static_cast<size_t>(tok) * n_embd + row0 + r] = 0.0f;
+        }
+        return;
+    }
+    // The wave's work is a sequence of steps, one group of kGroups slots of one row each, rows in order.  Two register
+    // sets take turns over the steps, each requested again as soon as its step is reduced (handing a look-ahead set
+    // over to "the current one" would be a copy, and a copy waits for the loads it copies).  The first two steps read
+    // their expert ids from the table itself, both before the first weight request (a look-up behind it would wait
+    // for the weights too); the later ones read the LDS copy.
+    const uint32_t n_groups = (n_slots + kGroups - 1) / kGroups, total = kRows * n_groups;
+    const uint32_t k1 = n_groups > 1 ? kGroups + grp : grp;                           // step 1: the row's second group,
+    const uint32_t row1 = n_groups > 1 ? row0 : (kRows > 1 ? row0 + 1 : n_embd);      // or the next row's first one
+    const uint32_t e0 = table.expert[first + (grp < n_slots ? grp : 0)], e1 = table.expert[first + (k1 < n_slots ? k1 : 0)];
+    bool ok0, ok1;
+    typename Q::Regs s0 = fetch_of(row0, grp, e0, &ok0), s1;
+    if (threadIdx.x < n_slots) {
+        s_expert[threadIdx.x] = stage_expert;
+        s_route[threadIdx.x] = stage_route;
+    }
 #pragma unroll
     for (int i = 0; i < kSpans; i++) {
         const uint32_t blk = wave + i * kDecodeWaves;
         if (blk < n_blocks) q8k_quantize_vals(mv[i], lane, s_qs + blk * 256, s_d + blk, s_bsums + blk * 16);
     }
+    s1 = fetch_of(row1, k1, e1, &ok1);
     __syncthreads();
-#pragma unroll 1
-    for (int r = 0; r < kRows; r++) {
-        const uint32_t row = row0 + r;
-        float acc = 0.0f;
-        for (uint32_t k0 = 0; k0 < n_slots; k0 += kGroups) {
-            const uint32_t k = k0 + grp;
-            bool nxt_ok;
-            // the next group of this row, or (kRows > 1) the first group of the next row
-            const bool wrap = kRows > 1 && k0 + kGroups >= n_slots;
-            const typename Q::Regs nxt = wrap ? fetch(r + 1 < kRows ? row + 1 : n_embd, grp, &nxt_ok) : fetch(row, k + kGroups, &nxt_ok);
-            float o = 0.0f;
-            if (cur_ok) {
-                const uint32_t ab = k * nb + b;
-                o = kquant_partial<kQuant>(cur, Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g), g);
-            }
-            o = seg_sum<kLanes>(o);
-            if (k < n_slots) o *= s_route[k];  // fanout.rs:306-308; only the group's last lane is read below
-#pragma unroll
-            for (int j = 0; j < kGroups; j++) {
-                const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
-                if (k0 + j < n_slots) acc += v;  // wave-uniform
-            }
-            cur = nxt;
-            cur_ok = nxt_ok;
+    // the request cursor stands at step 2, the reduce cursor at step 0 (row index and first slot of the group)
+    uint32_t fr = 0, fk0 = 0, cr = 0, ck0 = 0;
+    auto advance = [&](uint32_t &r, uint32_t &k0) {
+        k0 += kGroups;
+        if (k0 >= n_slots) {
+            k0 = 0;
+            r++;
         }
-        if (lane == 0 && row < n_embd) out[static_cast<size_t>(tok) * n_embd + row] = acc;
+    };
+    advance(fr, fk0);
+    advance(fr, fk0);
+    auto fetch_next = [&](bool *ok) {  // past the last step: dead lanes' block
+        const uint32_t k = fk0 + grp;
+        const typename Q::Regs r = fetch_of(fr < static_cast<uint32_t>(kRows) ? row0 + fr : n_embd, k, s_expert[k < n_slots ? k : 0], ok);
+        advance(fr, fk0);
+        return r;
+    };
+    float acc = 0.0f;
+    auto reduce = [&](const typename Q::Regs &regs, bool ok) {
+        const uint32_t k = ck0 + grp;
+        float o = 0.0f;
+        if (ok) {
+            const uint32_t ab = k * nb + b;
+            o = kquant_partial<kQuant>(regs, Q::load_act(s_qs + ab * 256, s_d[ab], s_bsums + ab * 16, g), g);
+        }
+        o = seg_sum<kLanes>(o);
+        if (k < n_slots) o *= s_route[k];  // fanout.rs:306-308; only the group's last lane is read below
+#pragma unroll
+        for (int j = 0; j < kGroups; j++) {
+            const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, o), j * kLanes + kLanes - 1));
+            if (ck0 + j < n_slots) acc += v;  // wave-uniform
+        }
+        if (ck0 + kGroups >= n_slots) {  // the row's last group
+            if (lane == 0 && row0 + cr < n_embd) out[static_cast<size_t>(tok) * n_embd + row0 + cr] = acc;
+            acc = 0.0f;
+        }
+        advance(cr, ck0);
+    };
+    // while both sets have a step left to request the requests are unconditional (the compiler's wait counts follow the
+    // issue order of the worst path); the last one to three steps are code of their own
+    uint32_t s = 0;
+    for (; s + 3 < total; s += 2) {
+        reduce(s0, ok0);
+        s0 = fetch_next(&ok0);
+        reduce(s1, ok1);
+        s1 = fetch_next(&ok1);
+    }
+    if (total - s == 3) {
+        reduce(s0, ok0);
+        s0 = fetch_next(&ok0);
+        reduce(s1, ok1);
+        reduce(s0, ok0);
+    } else {
+        reduce(s0, ok0);
+        if (total - s == 2) reduce(s1, ok1);
     }
 }
 
@@ -571,7 +621,10 @@ void launch_moe_down_token(const uint8_t *down_all, const MoeShared &shared, uin
 #undef RNB_LAUNCH_DT
 }
 
-bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x) {
+bool moe_decode_supported(size_t n_tokens, size_t n_slots, size_t max_per_token, size_t nb_in, size_t nb_mid, const void *x,
+                          uint32_t down_quant, const void *down, const void *down_shared) {
+    // the down kernel fetches Q6_K blocks without the odd-address path
+    if (down_quant == kQ6K && ((reinterpret_cast<uintptr_t>(down) | reinterpret_cast<uintptr_t>(down_shared)) & 1u) != 0) return false;
     return n_tokens >= 1 && n_tokens <= kMoeDecodeMaxTokens && n_slots >= 1 && n_slots <= kMoeDecodeMaxSlots &&
            max_per_token <= kMoeDecodeMaxPerToken && nb_in >= 1 && nb_in <= 16 && nb_mid >= 1 && nb_mid <= 16 &&
            max_per_token * nb_mid <= 64 && reinterpret_cast<uintptr_t>(x) % 16 == 0;

@@ -793,6 +793,28 @@ def test_moe_one_token_equals_batch_row(rnb, oracle, n_ff, n_embd, k, down_quant
         rnb.release(w)
 
 
+@pytest.mark.parametrize("tokens", [1, 3])
+@pytest.mark.parametrize("shift", [1, 2])
+def test_moe_decode_down_tensor_at_unaligned_device_address(rnb, oracle, tokens, shift):
+    """The down tensor as a sub-range of a resident parent, one or two bytes in: read at parent + offset on the device.  The
+    decode kernels fetch Q6_K blocks without the odd-address path, so at an odd address the call must take the general
+    sequence; either way the bits of the aligned call (the same arithmetic in both sequences)."""
+    n_expert, n_ff, n_embd, k = 6, 512, 768, 3
+    gate, up, down, x, e, r, t = _moe_case(oracle, n_expert, n_ff, n_embd, tokens, k, 9, Q6_K)
+    base = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, down, e, r, t, tokens, Q6_K, n_ff, n_embd, x)
+    rnb.release(down)
+    parent = np.zeros(down.size + 8, np.uint8)
+    parent[shift:shift + down.size] = down
+    rnb.prewarm([parent])
+    got = rnb.qwen35_sparse_experts_selected_base_by_token(gate, up, parent[shift:shift + down.size], e, r, t, tokens, Q6_K,
+                                                           n_ff, n_embd, x)
+    assert np.array_equal(got, base)
+    check_close(got, oracle.moe_sparse_experts_by_token(gate, up, down, n_expert, e, r, t, tokens, Q6_K, n_ff, n_embd, x), None,
+                f"moe decode, down tensor {shift} bytes in")
+    for w in (gate, up, parent):
+        rnb.release(w)
+
+
 @pytest.mark.parametrize("tokens,n_ff,n_embd,k,down_quant", [(2, 768, 2048, 8, Q6_K), (3, 256, 512, 1, Q4_K), (4, 512, 1280, 16, Q5_K),
                                                             (8, 768, 2048, 8, Q6_K), (5, 1024, 768, 3, Q6_K), (8, 2304, 512, 7, Q4_K),
                                                             (7, 256, 4096, 9, Q5_K)])
