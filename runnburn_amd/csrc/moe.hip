@@ -387,7 +387,8 @@ __global__ void __launch_bounds__(kWave *kDecodeWaves)
     __shared__ float s_route[kMoeDecodeMaxPerToken];
     // (every thread reads an entry, together with the first two steps' expert ids below and in front of the first weight
     // request: one wait for all table reads; the copy itself is written behind that request)
-    const uint32_t stage = first + (threadIdx.x < n_slots ? threadIdx.x : 0);
+    const uint32_t stage_at = first + (threadIdx.x < n_slots ? threadIdx.x : 0);
+    const uint32_t stage = stage_at < kMoeDecodeMaxSlots ? stage_at : 0;  // a last token without slots: first = the slot count
     const uint32_t stage_expert = table.expert[stage];
     const float stage_route = table.route[stage];
     // slot k of row `row`; past the token's slots the walk goes on with the next row's first slots
